@@ -1,0 +1,133 @@
+/* C ABI of the MI355X (gfx950) neighbor-list library.
+ *
+ * The two entry points, the three structs and the two enums below have the same names, field order, sizes and
+ * meaning as the ones every vesin binding is written against (reference: vesin/include/vesin.h:36-46 enum
+ * VesinAlgorithm, :49-78 VesinOptions, :81-89 VesinDeviceKind, :103-108 VesinDevice, :129-163 VesinNeighborList,
+ * :167 vesin_free, :191-200 vesin_neighbors), so an existing caller relinks against this library unchanged.
+ * A HIP device is addressed as `VesinCUDA`, which is what PyTorch-ROCm reports for its tensors.
+ *
+ * Layout on x86-64 (checked by tests/test_abi.py):
+ *   VesinOptions       32 bytes: cutoff@0, full@8, sorted@9, algorithm@12, n_threads@16, return_shifts@20,
+ *                                return_distances@21, return_vectors@22, skin@24
+ *   VesinDevice         8 bytes: type@0, device_id@4
+ *   VesinNeighborList  56 bytes: length@0, device@8, pairs@16, shifts@24, distances@32, vectors@40, opaque@48
+ */
+#ifndef VESIN_H
+#define VESIN_H
+
+#include <stddef.h>
+#include <stdint.h>
+#ifndef __cplusplus
+    #include <stdbool.h>
+#endif
+
+#if defined(VESIN_SHARED) && (defined(__GNUC__) || defined(__clang__))
+    #define VESIN_API __attribute__((visibility("default")))
+#else
+    #define VESIN_API
+#endif
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* How candidate pairs are enumerated. The result does not depend on the choice. */
+enum VesinAlgorithm {
+    VesinAutoAlgorithm = 0, /* pick from the number of points and the box */
+    VesinBruteForce = 1,    /* every point against every image of every point, tiled; for small systems */
+    VesinCellList = 2,      /* counting sort into cells + stencil search, O(n) */
+};
+
+struct VesinOptions {
+    double cutoff;             /* pairs with distance strictly below this are returned */
+    bool full;                 /* true: i->j and j->i; false: each pair once */
+    bool sorted;               /* true: pairs ordered by i (this library orders by (i, j, shift)) */
+    enum VesinAlgorithm algorithm;
+    int32_t n_threads;         /* CPU threads; must be >= 0; unused by the GPU path */
+    bool return_shifts;        /* fill VesinNeighborList::shifts */
+    bool return_distances;     /* fill VesinNeighborList::distances */
+    bool return_vectors;       /* fill VesinNeighborList::vectors */
+    double skin;               /* Verlet skin; only 0 is supported by this library */
+};
+
+enum VesinDeviceKind {
+    VesinUnknownDevice = 0, /* a zero-initialised list that owns nothing yet */
+    VesinCPU = 1,
+    VesinCUDA = 2,          /* a GPU; here: a HIP device */
+};
+
+struct VesinDevice {
+    enum VesinDeviceKind type;
+#ifdef __cplusplus
+    int device_id = 0;      /* GPU ordinal; 0 for the CPU */
+#else
+    int device_id;
+#endif
+};
+
+/* Output of one calculation. For pair k with points (i, j) and shift S, the vector is
+ * r_j - r_i + S . box (box vectors as rows). All arrays live on `device` and belong to the library: they stay
+ * valid until the next vesin_neighbors call on the same struct or vesin_free. */
+struct VESIN_API VesinNeighborList {
+#ifdef __cplusplus
+    VesinNeighborList():
+        length(0), device({VesinUnknownDevice, 0}), pairs(nullptr), shifts(nullptr), distances(nullptr),
+        vectors(nullptr) {}
+#endif
+    size_t length;           /* number of pairs */
+    struct VesinDevice device;
+    size_t (*pairs)[2];      /* [length][2] */
+    int32_t (*shifts)[3];    /* [length][3] when return_shifts, else NULL */
+    double* distances;       /* [length]    when return_distances, else NULL */
+    double (*vectors)[3];    /* [length][3] when return_vectors, else NULL */
+#ifdef __cplusplus
+    void* opaque = nullptr;  /* library-private state (device work buffers) */
+#else
+    void* opaque;
+#endif
+};
+
+/* Release everything a list owns and zero the struct. NULL is accepted. (reference: vesin.h:167) */
+void VESIN_API vesin_free(struct VesinNeighborList* neighbors);
+
+/* Compute the neighbor list of `n_points` points. (reference: vesin.h:191-200)
+ *
+ * With device.type == VesinCUDA, `points` ([n_points][3] doubles), `box` (3 box vectors as rows) and `periodic`
+ * (3 one-byte booleans) must be device memory of GPU `device.device_id`. `neighbors` must be zero-initialised
+ * before its first use and may be reused across calls. Work is issued on the null stream and the call returns
+ * after it completed. Returns EXIT_SUCCESS, or EXIT_FAILURE with *error_message pointing to a string owned by the
+ * library (left untouched on success). This library has no CPU engine: VesinCPU is refused with an error. */
+int VESIN_API vesin_neighbors(
+    const double (*points)[3],
+    size_t n_points,
+    const double box[3][3],
+    const bool periodic[3],
+    struct VesinDevice device,
+    struct VesinOptions options,
+    struct VesinNeighborList* neighbors,
+    const char** error_message
+);
+
+/* ---- additions of this library (no counterpart in the reference) ------------------------------------------ */
+
+/* Wall-clock breakdown of the most recent successful GPU call made through `neighbors`, measured with HIP events
+ * on the stream the kernels ran on. Recording is off until vesin_hip_enable_timings(1) was called (it adds event
+ * records to every call). Times are in milliseconds; stages that did not run report 0. */
+struct VesinHipTimings {
+    float total;        /* first launch to last kernel end */
+    float cell_build;   /* bounding box, cell assignment, cell scan, scatter, gather */
+    float count;        /* search, counting pass */
+    float scan;         /* device-wide scan of the per-wave counts */
+    float write;        /* search, writing pass: the kernel that produces the output arrays */
+    float sort;         /* radix sort of (i, j, shift) and payload gather */
+    uint64_t candidates;/* reserved, 0 */
+};
+
+void VESIN_API vesin_hip_enable_timings(int enabled);
+int VESIN_API vesin_hip_last_timings(const struct VesinNeighborList* neighbors, struct VesinHipTimings* timings);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif

@@ -1,0 +1,90 @@
+"""ctypes mirror of include/vesin.h (layouts asserted in tests/test_abi.py)."""
+
+import ctypes
+import os
+
+VesinAutoAlgorithm = 0
+VesinBruteForce = 1
+VesinCellList = 2
+
+VesinUnknownDevice = 0
+VesinCPU = 1
+VesinCUDA = 2
+
+
+class VesinDevice(ctypes.Structure):
+    _fields_ = [("type", ctypes.c_int), ("device_id", ctypes.c_int)]
+
+
+class VesinOptions(ctypes.Structure):
+    _fields_ = [
+        ("cutoff", ctypes.c_double),
+        ("full", ctypes.c_bool),
+        ("sorted", ctypes.c_bool),
+        ("algorithm", ctypes.c_int),
+        ("n_threads", ctypes.c_int32),
+        ("return_shifts", ctypes.c_bool),
+        ("return_distances", ctypes.c_bool),
+        ("return_vectors", ctypes.c_bool),
+        ("skin", ctypes.c_double),
+    ]
+
+
+class VesinNeighborList(ctypes.Structure):
+    _fields_ = [
+        ("length", ctypes.c_size_t),
+        ("device", VesinDevice),
+        ("pairs", ctypes.c_void_p),
+        ("shifts", ctypes.c_void_p),
+        ("distances", ctypes.c_void_p),
+        ("vectors", ctypes.c_void_p),
+        ("opaque", ctypes.c_void_p),
+    ]
+
+
+class VesinHipTimings(ctypes.Structure):
+    _fields_ = [
+        ("total", ctypes.c_float),
+        ("cell_build", ctypes.c_float),
+        ("count", ctypes.c_float),
+        ("scan", ctypes.c_float),
+        ("write", ctypes.c_float),
+        ("sort", ctypes.c_float),
+        ("candidates", ctypes.c_uint64),
+    ]
+
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.realpath(__file__)), "lib", "libvesin.so")
+
+_LIBRARY = None
+
+
+def get_library():
+    """Load libvesin.so. There is no fallback: without the compiled HIP library nothing can be computed."""
+    global _LIBRARY
+    if _LIBRARY is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it first with `python -m vesin_amd._build` "
+                "(hipcc, --offload-arch=gfx950)"
+            )
+        lib = ctypes.CDLL(LIB_PATH)
+        lib.vesin_neighbors.restype = ctypes.c_int
+        lib.vesin_neighbors.argtypes = [
+            ctypes.c_void_p,
+            ctypes.c_size_t,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            VesinDevice,
+            VesinOptions,
+            ctypes.POINTER(VesinNeighborList),
+            ctypes.POINTER(ctypes.c_char_p),
+        ]
+        lib.vesin_free.restype = None
+        lib.vesin_free.argtypes = [ctypes.POINTER(VesinNeighborList)]
+        lib.vesin_hip_enable_timings.restype = None
+        lib.vesin_hip_enable_timings.argtypes = [ctypes.c_int]
+        lib.vesin_hip_last_timings.restype = ctypes.c_int
+        lib.vesin_hip_last_timings.argtypes = [ctypes.POINTER(VesinNeighborList), ctypes.POINTER(VesinHipTimings)]
+        _LIBRARY = lib
+    return _LIBRARY

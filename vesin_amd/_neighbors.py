@@ -1,0 +1,257 @@
+"""``NeighborList``: the Python caller of the C ABI, with the interface of the reference's
+``vesin.NeighborList`` (python/vesin/vesin/_neighbors.py:69-381): same constructor arguments, same
+``compute(points, box, periodic, quantities, copy)`` contract, same dtypes and shapes of the results.
+
+The calculation always runs on a GPU through ``vesin_neighbors`` with ``device = {VesinCUDA, index}``:
+
+* torch tensors on a ``cuda`` device (what PyTorch-ROCm calls a HIP GPU) are used in place, and the results are
+  torch tensors on the same device (zero-copy views of the library's buffers when ``copy=False``);
+* numpy arrays (or anything numpy can convert) are uploaded to ``device`` (default ``cuda:0``) and the results come
+  back as numpy arrays.
+
+torch is only used to hold device memory; nothing is computed with it.
+"""
+
+import ctypes
+from typing import Sequence, Union
+
+import numpy as np
+
+from ._c_api import (
+    VesinAutoAlgorithm,
+    VesinBruteForce,
+    VesinCellList,
+    VesinCUDA,
+    VesinDevice,
+    VesinHipTimings,
+    VesinNeighborList,
+    VesinOptions,
+    VesinUnknownDevice,
+    get_library,
+)
+
+_ALGORITHMS = {
+    "auto": VesinAutoAlgorithm,
+    "brute_force": VesinBruteForce,
+    "cell_list": VesinCellList,
+}
+
+
+class _DeviceView:
+    """Expose a raw device pointer through ``__cuda_array_interface__`` so torch can wrap it without a copy."""
+
+    def __init__(self, pointer, shape, typestr, owner):
+        self._owner = owner
+        self.__cuda_array_interface__ = {
+            "shape": tuple(shape),
+            "typestr": typestr,
+            "data": (int(pointer), False),
+            "version": 2,
+            "strides": None,
+        }
+
+
+class NeighborList:
+    """A neighbor list calculator running on an AMD GPU."""
+
+    def __init__(
+        self,
+        cutoff: float,
+        full_list: bool,
+        sorted: bool = False,
+        algorithm: str = "auto",
+        skin: float = 0.0,
+        n_threads: int = 0,
+        device: str = "cuda:0",
+    ):
+        """
+        :param cutoff: spherical cutoff; pairs strictly closer than this are returned
+        :param full_list: return each pair twice (``i-j`` and ``j-i``) or only once
+        :param sorted: order the pairs by ``i`` (this implementation orders by ``(i, j, shift)``)
+        :param algorithm: ``"auto"``, ``"brute_force"`` or ``"cell_list"``
+        :param skin: Verlet skin; only ``0`` is supported
+        :param n_threads: accepted for compatibility (must be ``>= 0``); the GPU path does not use it
+        :param device: GPU used for inputs that are not already torch GPU tensors
+        """
+        self._lib = get_library()
+        self.cutoff = float(cutoff)
+        self.full_list = bool(full_list)
+        self.sorted = bool(sorted)
+        self.skin = float(skin)
+        self.algorithm = algorithm
+        self.n_threads = int(n_threads)
+        if self.n_threads < 0:
+            raise ValueError("n_threads must be zero or a positive integer")
+        self.device = device
+        self._neighbors = VesinNeighborList()
+
+    def __del__(self):
+        if hasattr(self, "_lib") and hasattr(self, "_neighbors"):
+            self._lib.vesin_free(ctypes.byref(self._neighbors))
+
+    @property
+    def algorithm(self) -> str:
+        return self._algorithm
+
+    @algorithm.setter
+    def algorithm(self, value: str):
+        algorithm = value.lower()
+        if algorithm not in _ALGORITHMS:
+            raise ValueError(
+                f"Unknown algorithm '{algorithm}'. Must be one of 'auto', 'brute_force', or 'cell_list'."
+            )
+        self._algorithm = algorithm
+        self._c_algorithm = _ALGORITHMS[algorithm]
+
+    def compute(
+        self,
+        points,
+        box,
+        periodic: Union[bool, Sequence[bool]],
+        quantities: str = "ij",
+        copy: bool = True,
+    ):
+        """Compute the neighbor list and return the requested ``quantities``, any of: ``i``, ``j``, ``P`` (both
+        indices), ``S`` (shifts), ``d`` (distances), ``D`` (vectors), as a tuple in the order asked for.
+
+        With ``copy=False`` the returned torch tensors alias the calculator's buffers and are invalidated by the
+        next ``compute`` or when the calculator is collected.
+        """
+        import torch
+
+        is_torch = isinstance(points, torch.Tensor)
+        if is_torch and points.device.type != "cuda":
+            raise RuntimeError(
+                "this implementation only computes on GPU tensors; move `points` to a cuda (HIP) device"
+            )
+        device = points.device if is_torch else torch.device(self.device)
+
+        if isinstance(periodic, (bool, np.bool_)):
+            periodic = [bool(periodic)] * 3
+
+        if is_torch:
+            box = torch.as_tensor(box)
+            initial_dtype = points.dtype
+            if box.dtype != initial_dtype:
+                raise RuntimeError(
+                    f"`points` and `box` must have the same dtype, got {points.dtype} and {box.dtype}"
+                )
+            if points.requires_grad or box.requires_grad:
+                raise RuntimeError("NeighborList.compute does not support autograd for torch tensors")
+            float_dtype = initial_dtype if initial_dtype.is_floating_point else torch.float64
+            to_result = lambda t: t  # noqa: E731
+        else:
+            points = np.asarray(points)
+            box = np.asarray(box)
+            initial_dtype = points.dtype
+            if box.dtype != initial_dtype:
+                raise RuntimeError(
+                    f"`points` and `box` must have the same dtype, got {points.dtype} and {box.dtype}"
+                )
+            np_float = initial_dtype if np.issubdtype(initial_dtype, np.floating) else np.float64
+            float_dtype = {np.dtype(np.float32): torch.float32, np.dtype(np.float64): torch.float64}.get(
+                np.dtype(np_float), torch.float64
+            )
+            points = torch.from_numpy(np.ascontiguousarray(points))
+            box = torch.from_numpy(np.ascontiguousarray(box))
+            to_result = lambda t: t.cpu().numpy()  # noqa: E731
+
+        if tuple(box.shape) != (3, 3):
+            raise ValueError("`box` must be a 3x3 matrix")
+        if points.dim() != 2 or points.shape[1] != 3:
+            raise ValueError("`points` must be a nx3 array")
+
+        periodic = torch.as_tensor(np.asarray(periodic).astype(np.bool_) if not isinstance(periodic, torch.Tensor) else periodic)
+        periodic = periodic.to(dtype=torch.bool, device=device).contiguous()
+        if tuple(periodic.shape) != (3,):
+            raise ValueError(
+                f"`periodic` must be a single boolean or a sequence of three booleans, got {periodic}"
+            )
+
+        points = points.to(device=device, dtype=torch.float64).contiguous()
+        box = box.to(device=device, dtype=torch.float64).contiguous()
+
+        options = VesinOptions()
+        options.cutoff = self.cutoff
+        options.full = self.full_list
+        options.sorted = self.sorted
+        options.algorithm = self._c_algorithm
+        options.n_threads = self.n_threads
+        options.return_shifts = "S" in quantities
+        options.return_distances = "d" in quantities
+        options.return_vectors = "D" in quantities
+        options.skin = self.skin
+
+        index = device.index if device.index is not None else torch.cuda.current_device()
+        c_device = VesinDevice(VesinCUDA, index)
+
+        if self._neighbors.device.type != VesinUnknownDevice and (
+            self._neighbors.device.type != c_device.type or self._neighbors.device.device_id != c_device.device_id
+        ):
+            # the list lives on another GPU: release it and start from a zeroed struct
+            self._lib.vesin_free(ctypes.byref(self._neighbors))
+            ctypes.memset(ctypes.byref(self._neighbors), 0, ctypes.sizeof(self._neighbors))
+
+        # inputs may still be in flight on torch's current stream
+        torch.cuda.current_stream(device).synchronize()
+
+        error_message = ctypes.c_char_p()
+        status = self._lib.vesin_neighbors(
+            points.data_ptr(),
+            points.shape[0],
+            box.data_ptr(),
+            periodic.data_ptr(),
+            c_device,
+            options,
+            ctypes.byref(self._neighbors),
+            ctypes.byref(error_message),
+        )
+        if status != 0:
+            raise RuntimeError(error_message.value.decode("utf8"))
+
+        n_pairs = self._neighbors.length
+        device_str = f"cuda:{index}"
+
+        def wrap(pointer, shape, typestr, dtype):
+            if n_pairs == 0:
+                return torch.empty(shape, dtype=dtype, device=device_str)
+            view = torch.as_tensor(_DeviceView(pointer, shape, typestr, self), device=device_str)
+            return view.clone() if copy else view
+
+        pairs = shifts = distances = vectors = None
+        if any(q in quantities for q in "ijP"):
+            pairs = wrap(self._neighbors.pairs, (n_pairs, 2), "<u8", torch.uint64)
+        if "S" in quantities:
+            shifts = wrap(self._neighbors.shifts, (n_pairs, 3), "<i4", torch.int32)
+        if "d" in quantities:
+            distances = wrap(self._neighbors.distances, (n_pairs,), "<f8", torch.float64).to(float_dtype)
+        if "D" in quantities:
+            vectors = wrap(self._neighbors.vectors, (n_pairs, 3), "<f8", torch.float64).to(float_dtype)
+
+        data = []
+        for quantity in quantities:
+            if quantity == "P":
+                data.append(to_result(pairs))
+            elif quantity == "i":
+                data.append(to_result(pairs[:, 0]))
+            elif quantity == "j":
+                data.append(to_result(pairs[:, 1]))
+            elif quantity == "S":
+                data.append(to_result(shifts))
+            elif quantity == "d":
+                data.append(to_result(distances))
+            elif quantity == "D":
+                data.append(to_result(vectors))
+        return tuple(data)
+
+    def timings(self):
+        """Per-stage GPU times (ms) of the last ``compute``; needs ``enable_timings(True)`` beforehand."""
+        timings = VesinHipTimings()
+        if self._lib.vesin_hip_last_timings(ctypes.byref(self._neighbors), ctypes.byref(timings)) != 0:
+            return None
+        return {name: getattr(timings, name) for name, _ in VesinHipTimings._fields_ if name != "candidates"}
+
+
+def enable_timings(enabled: bool = True):
+    """Make every later call record HIP events between its stages."""
+    get_library().vesin_hip_enable_timings(1 if enabled else 0)

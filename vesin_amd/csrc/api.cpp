@@ -1,0 +1,132 @@
+// The C ABI: argument validation, error-string ownership and dispatch to the HIP driver.
+//
+// Checks, their order and their texts are those of the reference's entry point (vesin/src/vesin.cpp:51-105), and
+// exceptions are turned into EXIT_FAILURE + message the same way (vesin/src/vesin.cpp:139-150). The difference is
+// the dispatch: a GPU device runs the HIP path, and VesinCPU is refused because this library ships no CPU engine.
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+
+#include <iostream>
+#include <stdexcept>
+#include <string>
+
+#include "driver.hpp"
+#include "vesin.h"
+
+// storage for messages built at run time; the caller only ever sees a pointer into it
+static thread_local std::string LAST_ERROR;
+
+static int fail(const char** error_message, const char* text) {
+    *error_message = text;
+    return EXIT_FAILURE;
+}
+
+extern "C" int vesin_neighbors(
+    const double (*points)[3],
+    size_t n_points,
+    const double box[3][3],
+    const bool periodic[3],
+    VesinDevice device,
+    VesinOptions options,
+    VesinNeighborList* neighbors,
+    const char** error_message
+) {
+    if (error_message == nullptr) {
+        return EXIT_FAILURE;
+    }
+    if (points == nullptr) {
+        return fail(error_message, "`points` can not be a NULL pointer");
+    }
+    if (box == nullptr) {
+        return fail(error_message, "`cell` can not be a NULL pointer");
+    }
+    if (neighbors == nullptr) {
+        return fail(error_message, "`neighbors` can not be a NULL pointer");
+    }
+    if (!std::isfinite(options.cutoff) || options.cutoff <= 0) {
+        return fail(error_message, "cutoff must be a finite, positive number");
+    }
+    if (options.cutoff <= 1e-6) {
+        return fail(error_message, "cutoff is too small");
+    }
+    if (!std::isfinite(options.skin) || options.skin < 0.0) {
+        // the reference sets this message without returning (vesin/src/vesin.cpp:80-82); a caching skin is not
+        // available here at all, so this is an error
+        return fail(error_message, "skin must be a finite, non-negative number");
+    }
+    if (options.n_threads < 0) {
+        return fail(error_message, "n_threads must be zero or a positive integer");
+    }
+    if (neighbors->device.type != VesinUnknownDevice && neighbors->device.type != device.type) {
+        return fail(error_message, "`neighbors` device and data `device` do not match, free the neighbors first");
+    }
+    if (device.type == VesinUnknownDevice) {
+        return fail(error_message, "got an unknown device type");
+    }
+
+    try {
+        if (device.type == VesinCUDA) {
+            if (options.skin > 0.0) {
+                throw std::runtime_error("a non-zero `skin` (Verlet caching) is not supported by the HIP path");
+            }
+            if (periodic == nullptr) {
+                throw std::runtime_error("`periodic` can not be a NULL pointer");
+            }
+            if (neighbors->device.type == VesinUnknownDevice) {
+                neighbors->device = device;
+            }
+            vesin_hip::neighbors(points, n_points, box, periodic, options, *neighbors);
+        } else if (device.type == VesinCPU) {
+            throw std::runtime_error(
+                "this library only implements GPU devices (VesinCUDA, i.e. HIP on ROCm); there is no CPU engine in it"
+            );
+        } else {
+            throw std::runtime_error("unknown device " + std::to_string(device.type));
+        }
+    } catch (const std::bad_alloc&) {
+        LAST_ERROR = "failed to allocate memory";
+        *error_message = LAST_ERROR.c_str();
+        return EXIT_FAILURE;
+    } catch (const std::exception& e) {
+        LAST_ERROR = e.what();
+        *error_message = LAST_ERROR.c_str();
+        return EXIT_FAILURE;
+    } catch (...) {
+        return fail(error_message, "fatal error: unknown type thrown as exception");
+    }
+    return EXIT_SUCCESS;
+}
+
+extern "C" void vesin_free(VesinNeighborList* neighbors) {
+    if (neighbors == nullptr) {
+        return;
+    }
+    try {
+        if (neighbors->device.type == VesinCUDA) {
+            vesin_hip::free_neighbors(*neighbors);
+        } else if (neighbors->device.type != VesinUnknownDevice) {
+            throw std::runtime_error(
+                "device " + std::to_string(neighbors->device.type) + " is not one this library allocates on"
+            );
+        }
+    } catch (const std::exception& e) {
+        std::cerr << "error in vesin_free: " << e.what() << std::endl;
+        return;
+    } catch (...) {
+        std::cerr << "fatal error in vesin_free, unknown type thrown as exception" << std::endl;
+        return;
+    }
+    std::memset(static_cast<void*>(neighbors), 0, sizeof(VesinNeighborList));
+}
+
+extern "C" void vesin_hip_enable_timings(int enabled) {
+    vesin_hip::enable_timings(enabled != 0);
+}
+
+extern "C" int vesin_hip_last_timings(const VesinNeighborList* neighbors, VesinHipTimings* timings) {
+    if (neighbors == nullptr || timings == nullptr || neighbors->device.type != VesinCUDA) {
+        return EXIT_FAILURE;
+    }
+    return vesin_hip::last_timings(*neighbors, *timings) ? EXIT_SUCCESS : EXIT_FAILURE;
+}

@@ -1,0 +1,291 @@
+// Cell-list construction on the GPU: projected bounding box, cell assignment in fractional coordinates,
+// counting sort of the points by cell (histogram -> device-wide scan -> scatter), and the per-cell pass that
+// puts every cell in a canonical order and lays the points out as structure-of-arrays for the search kernel.
+//
+// Reference roles replaced: compute_bounding_box (vesin/src/cuda/cell_list.cu:69-133), assign_cell_indices
+// (:279-333), count_particles_per_cell (:335-345), prefix_sum_cells (:347-390), scatter_particles (:392-421);
+// CPU twin CellList::add_point (vesin/src/cpu_cell_list.cpp:353-374).
+#ifndef VESIN_HIP_CELLS_CUH
+#define VESIN_HIP_CELLS_CUH
+
+#include "device_common.cuh"
+
+namespace vesin_hip {
+
+/// Cell-sorted copy of the points, one array per component so that 64 consecutive candidates load coalesced.
+struct SortedPoints {
+    double* x;
+    double* y;
+    double* z;
+    uint32_t* index; // original point index
+    int32_t* wx;     // number of box vectors the point was moved by to land inside the box
+    int32_t* wy;
+    int32_t* wz;
+};
+
+__global__ void init_status(DeviceStatus* status) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        status->total_pairs = 0;
+        status->first_bad_coordinate = 0xFFFFFFFFu;
+        status->n_tiles = 0;
+        for (int d = 0; d < 3; d++) {
+            status->frac_min[d] = ~0ull;
+            status->frac_max[d] = 0ull;
+        }
+    }
+}
+
+__device__ __forceinline__ void fractional(const GridParams& g, double x, double y, double z, double f[3]) {
+#pragma unroll
+    for (int d = 0; d < 3; d++) {
+        f[d] = x * g.Hinv[d] + y * g.Hinv[3 + d] + z * g.Hinv[6 + d];
+    }
+}
+
+__device__ __forceinline__ bool all_finite(double x, double y, double z, unsigned int& bad_axis) {
+    if (!isfinite(x)) {
+        bad_axis = 0;
+        return false;
+    }
+    if (!isfinite(y)) {
+        bad_axis = 1;
+        return false;
+    }
+    if (!isfinite(z)) {
+        bad_axis = 2;
+        return false;
+    }
+    return true;
+}
+
+/// Smallest and largest fractional coordinate over all points (needed for non-periodic directions), plus the
+/// check for non-finite input. Grid-stride loop, wave reduction, then one atomic per wave and direction.
+__global__ __launch_bounds__(BLOCK) void bounding_kernel(
+    const double* __restrict__ points, uint32_t n_points, GridParams g, DeviceStatus* status
+) {
+    double lo[3] = {INFINITY, INFINITY, INFINITY};
+    double hi[3] = {-INFINITY, -INFINITY, -INFINITY};
+    unsigned int bad = 0xFFFFFFFFu;
+
+    for (uint32_t i = blockIdx.x * BLOCK + threadIdx.x; i < n_points; i += gridDim.x * BLOCK) {
+        double x = points[3 * static_cast<size_t>(i) + 0];
+        double y = points[3 * static_cast<size_t>(i) + 1];
+        double z = points[3 * static_cast<size_t>(i) + 2];
+        unsigned int axis;
+        if (!all_finite(x, y, z, axis)) {
+            bad = min(bad, 3u * i + axis);
+            continue;
+        }
+        double f[3];
+        fractional(g, x, y, z, f);
+#pragma unroll
+        for (int d = 0; d < 3; d++) {
+            lo[d] = fmin(lo[d], f[d]);
+            hi[d] = fmax(hi[d], f[d]);
+        }
+    }
+
+#pragma unroll
+    for (int offset = WAVE / 2; offset > 0; offset >>= 1) {
+#pragma unroll
+        for (int d = 0; d < 3; d++) {
+            lo[d] = fmin(lo[d], __shfl_xor(lo[d], offset));
+            hi[d] = fmax(hi[d], __shfl_xor(hi[d], offset));
+        }
+        bad = min(bad, static_cast<unsigned int>(__shfl_xor(static_cast<int>(bad), offset)));
+    }
+
+    if (lane_id() == 0) {
+#pragma unroll
+        for (int d = 0; d < 3; d++) {
+            if (lo[d] <= hi[d]) {
+                atomicMin(&status->frac_min[d], ordered_bits(lo[d]));
+                atomicMax(&status->frac_max[d], ordered_bits(hi[d]));
+            }
+        }
+        if (bad != 0xFFFFFFFFu) {
+            atomicMin(&status->first_bad_coordinate, bad);
+        }
+    }
+}
+
+/// Cell coordinates and wrap shift of one point. Periodic directions: cell = floor(frac * n) brought back into
+/// [0, n) with the quotient kept as the wrap shift. Non-periodic directions: clamped, never wrapped.
+__device__ __forceinline__ void locate(
+    const GridParams& g, double x, double y, double z, int32_t cell[3], int32_t wrap[3]
+) {
+    double f[3];
+    fractional(g, x, y, z, f);
+#pragma unroll
+    for (int d = 0; d < 3; d++) {
+        const int32_t n = g.n[d];
+        if (g.periodic[d]) {
+            double scaled = floor(f[d] * static_cast<double>(n));
+            scaled = fmin(fmax(scaled, -2.0e9), 2.0e9);
+            int32_t c = static_cast<int32_t>(scaled);
+            int32_t q = c / n;
+            int32_t r = c - q * n;
+            if (r < 0) {
+                r += n;
+                q -= 1;
+            }
+            cell[d] = r;
+            wrap[d] = q;
+        } else {
+            double scaled = floor((f[d] - g.np_min[d]) * g.np_scale[d] * static_cast<double>(n));
+            scaled = fmin(fmax(scaled, 0.0), static_cast<double>(n - 1));
+            cell[d] = static_cast<int32_t>(scaled);
+            wrap[d] = 0;
+        }
+    }
+}
+
+/// One thread per point: cell id, wrap shift, and the histogram of points per cell. The value returned by the
+/// histogram atomic is kept as the point's provisional slot inside its cell.
+__global__ __launch_bounds__(BLOCK) void assign_cells(
+    const double* __restrict__ points, GridParams g,
+    uint32_t* __restrict__ cell_of, uint32_t* __restrict__ slot_of, int32_t* __restrict__ wrap_of,
+    uint32_t* __restrict__ cell_counts, DeviceStatus* status
+) {
+    uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
+    if (i >= g.n_points) {
+        return;
+    }
+    double x = points[3 * static_cast<size_t>(i) + 0];
+    double y = points[3 * static_cast<size_t>(i) + 1];
+    double z = points[3 * static_cast<size_t>(i) + 2];
+
+    int32_t cell[3] = {0, 0, 0};
+    int32_t wrap[3] = {0, 0, 0};
+    unsigned int axis;
+    if (all_finite(x, y, z, axis)) {
+        locate(g, x, y, z, cell, wrap);
+    } else {
+        atomicMin(&status->first_bad_coordinate, 3u * i + axis);
+    }
+
+    uint32_t linear = (static_cast<uint32_t>(cell[2]) * g.n[1] + cell[1]) * g.n[0] + cell[0];
+    cell_of[i] = linear;
+    slot_of[i] = atomicAdd(&cell_counts[linear], 1u);
+    wrap_of[3 * static_cast<size_t>(i) + 0] = wrap[0];
+    wrap_of[3 * static_cast<size_t>(i) + 1] = wrap[1];
+    wrap_of[3 * static_cast<size_t>(i) + 2] = wrap[2];
+}
+
+/// Counting-sort scatter: the point goes to (start of its cell) + (its provisional slot).
+__global__ __launch_bounds__(BLOCK) void scatter_points(
+    uint32_t n_points, const uint32_t* __restrict__ cell_of, const uint32_t* __restrict__ slot_of,
+    const uint64_t* __restrict__ cell_scan, uint32_t* __restrict__ provisional
+) {
+    uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
+    if (i >= n_points) {
+        return;
+    }
+    uint32_t start = static_cast<uint32_t>(cell_scan[cell_of[i]]);
+    provisional[start + slot_of[i]] = i;
+}
+
+constexpr uint32_t CANONICAL_LIMIT = 4096;
+
+/// One wave per cell. The atomics of assign_cells leave the points of a cell in arbitrary order; here they are
+/// ranked by original index (so the whole pipeline is deterministic), gathered into the structure-of-arrays
+/// layout, and the cell's 64-point tiles are appended to the tile list.
+__global__ __launch_bounds__(BLOCK) void gather_cells(
+    const double* __restrict__ points, const int32_t* __restrict__ wrap_of,
+    const uint32_t* __restrict__ provisional, const uint64_t* __restrict__ cell_scan, uint32_t n_cells,
+    SortedPoints sorted, Tile* __restrict__ tiles
+) {
+    const int lane = lane_id();
+    const uint32_t cell = blockIdx.x * WAVES_PER_BLOCK + threadIdx.x / WAVE;
+    if (cell >= n_cells) {
+        return;
+    }
+    const uint64_t here = cell_scan[cell];
+    const uint64_t next = cell_scan[cell + 1];
+    const uint32_t start = static_cast<uint32_t>(here);
+    const uint32_t count = static_cast<uint32_t>(next) - start;
+    const uint32_t first_tile = static_cast<uint32_t>(here >> 32);
+    if (count == 0) {
+        return;
+    }
+
+    for (uint32_t t = lane; t * 64u < count; t += WAVE) {
+        Tile tile;
+        tile.cell = cell;
+        tile.first = start + t * 64u;
+        tile.count = min(64u, count - t * 64u);
+        tile.pad = 0;
+        tiles[first_tile + t] = tile;
+    }
+
+    for (uint32_t base = 0; base < count; base += WAVE) {
+        uint32_t k = base + lane;
+        bool active = k < count;
+        uint32_t mine = active ? provisional[start + k] : 0xFFFFFFFFu;
+        uint32_t rank = k;
+        if (count <= CANONICAL_LIMIT) {
+            rank = 0;
+            for (uint32_t other = 0; other < count; other++) {
+                // same address in every lane: served as one broadcast load
+                rank += provisional[start + other] < mine ? 1u : 0u;
+            }
+        }
+        if (active) {
+            uint32_t to = start + rank;
+            sorted.index[to] = mine;
+            sorted.x[to] = points[3 * static_cast<size_t>(mine) + 0];
+            sorted.y[to] = points[3 * static_cast<size_t>(mine) + 1];
+            sorted.z[to] = points[3 * static_cast<size_t>(mine) + 2];
+            sorted.wx[to] = wrap_of[3 * static_cast<size_t>(mine) + 0];
+            sorted.wy[to] = wrap_of[3 * static_cast<size_t>(mine) + 1];
+            sorted.wz[to] = wrap_of[3 * static_cast<size_t>(mine) + 2];
+        }
+    }
+}
+
+/// The single-cell layout used by the brute-force / multi-image path: points keep their order, the one cell
+/// holds all of them, tiles are consecutive blocks of 64 points. Also performs the non-finite check.
+__global__ __launch_bounds__(BLOCK) void prepare_single_cell(
+    const double* __restrict__ points, GridParams g, SortedPoints sorted, Tile* __restrict__ tiles,
+    uint64_t* __restrict__ cell_scan, DeviceStatus* status
+) {
+    uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
+    const uint32_t n_tiles = (g.n_points + 63u) / 64u;
+    if (i == 0) {
+        cell_scan[0] = 0;
+        cell_scan[1] = static_cast<uint64_t>(g.n_points) | (static_cast<uint64_t>(n_tiles) << 32);
+    }
+    if (i < n_tiles) {
+        Tile tile;
+        tile.cell = 0;
+        tile.first = i * 64u;
+        tile.count = min(64u, g.n_points - i * 64u);
+        tile.pad = 0;
+        tiles[i] = tile;
+    }
+    if (i >= g.n_points) {
+        return;
+    }
+    double x = points[3 * static_cast<size_t>(i) + 0];
+    double y = points[3 * static_cast<size_t>(i) + 1];
+    double z = points[3 * static_cast<size_t>(i) + 2];
+    int32_t cell[3] = {0, 0, 0};
+    int32_t wrap[3] = {0, 0, 0};
+    unsigned int axis;
+    if (all_finite(x, y, z, axis)) {
+        locate(g, x, y, z, cell, wrap);
+    } else {
+        atomicMin(&status->first_bad_coordinate, 3u * i + axis);
+    }
+    sorted.index[i] = i;
+    sorted.x[i] = x;
+    sorted.y[i] = y;
+    sorted.z[i] = z;
+    sorted.wx[i] = wrap[0];
+    sorted.wy[i] = wrap[1];
+    sorted.wz[i] = wrap[2];
+}
+
+} // namespace vesin_hip
+
+#endif

@@ -1,0 +1,117 @@
+// Wave64 building blocks shared by the gfx950 kernels: lane ids, DPP scans, ballot compaction helpers.
+#ifndef VESIN_HIP_DEVICE_COMMON_CUH
+#define VESIN_HIP_DEVICE_COMMON_CUH
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace vesin_hip {
+
+constexpr int WAVE = 64;
+constexpr int BLOCK = 256;
+constexpr int WAVES_PER_BLOCK = BLOCK / WAVE;
+
+/// Everything a kernel needs to know about the box and the cell grid.
+struct GridParams {
+    double H[9];          // normalised box, row-major
+    double Hinv[9];       // inverse, row-major: frac[d] = sum_k r[k] * Hinv[3k + d]
+    double np_min[3];     // non-periodic directions: offset of the projected coordinate
+    double np_scale[3];   // non-periodic directions: 1 / extent
+    double cutoff2;
+    int32_t n[3];         // cells per direction
+    int32_t s[3];         // stencil radius per direction
+    int32_t periodic[3];
+    uint32_t n_points;
+    uint32_t n_cells;
+};
+
+/// One row of 64 i-points (or fewer) that one workgroup searches for.
+struct Tile {
+    uint32_t cell;   // linear cell index of these points
+    uint32_t first;  // position of the first point in the cell-sorted arrays
+    uint32_t count;  // 1..64
+    uint32_t pad;
+};
+
+/// Small block of results the host reads back after the counting pass.
+struct DeviceStatus {
+    unsigned long long total_pairs;
+    unsigned int first_bad_coordinate; // 3 * point + axis of the first non-finite coordinate, or 0xFFFFFFFF
+    unsigned int n_tiles;
+    unsigned long long frac_min[3];    // order-preserving encoding of the smallest / largest projected coordinate
+    unsigned long long frac_max[3];
+};
+
+__device__ __forceinline__ int lane_id() {
+    return static_cast<int>(__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)));
+}
+
+/// Number of set bits of `mask` below this lane: the slot of this lane after compaction.
+__device__ __forceinline__ uint32_t rank_in_mask(uint64_t mask) {
+    return __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(mask >> 32),
+                                     __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0u));
+}
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_or_zero(uint32_t v) {
+    // lanes without a valid source (or in rows that are masked off) receive 0
+    return static_cast<uint32_t>(
+        __builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, ROW_MASK, 0xf, false)
+    );
+}
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint64_t dpp_or_zero64(uint64_t v) {
+    uint32_t lo = dpp_or_zero<CTRL, ROW_MASK>(static_cast<uint32_t>(v));
+    uint32_t hi = dpp_or_zero<CTRL, ROW_MASK>(static_cast<uint32_t>(v >> 32));
+    return (static_cast<uint64_t>(hi) << 32) | lo;
+}
+
+/// Inclusive prefix sum over the 64 lanes of a wave, data moved with DPP only (row shifts inside each row of 16
+/// lanes, then row_bcast:15 and row_bcast:31 to carry row totals forward).
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
+    v += dpp_or_zero<0x111, 0xf>(v); // row_shr:1
+    v += dpp_or_zero<0x112, 0xf>(v); // row_shr:2
+    v += dpp_or_zero<0x114, 0xf>(v); // row_shr:4
+    v += dpp_or_zero<0x118, 0xf>(v); // row_shr:8
+    v += dpp_or_zero<0x142, 0xa>(v); // row_bcast:15 into rows 1 and 3
+    v += dpp_or_zero<0x143, 0xc>(v); // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
+__device__ __forceinline__ uint64_t wave_inclusive_scan(uint64_t v) {
+    v += dpp_or_zero64<0x111, 0xf>(v);
+    v += dpp_or_zero64<0x112, 0xf>(v);
+    v += dpp_or_zero64<0x114, 0xf>(v);
+    v += dpp_or_zero64<0x118, 0xf>(v);
+    v += dpp_or_zero64<0x142, 0xa>(v);
+    v += dpp_or_zero64<0x143, 0xc>(v);
+    return v;
+}
+
+__device__ __forceinline__ uint32_t read_lane(uint32_t v, int lane) {
+    return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), lane));
+}
+
+__device__ __forceinline__ uint64_t read_lane(uint64_t v, int lane) {
+    uint32_t lo = read_lane(static_cast<uint32_t>(v), lane);
+    uint32_t hi = read_lane(static_cast<uint32_t>(v >> 32), lane);
+    return (static_cast<uint64_t>(hi) << 32) | lo;
+}
+
+/// Doubles mapped to unsigned integers with the same ordering, for atomicMin / atomicMax.
+__device__ __forceinline__ unsigned long long ordered_bits(double x) {
+    unsigned long long bits = static_cast<unsigned long long>(__double_as_longlong(x));
+    return (bits & 0x8000000000000000ull) ? ~bits : (bits | 0x8000000000000000ull);
+}
+
+inline double ordered_bits_to_double(unsigned long long key) {
+    unsigned long long bits = (key & 0x8000000000000000ull) ? (key & 0x7FFFFFFFFFFFFFFFull) : ~key;
+    double x;
+    __builtin_memcpy(&x, &bits, sizeof(double));
+    return x;
+}
+
+} // namespace vesin_hip
+
+#endif

@@ -1,0 +1,591 @@
+// Host driver of the HIP neighbor-list path: owns the device work buffers kept in VesinNeighborList::opaque,
+// picks the grid, launches the kernel sequence on the null stream and sizes the outputs exactly (count pass ->
+// device-wide scan -> write pass), so no capacity guess and no overflow flag are needed.
+//
+// Reference role replaced: vesin::cuda::neighbors / allocate_output_buffers / finalize_output / free_neighbors
+// (vesin/src/vesin_cuda.cpp:819-923, :293-345, :783-817, :129-138) and the RAII buffers of
+// vesin/src/cuda_buffers.cpp.
+#include <hip/hip_runtime.h>
+
+#include <cerrno>
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+
+#include <atomic>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "cells.cuh"
+#include "device_common.cuh"
+#include "driver.hpp"
+#include "geometry.hpp"
+#include "scan.cuh"
+#include "search.cuh"
+#include "sort.cuh"
+
+namespace vesin_hip {
+
+#define HIP_CHECK(expr)                                                                                              \
+    do {                                                                                                             \
+        hipError_t status_ = (expr);                                                                                 \
+        if (status_ != hipSuccess) {                                                                                 \
+            throw std::runtime_error(std::string("HIP error in ") + #expr + ": " + hipGetErrorString(status_));      \
+        }                                                                                                            \
+    } while (false)
+
+static std::atomic<bool> TIMINGS_ENABLED{false};
+
+void enable_timings(bool enabled) {
+    TIMINGS_ENABLED.store(enabled);
+}
+
+namespace {
+
+/// Grow-only device allocation.
+struct DeviceBuffer {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+
+    void reserve(size_t wanted) {
+        if (wanted <= bytes) {
+            return;
+        }
+        release();
+        size_t padded = wanted + wanted / 4;
+        HIP_CHECK(hipMalloc(&ptr, padded));
+        bytes = padded;
+    }
+
+    void release() {
+        if (ptr != nullptr) {
+            (void)hipFree(ptr);
+            ptr = nullptr;
+            bytes = 0;
+        }
+    }
+};
+
+/// Hands out 256-byte aligned pieces of one allocation; first pass (base == nullptr) only measures.
+struct Carver {
+    char* base;
+    size_t used = 0;
+
+    explicit Carver(void* start): base(static_cast<char*>(start)) {}
+
+    template <typename T>
+    T* take(size_t count) {
+        size_t at = used;
+        used += (count * sizeof(T) + 255) & ~static_cast<size_t>(255);
+        return base == nullptr ? nullptr : reinterpret_cast<T*>(base + at);
+    }
+};
+
+enum Stage { T_START = 0, T_CELLS, T_COUNT, T_SCAN, T_WRITE_BEGIN, T_WRITE, T_SORT, T_STAGES };
+
+/// Private state of one VesinNeighborList (VesinNeighborList::opaque).
+struct HipExtras {
+    int device_id = 0;
+    DeviceBuffer work;
+    DeviceBuffer sort_work;
+    DeviceStatus* d_status = nullptr;
+    DeviceStatus* h_status = nullptr; // pinned
+    unsigned char* h_small = nullptr; // pinned: box (72 bytes) + periodic (3 bytes)
+    size_t capacity = 0;              // rows every allocated output array can hold
+    hipEvent_t events[T_STAGES] = {};
+    bool have_events = false;
+    bool timings_valid = false;
+    VesinHipTimings timings = {};
+
+    ~HipExtras() {
+        work.release();
+        sort_work.release();
+        if (d_status != nullptr) {
+            (void)hipFree(d_status);
+        }
+        if (h_status != nullptr) {
+            (void)hipHostFree(h_status);
+        }
+        if (h_small != nullptr) {
+            (void)hipHostFree(h_small);
+        }
+        if (have_events) {
+            for (auto& event : events) {
+                (void)hipEventDestroy(event);
+            }
+        }
+    }
+};
+
+HipExtras& extras_of(VesinNeighborList& neighbors) {
+    if (neighbors.opaque == nullptr) {
+        auto* extras = new HipExtras();
+        extras->device_id = neighbors.device.device_id;
+        neighbors.opaque = extras;
+        HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&extras->d_status), sizeof(DeviceStatus)));
+        HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&extras->h_status), sizeof(DeviceStatus), hipHostMallocDefault));
+        HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&extras->h_small), 128, hipHostMallocDefault));
+    }
+    return *static_cast<HipExtras*>(neighbors.opaque);
+}
+
+/// Device ordinal owning `ptr`, or -1 when it is not device memory.
+int device_of(const void* ptr) {
+    hipPointerAttribute_t attributes;
+    hipError_t status = hipPointerGetAttributes(&attributes, ptr);
+    if (status != hipSuccess) {
+        (void)hipGetLastError(); // clear the sticky error left by an unknown (host) pointer
+        return -1;
+    }
+    if (attributes.type != hipMemoryTypeDevice) {
+        return -1;
+    }
+    return attributes.device;
+}
+
+void free_outputs(VesinNeighborList& neighbors) {
+    if (neighbors.pairs != nullptr) {
+        (void)hipFree(neighbors.pairs);
+    }
+    if (neighbors.shifts != nullptr) {
+        (void)hipFree(neighbors.shifts);
+    }
+    if (neighbors.distances != nullptr) {
+        (void)hipFree(neighbors.distances);
+    }
+    if (neighbors.vectors != nullptr) {
+        (void)hipFree(neighbors.vectors);
+    }
+    neighbors.pairs = nullptr;
+    neighbors.shifts = nullptr;
+    neighbors.distances = nullptr;
+    neighbors.vectors = nullptr;
+}
+
+/// Make every requested output array hold `rows` rows and drop the ones that were not requested (like the CPU
+/// engine of the reference does, vesin/src/cpu_cell_list.cpp:605-627).
+void size_outputs(VesinNeighborList& neighbors, HipExtras& extras, size_t rows, const VesinOptions& options) {
+    if (rows > extras.capacity) {
+        free_outputs(neighbors);
+        size_t capacity = rows + rows / 8;
+        if (capacity < 1024) {
+            capacity = 1024;
+        }
+        extras.capacity = capacity;
+    }
+    if (extras.capacity == 0) {
+        extras.capacity = 1024;
+    }
+    const size_t capacity = extras.capacity;
+
+    auto drop = [](auto*& pointer) {
+        if (pointer != nullptr) {
+            (void)hipFree(pointer);
+            pointer = nullptr;
+        }
+    };
+    auto ensure = [&](auto*& pointer, size_t bytes) {
+        if (pointer == nullptr && hipMalloc(reinterpret_cast<void**>(&pointer), bytes) != hipSuccess) {
+            (void)hipGetLastError();
+            pointer = nullptr;
+            free_outputs(neighbors);
+            extras.capacity = 0;
+            throw std::bad_alloc();
+        }
+    };
+
+    ensure(neighbors.pairs, capacity * 2 * sizeof(size_t));
+    if (options.return_shifts) {
+        ensure(neighbors.shifts, capacity * 3 * sizeof(int32_t));
+    } else {
+        drop(neighbors.shifts);
+    }
+    if (options.return_distances) {
+        ensure(neighbors.distances, capacity * sizeof(double));
+    } else {
+        drop(neighbors.distances);
+    }
+    if (options.return_vectors) {
+        ensure(neighbors.vectors, capacity * 3 * sizeof(double));
+    } else {
+        drop(neighbors.vectors);
+    }
+}
+
+/// Optional user-imposed limit on pairs per point, kept for callers that rely on the reference's environment
+/// variable and its messages (vesin/src/vesin_cuda.cpp:871-884, :911-918). 0 = no limit.
+size_t pairs_per_point_limit() {
+    const char* text = std::getenv("VESIN_CUDA_MAX_PAIRS_PER_POINT");
+    if (text == nullptr) {
+        return 0;
+    }
+    size_t length = std::strlen(text);
+    char* end = nullptr;
+    errno = 0;
+    long long parsed = std::strtoll(text, &end, 10);
+    if (errno != 0 || end != text + length || parsed <= 0) {
+        throw std::runtime_error("Invalid value for VESIN_CUDA_MAX_PAIRS_PER_POINT: '" + std::string(text) + "'");
+    }
+    return static_cast<size_t>(parsed);
+}
+
+template <bool WRITE>
+void launch_search(bool full, uint32_t blocks, const SearchArgs& args, const GridParams& g, hipStream_t stream) {
+    if (blocks == 0) {
+        return;
+    }
+    constexpr int R = 2;
+    if (full) {
+        hipLaunchKernelGGL((search_kernel<WRITE, true, R>), dim3(blocks), dim3(BLOCK), 0, stream, args, g);
+    } else {
+        hipLaunchKernelGGL((search_kernel<WRITE, false, R>), dim3(blocks), dim3(BLOCK), 0, stream, args, g);
+    }
+}
+
+void non_finite_error(const double (*points)[3], unsigned int flat) {
+    size_t point = flat / 3;
+    int axis = static_cast<int>(flat % 3);
+    double value = 0.0;
+    HIP_CHECK(hipMemcpy(&value, &points[point][axis], sizeof(double), hipMemcpyDeviceToHost));
+    // same text as the CPU engine of the reference (vesin/src/types.hpp:163-169)
+    throw std::runtime_error(
+        "point " + std::to_string(point) + " has non-finite coordinate along axis " + std::to_string(axis) + ": " +
+        std::to_string(value)
+    );
+}
+
+} // namespace
+
+void neighbors(
+    const double (*points)[3],
+    size_t n_points,
+    const double box[3][3],
+    const bool periodic[3],
+    VesinOptions options,
+    VesinNeighborList& neighbors
+) {
+    const int device_id = neighbors.device.device_id;
+    int device_count = 0;
+    if (hipGetDeviceCount(&device_count) != hipSuccess || device_count == 0) {
+        (void)hipGetLastError();
+        throw std::runtime_error("no HIP device is available to this process");
+    }
+    if (device_id < 0 || device_id >= device_count) {
+        throw std::runtime_error("invalid GPU device_id " + std::to_string(device_id));
+    }
+
+    // same requirements and texts as the reference (vesin/src/vesin_cuda.cpp:831-854)
+    const int points_device = device_of(points);
+    if (points_device < 0) {
+        throw std::runtime_error("`points` pointer is not allocated on a CUDA device");
+    }
+    const int box_device = device_of(box);
+    if (box_device < 0) {
+        throw std::runtime_error("`box` pointer is not allocated on a CUDA device");
+    }
+    const int periodic_device = device_of(periodic);
+    if (periodic_device < 0) {
+        throw std::runtime_error("`periodic` pointer is not allocated on a CUDA device");
+    }
+    if (points_device != box_device) {
+        throw std::runtime_error("`points` and `box` do not exist on the same device");
+    }
+    if (points_device != periodic_device) {
+        throw std::runtime_error("`points` and `periodic` do not exist on the same device");
+    }
+    if (points_device != device_id) {
+        throw std::runtime_error("`points`, `box` and `periodic` device differs from input neighbors device_id");
+    }
+    if (n_points >= 0xFFFFFFF0ull) {
+        throw std::runtime_error("too many points: the GPU path indexes points with 32 bits");
+    }
+
+    HIP_CHECK(hipSetDevice(device_id));
+    HipExtras& extras = extras_of(neighbors);
+    extras.timings_valid = false;
+    const size_t pair_limit = pairs_per_point_limit();
+    hipStream_t stream = nullptr; // the null stream, like the reference (vesin/src/vesin_cuda.cpp:798)
+
+    const bool timed = TIMINGS_ENABLED.load();
+    if (timed && !extras.have_events) {
+        for (auto& event : extras.events) {
+            HIP_CHECK(hipEventCreate(&event));
+        }
+        extras.have_events = true;
+    }
+    auto mark = [&](Stage stage) {
+        if (timed) {
+            HIP_CHECK(hipEventRecord(extras.events[stage], stream));
+        }
+    };
+
+    // ---- box and periodicity come to the host once: 75 bytes
+    HIP_CHECK(hipMemcpyAsync(extras.h_small, box, 9 * sizeof(double), hipMemcpyDeviceToHost, stream));
+    HIP_CHECK(hipMemcpyAsync(extras.h_small + 72, periodic, 3, hipMemcpyDeviceToHost, stream));
+    HIP_CHECK(hipStreamSynchronize(stream));
+    double host_box[9];
+    bool host_periodic[3];
+    std::memcpy(host_box, extras.h_small, sizeof(host_box));
+    for (int d = 0; d < 3; d++) {
+        host_periodic[d] = extras.h_small[72 + d] != 0;
+    }
+    const HostBox hbox = normalise_box(host_box, host_periodic);
+
+    if (n_points == 0) {
+        size_outputs(neighbors, extras, 0, options);
+        neighbors.length = 0;
+        return;
+    }
+
+    GridParams g;
+    std::memset(&g, 0, sizeof(g));
+    for (int d = 0; d < 3; d++) {
+        for (int e = 0; e < 3; e++) {
+            g.H[3 * d + e] = hbox.H[d][e];
+            g.Hinv[3 * d + e] = hbox.Hinv[d][e];
+        }
+        g.periodic[d] = hbox.periodic[d] ? 1 : 0;
+        g.np_scale[d] = 1.0;
+    }
+    g.cutoff2 = options.cutoff * options.cutoff; // vesin/src/cpu_cell_list.cpp:77
+    g.n_points = static_cast<uint32_t>(n_points);
+
+    mark(T_START);
+    hipLaunchKernelGGL(init_status, dim3(1), dim3(1), 0, stream, extras.d_status);
+
+    // ---- extent of the points along non-periodic directions
+    const bool any_open = !(hbox.periodic[0] && hbox.periodic[1] && hbox.periodic[2]);
+    double lo[3] = {0, 0, 0};
+    double hi[3] = {0, 0, 0};
+    if (any_open) {
+        uint32_t blocks = static_cast<uint32_t>((n_points + BLOCK - 1) / BLOCK);
+        if (blocks > 2048) {
+            blocks = 2048;
+        }
+        hipLaunchKernelGGL(
+            bounding_kernel, dim3(blocks), dim3(BLOCK), 0, stream,
+            reinterpret_cast<const double*>(points), g.n_points, g, extras.d_status
+        );
+        HIP_CHECK(hipMemcpyAsync(extras.h_status, extras.d_status, sizeof(DeviceStatus), hipMemcpyDeviceToHost, stream));
+        HIP_CHECK(hipStreamSynchronize(stream));
+        if (extras.h_status->first_bad_coordinate != 0xFFFFFFFFu) {
+            non_finite_error(points, extras.h_status->first_bad_coordinate);
+        }
+        for (int d = 0; d < 3; d++) {
+            lo[d] = ordered_bits_to_double(extras.h_status->frac_min[d]);
+            hi[d] = ordered_bits_to_double(extras.h_status->frac_max[d]);
+        }
+    }
+
+    // ---- grid: the brute-force layout is one cell whose stencil enumerates periodic images
+    bool single_cell = options.algorithm == VesinBruteForce;
+    HostGrid grid = choose_grid(hbox, options.cutoff, n_points, lo, hi, single_cell);
+    if (options.algorithm == VesinAutoAlgorithm && !single_cell && (grid.n_cells == 1 || n_points < 32)) {
+        single_cell = true;
+        grid = choose_grid(hbox, options.cutoff, n_points, lo, hi, true);
+    }
+    for (int d = 0; d < 3; d++) {
+        g.n[d] = grid.n[d];
+        g.s[d] = grid.s[d];
+        g.np_min[d] = grid.np_min[d];
+        g.np_scale[d] = grid.np_scale[d];
+    }
+    g.n_cells = static_cast<uint32_t>(grid.n_cells);
+
+    // ---- carve the work buffers
+    const size_t n_cells = grid.n_cells;
+    const size_t tiles_bound = (single_cell ? 0 : std::min<size_t>(n_cells, n_points)) + n_points / 64 + 1;
+    uint32_t n_slices = 1;
+    if (tiles_bound < 1024) {
+        n_slices = static_cast<uint32_t>(std::min<size_t>(64, (1024 + tiles_bound - 1) / tiles_bound));
+    }
+    const size_t search_blocks = tiles_bound * n_slices;
+    const size_t n_slots = search_blocks * WAVES_PER_BLOCK;
+
+    uint32_t* cell_counts = nullptr;
+    uint64_t* cell_scan = nullptr;
+    uint32_t* cell_of = nullptr;
+    uint32_t* slot_of = nullptr;
+    int32_t* wrap_of = nullptr;
+    uint32_t* provisional = nullptr;
+    SortedPoints sorted = {};
+    Tile* tiles = nullptr;
+    uint32_t* counts = nullptr;
+    uint64_t* offsets = nullptr;
+    uint64_t* scan_scratch = nullptr;
+    const size_t scratch_elements = std::max(scan_scratch_elements(n_cells), scan_scratch_elements(n_slots));
+
+    auto carve = [&](Carver& carver) {
+        cell_counts = carver.take<uint32_t>(n_cells);
+        cell_scan = carver.take<uint64_t>(n_cells + 1);
+        if (!single_cell) {
+            cell_of = carver.take<uint32_t>(n_points);
+            slot_of = carver.take<uint32_t>(n_points);
+            wrap_of = carver.take<int32_t>(3 * n_points);
+            provisional = carver.take<uint32_t>(n_points);
+        }
+        sorted.x = carver.take<double>(n_points);
+        sorted.y = carver.take<double>(n_points);
+        sorted.z = carver.take<double>(n_points);
+        sorted.index = carver.take<uint32_t>(n_points);
+        sorted.wx = carver.take<int32_t>(n_points);
+        sorted.wy = carver.take<int32_t>(n_points);
+        sorted.wz = carver.take<int32_t>(n_points);
+        tiles = carver.take<Tile>(tiles_bound);
+        counts = carver.take<uint32_t>(n_slots);
+        offsets = carver.take<uint64_t>(n_slots + 1);
+        scan_scratch = carver.take<uint64_t>(scratch_elements);
+    };
+    Carver measure(nullptr);
+    carve(measure);
+    extras.work.reserve(measure.used);
+    Carver carver(extras.work.ptr);
+    carve(carver);
+
+    // ---- cell list
+    const uint32_t point_blocks = static_cast<uint32_t>((n_points + BLOCK - 1) / BLOCK);
+    const auto* flat_points = reinterpret_cast<const double*>(points);
+    if (single_cell) {
+        hipLaunchKernelGGL(
+            prepare_single_cell, dim3(point_blocks), dim3(BLOCK), 0, stream,
+            flat_points, g, sorted, tiles, cell_scan, extras.d_status
+        );
+    } else {
+        HIP_CHECK(hipMemsetAsync(cell_counts, 0, n_cells * sizeof(uint32_t), stream));
+        hipLaunchKernelGGL(
+            assign_cells, dim3(point_blocks), dim3(BLOCK), 0, stream,
+            flat_points, g, cell_of, slot_of, wrap_of, cell_counts, extras.d_status
+        );
+        exclusive_scan<SCAN_CELL_COUNTS>(cell_counts, n_cells, cell_scan, scan_scratch, stream);
+        hipLaunchKernelGGL(
+            scatter_points, dim3(point_blocks), dim3(BLOCK), 0, stream,
+            g.n_points, cell_of, slot_of, cell_scan, provisional
+        );
+        const uint32_t cell_blocks = static_cast<uint32_t>((n_cells + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK);
+        hipLaunchKernelGGL(
+            gather_cells, dim3(cell_blocks), dim3(BLOCK), 0, stream,
+            flat_points, wrap_of, provisional, cell_scan, g.n_cells, sorted, tiles
+        );
+    }
+    mark(T_CELLS);
+
+    // ---- pass 1: count
+    SearchArgs args = {};
+    args.sorted = sorted;
+    args.cell_scan = cell_scan;
+    args.tiles = tiles;
+    args.counts = counts;
+    args.offsets = offsets;
+    args.n_slices = n_slices;
+    launch_search<false>(options.full, static_cast<uint32_t>(search_blocks), args, g, stream);
+    mark(T_COUNT);
+
+    exclusive_scan<SCAN_U32>(counts, n_slots, offsets, scan_scratch, stream);
+    mark(T_SCAN);
+
+    HIP_CHECK(hipMemcpyAsync(extras.h_status, extras.d_status, sizeof(DeviceStatus), hipMemcpyDeviceToHost, stream));
+    HIP_CHECK(hipMemcpyAsync(
+        &extras.h_status->total_pairs, offsets + n_slots, sizeof(uint64_t), hipMemcpyDeviceToHost, stream
+    ));
+    HIP_CHECK(hipStreamSynchronize(stream));
+    if (extras.h_status->first_bad_coordinate != 0xFFFFFFFFu) {
+        non_finite_error(points, extras.h_status->first_bad_coordinate);
+    }
+    const size_t total = extras.h_status->total_pairs;
+
+    if (pair_limit != 0 && total > n_points * pair_limit) {
+        throw std::runtime_error(
+            "The number of neighbor pairs exceeds the maximum capacity of " + std::to_string(n_points * pair_limit) +
+            " (max_pairs_per_point=" + std::to_string(pair_limit) + "; n_points=" + std::to_string(n_points) + "). " +
+            "Consider reducing the cutoff distance, or explicitly setting " +
+            "VESIN_CUDA_MAX_PAIRS_PER_POINT as an environment variable."
+        );
+    }
+
+    // ---- pass 2: write
+    size_outputs(neighbors, extras, total, options);
+    SearchOutputs final_out;
+    final_out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
+    final_out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
+    final_out.distances = neighbors.distances;
+    final_out.vectors = reinterpret_cast<double*>(neighbors.vectors);
+
+    const bool sorting = options.sorted && total > 1;
+    SearchOutputs unsorted = final_out;
+    SortWorkspace sort_space = {};
+    if (sorting) {
+        // the write pass goes to scratch rows (shifts always present: they are part of the sort key); the sort's
+        // final gather fills the caller's arrays
+        const size_t table_entries = static_cast<size_t>(RADIX) * sort_blocks(total);
+        auto carve_sort = [&](Carver& c) {
+            unsorted.pairs = c.take<unsigned long long>(2 * total);
+            unsorted.shifts = c.take<int32_t>(3 * total);
+            unsorted.distances = options.return_distances ? c.take<double>(total) : nullptr;
+            unsorted.vectors = options.return_vectors ? c.take<double>(3 * total) : nullptr;
+            for (int b = 0; b < 2; b++) {
+                sort_space.keys[b] = c.take<uint64_t>(total);
+                sort_space.rows[b] = c.take<uint32_t>(total);
+            }
+            sort_space.table = c.take<uint32_t>(table_entries);
+            sort_space.table_scan = c.take<uint64_t>(table_entries + 1);
+            sort_space.scan_scratch = c.take<uint64_t>(scan_scratch_elements(table_entries));
+            sort_space.range = c.take<ShiftRange>(1);
+        };
+        Carver measure_sort(nullptr);
+        carve_sort(measure_sort);
+        extras.sort_work.reserve(measure_sort.used);
+        Carver sort_carver(extras.sort_work.ptr);
+        carve_sort(sort_carver);
+    }
+
+    mark(T_WRITE_BEGIN);
+    if (total > 0) {
+        args.out = unsorted;
+        launch_search<true>(options.full, static_cast<uint32_t>(search_blocks), args, g, stream);
+    }
+    mark(T_WRITE);
+
+    if (sorting) {
+        sort_pairs(unsorted, final_out, total, n_points, sort_space, stream);
+    }
+    mark(T_SORT);
+
+    HIP_CHECK(hipStreamSynchronize(stream));
+    HIP_CHECK(hipGetLastError());
+    neighbors.length = total;
+
+    if (timed) {
+        auto elapsed = [&](Stage from, Stage to) {
+            float ms = 0.0f;
+            HIP_CHECK(hipEventElapsedTime(&ms, extras.events[from], extras.events[to]));
+            return ms;
+        };
+        extras.timings.total = elapsed(T_START, T_SORT);
+        extras.timings.cell_build = elapsed(T_START, T_CELLS);
+        extras.timings.count = elapsed(T_CELLS, T_COUNT);
+        extras.timings.scan = elapsed(T_COUNT, T_SCAN);
+        extras.timings.write = elapsed(T_WRITE_BEGIN, T_WRITE);
+        extras.timings.sort = elapsed(T_WRITE, T_SORT);
+        extras.timings.candidates = 0;
+        extras.timings_valid = true;
+    }
+}
+
+void free_neighbors(VesinNeighborList& neighbors) {
+    HIP_CHECK(hipSetDevice(neighbors.device.device_id));
+    free_outputs(neighbors);
+    delete static_cast<HipExtras*>(neighbors.opaque);
+    neighbors.opaque = nullptr;
+}
+
+bool last_timings(const VesinNeighborList& neighbors, VesinHipTimings& timings) {
+    const auto* extras = static_cast<const HipExtras*>(neighbors.opaque);
+    if (extras == nullptr || !extras->timings_valid) {
+        return false;
+    }
+    timings = extras->timings;
+    return true;
+}
+
+} // namespace vesin_hip

@@ -1,0 +1,230 @@
+// Host-side box normalisation and grid selection for the HIP neighbor-list path.
+//
+// The box handling reproduces the semantics of the reference's BoundingBox (vesin/src/types.hpp:20-97): rows
+// of non-periodic directions are replaced by unit vectors orthogonal to the periodic ones, the box must be
+// invertible (|det| >= 1e-30), and the distance between opposite faces bounds how many cells fit per direction.
+// The operation order follows the reference so that the rows used for the shift vectors (T = S . H) carry the
+// same bits; this file must be compiled with -ffp-contract=off.
+//
+// The grid itself is this library's own choice (the pair set does not depend on it): cells are at least
+// cutoff * (1 + 1e-9) wide so that rounding in the cell assignment can never push a pair outside the stencil,
+// non-periodic directions are binned along the replaced (orthogonal) box rows, and the total number of cells
+// scales with the number of points.
+#ifndef VESIN_HIP_GEOMETRY_HPP
+#define VESIN_HIP_GEOMETRY_HPP
+
+#include <cmath>
+#include <cstddef>
+#include <cstdint>
+#include <stdexcept>
+
+namespace vesin_hip {
+
+struct HostBox {
+    double H[3][3];    // normalised box, one vector per row
+    double Hinv[3][3]; // inverse of H: fractional = cartesian (row vector) * Hinv
+    double face[3];    // distance between opposite faces (periodic directions only)
+    bool periodic[3];
+};
+
+namespace detail {
+    struct V3 {
+        double x, y, z;
+    };
+
+    inline double dot(V3 a, V3 b) {
+        return a.x * b.x + a.y * b.y + a.z * b.z;
+    }
+
+    inline V3 cross(V3 a, V3 b) {
+        return V3{a.y * b.z - a.z * b.y, a.z * b.x - a.x * b.z, a.x * b.y - a.y * b.x};
+    }
+
+    inline V3 unit(V3 a) {
+        double s = 1.0 / std::sqrt(dot(a, a));
+        return V3{s * a.x, s * a.y, s * a.z};
+    }
+
+    inline V3 get_row(const double m[3][3], int i) {
+        return V3{m[i][0], m[i][1], m[i][2]};
+    }
+
+    inline void put_row(double m[3][3], int i, V3 v) {
+        m[i][0] = v.x;
+        m[i][1] = v.y;
+        m[i][2] = v.z;
+    }
+} // namespace detail
+
+/// Build the normalised box. Throws std::runtime_error("the box matrix is not invertible") like the reference
+/// (types.hpp:75-78).
+inline HostBox normalise_box(const double box[9], const bool periodic[3]) {
+    using namespace detail;
+    HostBox out;
+    int n_periodic = 0;
+    int first = -1;
+    int second = -1;
+    for (int d = 0; d < 3; d++) {
+        out.periodic[d] = periodic[d];
+        for (int e = 0; e < 3; e++) {
+            out.H[d][e] = box[3 * d + e];
+        }
+        if (periodic[d]) {
+            n_periodic += 1;
+            if (first < 0) {
+                first = d;
+            } else if (second < 0) {
+                second = d;
+            }
+        }
+    }
+
+    if (n_periodic == 0) {
+        for (int d = 0; d < 3; d++) {
+            for (int e = 0; e < 3; e++) {
+                out.H[d][e] = d == e ? 1.0 : 0.0;
+            }
+        }
+    } else if (n_periodic == 1) {
+        V3 a = get_row(out.H, first);
+        V3 helper{0.0, 1.0, 0.0};
+        if (std::abs(dot(unit(a), helper)) > 0.9) {
+            helper = V3{0.0, 0.0, 1.0};
+        }
+        V3 c = unit(cross(a, helper));
+        V3 b = unit(cross(c, a));
+        put_row(out.H, (first + 1) % 3, b);
+        put_row(out.H, (first + 2) % 3, c);
+    } else if (n_periodic == 2) {
+        V3 c = unit(cross(get_row(out.H, first), get_row(out.H, second)));
+        put_row(out.H, 3 - first - second, c);
+    }
+
+    const auto& m = out.H;
+    double det = m[0][0] * (m[1][1] * m[2][2] - m[2][1] * m[1][2])
+               - m[0][1] * (m[1][0] * m[2][2] - m[1][2] * m[2][0])
+               + m[0][2] * (m[1][0] * m[2][1] - m[1][1] * m[2][0]);
+    if (!(std::abs(det) >= 1e-30)) {
+        throw std::runtime_error("the box matrix is not invertible");
+    }
+
+    out.Hinv[0][0] = (m[1][1] * m[2][2] - m[2][1] * m[1][2]) / det;
+    out.Hinv[0][1] = (m[0][2] * m[2][1] - m[0][1] * m[2][2]) / det;
+    out.Hinv[0][2] = (m[0][1] * m[1][2] - m[0][2] * m[1][1]) / det;
+    out.Hinv[1][0] = (m[1][2] * m[2][0] - m[1][0] * m[2][2]) / det;
+    out.Hinv[1][1] = (m[0][0] * m[2][2] - m[0][2] * m[2][0]) / det;
+    out.Hinv[1][2] = (m[1][0] * m[0][2] - m[0][0] * m[1][2]) / det;
+    out.Hinv[2][0] = (m[1][0] * m[2][1] - m[2][0] * m[1][1]) / det;
+    out.Hinv[2][1] = (m[2][0] * m[0][1] - m[0][0] * m[2][1]) / det;
+    out.Hinv[2][2] = (m[0][0] * m[1][1] - m[1][0] * m[0][1]) / det;
+
+    V3 a = get_row(out.H, 0);
+    V3 b = get_row(out.H, 1);
+    V3 c = get_row(out.H, 2);
+    out.face[0] = std::abs(dot(unit(cross(b, c)), a));
+    out.face[1] = std::abs(dot(unit(cross(c, a)), b));
+    out.face[2] = std::abs(dot(unit(cross(a, b)), c));
+    return out;
+}
+
+struct HostGrid {
+    int32_t n[3];          // cells per direction
+    int32_t s[3];          // stencil radius per direction (cells searched on each side)
+    double np_min[3];      // non-periodic directions: smallest projected coordinate
+    double np_scale[3];    // non-periodic directions: 1 / extent
+    uint64_t n_cells;
+};
+
+constexpr double CELL_MARGIN = 1.0 + 1e-9;
+constexpr int32_t MAX_STENCIL_RADIUS = 500;
+
+/// Choose the cell grid. `lo`/`hi` are the extrema of the fractional (projected) coordinates; they are only read
+/// for non-periodic directions. With `single_cell` every point goes to one cell and the stencil enumerates the
+/// periodic images directly (the brute-force and multi-image path).
+inline HostGrid choose_grid(
+    const HostBox& box, double cutoff, size_t n_points, const double lo[3], const double hi[3], bool single_cell
+) {
+    HostGrid grid;
+    double extent[3];
+    double cells[3];
+    const double padded = cutoff * CELL_MARGIN;
+
+    for (int d = 0; d < 3; d++) {
+        if (box.periodic[d]) {
+            extent[d] = box.face[d];
+            grid.np_min[d] = 0.0;
+            grid.np_scale[d] = 1.0;
+        } else {
+            // the replaced rows are unit vectors, so the projected coordinate is a length; add the same 1% margin
+            // and 1.0 floor as the reference (types.hpp:180-198) so that every point is strictly inside
+            double width = n_points > 0 ? hi[d] - lo[d] : 0.0;
+            if (!(width >= 1e-6)) {
+                width = 1.0;
+            }
+            extent[d] = width * 1.01;
+            if (extent[d] < 1.0) {
+                extent[d] = 1.0;
+            }
+            grid.np_min[d] = n_points > 0 ? lo[d] : 0.0;
+            grid.np_scale[d] = 1.0 / extent[d];
+        }
+
+        cells[d] = std::floor(extent[d] / padded);
+        if (!(cells[d] >= 1.0)) {
+            cells[d] = 1.0;
+        }
+        if (cells[d] > 1048576.0) {
+            cells[d] = 1048576.0;
+        }
+        if (single_cell) {
+            cells[d] = 1.0;
+        }
+    }
+
+    // keep the number of cells proportional to the number of points
+    double max_cells = 2.0 * static_cast<double>(n_points);
+    if (max_cells < 64.0) {
+        max_cells = 64.0;
+    }
+    if (max_cells > 16777216.0) {
+        max_cells = 16777216.0;
+    }
+    double total = cells[0] * cells[1] * cells[2];
+    if (total > max_cells) {
+        double shrink = std::cbrt(max_cells / total);
+        for (int d = 0; d < 3; d++) {
+            cells[d] = std::floor(cells[d] * shrink);
+            if (cells[d] < 1.0) {
+                cells[d] = 1.0;
+            }
+        }
+    }
+
+    grid.n_cells = 1;
+    for (int d = 0; d < 3; d++) {
+        grid.n[d] = static_cast<int32_t>(cells[d]);
+        grid.n_cells *= static_cast<uint64_t>(grid.n[d]);
+
+        double radius = std::ceil(padded * cells[d] / extent[d]);
+        if (!(radius >= 1.0)) {
+            radius = 1.0;
+        }
+        if (!box.periodic[d]) {
+            // nothing exists beyond the last cell of a non-periodic direction
+            if (radius > cells[d] - 1.0) {
+                radius = cells[d] - 1.0;
+            }
+        }
+        if (radius > static_cast<double>(MAX_STENCIL_RADIUS)) {
+            throw std::runtime_error(
+                "cutoff is too large for this box: more than 500 periodic images would be needed in one direction"
+            );
+        }
+        grid.s[d] = static_cast<int32_t>(radius);
+    }
+    return grid;
+}
+
+} // namespace vesin_hip
+
+#endif
