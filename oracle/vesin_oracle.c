@@ -158,7 +158,10 @@ static int box_init(bounding_box* b, const double box[9], const uint8_t periodic
     }
 
     double det = determinant(&b->matrix);
-    if (fabs(det) < 1e-30) {
+    /* The reference only tests `abs(det) < 1e-30`; a NaN determinant (a periodic direction with a zero box
+       vector) passes that test there and leads to undefined behaviour (NaN cell counts cast to integers). The
+       oracle refuses such a box instead of reproducing it. */
+    if (fabs(det) < 1e-30 || det != det) {
         snprintf(error, error_len, "the box matrix is not invertible");
         return 1;
     }

@@ -53,3 +53,22 @@ def assert_same_list(actual, expected, ordered=False, what=""):
                 scale = np.maximum(np.abs(expected[key]), 1e-300)
                 worst = float(np.max(np.abs(actual[key] - expected[key]) / scale))
                 raise AssertionError(f"{what}: {key} not bit-identical, worst relative difference {worst:.3e}")
+
+
+import pytest  # noqa: E402
+
+ENGINES = [pytest.param("oracle", id="oracle"), pytest.param("gpu", id="gpu", marks=pytest.mark.gpu)]
+
+
+def run_engine(engine, points, box, periodic, cutoff, full=True, sorted=False, quantities="ijSdD", algorithm="auto"):
+    """Same call against the CPU oracle or the HIP path."""
+    if engine == "oracle":
+        return oracle.neighbors(points, box, periodic, cutoff, full, sorted, quantities)
+    return gpu_neighbors(points, box, periodic, cutoff, full, sorted, quantities, algorithm)
+
+
+def ulp_close(actual, expected, ulps=4):
+    actual = np.asarray(actual, dtype=np.float64)
+    expected = np.asarray(expected, dtype=np.float64)
+    spacing = np.spacing(np.maximum(np.abs(actual), np.abs(expected)))
+    return bool(np.all(np.abs(actual - expected) <= ulps * spacing))

@@ -3,9 +3,11 @@ import sys
 
 import pytest
 
-ROOT = os.path.dirname(os.path.dirname(os.path.realpath(__file__)))
-if ROOT not in sys.path:
-    sys.path.insert(0, ROOT)
+TESTS = os.path.dirname(os.path.realpath(__file__))
+ROOT = os.path.dirname(TESTS)
+for path in (TESTS, ROOT):
+    if path not in sys.path:
+        sys.path.insert(0, path)
 
 
 def pytest_configure(config):

@@ -1,0 +1,46 @@
+"""Regenerate reference_checksums.json: run the COMPILED reference CPU path (oracle/_ref/libvesin_ref.so, built by
+oracle/Makefile from the reference's own sources) on every golden case and store order-independent fingerprints.
+
+Needs the reference checkout (for the build); run from the repository root:
+
+    python -m tests.golden.make_golden [--full-size]
+
+Small cases are always regenerated; full-size benchmark configurations are kept from the existing file unless
+--full-size is given (they take minutes and several GB of host memory).
+"""
+
+import json
+import os
+import sys
+
+import oracle
+from tests.golden import systems
+
+OUT = os.path.join(os.path.dirname(os.path.realpath(__file__)), "reference_checksums.json")
+
+
+def main():
+    full_size = "--full-size" in sys.argv
+    oracle.build()
+    if not oracle.have_ref():
+        raise SystemExit("oracle/_ref/libvesin_ref.so is missing: the reference checkout is needed to build it")
+
+    golden = {}
+    if os.path.exists(OUT):
+        with open(OUT) as fd:
+            golden = json.load(fd)
+
+    for name, points, box, periodic, cutoff, full in systems.golden_cases(full_size=full_size):
+        result = oracle.ref_neighbors(points, box, periodic, cutoff, full, False, "ijSdD")
+        entry = systems.fingerprints(result)
+        entry.update(cutoff=cutoff, full=full, n_points=int(len(points)))
+        golden[name] = entry
+        print(name, entry["n_pairs"], flush=True)
+        del result
+
+    with open(OUT, "w") as fd:
+        json.dump(golden, fd, indent=1, sort_keys=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,125 @@
+"""Host logic of the HIP driver (vesin_amd/csrc/geometry.hpp), checked on the CPU through a small g++-built shim:
+the normalised box, its inverse and the face distances must carry the same bits as the oracle's (they feed the
+shift vectors), and the grid must keep its covering guarantee."""
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import oracle
+from golden import systems
+
+HERE = os.path.dirname(os.path.realpath(__file__))
+ROOT = os.path.dirname(HERE)
+
+
+@pytest.fixture(scope="module")
+def probe(tmp_path_factory):
+    out = str(tmp_path_factory.mktemp("probe") / "libprobe.so")
+    subprocess.run(
+        ["g++", "-std=c++17", "-O2", "-ffp-contract=off", "-fPIC", "-shared", "-I", os.path.join(ROOT, "vesin_amd", "csrc"),
+         os.path.join(HERE, "host_probe.cpp"), "-o", out],
+        check=True,
+    )
+    lib = ctypes.CDLL(out)
+    lib.probe_box.argtypes = [ctypes.c_void_p] * 5
+    lib.probe_grid.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_double, ctypes.c_size_t, ctypes.c_void_p,
+                               ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    return lib
+
+
+def run_box(probe, box, periodic):
+    box = np.ascontiguousarray(box, dtype=np.float64)
+    periodic = np.ascontiguousarray(periodic, dtype=np.uint8)
+    H, Hinv, face = np.zeros((3, 3)), np.zeros((3, 3)), np.zeros(3)
+    status = probe.probe_box(box.ctypes.data, periodic.ctypes.data, H.ctypes.data, Hinv.ctypes.data, face.ctypes.data)
+    return status, H, Hinv, face
+
+
+def run_grid(probe, box, periodic, cutoff, n_points, lo, hi, single_cell=False):
+    box = np.ascontiguousarray(box, dtype=np.float64)
+    periodic = np.ascontiguousarray(periodic, dtype=np.uint8)
+    lo = np.ascontiguousarray(lo, dtype=np.float64)
+    hi = np.ascontiguousarray(hi, dtype=np.float64)
+    n, s = np.zeros(3, dtype=np.int32), np.zeros(3, dtype=np.int32)
+    status = probe.probe_grid(box.ctypes.data, periodic.ctypes.data, cutoff, n_points, lo.ctypes.data, hi.ctypes.data,
+                              int(single_cell), n.ctypes.data, s.ctypes.data)
+    return status, n, s
+
+
+@pytest.mark.parametrize("name", list(systems.small_systems()))
+@pytest.mark.parametrize("mask", range(8))
+def test_box_bits_match_the_oracle(probe, name, mask):
+    points, box, _ = systems.small_systems()[name]
+    periodic = np.array([(mask >> d) & 1 == 1 for d in range(3)])
+    if np.allclose(box, 0) and periodic.any():
+        box = systems.transformed((points, np.diag([11.0, 12.0, 13.0]), periodic), 5, False)[1]
+    try:
+        grid = oracle.neighbors(points, box, periodic, 4.0, return_grid=True)["grid"]
+    except RuntimeError as e:
+        assert "not invertible" in str(e)
+        assert run_box(probe, box, periodic)[0] == 1
+        return
+    status, H, Hinv, face = run_box(probe, box, periodic)
+    assert status == 0
+    assert np.array_equal(H, grid["matrix"])
+    assert np.array_equal(Hinv, grid["inverse"])
+    for d in range(3):
+        if periodic[d]:
+            assert face[d] == grid["face_distances"][d]
+
+
+def test_singular_box_is_refused(probe):
+    assert run_box(probe, np.zeros((3, 3)), [True, True, True])[0] == 1
+    assert run_box(probe, np.zeros((3, 3)), [False, False, False])[0] == 0  # box ignored
+    assert run_box(probe, np.diag([4.0, 4.5, 0.0]), [True, True, False])[0] == 0  # python/vesin/tests/_utils.py:186-194
+
+
+def test_grid_orthorhombic(probe):
+    lengths = np.array([10.7, 23.1, 37.9])
+    status, n, s = run_grid(probe, np.diag(lengths), [1, 1, 1], 5.0, 10000, [0] * 3, [0] * 3)
+    assert status == 0 and n.tolist() == [2, 4, 7] and s.tolist() == [1, 1, 1]
+    # cutoff above the box: images on each side
+    status, n, s = run_grid(probe, np.diag(lengths), [1, 1, 1], 25.0, 10000, [0] * 3, [0] * 3)
+    assert n.tolist() == [1, 1, 1] and s.tolist() == [3, 2, 1]
+    # an edge that is an exact multiple of the cutoff gets one cell less, never a cell of exactly the cutoff
+    status, n, s = run_grid(probe, np.diag([20.0, 20.0, 20.0]), [1, 1, 1], 5.0, 10000, [0] * 3, [0] * 3)
+    assert n.tolist() == [3, 3, 3] and s.tolist() == [1, 1, 1]
+
+
+def test_grid_covering_guarantee(probe):
+    rng = np.random.default_rng(0)
+    for _ in range(200):
+        box = rng.normal(size=(3, 3)) * rng.uniform(1, 30)
+        if abs(np.linalg.det(box)) < 1e-3:
+            continue
+        cutoff = rng.uniform(0.5, 12)
+        n_points = int(rng.integers(1, 100000))
+        status, n, s = run_grid(probe, box, [1, 1, 1], cutoff, n_points, [0] * 3, [0] * 3)
+        assert status == 0
+        _, _, _, face = run_box(probe, box, [1, 1, 1])
+        # s cells of width face / n must reach beyond the cutoff
+        assert np.all(s * face / n > cutoff)
+        assert np.prod(n.astype(np.int64)) <= max(64, 2 * n_points)
+
+
+def test_grid_open_directions_and_single_cell(probe):
+    box = np.diag([300.0, 300.0, 300.0])
+    status, n, s = run_grid(probe, box, [1, 1, 0], 4.5, 500000, [0, 0, -20.0], [0, 0, 330.0])
+    assert status == 0
+    assert n[2] == int(np.floor(350.0 * 1.01 / (4.5 * (1 + 1e-9)))) and s.tolist() == [1, 1, 1]
+    # a flat system along an open direction: one cell, nothing to search beyond it
+    status, n, s = run_grid(probe, box, [1, 1, 0], 4.5, 1000, [0, 0, 1.0], [0, 0, 1.0])
+    assert n[2] == 1 and s[2] == 0
+    status, n, s = run_grid(probe, np.diag([7.134] * 3), [1, 1, 1], 10.0, 64, [0] * 3, [0] * 3, single_cell=True)
+    assert n.tolist() == [1, 1, 1] and s.tolist() == [2, 2, 2]
+    status, n, s = run_grid(probe, box, [0, 0, 0], 4.5, 64, [0] * 3, [100.0] * 3, single_cell=True)
+    assert n.tolist() == [1, 1, 1] and s.tolist() == [0, 0, 0]
+
+
+def test_too_many_images_is_an_error(probe):
+    status, _, _ = run_grid(probe, np.eye(3) * 0.01, [1, 1, 1], 10.0, 10, [0] * 3, [0] * 3)
+    assert status == 1

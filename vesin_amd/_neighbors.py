@@ -195,9 +195,12 @@ class NeighborList:
         # inputs may still be in flight on torch's current stream
         torch.cuda.current_stream(device).synchronize()
 
+        # an empty tensor has no storage; the ABI still wants a device pointer
+        points_ptr = points.data_ptr() if points.shape[0] > 0 else box.data_ptr()
+
         error_message = ctypes.c_char_p()
         status = self._lib.vesin_neighbors(
-            points.data_ptr(),
+            points_ptr,
             points.shape[0],
             box.data_ptr(),
             periodic.data_ptr(),
