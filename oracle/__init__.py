@@ -13,6 +13,7 @@ The shipped library never does.
 import ctypes
 import os
 import subprocess
+import time
 
 import numpy as np
 
@@ -59,6 +60,9 @@ class _Grid(ctypes.Structure):
 
 
 _oracle = None
+
+# wall-clock seconds spent inside the C call of the most recent neighbors() / ref_neighbors()
+last_call_seconds = 0.0
 
 
 def _load_oracle():
@@ -123,8 +127,11 @@ def neighbors(points, box, periodic, cutoff, full=True, sorted=False, quantities
     out = _List()
     grid = _Grid()
     error = ctypes.create_string_buffer(512)
+    global last_call_seconds
+    start = time.perf_counter()
     status = lib.vesin_oracle_neighbors(points.ctypes.data, points.shape[0], box.ctypes.data, periodic.ctypes.data,
                                         ctypes.byref(options), ctypes.byref(out), ctypes.byref(grid), error, 512)
+    last_call_seconds = time.perf_counter() - start
     if status != 0:
         raise RuntimeError(error.value.decode("utf8"))
     try:
@@ -219,8 +226,11 @@ def ref_neighbors(points, box, periodic, cutoff, full=True, sorted=False, quanti
                           "d" in quantities, "D" in quantities, 0.0)
     out = _RefList()
     message = ctypes.c_char_p()
+    global last_call_seconds
+    start = time.perf_counter()
     status = lib.vesin_neighbors(points.ctypes.data, points.shape[0], box.ctypes.data, periodic.ctypes.data,
                                  _RefDevice(1, 0), options, ctypes.byref(out), ctypes.byref(message))
+    last_call_seconds = time.perf_counter() - start
     if status != 0:
         raise RuntimeError(message.value.decode("utf8"))
     try:
