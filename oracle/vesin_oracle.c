@@ -19,7 +19,7 @@
  *   vesin/src/threadpool.hpp:156-159      static contiguous chunks of cells per thread
  *   vesin/src/vesin.cpp:70-78             cutoff validation
  *
- * Parity status: every function here is pinned by tests/test_oracle_*.py against the literal vectors of the
+ * Parity status: every function here is pinned by tests/test_oracle.py and tests/test_known_answers.py against the literal vectors of the
  * reference's own tests, against closed forms / brute force, and (where oracle/_ref builds) against the compiled
  * reference itself.
  */
