@@ -12,7 +12,9 @@
 
 namespace vesin_hip {
 
-/// Cell-sorted copy of the points, one array per component so that 64 consecutive candidates load coalesced.
+/// Cell-sorted copy of the points, one array per component: 64 consecutive candidates load coalesced, and four
+/// consecutive points of a tile arrive with one scalar load per component. x, y, z and index are allocated with
+/// SORTED_PADDING extra elements so that those scalar loads may run past the last point.
 struct SortedPoints {
     double* x;
     double* y;
@@ -22,6 +24,8 @@ struct SortedPoints {
     int32_t* wy;
     int32_t* wz;
 };
+
+constexpr uint32_t SORTED_PADDING = 8;
 
 __global__ void init_status(DeviceStatus* status) {
     if (threadIdx.x == 0 && blockIdx.x == 0) {
@@ -209,15 +213,7 @@ __global__ __launch_bounds__(BLOCK) void gather_cells(
         return;
     }
 
-    for (uint32_t t = lane; t * 64u < count; t += WAVE) {
-        Tile tile;
-        tile.cell = cell;
-        tile.first = start + t * 64u;
-        tile.count = min(64u, count - t * 64u);
-        tile.pad = 0;
-        tiles[first_tile + t] = tile;
-    }
-
+    bool any_wrapped = false;
     for (uint32_t base = 0; base < count; base += WAVE) {
         uint32_t k = base + lane;
         bool active = k < count;
@@ -230,16 +226,32 @@ __global__ __launch_bounds__(BLOCK) void gather_cells(
                 rank += provisional[start + other] < mine ? 1u : 0u;
             }
         }
+        bool wrapped = false;
         if (active) {
             uint32_t to = start + rank;
+            const int32_t wx = wrap_of[3 * static_cast<size_t>(mine) + 0];
+            const int32_t wy = wrap_of[3 * static_cast<size_t>(mine) + 1];
+            const int32_t wz = wrap_of[3 * static_cast<size_t>(mine) + 2];
+            wrapped = (wx | wy | wz) != 0;
             sorted.index[to] = mine;
             sorted.x[to] = points[3 * static_cast<size_t>(mine) + 0];
             sorted.y[to] = points[3 * static_cast<size_t>(mine) + 1];
             sorted.z[to] = points[3 * static_cast<size_t>(mine) + 2];
-            sorted.wx[to] = wrap_of[3 * static_cast<size_t>(mine) + 0];
-            sorted.wy[to] = wrap_of[3 * static_cast<size_t>(mine) + 1];
-            sorted.wz[to] = wrap_of[3 * static_cast<size_t>(mine) + 2];
+            sorted.wx[to] = wx;
+            sorted.wy[to] = wy;
+            sorted.wz[to] = wz;
         }
+        any_wrapped = any_wrapped || (__ballot(wrapped) != 0);
+    }
+
+    // tiles of a cell holding a wrapped point take the search kernel's general path
+    for (uint32_t t = lane; t * 64u < count; t += WAVE) {
+        Tile tile;
+        tile.cell = cell;
+        tile.first = start + t * 64u;
+        tile.count = min(64u, count - t * 64u);
+        tile.wrapped = any_wrapped ? 1u : 0u;
+        tiles[first_tile + t] = tile;
     }
 }
 
@@ -255,35 +267,39 @@ __global__ __launch_bounds__(BLOCK) void prepare_single_cell(
         cell_scan[0] = 0;
         cell_scan[1] = static_cast<uint64_t>(g.n_points) | (static_cast<uint64_t>(n_tiles) << 32);
     }
-    if (i < n_tiles) {
+    bool wrapped = false;
+    if (i < g.n_points) {
+        const double x = points[3 * static_cast<size_t>(i) + 0];
+        const double y = points[3 * static_cast<size_t>(i) + 1];
+        const double z = points[3 * static_cast<size_t>(i) + 2];
+        int32_t cell[3] = {0, 0, 0};
+        int32_t wrap[3] = {0, 0, 0};
+        unsigned int axis;
+        if (all_finite(x, y, z, axis)) {
+            locate(g, x, y, z, cell, wrap);
+        } else {
+            atomicMin(&status->first_bad_coordinate, 3u * i + axis);
+        }
+        wrapped = (wrap[0] | wrap[1] | wrap[2]) != 0;
+        sorted.index[i] = i;
+        sorted.x[i] = x;
+        sorted.y[i] = y;
+        sorted.z[i] = z;
+        sorted.wx[i] = wrap[0];
+        sorted.wy[i] = wrap[1];
+        sorted.wz[i] = wrap[2];
+    }
+    // one wave covers exactly one tile of 64 consecutive points
+    const bool any_wrapped = __ballot(wrapped) != 0;
+    const uint32_t tile_id = i / 64u;
+    if (lane_id() == 0 && tile_id < n_tiles) {
         Tile tile;
         tile.cell = 0;
-        tile.first = i * 64u;
-        tile.count = min(64u, g.n_points - i * 64u);
-        tile.pad = 0;
-        tiles[i] = tile;
+        tile.first = tile_id * 64u;
+        tile.count = min(64u, g.n_points - tile_id * 64u);
+        tile.wrapped = any_wrapped ? 1u : 0u;
+        tiles[tile_id] = tile;
     }
-    if (i >= g.n_points) {
-        return;
-    }
-    double x = points[3 * static_cast<size_t>(i) + 0];
-    double y = points[3 * static_cast<size_t>(i) + 1];
-    double z = points[3 * static_cast<size_t>(i) + 2];
-    int32_t cell[3] = {0, 0, 0};
-    int32_t wrap[3] = {0, 0, 0};
-    unsigned int axis;
-    if (all_finite(x, y, z, axis)) {
-        locate(g, x, y, z, cell, wrap);
-    } else {
-        atomicMin(&status->first_bad_coordinate, 3u * i + axis);
-    }
-    sorted.index[i] = i;
-    sorted.x[i] = x;
-    sorted.y[i] = y;
-    sorted.z[i] = z;
-    sorted.wx[i] = wrap[0];
-    sorted.wy[i] = wrap[1];
-    sorted.wz[i] = wrap[2];
 }
 
 } // namespace vesin_hip

@@ -30,7 +30,7 @@ struct Tile {
     uint32_t cell;   // linear cell index of these points
     uint32_t first;  // position of the first point in the cell-sorted arrays
     uint32_t count;  // 1..64
-    uint32_t pad;
+    uint32_t wrapped;// 1 when a point of the cell was moved by a box vector to land inside the box
 };
 
 /// Small block of results the host reads back after the counting pass.

@@ -10,6 +10,7 @@
 #include <cerrno>
 #include <cmath>
 #include <cstdlib>
+#include <cstdio>
 #include <cstring>
 
 #include <atomic>
@@ -231,15 +232,24 @@ size_t pairs_per_point_limit() {
 }
 
 template <bool WRITE>
-void launch_search(bool full, uint32_t blocks, const SearchArgs& args, const GridParams& g, hipStream_t stream) {
-    if (blocks == 0) {
+void launch_search(bool full, const SearchArgs& args, const GridParams& g, hipStream_t stream) {
+    if (args.n_work == 0) {
         return;
     }
     constexpr int R = 2;
+    if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
+        int a = -1, b = -1;
+        (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&a, search_kernel<WRITE, true, R>, SEARCH_BLOCK, 0);
+        (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&b, search_kernel<WRITE, false, R>, SEARCH_BLOCK, 0);
+        hipFuncAttributes attr;
+        (void)hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(search_kernel<WRITE, true, R>));
+        fprintf(stderr, "search<%d>: blocks/CU full=%d half=%d regs=%d lds=%zu\n", int(WRITE), a, b, attr.numRegs, attr.sharedSizeBytes);
+    }
+    const uint32_t blocks = (args.n_work + SEARCH_WAVES - 1) / SEARCH_WAVES;
     if (full) {
-        hipLaunchKernelGGL((search_kernel<WRITE, true, R>), dim3(blocks), dim3(BLOCK), 0, stream, args, g);
+        hipLaunchKernelGGL((search_kernel<WRITE, true, R>), dim3(blocks), dim3(SEARCH_BLOCK), 0, stream, args, g);
     } else {
-        hipLaunchKernelGGL((search_kernel<WRITE, false, R>), dim3(blocks), dim3(BLOCK), 0, stream, args, g);
+        hipLaunchKernelGGL((search_kernel<WRITE, false, R>), dim3(blocks), dim3(SEARCH_BLOCK), 0, stream, args, g);
     }
 }
 
@@ -395,13 +405,17 @@ void neighbors(
 
     // ---- carve the work buffers
     const size_t n_cells = grid.n_cells;
-    const size_t tiles_bound = (single_cell ? 0 : std::min<size_t>(n_cells, n_points)) + n_points / 64 + 1;
+    // upper bound of the number of tiles, rounded up to what the search kernel's XCD-aware order needs
+    size_t tiles_bound = (single_cell ? 0 : std::min<size_t>(n_cells, n_points)) + n_points / 64 + 1;
+    constexpr size_t slot_multiple = N_XCD * SEARCH_WAVES;
+    tiles_bound = (tiles_bound + slot_multiple - 1) / slot_multiple * slot_multiple;
+    // small systems: several workgroups (of one wave each) share a tile, each taking a slice of its candidates
     uint32_t n_slices = 1;
-    if (tiles_bound < 1024) {
-        n_slices = static_cast<uint32_t>(std::min<size_t>(64, (1024 + tiles_bound - 1) / tiles_bound));
+    if (tiles_bound < 8192) {
+        n_slices = static_cast<uint32_t>(std::min<size_t>(256, (8192 + tiles_bound - 1) / tiles_bound));
     }
     const size_t search_blocks = tiles_bound * n_slices;
-    const size_t n_slots = search_blocks * WAVES_PER_BLOCK;
+    const size_t n_slots = search_blocks;
 
     uint32_t* cell_counts = nullptr;
     uint64_t* cell_scan = nullptr;
@@ -425,10 +439,10 @@ void neighbors(
             wrap_of = carver.take<int32_t>(3 * n_points);
             provisional = carver.take<uint32_t>(n_points);
         }
-        sorted.x = carver.take<double>(n_points);
-        sorted.y = carver.take<double>(n_points);
-        sorted.z = carver.take<double>(n_points);
-        sorted.index = carver.take<uint32_t>(n_points);
+        sorted.x = carver.take<double>(n_points + SORTED_PADDING);
+        sorted.y = carver.take<double>(n_points + SORTED_PADDING);
+        sorted.z = carver.take<double>(n_points + SORTED_PADDING);
+        sorted.index = carver.take<uint32_t>(n_points + SORTED_PADDING);
         sorted.wx = carver.take<int32_t>(n_points);
         sorted.wy = carver.take<int32_t>(n_points);
         sorted.wz = carver.take<int32_t>(n_points);
@@ -478,7 +492,8 @@ void neighbors(
     args.counts = counts;
     args.offsets = offsets;
     args.n_slices = n_slices;
-    launch_search<false>(options.full, static_cast<uint32_t>(search_blocks), args, g, stream);
+    args.n_work = static_cast<uint32_t>(search_blocks);
+    launch_search<false>(options.full, args, g, stream);
     mark(T_COUNT);
 
     exclusive_scan<SCAN_U32>(counts, n_slots, offsets, scan_scratch, stream);
@@ -542,7 +557,7 @@ void neighbors(
     mark(T_WRITE_BEGIN);
     if (total > 0) {
         args.out = unsorted;
-        launch_search<true>(options.full, static_cast<uint32_t>(search_blocks), args, g, stream);
+        launch_search<true>(options.full, args, g, stream);
     }
     mark(T_WRITE);
 

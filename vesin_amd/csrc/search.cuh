@@ -8,8 +8,10 @@
 //
 // Mapping: lanes hold candidates. A wave loads R groups of 64 consecutive candidates into registers (coalesced
 // reads from the cell-sorted structure-of-arrays), then loops over the tile's points `i`, whose coordinates come
-// in through scalar loads. Each (i, group) test costs 9-12 fp64 VALU operations and yields a 64-bit hit mask in
-// scalar registers.
+// in through scalar loads issued one iteration ahead. Each (i, group) test is 9 fp64 VALU operations (12 when a
+// shift vector has to be added) and yields a 64-bit hit mask in scalar registers. The loop is compiled in four
+// variants (candidates shifted or not, tile's own cell among them or not), picked per group batch, plus a general
+// variant for tiles holding points that were wrapped into the box.
 //
 // The same code runs twice:
 //   COUNT  adds up popcounts: one 32-bit total per wave, no atomics;
@@ -25,19 +27,27 @@
 //   keep iff d2 < cutoff*cutoff, d = sqrt(d2).
 // Adding T may be skipped in the test when S = 0 (it is +-0 and cannot change d2); the stored vector always adds it.
 //
+// Workgroups are dealt to the 8 XCDs round-robin by the hardware; the block index is remapped so that each XCD
+// walks one contiguous range of tiles (one slab of the grid) and its L2 sees the same cells again and again.
+//
 // Reference roles replaced: find_neighbors_cell_list (vesin/src/cuda/cell_list.cu:428-705), brute_force_*
 // (vesin/src/cuda/bruteforce.cu:241-573); CPU twin CellList::foreach_pair + callback
 // (vesin/src/cpu_cell_list.cpp:376-451, :100-163).
 #ifndef VESIN_HIP_SEARCH_CUH
 #define VESIN_HIP_SEARCH_CUH
 
+#include <type_traits>
+
 #include "cells.cuh"
 #include "device_common.cuh"
 
 namespace vesin_hip {
 
-constexpr int MAX_ENTRIES = 512; // stencil entries resident in LDS at a time
+constexpr int SEARCH_WAVES = 4;     // waves per workgroup; every wave works on its own tile, they never synchronise
+constexpr int SEARCH_BLOCK = SEARCH_WAVES * WAVE;
+constexpr int MAX_ENTRIES = 64;    // stencil entries resident in LDS at a time (27 for the usual 3x3x3 stencil)
 constexpr int RING = 128;        // tickets per wave ring (power of two, >= 2 * WAVE)
+constexpr int N_XCD = 8;
 
 struct SearchOutputs {
     unsigned long long* pairs; // [P][2]
@@ -50,10 +60,13 @@ struct SearchArgs {
     SortedPoints sorted;
     const uint64_t* cell_scan; // [n_cells + 1]: points before the cell | (tiles before the cell << 32)
     const Tile* tiles;
-    uint32_t* counts;          // COUNT: [gridDim.x * 4]
-    const uint64_t* offsets;   // WRITE: [gridDim.x * 4 + 1] exclusive scan of counts
+    uint32_t* counts;          // COUNT: [gridDim.x]
+    const uint64_t* offsets;   // WRITE: [gridDim.x + 1] exclusive scan of counts
     SearchOutputs out;
-    uint32_t n_slices;         // workgroups sharing one tile (each takes a slice of the candidates)
+    uint32_t n_slices;         // work items sharing one tile (each takes a slice of the candidates)
+    uint32_t n_work;           // work items = tile slots * n_slices; tile slots are a multiple of
+                               // N_XCD * SEARCH_WAVES and at least the number of tiles. counts / offsets are
+                               // indexed by work item.
 };
 
 __device__ __forceinline__ int32_t pack_shift(int32_t a, int32_t b, int32_t c) {
@@ -91,26 +104,311 @@ __device__ __forceinline__ bool half_keeps_self_image(int32_t sx, int32_t sy, in
     return true;
 }
 
-template <bool WRITE, bool FULL, int R>
-__global__ __launch_bounds__(BLOCK) void search_kernel(SearchArgs args, GridParams g) {
-    __shared__ uint32_t ent_prefix[MAX_ENTRIES + 1]; // candidates before each stencil entry
-    __shared__ uint32_t ent_start[MAX_ENTRIES];      // first sorted position of the entry's cell
-    __shared__ int32_t ent_shift[MAX_ENTRIES];       // packed cell shift, bit 30: same cell as the tile
-    __shared__ uint32_t wave_carry;
-    // tile points, for the redeem phase
-    __shared__ double tile_x[WAVE], tile_y[WAVE], tile_z[WAVE];
-    __shared__ uint32_t tile_index[WAVE];
-    __shared__ int32_t tile_wx[WAVE], tile_wy[WAVE], tile_wz[WAVE];
-    __shared__ uint16_t ring[WRITE ? WAVES_PER_BLOCK : 1][RING];
+/// R x 64 candidates held in registers by one wave.
+template <int R>
+struct Candidates {
+    double x[R], y[R], z[R];    // position (NaN for lanes past the end: never a hit)
+    double tx[R], ty[R], tz[R]; // shift vector against a tile point that was not wrapped
+    int32_t bx[R], by[R], bz[R];// cell shift minus the candidate's own wrap shift
+    uint32_t index[R];          // original index
+    uint32_t self_key[R];       // original index if the candidate is an unshifted member of the tile's cell, else ~0
+    uint32_t image_key[R];      // half lists: original index if the candidate is a shifted member of the tile's cell
+                                // whose shift the half-list rule keeps, else ~0
+    bool any_shift;             // some lane has a non-zero base shift
+    bool any_same;              // some lane is in the tile's own cell
+};
 
-    const int lane = lane_id();
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
-    const uint32_t tile_id = blockIdx.x / args.n_slices;
-    const uint32_t slice = blockIdx.x % args.n_slices;
-    const uint32_t n_tiles = static_cast<uint32_t>(args.cell_scan[g.n_cells] >> 32);
-    const size_t wave_slot = static_cast<size_t>(blockIdx.x) * WAVES_PER_BLOCK + wave;
+/// LDS of one wave. The counting pass only needs the stencil tables (the per-wave footprint decides how many
+/// waves a CU holds).
+struct SearchTables {
+    uint32_t ent_prefix[MAX_ENTRIES + 1]; // candidates before each stencil entry
+    uint32_t ent_start[MAX_ENTRIES];      // first sorted position of the entry's cell
+    int32_t ent_shift[MAX_ENTRIES];       // packed cell shift, bit 30: same cell as the tile
+    uint32_t n_candidates;
+};
 
-    if (tile_id >= n_tiles) {
+struct SearchSharedCount: SearchTables {
+    uint16_t ring[1];
+};
+
+struct SearchSharedWrite: SearchTables {
+    // the tile's points, for the redeem phase
+    double tile_x[WAVE], tile_y[WAVE], tile_z[WAVE];
+    uint32_t tile_index[WAVE];
+    int32_t tile_wx[WAVE], tile_wy[WAVE], tile_wz[WAVE];
+    uint16_t ring[RING];
+};
+
+/// Per-wave progress, kept in scalar registers.
+struct WaveState {
+    uint32_t total;      // COUNT: pairs found so far
+    uint64_t out_cursor; // WRITE: next output row of this wave
+    uint32_t head;       // tickets appended to the ring
+    uint32_t tail;       // tickets redeemed
+};
+
+/// Redeem up to 64 tickets: every lane rebuilds one pair from its ticket and stores one output row.
+template <int R>
+__device__ __forceinline__ void redeem(
+    uint32_t n, WaveState& state, const Candidates<R>& c, SearchSharedWrite& sh, const SearchOutputs& out,
+    const GridParams& g, bool tile_wrapped, int wave, int lane, double zero_tx, double zero_ty, double zero_tz
+) {
+    // tickets were written by other lanes of this wave: LDS operations of one wave complete in order, the fence only
+    // keeps the compiler from moving the read above the writes
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    const bool active = static_cast<uint32_t>(lane) < n;
+    const uint32_t ticket = sh.ring[(state.tail + lane) & (RING - 1)];
+    const int owner = ticket & 63;
+    const int which = (ticket >> 6) & 3;
+    const int il = active ? (ticket >> 8) & 63 : 0;
+    const bool need_shift = c.any_shift || tile_wrapped;
+
+    double xj = 0, yj = 0, zj = 0;
+    int32_t sx = 0, sy = 0, sz = 0;
+    uint32_t oj = 0;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const double px = __shfl(c.x[r], owner);
+        const double py = __shfl(c.y[r], owner);
+        const double pz = __shfl(c.z[r], owner);
+        const uint32_t po = static_cast<uint32_t>(__shfl(static_cast<int>(c.index[r]), owner));
+        int32_t pbx = 0, pby = 0, pbz = 0;
+        if (need_shift) {
+            pbx = __shfl(c.bx[r], owner);
+            pby = __shfl(c.by[r], owner);
+            pbz = __shfl(c.bz[r], owner);
+        }
+        if (R == 1 || which == r) {
+            xj = px;
+            yj = py;
+            zj = pz;
+            sx = pbx;
+            sy = pby;
+            sz = pbz;
+            oj = po;
+        }
+    }
+
+    // the stored vector always adds T, even when S = 0 (T = +-0 then): bit-identical zeros
+    double tx = zero_tx, ty = zero_ty, tz = zero_tz;
+    if (need_shift) {
+        if (tile_wrapped) {
+            sx += sh.tile_wx[il];
+            sy += sh.tile_wy[il];
+            sz += sh.tile_wz[il];
+        }
+        shift_vector(g, sx, sy, sz, tx, ty, tz);
+    }
+    const double vx = (xj - sh.tile_x[il]) + tx;
+    const double vy = (yj - sh.tile_y[il]) + ty;
+    const double vz = (zj - sh.tile_z[il]) + tz;
+
+    if (active) {
+        ulonglong2 pair;
+        pair.x = sh.tile_index[il];
+        pair.y = oj;
+        (reinterpret_cast<ulonglong2*>(out.pairs) + state.out_cursor)[lane] = pair;
+        if (out.shifts != nullptr) {
+            int32_t* s = out.shifts + 3 * state.out_cursor + 3 * lane;
+            s[0] = sx;
+            s[1] = sy;
+            s[2] = sz;
+        }
+        if (out.distances != nullptr) {
+            const double d2 = vx * vx + vy * vy + vz * vz;
+            (out.distances + state.out_cursor)[lane] = sqrt(d2);
+        }
+        if (out.vectors != nullptr) {
+            double* v = out.vectors + 3 * state.out_cursor + 3 * lane;
+            v[0] = vx;
+            v[1] = vy;
+            v[2] = vz;
+        }
+    }
+    state.out_cursor += n;
+    state.tail += n;
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+/// What happens to the hit mask of one (tile point, candidate group).
+template <bool WRITE, int R, typename Shared>
+__device__ __forceinline__ void consume(
+    uint64_t mask, int r, uint32_t i, WaveState& state, const Candidates<R>& c, Shared& sh,
+    const SearchOutputs& out, const GridParams& g, bool tile_wrapped, int wave, int lane, double zero_tx,
+    double zero_ty, double zero_tz
+) {
+    if (mask != 0) {
+        const uint32_t hits = __popcll(mask);
+        if constexpr (WRITE) {
+            if (__builtin_amdgcn_inverse_ballot_w64(mask)) {
+                const uint32_t at = (state.head + rank_in_mask(mask)) & (RING - 1);
+                sh.ring[at] = static_cast<uint16_t>(lane | (r << 6) | (i << 8));
+            }
+            state.head += hits;
+            if (state.head - state.tail >= WAVE) {
+                redeem<R>(WAVE, state, c, sh, out, g, tile_wrapped, wave, lane, zero_tx, zero_ty, zero_tz);
+            }
+        } else {
+            state.total += hits;
+        }
+    }
+}
+
+typedef uint32_t ScalarWords8 __attribute__((ext_vector_type(8)));
+typedef uint32_t ScalarWords4 __attribute__((ext_vector_type(4)));
+
+constexpr int POINTS_PER_LOAD = 4;
+
+/// Coordinates and original indices of four consecutive cell-sorted points, in scalar registers.
+struct FourPoints {
+    ScalarWords8 x, y, z;
+    ScalarWords4 index;
+};
+
+/// Four scalar loads (s_load_dwordx8 x3, s_load_dwordx4) issued back to back and waited for inside one asm
+/// statement, so the compiler never sees the registers before the data arrived. The addresses are wave-uniform.
+/// Reading up to three points past the end of a tile is harmless: the arrays are padded.
+__device__ __forceinline__ FourPoints load_four_points(
+    const double* x, const double* y, const double* z, const uint32_t* index
+) {
+    FourPoints p;
+    asm volatile(
+        "s_load_dwordx8 %0, %4, 0x0\n\t"
+        "s_load_dwordx8 %1, %5, 0x0\n\t"
+        "s_load_dwordx8 %2, %6, 0x0\n\t"
+        "s_load_dwordx4 %3, %7, 0x0\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&s"(p.x), "=&s"(p.y), "=&s"(p.z), "=&s"(p.index)
+        : "s"(x), "s"(y), "s"(z), "s"(index)
+    );
+    return p;
+}
+
+__device__ __forceinline__ double words_to_double(uint32_t lo, uint32_t hi) {
+    return __longlong_as_double(static_cast<long long>((static_cast<uint64_t>(hi) << 32) | lo));
+}
+
+/// Every tile point against the R x 64 candidates, for a tile none of whose points was wrapped: the shift of a
+/// pair is the candidate's base shift. SHIFTED / SAME say what this batch of candidates can contain.
+/// The tile's points come in through scalar loads, four points per round trip, and stay in scalar registers: the
+/// subtraction r_j - r_i takes them as scalar operands.
+template <bool WRITE, bool FULL, int R, bool SHIFTED, bool SAME, typename Shared>
+__device__ __forceinline__ void sweep_unwrapped(
+    const SortedPoints& sorted, uint32_t first_i, uint32_t n_i,
+    WaveState& state, const Candidates<R>& c, Shared& sh, const SearchOutputs& out,
+    const GridParams& g, int wave, int lane, double zero_tx, double zero_ty, double zero_tz
+) {
+    for (uint32_t i0 = 0; i0 < n_i; i0 += POINTS_PER_LOAD) {
+        const uint32_t at = first_i + i0;
+        const FourPoints p = load_four_points(sorted.x + at, sorted.y + at, sorted.z + at, sorted.index + at);
+#pragma unroll
+        for (int u = 0; u < POINTS_PER_LOAD; u++) {
+            if (u > 0 && i0 + u >= n_i) {
+                break;
+            }
+            const uint32_t i = i0 + u;
+            const double xi = words_to_double(p.x[2 * u], p.x[2 * u + 1]);
+            const double yi = words_to_double(p.y[2 * u], p.y[2 * u + 1]);
+            const double zi = words_to_double(p.z[2 * u], p.z[2 * u + 1]);
+            const uint32_t oi = p.index[u];
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                double vx = c.x[r] - xi;
+                double vy = c.y[r] - yi;
+                double vz = c.z[r] - zi;
+                if (SHIFTED) {
+                    vx += c.tx[r];
+                    vy += c.ty[r];
+                    vz += c.tz[r];
+                }
+                const double d2 = vx * vx + vy * vy + vz * vz;
+                // every condition is one compare whose lane mask lands in scalar registers; they are combined there
+                uint64_t mask = __ballot(d2 < g.cutoff2);
+                if (FULL) {
+                    if (SAME) {
+                        mask &= ~__ballot(c.self_key[r] == oi);
+                    }
+                } else {
+                    uint64_t keep = __ballot(oi < c.index[r]);
+                    if (SAME) {
+                        keep |= __ballot(c.image_key[r] == oi);
+                    }
+                    mask &= keep;
+                }
+                consume<WRITE, R>(mask, r, i, state, c, sh, out, g, false, wave, lane, zero_tx, zero_ty, zero_tz);
+            }
+        }
+    }
+}
+
+/// General variant: the tile holds wrapped points, so the shift depends on both points of a pair.
+template <bool WRITE, bool FULL, int R, typename Shared>
+__device__ __forceinline__ void sweep_wrapped(
+    const SortedPoints& sorted, uint32_t first_i, uint32_t n_i,
+    WaveState& state, const Candidates<R>& c, Shared& sh, const SearchOutputs& out,
+    const GridParams& g, int wave, int lane, double zero_tx, double zero_ty, double zero_tz
+) {
+    for (uint32_t i = 0; i < n_i; i++) {
+        const uint32_t at = first_i + i;
+        const double xi = sorted.x[at];
+        const double yi = sorted.y[at];
+        const double zi = sorted.z[at];
+        const uint32_t oi = sorted.index[at];
+        const int32_t wix = sorted.wx[at];
+        const int32_t wiy = sorted.wy[at];
+        const int32_t wiz = sorted.wz[at];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int32_t sx = c.bx[r] + wix;
+            const int32_t sy = c.by[r] + wiy;
+            const int32_t sz = c.bz[r] + wiz;
+            double tx, ty, tz;
+            shift_vector(g, sx, sy, sz, tx, ty, tz);
+            const double vx = (c.x[r] - xi) + tx;
+            const double vy = (c.y[r] - yi) + ty;
+            const double vz = (c.z[r] - zi) + tz;
+            const double d2 = vx * vx + vy * vy + vz * vz;
+            bool hit = d2 < g.cutoff2;
+            const bool zero = (sx | sy | sz) == 0;
+            const bool same_point = c.index[r] == oi;
+            if (FULL) {
+                hit = hit && !(same_point && zero);
+            } else {
+                const bool keep = oi < c.index[r] || (same_point && !zero && half_keeps_self_image(sx, sy, sz));
+                hit = hit && keep;
+            }
+            consume<WRITE, R>(__ballot(hit), r, i, state, c, sh, out, g, true, wave, lane, zero_tx, zero_ty, zero_tz);
+        }
+    }
+}
+
+/// LDS written by some lanes is about to be read by others of the same (only) wave of the workgroup: the
+/// hardware keeps one wave's LDS operations in order, this only stops the compiler from reordering them.
+__device__ __forceinline__ void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+}
+
+/// One work item: one tile (or one slice of its candidates) searched by one wave.
+template <bool WRITE, bool FULL, int R, typename Shared>
+__device__ __forceinline__ void search_work_item(
+    uint32_t work, const SearchArgs& args, const GridParams& g, Shared& sh, uint32_t n_tiles, int lane
+) {
+    const int wave = 0;
+    const uint32_t slice = work % args.n_slices;
+    const size_t wave_slot = work;
+
+    // XCD-aware order: the hardware deals workgroups to the 8 XCDs round-robin, so slot u (wave u % 4 of workgroup
+    // u / 4) runs on XCD (u / 4) % 8; each XCD walks its own contiguous range of tiles
+    const uint32_t slot = work / args.n_slices;
+    const uint32_t per_xcd = (n_tiles + N_XCD - 1) / N_XCD;
+    const uint32_t xcd = (slot / SEARCH_WAVES) % N_XCD;
+    const uint32_t within = (slot / (SEARCH_WAVES * N_XCD)) * SEARCH_WAVES + slot % SEARCH_WAVES;
+    const uint32_t tile_id = xcd * per_xcd + within;
+
+    if (within >= per_xcd || tile_id >= n_tiles) {
         if (!WRITE && lane == 0) {
             args.counts[wave_slot] = 0;
         }
@@ -132,53 +430,60 @@ __global__ __launch_bounds__(BLOCK) void search_kernel(SearchArgs args, GridPara
     const int32_t* __restrict__ pwy = args.sorted.wy;
     const int32_t* __restrict__ pwz = args.sorted.wz;
 
-    if (WRITE && threadIdx.x < n_i) {
-        uint32_t at = first_i + threadIdx.x;
-        tile_x[threadIdx.x] = px[at];
-        tile_y[threadIdx.x] = py[at];
-        tile_z[threadIdx.x] = pz[at];
-        tile_index[threadIdx.x] = pindex[at];
-        tile_wx[threadIdx.x] = pwx[at];
-        tile_wy[threadIdx.x] = pwy[at];
-        tile_wz[threadIdx.x] = pwz[at];
+    if constexpr (WRITE) {
+      if (static_cast<uint32_t>(lane) < n_i) {
+        const uint32_t at = first_i + lane;
+        sh.tile_x[lane] = px[at];
+        sh.tile_y[lane] = py[at];
+        sh.tile_z[lane] = pz[at];
+        sh.tile_index[lane] = pindex[at];
+        sh.tile_wx[lane] = pwx[at];
+        sh.tile_wy[lane] = pwy[at];
+        sh.tile_wz[lane] = pwz[at];
+      }
     }
+    const bool tile_wrapped = tile.wrapped != 0;
 
     const int32_t span_y = 2 * g.s[1] + 1;
     const int32_t span_z = 2 * g.s[2] + 1;
     const uint32_t n_entries = static_cast<uint32_t>(2 * g.s[0] + 1) * span_y * span_z;
 
-    uint32_t wave_total = 0;                 // COUNT
-    uint64_t out_cursor = 0;                 // WRITE: next output row of this wave
-    if (WRITE) {
-        out_cursor = args.offsets[wave_slot];
-    }
+    // shift vector of the zero shift: +0 or -0 per component, depending on the signs in H
+    double zero_tx, zero_ty, zero_tz;
+    shift_vector(g, 0, 0, 0, zero_tx, zero_ty, zero_tz);
+
+    WaveState state;
+    state.total = 0;
+    state.out_cursor = WRITE ? args.offsets[wave_slot] : 0;
+    state.head = 0;
+    state.tail = 0;
 
     for (uint32_t batch = 0; batch < n_entries; batch += MAX_ENTRIES) {
         const uint32_t n_batch = min(static_cast<uint32_t>(MAX_ENTRIES), n_entries - batch);
-        __syncthreads(); // everyone is done with the previous batch's tables (and the tile staging is visible)
+        wave_sync(); // done with the previous batch's tables
 
         // ---- stencil entries of this batch: neighbour cell, its cell shift, how many points it holds
-        for (uint32_t e = threadIdx.x; e < n_batch; e += BLOCK) {
+        for (uint32_t e = lane; e < n_batch; e += WAVE) {
             uint32_t linear = batch + e;
             int32_t dz = static_cast<int32_t>(linear % span_z) - g.s[2];
             int32_t dy = static_cast<int32_t>((linear / span_z) % span_y) - g.s[1];
             int32_t dx = static_cast<int32_t>(linear / (span_z * span_y)) - g.s[0];
-            int32_t c[3] = {cx + dx, cy + dy, cz + dz};
+            int32_t cell[3] = {cx + dx, cy + dy, cz + dz};
             int32_t q[3] = {0, 0, 0};
             bool valid = true;
 #pragma unroll
             for (int d = 0; d < 3; d++) {
                 const int32_t n = g.n[d];
                 if (g.periodic[d]) {
-                    int32_t quotient = c[d] / n;
-                    int32_t rest = c[d] - quotient * n;
+                    int32_t quotient = cell[d] / n;
+                    int32_t rest = cell[d] - quotient * n;
                     if (rest < 0) {
                         rest += n;
                         quotient -= 1;
                     }
                     q[d] = quotient;
-                    c[d] = rest;
-                } else if (c[d] < 0 || c[d] >= n) {
+                    cell[d] = rest;
+                } else if (cell[d] < 0 || cell[d] >= n) {
                     valid = false;
                 }
             }
@@ -186,7 +491,7 @@ __global__ __launch_bounds__(BLOCK) void search_kernel(SearchArgs args, GridPara
             uint32_t count = 0;
             int32_t packed = 0;
             if (valid) {
-                uint32_t neighbour = (static_cast<uint32_t>(c[2]) * g.n[1] + c[1]) * g.n[0] + c[0];
+                uint32_t neighbour = (static_cast<uint32_t>(cell[2]) * g.n[1] + cell[1]) * g.n[0] + cell[0];
                 start = static_cast<uint32_t>(args.cell_scan[neighbour]);
                 count = static_cast<uint32_t>(args.cell_scan[neighbour + 1]) - start;
                 packed = pack_shift(q[0], q[1], q[2]);
@@ -194,234 +499,149 @@ __global__ __launch_bounds__(BLOCK) void search_kernel(SearchArgs args, GridPara
                     packed |= 1 << 30;
                 }
             }
-            ent_start[e] = start;
-            ent_shift[e] = packed;
-            ent_prefix[e + 1] = count; // scanned in place below
+            sh.ent_start[e] = start;
+            sh.ent_shift[e] = packed;
+            sh.ent_prefix[e + 1] = count; // scanned in place below
         }
-        __syncthreads();
+        wave_sync();
 
-        if (wave == 0) {
+        {
             uint32_t carry = 0;
             for (uint32_t base = 0; base < n_batch; base += WAVE) {
                 uint32_t e = base + lane;
-                uint32_t v = e < n_batch ? ent_prefix[e + 1] : 0;
+                uint32_t v = e < n_batch ? sh.ent_prefix[e + 1] : 0;
                 uint32_t inclusive = wave_inclusive_scan(v) + carry;
                 if (e < n_batch) {
-                    ent_prefix[e + 1] = inclusive;
+                    sh.ent_prefix[e + 1] = inclusive;
                 }
                 carry = read_lane(inclusive, WAVE - 1);
             }
             if (lane == 0) {
-                ent_prefix[0] = 0;
-                wave_carry = carry;
+                sh.ent_prefix[0] = 0;
             }
+            sh.n_candidates = carry;
         }
-        __syncthreads();
+        wave_sync();
 
-        const uint32_t n_candidates = wave_carry;
+        const uint32_t n_candidates = __builtin_amdgcn_readfirstlane(sh.n_candidates);
         const uint32_t n_groups = (n_candidates + WAVE * R - 1) / (WAVE * R);
         const uint32_t per_slice = (n_groups + args.n_slices - 1) / args.n_slices;
         const uint32_t group_begin = slice * per_slice;
         const uint32_t group_end = min(n_groups, group_begin + per_slice);
 
-        for (uint32_t group = group_begin + wave; group < group_end; group += WAVES_PER_BLOCK) {
+        for (uint32_t group = group_begin; group < group_end; group++) {
             // ---- load R x 64 candidates into registers
-            double xj[R], yj[R], zj[R];   // position
-            double tx[R], ty[R], tz[R];   // shift vector for a tile point that was not wrapped
-            int32_t bx[R], by[R], bz[R];  // cell shift minus the candidate's own wrap shift
-            uint32_t oj[R];               // original index
-            bool same_cell[R];
-            bool any_shift[R];            // some lane of the group has a non-zero base shift
-            bool any_same[R];             // some lane of the group is in the tile's own cell
-
+            Candidates<R> c;
+            c.any_shift = false;
+            c.any_same = false;
 #pragma unroll
             for (int r = 0; r < R; r++) {
                 const uint32_t k = (group * R + r) * WAVE + lane;
                 const bool valid = k < n_candidates;
-                xj[r] = yj[r] = zj[r] = __builtin_nan("");
-                tx[r] = ty[r] = tz[r] = 0.0;
-                bx[r] = by[r] = bz[r] = 0;
-                oj[r] = 0xFFFFFFFFu;
-                same_cell[r] = false;
+                c.x[r] = c.y[r] = c.z[r] = __builtin_nan("");
+                c.tx[r] = c.ty[r] = c.tz[r] = 0.0;
+                c.bx[r] = c.by[r] = c.bz[r] = 0;
+                c.index[r] = 0xFFFFFFFFu;
+                c.self_key[r] = 0xFFFFFFFFu;
+                c.image_key[r] = 0xFFFFFFFFu;
+                bool same_cell = false;
                 if (valid) {
                     // largest e with ent_prefix[e] <= k
                     uint32_t lo = 0;
                     uint32_t hi = n_batch;
                     while (hi - lo > 1) {
                         uint32_t mid = (lo + hi) >> 1;
-                        if (ent_prefix[mid] <= k) {
+                        if (sh.ent_prefix[mid] <= k) {
                             lo = mid;
                         } else {
                             hi = mid;
                         }
                     }
-                    const uint32_t at = ent_start[lo] + (k - ent_prefix[lo]);
-                    const int32_t packed = ent_shift[lo];
+                    const uint32_t at = sh.ent_start[lo] + (k - sh.ent_prefix[lo]);
+                    const int32_t packed = sh.ent_shift[lo];
                     int32_t qx, qy, qz;
                     unpack_shift(packed, qx, qy, qz);
-                    same_cell[r] = (packed >> 30) & 1;
-                    xj[r] = px[at];
-                    yj[r] = py[at];
-                    zj[r] = pz[at];
-                    oj[r] = pindex[at];
-                    bx[r] = qx - pwx[at];
-                    by[r] = qy - pwy[at];
-                    bz[r] = qz - pwz[at];
-                    shift_vector(g, bx[r], by[r], bz[r], tx[r], ty[r], tz[r]);
+                    same_cell = (packed >> 30) & 1;
+                    c.x[r] = px[at];
+                    c.y[r] = py[at];
+                    c.z[r] = pz[at];
+                    c.index[r] = pindex[at];
+                    c.bx[r] = qx - pwx[at];
+                    c.by[r] = qy - pwy[at];
+                    c.bz[r] = qz - pwz[at];
                 }
-                any_shift[r] = __ballot((bx[r] | by[r] | bz[r]) != 0) != 0;
-                any_same[r] = __ballot(same_cell[r]) != 0;
+                const bool shifted = (c.bx[r] | c.by[r] | c.bz[r]) != 0;
+                if (same_cell) {
+                    if (!shifted) {
+                        c.self_key[r] = c.index[r];
+                    } else if (half_keeps_self_image(c.bx[r], c.by[r], c.bz[r])) {
+                        c.image_key[r] = c.index[r];
+                    }
+                }
+                c.any_shift = c.any_shift || (__ballot(shifted) != 0);
+                c.any_same = c.any_same || (__ballot(same_cell) != 0);
             }
-
-            uint32_t pending_head = 0; // tickets appended / redeemed for this group (ring positions)
-            uint32_t pending_tail = 0;
-
-            // ---- redeem up to 64 tickets: all lanes write one output row each
-            auto redeem = [&](uint32_t n) {
-                __builtin_amdgcn_wave_barrier();
-                const bool active = static_cast<uint32_t>(lane) < n;
-                const uint32_t ticket = static_cast<const volatile uint16_t*>(ring[WRITE ? wave : 0])[(pending_tail + lane) & (RING - 1)];
-                const int owner = ticket & 63;
-                const int which = (ticket >> 6) & 3;
-                const int il = active ? (ticket >> 8) & 63 : 0;
-
-                double cxj = 0, cyj = 0, czj = 0;
-                int32_t cbx = 0, cby = 0, cbz = 0;
-                uint32_t coj = 0;
+            if (c.any_shift) {
 #pragma unroll
                 for (int r = 0; r < R; r++) {
-                    double sx = __shfl(xj[r], owner);
-                    double sy = __shfl(yj[r], owner);
-                    double sz = __shfl(zj[r], owner);
-                    int32_t sbx = __shfl(bx[r], owner);
-                    int32_t sby = __shfl(by[r], owner);
-                    int32_t sbz = __shfl(bz[r], owner);
-                    uint32_t so = static_cast<uint32_t>(__shfl(static_cast<int>(oj[r]), owner));
-                    if (which == r) {
-                        cxj = sx;
-                        cyj = sy;
-                        czj = sz;
-                        cbx = sbx;
-                        cby = sby;
-                        cbz = sbz;
-                        coj = so;
-                    }
-                }
-
-                const int32_t sx = cbx + tile_wx[il];
-                const int32_t sy = cby + tile_wy[il];
-                const int32_t sz = cbz + tile_wz[il];
-                double ttx, tty, ttz;
-                shift_vector(g, sx, sy, sz, ttx, tty, ttz);
-                const double vx = (cxj - tile_x[il]) + ttx;
-                const double vy = (cyj - tile_y[il]) + tty;
-                const double vz = (czj - tile_z[il]) + ttz;
-                const double d2 = vx * vx + vy * vy + vz * vz;
-
-                if (active) {
-                    const uint64_t row = out_cursor + lane;
-                    ulonglong2 pair;
-                    pair.x = tile_index[il];
-                    pair.y = coj;
-                    reinterpret_cast<ulonglong2*>(args.out.pairs)[row] = pair;
-                    if (args.out.shifts != nullptr) {
-                        int32_t* s = args.out.shifts + 3 * row;
-                        s[0] = sx;
-                        s[1] = sy;
-                        s[2] = sz;
-                    }
-                    if (args.out.distances != nullptr) {
-                        args.out.distances[row] = sqrt(d2);
-                    }
-                    if (args.out.vectors != nullptr) {
-                        double* v = args.out.vectors + 3 * row;
-                        v[0] = vx;
-                        v[1] = vy;
-                        v[2] = vz;
-                    }
-                }
-                out_cursor += n;
-                pending_tail += n;
-                __builtin_amdgcn_wave_barrier();
-            };
-
-            // ---- every tile point against the R x 64 candidates
-            for (uint32_t i = 0; i < n_i; i++) {
-                const uint32_t at = first_i + i;
-                const double xi = px[at];
-                const double yi = py[at];
-                const double zi = pz[at];
-                const uint32_t oi = pindex[at];
-                const int32_t wix = pwx[at];
-                const int32_t wiy = pwy[at];
-                const int32_t wiz = pwz[at];
-                const bool i_wrapped = (wix | wiy | wiz) != 0;
-
-#pragma unroll
-                for (int r = 0; r < R; r++) {
-                    double vx = xj[r] - xi;
-                    double vy = yj[r] - yi;
-                    double vz = zj[r] - zi;
-                    if (i_wrapped) {
-                        double ttx, tty, ttz;
-                        shift_vector(g, bx[r] + wix, by[r] + wiy, bz[r] + wiz, ttx, tty, ttz);
-                        vx += ttx;
-                        vy += tty;
-                        vz += ttz;
-                    } else if (any_shift[r]) {
-                        vx += tx[r];
-                        vy += ty[r];
-                        vz += tz[r];
-                    }
-                    const double d2 = vx * vx + vy * vy + vz * vz;
-                    bool hit = d2 < g.cutoff2;
-
-                    if (FULL) {
-                        if (any_same[r]) {
-                            // a point is not its own neighbour unless a non-zero shift separates the two
-                            const bool zero = ((bx[r] + wix) | (by[r] + wiy) | (bz[r] + wiz)) == 0;
-                            hit = hit && !(oj[r] == oi && zero);
-                        }
-                    } else {
-                        bool keep = oi < oj[r];
-                        if (any_same[r]) {
-                            const int32_t sx = bx[r] + wix;
-                            const int32_t sy = by[r] + wiy;
-                            const int32_t sz = bz[r] + wiz;
-                            const bool zero = (sx | sy | sz) == 0;
-                            keep = keep || (oj[r] == oi && !zero && half_keeps_self_image(sx, sy, sz));
-                        }
-                        hit = hit && keep;
-                    }
-
-                    const uint64_t mask = __ballot(hit);
-                    if (mask != 0) {
-                        const uint32_t hits = __popcll(mask);
-                        if (WRITE) {
-                            if (hit) {
-                                const uint32_t slot = (pending_head + rank_in_mask(mask)) & (RING - 1);
-                                static_cast<volatile uint16_t*>(ring[wave])[slot] =
-                                    static_cast<uint16_t>(lane | (r << 6) | (i << 8));
-                            }
-                            pending_head += hits;
-                            if (pending_head - pending_tail >= WAVE) {
-                                redeem(WAVE);
-                            }
-                        } else {
-                            wave_total += hits;
-                        }
-                    }
+                    shift_vector(g, c.bx[r], c.by[r], c.bz[r], c.tx[r], c.ty[r], c.tz[r]);
                 }
             }
 
-            if (WRITE && pending_head != pending_tail) {
-                redeem(pending_head - pending_tail);
+            state.head = 0;
+            state.tail = 0;
+
+#define VESIN_SWEEP(SHIFTED, SAME)                                                                                    \
+    sweep_unwrapped<WRITE, FULL, R, SHIFTED, SAME>(                                                                   \
+        args.sorted, first_i, n_i, state, c, sh, args.out, g, wave, lane, zero_tx, zero_ty, zero_tz                   \
+    )
+            if (tile_wrapped) {
+                sweep_wrapped<WRITE, FULL, R>(
+                    args.sorted, first_i, n_i, state, c, sh, args.out, g, wave, lane, zero_tx, zero_ty, zero_tz
+                );
+            } else if (c.any_shift) {
+                if (c.any_same) {
+                    VESIN_SWEEP(true, true);
+                } else {
+                    VESIN_SWEEP(true, false);
+                }
+            } else {
+                if (c.any_same) {
+                    VESIN_SWEEP(false, true);
+                } else {
+                    VESIN_SWEEP(false, false);
+                }
+            }
+#undef VESIN_SWEEP
+
+            // the candidates leave the registers with this group: redeem what is left
+            if constexpr (WRITE) {
+                if (state.head != state.tail) {
+                    redeem<R>(
+                        state.head - state.tail, state, c, sh, args.out, g, tile_wrapped, wave, lane, zero_tx, zero_ty,
+                        zero_tz
+                    );
+                }
             }
         }
     }
 
     if (!WRITE && lane == 0) {
-        args.counts[wave_slot] = wave_total;
+        args.counts[wave_slot] = state.total;
+    }
+}
+
+/// Four independent waves per workgroup, one work item each (single-wave workgroups would cap the number of
+/// waves a CU holds well below what the registers allow).
+template <bool WRITE, bool FULL, int R>
+__global__ __launch_bounds__(SEARCH_BLOCK) void search_kernel(SearchArgs args, GridParams g) {
+    __shared__ std::conditional_t<WRITE, SearchSharedWrite, SearchSharedCount> shared[SEARCH_WAVES];
+    const int lane = lane_id();
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    const uint32_t n_tiles = static_cast<uint32_t>(args.cell_scan[g.n_cells] >> 32);
+    const uint32_t work = blockIdx.x * SEARCH_WAVES + wave;
+    if (work < args.n_work) {
+        search_work_item<WRITE, FULL, R>(work, args, g, shared[wave], n_tiles, lane);
     }
 }
 
