@@ -10,7 +10,6 @@
 #include <cerrno>
 #include <cmath>
 #include <cstdlib>
-#include <cstdio>
 #include <cstring>
 
 #include <atomic>
@@ -237,14 +236,6 @@ void launch_search(bool full, const SearchArgs& args, const GridParams& g, hipSt
         return;
     }
     constexpr int R = 2;
-    if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
-        int a = -1, b = -1;
-        (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&a, search_kernel<WRITE, true, R>, SEARCH_BLOCK, 0);
-        (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&b, search_kernel<WRITE, false, R>, SEARCH_BLOCK, 0);
-        hipFuncAttributes attr;
-        (void)hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(search_kernel<WRITE, true, R>));
-        fprintf(stderr, "search<%d>: blocks/CU full=%d half=%d regs=%d lds=%zu\n", int(WRITE), a, b, attr.numRegs, attr.sharedSizeBytes);
-    }
     const uint32_t blocks = (args.n_work + SEARCH_WAVES - 1) / SEARCH_WAVES;
     if (full) {
         hipLaunchKernelGGL((search_kernel<WRITE, true, R>), dim3(blocks), dim3(SEARCH_BLOCK), 0, stream, args, g);

@@ -1,17 +1,19 @@
 // Stencil search over the cell grid: the kernel that decides pair membership and produces the output arrays.
 //
-// One workgroup (4 waves) owns one tile = up to 64 points `i` of one cell. The candidates `j` are the points of
-// every cell in the (2s+1)^3 stencil around that cell, periodic images included (a cell may appear several
-// times with different cell shifts when the box is narrower than the stencil: that is the multi-image path; with a
-// single cell the stencil enumerates images only and the kernel is a tiled brute force, optionally split over
-// several workgroups per tile).
+// One wave owns one tile = up to 64 points `i` of one cell. The candidates `j` are the points of the cells in
+// the upper half of the (2s+1)^3 stencil around that cell (offsets that are lexicographically positive, plus the
+// cell itself restricted to later points), periodic images included: every unordered pair {(i, j, S), (j, i, -S)}
+// is tested exactly once, by the tile of one of its two points, and both rows are produced from that one test.
+// A cell may appear several times in the stencil with different cell shifts when the box is narrower than the
+// stencil: that is the multi-image path; with a single cell the stencil enumerates images only and the kernel is
+// a tiled brute force, the candidates of a tile being sliced over several waves.
 //
 // Mapping: lanes hold candidates. A wave loads R groups of 64 consecutive candidates into registers (coalesced
-// reads from the cell-sorted structure-of-arrays), then loops over the tile's points `i`, whose coordinates come
-// in through scalar loads issued one iteration ahead. Each (i, group) test is 9 fp64 VALU operations (12 when a
-// shift vector has to be added) and yields a 64-bit hit mask in scalar registers. The loop is compiled in four
-// variants (candidates shifted or not, tile's own cell among them or not), picked per group batch, plus a general
-// variant for tiles holding points that were wrapped into the box.
+// reads from the cell-sorted structure-of-arrays), then loops over the tile's points, whose coordinates come in
+// through scalar loads (four points per round trip) and are used as scalar operands. One (i, group) test is 9 fp64
+// VALU operations (12 when a shift vector has to be added) and yields a 64-bit hit mask in scalar registers. The
+// loop is compiled in four variants (candidates shifted or not, tile's own cell among them or not), picked per
+// group batch, plus a general variant for tiles holding points that were wrapped into the box.
 //
 // The same code runs twice:
 //   COUNT  adds up popcounts: one 32-bit total per wave, no atomics;
@@ -19,15 +21,18 @@
 //          compacts: hit lanes drop a 16-bit ticket (lane, group, i) into a per-wave LDS ring at the slot given by
 //          mbcnt of the mask; whenever 64 tickets are pending, all 64 lanes redeem one each, pulling the
 //          candidate's data out of the owning lane with ds_bpermute, recomputing shift / vector / distance and
-//          storing 64 consecutive output rows.
+//          storing the rows: (i, j, S) and its mirror (j, i, -S) for a full list, the one of the two that the
+//          half-list rule keeps otherwise. A wave's rows are consecutive in the output.
 //
 // Arithmetic (bit-for-bit the CPU reference, vesin/src/cpu_cell_list.cpp:135-138 and vesin/src/types.hpp:232-243,
 // vesin/src/math.hpp:14-16,111-117; compile with -ffp-contract=off):
 //   T_k = S0*H0k + S1*H1k + S2*H2k (left to right), v_k = (r_jk - r_ik) + T_k, d2 = v0*v0 + v1*v1 + v2*v2,
 //   keep iff d2 < cutoff*cutoff, d = sqrt(d2).
 // Adding T may be skipped in the test when S = 0 (it is +-0 and cannot change d2); the stored vector always adds it.
+// The mirror row is exact as well: r_i - r_j and T(-S) are the exact negations of r_j - r_i and T(S) (T(0) is not
+// negated), so d2 is the same number and the vector is recomputed as (r_i - r_j) + T(-S).
 //
-// Workgroups are dealt to the 8 XCDs round-robin by the hardware; the block index is remapped so that each XCD
+// Workgroups are dealt to the 8 XCDs round-robin by the hardware; the work index is remapped so that each XCD
 // walks one contiguous range of tiles (one slab of the grid) and its L2 sees the same cells again and again.
 //
 // Reference roles replaced: find_neighbors_cell_list (vesin/src/cuda/cell_list.cu:428-705), brute_force_*
@@ -43,10 +48,10 @@
 
 namespace vesin_hip {
 
-constexpr int SEARCH_WAVES = 4;     // waves per workgroup; every wave works on its own tile, they never synchronise
+constexpr int SEARCH_WAVES = 4;    // waves per workgroup; every wave works on its own tile, they never synchronise
 constexpr int SEARCH_BLOCK = SEARCH_WAVES * WAVE;
-constexpr int MAX_ENTRIES = 64;    // stencil entries resident in LDS at a time (27 for the usual 3x3x3 stencil)
-constexpr int RING = 128;        // tickets per wave ring (power of two, >= 2 * WAVE)
+constexpr int MAX_ENTRIES = 64;    // stencil entries resident in LDS at a time (14 for the usual 3x3x3 stencil)
+constexpr int RING = 128;          // tickets per wave ring (power of two, >= 2 * WAVE)
 constexpr int N_XCD = 8;
 
 struct SearchOutputs {
@@ -60,13 +65,12 @@ struct SearchArgs {
     SortedPoints sorted;
     const uint64_t* cell_scan; // [n_cells + 1]: points before the cell | (tiles before the cell << 32)
     const Tile* tiles;
-    uint32_t* counts;          // COUNT: [gridDim.x]
-    const uint64_t* offsets;   // WRITE: [gridDim.x + 1] exclusive scan of counts
+    uint32_t* counts;          // COUNT: rows produced by every work item
+    const uint64_t* offsets;   // WRITE: exclusive scan of counts
     SearchOutputs out;
     uint32_t n_slices;         // work items sharing one tile (each takes a slice of the candidates)
     uint32_t n_work;           // work items = tile slots * n_slices; tile slots are a multiple of
-                               // N_XCD * SEARCH_WAVES and at least the number of tiles. counts / offsets are
-                               // indexed by work item.
+                               // N_XCD * SEARCH_WAVES and at least the number of tiles
 };
 
 __device__ __forceinline__ int32_t pack_shift(int32_t a, int32_t b, int32_t c) {
@@ -110,20 +114,17 @@ struct Candidates {
     double x[R], y[R], z[R];    // position (NaN for lanes past the end: never a hit)
     double tx[R], ty[R], tz[R]; // shift vector against a tile point that was not wrapped
     int32_t bx[R], by[R], bz[R];// cell shift minus the candidate's own wrap shift
-    uint32_t index[R];          // original index
-    uint32_t self_key[R];       // original index if the candidate is an unshifted member of the tile's cell, else ~0
-    uint32_t image_key[R];      // half lists: original index if the candidate is a shifted member of the tile's cell
-                                // whose shift the half-list rule keeps, else ~0
+    uint32_t position[R];       // position in the cell-sorted arrays if the candidate comes from the tile's own
+                                // cell with a zero cell shift (only later points are partners), else ~0
     bool any_shift;             // some lane has a non-zero base shift
-    bool any_same;              // some lane is in the tile's own cell
+    bool any_same;              // some lane comes from the tile's own, unshifted cell
 };
 
-/// LDS of one wave. The counting pass only needs the stencil tables (the per-wave footprint decides how many
-/// waves a CU holds).
+/// LDS of one wave. The counting pass only needs the stencil tables.
 struct SearchTables {
     uint32_t ent_prefix[MAX_ENTRIES + 1]; // candidates before each stencil entry
     uint32_t ent_start[MAX_ENTRIES];      // first sorted position of the entry's cell
-    int32_t ent_shift[MAX_ENTRIES];       // packed cell shift, bit 30: same cell as the tile
+    int32_t ent_shift[MAX_ENTRIES];       // packed cell shift, bit 30: the tile's own cell with a zero cell shift
     uint32_t n_candidates;
 };
 
@@ -131,124 +132,182 @@ struct SearchSharedCount: SearchTables {
     uint16_t ring[1];
 };
 
+constexpr int MAX_R = 2;
+
 struct SearchSharedWrite: SearchTables {
     // the tile's points, for the redeem phase
     double tile_x[WAVE], tile_y[WAVE], tile_z[WAVE];
     uint32_t tile_index[WAVE];
     int32_t tile_wx[WAVE], tile_wy[WAVE], tile_wz[WAVE];
+    // the candidates currently held in registers, where any lane can fetch them when it redeems a ticket
+    double cand_x[MAX_R * WAVE], cand_y[MAX_R * WAVE], cand_z[MAX_R * WAVE];
+    uint32_t cand_index[MAX_R * WAVE];
+    int32_t cand_bx[MAX_R * WAVE], cand_by[MAX_R * WAVE], cand_bz[MAX_R * WAVE];
     uint16_t ring[RING];
 };
 
 /// Per-wave progress, kept in scalar registers.
 struct WaveState {
-    uint32_t total;      // COUNT: pairs found so far
+    uint32_t total;      // COUNT: hits found so far
     uint64_t out_cursor; // WRITE: next output row of this wave
     uint32_t head;       // tickets appended to the ring
     uint32_t tail;       // tickets redeemed
 };
 
-/// Redeem up to 64 tickets: every lane rebuilds one pair from its ticket and stores one output row.
-template <int R>
+/// Constants of one work item.
+struct SweepContext {
+    double zero_tx, zero_ty, zero_tz; // shift vector of the zero shift: +0 or -0 per component
+    bool tile_wrapped;
+    int lane;
+};
+
+/// Redeem up to 64 tickets: every lane rebuilds one pair from its ticket and stores its row(s).
+template <bool FULL, int R>
 __device__ __forceinline__ void redeem(
     uint32_t n, WaveState& state, const Candidates<R>& c, SearchSharedWrite& sh, const SearchOutputs& out,
-    const GridParams& g, bool tile_wrapped, int wave, int lane, double zero_tx, double zero_ty, double zero_tz
+    const GridParams& g, const SweepContext& ctx
 ) {
     // tickets were written by other lanes of this wave: LDS operations of one wave complete in order, the fence only
     // keeps the compiler from moving the read above the writes
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
+    const int lane = ctx.lane;
     const bool active = static_cast<uint32_t>(lane) < n;
     const uint32_t ticket = sh.ring[(state.tail + lane) & (RING - 1)];
-    const int owner = ticket & 63;
-    const int which = (ticket >> 6) & 3;
+    const int slot = active ? ticket & (MAX_R * WAVE - 1) : 0; // group r, lane l -> r * 64 + l
     const int il = active ? (ticket >> 8) & 63 : 0;
-    const bool need_shift = c.any_shift || tile_wrapped;
+    const bool need_shift = c.any_shift || ctx.tile_wrapped;
 
-    double xj = 0, yj = 0, zj = 0;
+    const double xj = sh.cand_x[slot];
+    const double yj = sh.cand_y[slot];
+    const double zj = sh.cand_z[slot];
+    const uint32_t oj = sh.cand_index[slot];
     int32_t sx = 0, sy = 0, sz = 0;
-    uint32_t oj = 0;
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-        const double px = __shfl(c.x[r], owner);
-        const double py = __shfl(c.y[r], owner);
-        const double pz = __shfl(c.z[r], owner);
-        const uint32_t po = static_cast<uint32_t>(__shfl(static_cast<int>(c.index[r]), owner));
-        int32_t pbx = 0, pby = 0, pbz = 0;
-        if (need_shift) {
-            pbx = __shfl(c.bx[r], owner);
-            pby = __shfl(c.by[r], owner);
-            pbz = __shfl(c.bz[r], owner);
-        }
-        if (R == 1 || which == r) {
-            xj = px;
-            yj = py;
-            zj = pz;
-            sx = pbx;
-            sy = pby;
-            sz = pbz;
-            oj = po;
-        }
+    if (need_shift) {
+        sx = sh.cand_bx[slot];
+        sy = sh.cand_by[slot];
+        sz = sh.cand_bz[slot];
     }
 
-    // the stored vector always adds T, even when S = 0 (T = +-0 then): bit-identical zeros
-    double tx = zero_tx, ty = zero_ty, tz = zero_tz;
+    const double xi = sh.tile_x[il];
+    const double yi = sh.tile_y[il];
+    const double zi = sh.tile_z[il];
+    const uint32_t oi = sh.tile_index[il];
+
+    // the stored vector always adds T, even when S = 0 (T = +-0 then): bit-identical zeros.
+    // (tx, ty, tz) = T(S); (mx, my, mz) = T(-S), which is -T(S) exactly unless S = 0
+    double tx = ctx.zero_tx, ty = ctx.zero_ty, tz = ctx.zero_tz;
+    double mx = ctx.zero_tx, my = ctx.zero_ty, mz = ctx.zero_tz;
     if (need_shift) {
-        if (tile_wrapped) {
+        if (ctx.tile_wrapped) {
             sx += sh.tile_wx[il];
             sy += sh.tile_wy[il];
             sz += sh.tile_wz[il];
         }
         shift_vector(g, sx, sy, sz, tx, ty, tz);
+        if ((sx | sy | sz) != 0) {
+            mx = -tx;
+            my = -ty;
+            mz = -tz;
+        }
     }
-    const double vx = (xj - sh.tile_x[il]) + tx;
-    const double vy = (yj - sh.tile_y[il]) + ty;
-    const double vz = (zj - sh.tile_z[il]) + tz;
+    const double vx = (xj - xi) + tx;
+    const double vy = (yj - yi) + ty;
+    const double vz = (zj - zi) + tz;
+    const double wx = (xi - xj) + mx;
+    const double wy = (yi - yj) + my;
+    const double wz = (zi - zj) + mz;
+    const double d2 = vx * vx + vy * vy + vz * vz;
 
-    if (active) {
-        ulonglong2 pair;
-        pair.x = sh.tile_index[il];
-        pair.y = oj;
-        (reinterpret_cast<ulonglong2*>(out.pairs) + state.out_cursor)[lane] = pair;
-        if (out.shifts != nullptr) {
-            int32_t* s = out.shifts + 3 * state.out_cursor + 3 * lane;
-            s[0] = sx;
-            s[1] = sy;
-            s[2] = sz;
+    if (FULL) {
+        // two rows per ticket: the n pairs first, then their n mirrors, so that every store instruction of the
+        // wave covers one dense, contiguous range
+        if (active) {
+            const uint64_t forward_row = state.out_cursor + lane;
+            const uint64_t mirror_row = forward_row + n;
+            ulonglong2 forward, backward;
+            forward.x = oi;
+            forward.y = oj;
+            backward.x = oj;
+            backward.y = oi;
+            reinterpret_cast<ulonglong2*>(out.pairs)[forward_row] = forward;
+            reinterpret_cast<ulonglong2*>(out.pairs)[mirror_row] = backward;
+            if (out.shifts != nullptr) {
+                int32_t* s = out.shifts + 3 * forward_row;
+                s[0] = sx;
+                s[1] = sy;
+                s[2] = sz;
+                int32_t* m = out.shifts + 3 * mirror_row;
+                m[0] = -sx;
+                m[1] = -sy;
+                m[2] = -sz;
+            }
+            if (out.distances != nullptr) {
+                const double d = sqrt(d2);
+                out.distances[forward_row] = d;
+                out.distances[mirror_row] = d;
+            }
+            if (out.vectors != nullptr) {
+                double* v = out.vectors + 3 * forward_row;
+                v[0] = vx;
+                v[1] = vy;
+                v[2] = vz;
+                double* m = out.vectors + 3 * mirror_row;
+                m[0] = wx;
+                m[1] = wy;
+                m[2] = wz;
+            }
         }
-        if (out.distances != nullptr) {
-            const double d2 = vx * vx + vy * vy + vz * vz;
-            (out.distances + state.out_cursor)[lane] = sqrt(d2);
+        state.out_cursor += 2 * n;
+    } else {
+        // one row per ticket, oriented like the reference's half list: smaller original index first; a point with
+        // its own image keeps the shift the half-list rule accepts
+        const bool flip = oi > oj || (oi == oj && !half_keeps_self_image(sx, sy, sz));
+        if (active) {
+            const uint64_t row = state.out_cursor + lane;
+            ulonglong2 pair;
+            pair.x = flip ? oj : oi;
+            pair.y = flip ? oi : oj;
+            reinterpret_cast<ulonglong2*>(out.pairs)[row] = pair;
+            if (out.shifts != nullptr) {
+                int32_t* s = out.shifts + 3 * row;
+                s[0] = flip ? -sx : sx;
+                s[1] = flip ? -sy : sy;
+                s[2] = flip ? -sz : sz;
+            }
+            if (out.distances != nullptr) {
+                out.distances[row] = sqrt(d2);
+            }
+            if (out.vectors != nullptr) {
+                double* v = out.vectors + 3 * row;
+                v[0] = flip ? wx : vx;
+                v[1] = flip ? wy : vy;
+                v[2] = flip ? wz : vz;
+            }
         }
-        if (out.vectors != nullptr) {
-            double* v = out.vectors + 3 * state.out_cursor + 3 * lane;
-            v[0] = vx;
-            v[1] = vy;
-            v[2] = vz;
-        }
+        state.out_cursor += n;
     }
-    state.out_cursor += n;
     state.tail += n;
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
 }
 
 /// What happens to the hit mask of one (tile point, candidate group).
-template <bool WRITE, int R, typename Shared>
+template <bool WRITE, bool FULL, int R, typename Shared>
 __device__ __forceinline__ void consume(
-    uint64_t mask, int r, uint32_t i, WaveState& state, const Candidates<R>& c, Shared& sh,
-    const SearchOutputs& out, const GridParams& g, bool tile_wrapped, int wave, int lane, double zero_tx,
-    double zero_ty, double zero_tz
+    uint64_t mask, int r, uint32_t i, WaveState& state, const Candidates<R>& c, Shared& sh, const SearchOutputs& out,
+    const GridParams& g, const SweepContext& ctx
 ) {
     if (mask != 0) {
         const uint32_t hits = __popcll(mask);
         if constexpr (WRITE) {
             if (__builtin_amdgcn_inverse_ballot_w64(mask)) {
                 const uint32_t at = (state.head + rank_in_mask(mask)) & (RING - 1);
-                sh.ring[at] = static_cast<uint16_t>(lane | (r << 6) | (i << 8));
+                sh.ring[at] = static_cast<uint16_t>(ctx.lane | (r << 6) | (i << 8));
             }
             state.head += hits;
             if (state.head - state.tail >= WAVE) {
-                redeem<R>(WAVE, state, c, sh, out, g, tile_wrapped, wave, lane, zero_tx, zero_ty, zero_tz);
+                redeem<FULL, R>(WAVE, state, c, sh, out, g, ctx);
             }
         } else {
             state.total += hits;
@@ -257,31 +316,26 @@ __device__ __forceinline__ void consume(
 }
 
 typedef uint32_t ScalarWords8 __attribute__((ext_vector_type(8)));
-typedef uint32_t ScalarWords4 __attribute__((ext_vector_type(4)));
 
 constexpr int POINTS_PER_LOAD = 4;
 
-/// Coordinates and original indices of four consecutive cell-sorted points, in scalar registers.
+/// Coordinates of four consecutive cell-sorted points, in scalar registers.
 struct FourPoints {
     ScalarWords8 x, y, z;
-    ScalarWords4 index;
 };
 
-/// Four scalar loads (s_load_dwordx8 x3, s_load_dwordx4) issued back to back and waited for inside one asm
-/// statement, so the compiler never sees the registers before the data arrived. The addresses are wave-uniform.
-/// Reading up to three points past the end of a tile is harmless: the arrays are padded.
-__device__ __forceinline__ FourPoints load_four_points(
-    const double* x, const double* y, const double* z, const uint32_t* index
-) {
+/// Three scalar loads (s_load_dwordx8) issued back to back and waited for inside one asm statement, so the
+/// compiler never sees the registers before the data arrived. The addresses are wave-uniform. Reading up to three
+/// points past the end of a tile is harmless: the arrays are padded.
+__device__ __forceinline__ FourPoints load_four_points(const double* x, const double* y, const double* z) {
     FourPoints p;
     asm volatile(
-        "s_load_dwordx8 %0, %4, 0x0\n\t"
-        "s_load_dwordx8 %1, %5, 0x0\n\t"
-        "s_load_dwordx8 %2, %6, 0x0\n\t"
-        "s_load_dwordx4 %3, %7, 0x0\n\t"
+        "s_load_dwordx8 %0, %3, 0x0\n\t"
+        "s_load_dwordx8 %1, %4, 0x0\n\t"
+        "s_load_dwordx8 %2, %5, 0x0\n\t"
         "s_waitcnt lgkmcnt(0)"
-        : "=&s"(p.x), "=&s"(p.y), "=&s"(p.z), "=&s"(p.index)
-        : "s"(x), "s"(y), "s"(z), "s"(index)
+        : "=&s"(p.x), "=&s"(p.y), "=&s"(p.z)
+        : "s"(x), "s"(y), "s"(z)
     );
     return p;
 }
@@ -292,17 +346,15 @@ __device__ __forceinline__ double words_to_double(uint32_t lo, uint32_t hi) {
 
 /// Every tile point against the R x 64 candidates, for a tile none of whose points was wrapped: the shift of a
 /// pair is the candidate's base shift. SHIFTED / SAME say what this batch of candidates can contain.
-/// The tile's points come in through scalar loads, four points per round trip, and stay in scalar registers: the
-/// subtraction r_j - r_i takes them as scalar operands.
 template <bool WRITE, bool FULL, int R, bool SHIFTED, bool SAME, typename Shared>
 __device__ __forceinline__ void sweep_unwrapped(
     const SortedPoints& sorted, uint32_t first_i, uint32_t n_i,
     WaveState& state, const Candidates<R>& c, Shared& sh, const SearchOutputs& out,
-    const GridParams& g, int wave, int lane, double zero_tx, double zero_ty, double zero_tz
+    const GridParams& g, const SweepContext& ctx
 ) {
     for (uint32_t i0 = 0; i0 < n_i; i0 += POINTS_PER_LOAD) {
         const uint32_t at = first_i + i0;
-        const FourPoints p = load_four_points(sorted.x + at, sorted.y + at, sorted.z + at, sorted.index + at);
+        const FourPoints p = load_four_points(sorted.x + at, sorted.y + at, sorted.z + at);
 #pragma unroll
         for (int u = 0; u < POINTS_PER_LOAD; u++) {
             if (u > 0 && i0 + u >= n_i) {
@@ -312,7 +364,6 @@ __device__ __forceinline__ void sweep_unwrapped(
             const double xi = words_to_double(p.x[2 * u], p.x[2 * u + 1]);
             const double yi = words_to_double(p.y[2 * u], p.y[2 * u + 1]);
             const double zi = words_to_double(p.z[2 * u], p.z[2 * u + 1]);
-            const uint32_t oi = p.index[u];
 #pragma unroll
             for (int r = 0; r < R; r++) {
                 double vx = c.x[r] - xi;
@@ -324,20 +375,13 @@ __device__ __forceinline__ void sweep_unwrapped(
                     vz += c.tz[r];
                 }
                 const double d2 = vx * vx + vy * vy + vz * vz;
-                // every condition is one compare whose lane mask lands in scalar registers; they are combined there
+                // each condition is one compare whose lane mask lands in scalar registers; they are combined there
                 uint64_t mask = __ballot(d2 < g.cutoff2);
-                if (FULL) {
-                    if (SAME) {
-                        mask &= ~__ballot(c.self_key[r] == oi);
-                    }
-                } else {
-                    uint64_t keep = __ballot(oi < c.index[r]);
-                    if (SAME) {
-                        keep |= __ballot(c.image_key[r] == oi);
-                    }
-                    mask &= keep;
+                if (SAME) {
+                    // inside the tile's own cell only later points are partners (earlier ones find this point)
+                    mask &= __ballot(c.position[r] > at + u);
                 }
-                consume<WRITE, R>(mask, r, i, state, c, sh, out, g, false, wave, lane, zero_tx, zero_ty, zero_tz);
+                consume<WRITE, FULL, R>(mask, r, i, state, c, sh, out, g, ctx);
             }
         }
     }
@@ -348,44 +392,32 @@ template <bool WRITE, bool FULL, int R, typename Shared>
 __device__ __forceinline__ void sweep_wrapped(
     const SortedPoints& sorted, uint32_t first_i, uint32_t n_i,
     WaveState& state, const Candidates<R>& c, Shared& sh, const SearchOutputs& out,
-    const GridParams& g, int wave, int lane, double zero_tx, double zero_ty, double zero_tz
+    const GridParams& g, const SweepContext& ctx
 ) {
     for (uint32_t i = 0; i < n_i; i++) {
         const uint32_t at = first_i + i;
         const double xi = sorted.x[at];
         const double yi = sorted.y[at];
         const double zi = sorted.z[at];
-        const uint32_t oi = sorted.index[at];
         const int32_t wix = sorted.wx[at];
         const int32_t wiy = sorted.wy[at];
         const int32_t wiz = sorted.wz[at];
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            const int32_t sx = c.bx[r] + wix;
-            const int32_t sy = c.by[r] + wiy;
-            const int32_t sz = c.bz[r] + wiz;
             double tx, ty, tz;
-            shift_vector(g, sx, sy, sz, tx, ty, tz);
+            shift_vector(g, c.bx[r] + wix, c.by[r] + wiy, c.bz[r] + wiz, tx, ty, tz);
             const double vx = (c.x[r] - xi) + tx;
             const double vy = (c.y[r] - yi) + ty;
             const double vz = (c.z[r] - zi) + tz;
             const double d2 = vx * vx + vy * vy + vz * vz;
-            bool hit = d2 < g.cutoff2;
-            const bool zero = (sx | sy | sz) == 0;
-            const bool same_point = c.index[r] == oi;
-            if (FULL) {
-                hit = hit && !(same_point && zero);
-            } else {
-                const bool keep = oi < c.index[r] || (same_point && !zero && half_keeps_self_image(sx, sy, sz));
-                hit = hit && keep;
-            }
-            consume<WRITE, R>(__ballot(hit), r, i, state, c, sh, out, g, true, wave, lane, zero_tx, zero_ty, zero_tz);
+            const uint64_t mask = __ballot(d2 < g.cutoff2) & __ballot(c.position[r] > at);
+            consume<WRITE, FULL, R>(mask, r, i, state, c, sh, out, g, ctx);
         }
     }
 }
 
-/// LDS written by some lanes is about to be read by others of the same (only) wave of the workgroup: the
-/// hardware keeps one wave's LDS operations in order, this only stops the compiler from reordering them.
+/// LDS written by some lanes is about to be read by others of the same wave: the hardware keeps one wave's LDS
+/// operations in order, this only stops the compiler from reordering them.
 __device__ __forceinline__ void wave_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
     __builtin_amdgcn_wave_barrier();
@@ -396,9 +428,7 @@ template <bool WRITE, bool FULL, int R, typename Shared>
 __device__ __forceinline__ void search_work_item(
     uint32_t work, const SearchArgs& args, const GridParams& g, Shared& sh, uint32_t n_tiles, int lane
 ) {
-    const int wave = 0;
     const uint32_t slice = work % args.n_slices;
-    const size_t wave_slot = work;
 
     // XCD-aware order: the hardware deals workgroups to the 8 XCDs round-robin, so slot u (wave u % 4 of workgroup
     // u / 4) runs on XCD (u / 4) % 8; each XCD walks its own contiguous range of tiles
@@ -410,7 +440,7 @@ __device__ __forceinline__ void search_work_item(
 
     if (within >= per_xcd || tile_id >= n_tiles) {
         if (!WRITE && lane == 0) {
-            args.counts[wave_slot] = 0;
+            args.counts[work] = 0;
         }
         return;
     }
@@ -431,30 +461,34 @@ __device__ __forceinline__ void search_work_item(
     const int32_t* __restrict__ pwz = args.sorted.wz;
 
     if constexpr (WRITE) {
-      if (static_cast<uint32_t>(lane) < n_i) {
-        const uint32_t at = first_i + lane;
-        sh.tile_x[lane] = px[at];
-        sh.tile_y[lane] = py[at];
-        sh.tile_z[lane] = pz[at];
-        sh.tile_index[lane] = pindex[at];
-        sh.tile_wx[lane] = pwx[at];
-        sh.tile_wy[lane] = pwy[at];
-        sh.tile_wz[lane] = pwz[at];
-      }
+        if (static_cast<uint32_t>(lane) < n_i) {
+            const uint32_t at = first_i + lane;
+            sh.tile_x[lane] = px[at];
+            sh.tile_y[lane] = py[at];
+            sh.tile_z[lane] = pz[at];
+            sh.tile_index[lane] = pindex[at];
+            sh.tile_wx[lane] = pwx[at];
+            sh.tile_wy[lane] = pwy[at];
+            sh.tile_wz[lane] = pwz[at];
+        }
     }
-    const bool tile_wrapped = tile.wrapped != 0;
 
+    SweepContext ctx;
+    ctx.tile_wrapped = tile.wrapped != 0;
+    ctx.lane = lane;
+    shift_vector(g, 0, 0, 0, ctx.zero_tx, ctx.zero_ty, ctx.zero_tz);
+
+    // upper half of the stencil: linear offsets from the centre (the cell itself) to the last one, in the order
+    // dx major, dz minor, are exactly the lexicographically non-negative offsets
     const int32_t span_y = 2 * g.s[1] + 1;
     const int32_t span_z = 2 * g.s[2] + 1;
-    const uint32_t n_entries = static_cast<uint32_t>(2 * g.s[0] + 1) * span_y * span_z;
-
-    // shift vector of the zero shift: +0 or -0 per component, depending on the signs in H
-    double zero_tx, zero_ty, zero_tz;
-    shift_vector(g, 0, 0, 0, zero_tx, zero_ty, zero_tz);
+    const uint32_t n_stencil = static_cast<uint32_t>(2 * g.s[0] + 1) * span_y * span_z;
+    const uint32_t centre = n_stencil / 2;
+    const uint32_t n_entries = n_stencil - centre;
 
     WaveState state;
     state.total = 0;
-    state.out_cursor = WRITE ? args.offsets[wave_slot] : 0;
+    state.out_cursor = WRITE ? args.offsets[work] : 0;
     state.head = 0;
     state.tail = 0;
 
@@ -464,7 +498,7 @@ __device__ __forceinline__ void search_work_item(
 
         // ---- stencil entries of this batch: neighbour cell, its cell shift, how many points it holds
         for (uint32_t e = lane; e < n_batch; e += WAVE) {
-            uint32_t linear = batch + e;
+            const uint32_t linear = centre + batch + e;
             int32_t dz = static_cast<int32_t>(linear % span_z) - g.s[2];
             int32_t dy = static_cast<int32_t>((linear / span_z) % span_y) - g.s[1];
             int32_t dx = static_cast<int32_t>(linear / (span_z * span_y)) - g.s[0];
@@ -495,7 +529,7 @@ __device__ __forceinline__ void search_work_item(
                 start = static_cast<uint32_t>(args.cell_scan[neighbour]);
                 count = static_cast<uint32_t>(args.cell_scan[neighbour + 1]) - start;
                 packed = pack_shift(q[0], q[1], q[2]);
-                if (neighbour == tile.cell) {
+                if (linear == centre) {
                     packed |= 1 << 30;
                 }
             }
@@ -541,9 +575,7 @@ __device__ __forceinline__ void search_work_item(
                 c.x[r] = c.y[r] = c.z[r] = __builtin_nan("");
                 c.tx[r] = c.ty[r] = c.tz[r] = 0.0;
                 c.bx[r] = c.by[r] = c.bz[r] = 0;
-                c.index[r] = 0xFFFFFFFFu;
-                c.self_key[r] = 0xFFFFFFFFu;
-                c.image_key[r] = 0xFFFFFFFFu;
+                c.position[r] = 0xFFFFFFFFu;
                 bool same_cell = false;
                 if (valid) {
                     // largest e with ent_prefix[e] <= k
@@ -565,19 +597,24 @@ __device__ __forceinline__ void search_work_item(
                     c.x[r] = px[at];
                     c.y[r] = py[at];
                     c.z[r] = pz[at];
-                    c.index[r] = pindex[at];
                     c.bx[r] = qx - pwx[at];
                     c.by[r] = qy - pwy[at];
                     c.bz[r] = qz - pwz[at];
-                }
-                const bool shifted = (c.bx[r] | c.by[r] | c.bz[r]) != 0;
-                if (same_cell) {
-                    if (!shifted) {
-                        c.self_key[r] = c.index[r];
-                    } else if (half_keeps_self_image(c.bx[r], c.by[r], c.bz[r])) {
-                        c.image_key[r] = c.index[r];
+                    if (same_cell) {
+                        c.position[r] = at;
+                    }
+                    if constexpr (WRITE) {
+                        const int slot = r * WAVE + lane;
+                        sh.cand_x[slot] = c.x[r];
+                        sh.cand_y[slot] = c.y[r];
+                        sh.cand_z[slot] = c.z[r];
+                        sh.cand_index[slot] = pindex[at];
+                        sh.cand_bx[slot] = c.bx[r];
+                        sh.cand_by[slot] = c.by[r];
+                        sh.cand_bz[slot] = c.bz[r];
                     }
                 }
+                const bool shifted = (c.bx[r] | c.by[r] | c.bz[r]) != 0;
                 c.any_shift = c.any_shift || (__ballot(shifted) != 0);
                 c.any_same = c.any_same || (__ballot(same_cell) != 0);
             }
@@ -590,15 +627,14 @@ __device__ __forceinline__ void search_work_item(
 
             state.head = 0;
             state.tail = 0;
+            if constexpr (WRITE) {
+                wave_sync(); // candidate records are in LDS before any ticket is redeemed
+            }
 
 #define VESIN_SWEEP(SHIFTED, SAME)                                                                                    \
-    sweep_unwrapped<WRITE, FULL, R, SHIFTED, SAME>(                                                                   \
-        args.sorted, first_i, n_i, state, c, sh, args.out, g, wave, lane, zero_tx, zero_ty, zero_tz                   \
-    )
-            if (tile_wrapped) {
-                sweep_wrapped<WRITE, FULL, R>(
-                    args.sorted, first_i, n_i, state, c, sh, args.out, g, wave, lane, zero_tx, zero_ty, zero_tz
-                );
+    sweep_unwrapped<WRITE, FULL, R, SHIFTED, SAME>(args.sorted, first_i, n_i, state, c, sh, args.out, g, ctx)
+            if (ctx.tile_wrapped) {
+                sweep_wrapped<WRITE, FULL, R>(args.sorted, first_i, n_i, state, c, sh, args.out, g, ctx);
             } else if (c.any_shift) {
                 if (c.any_same) {
                     VESIN_SWEEP(true, true);
@@ -617,22 +653,19 @@ __device__ __forceinline__ void search_work_item(
             // the candidates leave the registers with this group: redeem what is left
             if constexpr (WRITE) {
                 if (state.head != state.tail) {
-                    redeem<R>(
-                        state.head - state.tail, state, c, sh, args.out, g, tile_wrapped, wave, lane, zero_tx, zero_ty,
-                        zero_tz
-                    );
+                    redeem<FULL, R>(state.head - state.tail, state, c, sh, args.out, g, ctx);
                 }
             }
         }
     }
 
     if (!WRITE && lane == 0) {
-        args.counts[wave_slot] = state.total;
+        // a full list gets two rows per hit: the pair and its mirror
+        args.counts[work] = FULL ? 2 * state.total : state.total;
     }
 }
 
-/// Four independent waves per workgroup, one work item each (single-wave workgroups would cap the number of
-/// waves a CU holds well below what the registers allow).
+/// Four independent waves per workgroup, one work item each.
 template <bool WRITE, bool FULL, int R>
 __global__ __launch_bounds__(SEARCH_BLOCK) void search_kernel(SearchArgs args, GridParams g) {
     __shared__ std::conditional_t<WRITE, SearchSharedWrite, SearchSharedCount> shared[SEARCH_WAVES];
