@@ -27,15 +27,28 @@ struct SortedPoints {
 
 constexpr uint32_t SORTED_PADDING = 8;
 
-__global__ void init_status(DeviceStatus* status) {
-    if (threadIdx.x == 0 && blockIdx.x == 0) {
+/// First kernel of a call: box and periodicity go to pinned host memory (the host picks the grid from them), and
+/// the status block is reset.
+__global__ void fetch_box(
+    const double* __restrict__ box, const bool* __restrict__ periodic, unsigned char* host_small, DeviceStatus* status
+) {
+    const int t = threadIdx.x;
+    if (t < 9) {
+        reinterpret_cast<double*>(host_small)[t] = box[t];
+    } else if (t < 12) {
+        host_small[72 + (t - 9)] = periodic[t - 9] ? 1 : 0;
+    } else if (t == 12) {
         status->total_pairs = 0;
         status->first_bad_coordinate = 0xFFFFFFFFu;
-        status->n_tiles = 0;
-        for (int d = 0; d < 3; d++) {
-            status->frac_min[d] = ~0ull;
-            status->frac_max[d] = 0ull;
-        }
+    }
+}
+
+/// After the counting pass: what the host needs to know goes to pinned host memory, read after the next
+/// synchronisation of the stream.
+__global__ void publish_status(const DeviceStatus* status, const uint64_t* total, DeviceStatus* host_status) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        host_status->first_bad_coordinate = status->first_bad_coordinate;
+        host_status->total_pairs = *total;
     }
 }
 
@@ -63,10 +76,12 @@ __device__ __forceinline__ bool all_finite(double x, double y, double z, unsigne
 }
 
 /// Smallest and largest fractional coordinate over all points (needed for non-periodic directions), plus the
-/// check for non-finite input. Grid-stride loop, wave reduction, then one atomic per wave and direction.
+/// check for non-finite input. Grid-stride loop, wave then workgroup reduction; every workgroup reports to its own
+/// slot of `host_bounds` (pinned host memory), so no atomics are involved.
 __global__ __launch_bounds__(BLOCK) void bounding_kernel(
-    const double* __restrict__ points, uint32_t n_points, GridParams g, DeviceStatus* status
+    const double* __restrict__ points, uint32_t n_points, GridParams g, BlockBounds* host_bounds
 ) {
+    __shared__ BlockBounds partial[WAVES_PER_BLOCK];
     double lo[3] = {INFINITY, INFINITY, INFINITY};
     double hi[3] = {-INFINITY, -INFINITY, -INFINITY};
     unsigned int bad = 0xFFFFFFFFu;
@@ -100,16 +115,27 @@ __global__ __launch_bounds__(BLOCK) void bounding_kernel(
     }
 
     if (lane_id() == 0) {
+        BlockBounds& mine = partial[threadIdx.x / WAVE];
 #pragma unroll
         for (int d = 0; d < 3; d++) {
-            if (lo[d] <= hi[d]) {
-                atomicMin(&status->frac_min[d], ordered_bits(lo[d]));
-                atomicMax(&status->frac_max[d], ordered_bits(hi[d]));
+            mine.lo[d] = lo[d];
+            mine.hi[d] = hi[d];
+        }
+        mine.first_bad_coordinate = bad;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        BlockBounds all = partial[0];
+        for (int w = 1; w < WAVES_PER_BLOCK; w++) {
+#pragma unroll
+            for (int d = 0; d < 3; d++) {
+                all.lo[d] = fmin(all.lo[d], partial[w].lo[d]);
+                all.hi[d] = fmax(all.hi[d], partial[w].hi[d]);
             }
+            all.first_bad_coordinate = min(all.first_bad_coordinate, partial[w].first_bad_coordinate);
         }
-        if (bad != 0xFFFFFFFFu) {
-            atomicMin(&status->first_bad_coordinate, bad);
-        }
+        all.padding = 0;
+        host_bounds[blockIdx.x] = all;
     }
 }
 
@@ -145,35 +171,65 @@ __device__ __forceinline__ void locate(
 }
 
 /// One thread per point: cell id, wrap shift, and the histogram of points per cell. The value returned by the
-/// histogram atomic is kept as the point's provisional slot inside its cell.
+/// histogram atomic is kept as the point's provisional slot inside its cell. Lanes of a wave that fall in the same
+/// cell (the usual case for spatially coherent input) are grouped first, for up to ASSIGN_ROUNDS distinct cells
+/// per wave, so that one lane per group issues the atomic for all of them.
+constexpr int ASSIGN_ROUNDS = 8;
+
 __global__ __launch_bounds__(BLOCK) void assign_cells(
     const double* __restrict__ points, GridParams g,
     uint32_t* __restrict__ cell_of, uint32_t* __restrict__ slot_of, int32_t* __restrict__ wrap_of,
     uint32_t* __restrict__ cell_counts, DeviceStatus* status
 ) {
-    uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
-    if (i >= g.n_points) {
-        return;
-    }
-    double x = points[3 * static_cast<size_t>(i) + 0];
-    double y = points[3 * static_cast<size_t>(i) + 1];
-    double z = points[3 * static_cast<size_t>(i) + 2];
+    const uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
+    const bool active = i < g.n_points;
+    const int lane = lane_id();
 
     int32_t cell[3] = {0, 0, 0};
     int32_t wrap[3] = {0, 0, 0};
-    unsigned int axis;
-    if (all_finite(x, y, z, axis)) {
-        locate(g, x, y, z, cell, wrap);
-    } else {
-        atomicMin(&status->first_bad_coordinate, 3u * i + axis);
+    if (active) {
+        double x = points[3 * static_cast<size_t>(i) + 0];
+        double y = points[3 * static_cast<size_t>(i) + 1];
+        double z = points[3 * static_cast<size_t>(i) + 2];
+        unsigned int axis;
+        if (all_finite(x, y, z, axis)) {
+            locate(g, x, y, z, cell, wrap);
+        } else {
+            atomicMin(&status->first_bad_coordinate, 3u * i + axis);
+        }
+    }
+    const uint32_t linear = (static_cast<uint32_t>(cell[2]) * g.n[1] + cell[1]) * g.n[0] + cell[0];
+
+    uint64_t group = 1ull << lane; // lanes left over after the rounds stand alone
+    bool pending = active;
+    for (int round = 0; round < ASSIGN_ROUNDS; round++) {
+        const uint64_t remaining = __ballot(pending);
+        if (remaining == 0) {
+            break;
+        }
+        const int leader = __ffsll(static_cast<unsigned long long>(remaining)) - 1;
+        const uint32_t leader_cell = read_lane(linear, leader);
+        const bool same = pending && linear == leader_cell;
+        const uint64_t members = __ballot(same);
+        if (same) {
+            group = members;
+            pending = false;
+        }
     }
 
-    uint32_t linear = (static_cast<uint32_t>(cell[2]) * g.n[1] + cell[1]) * g.n[0] + cell[0];
-    cell_of[i] = linear;
-    slot_of[i] = atomicAdd(&cell_counts[linear], 1u);
-    wrap_of[3 * static_cast<size_t>(i) + 0] = wrap[0];
-    wrap_of[3 * static_cast<size_t>(i) + 1] = wrap[1];
-    wrap_of[3 * static_cast<size_t>(i) + 2] = wrap[2];
+    const int first = __ffsll(static_cast<unsigned long long>(group)) - 1;
+    uint32_t base = 0;
+    if (active && lane == first) {
+        base = atomicAdd(&cell_counts[linear], static_cast<uint32_t>(__popcll(group)));
+    }
+    base = static_cast<uint32_t>(__shfl(static_cast<int>(base), first));
+    if (active) {
+        cell_of[i] = linear;
+        slot_of[i] = base + rank_in_mask(group);
+        wrap_of[3 * static_cast<size_t>(i) + 0] = wrap[0];
+        wrap_of[3 * static_cast<size_t>(i) + 1] = wrap[1];
+        wrap_of[3 * static_cast<size_t>(i) + 2] = wrap[2];
+    }
 }
 
 /// Counting-sort scatter: the point goes to (start of its cell) + (its provisional slot).
@@ -191,67 +247,58 @@ __global__ __launch_bounds__(BLOCK) void scatter_points(
 
 constexpr uint32_t CANONICAL_LIMIT = 4096;
 
-/// One wave per cell. The atomics of assign_cells leave the points of a cell in arbitrary order; here they are
-/// ranked by original index (so the whole pipeline is deterministic), gathered into the structure-of-arrays
-/// layout, and the cell's 64-point tiles are appended to the tile list.
-__global__ __launch_bounds__(BLOCK) void gather_cells(
-    const double* __restrict__ points, const int32_t* __restrict__ wrap_of,
-    const uint32_t* __restrict__ provisional, const uint64_t* __restrict__ cell_scan, uint32_t n_cells,
+/// One thread per slot of the counting sort. The atomics of assign_cells leave the points of a cell in arbitrary
+/// order; here every point is ranked by original index among the points of its cell (so the whole pipeline is
+/// deterministic), gathered into the structure-of-arrays layout, and the first point of every run of 64 appends
+/// the tile to the tile list. Work is proportional to the number of points, whatever the number of empty cells.
+/// `tiles[].wrapped` must be zero on entry: points moved by a box vector set it with an atomic.
+__global__ __launch_bounds__(BLOCK) void gather_points(
+    const double* __restrict__ points, const int32_t* __restrict__ wrap_of, const uint32_t* __restrict__ cell_of,
+    const uint32_t* __restrict__ provisional, const uint64_t* __restrict__ cell_scan, uint32_t n_points,
     SortedPoints sorted, Tile* __restrict__ tiles
 ) {
-    const int lane = lane_id();
-    const uint32_t cell = blockIdx.x * WAVES_PER_BLOCK + threadIdx.x / WAVE;
-    if (cell >= n_cells) {
+    const uint32_t p = blockIdx.x * BLOCK + threadIdx.x;
+    if (p >= n_points) {
         return;
     }
+    const uint32_t mine = provisional[p];
+    const uint32_t cell = cell_of[mine];
     const uint64_t here = cell_scan[cell];
-    const uint64_t next = cell_scan[cell + 1];
     const uint32_t start = static_cast<uint32_t>(here);
-    const uint32_t count = static_cast<uint32_t>(next) - start;
+    const uint32_t count = static_cast<uint32_t>(cell_scan[cell + 1]) - start;
     const uint32_t first_tile = static_cast<uint32_t>(here >> 32);
-    if (count == 0) {
-        return;
+
+    uint32_t rank = p - start;
+    if (count <= CANONICAL_LIMIT) {
+        rank = 0;
+        // neighbouring lanes share the cell, so these loads hit the same few cache lines
+        for (uint32_t other = 0; other < count; other++) {
+            rank += provisional[start + other] < mine ? 1u : 0u;
+        }
     }
 
-    bool any_wrapped = false;
-    for (uint32_t base = 0; base < count; base += WAVE) {
-        uint32_t k = base + lane;
-        bool active = k < count;
-        uint32_t mine = active ? provisional[start + k] : 0xFFFFFFFFu;
-        uint32_t rank = k;
-        if (count <= CANONICAL_LIMIT) {
-            rank = 0;
-            for (uint32_t other = 0; other < count; other++) {
-                // same address in every lane: served as one broadcast load
-                rank += provisional[start + other] < mine ? 1u : 0u;
-            }
-        }
-        bool wrapped = false;
-        if (active) {
-            uint32_t to = start + rank;
-            const int32_t wx = wrap_of[3 * static_cast<size_t>(mine) + 0];
-            const int32_t wy = wrap_of[3 * static_cast<size_t>(mine) + 1];
-            const int32_t wz = wrap_of[3 * static_cast<size_t>(mine) + 2];
-            wrapped = (wx | wy | wz) != 0;
-            sorted.index[to] = mine;
-            sorted.x[to] = points[3 * static_cast<size_t>(mine) + 0];
-            sorted.y[to] = points[3 * static_cast<size_t>(mine) + 1];
-            sorted.z[to] = points[3 * static_cast<size_t>(mine) + 2];
-            sorted.wx[to] = wx;
-            sorted.wy[to] = wy;
-            sorted.wz[to] = wz;
-        }
-        any_wrapped = any_wrapped || (__ballot(wrapped) != 0);
+    const uint32_t to = start + rank;
+    const int32_t wx = wrap_of[3 * static_cast<size_t>(mine) + 0];
+    const int32_t wy = wrap_of[3 * static_cast<size_t>(mine) + 1];
+    const int32_t wz = wrap_of[3 * static_cast<size_t>(mine) + 2];
+    sorted.index[to] = mine;
+    sorted.x[to] = points[3 * static_cast<size_t>(mine) + 0];
+    sorted.y[to] = points[3 * static_cast<size_t>(mine) + 1];
+    sorted.z[to] = points[3 * static_cast<size_t>(mine) + 2];
+    sorted.wx[to] = wx;
+    sorted.wy[to] = wy;
+    sorted.wz[to] = wz;
+    if ((wx | wy | wz) != 0) {
+        // tiles holding a wrapped point take the search kernel's general path
+        atomicOr(&tiles[first_tile + rank / 64u].wrapped, 1u);
     }
 
-    // tiles of a cell holding a wrapped point take the search kernel's general path
-    for (uint32_t t = lane; t * 64u < count; t += WAVE) {
-        Tile tile;
-        tile.cell = cell;
-        tile.first = start + t * 64u;
-        tile.count = min(64u, count - t * 64u);
-        tile.wrapped = any_wrapped ? 1u : 0u;
-        tiles[first_tile + t] = tile;
+    const uint32_t k = p - start;
+    if (k % 64u == 0) {
+        Tile* tile = &tiles[first_tile + k / 64u];
+        tile->cell = cell;
+        tile->first = start + k;
+        tile->count = min(64u, count - k);
     }
 }
 

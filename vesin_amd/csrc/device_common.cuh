@@ -37,10 +37,18 @@ struct Tile {
 struct DeviceStatus {
     unsigned long long total_pairs;
     unsigned int first_bad_coordinate; // 3 * point + axis of the first non-finite coordinate, or 0xFFFFFFFF
-    unsigned int n_tiles;
-    unsigned long long frac_min[3];    // order-preserving encoding of the smallest / largest projected coordinate
-    unsigned long long frac_max[3];
+    unsigned int padding;
 };
+
+/// What one workgroup of the bounding pass reports (to pinned host memory; the host folds the workgroups).
+struct BlockBounds {
+    double lo[3]; // smallest / largest projected coordinate; lo > hi when the workgroup saw no finite point
+    double hi[3];
+    unsigned int first_bad_coordinate;
+    unsigned int padding;
+};
+
+constexpr int BOUNDING_BLOCKS = 256;
 
 __device__ __forceinline__ int lane_id() {
     return static_cast<int>(__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)));
@@ -97,19 +105,6 @@ __device__ __forceinline__ uint64_t read_lane(uint64_t v, int lane) {
     uint32_t lo = read_lane(static_cast<uint32_t>(v), lane);
     uint32_t hi = read_lane(static_cast<uint32_t>(v >> 32), lane);
     return (static_cast<uint64_t>(hi) << 32) | lo;
-}
-
-/// Doubles mapped to unsigned integers with the same ordering, for atomicMin / atomicMax.
-__device__ __forceinline__ unsigned long long ordered_bits(double x) {
-    unsigned long long bits = static_cast<unsigned long long>(__double_as_longlong(x));
-    return (bits & 0x8000000000000000ull) ? ~bits : (bits | 0x8000000000000000ull);
-}
-
-inline double ordered_bits_to_double(unsigned long long key) {
-    unsigned long long bits = (key & 0x8000000000000000ull) ? (key & 0x7FFFFFFFFFFFFFFFull) : ~key;
-    double x;
-    __builtin_memcpy(&x, &bits, sizeof(double));
-    return x;
 }
 
 } // namespace vesin_hip

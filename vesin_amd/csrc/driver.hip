@@ -12,6 +12,7 @@
 #include <cstdlib>
 #include <cstring>
 
+#include <algorithm>
 #include <atomic>
 #include <stdexcept>
 #include <string>
@@ -92,6 +93,7 @@ struct HipExtras {
     DeviceStatus* d_status = nullptr;
     DeviceStatus* h_status = nullptr; // pinned
     unsigned char* h_small = nullptr; // pinned: box (72 bytes) + periodic (3 bytes)
+    BlockBounds* h_bounds = nullptr;  // pinned: one slot per workgroup of the bounding pass
     size_t capacity = 0;              // rows every allocated output array can hold
     hipEvent_t events[T_STAGES] = {};
     bool have_events = false;
@@ -110,6 +112,9 @@ struct HipExtras {
         if (h_small != nullptr) {
             (void)hipHostFree(h_small);
         }
+        if (h_bounds != nullptr) {
+            (void)hipHostFree(h_bounds);
+        }
         if (have_events) {
             for (auto& event : events) {
                 (void)hipEventDestroy(event);
@@ -126,6 +131,9 @@ HipExtras& extras_of(VesinNeighborList& neighbors) {
         HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&extras->d_status), sizeof(DeviceStatus)));
         HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&extras->h_status), sizeof(DeviceStatus), hipHostMallocDefault));
         HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&extras->h_small), 128, hipHostMallocDefault));
+        HIP_CHECK(hipHostMalloc(
+            reinterpret_cast<void**>(&extras->h_bounds), BOUNDING_BLOCKS * sizeof(BlockBounds), hipHostMallocDefault
+        ));
     }
     return *static_cast<HipExtras*>(neighbors.opaque);
 }
@@ -322,8 +330,10 @@ void neighbors(
     };
 
     // ---- box and periodicity come to the host once: 75 bytes
-    HIP_CHECK(hipMemcpyAsync(extras.h_small, box, 9 * sizeof(double), hipMemcpyDeviceToHost, stream));
-    HIP_CHECK(hipMemcpyAsync(extras.h_small + 72, periodic, 3, hipMemcpyDeviceToHost, stream));
+    hipLaunchKernelGGL(
+        fetch_box, dim3(1), dim3(64), 0, stream,
+        reinterpret_cast<const double*>(box), periodic, extras.h_small, extras.d_status
+    );
     HIP_CHECK(hipStreamSynchronize(stream));
     double host_box[9];
     bool host_periodic[3];
@@ -353,29 +363,33 @@ void neighbors(
     g.n_points = static_cast<uint32_t>(n_points);
 
     mark(T_START);
-    hipLaunchKernelGGL(init_status, dim3(1), dim3(1), 0, stream, extras.d_status);
 
     // ---- extent of the points along non-periodic directions
     const bool any_open = !(hbox.periodic[0] && hbox.periodic[1] && hbox.periodic[2]);
     double lo[3] = {0, 0, 0};
     double hi[3] = {0, 0, 0};
     if (any_open) {
-        uint32_t blocks = static_cast<uint32_t>((n_points + BLOCK - 1) / BLOCK);
-        if (blocks > 2048) {
-            blocks = 2048;
-        }
+        const uint32_t blocks = static_cast<uint32_t>(std::min<size_t>(BOUNDING_BLOCKS, (n_points + BLOCK - 1) / BLOCK));
         hipLaunchKernelGGL(
             bounding_kernel, dim3(blocks), dim3(BLOCK), 0, stream,
-            reinterpret_cast<const double*>(points), g.n_points, g, extras.d_status
+            reinterpret_cast<const double*>(points), g.n_points, g, extras.h_bounds
         );
-        HIP_CHECK(hipMemcpyAsync(extras.h_status, extras.d_status, sizeof(DeviceStatus), hipMemcpyDeviceToHost, stream));
         HIP_CHECK(hipStreamSynchronize(stream));
-        if (extras.h_status->first_bad_coordinate != 0xFFFFFFFFu) {
-            non_finite_error(points, extras.h_status->first_bad_coordinate);
-        }
+        unsigned int bad = 0xFFFFFFFFu;
         for (int d = 0; d < 3; d++) {
-            lo[d] = ordered_bits_to_double(extras.h_status->frac_min[d]);
-            hi[d] = ordered_bits_to_double(extras.h_status->frac_max[d]);
+            lo[d] = INFINITY;
+            hi[d] = -INFINITY;
+        }
+        for (uint32_t block = 0; block < blocks; block++) {
+            const BlockBounds& part = extras.h_bounds[block];
+            bad = std::min(bad, part.first_bad_coordinate);
+            for (int d = 0; d < 3; d++) {
+                lo[d] = std::fmin(lo[d], part.lo[d]);
+                hi[d] = std::fmax(hi[d], part.hi[d]);
+            }
+        }
+        if (bad != 0xFFFFFFFFu) {
+            non_finite_error(points, bad);
         }
     }
 
@@ -422,7 +436,9 @@ void neighbors(
     const size_t scratch_elements = std::max(scan_scratch_elements(n_cells), scan_scratch_elements(n_slots));
 
     auto carve = [&](Carver& carver) {
+        // cell_counts and tiles are adjacent: one fill clears the histogram and the tiles' flags
         cell_counts = carver.take<uint32_t>(n_cells);
+        tiles = carver.take<Tile>(tiles_bound);
         cell_scan = carver.take<uint64_t>(n_cells + 1);
         if (!single_cell) {
             cell_of = carver.take<uint32_t>(n_points);
@@ -437,7 +453,6 @@ void neighbors(
         sorted.wx = carver.take<int32_t>(n_points);
         sorted.wy = carver.take<int32_t>(n_points);
         sorted.wz = carver.take<int32_t>(n_points);
-        tiles = carver.take<Tile>(tiles_bound);
         counts = carver.take<uint32_t>(n_slots);
         offsets = carver.take<uint64_t>(n_slots + 1);
         scan_scratch = carver.take<uint64_t>(scratch_elements);
@@ -457,7 +472,8 @@ void neighbors(
             flat_points, g, sorted, tiles, cell_scan, extras.d_status
         );
     } else {
-        HIP_CHECK(hipMemsetAsync(cell_counts, 0, n_cells * sizeof(uint32_t), stream));
+        const size_t to_clear = reinterpret_cast<char*>(tiles + tiles_bound) - reinterpret_cast<char*>(cell_counts);
+        HIP_CHECK(hipMemsetAsync(cell_counts, 0, to_clear, stream));
         hipLaunchKernelGGL(
             assign_cells, dim3(point_blocks), dim3(BLOCK), 0, stream,
             flat_points, g, cell_of, slot_of, wrap_of, cell_counts, extras.d_status
@@ -467,10 +483,9 @@ void neighbors(
             scatter_points, dim3(point_blocks), dim3(BLOCK), 0, stream,
             g.n_points, cell_of, slot_of, cell_scan, provisional
         );
-        const uint32_t cell_blocks = static_cast<uint32_t>((n_cells + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK);
         hipLaunchKernelGGL(
-            gather_cells, dim3(cell_blocks), dim3(BLOCK), 0, stream,
-            flat_points, wrap_of, provisional, cell_scan, g.n_cells, sorted, tiles
+            gather_points, dim3(point_blocks), dim3(BLOCK), 0, stream,
+            flat_points, wrap_of, cell_of, provisional, cell_scan, g.n_points, sorted, tiles
         );
     }
     mark(T_CELLS);
@@ -490,10 +505,30 @@ void neighbors(
     exclusive_scan<SCAN_U32>(counts, n_slots, offsets, scan_scratch, stream);
     mark(T_SCAN);
 
-    HIP_CHECK(hipMemcpyAsync(extras.h_status, extras.d_status, sizeof(DeviceStatus), hipMemcpyDeviceToHost, stream));
-    HIP_CHECK(hipMemcpyAsync(
-        &extras.h_status->total_pairs, offsets + n_slots, sizeof(uint64_t), hipMemcpyDeviceToHost, stream
-    ));
+    hipLaunchKernelGGL(publish_status, dim3(1), dim3(1), 0, stream, extras.d_status, offsets + n_slots, extras.h_status);
+
+    auto outputs_of = [&]() {
+        SearchOutputs out;
+        out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
+        out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
+        out.distances = neighbors.distances;
+        out.vectors = reinterpret_cast<double*>(neighbors.vectors);
+        return out;
+    };
+
+    // ---- pass 2: write. Without sorting the rows go straight to the caller's arrays, and the launch does not
+    // wait for the host to learn their number: the arrays keep the capacity of earlier calls, and a launch that
+    // would overflow them writes nothing and is repeated once they have grown.
+    const bool speculative = !options.sorted;
+    if (speculative) {
+        size_outputs(neighbors, extras, 0, options);
+        args.out = outputs_of();
+        args.capacity = extras.capacity;
+        mark(T_WRITE_BEGIN);
+        launch_search<true>(options.full, args, g, stream);
+        mark(T_WRITE);
+    }
+
     HIP_CHECK(hipStreamSynchronize(stream));
     if (extras.h_status->first_bad_coordinate != 0xFFFFFFFFu) {
         non_finite_error(points, extras.h_status->first_bad_coordinate);
@@ -509,13 +544,9 @@ void neighbors(
         );
     }
 
-    // ---- pass 2: write
+    const bool fits = total <= extras.capacity;
     size_outputs(neighbors, extras, total, options);
-    SearchOutputs final_out;
-    final_out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
-    final_out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
-    final_out.distances = neighbors.distances;
-    final_out.vectors = reinterpret_cast<double*>(neighbors.vectors);
+    const SearchOutputs final_out = outputs_of();
 
     const bool sorting = options.sorted && total > 1;
     SearchOutputs unsorted = final_out;
@@ -545,19 +576,24 @@ void neighbors(
         carve_sort(sort_carver);
     }
 
-    mark(T_WRITE_BEGIN);
-    if (total > 0) {
-        args.out = unsorted;
-        launch_search<true>(options.full, args, g, stream);
+    if (!speculative || !fits) {
+        mark(T_WRITE_BEGIN);
+        if (total > 0) {
+            args.out = unsorted;
+            args.capacity = sorting ? total : extras.capacity;
+            launch_search<true>(options.full, args, g, stream);
+        }
+        mark(T_WRITE);
     }
-    mark(T_WRITE);
 
     if (sorting) {
         sort_pairs(unsorted, final_out, total, n_points, sort_space, stream);
     }
     mark(T_SORT);
 
-    HIP_CHECK(hipStreamSynchronize(stream));
+    if (!speculative || !fits || timed) {
+        HIP_CHECK(hipStreamSynchronize(stream));
+    }
     HIP_CHECK(hipGetLastError());
     neighbors.length = total;
 

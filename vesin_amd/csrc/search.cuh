@@ -71,6 +71,7 @@ struct SearchArgs {
     uint32_t n_slices;         // work items sharing one tile (each takes a slice of the candidates)
     uint32_t n_work;           // work items = tile slots * n_slices; tile slots are a multiple of
                                // N_XCD * SEARCH_WAVES and at least the number of tiles
+    uint64_t capacity;         // WRITE: rows the output arrays hold; a launch that would overflow writes nothing
 };
 
 __device__ __forceinline__ int32_t pack_shift(int32_t a, int32_t b, int32_t c) {
@@ -673,6 +674,11 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void search_kernel(SearchArgs args, G
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     const uint32_t n_tiles = static_cast<uint32_t>(args.cell_scan[g.n_cells] >> 32);
     const uint32_t work = blockIdx.x * SEARCH_WAVES + wave;
+    if (WRITE && args.offsets[args.n_work] > args.capacity) {
+        // launched before the host knew the number of rows, and they do not fit: the host grows the arrays and
+        // launches again
+        return;
+    }
     if (work < args.n_work) {
         search_work_item<WRITE, FULL, R>(work, args, g, shared[wave], n_tiles, lane);
     }
