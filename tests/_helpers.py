@@ -14,17 +14,48 @@ def gpu_neighbors(points, box, periodic, cutoff, full=True, sorted=False, quanti
 
     calculator = NeighborList(cutoff=cutoff, full_list=full, sorted=sorted, algorithm=algorithm)
     letters = "P" + "".join(q for q in "SdD" if q in quantities)
-    outputs = calculator.compute(
-        torch.as_tensor(np.ascontiguousarray(points, dtype=np.float64), device="cuda:0"),
-        torch.as_tensor(np.ascontiguousarray(box, dtype=np.float64), device="cuda:0"),
-        periodic,
-        letters,
-        copy=True,
-    )
     names = {"P": "pairs", "S": "shifts", "d": "distances", "D": "vectors"}
-    result = {names[q]: out.cpu().numpy() for q, out in zip(letters, outputs)}
+    device_points = torch.as_tensor(np.ascontiguousarray(points, dtype=np.float64), device="cuda:0")
+    device_box = torch.as_tensor(np.ascontiguousarray(box, dtype=np.float64), device="cuda:0")
+
+    # The first call of a list sizes the outputs with the two-pass search; later calls of an unsorted list go
+    # through the single-pass search into the arrays they kept. Both must give the same rows.
+    results = []
+    for _ in range(2):
+        outputs = calculator.compute(device_points, device_box, periodic, letters, copy=True)
+        results.append({names[q]: out.cpu().numpy() for q, out in zip(letters, outputs)})
     del calculator
-    return result
+    first, second = results
+    if sorted:
+        for key in first:
+            assert np.array_equal(first[key], second[key]), f"second call differs from the first: {key}"
+    elif len(first["pairs"]) > 2_000_000:
+        # too many rows to sort twice within a test's time: order-independent fingerprints of the rows
+        from golden import systems
+
+        assert systems.fingerprints(first) == systems.fingerprints(second), "second call differs from the first"
+    else:
+        a = _fully_ordered(first)
+        b = _fully_ordered(second)
+        for key in a:
+            assert a[key].shape == b[key].shape, (
+                f"second call has {b[key].shape[0]} rows of {key}, the first had {a[key].shape[0]}"
+            )
+            assert np.array_equal(a[key], b[key]), f"second call differs from the first: {key}"
+    return second
+
+
+def _fully_ordered(result):
+    """Rows sorted by every column present, so that two row orders of one list compare equal even when the shifts
+    that tell the images of a pair apart were not requested."""
+    n = len(result["pairs"])
+    columns = []
+    for key in ("vectors", "distances", "shifts", "pairs"):
+        if key in result:
+            block = result[key].reshape(n, -1)
+            columns += [block[:, c] for c in range(block.shape[1] - 1, -1, -1)]
+    order = np.lexsort(columns) if n else np.arange(0)
+    return {key: value[order] for key, value in result.items()}
 
 
 def near_cutoff_count(result, cutoff):

@@ -1,0 +1,163 @@
+"""The two ways the HIP path produces an unsorted list must agree (``-m gpu``).
+
+A list's first call sizes the output arrays with the two-pass search (count, scan, write). Later calls go through the
+single-pass search (sweep with hit columns, chained row offsets, replay) straight into the arrays they kept, and fall
+back to the two passes when the rows do not fit or the problem has a shape the single pass does not cover. Every
+branch of that decision is driven here and compared with the CPU oracle."""
+
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from _helpers import assert_same_list
+from golden import systems
+from vesin_amd import NeighborList, configs, enable_timings
+
+pytestmark = pytest.mark.gpu
+
+NAMES = {"P": "pairs", "S": "shifts", "d": "distances", "D": "vectors"}
+
+
+def on_device(points, box):
+    import torch
+
+    return (
+        torch.as_tensor(np.ascontiguousarray(points, dtype=np.float64), device="cuda:0"),
+        torch.as_tensor(np.ascontiguousarray(box, dtype=np.float64), device="cuda:0"),
+    )
+
+
+def call(calculator, points, box, periodic, letters="PSdD"):
+    device_points, device_box = on_device(points, box)
+    outputs = calculator.compute(device_points, device_box, periodic, letters, copy=True)
+    return {NAMES[q]: out.cpu().numpy() for q, out in zip(letters, outputs)}
+
+
+@pytest.fixture
+def timings():
+    enable_timings(True)
+    yield
+    enable_timings(False)
+
+
+def used_single_pass(calculator):
+    stages = calculator.timings()
+    return stages["count"] == 0 and stages["scan"] == 0 and stages["write"] > 0
+
+
+@pytest.mark.parametrize("full", [True, False], ids=["full", "half"])
+def test_second_call_is_single_pass_and_matches(timings, full):
+    points, box, periodic, _ = configs.config1(10)
+    expected = oracle.neighbors(points, box, periodic, 5.0, full, False, "ijSdD")
+    calculator = NeighborList(cutoff=5.0, full_list=full)
+    first = call(calculator, points, box, periodic)
+    assert not used_single_pass(calculator)
+    assert_same_list(first, expected, what="first call")
+    for repeat in range(3):
+        again = call(calculator, points, box, periodic)
+        assert used_single_pass(calculator)
+        assert_same_list(again, expected, what=f"call {repeat + 2}")
+
+
+def test_single_pass_is_deterministic(timings):
+    points, box, periodic, _ = configs.config1(12)
+    calculator = NeighborList(cutoff=5.0, full_list=True)
+    call(calculator, points, box, periodic)
+    second = call(calculator, points, box, periodic)
+    third = call(calculator, points, box, periodic)
+    assert used_single_pass(calculator)
+    for key in second:
+        assert np.array_equal(second[key], third[key]), key
+
+
+def test_environment_switch_keeps_the_two_passes(timings):
+    points, box, periodic, _ = configs.config1(8)
+    calculator = NeighborList(cutoff=5.0, full_list=True)
+    call(calculator, points, box, periodic)
+    os.environ["VESIN_HIP_SEARCH"] = "two-pass"
+    try:
+        call(calculator, points, box, periodic)
+        assert not used_single_pass(calculator)
+    finally:
+        del os.environ["VESIN_HIP_SEARCH"]
+    call(calculator, points, box, periodic)
+    assert used_single_pass(calculator)
+
+
+def test_rows_that_do_not_fit_fall_back(timings):
+    # same list, then a system with eight times the rows: the single pass finds the arrays too small, writes nothing
+    # out of bounds, and the two passes start over
+    small = configs.config1(6)
+    large = configs.config1(12)
+    calculator = NeighborList(cutoff=5.0, full_list=True)
+    call(calculator, *small[:3])
+    grown = call(calculator, *large[:3])
+    assert not used_single_pass(calculator)
+    assert_same_list(grown, oracle.neighbors(*large[:3], 5.0, True, False, "ijSdD"), what="grown")
+    # and back: the small system now fits with room to spare
+    shrunk = call(calculator, *small[:3])
+    assert used_single_pass(calculator)
+    assert_same_list(shrunk, oracle.neighbors(*small[:3], 5.0, True, False, "ijSdD"), what="shrunk")
+
+
+def test_crowded_tiles_are_left_to_the_write_pass(timings):
+    # a dense blob inside a sparse gas: tiles of the blob see more candidates than the single pass keeps columns
+    # for; they are counted and placed by it and written by the write pass
+    rng = np.random.default_rng(21)
+    gas = rng.random((4000, 3)) * 40.0
+    blob = rng.random((1500, 3)) * 3.0 + 18.0
+    points = np.concatenate([gas, blob])
+    box = np.eye(3) * 40.0
+    expected = oracle.neighbors(points, box, True, 2.5, True, False, "ijSdD")
+    calculator = NeighborList(cutoff=2.5, full_list=True)
+    first = call(calculator, points, box, True)
+    second = call(calculator, points, box, True)
+    assert used_single_pass(calculator)
+    assert_same_list(first, expected, what="two-pass")
+    assert_same_list(second, expected, what="single pass with deferred tiles")
+
+
+def test_shifts_beyond_the_packing_fall_back():
+    # points thousands of boxes away: their shifts do not fit the 10-bit fields of the single pass
+    rng = np.random.default_rng(6)
+    points, box, periodic = systems.read_xyz("carbon")
+    points = points + rng.integers(-3000, 3000, size=(len(points), 3)).astype(float) @ box
+    expected = oracle.neighbors(points, box, periodic, 5.0, True, False, "ijSdD")
+    calculator = NeighborList(cutoff=5.0, full_list=True)
+    for repeat in range(3):
+        assert_same_list(call(calculator, points, box, periodic), expected, what=f"call {repeat + 1}")
+
+
+@pytest.mark.parametrize("letters", ["P", "PS", "Pd", "PD", "PSdD"])
+def test_single_pass_with_every_output(letters):
+    points, box, periodic = systems.read_xyz("carbon")
+    quantities = "ij" + letters[1:]
+    expected = oracle.neighbors(points, box, periodic, 4.0, True, False, "ijSdD")
+    calculator = NeighborList(cutoff=4.0, full_list=True)
+    call(calculator, points, box, periodic, letters)
+    again = call(calculator, points, box, periodic, letters)
+    if "S" in letters:
+        assert_same_list(again, {k: v for k, v in expected.items() if k in again}, what=quantities)
+    else:
+        # without shifts the images of one pair have no order of their own: compare as multisets
+        assert len(again["pairs"]) == len(expected["pairs"])
+        keys = ["pairs"] + [k for k in ("distances", "vectors") if k in again]
+        for key in keys:
+            a = np.sort(again[key].reshape(len(again["pairs"]), -1), axis=0)
+            b = np.sort(expected[key].reshape(len(expected["pairs"]), -1), axis=0)
+            assert np.array_equal(a, b), key
+
+
+def test_wrapped_tiles_in_the_single_pass(timings):
+    # half of the points sit one or two boxes away: their tiles take the per-point shift path of both searches
+    rng = np.random.default_rng(9)
+    points, box, periodic, _ = configs.config1(6)
+    points = points + rng.integers(-2, 3, size=(len(points), 3)).astype(float) @ box
+    expected = oracle.neighbors(points, box, periodic, 5.0, False, False, "ijSdD")
+    calculator = NeighborList(cutoff=5.0, full_list=False)
+    call(calculator, points, box, periodic)
+    again = call(calculator, points, box, periodic)
+    assert used_single_pass(calculator)
+    assert_same_list(again, expected)

@@ -12,6 +12,18 @@
 
 namespace vesin_hip {
 
+/// What the single-pass search kernel tells the host besides the rows themselves.
+struct FusedStatus {
+    unsigned long long total_rows; // written by the last workgroup
+    unsigned long long deferred_rows; // rows of the deferred work items
+    unsigned int general;          // work items outside of the shape that kernel covers
+    unsigned int deferred;         // work items that kernel counted and placed but left to the write pass
+    unsigned int overflow;         // workgroups whose rows did not fit the output arrays
+    unsigned int chain_timeout;    // waves that gave up waiting for an earlier workgroup
+    unsigned int first_bad_coordinate;
+    unsigned int padding;
+};
+
 /// Cell-sorted copy of the points, one array per component: 64 consecutive candidates load coalesced, and four
 /// consecutive points of a tile arrive with one scalar load per component. x, y, z and index are allocated with
 /// SORTED_PADDING extra elements so that those scalar loads may run past the last point.
@@ -49,6 +61,15 @@ __global__ void publish_status(const DeviceStatus* status, const uint64_t* total
     if (threadIdx.x == 0 && blockIdx.x == 0) {
         host_status->first_bad_coordinate = status->first_bad_coordinate;
         host_status->total_pairs = *total;
+    }
+}
+
+/// Same after the single-pass search.
+__global__ void publish_fused_status(const DeviceStatus* status, const FusedStatus* fused, FusedStatus* host_fused) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        FusedStatus copy = *fused;
+        copy.first_bad_coordinate = status->first_bad_coordinate;
+        *host_fused = copy;
     }
 }
 

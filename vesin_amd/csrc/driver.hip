@@ -9,6 +9,7 @@
 
 #include <cerrno>
 #include <cmath>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 
@@ -21,6 +22,7 @@
 #include "cells.cuh"
 #include "device_common.cuh"
 #include "driver.hpp"
+#include "fused.cuh"
 #include "geometry.hpp"
 #include "scan.cuh"
 #include "search.cuh"
@@ -40,6 +42,12 @@ static std::atomic<bool> TIMINGS_ENABLED{false};
 
 void enable_timings(bool enabled) {
     TIMINGS_ENABLED.store(enabled);
+}
+
+/// VESIN_HIP_SEARCH=two-pass keeps every call on the count / scan / write sequence (for comparisons and tests).
+static bool two_pass_only() {
+    const char* text = std::getenv("VESIN_HIP_SEARCH");
+    return text != nullptr && std::strcmp(text, "two-pass") == 0;
 }
 
 namespace {
@@ -83,6 +91,8 @@ struct Carver {
     }
 };
 
+constexpr int SINGLE_PASS_REST = 64;
+
 enum Stage { T_START = 0, T_CELLS, T_COUNT, T_SCAN, T_WRITE_BEGIN, T_WRITE, T_SORT, T_STAGES };
 
 /// Private state of one VesinNeighborList (VesinNeighborList::opaque).
@@ -94,7 +104,9 @@ struct HipExtras {
     DeviceStatus* h_status = nullptr; // pinned
     unsigned char* h_small = nullptr; // pinned: box (72 bytes) + periodic (3 bytes)
     BlockBounds* h_bounds = nullptr;  // pinned: one slot per workgroup of the bounding pass
+    FusedStatus* h_fused = nullptr;   // pinned
     size_t capacity = 0;              // rows every allocated output array can hold
+    int single_pass_rest = 0;         // calls left before the single-pass search is tried again after it did not fit
     hipEvent_t events[T_STAGES] = {};
     bool have_events = false;
     bool timings_valid = false;
@@ -115,6 +127,9 @@ struct HipExtras {
         if (h_bounds != nullptr) {
             (void)hipHostFree(h_bounds);
         }
+        if (h_fused != nullptr) {
+            (void)hipHostFree(h_fused);
+        }
         if (have_events) {
             for (auto& event : events) {
                 (void)hipEventDestroy(event);
@@ -134,6 +149,7 @@ HipExtras& extras_of(VesinNeighborList& neighbors) {
         HIP_CHECK(hipHostMalloc(
             reinterpret_cast<void**>(&extras->h_bounds), BOUNDING_BLOCKS * sizeof(BlockBounds), hipHostMallocDefault
         ));
+        HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&extras->h_fused), sizeof(FusedStatus), hipHostMallocDefault));
     }
     return *static_cast<HipExtras*>(neighbors.opaque);
 }
@@ -422,7 +438,11 @@ void neighbors(
     const size_t search_blocks = tiles_bound * n_slices;
     const size_t n_slots = search_blocks;
 
+    const size_t search_workgroups = (search_blocks + SEARCH_WAVES - 1) / SEARCH_WAVES;
     uint32_t* cell_counts = nullptr;
+    const size_t chain_groups = (search_workgroups + CHAIN_GROUP - 1) / CHAIN_GROUP;
+    Chain chain = {};
+    FusedStatus* fused_status = nullptr;
     uint64_t* cell_scan = nullptr;
     uint32_t* cell_of = nullptr;
     uint32_t* slot_of = nullptr;
@@ -436,9 +456,13 @@ void neighbors(
     const size_t scratch_elements = std::max(scan_scratch_elements(n_cells), scan_scratch_elements(n_slots));
 
     auto carve = [&](Carver& carver) {
-        // cell_counts and tiles are adjacent: one fill clears the histogram and the tiles' flags
+        // adjacent, so that one fill clears the histogram, the tiles' flags and the state of the single-pass search
         cell_counts = carver.take<uint32_t>(n_cells);
         tiles = carver.take<Tile>(tiles_bound);
+        chain.blocks = carver.take<uint64_t>(search_workgroups);
+        chain.groups = carver.take<uint64_t>(chain_groups);
+        chain.bases = carver.take<uint64_t>(chain_groups);
+        fused_status = carver.take<FusedStatus>(1);
         cell_scan = carver.take<uint64_t>(n_cells + 1);
         if (!single_cell) {
             cell_of = carver.take<uint32_t>(n_points);
@@ -466,14 +490,16 @@ void neighbors(
     // ---- cell list
     const uint32_t point_blocks = static_cast<uint32_t>((n_points + BLOCK - 1) / BLOCK);
     const auto* flat_points = reinterpret_cast<const double*>(points);
+    {
+        const size_t to_clear = reinterpret_cast<char*>(fused_status + 1) - reinterpret_cast<char*>(cell_counts);
+        HIP_CHECK(hipMemsetAsync(cell_counts, 0, to_clear, stream));
+    }
     if (single_cell) {
         hipLaunchKernelGGL(
             prepare_single_cell, dim3(point_blocks), dim3(BLOCK), 0, stream,
             flat_points, g, sorted, tiles, cell_scan, extras.d_status
         );
     } else {
-        const size_t to_clear = reinterpret_cast<char*>(tiles + tiles_bound) - reinterpret_cast<char*>(cell_counts);
-        HIP_CHECK(hipMemsetAsync(cell_counts, 0, to_clear, stream));
         hipLaunchKernelGGL(
             assign_cells, dim3(point_blocks), dim3(BLOCK), 0, stream,
             flat_points, g, cell_of, slot_of, wrap_of, cell_counts, extras.d_status
@@ -490,7 +516,6 @@ void neighbors(
     }
     mark(T_CELLS);
 
-    // ---- pass 1: count
     SearchArgs args = {};
     args.sorted = sorted;
     args.cell_scan = cell_scan;
@@ -499,13 +524,6 @@ void neighbors(
     args.offsets = offsets;
     args.n_slices = n_slices;
     args.n_work = static_cast<uint32_t>(search_blocks);
-    launch_search<false>(options.full, args, g, stream);
-    mark(T_COUNT);
-
-    exclusive_scan<SCAN_U32>(counts, n_slots, offsets, scan_scratch, stream);
-    mark(T_SCAN);
-
-    hipLaunchKernelGGL(publish_status, dim3(1), dim3(1), 0, stream, extras.d_status, offsets + n_slots, extras.h_status);
 
     auto outputs_of = [&]() {
         SearchOutputs out;
@@ -515,6 +533,102 @@ void neighbors(
         out.vectors = reinterpret_cast<double*>(neighbors.vectors);
         return out;
     };
+    auto check_pair_limit = [&](size_t total) {
+        if (pair_limit != 0 && total > n_points * pair_limit) {
+            throw std::runtime_error(
+                "The number of neighbor pairs exceeds the maximum capacity of " + std::to_string(n_points * pair_limit) +
+                " (max_pairs_per_point=" + std::to_string(pair_limit) + "; n_points=" + std::to_string(n_points) + "). " +
+                "Consider reducing the cutoff distance, or explicitly setting " +
+                "VESIN_CUDA_MAX_PAIRS_PER_POINT as an environment variable."
+            );
+        }
+    };
+    auto elapsed = [&](Stage from, Stage to) {
+        float ms = 0.0f;
+        HIP_CHECK(hipEventElapsedTime(&ms, extras.events[from], extras.events[to]));
+        return ms;
+    };
+
+    // ---- single-pass search straight into the arrays kept from earlier calls. It does not cover every shape of
+    // problem and the rows may not fit: in both cases nothing is lost but time, the two passes below start over.
+    bool try_single_pass = !options.sorted && extras.capacity > 0 && !two_pass_only();
+    if (try_single_pass && extras.single_pass_rest > 0) {
+        extras.single_pass_rest -= 1;
+        try_single_pass = false;
+    }
+    if (try_single_pass) {
+        size_outputs(neighbors, extras, 0, options);
+        FusedArgs fargs = {};
+        fargs.search = args;
+        fargs.search.out = outputs_of();
+        fargs.search.capacity = extras.capacity;
+        fargs.chain = chain;
+        fargs.first_rows = offsets;
+        fargs.status = fused_status;
+        const uint32_t blocks = static_cast<uint32_t>(search_workgroups);
+        if (options.full) {
+            hipLaunchKernelGGL(fused_search_kernel<true>, dim3(blocks), dim3(SEARCH_BLOCK), 0, stream, fargs, g);
+        } else {
+            hipLaunchKernelGGL(fused_search_kernel<false>, dim3(blocks), dim3(SEARCH_BLOCK), 0, stream, fargs, g);
+        }
+        mark(T_WRITE);
+        hipLaunchKernelGGL(publish_fused_status, dim3(1), dim3(1), 0, stream, extras.d_status, fused_status, extras.h_fused);
+        HIP_CHECK(hipStreamSynchronize(stream));
+        const FusedStatus result = *extras.h_fused;
+        if (result.first_bad_coordinate != 0xFFFFFFFFu) {
+            non_finite_error(points, result.first_bad_coordinate);
+        }
+        if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
+            std::fprintf(
+                stderr, "single pass: rows %llu general %u deferred %u overflow %u timeout %u (cells %u %u %u, capacity %zu)\n",
+                result.total_rows, result.general, result.deferred, result.overflow, result.chain_timeout, g.n[0], g.n[1], g.n[2],
+                extras.capacity
+            );
+        }
+        if (result.chain_timeout != 0) {
+            throw std::runtime_error("internal error: the single-pass search gave up waiting for an earlier workgroup");
+        }
+        if (result.general == 0 && result.overflow == 0) {
+            check_pair_limit(result.total_rows);
+            if (result.deferred != 0) {
+                // work items too large for the single pass: their rows are counted and placed, the write pass of
+                // the two-pass search produces them
+                SearchArgs rest = fargs.search;
+                rest.only = counts;
+                rest.capacity = ~0ull;
+                launch_search<true>(options.full, rest, g, stream);
+                mark(T_WRITE);
+                HIP_CHECK(hipStreamSynchronize(stream));
+                if (result.deferred_rows > result.total_rows / 8) {
+                    // a system dominated by crowded tiles is searched twice this way: the two passes do better
+                    extras.single_pass_rest = SINGLE_PASS_REST;
+                }
+            }
+            HIP_CHECK(hipGetLastError());
+            neighbors.length = result.total_rows;
+            if (timed) {
+                extras.timings = {};
+                extras.timings.total = elapsed(T_START, T_WRITE);
+                extras.timings.cell_build = elapsed(T_START, T_CELLS);
+                extras.timings.write = elapsed(T_CELLS, T_WRITE);
+                extras.timings_valid = true;
+            }
+            return;
+        }
+        if (result.general != 0) {
+            // the shape of this system is not the single-pass kernel's: leave it alone for a while
+            extras.single_pass_rest = SINGLE_PASS_REST;
+        }
+    }
+
+    // ---- pass 1: count
+    launch_search<false>(options.full, args, g, stream);
+    mark(T_COUNT);
+
+    exclusive_scan<SCAN_U32>(counts, n_slots, offsets, scan_scratch, stream);
+    mark(T_SCAN);
+
+    hipLaunchKernelGGL(publish_status, dim3(1), dim3(1), 0, stream, extras.d_status, offsets + n_slots, extras.h_status);
 
     // ---- pass 2: write. Without sorting the rows go straight to the caller's arrays, and the launch does not
     // wait for the host to learn their number: the arrays keep the capacity of earlier calls, and a launch that
@@ -535,14 +649,7 @@ void neighbors(
     }
     const size_t total = extras.h_status->total_pairs;
 
-    if (pair_limit != 0 && total > n_points * pair_limit) {
-        throw std::runtime_error(
-            "The number of neighbor pairs exceeds the maximum capacity of " + std::to_string(n_points * pair_limit) +
-            " (max_pairs_per_point=" + std::to_string(pair_limit) + "; n_points=" + std::to_string(n_points) + "). " +
-            "Consider reducing the cutoff distance, or explicitly setting " +
-            "VESIN_CUDA_MAX_PAIRS_PER_POINT as an environment variable."
-        );
-    }
+    check_pair_limit(total);
 
     const bool fits = total <= extras.capacity;
     size_outputs(neighbors, extras, total, options);
@@ -598,11 +705,6 @@ void neighbors(
     neighbors.length = total;
 
     if (timed) {
-        auto elapsed = [&](Stage from, Stage to) {
-            float ms = 0.0f;
-            HIP_CHECK(hipEventElapsedTime(&ms, extras.events[from], extras.events[to]));
-            return ms;
-        };
         extras.timings.total = elapsed(T_START, T_SORT);
         extras.timings.cell_build = elapsed(T_START, T_CELLS);
         extras.timings.count = elapsed(T_CELLS, T_COUNT);

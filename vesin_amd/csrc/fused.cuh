@@ -1,0 +1,791 @@
+// Single-pass stencil search: count, place and write the rows of every tile in one kernel.
+//
+// The two-pass search (search.cuh) evaluates every candidate pair twice, once to count and once to write, with a
+// device-wide scan between the two launches. Here a wave keeps the outcome of its tests instead: while it sweeps the
+// tile's points over 64 candidates held in registers, every candidate lane shifts the hit bit of each tile point into
+// a 64-bit column (one v_addc per test, fed by the compare's lane mask). After the sweep the wave knows its number of
+// rows; the workgroups then chain their totals (64-bit words holding a flag and a value, written and polled with
+// device-scope atomics; decoupled look-back over groups of workgroups), which hands every wave its first output row.
+// The wave finally replays its columns: each round every lane with hits left peels one bit off its column and drops
+// a ticket (candidate slot, tile point) into the wave's LDS ring; whenever 64 tickets are pending all lanes redeem
+// one each, exactly like the write pass of the two-pass search, and store dense rows.
+//
+// A workgroup waits only for workgroups with a smaller index, which the hardware started earlier, so the chain always
+// advances; the wait is bounded anyway, and a wave that runs out of patience raises a flag for the host instead of
+// spinning for ever.
+//
+// A work item with more than FUSED_UNITS x 64 candidates cannot keep its columns: it is swept and counted here, its
+// rows are placed by the chain like all others, and its first row goes to `offsets` with a mark in `counts`; the
+// host then launches the write pass of the two-pass search for the marked work items only.
+//
+// This kernel covers the common shape of the problem: at most MAX_ENTRIES stencil entries, shifts that fit the
+// 10-bit packing. A work item outside of that shape raises the `general` count and produces nothing; the host then
+// runs the two-pass search for the whole call.
+//
+// Arithmetic and row conventions are those of search.cuh.
+#ifndef VESIN_HIP_FUSED_CUH
+#define VESIN_HIP_FUSED_CUH
+
+#include "search.cuh"
+
+namespace vesin_hip {
+
+constexpr int FUSED_UNITS = 8;          // 64-candidate units of one work item whose columns stay in registers
+constexpr int FUSED_SLOTS = 2 * WAVE;   // candidate records in LDS: two units, so that tickets survive a unit change
+constexpr int32_t PACKED_SHIFT_LIMIT = 500;
+constexpr uint32_t CHAIN_SPIN_LIMIT = 1u << 18;
+constexpr uint32_t CHAIN_GROUP = 32;    // workgroups per group of the chain (at most 64)
+
+constexpr uint64_t CHAIN_FLAG_SHIFT = 62;
+constexpr uint64_t CHAIN_AGGREGATE = 1ull << CHAIN_FLAG_SHIFT; // value = rows of this workgroup
+constexpr uint64_t CHAIN_PREFIX = 2ull << CHAIN_FLAG_SHIFT;    // value = rows of this and all earlier workgroups
+constexpr uint64_t CHAIN_VALUE = (1ull << CHAIN_FLAG_SHIFT) - 1;
+
+/// The words through which the workgroups learn where their rows start; all zero on entry.
+struct Chain {
+    uint64_t* blocks; // [workgroups]: flag | rows of the workgroup
+    uint64_t* groups; // [groups]: flag | rows of the group, later of all groups up to this one
+    uint64_t* bases;  // [groups]: flag | rows of all earlier groups
+};
+
+struct FusedArgs {
+    SearchArgs search;
+    uint64_t* first_rows; // [work items]: first output row of the work items left to the write pass
+    Chain chain;
+    FusedStatus* status; // zero on entry
+};
+
+/// LDS of one wave.
+struct FusedWaveShared: SearchTables {
+    double tile_x[WAVE], tile_y[WAVE], tile_z[WAVE];
+    uint32_t tile_index[WAVE];
+    int32_t tile_wx[WAVE], tile_wy[WAVE], tile_wz[WAVE];
+    double cand_x[FUSED_SLOTS], cand_y[FUSED_SLOTS], cand_z[FUSED_SLOTS];
+    uint32_t cand_index[FUSED_SLOTS];
+    int32_t cand_shift[FUSED_SLOTS]; // packed: cell shift minus the candidate's own wrap shift
+    uint16_t ring[RING];
+};
+
+struct FusedShared {
+    FusedWaveShared wave[SEARCH_WAVES];
+    uint32_t rows[SEARCH_WAVES];
+    uint64_t base;     // first output row of the workgroup
+    uint32_t writable; // the workgroup's rows fit the output arrays
+};
+
+/// col = 2 * col + (this lane's bit of mask): one VALU instruction, the mask is the carry-in.
+__device__ __forceinline__ uint32_t shift_in(uint32_t col, uint64_t mask) {
+    uint32_t result;
+    uint64_t carry_out;
+    asm("v_addc_co_u32_e64 %0, %1, %2, %2, %3" : "=v"(result), "=s"(carry_out) : "v"(col), "s"(mask));
+    return result;
+}
+
+/// One candidate per lane: where it is, what it is shifted by.
+struct UnitCandidates {
+    uint32_t at;     // position in the cell-sorted arrays (valid lanes)
+    int32_t bx, by, bz;
+    bool valid;
+    bool same_cell;  // from the tile's own cell with a zero cell shift
+};
+
+__device__ __forceinline__ UnitCandidates locate_unit(
+    const SearchTables& sh, uint32_t n_batch, uint32_t n_candidates, uint32_t k, const SortedPoints& sorted
+) {
+    UnitCandidates u;
+    u.valid = k < n_candidates;
+    u.at = 0;
+    u.bx = u.by = u.bz = 0;
+    u.same_cell = false;
+    if (u.valid) {
+        int32_t packed;
+        locate_candidate(sh, n_batch, k, u.at, packed);
+        int32_t qx, qy, qz;
+        unpack_shift(packed, qx, qy, qz);
+        u.same_cell = (packed >> 30) & 1;
+        u.bx = qx - sorted.wx[u.at];
+        u.by = qy - sorted.wy[u.at];
+        u.bz = qz - sorted.wz[u.at];
+    }
+    return u;
+}
+
+/// Registers of the sweep: R x 64 candidates.
+template <int R>
+struct SweepCandidates {
+    double x[R], y[R], z[R];
+    double tx[R], ty[R], tz[R];
+    int32_t shift[R];      // packed
+    uint32_t position[R];  // see Candidates::position
+};
+
+/// Up to 32 consecutive tile points (from cell-sorted position `first`) against the R x 64 candidates; every
+/// candidate lane shifts its hit bits into `column` (the first point ends up in the highest bit used). Returns the
+/// number of hits.
+template <int R, bool SHIFTED, bool SAME>
+__device__ __forceinline__ uint32_t sweep_half(
+    const SortedPoints& sorted, uint32_t first, uint32_t count, const SweepCandidates<R>& c, double cutoff2,
+    uint32_t (&column)[R]
+) {
+    uint32_t total = 0;
+    for (uint32_t i0 = 0; i0 < count; i0 += POINTS_PER_LOAD) {
+        const uint32_t at = first + i0;
+        const FourPoints p = load_four_points(sorted.x + at, sorted.y + at, sorted.z + at);
+#pragma unroll
+        for (int u = 0; u < POINTS_PER_LOAD; u++) {
+            if (u > 0 && i0 + u >= count) {
+                break;
+            }
+            const double xi = words_to_double(p.x[2 * u], p.x[2 * u + 1]);
+            const double yi = words_to_double(p.y[2 * u], p.y[2 * u + 1]);
+            const double zi = words_to_double(p.z[2 * u], p.z[2 * u + 1]);
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                double vx = c.x[r] - xi;
+                double vy = c.y[r] - yi;
+                double vz = c.z[r] - zi;
+                if (SHIFTED) {
+                    vx += c.tx[r];
+                    vy += c.ty[r];
+                    vz += c.tz[r];
+                }
+                const double d2 = vx * vx + vy * vy + vz * vz;
+                uint64_t mask = __ballot(d2 < cutoff2);
+                if (SAME) {
+                    mask &= __ballot(c.position[r] > at + u);
+                }
+                total += __popcll(mask);
+                column[r] = shift_in(column[r], mask);
+            }
+        }
+    }
+    return total;
+}
+
+/// Every tile point against the R x 64 candidates: points 0..31 go to the `lo` columns, 32..63 to `hi`.
+template <int R, bool SHIFTED, bool SAME>
+__device__ __forceinline__ uint32_t sweep_columns(
+    const SortedPoints& sorted, uint32_t first_i, uint32_t n_i, const SweepCandidates<R>& c, double cutoff2,
+    uint32_t (&lo)[R], uint32_t (&hi)[R]
+) {
+    uint32_t total = sweep_half<R, SHIFTED, SAME>(sorted, first_i, min(n_i, 32u), c, cutoff2, lo);
+    if (n_i > 32) {
+        total += sweep_half<R, SHIFTED, SAME>(sorted, first_i + 32, n_i - 32, c, cutoff2, hi);
+    }
+    return total;
+}
+
+/// Variant for a tile holding points that were wrapped into the box: the shift of a pair depends on both points.
+template <int R>
+__device__ __forceinline__ uint32_t sweep_columns_wrapped(
+    const SortedPoints& sorted, uint32_t first_i, uint32_t n_i, const SweepCandidates<R>& c, const GridParams& g,
+    uint32_t (&lo)[R], uint32_t (&hi)[R]
+) {
+    uint32_t total = 0;
+    for (uint32_t i = 0; i < n_i; i++) {
+        if (i == 32) {
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                hi[r] = lo[r];
+                lo[r] = 0;
+            }
+        }
+        const uint32_t at = first_i + i;
+        const double xi = sorted.x[at];
+        const double yi = sorted.y[at];
+        const double zi = sorted.z[at];
+        const int32_t wix = sorted.wx[at];
+        const int32_t wiy = sorted.wy[at];
+        const int32_t wiz = sorted.wz[at];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            int32_t bx, by, bz;
+            unpack_shift(c.shift[r], bx, by, bz);
+            double tx, ty, tz;
+            shift_vector(g, bx + wix, by + wiy, bz + wiz, tx, ty, tz);
+            const double vx = (c.x[r] - xi) + tx;
+            const double vy = (c.y[r] - yi) + ty;
+            const double vz = (c.z[r] - zi) + tz;
+            const double d2 = vx * vx + vy * vy + vz * vz;
+            const uint64_t mask = __ballot(d2 < g.cutoff2) & __ballot(c.position[r] > at);
+            total += __popcll(mask);
+            lo[r] = shift_in(lo[r], mask);
+        }
+    }
+    if (n_i > 32) {
+        // the first 32 points were parked in `hi` while the rest went through `lo`
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const uint32_t rest = lo[r];
+            lo[r] = hi[r];
+            hi[r] = rest;
+        }
+    }
+    return total;
+}
+
+/// Constants of the replay phase of one work item.
+struct ReplayContext {
+    double zero_tx, zero_ty, zero_tz;
+    bool need_shift;   // some candidate of the work item has a non-zero shift, or the tile holds wrapped points
+    bool tile_wrapped;
+    int lane;
+};
+
+struct ReplayState {
+    uint64_t out_cursor;
+    uint32_t head;
+    uint32_t tail;
+    uint32_t batch; // tickets the next redeem takes: 64, or fewer to bring the cursor to a multiple of ROW_ALIGN
+};
+
+/// Stores of 64 consecutive rows are fastest when they start on whole cache lines in all three arrays (16, 12 and
+/// 8 bytes per row): at multiples of 32 rows. A wave's first row is wherever the rows before it ended, so its first
+/// redeem takes just enough tickets to reach such a boundary.
+constexpr uint32_t ROW_ALIGN = 32;
+
+template <bool FULL>
+__device__ __forceinline__ uint32_t aligning_batch(uint64_t cursor) {
+    const uint32_t off = static_cast<uint32_t>(cursor) & (ROW_ALIGN - 1);
+    if (off == 0) {
+        return WAVE;
+    }
+    // a full list writes two rows per ticket (its cursor is always even)
+    return FULL ? (ROW_ALIGN - off) / 2 : ROW_ALIGN - off;
+}
+
+/// Redeem n <= 64 tickets: same rows as `redeem` of the two-pass search, candidates and tile points read from LDS.
+template <bool FULL>
+__device__ __forceinline__ void redeem_fused(
+    uint32_t n, ReplayState& state, FusedWaveShared& sh, const SearchOutputs& out, const GridParams& g,
+    const ReplayContext& ctx
+) {
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    const int lane = ctx.lane;
+    const bool active = static_cast<uint32_t>(lane) < n;
+    const uint32_t ticket = sh.ring[(state.tail + lane) & (RING - 1)];
+    const int slot = active ? ticket & (FUSED_SLOTS - 1) : 0;
+    const int il = active ? (ticket >> 8) & 63 : 0;
+
+    const double xj = sh.cand_x[slot];
+    const double yj = sh.cand_y[slot];
+    const double zj = sh.cand_z[slot];
+    const uint32_t oj = sh.cand_index[slot];
+    const double xi = sh.tile_x[il];
+    const double yi = sh.tile_y[il];
+    const double zi = sh.tile_z[il];
+    const uint32_t oi = sh.tile_index[il];
+
+    int32_t sx = 0, sy = 0, sz = 0;
+    double tx = ctx.zero_tx, ty = ctx.zero_ty, tz = ctx.zero_tz;
+    double mx = ctx.zero_tx, my = ctx.zero_ty, mz = ctx.zero_tz;
+    if (ctx.need_shift) {
+        unpack_shift(sh.cand_shift[slot], sx, sy, sz);
+        if (ctx.tile_wrapped) {
+            sx += sh.tile_wx[il];
+            sy += sh.tile_wy[il];
+            sz += sh.tile_wz[il];
+        }
+        shift_vector(g, sx, sy, sz, tx, ty, tz);
+        if ((sx | sy | sz) != 0) {
+            mx = -tx;
+            my = -ty;
+            mz = -tz;
+        }
+    }
+    const double vx = (xj - xi) + tx;
+    const double vy = (yj - yi) + ty;
+    const double vz = (zj - zi) + tz;
+    const double wx = (xi - xj) + mx;
+    const double wy = (yi - yj) + my;
+    const double wz = (zi - zj) + mz;
+    const double d2 = vx * vx + vy * vy + vz * vz;
+
+    if (FULL) {
+        if (active) {
+            const uint64_t forward_row = state.out_cursor + lane;
+            const uint64_t mirror_row = forward_row + n;
+            ulonglong2 forward, backward;
+            forward.x = oi;
+            forward.y = oj;
+            backward.x = oj;
+            backward.y = oi;
+            reinterpret_cast<ulonglong2*>(out.pairs)[forward_row] = forward;
+            reinterpret_cast<ulonglong2*>(out.pairs)[mirror_row] = backward;
+            if (out.shifts != nullptr) {
+                int32_t* s = out.shifts + 3 * forward_row;
+                s[0] = sx;
+                s[1] = sy;
+                s[2] = sz;
+                int32_t* m = out.shifts + 3 * mirror_row;
+                m[0] = -sx;
+                m[1] = -sy;
+                m[2] = -sz;
+            }
+            if (out.distances != nullptr) {
+                const double d = sqrt(d2);
+                out.distances[forward_row] = d;
+                out.distances[mirror_row] = d;
+            }
+            if (out.vectors != nullptr) {
+                double* v = out.vectors + 3 * forward_row;
+                v[0] = vx;
+                v[1] = vy;
+                v[2] = vz;
+                double* m = out.vectors + 3 * mirror_row;
+                m[0] = wx;
+                m[1] = wy;
+                m[2] = wz;
+            }
+        }
+        state.out_cursor += 2 * n;
+    } else {
+        const bool flip = oi > oj || (oi == oj && !half_keeps_self_image(sx, sy, sz));
+        if (active) {
+            const uint64_t row = state.out_cursor + lane;
+            ulonglong2 pair;
+            pair.x = flip ? oj : oi;
+            pair.y = flip ? oi : oj;
+            reinterpret_cast<ulonglong2*>(out.pairs)[row] = pair;
+            if (out.shifts != nullptr) {
+                int32_t* s = out.shifts + 3 * row;
+                s[0] = flip ? -sx : sx;
+                s[1] = flip ? -sy : sy;
+                s[2] = flip ? -sz : sz;
+            }
+            if (out.distances != nullptr) {
+                out.distances[row] = sqrt(d2);
+            }
+            if (out.vectors != nullptr) {
+                double* v = out.vectors + 3 * row;
+                v[0] = flip ? wx : vx;
+                v[1] = flip ? wy : vy;
+                v[2] = flip ? wz : vz;
+            }
+        }
+        state.out_cursor += n;
+    }
+    state.tail += n;
+    state.batch = aligning_batch<FULL>(state.out_cursor);
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+/// What one wave carries from the sweep to the replay.
+struct WorkItem {
+    bool valid;          // there is a tile for this work item and it fits the shape of this kernel
+    bool deferred;       // too many candidates to keep the columns: counted here, written by the write pass
+    bool any_shift;
+    bool tile_wrapped;
+    uint32_t first_i, n_i;
+    uint32_t n_batch, n_candidates;
+    uint32_t unit_begin, n_units;
+    uint32_t hits;
+};
+
+__device__ __forceinline__ uint64_t chain_load(const uint64_t* word) {
+    return __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ void chain_store(uint64_t* word, uint64_t value) {
+    __hip_atomic_store(word, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+/// Bounded wait between two polls of the chain; returns false when patience ran out.
+__device__ __forceinline__ bool chain_wait(uint32_t& spins, int lane, FusedStatus* status) {
+    spins += 1;
+    if (spins > CHAIN_SPIN_LIMIT) {
+        if (lane == 0) {
+            atomicAdd(&status->chain_timeout, 1u);
+        }
+        return false;
+    }
+    __builtin_amdgcn_s_sleep(8);
+    return true;
+}
+
+/// Sum of the rows of all earlier workgroups. Called by one full wave of every workgroup.
+///
+/// Two levels keep the polling light. Every workgroup publishes its rows in `chain.blocks`. Workgroups form groups
+/// of CHAIN_GROUP consecutive ones; the last workgroup of a group waits for the rows of the others, publishes the
+/// group's rows in `chain.groups`, finds the rows of all earlier groups by decoupled look-back over that (short)
+/// array, and publishes them in `chain.bases`. The other workgroups of the group poll that one word, then add the
+/// rows of the earlier workgroups of their group. Every word carries its own flag, so no fences are needed.
+__device__ __forceinline__ uint64_t chain_position(
+    const Chain& chain, uint32_t block, uint32_t n_blocks, uint64_t own_rows, int lane, FusedStatus* status
+) {
+    if (lane == 0) {
+        chain_store(&chain.blocks[block], CHAIN_AGGREGATE | own_rows);
+    }
+    const uint32_t group = block / CHAIN_GROUP;
+    const uint32_t group_first = group * CHAIN_GROUP;
+    const uint32_t member = block - group_first;
+    const bool leader = member == CHAIN_GROUP - 1 || block == n_blocks - 1;
+    uint32_t spins = 0;
+
+    uint64_t group_before = 0;
+    if (leader) {
+        // ---- rows of the group: lanes 0..member-1 watch the other workgroups
+        uint64_t rows_of_member = 0;
+        while (true) {
+            uint64_t word = CHAIN_AGGREGATE;
+            if (static_cast<uint32_t>(lane) < member) {
+                word = chain_load(&chain.blocks[group_first + lane]);
+            }
+            rows_of_member = word & CHAIN_VALUE;
+            if (__ballot((word >> CHAIN_FLAG_SHIFT) == 0) == 0 || !chain_wait(spins, lane, status)) {
+                break;
+            }
+        }
+        const uint64_t group_rows = read_lane(wave_inclusive_scan(rows_of_member), WAVE - 1) + own_rows;
+        if (group == 0) {
+            if (lane == 0) {
+                chain_store(&chain.groups[0], CHAIN_PREFIX | group_rows);
+            }
+        } else {
+            if (lane == 0) {
+                chain_store(&chain.groups[group], CHAIN_AGGREGATE | group_rows);
+            }
+            // ---- decoupled look-back over the groups: lane l looks at group nearest - l
+            int64_t nearest = static_cast<int64_t>(group) - 1;
+            bool done = false;
+            while (!done) {
+                const int64_t at = nearest - lane;
+                uint64_t word = CHAIN_PREFIX; // before the first group: nothing
+                if (at >= 0) {
+                    word = chain_load(&chain.groups[at]);
+                }
+                const uint64_t flag = word >> CHAIN_FLAG_SHIFT;
+                const uint64_t is_prefix = __ballot(flag == 2);
+                const uint64_t is_missing = __ballot(flag == 0);
+                // lanes [0, usable) hold aggregates, possibly ended by a prefix
+                const uint32_t first_prefix =
+                    is_prefix != 0 ? __ffsll(static_cast<unsigned long long>(is_prefix)) - 1 : WAVE;
+                const uint32_t first_missing =
+                    is_missing != 0 ? __ffsll(static_cast<unsigned long long>(is_missing)) - 1 : WAVE;
+                const bool reaches_prefix = first_prefix < first_missing;
+                const uint32_t usable = reaches_prefix ? first_prefix + 1 : first_missing;
+
+                uint64_t value = static_cast<uint32_t>(lane) < usable ? (word & CHAIN_VALUE) : 0;
+                value = wave_inclusive_scan(value);
+                group_before += read_lane(value, WAVE - 1);
+                nearest -= usable;
+                if (reaches_prefix) {
+                    done = true;
+                } else if (usable == 0 && !chain_wait(spins, lane, status)) {
+                    done = true;
+                }
+            }
+            if (lane == 0) {
+                chain_store(&chain.groups[group], CHAIN_PREFIX | ((group_before + group_rows) & CHAIN_VALUE));
+            }
+        }
+        if (lane == 0) {
+            chain_store(&chain.bases[group], CHAIN_PREFIX | (group_before & CHAIN_VALUE));
+        }
+        // rows of the earlier workgroups of this group: everything but the own rows
+        return group_before + (group_rows - own_rows);
+    }
+
+    // ---- not the leader: wait for the group's base, then add the earlier members (all published by then)
+    while (true) {
+        const uint64_t word = chain_load(&chain.bases[group]);
+        if ((word >> CHAIN_FLAG_SHIFT) != 0) {
+            group_before = word & CHAIN_VALUE;
+            break;
+        }
+        if (!chain_wait(spins, lane, status)) {
+            break;
+        }
+    }
+    uint64_t rows_of_member = 0;
+    if (static_cast<uint32_t>(lane) < member) {
+        rows_of_member = chain_load(&chain.blocks[group_first + lane]) & CHAIN_VALUE;
+    }
+    return group_before + read_lane(wave_inclusive_scan(rows_of_member), WAVE - 1);
+}
+
+/// Four waves per workgroup, one work item each; they meet twice: to add up their rows, and to learn their place.
+template <bool FULL>
+__global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fargs, GridParams g) {
+    constexpr int R = 2;
+    __shared__ FusedShared shared;
+    const SearchArgs& args = fargs.search;
+    const int lane = lane_id();
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    FusedWaveShared& sh = shared.wave[wave];
+    const uint32_t n_tiles = static_cast<uint32_t>(args.cell_scan[g.n_cells] >> 32);
+    const uint32_t work = blockIdx.x * SEARCH_WAVES + wave;
+    const SortedPoints& sorted = args.sorted;
+
+    WorkItem item;
+    item.valid = false;
+    item.deferred = false;
+    item.any_shift = false;
+    item.tile_wrapped = false;
+    item.hits = 0;
+    item.n_units = 0;
+    item.unit_begin = 0;
+    item.first_i = 0;
+    item.n_i = 0;
+    item.n_batch = 0;
+    item.n_candidates = 0;
+    // hit columns of the work item's units; indexed with wave-uniform values only
+    uint32_t columns_lo[FUSED_UNITS];
+    uint32_t columns_hi[FUSED_UNITS];
+#pragma unroll
+    for (int u = 0; u < FUSED_UNITS; u++) {
+        columns_lo[u] = 0;
+        columns_hi[u] = 0;
+    }
+
+    // ---- phase 1: sweep, keep the columns
+    bool general = false;
+    if (work < args.n_work) {
+        const uint32_t slice = work % args.n_slices;
+        const uint32_t slot = work / args.n_slices;
+        const uint32_t per_xcd = (n_tiles + N_XCD - 1) / N_XCD;
+        const uint32_t xcd = (slot / SEARCH_WAVES) % N_XCD;
+        const uint32_t within = (slot / (SEARCH_WAVES * N_XCD)) * SEARCH_WAVES + slot % SEARCH_WAVES;
+        const uint32_t tile_id = xcd * per_xcd + within;
+
+        if (within < per_xcd && tile_id < n_tiles) {
+            const Tile tile = args.tiles[tile_id];
+            item.n_i = tile.count;
+            item.first_i = tile.first;
+            item.tile_wrapped = tile.wrapped != 0;
+            const int32_t cx = tile.cell % g.n[0];
+            const int32_t cy = (tile.cell / g.n[0]) % g.n[1];
+            const int32_t cz = tile.cell / (g.n[0] * g.n[1]);
+
+            const int32_t span_y = 2 * g.s[1] + 1;
+            const int32_t span_z = 2 * g.s[2] + 1;
+            const uint32_t n_stencil = static_cast<uint32_t>(2 * g.s[0] + 1) * span_y * span_z;
+            const uint32_t centre = n_stencil / 2;
+            const uint32_t n_entries = n_stencil - centre;
+
+            if (n_entries > MAX_ENTRIES) {
+                general = true;
+            } else {
+                if (static_cast<uint32_t>(lane) < item.n_i) {
+                    const uint32_t at = item.first_i + lane;
+                    sh.tile_x[lane] = sorted.x[at];
+                    sh.tile_y[lane] = sorted.y[at];
+                    sh.tile_z[lane] = sorted.z[at];
+                    sh.tile_index[lane] = sorted.index[at];
+                    sh.tile_wx[lane] = sorted.wx[at];
+                    sh.tile_wy[lane] = sorted.wy[at];
+                    sh.tile_wz[lane] = sorted.wz[at];
+                }
+                item.n_batch = n_entries;
+                fill_stencil_tables(sh, lane, centre, n_entries, cx, cy, cz, span_y, span_z, g, args.cell_scan);
+                item.n_candidates = __builtin_amdgcn_readfirstlane(sh.n_candidates);
+
+                const uint32_t n_groups = (item.n_candidates + WAVE * R - 1) / (WAVE * R);
+                const uint32_t per_slice = (n_groups + args.n_slices - 1) / args.n_slices;
+                const uint32_t group_begin = min(n_groups, slice * per_slice);
+                const uint32_t group_end = min(n_groups, group_begin + per_slice);
+                item.unit_begin = group_begin * R;
+                item.n_units = (group_end - group_begin) * R;
+                item.deferred = item.n_units > FUSED_UNITS;
+            }
+
+            if (!general) {
+                item.valid = true;
+                for (uint32_t pair = 0; pair < item.n_units / R; pair++) {
+                    SweepCandidates<R> c;
+                    bool any_shift = false;
+                    bool any_same = false;
+                    bool too_far = false;
+#pragma unroll
+                    for (int r = 0; r < R; r++) {
+                        const uint32_t k = (item.unit_begin + pair * R + r) * WAVE + lane;
+                        const UnitCandidates u = locate_unit(sh, item.n_batch, item.n_candidates, k, sorted);
+                        c.x[r] = c.y[r] = c.z[r] = __builtin_nan("");
+                        c.tx[r] = c.ty[r] = c.tz[r] = 0.0;
+                        c.position[r] = 0xFFFFFFFFu;
+                        if (u.valid) {
+                            c.x[r] = sorted.x[u.at];
+                            c.y[r] = sorted.y[u.at];
+                            c.z[r] = sorted.z[u.at];
+                            if (u.same_cell) {
+                                c.position[r] = u.at;
+                            }
+                        }
+                        c.shift[r] = pack_shift(u.bx, u.by, u.bz);
+                        const bool shifted = (u.bx | u.by | u.bz) != 0;
+                        const bool far = abs(u.bx) > PACKED_SHIFT_LIMIT || abs(u.by) > PACKED_SHIFT_LIMIT ||
+                                         abs(u.bz) > PACKED_SHIFT_LIMIT;
+                        any_shift = any_shift || (__ballot(shifted) != 0);
+                        any_same = any_same || (__ballot(u.same_cell) != 0);
+                        too_far = too_far || (__ballot(far) != 0);
+                        if (shifted) {
+                            shift_vector(g, u.bx, u.by, u.bz, c.tx[r], c.ty[r], c.tz[r]);
+                        }
+                    }
+                    if (too_far) {
+                        general = true;
+                        break;
+                    }
+                    item.any_shift = item.any_shift || any_shift;
+
+                    uint32_t lo[R] = {0, 0};
+                    uint32_t hi[R] = {0, 0};
+                    uint32_t hits;
+                    if (item.tile_wrapped) {
+                        hits = sweep_columns_wrapped<R>(sorted, item.first_i, item.n_i, c, g, lo, hi);
+                    } else if (any_shift) {
+                        if (any_same) {
+                            hits = sweep_columns<R, true, true>(sorted, item.first_i, item.n_i, c, g.cutoff2, lo, hi);
+                        } else {
+                            hits = sweep_columns<R, true, false>(sorted, item.first_i, item.n_i, c, g.cutoff2, lo, hi);
+                        }
+                    } else {
+                        if (any_same) {
+                            hits = sweep_columns<R, false, true>(sorted, item.first_i, item.n_i, c, g.cutoff2, lo, hi);
+                        } else {
+                            hits = sweep_columns<R, false, false>(sorted, item.first_i, item.n_i, c, g.cutoff2, lo, hi);
+                        }
+                    }
+                    item.hits += hits;
+                    if (pair * R < FUSED_UNITS) {
+#pragma unroll
+                        for (int r = 0; r < R; r++) {
+                            columns_lo[pair * R + r] = lo[r];
+                            columns_hi[pair * R + r] = hi[r];
+                        }
+                    }
+                }
+            }
+            if (general) {
+                item.valid = false;
+                item.hits = 0;
+                if (lane == 0) {
+                    atomicAdd(&fargs.status->general, 1u);
+                }
+            }
+        }
+    }
+
+    // ---- phase 2: the workgroup's rows, then its place in the output
+    const uint32_t own_rows = FULL ? 2 * item.hits : item.hits;
+    if (lane == 0) {
+        shared.rows[wave] = own_rows;
+    }
+    __syncthreads();
+    uint64_t rows_before_wave = 0;
+    uint64_t block_rows = 0;
+#pragma unroll
+    for (int w = 0; w < SEARCH_WAVES; w++) {
+        const uint32_t rows = shared.rows[w];
+        rows_before_wave += static_cast<uint32_t>(w) < wave ? rows : 0;
+        block_rows += rows;
+    }
+    if (wave == 0) {
+        const uint64_t before = chain_position(fargs.chain, blockIdx.x, gridDim.x, block_rows, lane, fargs.status);
+        const bool fits = before + block_rows <= args.capacity;
+        if (lane == 0) {
+            shared.base = before;
+            shared.writable = fits ? 1u : 0u;
+            if (!fits) {
+                atomicAdd(&fargs.status->overflow, 1u);
+            }
+            if (blockIdx.x == gridDim.x - 1) {
+                fargs.status->total_rows = before + block_rows;
+            }
+        }
+    }
+    __syncthreads();
+    const bool leave_to_write_pass = item.valid && item.deferred && item.hits != 0 && shared.writable != 0;
+    if (work < args.n_work && lane == 0) {
+        args.counts[work] = leave_to_write_pass ? 1u : 0u;
+        if (leave_to_write_pass) {
+            fargs.first_rows[work] = shared.base + rows_before_wave;
+            atomicAdd(&fargs.status->deferred, 1u);
+            atomicAdd(&fargs.status->deferred_rows, static_cast<unsigned long long>(own_rows));
+        }
+    }
+    if (!item.valid || item.deferred || item.hits == 0 || shared.writable == 0) {
+        return;
+    }
+
+    // ---- phase 3: replay the columns, write the rows
+    ReplayContext ctx;
+    ctx.lane = lane;
+    ctx.tile_wrapped = item.tile_wrapped;
+    ctx.need_shift = item.any_shift || item.tile_wrapped;
+    shift_vector(g, 0, 0, 0, ctx.zero_tx, ctx.zero_ty, ctx.zero_tz);
+
+    ReplayState state;
+    state.out_cursor = shared.base + rows_before_wave;
+    state.head = 0;
+    state.tail = 0;
+    state.batch = aligning_batch<FULL>(state.out_cursor);
+    // number of tile points in each half of a column
+    const uint32_t n_lo = min(item.n_i, 32u);
+    const uint32_t n_hi = item.n_i - n_lo;
+    uint32_t filled[2] = {0, 0}; // value of head when the unit in each half of the candidate records was done
+
+    for (uint32_t unit = 0; unit < item.n_units; unit++) {
+        uint32_t lo = columns_lo[unit];
+        uint32_t hi = columns_hi[unit];
+        if (__ballot((lo | hi) != 0) == 0) {
+            continue;
+        }
+        const uint32_t half = unit & 1;
+        if (half == 0 ? state.tail < filled[0] : state.tail < filled[1]) {
+            // pending tickets still point into the records about to be replaced
+            redeem_fused<FULL>(state.head - state.tail, state, sh, args.out, g, ctx);
+        }
+        const uint32_t k = (item.unit_begin + unit) * WAVE + lane;
+        const UnitCandidates u = locate_unit(sh, item.n_batch, item.n_candidates, k, sorted);
+        if (u.valid) {
+            const int record = half * WAVE + lane;
+            sh.cand_x[record] = sorted.x[u.at];
+            sh.cand_y[record] = sorted.y[u.at];
+            sh.cand_z[record] = sorted.z[u.at];
+            sh.cand_index[record] = sorted.index[u.at];
+            sh.cand_shift[record] = pack_shift(u.bx, u.by, u.bz);
+        }
+        wave_sync();
+
+        while (true) {
+            const bool has = (lo | hi) != 0;
+            const uint64_t mask = __ballot(has);
+            if (mask == 0) {
+                break;
+            }
+            if (has) {
+                uint32_t point;
+                if (lo != 0) {
+                    const uint32_t bit = __builtin_ctz(lo);
+                    lo &= lo - 1;
+                    point = n_lo - 1 - bit;
+                } else {
+                    const uint32_t bit = __builtin_ctz(hi);
+                    hi &= hi - 1;
+                    point = 32 + n_hi - 1 - bit;
+                }
+                const uint32_t at = (state.head + rank_in_mask(mask)) & (RING - 1);
+                sh.ring[at] = static_cast<uint16_t>((half * WAVE + lane) | (point << 8));
+            }
+            state.head += __popcll(mask);
+            while (state.head - state.tail >= state.batch) {
+                redeem_fused<FULL>(state.batch, state, sh, args.out, g, ctx);
+            }
+        }
+        if (half == 0) {
+            filled[0] = state.head;
+        } else {
+            filled[1] = state.head;
+        }
+    }
+    if (state.head != state.tail) {
+        redeem_fused<FULL>(state.head - state.tail, state, sh, args.out, g, ctx);
+    }
+}
+
+} // namespace vesin_hip
+
+#endif

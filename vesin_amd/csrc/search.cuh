@@ -72,6 +72,7 @@ struct SearchArgs {
     uint32_t n_work;           // work items = tile slots * n_slices; tile slots are a multiple of
                                // N_XCD * SEARCH_WAVES and at least the number of tiles
     uint64_t capacity;         // WRITE: rows the output arrays hold; a launch that would overflow writes nothing
+    const uint32_t* only;      // WRITE: when not null, only work items with a non-zero entry are processed
 };
 
 __device__ __forceinline__ int32_t pack_shift(int32_t a, int32_t b, int32_t c) {
@@ -146,6 +147,99 @@ struct SearchSharedWrite: SearchTables {
     int32_t cand_bx[MAX_R * WAVE], cand_by[MAX_R * WAVE], cand_bz[MAX_R * WAVE];
     uint16_t ring[RING];
 };
+
+/// LDS written by some lanes is about to be read by others of the same wave: the hardware keeps one wave's LDS
+/// operations in order, this only stops the compiler from reordering them.
+__device__ __forceinline__ void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+}
+
+/// Stencil entries [first_linear, first_linear + n_batch) around cell (cx, cy, cz) go to the wave's LDS tables:
+/// neighbour cell start, packed cell shift, and the running number of candidates (scanned in place). Linear stencil
+/// offsets run dx major, dz minor.
+__device__ __forceinline__ void fill_stencil_tables(
+    SearchTables& sh, int lane, uint32_t first_linear, uint32_t n_batch, int32_t cx, int32_t cy, int32_t cz,
+    int32_t span_y, int32_t span_z, const GridParams& g, const uint64_t* __restrict__ cell_scan
+) {
+    const uint32_t centre = static_cast<uint32_t>(2 * g.s[0] + 1) * span_y * span_z / 2;
+    for (uint32_t e = lane; e < n_batch; e += WAVE) {
+        const uint32_t linear = first_linear + e;
+        int32_t dz = static_cast<int32_t>(linear % span_z) - g.s[2];
+        int32_t dy = static_cast<int32_t>((linear / span_z) % span_y) - g.s[1];
+        int32_t dx = static_cast<int32_t>(linear / (span_z * span_y)) - g.s[0];
+        int32_t cell[3] = {cx + dx, cy + dy, cz + dz};
+        int32_t q[3] = {0, 0, 0};
+        bool valid = true;
+#pragma unroll
+        for (int d = 0; d < 3; d++) {
+            const int32_t n = g.n[d];
+            if (g.periodic[d]) {
+                int32_t quotient = cell[d] / n;
+                int32_t rest = cell[d] - quotient * n;
+                if (rest < 0) {
+                    rest += n;
+                    quotient -= 1;
+                }
+                q[d] = quotient;
+                cell[d] = rest;
+            } else if (cell[d] < 0 || cell[d] >= n) {
+                valid = false;
+            }
+        }
+        uint32_t start = 0;
+        uint32_t count = 0;
+        int32_t packed = 0;
+        if (valid) {
+            uint32_t neighbour = (static_cast<uint32_t>(cell[2]) * g.n[1] + cell[1]) * g.n[0] + cell[0];
+            start = static_cast<uint32_t>(cell_scan[neighbour]);
+            count = static_cast<uint32_t>(cell_scan[neighbour + 1]) - start;
+            packed = pack_shift(q[0], q[1], q[2]);
+            if (linear == centre) {
+                packed |= 1 << 30;
+            }
+        }
+        sh.ent_start[e] = start;
+        sh.ent_shift[e] = packed;
+        sh.ent_prefix[e + 1] = count; // scanned in place below
+    }
+    wave_sync();
+
+    uint32_t carry = 0;
+    for (uint32_t base = 0; base < n_batch; base += WAVE) {
+        uint32_t e = base + lane;
+        uint32_t v = e < n_batch ? sh.ent_prefix[e + 1] : 0;
+        uint32_t inclusive = wave_inclusive_scan(v) + carry;
+        if (e < n_batch) {
+            sh.ent_prefix[e + 1] = inclusive;
+        }
+        carry = read_lane(inclusive, WAVE - 1);
+    }
+    if (lane == 0) {
+        sh.ent_prefix[0] = 0;
+    }
+    sh.n_candidates = carry;
+    wave_sync();
+}
+
+/// Candidate number k of the tables: its position in the cell-sorted arrays and the packed shift of its cell.
+__device__ __forceinline__ void locate_candidate(
+    const SearchTables& sh, uint32_t n_batch, uint32_t k, uint32_t& at, int32_t& packed
+) {
+    // largest e with ent_prefix[e] <= k
+    uint32_t lo = 0;
+    uint32_t hi = n_batch;
+    while (hi - lo > 1) {
+        uint32_t mid = (lo + hi) >> 1;
+        if (sh.ent_prefix[mid] <= k) {
+            lo = mid;
+        } else {
+            hi = mid;
+        }
+    }
+    at = sh.ent_start[lo] + (k - sh.ent_prefix[lo]);
+    packed = sh.ent_shift[lo];
+}
 
 /// Per-wave progress, kept in scalar registers.
 struct WaveState {
@@ -417,13 +511,6 @@ __device__ __forceinline__ void sweep_wrapped(
     }
 }
 
-/// LDS written by some lanes is about to be read by others of the same wave: the hardware keeps one wave's LDS
-/// operations in order, this only stops the compiler from reordering them.
-__device__ __forceinline__ void wave_sync() {
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
-    __builtin_amdgcn_wave_barrier();
-}
-
 /// One work item: one tile (or one slice of its candidates) searched by one wave.
 template <bool WRITE, bool FULL, int R, typename Shared>
 __device__ __forceinline__ void search_work_item(
@@ -497,66 +584,7 @@ __device__ __forceinline__ void search_work_item(
         const uint32_t n_batch = min(static_cast<uint32_t>(MAX_ENTRIES), n_entries - batch);
         wave_sync(); // done with the previous batch's tables
 
-        // ---- stencil entries of this batch: neighbour cell, its cell shift, how many points it holds
-        for (uint32_t e = lane; e < n_batch; e += WAVE) {
-            const uint32_t linear = centre + batch + e;
-            int32_t dz = static_cast<int32_t>(linear % span_z) - g.s[2];
-            int32_t dy = static_cast<int32_t>((linear / span_z) % span_y) - g.s[1];
-            int32_t dx = static_cast<int32_t>(linear / (span_z * span_y)) - g.s[0];
-            int32_t cell[3] = {cx + dx, cy + dy, cz + dz};
-            int32_t q[3] = {0, 0, 0};
-            bool valid = true;
-#pragma unroll
-            for (int d = 0; d < 3; d++) {
-                const int32_t n = g.n[d];
-                if (g.periodic[d]) {
-                    int32_t quotient = cell[d] / n;
-                    int32_t rest = cell[d] - quotient * n;
-                    if (rest < 0) {
-                        rest += n;
-                        quotient -= 1;
-                    }
-                    q[d] = quotient;
-                    cell[d] = rest;
-                } else if (cell[d] < 0 || cell[d] >= n) {
-                    valid = false;
-                }
-            }
-            uint32_t start = 0;
-            uint32_t count = 0;
-            int32_t packed = 0;
-            if (valid) {
-                uint32_t neighbour = (static_cast<uint32_t>(cell[2]) * g.n[1] + cell[1]) * g.n[0] + cell[0];
-                start = static_cast<uint32_t>(args.cell_scan[neighbour]);
-                count = static_cast<uint32_t>(args.cell_scan[neighbour + 1]) - start;
-                packed = pack_shift(q[0], q[1], q[2]);
-                if (linear == centre) {
-                    packed |= 1 << 30;
-                }
-            }
-            sh.ent_start[e] = start;
-            sh.ent_shift[e] = packed;
-            sh.ent_prefix[e + 1] = count; // scanned in place below
-        }
-        wave_sync();
-
-        {
-            uint32_t carry = 0;
-            for (uint32_t base = 0; base < n_batch; base += WAVE) {
-                uint32_t e = base + lane;
-                uint32_t v = e < n_batch ? sh.ent_prefix[e + 1] : 0;
-                uint32_t inclusive = wave_inclusive_scan(v) + carry;
-                if (e < n_batch) {
-                    sh.ent_prefix[e + 1] = inclusive;
-                }
-                carry = read_lane(inclusive, WAVE - 1);
-            }
-            if (lane == 0) {
-                sh.ent_prefix[0] = 0;
-            }
-            sh.n_candidates = carry;
-        }
-        wave_sync();
+        fill_stencil_tables(sh, lane, centre + batch, n_batch, cx, cy, cz, span_y, span_z, g, args.cell_scan);
 
         const uint32_t n_candidates = __builtin_amdgcn_readfirstlane(sh.n_candidates);
         const uint32_t n_groups = (n_candidates + WAVE * R - 1) / (WAVE * R);
@@ -579,19 +607,9 @@ __device__ __forceinline__ void search_work_item(
                 c.position[r] = 0xFFFFFFFFu;
                 bool same_cell = false;
                 if (valid) {
-                    // largest e with ent_prefix[e] <= k
-                    uint32_t lo = 0;
-                    uint32_t hi = n_batch;
-                    while (hi - lo > 1) {
-                        uint32_t mid = (lo + hi) >> 1;
-                        if (sh.ent_prefix[mid] <= k) {
-                            lo = mid;
-                        } else {
-                            hi = mid;
-                        }
-                    }
-                    const uint32_t at = sh.ent_start[lo] + (k - sh.ent_prefix[lo]);
-                    const int32_t packed = sh.ent_shift[lo];
+                    uint32_t at;
+                    int32_t packed;
+                    locate_candidate(sh, n_batch, k, at, packed);
                     int32_t qx, qy, qz;
                     unpack_shift(packed, qx, qy, qz);
                     same_cell = (packed >> 30) & 1;
@@ -680,6 +698,9 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void search_kernel(SearchArgs args, G
         return;
     }
     if (work < args.n_work) {
+        if (WRITE && args.only != nullptr && args.only[work] == 0) {
+            return;
+        }
         search_work_item<WRITE, FULL, R>(work, args, g, shared[wave], n_tiles, lane);
     }
 }
