@@ -97,6 +97,15 @@ __device__ __forceinline__ uint64_t wave_inclusive_scan(uint64_t v) {
     return v;
 }
 
+/// A value that is the same in every lane, moved to scalar registers (tells the compiler it is wave-uniform).
+__device__ __forceinline__ uint32_t uniform(uint32_t v) {
+    return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(v)));
+}
+
+__device__ __forceinline__ uint64_t uniform(uint64_t v) {
+    return (static_cast<uint64_t>(uniform(static_cast<uint32_t>(v >> 32))) << 32) | uniform(static_cast<uint32_t>(v));
+}
+
 __device__ __forceinline__ uint32_t read_lane(uint32_t v, int lane) {
     return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), lane));
 }

@@ -230,6 +230,8 @@ struct ReplayContext {
     bool need_shift;   // some candidate of the work item has a non-zero shift, or the tile holds wrapped points
     bool tile_wrapped;
     int lane;
+    uint32_t last_lo; // tile point of bit 0 of the low half of a column: min(n_i, 32) - 1
+    uint32_t last_hi; // same for the high half: n_i - 1
 };
 
 struct ReplayState {
@@ -265,8 +267,12 @@ __device__ __forceinline__ void redeem_fused(
     const int lane = ctx.lane;
     const bool active = static_cast<uint32_t>(lane) < n;
     const uint32_t ticket = sh.ring[(state.tail + lane) & (RING - 1)];
+    // ticket: candidate record (7 bits), bit of the column (5 bits, from bit 8), half of the column (bit 13); the
+    // first point of a half sits in the highest bit used
     const int slot = active ? ticket & (FUSED_SLOTS - 1) : 0;
-    const int il = active ? (ticket >> 8) & 63 : 0;
+    const uint32_t bit = (ticket >> 8) & 31;
+    const bool high = (ticket >> 13) & 1;
+    const int il = active ? static_cast<int>((high ? ctx.last_hi : ctx.last_lo) - bit) : 0;
 
     const double xj = sh.cand_x[slot];
     const double yj = sh.cand_y[slot];
@@ -302,38 +308,43 @@ __device__ __forceinline__ void redeem_fused(
     const double wz = (zi - zj) + mz;
     const double d2 = vx * vx + vy * vy + vz * vz;
 
+    // rows of this redeem start at the (wave-uniform) cursor: every address is a scalar base plus a 32-bit lane offset
+    const uint64_t cursor = state.out_cursor;
+    const uint32_t ulane = static_cast<uint32_t>(lane);
     if (FULL) {
         if (active) {
-            const uint64_t forward_row = state.out_cursor + lane;
-            const uint64_t mirror_row = forward_row + n;
+            char* pair_rows = reinterpret_cast<char*>(out.pairs) + cursor * 16;
             ulonglong2 forward, backward;
             forward.x = oi;
             forward.y = oj;
             backward.x = oj;
             backward.y = oi;
-            reinterpret_cast<ulonglong2*>(out.pairs)[forward_row] = forward;
-            reinterpret_cast<ulonglong2*>(out.pairs)[mirror_row] = backward;
+            *reinterpret_cast<ulonglong2*>(pair_rows + ulane * 16u) = forward;
+            *reinterpret_cast<ulonglong2*>(pair_rows + n * 16u + ulane * 16u) = backward;
             if (out.shifts != nullptr) {
-                int32_t* s = out.shifts + 3 * forward_row;
+                char* shift_rows = reinterpret_cast<char*>(out.shifts) + cursor * 12;
+                int32_t* s = reinterpret_cast<int32_t*>(shift_rows + ulane * 12u);
                 s[0] = sx;
                 s[1] = sy;
                 s[2] = sz;
-                int32_t* m = out.shifts + 3 * mirror_row;
+                int32_t* m = reinterpret_cast<int32_t*>(shift_rows + n * 12u + ulane * 12u);
                 m[0] = -sx;
                 m[1] = -sy;
                 m[2] = -sz;
             }
             if (out.distances != nullptr) {
+                char* distance_rows = reinterpret_cast<char*>(out.distances) + cursor * 8;
                 const double d = sqrt(d2);
-                out.distances[forward_row] = d;
-                out.distances[mirror_row] = d;
+                *reinterpret_cast<double*>(distance_rows + ulane * 8u) = d;
+                *reinterpret_cast<double*>(distance_rows + n * 8u + ulane * 8u) = d;
             }
             if (out.vectors != nullptr) {
-                double* v = out.vectors + 3 * forward_row;
+                char* vector_rows = reinterpret_cast<char*>(out.vectors) + cursor * 24;
+                double* v = reinterpret_cast<double*>(vector_rows + ulane * 24u);
                 v[0] = vx;
                 v[1] = vy;
                 v[2] = vz;
-                double* m = out.vectors + 3 * mirror_row;
+                double* m = reinterpret_cast<double*>(vector_rows + n * 24u + ulane * 24u);
                 m[0] = wx;
                 m[1] = wy;
                 m[2] = wz;
@@ -343,22 +354,21 @@ __device__ __forceinline__ void redeem_fused(
     } else {
         const bool flip = oi > oj || (oi == oj && !half_keeps_self_image(sx, sy, sz));
         if (active) {
-            const uint64_t row = state.out_cursor + lane;
             ulonglong2 pair;
             pair.x = flip ? oj : oi;
             pair.y = flip ? oi : oj;
-            reinterpret_cast<ulonglong2*>(out.pairs)[row] = pair;
+            *reinterpret_cast<ulonglong2*>(reinterpret_cast<char*>(out.pairs) + cursor * 16 + ulane * 16u) = pair;
             if (out.shifts != nullptr) {
-                int32_t* s = out.shifts + 3 * row;
+                int32_t* s = reinterpret_cast<int32_t*>(reinterpret_cast<char*>(out.shifts) + cursor * 12 + ulane * 12u);
                 s[0] = flip ? -sx : sx;
                 s[1] = flip ? -sy : sy;
                 s[2] = flip ? -sz : sz;
             }
             if (out.distances != nullptr) {
-                out.distances[row] = sqrt(d2);
+                *reinterpret_cast<double*>(reinterpret_cast<char*>(out.distances) + cursor * 8 + ulane * 8u) = sqrt(d2);
             }
             if (out.vectors != nullptr) {
-                double* v = out.vectors + 3 * row;
+                double* v = reinterpret_cast<double*>(reinterpret_cast<char*>(out.vectors) + cursor * 24 + ulane * 24u);
                 v[0] = flip ? wx : vx;
                 v[1] = flip ? wy : vy;
                 v[2] = flip ? wz : vz;
@@ -678,7 +688,7 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fa
     uint64_t block_rows = 0;
 #pragma unroll
     for (int w = 0; w < SEARCH_WAVES; w++) {
-        const uint32_t rows = shared.rows[w];
+        const uint32_t rows = uniform(shared.rows[w]);
         rows_before_wave += static_cast<uint32_t>(w) < wave ? rows : 0;
         block_rows += rows;
     }
@@ -697,16 +707,18 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fa
         }
     }
     __syncthreads();
-    const bool leave_to_write_pass = item.valid && item.deferred && item.hits != 0 && shared.writable != 0;
+    const uint64_t block_base = uniform(shared.base);
+    const bool writable = uniform(shared.writable) != 0;
+    const bool leave_to_write_pass = item.valid && item.deferred && item.hits != 0 && writable;
     if (work < args.n_work && lane == 0) {
         args.counts[work] = leave_to_write_pass ? 1u : 0u;
         if (leave_to_write_pass) {
-            fargs.first_rows[work] = shared.base + rows_before_wave;
+            fargs.first_rows[work] = block_base + rows_before_wave;
             atomicAdd(&fargs.status->deferred, 1u);
             atomicAdd(&fargs.status->deferred_rows, static_cast<unsigned long long>(own_rows));
         }
     }
-    if (!item.valid || item.deferred || item.hits == 0 || shared.writable == 0) {
+    if (!item.valid || item.deferred || item.hits == 0 || !writable) {
         return;
     }
 
@@ -718,13 +730,12 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fa
     shift_vector(g, 0, 0, 0, ctx.zero_tx, ctx.zero_ty, ctx.zero_tz);
 
     ReplayState state;
-    state.out_cursor = shared.base + rows_before_wave;
+    state.out_cursor = block_base + rows_before_wave;
     state.head = 0;
     state.tail = 0;
     state.batch = aligning_batch<FULL>(state.out_cursor);
-    // number of tile points in each half of a column
-    const uint32_t n_lo = min(item.n_i, 32u);
-    const uint32_t n_hi = item.n_i - n_lo;
+    ctx.last_lo = min(item.n_i, 32u) - 1;
+    ctx.last_hi = item.n_i - 1;
     uint32_t filled[2] = {0, 0}; // value of head when the unit in each half of the candidate records was done
 
     for (uint32_t unit = 0; unit < item.n_units; unit++) {
@@ -750,29 +761,28 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fa
         }
         wave_sync();
 
-        while (true) {
-            const bool has = (lo | hi) != 0;
-            const uint64_t mask = __ballot(has);
-            if (mask == 0) {
-                break;
-            }
-            if (has) {
-                uint32_t point;
-                if (lo != 0) {
-                    const uint32_t bit = __builtin_ctz(lo);
-                    lo &= lo - 1;
-                    point = n_lo - 1 - bit;
-                } else {
-                    const uint32_t bit = __builtin_ctz(hi);
-                    hi &= hi - 1;
-                    point = 32 + n_hi - 1 - bit;
+        // every round, each lane with hits left peels one bit off its column and drops a ticket; the low half of
+        // the columns first, then (tiles of more than 32 points) the high half
+        const uint32_t record = half * WAVE + lane;
+#pragma nounroll
+        for (int part = 0; part < 2; part++) {
+            uint32_t column = part == 0 ? lo : hi;
+            const uint32_t tag = record | (part << 13);
+            while (true) {
+                const uint64_t mask = __ballot(column != 0);
+                if (mask == 0) {
+                    break;
                 }
-                const uint32_t at = (state.head + rank_in_mask(mask)) & (RING - 1);
-                sh.ring[at] = static_cast<uint16_t>((half * WAVE + lane) | (point << 8));
-            }
-            state.head += __popcll(mask);
-            while (state.head - state.tail >= state.batch) {
-                redeem_fused<FULL>(state.batch, state, sh, args.out, g, ctx);
+                if (column != 0) {
+                    const uint32_t bit = __builtin_ctz(column);
+                    column &= column - 1;
+                    const uint32_t at = (state.head + rank_in_mask(mask)) & (RING - 1);
+                    sh.ring[at] = static_cast<uint16_t>(tag | (bit << 8));
+                }
+                state.head += __popcll(mask);
+                while (state.head - state.tail >= state.batch) {
+                    redeem_fused<FULL>(state.batch, state, sh, args.out, g, ctx);
+                }
             }
         }
         if (half == 0) {
