@@ -61,15 +61,34 @@ def test_second_call_is_single_pass_and_matches(timings, full):
         assert_same_list(again, expected, what=f"call {repeat + 2}")
 
 
-def test_single_pass_is_deterministic(timings):
+@pytest.mark.parametrize("full", [True, False], ids=["full", "half"])
+def test_ordered_rows_are_the_same_on_every_run(timings, monkeypatch, full):
+    # VESIN_HIP_ROWS=ordered: rows in work-item order, placed by the chain of workgroup totals
+    monkeypatch.setenv("VESIN_HIP_ROWS", "ordered")
     points, box, periodic, _ = configs.config1(12)
-    calculator = NeighborList(cutoff=5.0, full_list=True)
+    expected = oracle.neighbors(points, box, periodic, 5.0, full, False, "ijSdD")
+    calculator = NeighborList(cutoff=5.0, full_list=full)
     call(calculator, points, box, periodic)
     second = call(calculator, points, box, periodic)
     third = call(calculator, points, box, periodic)
     assert used_single_pass(calculator)
     for key in second:
         assert np.array_equal(second[key], third[key]), key
+    assert_same_list(second, expected)
+
+
+def test_ordered_rows_with_crowded_tiles_and_growth(timings, monkeypatch):
+    monkeypatch.setenv("VESIN_HIP_ROWS", "ordered")
+    rng = np.random.default_rng(22)
+    points = np.concatenate([rng.random((3000, 3)) * 30.0, rng.random((1200, 3)) * 2.5 + 10.0])
+    box = np.eye(3) * 30.0
+    expected = oracle.neighbors(points, box, True, 2.5, True, False, "ijSdD")
+    calculator = NeighborList(cutoff=2.5, full_list=True)
+    small = configs.config1(4)
+    call(calculator, *small[:3])
+    assert_same_list(call(calculator, points, box, True), expected, what="grown")
+    assert_same_list(call(calculator, points, box, True), expected, what="single pass")
+    assert used_single_pass(calculator)
 
 
 def test_environment_switch_keeps_the_two_passes(timings):

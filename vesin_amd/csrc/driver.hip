@@ -44,6 +44,13 @@ void enable_timings(bool enabled) {
     TIMINGS_ENABLED.store(enabled);
 }
 
+/// VESIN_HIP_ROWS=ordered makes the single-pass search place the rows in work-item order (identical from run to
+/// run) instead of order of arrival; costs about a tenth of the kernel's time.
+static bool ordered_rows() {
+    const char* text = std::getenv("VESIN_HIP_ROWS");
+    return text != nullptr && std::strcmp(text, "ordered") == 0;
+}
+
 /// VESIN_HIP_SEARCH=two-pass keeps every call on the count / scan / write sequence (for comparisons and tests).
 static bool two_pass_only() {
     const char* text = std::getenv("VESIN_HIP_SEARCH");
@@ -566,11 +573,10 @@ void neighbors(
         fargs.first_rows = offsets;
         fargs.status = fused_status;
         const uint32_t blocks = static_cast<uint32_t>(search_workgroups);
-        if (options.full) {
-            hipLaunchKernelGGL(fused_search_kernel<true>, dim3(blocks), dim3(SEARCH_BLOCK), 0, stream, fargs, g);
-        } else {
-            hipLaunchKernelGGL(fused_search_kernel<false>, dim3(blocks), dim3(SEARCH_BLOCK), 0, stream, fargs, g);
-        }
+        const bool ordered = ordered_rows();
+        auto kernel = options.full ? (ordered ? fused_search_kernel<true, true> : fused_search_kernel<true, false>)
+                                   : (ordered ? fused_search_kernel<false, true> : fused_search_kernel<false, false>);
+        hipLaunchKernelGGL(kernel, dim3(blocks), dim3(SEARCH_BLOCK), 0, stream, fargs, g);
         mark(T_WRITE);
         hipLaunchKernelGGL(publish_fused_status, dim3(1), dim3(1), 0, stream, extras.d_status, fused_status, extras.h_fused);
         HIP_CHECK(hipStreamSynchronize(stream));

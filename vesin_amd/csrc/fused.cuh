@@ -516,8 +516,11 @@ __device__ __forceinline__ uint64_t chain_position(
     return group_before + read_lane(wave_inclusive_scan(rows_of_member), WAVE - 1);
 }
 
-/// Four waves per workgroup, one work item each; they meet twice: to add up their rows, and to learn their place.
-template <bool FULL>
+/// Four waves per workgroup, one work item each. ORDERED: the rows come out in work-item order, the same on every
+/// run (the waves of a workgroup meet twice: to add up their rows, and to learn their place from the chain).
+/// Otherwise the waves never wait for one another and the rows come out in order of arrival, which varies from run
+/// to run like the order of the reference's GPU kernels (vesin/src/cuda/cell_list.cu:664, an atomic per pair there).
+template <bool FULL, bool ORDERED>
 __global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fargs, GridParams g) {
     constexpr int R = 2;
     __shared__ FusedShared shared;
@@ -678,42 +681,58 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fa
         }
     }
 
-    // ---- phase 2: the workgroup's rows, then its place in the output
+    // ---- phase 2: the place of the wave's rows in the output
     const uint32_t own_rows = FULL ? 2 * item.hits : item.hits;
-    if (lane == 0) {
-        shared.rows[wave] = own_rows;
-    }
-    __syncthreads();
-    uint64_t rows_before_wave = 0;
-    uint64_t block_rows = 0;
-#pragma unroll
-    for (int w = 0; w < SEARCH_WAVES; w++) {
-        const uint32_t rows = uniform(shared.rows[w]);
-        rows_before_wave += static_cast<uint32_t>(w) < wave ? rows : 0;
-        block_rows += rows;
-    }
-    if (wave == 0) {
-        const uint64_t before = chain_position(fargs.chain, blockIdx.x, gridDim.x, block_rows, lane, fargs.status);
-        const bool fits = before + block_rows <= args.capacity;
+    uint64_t first_row;
+    bool writable;
+    if (ORDERED) {
+        // rows in work-item order: the workgroup adds up its waves, then chains with the earlier workgroups
         if (lane == 0) {
-            shared.base = before;
-            shared.writable = fits ? 1u : 0u;
-            if (!fits) {
-                atomicAdd(&fargs.status->overflow, 1u);
-            }
-            if (blockIdx.x == gridDim.x - 1) {
-                fargs.status->total_rows = before + block_rows;
+            shared.rows[wave] = own_rows;
+        }
+        __syncthreads();
+        uint64_t rows_before_wave = 0;
+        uint64_t block_rows = 0;
+#pragma unroll
+        for (int w = 0; w < SEARCH_WAVES; w++) {
+            const uint32_t rows = uniform(shared.rows[w]);
+            rows_before_wave += static_cast<uint32_t>(w) < wave ? rows : 0;
+            block_rows += rows;
+        }
+        if (wave == 0) {
+            const uint64_t before = chain_position(fargs.chain, blockIdx.x, gridDim.x, block_rows, lane, fargs.status);
+            const bool fits = before + block_rows <= args.capacity;
+            if (lane == 0) {
+                shared.base = before;
+                shared.writable = fits ? 1u : 0u;
+                if (!fits) {
+                    atomicAdd(&fargs.status->overflow, 1u);
+                }
+                if (blockIdx.x == gridDim.x - 1) {
+                    fargs.status->total_rows = before + block_rows;
+                }
             }
         }
+        __syncthreads();
+        first_row = uniform(shared.base) + rows_before_wave;
+        writable = uniform(shared.writable) != 0;
+    } else {
+        // rows in order of arrival: one atomic per wave on the running total, no wave waits for another
+        unsigned long long before = 0;
+        if (lane == 0 && own_rows != 0) {
+            before = atomicAdd(&fargs.status->total_rows, static_cast<unsigned long long>(own_rows));
+        }
+        first_row = uniform(static_cast<uint64_t>(before));
+        writable = first_row + own_rows <= args.capacity;
+        if (!writable && lane == 0) {
+            atomicAdd(&fargs.status->overflow, 1u);
+        }
     }
-    __syncthreads();
-    const uint64_t block_base = uniform(shared.base);
-    const bool writable = uniform(shared.writable) != 0;
     const bool leave_to_write_pass = item.valid && item.deferred && item.hits != 0 && writable;
     if (work < args.n_work && lane == 0) {
         args.counts[work] = leave_to_write_pass ? 1u : 0u;
         if (leave_to_write_pass) {
-            fargs.first_rows[work] = block_base + rows_before_wave;
+            fargs.first_rows[work] = first_row;
             atomicAdd(&fargs.status->deferred, 1u);
             atomicAdd(&fargs.status->deferred_rows, static_cast<unsigned long long>(own_rows));
         }
@@ -730,7 +749,7 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fa
     shift_vector(g, 0, 0, 0, ctx.zero_tx, ctx.zero_ty, ctx.zero_tz);
 
     ReplayState state;
-    state.out_cursor = block_base + rows_before_wave;
+    state.out_cursor = first_row;
     state.head = 0;
     state.tail = 0;
     state.batch = aligning_batch<FULL>(state.out_cursor);
