@@ -116,6 +116,17 @@ __device__ __forceinline__ uint64_t read_lane(uint64_t v, int lane) {
     return (static_cast<uint64_t>(hi) << 32) | lo;
 }
 
+typedef unsigned long long PairRow __attribute__((ext_vector_type(2)));
+typedef int32_t ShiftRow __attribute__((ext_vector_type(3), aligned(4)));
+typedef double VectorHead __attribute__((ext_vector_type(2), aligned(8))); // first two of the three components
+
+/// Output rows are written once and never read by this kernel: non-temporal stores keep them from displacing the
+/// cell-sorted points in L2.
+template <typename T>
+__device__ __forceinline__ void stream_store(void* address, T value) {
+    __builtin_nontemporal_store(value, reinterpret_cast<T*>(address));
+}
+
 } // namespace vesin_hip
 
 #endif

@@ -314,64 +314,45 @@ __device__ __forceinline__ void redeem_fused(
     if (FULL) {
         if (active) {
             char* pair_rows = reinterpret_cast<char*>(out.pairs) + cursor * 16;
-            ulonglong2 forward, backward;
-            forward.x = oi;
-            forward.y = oj;
-            backward.x = oj;
-            backward.y = oi;
-            *reinterpret_cast<ulonglong2*>(pair_rows + ulane * 16u) = forward;
-            *reinterpret_cast<ulonglong2*>(pair_rows + n * 16u + ulane * 16u) = backward;
+            stream_store(pair_rows + ulane * 16u, PairRow{oi, oj});
+            stream_store(pair_rows + n * 16u + ulane * 16u, PairRow{oj, oi});
             if (out.shifts != nullptr) {
                 char* shift_rows = reinterpret_cast<char*>(out.shifts) + cursor * 12;
-                int32_t* s = reinterpret_cast<int32_t*>(shift_rows + ulane * 12u);
-                s[0] = sx;
-                s[1] = sy;
-                s[2] = sz;
-                int32_t* m = reinterpret_cast<int32_t*>(shift_rows + n * 12u + ulane * 12u);
-                m[0] = -sx;
-                m[1] = -sy;
-                m[2] = -sz;
+                stream_store(shift_rows + ulane * 12u, ShiftRow{sx, sy, sz});
+                stream_store(shift_rows + n * 12u + ulane * 12u, ShiftRow{-sx, -sy, -sz});
             }
             if (out.distances != nullptr) {
                 char* distance_rows = reinterpret_cast<char*>(out.distances) + cursor * 8;
                 const double d = sqrt(d2);
-                *reinterpret_cast<double*>(distance_rows + ulane * 8u) = d;
-                *reinterpret_cast<double*>(distance_rows + n * 8u + ulane * 8u) = d;
+                stream_store(distance_rows + ulane * 8u, d);
+                stream_store(distance_rows + n * 8u + ulane * 8u, d);
             }
             if (out.vectors != nullptr) {
                 char* vector_rows = reinterpret_cast<char*>(out.vectors) + cursor * 24;
-                double* v = reinterpret_cast<double*>(vector_rows + ulane * 24u);
-                v[0] = vx;
-                v[1] = vy;
-                v[2] = vz;
-                double* m = reinterpret_cast<double*>(vector_rows + n * 24u + ulane * 24u);
-                m[0] = wx;
-                m[1] = wy;
-                m[2] = wz;
+                stream_store(vector_rows + ulane * 24u, VectorHead{vx, vy});
+                stream_store(vector_rows + ulane * 24u + 16u, vz);
+                stream_store(vector_rows + n * 24u + ulane * 24u, VectorHead{wx, wy});
+                stream_store(vector_rows + n * 24u + ulane * 24u + 16u, wz);
             }
         }
         state.out_cursor += 2 * n;
     } else {
         const bool flip = oi > oj || (oi == oj && !half_keeps_self_image(sx, sy, sz));
         if (active) {
-            ulonglong2 pair;
-            pair.x = flip ? oj : oi;
-            pair.y = flip ? oi : oj;
-            *reinterpret_cast<ulonglong2*>(reinterpret_cast<char*>(out.pairs) + cursor * 16 + ulane * 16u) = pair;
+            stream_store(reinterpret_cast<char*>(out.pairs) + cursor * 16 + ulane * 16u, PairRow{flip ? oj : oi, flip ? oi : oj});
             if (out.shifts != nullptr) {
-                int32_t* s = reinterpret_cast<int32_t*>(reinterpret_cast<char*>(out.shifts) + cursor * 12 + ulane * 12u);
-                s[0] = flip ? -sx : sx;
-                s[1] = flip ? -sy : sy;
-                s[2] = flip ? -sz : sz;
+                stream_store(
+                    reinterpret_cast<char*>(out.shifts) + cursor * 12 + ulane * 12u,
+                    ShiftRow{flip ? -sx : sx, flip ? -sy : sy, flip ? -sz : sz}
+                );
             }
             if (out.distances != nullptr) {
-                *reinterpret_cast<double*>(reinterpret_cast<char*>(out.distances) + cursor * 8 + ulane * 8u) = sqrt(d2);
+                stream_store(reinterpret_cast<char*>(out.distances) + cursor * 8 + ulane * 8u, sqrt(d2));
             }
             if (out.vectors != nullptr) {
-                double* v = reinterpret_cast<double*>(reinterpret_cast<char*>(out.vectors) + cursor * 24 + ulane * 24u);
-                v[0] = flip ? wx : vx;
-                v[1] = flip ? wy : vy;
-                v[2] = flip ? wz : vz;
+                char* row = reinterpret_cast<char*>(out.vectors) + cursor * 24 + ulane * 24u;
+                stream_store(row, VectorHead{flip ? wx : vx, flip ? wy : vy});
+                stream_store(row + 16u, flip ? wz : vz);
             }
         }
         state.out_cursor += n;
