@@ -112,6 +112,7 @@ struct HipExtras {
     unsigned char* h_small = nullptr; // pinned: box (72 bytes) + periodic (3 bytes)
     BlockBounds* h_bounds = nullptr;  // pinned: one slot per workgroup of the bounding pass
     FusedStatus* h_fused = nullptr;   // pinned
+    ShiftRange* h_shift_ranges = nullptr; // pinned: one slot per workgroup of the sort's range pass
     size_t capacity = 0;              // rows every allocated output array can hold
     int single_pass_rest = 0;         // calls left before the single-pass search is tried again after it did not fit
     hipEvent_t events[T_STAGES] = {};
@@ -137,6 +138,9 @@ struct HipExtras {
         if (h_fused != nullptr) {
             (void)hipHostFree(h_fused);
         }
+        if (h_shift_ranges != nullptr) {
+            (void)hipHostFree(h_shift_ranges);
+        }
         if (have_events) {
             for (auto& event : events) {
                 (void)hipEventDestroy(event);
@@ -157,6 +161,9 @@ HipExtras& extras_of(VesinNeighborList& neighbors) {
             reinterpret_cast<void**>(&extras->h_bounds), BOUNDING_BLOCKS * sizeof(BlockBounds), hipHostMallocDefault
         ));
         HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&extras->h_fused), sizeof(FusedStatus), hipHostMallocDefault));
+        HIP_CHECK(hipHostMalloc(
+            reinterpret_cast<void**>(&extras->h_shift_ranges), SHIFT_RANGE_BLOCKS * sizeof(ShiftRange), hipHostMallocDefault
+        ));
     }
     return *static_cast<HipExtras*>(neighbors.opaque);
 }
@@ -664,6 +671,7 @@ void neighbors(
     const bool sorting = options.sorted && total > 1;
     SearchOutputs unsorted = final_out;
     SortWorkspace sort_space = {};
+    sort_space.host_ranges = extras.h_shift_ranges;
     if (sorting) {
         // the write pass goes to scratch rows (shifts always present: they are part of the sort key); the sort's
         // final gather fills the caller's arrays
@@ -680,7 +688,6 @@ void neighbors(
             sort_space.table = c.take<uint32_t>(table_entries);
             sort_space.table_scan = c.take<uint64_t>(table_entries + 1);
             sort_space.scan_scratch = c.take<uint64_t>(scan_scratch_elements(table_entries));
-            sort_space.range = c.take<ShiftRange>(1);
         };
         Carver measure_sort(nullptr);
         carve_sort(measure_sort);

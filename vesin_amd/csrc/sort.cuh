@@ -17,6 +17,7 @@
 #include "scan.cuh"
 #include "search.cuh"
 
+#include <algorithm>
 #include <stdexcept>
 #include <string>
 
@@ -43,16 +44,14 @@ struct KeyLayout {
     uint32_t use_j_and_shift;
 };
 
-__global__ void init_shift_range(ShiftRange* range) {
-    if (threadIdx.x == 0 && blockIdx.x == 0) {
-        for (int d = 0; d < 3; d++) {
-            range->lo[d] = 0x7fffffff;
-            range->hi[d] = -0x7fffffff - 1;
-        }
-    }
-}
+constexpr int SHIFT_RANGE_BLOCKS = 256;
 
-__global__ __launch_bounds__(BLOCK) void shift_range_kernel(const int32_t* __restrict__ shifts, size_t n, ShiftRange* range) {
+/// Range of the shifts of all rows: grid-stride loop, wave then workgroup reduction; every workgroup reports to its
+/// own slot of `host_ranges` (pinned host memory, folded by the host), so no atomics are involved.
+__global__ __launch_bounds__(BLOCK) void shift_range_kernel(
+    const int32_t* __restrict__ shifts, size_t n, ShiftRange* host_ranges
+) {
+    __shared__ ShiftRange partial[WAVES_PER_BLOCK];
     int lo[3] = {0x7fffffff, 0x7fffffff, 0x7fffffff};
     int hi[3] = {-0x7fffffff - 1, -0x7fffffff - 1, -0x7fffffff - 1};
     for (size_t k = static_cast<size_t>(blockIdx.x) * BLOCK + threadIdx.x; k < n; k += static_cast<size_t>(gridDim.x) * BLOCK) {
@@ -74,9 +73,21 @@ __global__ __launch_bounds__(BLOCK) void shift_range_kernel(const int32_t* __res
     if (lane_id() == 0) {
 #pragma unroll
         for (int d = 0; d < 3; d++) {
-            atomicMin(&range->lo[d], lo[d]);
-            atomicMax(&range->hi[d], hi[d]);
+            partial[threadIdx.x / WAVE].lo[d] = lo[d];
+            partial[threadIdx.x / WAVE].hi[d] = hi[d];
         }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        ShiftRange all = partial[0];
+        for (int w = 1; w < WAVES_PER_BLOCK; w++) {
+#pragma unroll
+            for (int d = 0; d < 3; d++) {
+                all.lo[d] = min(all.lo[d], partial[w].lo[d]);
+                all.hi[d] = max(all.hi[d], partial[w].hi[d]);
+            }
+        }
+        host_ranges[blockIdx.x] = all;
     }
 }
 
@@ -239,7 +250,7 @@ struct SortWorkspace {
     uint32_t* table;
     uint64_t* table_scan;
     uint64_t* scan_scratch;
-    ShiftRange* range;
+    ShiftRange* host_ranges; // pinned host memory, SHIFT_RANGE_BLOCKS entries
 };
 
 inline size_t sort_blocks(size_t n) {
@@ -273,13 +284,17 @@ inline void sort_pairs(
     }
     const uint32_t n_key_blocks = static_cast<uint32_t>((n + BLOCK - 1) / BLOCK);
 
-    hipLaunchKernelGGL(init_shift_range, dim3(1), dim3(1), 0, stream, w.range);
-    uint32_t range_blocks = n_key_blocks > 4096 ? 4096 : n_key_blocks;
-    hipLaunchKernelGGL(shift_range_kernel, dim3(range_blocks), dim3(BLOCK), 0, stream, from.shifts, n, w.range);
-    ShiftRange range;
-    if (hipMemcpyAsync(&range, w.range, sizeof(ShiftRange), hipMemcpyDeviceToHost, stream) != hipSuccess ||
-        hipStreamSynchronize(stream) != hipSuccess) {
+    const uint32_t range_blocks = n_key_blocks > SHIFT_RANGE_BLOCKS ? SHIFT_RANGE_BLOCKS : n_key_blocks;
+    hipLaunchKernelGGL(shift_range_kernel, dim3(range_blocks), dim3(BLOCK), 0, stream, from.shifts, n, w.host_ranges);
+    if (hipStreamSynchronize(stream) != hipSuccess) {
         throw std::runtime_error("HIP error while reading the range of the shifts");
+    }
+    ShiftRange range = w.host_ranges[0];
+    for (uint32_t block = 1; block < range_blocks; block++) {
+        for (int d = 0; d < 3; d++) {
+            range.lo[d] = std::min(range.lo[d], w.host_ranges[block].lo[d]);
+            range.hi[d] = std::max(range.hi[d], w.host_ranges[block].hi[d]);
+        }
     }
 
     KeyLayout layout = {};
