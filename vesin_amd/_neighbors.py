@@ -161,8 +161,17 @@ class NeighborList:
         if points.dim() != 2 or points.shape[1] != 3:
             raise ValueError("`points` must be a nx3 array")
 
-        periodic = torch.as_tensor(np.asarray(periodic).astype(np.bool_) if not isinstance(periodic, torch.Tensor) else periodic)
-        periodic = periodic.to(dtype=torch.bool, device=device).contiguous()
+        if isinstance(periodic, torch.Tensor):
+            periodic = periodic.to(dtype=torch.bool, device=device).contiguous()
+        else:
+            # the three flags rarely change between calls: keep their device copy
+            flags = np.asarray(periodic).astype(np.bool_)
+            key = (flags.tobytes(), flags.shape, str(device))
+            cached = getattr(self, "_periodic_on_device", None)
+            if cached is None or cached[0] != key:
+                cached = (key, torch.as_tensor(flags).to(device=device))
+                self._periodic_on_device = cached
+            periodic = cached[1]
         if tuple(periodic.shape) != (3,):
             raise ValueError(
                 f"`periodic` must be a single boolean or a sequence of three booleans, got {periodic}"

@@ -266,6 +266,47 @@ __global__ __launch_bounds__(BLOCK) void scatter_points(
     provisional[start + slot_of[i]] = i;
 }
 
+/// Counting-sort scatter straight into the structure-of-arrays layout, for callers that do not need the order of
+/// the points inside a cell to be the same on every run: the slot handed out by the histogram atomic is final.
+/// Also appends the cell's tiles. `tiles[].wrapped` must be zero on entry.
+__global__ __launch_bounds__(BLOCK) void place_points(
+    const double* __restrict__ points, const int32_t* __restrict__ wrap_of, const uint32_t* __restrict__ cell_of,
+    const uint32_t* __restrict__ slot_of, const uint64_t* __restrict__ cell_scan, uint32_t n_points,
+    SortedPoints sorted, Tile* __restrict__ tiles
+) {
+    const uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
+    if (i >= n_points) {
+        return;
+    }
+    const uint32_t cell = cell_of[i];
+    const uint64_t here = cell_scan[cell];
+    const uint32_t start = static_cast<uint32_t>(here);
+    const uint32_t count = static_cast<uint32_t>(cell_scan[cell + 1]) - start;
+    const uint32_t first_tile = static_cast<uint32_t>(here >> 32);
+    const uint32_t k = slot_of[i];
+    const uint32_t to = start + k;
+
+    const int32_t wx = wrap_of[3 * static_cast<size_t>(i) + 0];
+    const int32_t wy = wrap_of[3 * static_cast<size_t>(i) + 1];
+    const int32_t wz = wrap_of[3 * static_cast<size_t>(i) + 2];
+    sorted.index[to] = i;
+    sorted.x[to] = points[3 * static_cast<size_t>(i) + 0];
+    sorted.y[to] = points[3 * static_cast<size_t>(i) + 1];
+    sorted.z[to] = points[3 * static_cast<size_t>(i) + 2];
+    sorted.wx[to] = wx;
+    sorted.wy[to] = wy;
+    sorted.wz[to] = wz;
+    if ((wx | wy | wz) != 0) {
+        atomicOr(&tiles[first_tile + k / 64u].wrapped, 1u);
+    }
+    if (k % 64u == 0) {
+        Tile* tile = &tiles[first_tile + k / 64u];
+        tile->cell = cell;
+        tile->first = to;
+        tile->count = min(64u, count - k);
+    }
+}
+
 constexpr uint32_t CANONICAL_LIMIT = 4096;
 
 /// One thread per slot of the counting sort. The atomics of assign_cells leave the points of a cell in arbitrary

@@ -519,14 +519,22 @@ void neighbors(
             flat_points, g, cell_of, slot_of, wrap_of, cell_counts, extras.d_status
         );
         exclusive_scan<SCAN_CELL_COUNTS>(cell_counts, n_cells, cell_scan, scan_scratch, stream);
-        hipLaunchKernelGGL(
-            scatter_points, dim3(point_blocks), dim3(BLOCK), 0, stream,
-            g.n_points, cell_of, slot_of, cell_scan, provisional
-        );
-        hipLaunchKernelGGL(
-            gather_points, dim3(point_blocks), dim3(BLOCK), 0, stream,
-            flat_points, wrap_of, cell_of, provisional, cell_scan, g.n_points, sorted, tiles
-        );
+        if (ordered_rows()) {
+            // the same order of the points inside every cell on every run
+            hipLaunchKernelGGL(
+                scatter_points, dim3(point_blocks), dim3(BLOCK), 0, stream,
+                g.n_points, cell_of, slot_of, cell_scan, provisional
+            );
+            hipLaunchKernelGGL(
+                gather_points, dim3(point_blocks), dim3(BLOCK), 0, stream,
+                flat_points, wrap_of, cell_of, provisional, cell_scan, g.n_points, sorted, tiles
+            );
+        } else {
+            hipLaunchKernelGGL(
+                place_points, dim3(point_blocks), dim3(BLOCK), 0, stream,
+                flat_points, wrap_of, cell_of, slot_of, cell_scan, g.n_points, sorted, tiles
+            );
+        }
     }
     mark(T_CELLS);
 
