@@ -1,13 +1,13 @@
 """Headline benchmark: neighbor pairs per second of the HIP path on one MI355X.
 
-One "step" is one ``vesin_neighbors`` call (the whole job: cell list, count pass, scan, write pass, final device
-sync) on the 1,000,000-atom jittered diamond configuration, cutoff 5 A, full list, unsorted, returning i, j, S, d,
+One "step" is one ``vesin_neighbors`` call (the whole job: cell list, single-pass search into the arrays the list
+kept from its first call, final device sync) on the 1,000,000-atom jittered diamond configuration, cutoff 5 A, full list, unsorted, returning i, j, S, d,
 with the inputs already resident in HBM. Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
 
 The line carries, next to the throughput:
-* ``roofline``: the dominant kernel (the write pass of the search) against the 8 TB/s HBM peak, from its
+* ``roofline``: the dominant kernel (the single-pass search, fused_search_kernel) against the 8 TB/s HBM peak, from its
   algorithmic bytes (24 B per point read + 36 B per pair written) and its launch duration measured with HIP events
   on the stream it runs on (``vesin_hip_last_timings``);
 * ``cpu_baseline``: the reference's CPU path (the compiled reference in oracle/_ref when present, otherwise the C
@@ -26,9 +26,10 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes moved by ONE launch of the write-pass kernel on this workload, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE runs scaled by a copy kernel of known size (profiles/search_write_config1_pmc.txt); None = not measured.
-WRITE_KERNEL_TRAFFIC_BYTES = None
+# HBM bytes moved by ONE launch of the single-pass search kernel on this workload, from rocprofv3 --pmc FETCH_SIZE
+# and WRITE_SIZE runs scaled by a device copy of known size (profiles/fused_search_config1_pmc.txt):
+# 94.7 MB fetched + 3216.3 MB written. Only meaningful for the default 1M-atom workload.
+SEARCH_KERNEL_TRAFFIC_BYTES = 3_311_000_000
 
 
 def main():
@@ -113,12 +114,12 @@ def main():
     achieved = algorithmic_bytes / (write_ms * 1e-3) / 1e9
     roofline = {
         "bound": "hbm",
-        "kernel": "search_kernel<WRITE> (write pass)",
+        "kernel": "fused_search_kernel (single-pass search)" if stages["count"] == 0 else "search_kernel<WRITE> (write pass)",
         "achieved": round(achieved, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4),
-        "traffic": WRITE_KERNEL_TRAFFIC_BYTES,
+        "traffic": SEARCH_KERNEL_TRAFFIC_BYTES if (args.replicas == 50 and stages["count"] == 0) else None,
         "algorithmic_bytes": algorithmic_bytes,
         "kernel_ms": round(write_ms, 4),
         "whole_call_frac": round(algorithmic_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
