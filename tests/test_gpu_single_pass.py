@@ -180,3 +180,34 @@ def test_wrapped_tiles_in_the_single_pass(timings):
     again = call(calculator, points, box, periodic)
     assert used_single_pass(calculator)
     assert_same_list(again, expected)
+
+
+def test_a_box_that_changes_between_calls():
+    # later calls of a list start with the box of the call before and check it when they synchronise: a changed box
+    # must be noticed and the call redone, whatever the sequence
+    rng = np.random.default_rng(12)
+    points, box, periodic, _ = configs.config1(6)
+    boxes = [box, box, box, box * 1.03, box * 1.03, box, box * 0.99, box * 0.99, box * 0.99]
+    calculator = NeighborList(cutoff=5.0, full_list=True)
+    for step, current in enumerate(boxes):
+        moved = points * (current[0, 0] / box[0, 0]) + rng.normal(scale=0.01, size=points.shape)
+        expected = oracle.neighbors(moved, current, periodic, 5.0, True, False, "ijSdD")
+        assert_same_list(call(calculator, moved, current, periodic), expected, what=f"step {step}")
+    # the flags are part of what is remembered
+    open_box = oracle.neighbors(points, box, [True, False, True], 5.0, True, False, "ijSdD")
+    assert_same_list(call(calculator, points, box, [True, False, True]), open_box, what="periodicity changed")
+    assert_same_list(call(calculator, points, box, [True, False, True]), open_box, what="periodicity kept")
+
+
+def test_a_box_that_becomes_singular():
+    points, box, periodic, _ = configs.config1(4)
+    calculator = NeighborList(cutoff=5.0, full_list=True)
+    for _ in range(3):
+        call(calculator, points, box, periodic)
+    flat = box.copy()
+    flat[2] = flat[1]
+    with pytest.raises(RuntimeError, match="the box matrix is not invertible"):
+        call(calculator, points, flat, periodic)
+    # and the list is still usable
+    expected = oracle.neighbors(points, box, periodic, 5.0, True, False, "ijSdD")
+    assert_same_list(call(calculator, points, box, periodic), expected)

@@ -165,9 +165,17 @@ __device__ __forceinline__ void fill_stencil_tables(
     const uint32_t centre = static_cast<uint32_t>(2 * g.s[0] + 1) * span_y * span_z / 2;
     for (uint32_t e = lane; e < n_batch; e += WAVE) {
         const uint32_t linear = first_linear + e;
-        int32_t dz = static_cast<int32_t>(linear % span_z) - g.s[2];
-        int32_t dy = static_cast<int32_t>((linear / span_z) % span_y) - g.s[1];
-        int32_t dx = static_cast<int32_t>(linear / (span_z * span_y)) - g.s[0];
+        int32_t dx, dy, dz;
+        if (span_y == 3 && span_z == 3) {
+            // the usual stencil of radius one: divisions by constants
+            dz = static_cast<int32_t>(linear % 3u) - 1;
+            dy = static_cast<int32_t>((linear / 3u) % 3u) - 1;
+            dx = static_cast<int32_t>(linear / 9u) - g.s[0];
+        } else {
+            dz = static_cast<int32_t>(linear % span_z) - g.s[2];
+            dy = static_cast<int32_t>((linear / span_z) % span_y) - g.s[1];
+            dx = static_cast<int32_t>(linear / (span_z * span_y)) - g.s[0];
+        }
         int32_t cell[3] = {cx + dx, cy + dy, cz + dz};
         int32_t q[3] = {0, 0, 0};
         bool valid = true;
@@ -175,14 +183,25 @@ __device__ __forceinline__ void fill_stencil_tables(
         for (int d = 0; d < 3; d++) {
             const int32_t n = g.n[d];
             if (g.periodic[d]) {
-                int32_t quotient = cell[d] / n;
-                int32_t rest = cell[d] - quotient * n;
-                if (rest < 0) {
-                    rest += n;
-                    quotient -= 1;
+                if (g.s[d] <= n) {
+                    // the neighbour is at most one box away: no division needed
+                    if (cell[d] < 0) {
+                        cell[d] += n;
+                        q[d] = -1;
+                    } else if (cell[d] >= n) {
+                        cell[d] -= n;
+                        q[d] = 1;
+                    }
+                } else {
+                    int32_t quotient = cell[d] / n;
+                    int32_t rest = cell[d] - quotient * n;
+                    if (rest < 0) {
+                        rest += n;
+                        quotient -= 1;
+                    }
+                    q[d] = quotient;
+                    cell[d] = rest;
                 }
-                q[d] = quotient;
-                cell[d] = rest;
             } else if (cell[d] < 0 || cell[d] >= n) {
                 valid = false;
             }
