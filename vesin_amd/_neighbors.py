@@ -224,11 +224,21 @@ class NeighborList:
         n_pairs = self._neighbors.length
         device_str = f"cuda:{index}"
 
+        views = self.__dict__.setdefault("_views", {})
+
         def wrap(pointer, shape, typestr, dtype):
             if n_pairs == 0:
                 return torch.empty(shape, dtype=dtype, device=device_str)
-            view = torch.as_tensor(_DeviceView(pointer, shape, typestr, self), device=device_str)
-            return view.clone() if copy else view
+            if copy:
+                return torch.as_tensor(_DeviceView(pointer, shape, typestr, self), device=device_str).clone()
+            # the arrays are kept between calls: the same pointer and shape give the same view (views refer to
+            # the calculator, so only callers who asked for views make it refer to itself)
+            key = (pointer, shape, typestr, device_str)
+            cached = views.get(typestr + str(len(shape)))
+            if cached is None or cached[0] != key:
+                cached = (key, torch.as_tensor(_DeviceView(pointer, shape, typestr, self), device=device_str))
+                views[typestr + str(len(shape))] = cached
+            return cached[1]
 
         pairs = shifts = distances = vectors = None
         if any(q in quantities for q in "ijP"):
