@@ -123,6 +123,35 @@ struct VesinHipTimings {
     uint64_t candidates;/* reserved, 0 */
 };
 
+/* Neighbor lists of many systems that share the options, computed by one sequence of launches (thousands of small
+ * systems cost about as much as one large one with as many points, instead of thousands of calls). Per system the
+ * rows are exactly those of vesin_neighbors on that system alone; only their order may differ.
+ *
+ *   points       device: the points of all systems, one system after the other
+ *   first_point  host, n_systems + 1 entries: first_point[s] is the index in `points` of the first point of system
+ *                s, first_point[n_systems] the total number of points
+ *   boxes        device: n_systems boxes (3x3 each, rows = box vectors)
+ *   periodic     device: n_systems x 3 flags; every system must be periodic in all three directions
+ *   neighbors    receives all rows, system after system; the indices in `pairs` count from the first point of the
+ *                row's system. Same ownership rules as for vesin_neighbors; the same struct may be used with both.
+ *   first_pair   host, n_systems + 1 entries, filled on success: rows [first_pair[s], first_pair[s + 1]) belong to
+ *                system s
+ *
+ * options.sorted must be false. Returns EXIT_SUCCESS / EXIT_FAILURE like vesin_neighbors, with the same message
+ * ownership. */
+int VESIN_API vesin_hip_neighbors_batch(
+    const double (*points)[3],
+    const size_t* first_point,
+    size_t n_systems,
+    const double (*boxes)[3][3],
+    const bool (*periodic)[3],
+    struct VesinDevice device,
+    struct VesinOptions options,
+    struct VesinNeighborList* neighbors,
+    size_t* first_pair,
+    const char** error_message
+);
+
 void VESIN_API vesin_hip_enable_timings(int enabled);
 int VESIN_API vesin_hip_last_timings(const struct VesinNeighborList* neighbors, struct VesinHipTimings* timings);
 

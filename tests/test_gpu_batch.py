@@ -1,0 +1,108 @@
+"""``vesin_hip_neighbors_batch``: many systems in one call give, per system, the rows of a call on that system alone
+(``-m gpu``)."""
+
+import numpy as np
+import pytest
+
+import oracle
+from _helpers import assert_same_list
+from golden import systems
+from vesin_amd import NeighborList, configs
+
+pytestmark = pytest.mark.gpu
+
+NAMES = {"P": "pairs", "S": "shifts", "d": "distances", "D": "vectors"}
+
+
+def run_batch(calculator, all_points, all_boxes, letters="PSdD", periodic=True):
+    import torch
+
+    first_point = np.cumsum([0] + [len(p) for p in all_points])
+    points = torch.as_tensor(np.concatenate(all_points).astype(np.float64), device="cuda:0")
+    boxes = torch.as_tensor(np.stack(all_boxes).astype(np.float64), device="cuda:0")
+    outputs, first_pair = calculator.compute_batch(points, first_point, boxes, periodic, letters)
+    whole = {NAMES[q]: out.cpu().numpy() for q, out in zip(letters, outputs)}
+    per_system = []
+    for s in range(len(all_points)):
+        rows = slice(int(first_pair[s]), int(first_pair[s + 1]))
+        per_system.append({key: value[rows] for key, value in whole.items()})
+    assert first_pair[0] == 0 and first_pair[-1] == len(whole["pairs"])
+    return per_system
+
+
+@pytest.mark.parametrize("full", [True, False], ids=["full", "half"])
+def test_replicas_of_the_small_cell_case(full):
+    # 64 atoms, cutoff above the box: one cell, 5^3 images (the multi-image path), 48 systems at once
+    replicas = [configs.config3(r) for r in range(48)]
+    cutoff = replicas[0][3]["cutoff"]
+    calculator = NeighborList(cutoff=cutoff, full_list=full)
+    lists = run_batch(calculator, [r[0] for r in replicas], [r[1] for r in replicas])
+    for r, (points, box, periodic, _) in enumerate(replicas):
+        expected = oracle.neighbors(points, box, periodic, cutoff, full, False, "ijSdD")
+        assert_same_list(lists[r], expected, what=f"replica {r}")
+
+
+def test_systems_of_different_sizes_and_shapes():
+    rng = np.random.default_rng(31)
+    all_points, all_boxes = [], []
+    # a triclinic box with a few hundred points (a real cell list), tiny systems, an empty one, a larger cube
+    points, box, _ = systems.read_xyz("carbon")
+    all_points.append(points)
+    all_boxes.append(box)
+    for n in (1, 2, 0, 33, 700):
+        edge = 6.0 + 2.0 * rng.random()
+        box = np.eye(3) * edge + 0.3 * rng.normal(size=(3, 3))
+        all_boxes.append(box)
+        all_points.append(rng.random((n, 3)) @ box + rng.integers(-2, 3, size=(n, 3)) @ box)
+    big = configs.config1(5)
+    all_points.append(big[0])
+    all_boxes.append(big[1])
+    for full in (True, False):
+        calculator = NeighborList(cutoff=4.0, full_list=full)
+        lists = run_batch(calculator, all_points, all_boxes)
+        for s, (points, box) in enumerate(zip(all_points, all_boxes)):
+            expected = oracle.neighbors(points, box, True, 4.0, full, False, "ijSdD")
+            assert_same_list(lists[s], expected, what=f"system {s} full={full}")
+
+
+def test_batch_of_one_equals_the_single_call():
+    points, box, periodic, _ = configs.config1(8)
+    calculator = NeighborList(cutoff=5.0, full_list=True)
+    (alone,) = run_batch(calculator, [points], [box])
+    expected = oracle.neighbors(points, box, periodic, 5.0, True, False, "ijSdD")
+    assert_same_list(alone, expected)
+    # the same struct then serves a single call
+    import torch
+
+    out = calculator.compute(torch.as_tensor(points, device="cuda:0"), torch.as_tensor(box, device="cuda:0"), True, "PSdD")
+    single = {NAMES[q]: t.cpu().numpy() for q, t in zip("PSdD", out)}
+    assert_same_list(single, expected)
+
+
+def test_batch_errors():
+    import torch
+
+    points, box, periodic, _ = configs.config3(0)
+    device_points = torch.as_tensor(points, device="cuda:0")
+    boxes = torch.as_tensor(box[None], device="cuda:0")
+    with pytest.raises(RuntimeError, match="sorted output is not available for a batch"):
+        NeighborList(cutoff=5.0, full_list=True, sorted=True).compute_batch(device_points, [0, len(points)], boxes)
+    with pytest.raises(RuntimeError, match="not periodic in all directions"):
+        flags = torch.as_tensor([[True, False, True]], device="cuda:0")
+        NeighborList(cutoff=5.0, full_list=True).compute_batch(device_points, [0, len(points)], boxes, flags)
+    with pytest.raises(RuntimeError, match="must not decrease"):
+        NeighborList(cutoff=5.0, full_list=True).compute_batch(device_points, [0, 70, len(points)], torch.cat([boxes, boxes]))
+    singular = boxes.clone()
+    singular[0, 2] = singular[0, 1]
+    with pytest.raises(RuntimeError, match="the box matrix is not invertible"):
+        NeighborList(cutoff=5.0, full_list=True).compute_batch(device_points, [0, len(points)], singular)
+
+
+def test_outputs_on_request_only():
+    replicas = [configs.config3(r) for r in range(4)]
+    calculator = NeighborList(cutoff=10.0, full_list=True)
+    lists = run_batch(calculator, [r[0] for r in replicas], [r[1] for r in replicas], letters="Pd")
+    for r, (points, box, periodic, _) in enumerate(replicas):
+        expected = oracle.neighbors(points, box, periodic, 10.0, True, False, "ijSd")
+        assert len(lists[r]["pairs"]) == len(expected["pairs"])
+        assert np.array_equal(np.sort(lists[r]["distances"]), np.sort(expected["distances"]))

@@ -68,6 +68,13 @@ def get_library():
                 f"{LIB_PATH} is missing: build it first with `python -m vesin_amd._build` "
                 "(hipcc, --offload-arch=gfx950)"
             )
+        # PyTorch-ROCm ships its own HIP runtime. A process must use one runtime only (device pointers and streams
+        # of one are unknown to another): torch goes first, so that the library's HIP symbols resolve to the
+        # runtime that owns the caller's tensors.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         lib = ctypes.CDLL(LIB_PATH)
         lib.vesin_neighbors.restype = ctypes.c_int
         lib.vesin_neighbors.argtypes = [
@@ -82,6 +89,19 @@ def get_library():
         ]
         lib.vesin_free.restype = None
         lib.vesin_free.argtypes = [ctypes.POINTER(VesinNeighborList)]
+        lib.vesin_hip_neighbors_batch.restype = ctypes.c_int
+        lib.vesin_hip_neighbors_batch.argtypes = [
+            ctypes.c_void_p,
+            ctypes.POINTER(ctypes.c_size_t),
+            ctypes.c_size_t,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            VesinDevice,
+            VesinOptions,
+            ctypes.POINTER(VesinNeighborList),
+            ctypes.POINTER(ctypes.c_size_t),
+            ctypes.POINTER(ctypes.c_char_p),
+        ]
         lib.vesin_hip_enable_timings.restype = None
         lib.vesin_hip_enable_timings.argtypes = [ctypes.c_int]
         lib.vesin_hip_last_timings.restype = ctypes.c_int

@@ -266,6 +266,90 @@ class NeighborList:
                 data.append(to_result(vectors))
         return tuple(data)
 
+    def compute_batch(self, points, first_point, boxes, periodic=True, quantities: str = "ij", copy: bool = True):
+        """Neighbor lists of many fully periodic systems in one go (``vesin_hip_neighbors_batch``).
+
+        ``points``: (N, 3) GPU tensor with the systems one after the other; ``first_point``: n_systems + 1 integers,
+        where each system starts; ``boxes``: (n_systems, 3, 3) GPU tensor; ``periodic``: ``True`` or an
+        (n_systems, 3) boolean tensor. Returns ``(outputs, first_pair)``: the requested quantities for all systems
+        (indices count inside each system) and the n_systems + 1 row offsets of the systems as a numpy array.
+        """
+        import torch
+
+        if not isinstance(points, torch.Tensor) or points.device.type != "cuda":
+            raise RuntimeError("compute_batch takes torch tensors on a cuda (HIP) device")
+        device = points.device
+        first_point = np.ascontiguousarray(first_point, dtype=np.uint64)
+        n_systems = len(first_point) - 1
+        points = points.to(dtype=torch.float64).contiguous()
+        boxes = torch.as_tensor(boxes).to(device=device, dtype=torch.float64).contiguous()
+        if tuple(boxes.shape) != (n_systems, 3, 3):
+            raise ValueError("`boxes` must hold one 3x3 matrix per system")
+        if isinstance(periodic, (bool, np.bool_)):
+            periodic = torch.full((n_systems, 3), bool(periodic), dtype=torch.bool, device=device)
+        else:
+            periodic = torch.as_tensor(periodic).to(device=device, dtype=torch.bool).contiguous()
+        if tuple(periodic.shape) != (n_systems, 3):
+            raise ValueError("`periodic` must hold three flags per system")
+
+        options = VesinOptions()
+        options.cutoff = self.cutoff
+        options.full = self.full_list
+        options.sorted = self.sorted
+        options.algorithm = self._c_algorithm
+        options.n_threads = self.n_threads
+        options.return_shifts = "S" in quantities
+        options.return_distances = "d" in quantities
+        options.return_vectors = "D" in quantities
+        options.skin = self.skin
+
+        index = device.index if device.index is not None else torch.cuda.current_device()
+        torch.cuda.current_stream(device).synchronize()
+        first_pair = np.zeros(n_systems + 1, dtype=np.uint64)
+        error_message = ctypes.c_char_p()
+        status = self._lib.vesin_hip_neighbors_batch(
+            points.data_ptr() if points.shape[0] > 0 else boxes.data_ptr(),
+            first_point.ctypes.data_as(ctypes.POINTER(ctypes.c_size_t)),
+            n_systems,
+            boxes.data_ptr(),
+            periodic.data_ptr(),
+            VesinDevice(VesinCUDA, index),
+            options,
+            ctypes.byref(self._neighbors),
+            first_pair.ctypes.data_as(ctypes.POINTER(ctypes.c_size_t)),
+            ctypes.byref(error_message),
+        )
+        if status != 0:
+            raise RuntimeError(error_message.value.decode("utf8"))
+
+        n_pairs = self._neighbors.length
+        device_str = f"cuda:{index}"
+
+        def wrap(pointer, shape, typestr, dtype):
+            if n_pairs == 0:
+                return torch.empty(shape, dtype=dtype, device=device_str)
+            view = torch.as_tensor(_DeviceView(pointer, shape, typestr, self), device=device_str)
+            return view.clone() if copy else view
+
+        data = []
+        pairs = None
+        for quantity in quantities:
+            if quantity in "ijP" and pairs is None:
+                pairs = wrap(self._neighbors.pairs, (n_pairs, 2), "<u8", torch.uint64)
+            if quantity == "P":
+                data.append(pairs)
+            elif quantity == "i":
+                data.append(pairs[:, 0])
+            elif quantity == "j":
+                data.append(pairs[:, 1])
+            elif quantity == "S":
+                data.append(wrap(self._neighbors.shifts, (n_pairs, 3), "<i4", torch.int32))
+            elif quantity == "d":
+                data.append(wrap(self._neighbors.distances, (n_pairs,), "<f8", torch.float64))
+            elif quantity == "D":
+                data.append(wrap(self._neighbors.vectors, (n_pairs, 3), "<f8", torch.float64))
+        return tuple(data), first_pair
+
     def timings(self):
         """Per-stage GPU times (ms) of the last ``compute``; needs ``enable_timings(True)`` beforehand."""
         timings = VesinHipTimings()

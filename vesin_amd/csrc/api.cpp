@@ -98,6 +98,80 @@ extern "C" int vesin_neighbors(
     return EXIT_SUCCESS;
 }
 
+extern "C" int vesin_hip_neighbors_batch(
+    const double (*points)[3],
+    const size_t* first_point,
+    size_t n_systems,
+    const double (*boxes)[3][3],
+    const bool (*periodic)[3],
+    VesinDevice device,
+    VesinOptions options,
+    VesinNeighborList* neighbors,
+    size_t* first_pair,
+    const char** error_message
+) {
+    if (error_message == nullptr) {
+        return EXIT_FAILURE;
+    }
+    if (first_point == nullptr) {
+        return fail(error_message, "`first_point` can not be a NULL pointer");
+    }
+    if (first_pair == nullptr) {
+        return fail(error_message, "`first_pair` can not be a NULL pointer");
+    }
+    if (boxes == nullptr) {
+        return fail(error_message, "`cell` can not be a NULL pointer");
+    }
+    if (periodic == nullptr) {
+        return fail(error_message, "`periodic` can not be a NULL pointer");
+    }
+    if (neighbors == nullptr) {
+        return fail(error_message, "`neighbors` can not be a NULL pointer");
+    }
+    if (n_systems > 0 && points == nullptr && first_point[n_systems] > 0) {
+        return fail(error_message, "`points` can not be a NULL pointer");
+    }
+    if (!std::isfinite(options.cutoff) || options.cutoff <= 0) {
+        return fail(error_message, "cutoff must be a finite, positive number");
+    }
+    if (options.cutoff <= 1e-6) {
+        return fail(error_message, "cutoff is too small");
+    }
+    if (!std::isfinite(options.skin) || options.skin < 0.0) {
+        return fail(error_message, "skin must be a finite, non-negative number");
+    }
+    if (options.n_threads < 0) {
+        return fail(error_message, "n_threads must be zero or a positive integer");
+    }
+    if (device.type != VesinCUDA) {
+        return fail(error_message, "a batch of systems is only computed on a GPU device (VesinCUDA, i.e. HIP on ROCm)");
+    }
+    if (neighbors->device.type != VesinUnknownDevice && neighbors->device.type != device.type) {
+        return fail(error_message, "`neighbors` device and data `device` do not match, free the neighbors first");
+    }
+
+    try {
+        if (options.skin > 0.0) {
+            throw std::runtime_error("a non-zero `skin` (Verlet caching) is not supported by the HIP path");
+        }
+        if (neighbors->device.type == VesinUnknownDevice) {
+            neighbors->device = device;
+        }
+        vesin_hip::neighbors_batch(points, first_point, n_systems, boxes, periodic, options, *neighbors, first_pair);
+    } catch (const std::bad_alloc&) {
+        LAST_ERROR = "failed to allocate memory";
+        *error_message = LAST_ERROR.c_str();
+        return EXIT_FAILURE;
+    } catch (const std::exception& e) {
+        LAST_ERROR = e.what();
+        *error_message = LAST_ERROR.c_str();
+        return EXIT_FAILURE;
+    } catch (...) {
+        return fail(error_message, "fatal error: unknown type thrown as exception");
+    }
+    return EXIT_SUCCESS;
+}
+
 extern "C" void vesin_free(VesinNeighborList* neighbors) {
     if (neighbors == nullptr) {
         return;

@@ -272,7 +272,8 @@ __global__ __launch_bounds__(BLOCK) void scatter_points(
 __global__ __launch_bounds__(BLOCK) void place_points(
     const double* __restrict__ points, const int32_t* __restrict__ wrap_of, const uint32_t* __restrict__ cell_of,
     const uint32_t* __restrict__ slot_of, const uint64_t* __restrict__ cell_scan, uint32_t n_points,
-    SortedPoints sorted, Tile* __restrict__ tiles
+    SortedPoints sorted, Tile* __restrict__ tiles,
+    const uint32_t* __restrict__ system_of, const uint32_t* __restrict__ first_point
 ) {
     const uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
     if (i >= n_points) {
@@ -289,7 +290,10 @@ __global__ __launch_bounds__(BLOCK) void place_points(
     const int32_t wx = wrap_of[3 * static_cast<size_t>(i) + 0];
     const int32_t wy = wrap_of[3 * static_cast<size_t>(i) + 1];
     const int32_t wz = wrap_of[3 * static_cast<size_t>(i) + 2];
-    sorted.index[to] = i;
+    // in a batch (system_of not null) the index counts from the first point of the point's system, and the tile
+    // carries the system above its flag bit
+    const uint32_t system = system_of != nullptr ? system_of[i] : 0;
+    sorted.index[to] = system_of != nullptr ? i - first_point[system] : i;
     sorted.x[to] = points[3 * static_cast<size_t>(i) + 0];
     sorted.y[to] = points[3 * static_cast<size_t>(i) + 1];
     sorted.z[to] = points[3 * static_cast<size_t>(i) + 2];
@@ -304,7 +308,57 @@ __global__ __launch_bounds__(BLOCK) void place_points(
         tile->cell = cell;
         tile->first = to;
         tile->count = min(64u, count - k);
+        if (system != 0) {
+            atomicOr(&tile->wrapped, system << 1);
+        }
     }
+}
+
+/// assign_cells for many systems at once: every point looks up its system (binary search in `first_point`), uses
+/// that system's grid, and counts itself in the system's range of cells.
+__global__ __launch_bounds__(BLOCK) void assign_cells_batch(
+    const double* __restrict__ points, uint32_t n_points, const GridParams* __restrict__ grids,
+    const uint32_t* __restrict__ first_point, const uint32_t* __restrict__ cell_base, uint32_t n_systems,
+    uint32_t* __restrict__ cell_of, uint32_t* __restrict__ slot_of, int32_t* __restrict__ wrap_of,
+    uint32_t* __restrict__ system_of, uint32_t* __restrict__ cell_counts, DeviceStatus* status
+) {
+    const uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
+    if (i >= n_points) {
+        return;
+    }
+    // largest s with first_point[s] <= i
+    uint32_t lo = 0;
+    uint32_t hi = n_systems;
+    while (hi - lo > 1) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (first_point[mid] <= i) {
+            lo = mid;
+        } else {
+            hi = mid;
+        }
+    }
+    const uint32_t system = lo;
+    const GridParams& g = grids[system];
+
+    const double x = points[3 * static_cast<size_t>(i) + 0];
+    const double y = points[3 * static_cast<size_t>(i) + 1];
+    const double z = points[3 * static_cast<size_t>(i) + 2];
+    int32_t cell[3] = {0, 0, 0};
+    int32_t wrap[3] = {0, 0, 0};
+    unsigned int axis;
+    if (all_finite(x, y, z, axis)) {
+        locate(g, x, y, z, cell, wrap);
+    } else {
+        atomicMin(&status->first_bad_coordinate, 3u * i + axis);
+    }
+    const uint32_t linear =
+        cell_base[system] + (static_cast<uint32_t>(cell[2]) * g.n[1] + cell[1]) * g.n[0] + cell[0];
+    cell_of[i] = linear;
+    slot_of[i] = atomicAdd(&cell_counts[linear], 1u);
+    system_of[i] = system;
+    wrap_of[3 * static_cast<size_t>(i) + 0] = wrap[0];
+    wrap_of[3 * static_cast<size_t>(i) + 1] = wrap[1];
+    wrap_of[3 * static_cast<size_t>(i) + 2] = wrap[2];
 }
 
 constexpr uint32_t CANONICAL_LIMIT = 4096;

@@ -603,7 +603,8 @@ bool compute(
         } else {
             hipLaunchKernelGGL(
                 place_points, dim3(point_blocks), dim3(BLOCK), 0, stream,
-                flat_points, wrap_of, cell_of, slot_of, cell_scan, g.n_points, sorted, tiles
+                flat_points, wrap_of, cell_of, slot_of, cell_scan, g.n_points, sorted, tiles,
+                static_cast<const uint32_t*>(nullptr), static_cast<const uint32_t*>(nullptr)
             );
         }
     }
@@ -816,6 +817,296 @@ bool compute(
 }
 
 } // namespace
+
+
+namespace {
+
+/// first_pair[s] = first output row of system s (offsets are kept per tile-major work item), first_pair[n] = total.
+__global__ void system_rows_kernel(
+    const uint64_t* __restrict__ cell_scan, const uint32_t* __restrict__ cell_base, const uint64_t* __restrict__ offsets,
+    uint32_t n_systems, uint32_t n_slices, uint32_t n_slots, unsigned long long* __restrict__ first_pair
+) {
+    const uint32_t s = blockIdx.x * BLOCK + threadIdx.x;
+    if (s > n_systems) {
+        return;
+    }
+    if (s == n_systems) {
+        first_pair[s] = offsets[n_slots];
+        return;
+    }
+    const uint32_t first_tile = static_cast<uint32_t>(cell_scan[cell_base[s]] >> 32);
+    first_pair[s] = offsets[static_cast<size_t>(first_tile) * n_slices];
+}
+
+template <bool WRITE>
+void launch_search_batch(bool full, const SearchArgs& args, hipStream_t stream) {
+    if (args.n_work == 0) {
+        return;
+    }
+    constexpr int R = 2;
+    const uint32_t blocks = (args.n_work + SEARCH_WAVES - 1) / SEARCH_WAVES;
+    if (full) {
+        hipLaunchKernelGGL((search_kernel_batch<WRITE, true, R>), dim3(blocks), dim3(SEARCH_BLOCK), 0, stream, args);
+    } else {
+        hipLaunchKernelGGL((search_kernel_batch<WRITE, false, R>), dim3(blocks), dim3(SEARCH_BLOCK), 0, stream, args);
+    }
+}
+
+} // namespace
+
+void neighbors_batch(
+    const double (*points)[3],
+    const size_t* first_point,
+    size_t n_systems,
+    const double (*boxes)[3][3],
+    const bool (*periodic)[3],
+    VesinOptions options,
+    VesinNeighborList& neighbors,
+    size_t* first_pair
+) {
+    const int device_id = neighbors.device.device_id;
+    int device_count = 0;
+    if (hipGetDeviceCount(&device_count) != hipSuccess || device_count == 0) {
+        (void)hipGetLastError();
+        throw std::runtime_error("no HIP device is available to this process");
+    }
+    if (device_id < 0 || device_id >= device_count) {
+        throw std::runtime_error("invalid GPU device_id " + std::to_string(device_id));
+    }
+    if (n_systems == 0) {
+        throw std::runtime_error("a batch needs at least one system");
+    }
+    for (size_t s = 0; s < n_systems; s++) {
+        if (first_point[s + 1] < first_point[s]) {
+            throw std::runtime_error("`first_point` must not decrease");
+        }
+    }
+    if (first_point[0] != 0) {
+        throw std::runtime_error("`first_point` must start at 0");
+    }
+    const size_t n_points = first_point[n_systems];
+    if (n_points >= 0xFFFFFFF0ull || n_systems >= 0x7FFFFFF0ull) {
+        throw std::runtime_error("too many points or systems: the GPU path indexes them with 32 bits");
+    }
+    if (options.sorted) {
+        throw std::runtime_error("sorted output is not available for a batch of systems");
+    }
+    if (device_of(points) != device_id && n_points > 0) {
+        throw std::runtime_error("`points` pointer is not allocated on the GPU of the neighbor list");
+    }
+    if (device_of(boxes) != device_id) {
+        throw std::runtime_error("`boxes` pointer is not allocated on the GPU of the neighbor list");
+    }
+    if (device_of(periodic) != device_id) {
+        throw std::runtime_error("`periodic` pointer is not allocated on the GPU of the neighbor list");
+    }
+
+    HIP_CHECK(hipSetDevice(device_id));
+    HipExtras& extras = extras_of(neighbors);
+    extras.timings_valid = false;
+    extras.have_last_box = false; // the work buffers of the single-system path are about to be reused
+    hipStream_t stream = nullptr;
+    const size_t pair_limit = pairs_per_point_limit();
+
+    // ---- every system's box comes to the host: the grids are picked there
+    std::vector<double> host_boxes(9 * n_systems);
+    std::vector<unsigned char> host_periodic(3 * n_systems);
+    HIP_CHECK(hipMemcpy(host_boxes.data(), boxes, host_boxes.size() * sizeof(double), hipMemcpyDeviceToHost));
+    HIP_CHECK(hipMemcpy(host_periodic.data(), periodic, host_periodic.size(), hipMemcpyDeviceToHost));
+
+    std::vector<GridParams> grids(n_systems);
+    std::vector<uint32_t> cell_base_host(n_systems + 1);
+    std::vector<uint32_t> first_point_host(n_systems + 1);
+    uint64_t total_cells = 0;
+    const double zeros[3] = {0.0, 0.0, 0.0};
+    for (size_t s = 0; s < n_systems; s++) {
+        bool flags[3];
+        for (int d = 0; d < 3; d++) {
+            flags[d] = host_periodic[3 * s + d] != 0;
+        }
+        if (!(flags[0] && flags[1] && flags[2])) {
+            throw std::runtime_error(
+                "system " + std::to_string(s) + " is not periodic in all directions: a batch only takes fully periodic systems"
+            );
+        }
+        const HostBox hbox = normalise_box(&host_boxes[9 * s], flags);
+        const size_t n_here = first_point[s + 1] - first_point[s];
+        bool single_cell = options.algorithm == VesinBruteForce;
+        HostGrid grid = choose_grid(hbox, options.cutoff, n_here, zeros, zeros, single_cell);
+        if (options.algorithm == VesinAutoAlgorithm && !single_cell && (grid.n_cells == 1 || n_here < 32)) {
+            grid = choose_grid(hbox, options.cutoff, n_here, zeros, zeros, true);
+        }
+        GridParams& g = grids[s];
+        std::memset(&g, 0, sizeof(g));
+        for (int d = 0; d < 3; d++) {
+            for (int e = 0; e < 3; e++) {
+                g.H[3 * d + e] = hbox.H[d][e];
+                g.Hinv[3 * d + e] = hbox.Hinv[d][e];
+            }
+            g.periodic[d] = 1;
+            g.n[d] = grid.n[d];
+            g.s[d] = grid.s[d];
+            g.np_min[d] = grid.np_min[d];
+            g.np_scale[d] = grid.np_scale[d];
+        }
+        g.cutoff2 = options.cutoff * options.cutoff;
+        g.n_points = static_cast<uint32_t>(n_here);
+        g.n_cells = static_cast<uint32_t>(grid.n_cells);
+        cell_base_host[s] = static_cast<uint32_t>(total_cells);
+        first_point_host[s] = static_cast<uint32_t>(first_point[s]);
+        total_cells += grid.n_cells;
+        if (total_cells >= 0xFFFFFFF0ull) {
+            throw std::runtime_error("too many cells in this batch");
+        }
+    }
+    cell_base_host[n_systems] = static_cast<uint32_t>(total_cells);
+    first_point_host[n_systems] = static_cast<uint32_t>(n_points);
+
+    if (n_points == 0) {
+        size_outputs(neighbors, extras, 0, options);
+        neighbors.length = 0;
+        for (size_t s = 0; s <= n_systems; s++) {
+            first_pair[s] = 0;
+        }
+        return;
+    }
+
+    // ---- work buffers
+    size_t tiles_bound = std::min<size_t>(total_cells, n_points) + n_points / 64 + 1;
+    constexpr size_t slot_multiple = N_XCD * SEARCH_WAVES;
+    tiles_bound = (tiles_bound + slot_multiple - 1) / slot_multiple * slot_multiple;
+    uint32_t n_slices = 1;
+    if (tiles_bound < 8192) {
+        n_slices = static_cast<uint32_t>(std::min<size_t>(256, (8192 + tiles_bound - 1) / tiles_bound));
+    }
+    const size_t n_slots = tiles_bound * n_slices;
+
+    uint32_t* cell_counts = nullptr;
+    Tile* tiles = nullptr;
+    uint64_t* cell_scan = nullptr;
+    uint32_t* cell_of = nullptr;
+    uint32_t* slot_of = nullptr;
+    uint32_t* system_of = nullptr;
+    int32_t* wrap_of = nullptr;
+    SortedPoints sorted = {};
+    uint32_t* counts = nullptr;
+    uint64_t* offsets = nullptr;
+    uint64_t* scan_scratch = nullptr;
+    GridParams* d_grids = nullptr;
+    uint32_t* d_first_point = nullptr;
+    uint32_t* d_cell_base = nullptr;
+    unsigned long long* d_first_pair = nullptr;
+    const size_t scratch_elements = std::max(scan_scratch_elements(total_cells), scan_scratch_elements(n_slots));
+    auto carve = [&](Carver& carver) {
+        cell_counts = carver.take<uint32_t>(total_cells);
+        tiles = carver.take<Tile>(tiles_bound);
+        cell_scan = carver.take<uint64_t>(total_cells + 1);
+        cell_of = carver.take<uint32_t>(n_points);
+        slot_of = carver.take<uint32_t>(n_points);
+        system_of = carver.take<uint32_t>(n_points);
+        wrap_of = carver.take<int32_t>(3 * n_points);
+        sorted.x = carver.take<double>(n_points + SORTED_PADDING);
+        sorted.y = carver.take<double>(n_points + SORTED_PADDING);
+        sorted.z = carver.take<double>(n_points + SORTED_PADDING);
+        sorted.index = carver.take<uint32_t>(n_points + SORTED_PADDING);
+        sorted.wx = carver.take<int32_t>(n_points);
+        sorted.wy = carver.take<int32_t>(n_points);
+        sorted.wz = carver.take<int32_t>(n_points);
+        counts = carver.take<uint32_t>(n_slots);
+        offsets = carver.take<uint64_t>(n_slots + 1);
+        scan_scratch = carver.take<uint64_t>(scratch_elements);
+        d_grids = carver.take<GridParams>(n_systems);
+        d_first_point = carver.take<uint32_t>(n_systems + 1);
+        d_cell_base = carver.take<uint32_t>(n_systems + 1);
+        d_first_pair = carver.take<unsigned long long>(n_systems + 1);
+    };
+    Carver measure(nullptr);
+    carve(measure);
+    extras.work.reserve(measure.used);
+    Carver carver(extras.work.ptr);
+    carve(carver);
+
+    HIP_CHECK(hipMemcpyAsync(d_grids, grids.data(), n_systems * sizeof(GridParams), hipMemcpyHostToDevice, stream));
+    HIP_CHECK(hipMemcpyAsync(
+        d_first_point, first_point_host.data(), (n_systems + 1) * sizeof(uint32_t), hipMemcpyHostToDevice, stream
+    ));
+    HIP_CHECK(hipMemcpyAsync(
+        d_cell_base, cell_base_host.data(), (n_systems + 1) * sizeof(uint32_t), hipMemcpyHostToDevice, stream
+    ));
+
+    // ---- cell lists of all systems, in one sequence of launches
+    const uint32_t point_blocks = static_cast<uint32_t>((n_points + BLOCK - 1) / BLOCK);
+    const auto* flat_points = reinterpret_cast<const double*>(points);
+    hipLaunchKernelGGL(
+        fetch_box, dim3(1), dim3(64), 0, stream,
+        reinterpret_cast<const double*>(boxes), reinterpret_cast<const bool*>(periodic), extras.h_small, extras.d_status
+    );
+    {
+        const size_t to_clear = reinterpret_cast<char*>(tiles + tiles_bound) - reinterpret_cast<char*>(cell_counts);
+        HIP_CHECK(hipMemsetAsync(cell_counts, 0, to_clear, stream));
+        HIP_CHECK(hipMemsetAsync(counts, 0, n_slots * sizeof(uint32_t), stream));
+    }
+    hipLaunchKernelGGL(
+        assign_cells_batch, dim3(point_blocks), dim3(BLOCK), 0, stream,
+        flat_points, static_cast<uint32_t>(n_points), d_grids, d_first_point, d_cell_base,
+        static_cast<uint32_t>(n_systems), cell_of, slot_of, wrap_of, system_of, cell_counts, extras.d_status
+    );
+    exclusive_scan<SCAN_CELL_COUNTS>(cell_counts, total_cells, cell_scan, scan_scratch, stream);
+    hipLaunchKernelGGL(
+        place_points, dim3(point_blocks), dim3(BLOCK), 0, stream,
+        flat_points, wrap_of, cell_of, slot_of, cell_scan, static_cast<uint32_t>(n_points), sorted, tiles,
+        system_of, d_first_point
+    );
+
+    // ---- count, scan, write
+    SearchArgs args = {};
+    args.sorted = sorted;
+    args.cell_scan = cell_scan;
+    args.tiles = tiles;
+    args.counts = counts;
+    args.offsets = offsets;
+    args.n_slices = n_slices;
+    args.n_work = static_cast<uint32_t>(n_slots);
+    args.grids = d_grids;
+    args.cell_base = d_cell_base;
+    args.total_cells = static_cast<uint32_t>(total_cells);
+    launch_search_batch<false>(options.full, args, stream);
+    exclusive_scan<SCAN_U32>(counts, n_slots, offsets, scan_scratch, stream);
+    hipLaunchKernelGGL(publish_status, dim3(1), dim3(1), 0, stream, extras.d_status, offsets + n_slots, extras.h_status);
+    HIP_CHECK(hipStreamSynchronize(stream));
+    if (extras.h_status->first_bad_coordinate != 0xFFFFFFFFu) {
+        non_finite_error(points, extras.h_status->first_bad_coordinate);
+    }
+    const size_t total = extras.h_status->total_pairs;
+    if (pair_limit != 0 && total > n_points * pair_limit) {
+        throw std::runtime_error(
+            "The number of neighbor pairs exceeds the maximum capacity of " + std::to_string(n_points * pair_limit) +
+            " (max_pairs_per_point=" + std::to_string(pair_limit) + "; n_points=" + std::to_string(n_points) + "). " +
+            "Consider reducing the cutoff distance, or explicitly setting " +
+            "VESIN_CUDA_MAX_PAIRS_PER_POINT as an environment variable."
+        );
+    }
+
+    size_outputs(neighbors, extras, total, options);
+    args.out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
+    args.out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
+    args.out.distances = neighbors.distances;
+    args.out.vectors = reinterpret_cast<double*>(neighbors.vectors);
+    args.capacity = extras.capacity;
+    if (total > 0) {
+        launch_search_batch<true>(options.full, args, stream);
+    }
+    const uint32_t system_blocks = static_cast<uint32_t>((n_systems + 1 + BLOCK - 1) / BLOCK);
+    hipLaunchKernelGGL(
+        system_rows_kernel, dim3(system_blocks), dim3(BLOCK), 0, stream,
+        cell_scan, d_cell_base, offsets, static_cast<uint32_t>(n_systems), n_slices, static_cast<uint32_t>(n_slots), d_first_pair
+    );
+    static_assert(sizeof(size_t) == sizeof(unsigned long long), "size_t is 64 bits wide here");
+    HIP_CHECK(hipMemcpyAsync(first_pair, d_first_pair, (n_systems + 1) * sizeof(size_t), hipMemcpyDeviceToHost, stream));
+    HIP_CHECK(hipStreamSynchronize(stream));
+    HIP_CHECK(hipGetLastError());
+    neighbors.length = total;
+}
 
 void free_neighbors(VesinNeighborList& neighbors) {
     HIP_CHECK(hipSetDevice(neighbors.device.device_id));

@@ -17,6 +17,21 @@ void neighbors(
     VesinNeighborList& neighbors
 );
 
+/// The lists of many (fully periodic) systems in one sequence of launches. `points`, `boxes`, `periodic` are device
+/// memory holding the systems one after the other; `first_point` (host, n_systems + 1 entries) says where each
+/// system starts. Rows come out system after system with indices counted inside each system; `first_pair` (host,
+/// n_systems + 1 entries) receives where each system's rows start.
+void neighbors_batch(
+    const double (*points)[3],
+    const size_t* first_point,
+    size_t n_systems,
+    const double (*boxes)[3][3],
+    const bool (*periodic)[3],
+    VesinOptions options,
+    VesinNeighborList& neighbors,
+    size_t* first_pair
+);
+
 /// Free the outputs and the private state of a GPU list (does not zero the struct).
 void free_neighbors(VesinNeighborList& neighbors);
 

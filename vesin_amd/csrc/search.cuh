@@ -73,7 +73,16 @@ struct SearchArgs {
                                // N_XCD * SEARCH_WAVES and at least the number of tiles
     uint64_t capacity;         // WRITE: rows the output arrays hold; a launch that would overflow writes nothing
     const uint32_t* only;      // WRITE: when not null, only work items with a non-zero entry are processed
+    // many systems in one launch (batched entry point); null / zero otherwise
+    const GridParams* grids;   // one per system
+    const uint32_t* cell_base; // first cell of every system in the concatenated grids, n_systems + 1 entries
+    uint32_t total_cells;
 };
+
+/// In a batch the tile remembers its system next to the flag: bit 0 = holds wrapped points, bits 1.. = system.
+__device__ __forceinline__ uint32_t tile_system(const Tile& tile) {
+    return tile.wrapped >> 1;
+}
 
 __device__ __forceinline__ int32_t pack_shift(int32_t a, int32_t b, int32_t c) {
     // three signed 10-bit fields
@@ -531,9 +540,9 @@ __device__ __forceinline__ void sweep_wrapped(
 }
 
 /// One work item: one tile (or one slice of its candidates) searched by one wave.
-template <bool WRITE, bool FULL, int R, typename Shared>
+template <bool WRITE, bool FULL, int R, bool BATCH, typename Shared>
 __device__ __forceinline__ void search_work_item(
-    uint32_t work, const SearchArgs& args, const GridParams& g, Shared& sh, uint32_t n_tiles, int lane
+    uint32_t work, const SearchArgs& args, const GridParams& single_grid, Shared& sh, uint32_t n_tiles, int lane
 ) {
     const uint32_t slice = work % args.n_slices;
 
@@ -546,18 +555,33 @@ __device__ __forceinline__ void search_work_item(
     const uint32_t tile_id = xcd * per_xcd + within;
 
     if (within >= per_xcd || tile_id >= n_tiles) {
-        if (!WRITE && lane == 0) {
+        if (!WRITE && !BATCH && lane == 0) {
             args.counts[work] = 0;
         }
         return;
     }
+    // In a batch the rows of a work item are counted and placed under its tile's number, not under the number of
+    // the wave that happens to run it: the rows of one system stay together (the host clears `counts` first).
+    const uint32_t row_slot = BATCH ? tile_id * args.n_slices + slice : work;
 
     const Tile tile = args.tiles[tile_id];
     const uint32_t n_i = tile.count;
     const uint32_t first_i = tile.first;
-    const int32_t cx = tile.cell % g.n[0];
-    const int32_t cy = (tile.cell / g.n[0]) % g.n[1];
-    const int32_t cz = tile.cell / (g.n[0] * g.n[1]);
+
+    // the grid: the kernel's argument, or this tile's system's
+    GridParams batch_grid;
+    uint32_t first_cell = 0;
+    if (BATCH) {
+        const uint32_t system = tile_system(tile);
+        batch_grid = args.grids[system];
+        first_cell = args.cell_base[system];
+    }
+    const GridParams& g = BATCH ? batch_grid : single_grid;
+    const uint64_t* __restrict__ cell_scan = args.cell_scan + first_cell;
+    const uint32_t local_cell = tile.cell - first_cell;
+    const int32_t cx = local_cell % g.n[0];
+    const int32_t cy = (local_cell / g.n[0]) % g.n[1];
+    const int32_t cz = local_cell / (g.n[0] * g.n[1]);
 
     const double* __restrict__ px = args.sorted.x;
     const double* __restrict__ py = args.sorted.y;
@@ -581,7 +605,7 @@ __device__ __forceinline__ void search_work_item(
     }
 
     SweepContext ctx;
-    ctx.tile_wrapped = tile.wrapped != 0;
+    ctx.tile_wrapped = (tile.wrapped & 1u) != 0;
     ctx.lane = lane;
     shift_vector(g, 0, 0, 0, ctx.zero_tx, ctx.zero_ty, ctx.zero_tz);
 
@@ -595,7 +619,7 @@ __device__ __forceinline__ void search_work_item(
 
     WaveState state;
     state.total = 0;
-    state.out_cursor = WRITE ? args.offsets[work] : 0;
+    state.out_cursor = WRITE ? args.offsets[row_slot] : 0;
     state.head = 0;
     state.tail = 0;
 
@@ -603,7 +627,7 @@ __device__ __forceinline__ void search_work_item(
         const uint32_t n_batch = min(static_cast<uint32_t>(MAX_ENTRIES), n_entries - batch);
         wave_sync(); // done with the previous batch's tables
 
-        fill_stencil_tables(sh, lane, centre + batch, n_batch, cx, cy, cz, span_y, span_z, g, args.cell_scan);
+        fill_stencil_tables(sh, lane, centre + batch, n_batch, cx, cy, cz, span_y, span_z, g, cell_scan);
 
         const uint32_t n_candidates = __builtin_amdgcn_readfirstlane(sh.n_candidates);
         const uint32_t n_groups = (n_candidates + WAVE * R - 1) / (WAVE * R);
@@ -699,7 +723,7 @@ __device__ __forceinline__ void search_work_item(
 
     if (!WRITE && lane == 0) {
         // a full list gets two rows per hit: the pair and its mirror
-        args.counts[work] = FULL ? 2 * state.total : state.total;
+        args.counts[row_slot] = FULL ? 2 * state.total : state.total;
     }
 }
 
@@ -720,7 +744,21 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void search_kernel(SearchArgs args, G
         if (WRITE && args.only != nullptr && args.only[work] == 0) {
             return;
         }
-        search_work_item<WRITE, FULL, R>(work, args, g, shared[wave], n_tiles, lane);
+        search_work_item<WRITE, FULL, R, false>(work, args, g, shared[wave], n_tiles, lane);
+    }
+}
+
+/// The same search over the tiles of many systems: every tile brings its system's grid along.
+template <bool WRITE, bool FULL, int R>
+__global__ __launch_bounds__(SEARCH_BLOCK) void search_kernel_batch(SearchArgs args) {
+    __shared__ std::conditional_t<WRITE, SearchSharedWrite, SearchSharedCount> shared[SEARCH_WAVES];
+    const int lane = lane_id();
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    const uint32_t n_tiles = static_cast<uint32_t>(args.cell_scan[args.total_cells] >> 32);
+    const uint32_t work = blockIdx.x * SEARCH_WAVES + wave;
+    if (work < args.n_work) {
+        GridParams unused;
+        search_work_item<WRITE, FULL, R, true>(work, args, unused, shared[wave], n_tiles, lane);
     }
 }
 
