@@ -241,21 +241,6 @@ struct ReplayState {
     uint32_t batch; // tickets the next redeem takes: 64, or fewer to bring the cursor to a multiple of ROW_ALIGN
 };
 
-/// Stores of 64 consecutive rows are fastest when they start on whole cache lines in all three arrays (16, 12 and
-/// 8 bytes per row): at multiples of 32 rows. A wave's first row is wherever the rows before it ended, so its first
-/// redeem takes just enough tickets to reach such a boundary.
-constexpr uint32_t ROW_ALIGN = 32;
-
-template <bool FULL>
-__device__ __forceinline__ uint32_t aligning_batch(uint64_t cursor) {
-    const uint32_t off = static_cast<uint32_t>(cursor) & (ROW_ALIGN - 1);
-    if (off == 0) {
-        return WAVE;
-    }
-    // a full list writes two rows per ticket (its cursor is always even)
-    return FULL ? (ROW_ALIGN - off) / 2 : ROW_ALIGN - off;
-}
-
 /// Redeem n <= 64 tickets: same rows as `redeem` of the two-pass search, candidates and tile points read from LDS.
 template <bool FULL>
 __device__ __forceinline__ void redeem_fused(

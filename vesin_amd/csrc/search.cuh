@@ -269,12 +269,28 @@ __device__ __forceinline__ void locate_candidate(
     packed = sh.ent_shift[lo];
 }
 
+/// Stores of 64 consecutive rows are fastest when they start on whole cache lines in all three arrays (16, 12 and
+/// 8 bytes per row): at multiples of 32 rows. A wave's first row is wherever the rows before it ended, so its first
+/// redeem takes just enough tickets to reach such a boundary.
+constexpr uint32_t ROW_ALIGN = 32;
+
+template <bool FULL>
+__device__ __forceinline__ uint32_t aligning_batch(uint64_t cursor) {
+    const uint32_t off = static_cast<uint32_t>(cursor) & (ROW_ALIGN - 1);
+    if (off == 0) {
+        return WAVE;
+    }
+    // a full list writes two rows per ticket (its cursor is always even)
+    return FULL ? (ROW_ALIGN - off) / 2 : ROW_ALIGN - off;
+}
+
 /// Per-wave progress, kept in scalar registers.
 struct WaveState {
     uint32_t total;      // COUNT: hits found so far
     uint64_t out_cursor; // WRITE: next output row of this wave
     uint32_t head;       // tickets appended to the ring
     uint32_t tail;       // tickets redeemed
+    uint32_t batch;      // WRITE: tickets the next redeem takes, see aligning_batch
 };
 
 /// Constants of one work item.
@@ -348,37 +364,22 @@ __device__ __forceinline__ void redeem(
         if (active) {
             const uint64_t forward_row = state.out_cursor + lane;
             const uint64_t mirror_row = forward_row + n;
-            ulonglong2 forward, backward;
-            forward.x = oi;
-            forward.y = oj;
-            backward.x = oj;
-            backward.y = oi;
-            reinterpret_cast<ulonglong2*>(out.pairs)[forward_row] = forward;
-            reinterpret_cast<ulonglong2*>(out.pairs)[mirror_row] = backward;
+            stream_store(reinterpret_cast<PairRow*>(out.pairs) + forward_row, PairRow{oi, oj});
+            stream_store(reinterpret_cast<PairRow*>(out.pairs) + mirror_row, PairRow{oj, oi});
             if (out.shifts != nullptr) {
-                int32_t* s = out.shifts + 3 * forward_row;
-                s[0] = sx;
-                s[1] = sy;
-                s[2] = sz;
-                int32_t* m = out.shifts + 3 * mirror_row;
-                m[0] = -sx;
-                m[1] = -sy;
-                m[2] = -sz;
+                stream_store(out.shifts + 3 * forward_row, ShiftRow{sx, sy, sz});
+                stream_store(out.shifts + 3 * mirror_row, ShiftRow{-sx, -sy, -sz});
             }
             if (out.distances != nullptr) {
                 const double d = sqrt(d2);
-                out.distances[forward_row] = d;
-                out.distances[mirror_row] = d;
+                stream_store(out.distances + forward_row, d);
+                stream_store(out.distances + mirror_row, d);
             }
             if (out.vectors != nullptr) {
-                double* v = out.vectors + 3 * forward_row;
-                v[0] = vx;
-                v[1] = vy;
-                v[2] = vz;
-                double* m = out.vectors + 3 * mirror_row;
-                m[0] = wx;
-                m[1] = wy;
-                m[2] = wz;
+                stream_store(out.vectors + 3 * forward_row, VectorHead{vx, vy});
+                stream_store(out.vectors + 3 * forward_row + 2, vz);
+                stream_store(out.vectors + 3 * mirror_row, VectorHead{wx, wy});
+                stream_store(out.vectors + 3 * mirror_row + 2, wz);
             }
         }
         state.out_cursor += 2 * n;
@@ -388,29 +389,22 @@ __device__ __forceinline__ void redeem(
         const bool flip = oi > oj || (oi == oj && !half_keeps_self_image(sx, sy, sz));
         if (active) {
             const uint64_t row = state.out_cursor + lane;
-            ulonglong2 pair;
-            pair.x = flip ? oj : oi;
-            pair.y = flip ? oi : oj;
-            reinterpret_cast<ulonglong2*>(out.pairs)[row] = pair;
+            stream_store(reinterpret_cast<PairRow*>(out.pairs) + row, PairRow{flip ? oj : oi, flip ? oi : oj});
             if (out.shifts != nullptr) {
-                int32_t* s = out.shifts + 3 * row;
-                s[0] = flip ? -sx : sx;
-                s[1] = flip ? -sy : sy;
-                s[2] = flip ? -sz : sz;
+                stream_store(out.shifts + 3 * row, ShiftRow{flip ? -sx : sx, flip ? -sy : sy, flip ? -sz : sz});
             }
             if (out.distances != nullptr) {
-                out.distances[row] = sqrt(d2);
+                stream_store(out.distances + row, sqrt(d2));
             }
             if (out.vectors != nullptr) {
-                double* v = out.vectors + 3 * row;
-                v[0] = flip ? wx : vx;
-                v[1] = flip ? wy : vy;
-                v[2] = flip ? wz : vz;
+                stream_store(out.vectors + 3 * row, VectorHead{flip ? wx : vx, flip ? wy : vy});
+                stream_store(out.vectors + 3 * row + 2, flip ? wz : vz);
             }
         }
         state.out_cursor += n;
     }
     state.tail += n;
+    state.batch = aligning_batch<FULL>(state.out_cursor);
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
 }
@@ -429,8 +423,8 @@ __device__ __forceinline__ void consume(
                 sh.ring[at] = static_cast<uint16_t>(ctx.lane | (r << 6) | (i << 8));
             }
             state.head += hits;
-            if (state.head - state.tail >= WAVE) {
-                redeem<FULL, R>(WAVE, state, c, sh, out, g, ctx);
+            while (state.head - state.tail >= state.batch) {
+                redeem<FULL, R>(state.batch, state, c, sh, out, g, ctx);
             }
         } else {
             state.total += hits;
@@ -622,6 +616,7 @@ __device__ __forceinline__ void search_work_item(
     state.out_cursor = WRITE ? args.offsets[row_slot] : 0;
     state.head = 0;
     state.tail = 0;
+    state.batch = aligning_batch<FULL>(state.out_cursor);
 
     for (uint32_t batch = 0; batch < n_entries; batch += MAX_ENTRIES) {
         const uint32_t n_batch = min(static_cast<uint32_t>(MAX_ENTRIES), n_entries - batch);
