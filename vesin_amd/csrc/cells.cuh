@@ -301,13 +301,13 @@ __global__ __launch_bounds__(BLOCK) void place_points(
     sorted.wy[to] = wy;
     sorted.wz[to] = wz;
     if ((wx | wy | wz) != 0) {
-        atomicOr(&tiles[first_tile + k / 64u].wrapped, 1u);
+        atomicOr(&tiles[first_tile + k / TILE_POINTS].wrapped, 1u);
     }
-    if (k % 64u == 0) {
-        Tile* tile = &tiles[first_tile + k / 64u];
+    if (k % TILE_POINTS == 0) {
+        Tile* tile = &tiles[first_tile + k / TILE_POINTS];
         tile->cell = cell;
         tile->first = to;
-        tile->count = min(64u, count - k);
+        tile->count = min(TILE_POINTS, count - k);
         if (system != 0) {
             atomicOr(&tile->wrapped, system << 1);
         }
@@ -406,15 +406,15 @@ __global__ __launch_bounds__(BLOCK) void gather_points(
     sorted.wz[to] = wz;
     if ((wx | wy | wz) != 0) {
         // tiles holding a wrapped point take the search kernel's general path
-        atomicOr(&tiles[first_tile + rank / 64u].wrapped, 1u);
+        atomicOr(&tiles[first_tile + rank / TILE_POINTS].wrapped, 1u);
     }
 
     const uint32_t k = p - start;
-    if (k % 64u == 0) {
-        Tile* tile = &tiles[first_tile + k / 64u];
+    if (k % TILE_POINTS == 0) {
+        Tile* tile = &tiles[first_tile + k / TILE_POINTS];
         tile->cell = cell;
         tile->first = start + k;
-        tile->count = min(64u, count - k);
+        tile->count = min(TILE_POINTS, count - k);
     }
 }
 
@@ -425,7 +425,7 @@ __global__ __launch_bounds__(BLOCK) void prepare_single_cell(
     uint64_t* __restrict__ cell_scan, DeviceStatus* status
 ) {
     uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
-    const uint32_t n_tiles = (g.n_points + 63u) / 64u;
+    const uint32_t n_tiles = (g.n_points + TILE_POINTS - 1) / TILE_POINTS;
     if (i == 0) {
         cell_scan[0] = 0;
         cell_scan[1] = static_cast<uint64_t>(g.n_points) | (static_cast<uint64_t>(n_tiles) << 32);
@@ -452,15 +452,17 @@ __global__ __launch_bounds__(BLOCK) void prepare_single_cell(
         sorted.wy[i] = wrap[1];
         sorted.wz[i] = wrap[2];
     }
-    // one wave covers exactly one tile of 64 consecutive points
-    const bool any_wrapped = __ballot(wrapped) != 0;
-    const uint32_t tile_id = i / 64u;
-    if (lane_id() == 0 && tile_id < n_tiles) {
+    // a wave covers WAVE / TILE_POINTS whole tiles of consecutive points
+    const uint64_t wrapped_lanes = __ballot(wrapped);
+    const uint32_t tile_id = i / TILE_POINTS;
+    const uint32_t first_lane = (lane_id() / TILE_POINTS) * TILE_POINTS;
+    const uint64_t tile_lanes = ((TILE_POINTS == WAVE ? 0ull : (1ull << TILE_POINTS)) - 1ull) << first_lane;
+    if (lane_id() % TILE_POINTS == 0 && tile_id < n_tiles) {
         Tile tile;
         tile.cell = 0;
-        tile.first = tile_id * 64u;
-        tile.count = min(64u, g.n_points - tile_id * 64u);
-        tile.wrapped = any_wrapped ? 1u : 0u;
+        tile.first = tile_id * TILE_POINTS;
+        tile.count = min(TILE_POINTS, g.n_points - tile_id * TILE_POINTS);
+        tile.wrapped = (wrapped_lanes & tile_lanes) != 0 ? 1u : 0u;
         tiles[tile_id] = tile;
     }
 }

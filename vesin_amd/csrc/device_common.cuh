@@ -9,6 +9,13 @@ namespace vesin_hip {
 
 constexpr int WAVE = 64;
 constexpr int BLOCK = 256;
+
+/// Points `i` one wave searches for at a time (a tile). 32 keeps the hit column of a candidate in one register and the
+/// tile's LDS record small, which buys a sixth wave per SIMD in the single-pass search; cells with more points
+/// simply make several tiles.
+constexpr uint32_t TILE_POINTS = 32;
+constexpr uint32_t TILE_SHIFT = 5;
+static_assert((1u << TILE_SHIFT) == TILE_POINTS, "TILE_SHIFT is log2 of TILE_POINTS");
 constexpr int WAVES_PER_BLOCK = BLOCK / WAVE;
 
 /// Everything a kernel needs to know about the box and the cell grid.
@@ -25,11 +32,11 @@ struct GridParams {
     uint32_t n_cells;
 };
 
-/// One row of 64 i-points (or fewer) that one workgroup searches for.
+/// One row of TILE_POINTS i-points (or fewer) that one wave searches for.
 struct Tile {
     uint32_t cell;   // linear cell index of these points
     uint32_t first;  // position of the first point in the cell-sorted arrays
-    uint32_t count;  // 1..64
+    uint32_t count;  // 1..TILE_POINTS
     uint32_t wrapped;// 1 when a point of the cell was moved by a box vector to land inside the box
 };
 

@@ -512,7 +512,7 @@ bool compute(
     // ---- carve the work buffers
     const size_t n_cells = grid.n_cells;
     // upper bound of the number of tiles, rounded up to what the search kernel's XCD-aware order needs
-    size_t tiles_bound = (single_cell ? 0 : std::min<size_t>(n_cells, n_points)) + n_points / 64 + 1;
+    size_t tiles_bound = (single_cell ? 0 : std::min<size_t>(n_cells, n_points)) + n_points / TILE_POINTS + 1;
     constexpr size_t slot_multiple = N_XCD * SEARCH_WAVES;
     tiles_bound = (tiles_bound + slot_multiple - 1) / slot_multiple * slot_multiple;
     // small systems: several workgroups (of one wave each) share a tile, each taking a slice of its candidates
@@ -972,7 +972,7 @@ void neighbors_batch(
     }
 
     // ---- work buffers
-    size_t tiles_bound = std::min<size_t>(total_cells, n_points) + n_points / 64 + 1;
+    size_t tiles_bound = std::min<size_t>(total_cells, n_points) + n_points / TILE_POINTS + 1;
     constexpr size_t slot_multiple = N_XCD * SEARCH_WAVES;
     tiles_bound = (tiles_bound + slot_multiple - 1) / slot_multiple * slot_multiple;
     uint32_t n_slices = 1;

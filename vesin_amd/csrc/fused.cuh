@@ -3,7 +3,7 @@
 // The two-pass search (search.cuh) evaluates every candidate pair twice, once to count and once to write, with a
 // device-wide scan between the two launches. Here a wave keeps the outcome of its tests instead: while it sweeps the
 // tile's points over 64 candidates held in registers, every candidate lane shifts the hit bit of each tile point into
-// a 64-bit column (one v_addc per test, fed by the compare's lane mask). After the sweep the wave knows its number of
+// a 32-bit column (one v_addc per test, fed by the compare's lane mask; a tile has at most 32 points). After the sweep the wave knows its number of
 // rows; the workgroups then chain their totals (64-bit words holding a flag and a value, written and polled with
 // device-scope atomics; decoupled look-back over groups of workgroups), which hands every wave its first output row.
 // The wave finally replays its columns: each round every lane with hits left peels one bit off its column and drops
@@ -57,9 +57,9 @@ struct FusedArgs {
 
 /// LDS of one wave.
 struct FusedWaveShared: SearchTables {
-    double tile_x[WAVE], tile_y[WAVE], tile_z[WAVE];
-    uint32_t tile_index[WAVE];
-    int32_t tile_wx[WAVE], tile_wy[WAVE], tile_wz[WAVE];
+    double tile_x[TILE_POINTS], tile_y[TILE_POINTS], tile_z[TILE_POINTS];
+    uint32_t tile_index[TILE_POINTS];
+    int32_t tile_wx[TILE_POINTS], tile_wy[TILE_POINTS], tile_wz[TILE_POINTS];
     double cand_x[FUSED_SLOTS], cand_y[FUSED_SLOTS], cand_z[FUSED_SLOTS];
     uint32_t cand_index[FUSED_SLOTS];
     int32_t cand_shift[FUSED_SLOTS]; // packed: cell shift minus the candidate's own wrap shift
@@ -119,11 +119,12 @@ struct SweepCandidates {
     uint32_t position[R];  // see Candidates::position
 };
 
-/// Up to 32 consecutive tile points (from cell-sorted position `first`) against the R x 64 candidates; every
-/// candidate lane shifts its hit bits into `column` (the first point ends up in the highest bit used). Returns the
-/// number of hits.
+static_assert(TILE_POINTS <= 32, "the hit column of a candidate is one 32-bit register");
+
+/// The tile's points (from cell-sorted position `first`) against the R x 64 candidates; every candidate lane
+/// shifts its hit bits into `column` (the first point ends up in the highest bit used). Returns the number of hits.
 template <int R, bool SHIFTED, bool SAME>
-__device__ __forceinline__ uint32_t sweep_half(
+__device__ __forceinline__ uint32_t sweep_columns(
     const SortedPoints& sorted, uint32_t first, uint32_t count, const SweepCandidates<R>& c, double cutoff2,
     uint32_t (&column)[R]
 ) {
@@ -162,34 +163,14 @@ __device__ __forceinline__ uint32_t sweep_half(
     return total;
 }
 
-/// Every tile point against the R x 64 candidates: points 0..31 go to the `lo` columns, 32..63 to `hi`.
-template <int R, bool SHIFTED, bool SAME>
-__device__ __forceinline__ uint32_t sweep_columns(
-    const SortedPoints& sorted, uint32_t first_i, uint32_t n_i, const SweepCandidates<R>& c, double cutoff2,
-    uint32_t (&lo)[R], uint32_t (&hi)[R]
-) {
-    uint32_t total = sweep_half<R, SHIFTED, SAME>(sorted, first_i, min(n_i, 32u), c, cutoff2, lo);
-    if (n_i > 32) {
-        total += sweep_half<R, SHIFTED, SAME>(sorted, first_i + 32, n_i - 32, c, cutoff2, hi);
-    }
-    return total;
-}
-
 /// Variant for a tile holding points that were wrapped into the box: the shift of a pair depends on both points.
 template <int R>
 __device__ __forceinline__ uint32_t sweep_columns_wrapped(
     const SortedPoints& sorted, uint32_t first_i, uint32_t n_i, const SweepCandidates<R>& c, const GridParams& g,
-    uint32_t (&lo)[R], uint32_t (&hi)[R]
+    uint32_t (&column)[R]
 ) {
     uint32_t total = 0;
     for (uint32_t i = 0; i < n_i; i++) {
-        if (i == 32) {
-#pragma unroll
-            for (int r = 0; r < R; r++) {
-                hi[r] = lo[r];
-                lo[r] = 0;
-            }
-        }
         const uint32_t at = first_i + i;
         const double xi = sorted.x[at];
         const double yi = sorted.y[at];
@@ -209,16 +190,7 @@ __device__ __forceinline__ uint32_t sweep_columns_wrapped(
             const double d2 = vx * vx + vy * vy + vz * vz;
             const uint64_t mask = __ballot(d2 < g.cutoff2) & __ballot(c.position[r] > at);
             total += __popcll(mask);
-            lo[r] = shift_in(lo[r], mask);
-        }
-    }
-    if (n_i > 32) {
-        // the first 32 points were parked in `hi` while the rest went through `lo`
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            const uint32_t rest = lo[r];
-            lo[r] = hi[r];
-            hi[r] = rest;
+            column[r] = shift_in(column[r], mask);
         }
     }
     return total;
@@ -230,8 +202,7 @@ struct ReplayContext {
     bool need_shift;   // some candidate of the work item has a non-zero shift, or the tile holds wrapped points
     bool tile_wrapped;
     int lane;
-    uint32_t last_lo; // tile point of bit 0 of the low half of a column: min(n_i, 32) - 1
-    uint32_t last_hi; // same for the high half: n_i - 1
+    uint32_t last;     // tile point of bit 0 of a column: n_i - 1
 };
 
 struct ReplayState {
@@ -252,12 +223,11 @@ __device__ __forceinline__ void redeem_fused(
     const int lane = ctx.lane;
     const bool active = static_cast<uint32_t>(lane) < n;
     const uint32_t ticket = sh.ring[(state.tail + lane) & (RING - 1)];
-    // ticket: candidate record (7 bits), bit of the column (5 bits, from bit 8), half of the column (bit 13); the
-    // first point of a half sits in the highest bit used
+    // ticket: candidate record (7 bits), bit of the column (5 bits, from bit 8); the tile's first point sits in the
+    // highest bit used
     const int slot = active ? ticket & (FUSED_SLOTS - 1) : 0;
     const uint32_t bit = (ticket >> 8) & 31;
-    const bool high = (ticket >> 13) & 1;
-    const int il = active ? static_cast<int>((high ? ctx.last_hi : ctx.last_lo) - bit) : 0;
+    const int il = active ? static_cast<int>(ctx.last - bit) : 0;
 
     const double xj = sh.cand_x[slot];
     const double yj = sh.cand_y[slot];
@@ -511,12 +481,10 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fa
     item.n_batch = 0;
     item.n_candidates = 0;
     // hit columns of the work item's units; indexed with wave-uniform values only
-    uint32_t columns_lo[FUSED_UNITS];
-    uint32_t columns_hi[FUSED_UNITS];
+    uint32_t columns[FUSED_UNITS];
 #pragma unroll
     for (int u = 0; u < FUSED_UNITS; u++) {
-        columns_lo[u] = 0;
-        columns_hi[u] = 0;
+        columns[u] = 0;
     }
 
     // ---- phase 1: sweep, keep the columns
@@ -609,30 +577,28 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fa
                     }
                     item.any_shift = item.any_shift || any_shift;
 
-                    uint32_t lo[R] = {0, 0};
-                    uint32_t hi[R] = {0, 0};
+                    uint32_t column[R] = {0, 0};
                     uint32_t hits;
                     if (item.tile_wrapped) {
-                        hits = sweep_columns_wrapped<R>(sorted, item.first_i, item.n_i, c, g, lo, hi);
+                        hits = sweep_columns_wrapped<R>(sorted, item.first_i, item.n_i, c, g, column);
                     } else if (any_shift) {
                         if (any_same) {
-                            hits = sweep_columns<R, true, true>(sorted, item.first_i, item.n_i, c, g.cutoff2, lo, hi);
+                            hits = sweep_columns<R, true, true>(sorted, item.first_i, item.n_i, c, g.cutoff2, column);
                         } else {
-                            hits = sweep_columns<R, true, false>(sorted, item.first_i, item.n_i, c, g.cutoff2, lo, hi);
+                            hits = sweep_columns<R, true, false>(sorted, item.first_i, item.n_i, c, g.cutoff2, column);
                         }
                     } else {
                         if (any_same) {
-                            hits = sweep_columns<R, false, true>(sorted, item.first_i, item.n_i, c, g.cutoff2, lo, hi);
+                            hits = sweep_columns<R, false, true>(sorted, item.first_i, item.n_i, c, g.cutoff2, column);
                         } else {
-                            hits = sweep_columns<R, false, false>(sorted, item.first_i, item.n_i, c, g.cutoff2, lo, hi);
+                            hits = sweep_columns<R, false, false>(sorted, item.first_i, item.n_i, c, g.cutoff2, column);
                         }
                     }
                     item.hits += hits;
                     if (pair * R < FUSED_UNITS) {
 #pragma unroll
                         for (int r = 0; r < R; r++) {
-                            columns_lo[pair * R + r] = lo[r];
-                            columns_hi[pair * R + r] = hi[r];
+                            columns[pair * R + r] = column[r];
                         }
                     }
                 }
@@ -719,14 +685,12 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fa
     state.head = 0;
     state.tail = 0;
     state.batch = aligning_batch<FULL>(state.out_cursor);
-    ctx.last_lo = min(item.n_i, 32u) - 1;
-    ctx.last_hi = item.n_i - 1;
+    ctx.last = item.n_i - 1;
     uint32_t filled[2] = {0, 0}; // value of head when the unit in each half of the candidate records was done
 
     for (uint32_t unit = 0; unit < item.n_units; unit++) {
-        uint32_t lo = columns_lo[unit];
-        uint32_t hi = columns_hi[unit];
-        if (__ballot((lo | hi) != 0) == 0) {
+        uint32_t column = columns[unit];
+        if (__ballot(column != 0) == 0) {
             continue;
         }
         const uint32_t half = unit & 1;
@@ -746,28 +710,22 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fa
         }
         wave_sync();
 
-        // every round, each lane with hits left peels one bit off its column and drops a ticket; the low half of
-        // the columns first, then (tiles of more than 32 points) the high half
+        // every round, each lane with hits left peels one bit off its column and drops a ticket
         const uint32_t record = half * WAVE + lane;
-#pragma nounroll
-        for (int part = 0; part < 2; part++) {
-            uint32_t column = part == 0 ? lo : hi;
-            const uint32_t tag = record | (part << 13);
-            while (true) {
-                const uint64_t mask = __ballot(column != 0);
-                if (mask == 0) {
-                    break;
-                }
-                if (column != 0) {
-                    const uint32_t bit = __builtin_ctz(column);
-                    column &= column - 1;
-                    const uint32_t at = (state.head + rank_in_mask(mask)) & (RING - 1);
-                    sh.ring[at] = static_cast<uint16_t>(tag | (bit << 8));
-                }
-                state.head += __popcll(mask);
-                while (state.head - state.tail >= state.batch) {
-                    redeem_fused<FULL>(state.batch, state, sh, args.out, g, ctx);
-                }
+        while (true) {
+            const uint64_t mask = __ballot(column != 0);
+            if (mask == 0) {
+                break;
+            }
+            if (column != 0) {
+                const uint32_t bit = __builtin_ctz(column);
+                column &= column - 1;
+                const uint32_t at = (state.head + rank_in_mask(mask)) & (RING - 1);
+                sh.ring[at] = static_cast<uint16_t>(record | (bit << 8));
+            }
+            state.head += __popcll(mask);
+            while (state.head - state.tail >= state.batch) {
+                redeem_fused<FULL>(state.batch, state, sh, args.out, g, ctx);
             }
         }
         if (half == 0) {

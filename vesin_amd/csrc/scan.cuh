@@ -16,7 +16,7 @@ constexpr int SCAN_TILE = BLOCK * SCAN_ITEMS; // 2048 elements per workgroup
 /// What the scan reads.
 enum ScanInput {
     SCAN_U32 = 0,        // plain 32-bit counts
-    SCAN_CELL_COUNTS = 1,// 32-bit points-per-cell; scanned value = count | (number of 64-point tiles << 32)
+    SCAN_CELL_COUNTS = 1,// 32-bit points-per-cell; scanned value = count | (number of tiles << 32)
     SCAN_U64 = 2,        // 64-bit values (tile sums of a previous level)
 };
 
@@ -27,7 +27,7 @@ __device__ __forceinline__ uint64_t scan_load(const void* in, size_t i) {
     }
     uint32_t v = static_cast<const uint32_t*>(in)[i];
     if (INPUT == SCAN_CELL_COUNTS) {
-        return static_cast<uint64_t>(v) | (static_cast<uint64_t>((v + 63u) >> 6) << 32);
+        return static_cast<uint64_t>(v) | (static_cast<uint64_t>((v + TILE_POINTS - 1) >> TILE_SHIFT) << 32);
     }
     return v;
 }

@@ -147,9 +147,9 @@ constexpr int MAX_R = 2;
 
 struct SearchSharedWrite: SearchTables {
     // the tile's points, for the redeem phase
-    double tile_x[WAVE], tile_y[WAVE], tile_z[WAVE];
-    uint32_t tile_index[WAVE];
-    int32_t tile_wx[WAVE], tile_wy[WAVE], tile_wz[WAVE];
+    double tile_x[TILE_POINTS], tile_y[TILE_POINTS], tile_z[TILE_POINTS];
+    uint32_t tile_index[TILE_POINTS];
+    int32_t tile_wx[TILE_POINTS], tile_wy[TILE_POINTS], tile_wz[TILE_POINTS];
     // the candidates currently held in registers, where any lane can fetch them when it redeems a ticket
     double cand_x[MAX_R * WAVE], cand_y[MAX_R * WAVE], cand_z[MAX_R * WAVE];
     uint32_t cand_index[MAX_R * WAVE];
