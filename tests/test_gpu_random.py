@@ -1,0 +1,85 @@
+"""Randomised differential test of the HIP path against the CPU oracle (``-m gpu``): many small systems with random
+boxes, periodicity, densities and cutoffs go through ONE reused list per option set, so that consecutive calls
+exercise the single-pass search, its fallbacks (growth, crowded tiles, wrapped points), the remembered box and the
+sliced small-system layout in whatever order the generator produces them."""
+
+import numpy as np
+import pytest
+
+import oracle
+from _helpers import assert_same_list
+from vesin_amd import NeighborList
+
+pytestmark = pytest.mark.gpu
+
+NAMES = {"P": "pairs", "S": "shifts", "d": "distances", "D": "vectors"}
+
+
+def random_system(rng):
+    kind = rng.integers(0, 6)
+    n = int(rng.choice([1, 2, 3, 17, 64, 65, 200, 700, 1500]))
+    edge = float(rng.uniform(3.0, 14.0))
+    if kind == 0:  # cubic
+        box = np.eye(3) * edge
+    elif kind == 1:  # orthorhombic, one short axis (several images along it)
+        box = np.diag([edge, edge * rng.uniform(0.2, 0.5), edge * rng.uniform(0.8, 1.6)])
+    else:  # triclinic
+        box = np.eye(3) * edge + rng.normal(scale=0.25 * edge, size=(3, 3)) * (np.arange(3)[:, None] > np.arange(3)[None, :])
+    periodic = [bool(b) for b in rng.integers(0, 2, size=3)] if rng.random() < 0.5 else [True, True, True]
+    points = rng.random((n, 3)) @ box
+    if kind == 3:  # a crowded corner
+        points[: n // 2] = points[: n // 2] * 0.15
+    if kind == 4:  # points far outside the box
+        points = points + rng.integers(-3, 4, size=(n, 3)) @ box
+    if kind == 5 and n > 3:  # coincident points
+        points[1] = points[0]
+        points[-1] = points[-2]
+    return points, box, periodic
+
+
+@pytest.mark.parametrize("full", [True, False], ids=["full", "half"])
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_random_systems_on_one_reused_list(seed, full):
+    import torch
+
+    rng = np.random.default_rng(1000 + seed)
+    cutoff = float(rng.choice([1.5, 2.5, 3.7]))
+    calculator = NeighborList(cutoff=cutoff, full_list=full)
+    for step in range(14):
+        points, box, periodic = random_system(rng)
+        expected = oracle.neighbors(points, box, periodic, cutoff, full, False, "ijSdD")
+        for repeat in range(2):  # the second call on the same input meets the remembered box and kept arrays
+            outputs = calculator.compute(
+                torch.as_tensor(points, device="cuda:0"), torch.as_tensor(box, device="cuda:0"), periodic, "PSdD"
+            )
+            actual = {NAMES[q]: t.cpu().numpy() for q, t in zip("PSdD", outputs)}
+            assert_same_list(actual, expected, what=f"seed {seed} step {step} repeat {repeat} n={len(points)} periodic={periodic}")
+
+
+def test_random_batches():
+    import torch
+
+    rng = np.random.default_rng(77)
+    for trial in range(4):
+        cutoff = float(rng.choice([2.0, 3.0]))
+        full = bool(rng.integers(0, 2))
+        n_systems = int(rng.integers(1, 12))
+        all_points, all_boxes = [], []
+        for _ in range(n_systems):
+            points, box, _ = random_system(rng)
+            all_points.append(points)
+            all_boxes.append(box)
+        first_point = np.cumsum([0] + [len(p) for p in all_points])
+        calculator = NeighborList(cutoff=cutoff, full_list=full)
+        outputs, first_pair = calculator.compute_batch(
+            torch.as_tensor(np.concatenate(all_points), device="cuda:0"),
+            first_point,
+            torch.as_tensor(np.stack(all_boxes), device="cuda:0"),
+            True,
+            "PSdD",
+        )
+        whole = {NAMES[q]: t.cpu().numpy() for q, t in zip("PSdD", outputs)}
+        for s in range(n_systems):
+            rows = slice(int(first_pair[s]), int(first_pair[s + 1]))
+            expected = oracle.neighbors(all_points[s], all_boxes[s], True, cutoff, full, False, "ijSdD")
+            assert_same_list({k: v[rows] for k, v in whole.items()}, expected, what=f"trial {trial} system {s}")
