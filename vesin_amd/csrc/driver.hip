@@ -60,6 +60,31 @@ static bool two_pass_only() {
 
 namespace {
 
+/// Makes `device` current for a scope and gives the caller's device back afterwards.
+struct DeviceGuard {
+    int previous = -1;
+    int wanted;
+
+    explicit DeviceGuard(int device): wanted(device) {
+        if (hipGetDevice(&previous) != hipSuccess) {
+            (void)hipGetLastError();
+            previous = -1;
+        }
+        if (previous != wanted) {
+            HIP_CHECK(hipSetDevice(wanted));
+        }
+    }
+
+    ~DeviceGuard() {
+        if (previous >= 0 && previous != wanted) {
+            (void)hipSetDevice(previous);
+        }
+    }
+
+    DeviceGuard(const DeviceGuard&) = delete;
+    DeviceGuard& operator=(const DeviceGuard&) = delete;
+};
+
 /// Grow-only device allocation.
 struct DeviceBuffer {
     void* ptr = nullptr;
@@ -351,7 +376,7 @@ void neighbors(
         throw std::runtime_error("too many points: the GPU path indexes points with 32 bits");
     }
 
-    HIP_CHECK(hipSetDevice(device_id));
+    const DeviceGuard guard(device_id);
     HipExtras& extras = extras_of(neighbors);
     extras.timings_valid = false;
 
@@ -901,7 +926,7 @@ void neighbors_batch(
         throw std::runtime_error("`periodic` pointer is not allocated on the GPU of the neighbor list");
     }
 
-    HIP_CHECK(hipSetDevice(device_id));
+    const DeviceGuard guard(device_id);
     HipExtras& extras = extras_of(neighbors);
     extras.timings_valid = false;
     extras.have_last_box = false; // the work buffers of the single-system path are about to be reused
@@ -1109,7 +1134,7 @@ void neighbors_batch(
 }
 
 void free_neighbors(VesinNeighborList& neighbors) {
-    HIP_CHECK(hipSetDevice(neighbors.device.device_id));
+    const DeviceGuard guard(neighbors.device.device_id);
     free_outputs(neighbors);
     delete static_cast<HipExtras*>(neighbors.opaque);
     neighbors.opaque = nullptr;
