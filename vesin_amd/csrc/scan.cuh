@@ -105,6 +105,42 @@ __global__ __launch_bounds__(BLOCK) void scan_tile_write(
     }
 }
 
+/// scan_tile_write for inputs of at most BLOCK tiles: instead of reading its offset from a scanned array of tile
+/// sums, every workgroup adds up the sums of the tiles before its own (one per thread). Saves the launch of the
+/// middle level.
+template <int INPUT>
+__global__ __launch_bounds__(BLOCK) void scan_tile_write_few(
+    const void* __restrict__ in, size_t n, const uint64_t* __restrict__ sums, uint64_t* __restrict__ out
+) {
+    __shared__ uint64_t wave_sums[WAVES_PER_BLOCK];
+    uint64_t before = threadIdx.x < blockIdx.x ? sums[threadIdx.x] : 0;
+    uint64_t offset;
+    block_exclusive_scan(before, offset, wave_sums);
+
+    size_t base = static_cast<size_t>(blockIdx.x) * SCAN_TILE + static_cast<size_t>(threadIdx.x) * SCAN_ITEMS;
+    uint64_t items[SCAN_ITEMS];
+    uint64_t local = 0;
+#pragma unroll
+    for (int k = 0; k < SCAN_ITEMS; k++) {
+        size_t i = base + k;
+        items[k] = i < n ? scan_load<INPUT>(in, i) : 0;
+        local += items[k];
+    }
+    uint64_t total;
+    uint64_t running = block_exclusive_scan(local, total, wave_sums) + offset;
+#pragma unroll
+    for (int k = 0; k < SCAN_ITEMS; k++) {
+        size_t i = base + k;
+        if (i < n) {
+            out[i] = running;
+        }
+        running += items[k];
+        if (i + 1 == n) {
+            out[n] = running;
+        }
+    }
+}
+
 inline size_t scan_tiles(size_t n) {
     return n == 0 ? 1 : (n + SCAN_TILE - 1) / SCAN_TILE;
 }
@@ -131,6 +167,10 @@ inline void exclusive_scan(const void* in, size_t n, uint64_t* out, uint64_t* sc
     uint64_t* sums = scratch;
     uint64_t* offsets = scratch + (tiles + 1);
     hipLaunchKernelGGL(scan_tile_sums<INPUT>, dim3(tiles), dim3(BLOCK), 0, stream, in, n, sums);
+    if (tiles <= BLOCK) {
+        hipLaunchKernelGGL(scan_tile_write_few<INPUT>, dim3(tiles), dim3(BLOCK), 0, stream, in, n, sums, out);
+        return;
+    }
     exclusive_scan<SCAN_U64>(sums, tiles, offsets, scratch + 2 * (tiles + 1), stream);
     hipLaunchKernelGGL(scan_tile_write<INPUT>, dim3(tiles), dim3(BLOCK), 0, stream, in, n, offsets, out);
 }
