@@ -211,3 +211,16 @@ def test_a_box_that_becomes_singular():
     # and the list is still usable
     expected = oracle.neighbors(points, box, periodic, 5.0, True, False, "ijSdD")
     assert_same_list(call(calculator, points, box, periodic), expected)
+
+
+def test_stencils_larger_than_the_single_pass_tables(timings):
+    # cutoff almost three box lengths: 7^3 images, more stencil entries than the single pass keeps in LDS; every
+    # call of the list falls back to the two passes (which walk the stencil in batches)
+    rng = np.random.default_rng(41)
+    box = np.array([[3.1, 0.0, 0.0], [0.4, 2.9, 0.0], [-0.3, 0.5, 3.3]])
+    points = rng.random((40, 3)) @ box
+    expected = oracle.neighbors(points, box, True, 8.0, True, False, "ijSdD")
+    calculator = NeighborList(cutoff=8.0, full_list=True)
+    for repeat in range(3):
+        assert_same_list(call(calculator, points, box, True), expected, what=f"call {repeat + 1}")
+        assert not used_single_pass(calculator)
