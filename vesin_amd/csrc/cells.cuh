@@ -55,6 +55,31 @@ __global__ void fetch_box(
     }
 }
 
+/// Clears `n_blocks16` 16-byte blocks from `begin` (the histogram, the tiles' flags and the state of the single-pass
+/// search live next to each other), and does the work of fetch_box on the way when `box` is not null: one launch
+/// at the start of a call instead of a fetch and two fills.
+__global__ __launch_bounds__(BLOCK) void clear_and_fetch(
+    uint4* __restrict__ begin, size_t n_blocks16, const double* __restrict__ box, const bool* __restrict__ periodic,
+    unsigned char* host_small, DeviceStatus* status
+) {
+    if (box != nullptr && blockIdx.x == 0) {
+        const int t = threadIdx.x;
+        if (t < 9) {
+            reinterpret_cast<double*>(host_small)[t] = box[t];
+        } else if (t < 12) {
+            host_small[72 + (t - 9)] = periodic[t - 9] ? 1 : 0;
+        } else if (t == 12) {
+            status->total_pairs = 0;
+            status->first_bad_coordinate = 0xFFFFFFFFu;
+        }
+    }
+    const uint4 zero = {0u, 0u, 0u, 0u};
+    for (size_t k = static_cast<size_t>(blockIdx.x) * BLOCK + threadIdx.x; k < n_blocks16;
+         k += static_cast<size_t>(gridDim.x) * BLOCK) {
+        begin[k] = zero;
+    }
+}
+
 /// After the counting pass: what the host needs to know goes to pinned host memory, read after the next
 /// synchronisation of the stream.
 __global__ void publish_status(const DeviceStatus* status, const uint64_t* total, DeviceStatus* host_status) {
@@ -245,11 +270,14 @@ __global__ __launch_bounds__(BLOCK) void assign_cells(
     }
     base = static_cast<uint32_t>(__shfl(static_cast<int>(base), first));
     if (active) {
-        cell_of[i] = linear;
         slot_of[i] = base + rank_in_mask(group);
-        wrap_of[3 * static_cast<size_t>(i) + 0] = wrap[0];
-        wrap_of[3 * static_cast<size_t>(i) + 1] = wrap[1];
-        wrap_of[3 * static_cast<size_t>(i) + 2] = wrap[2];
+        // callers that place the points with `place_points` do not need these: it locates the point again
+        if (cell_of != nullptr) {
+            cell_of[i] = linear;
+            wrap_of[3 * static_cast<size_t>(i) + 0] = wrap[0];
+            wrap_of[3 * static_cast<size_t>(i) + 1] = wrap[1];
+            wrap_of[3 * static_cast<size_t>(i) + 2] = wrap[2];
+        }
     }
 }
 
@@ -268,18 +296,42 @@ __global__ __launch_bounds__(BLOCK) void scatter_points(
 
 /// Counting-sort scatter straight into the structure-of-arrays layout, for callers that do not need the order of
 /// the points inside a cell to be the same on every run: the slot handed out by the histogram atomic is final.
-/// Also appends the cell's tiles. `tiles[].wrapped` must be zero on entry.
+/// Also appends the cell's tiles. `tiles[].wrapped` must be zero on entry. Cell and wrap shift of the point come
+/// from `cell_of` / `wrap_of` when given (a batch of systems), else the point is located again with `g`: cheaper
+/// than carrying 16 bytes per point from assign_cells through memory.
 __global__ __launch_bounds__(BLOCK) void place_points(
-    const double* __restrict__ points, const int32_t* __restrict__ wrap_of, const uint32_t* __restrict__ cell_of,
-    const uint32_t* __restrict__ slot_of, const uint64_t* __restrict__ cell_scan, uint32_t n_points,
-    SortedPoints sorted, Tile* __restrict__ tiles,
+    const double* __restrict__ points, GridParams g, const int32_t* __restrict__ wrap_of,
+    const uint32_t* __restrict__ cell_of, const uint32_t* __restrict__ slot_of,
+    const uint64_t* __restrict__ cell_scan, uint32_t n_points, SortedPoints sorted, Tile* __restrict__ tiles,
     const uint32_t* __restrict__ system_of, const uint32_t* __restrict__ first_point
 ) {
     const uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
     if (i >= n_points) {
         return;
     }
-    const uint32_t cell = cell_of[i];
+    const double x = points[3 * static_cast<size_t>(i) + 0];
+    const double y = points[3 * static_cast<size_t>(i) + 1];
+    const double z = points[3 * static_cast<size_t>(i) + 2];
+    uint32_t cell;
+    int32_t wx, wy, wz;
+    if (cell_of != nullptr) {
+        cell = cell_of[i];
+        wx = wrap_of[3 * static_cast<size_t>(i) + 0];
+        wy = wrap_of[3 * static_cast<size_t>(i) + 1];
+        wz = wrap_of[3 * static_cast<size_t>(i) + 2];
+    } else {
+        // same inputs and code as in assign_cells: the same cell
+        int32_t where[3] = {0, 0, 0};
+        int32_t wrap[3] = {0, 0, 0};
+        unsigned int axis;
+        if (all_finite(x, y, z, axis)) {
+            locate(g, x, y, z, where, wrap);
+        }
+        cell = (static_cast<uint32_t>(where[2]) * g.n[1] + where[1]) * g.n[0] + where[0];
+        wx = wrap[0];
+        wy = wrap[1];
+        wz = wrap[2];
+    }
     const uint64_t here = cell_scan[cell];
     const uint32_t start = static_cast<uint32_t>(here);
     const uint32_t count = static_cast<uint32_t>(cell_scan[cell + 1]) - start;
@@ -287,16 +339,13 @@ __global__ __launch_bounds__(BLOCK) void place_points(
     const uint32_t k = slot_of[i];
     const uint32_t to = start + k;
 
-    const int32_t wx = wrap_of[3 * static_cast<size_t>(i) + 0];
-    const int32_t wy = wrap_of[3 * static_cast<size_t>(i) + 1];
-    const int32_t wz = wrap_of[3 * static_cast<size_t>(i) + 2];
     // in a batch (system_of not null) the index counts from the first point of the point's system, and the tile
     // carries the system above its flag bit
     const uint32_t system = system_of != nullptr ? system_of[i] : 0;
     sorted.index[to] = system_of != nullptr ? i - first_point[system] : i;
-    sorted.x[to] = points[3 * static_cast<size_t>(i) + 0];
-    sorted.y[to] = points[3 * static_cast<size_t>(i) + 1];
-    sorted.z[to] = points[3 * static_cast<size_t>(i) + 2];
+    sorted.x[to] = x;
+    sorted.y[to] = y;
+    sorted.z[to] = z;
     sorted.wx[to] = wx;
     sorted.wy[to] = wy;
     sorted.wz[to] = wz;

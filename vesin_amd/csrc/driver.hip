@@ -441,15 +441,21 @@ bool compute(
         }
     };
 
-    // ---- box and periodicity come to the host once: 75 bytes
-    hipLaunchKernelGGL(
-        fetch_box, dim3(1), dim3(64), 0, stream,
-        reinterpret_cast<const double*>(box), periodic, extras.h_small, extras.d_status
-    );
+    // ---- box and periodicity come to the host once: 75 bytes. A call that starts from the remembered box fetches
+    // them with its first fill kernel instead (see below).
+    auto launch_fetch = [&]() {
+        hipLaunchKernelGGL(
+            fetch_box, dim3(1), dim3(64), 0, stream,
+            reinterpret_cast<const double*>(box), periodic, extras.h_small, extras.d_status
+        );
+    };
+    bool fetched = false;
     unsigned char used_box[BOX_BYTES];
     if (speculate) {
         std::memcpy(used_box, extras.last_box, BOX_BYTES);
     } else {
+        launch_fetch();
+        fetched = true;
         HIP_CHECK(hipStreamSynchronize(stream));
         std::memcpy(used_box, extras.h_small, BOX_BYTES);
         std::memcpy(extras.last_box, used_box, BOX_BYTES);
@@ -492,6 +498,10 @@ bool compute(
     double lo[3] = {0, 0, 0};
     double hi[3] = {0, 0, 0};
     if (any_open) {
+        if (!fetched) {
+            launch_fetch(); // the synchronisation below is where a remembered box is checked first
+            fetched = true;
+        }
         const uint32_t blocks = static_cast<uint32_t>(std::min<size_t>(BOUNDING_BLOCKS, (n_points + BLOCK - 1) / BLOCK));
         hipLaunchKernelGGL(
             bounding_kernel, dim3(blocks), dim3(BLOCK), 0, stream,
@@ -601,8 +611,16 @@ bool compute(
     const uint32_t point_blocks = static_cast<uint32_t>((n_points + BLOCK - 1) / BLOCK);
     const auto* flat_points = reinterpret_cast<const double*>(points);
     {
+        // every piece of the work buffer is padded to 256 bytes: clearing whole 16-byte blocks stays inside
         const size_t to_clear = reinterpret_cast<char*>(fused_status + 1) - reinterpret_cast<char*>(cell_counts);
-        HIP_CHECK(hipMemsetAsync(cell_counts, 0, to_clear, stream));
+        const size_t blocks16 = (to_clear + 15) / 16;
+        const uint32_t fill_blocks = static_cast<uint32_t>(std::min<size_t>(1024, (blocks16 + BLOCK - 1) / BLOCK));
+        hipLaunchKernelGGL(
+            clear_and_fetch, dim3(fill_blocks), dim3(BLOCK), 0, stream,
+            reinterpret_cast<uint4*>(cell_counts), blocks16,
+            fetched ? static_cast<const double*>(nullptr) : reinterpret_cast<const double*>(box), periodic,
+            extras.h_small, extras.d_status
+        );
     }
     if (single_cell) {
         hipLaunchKernelGGL(
@@ -610,12 +628,14 @@ bool compute(
             flat_points, g, sorted, tiles, cell_scan, extras.d_status
         );
     } else {
+        const bool ordered = ordered_rows();
         hipLaunchKernelGGL(
             assign_cells, dim3(point_blocks), dim3(BLOCK), 0, stream,
-            flat_points, g, cell_of, slot_of, wrap_of, cell_counts, extras.d_status
+            flat_points, g, ordered ? cell_of : static_cast<uint32_t*>(nullptr), slot_of,
+            ordered ? wrap_of : static_cast<int32_t*>(nullptr), cell_counts, extras.d_status
         );
         exclusive_scan<SCAN_CELL_COUNTS>(cell_counts, n_cells, cell_scan, scan_scratch, stream);
-        if (ordered_rows()) {
+        if (ordered) {
             // the same order of the points inside every cell on every run
             hipLaunchKernelGGL(
                 scatter_points, dim3(point_blocks), dim3(BLOCK), 0, stream,
@@ -628,7 +648,8 @@ bool compute(
         } else {
             hipLaunchKernelGGL(
                 place_points, dim3(point_blocks), dim3(BLOCK), 0, stream,
-                flat_points, wrap_of, cell_of, slot_of, cell_scan, g.n_points, sorted, tiles,
+                flat_points, g, static_cast<const int32_t*>(nullptr), static_cast<const uint32_t*>(nullptr), slot_of,
+                cell_scan, g.n_points, sorted, tiles,
                 static_cast<const uint32_t*>(nullptr), static_cast<const uint32_t*>(nullptr)
             );
         }
@@ -1079,7 +1100,7 @@ void neighbors_batch(
     exclusive_scan<SCAN_CELL_COUNTS>(cell_counts, total_cells, cell_scan, scan_scratch, stream);
     hipLaunchKernelGGL(
         place_points, dim3(point_blocks), dim3(BLOCK), 0, stream,
-        flat_points, wrap_of, cell_of, slot_of, cell_scan, static_cast<uint32_t>(n_points), sorted, tiles,
+        flat_points, GridParams{}, wrap_of, cell_of, slot_of, cell_scan, static_cast<uint32_t>(n_points), sorted, tiles,
         system_of, d_first_point
     );
 
