@@ -398,7 +398,11 @@ void neighbors(
             failure = std::current_exception();
         }
         if (failed) {
-            // the error may be a consequence of the wrong box: find out
+            // the error may be a consequence of the wrong box: fetch the one of this call and find out
+            hipLaunchKernelGGL(
+                fetch_box, dim3(1), dim3(64), 0, nullptr,
+                reinterpret_cast<const double*>(box), periodic, extras.h_small, extras.d_status
+            );
             HIP_CHECK(hipStreamSynchronize(nullptr));
             box_was_right = std::memcmp(extras.h_small, extras.last_box, BOX_BYTES) == 0;
             if (box_was_right) {
@@ -458,8 +462,7 @@ bool compute(
         fetched = true;
         HIP_CHECK(hipStreamSynchronize(stream));
         std::memcpy(used_box, extras.h_small, BOX_BYTES);
-        std::memcpy(extras.last_box, used_box, BOX_BYTES);
-        extras.have_last_box = true;
+        extras.have_last_box = false; // remembered once it proved usable, below
     }
     // valid after any synchronisation of the stream that follows the launch of fetch_box
     auto box_was_right = [&]() { return std::memcmp(extras.h_small, used_box, BOX_BYTES) == 0; };
@@ -471,6 +474,10 @@ bool compute(
         host_periodic[d] = used_box[72 + d] != 0;
     }
     const HostBox hbox = normalise_box(host_box, host_periodic);
+    if (!speculate) {
+        std::memcpy(extras.last_box, used_box, BOX_BYTES);
+        extras.have_last_box = true;
+    }
 
     if (n_points == 0) {
         size_outputs(neighbors, extras, 0, options);
