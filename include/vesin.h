@@ -152,6 +152,31 @@ int VESIN_API vesin_hip_neighbors_batch(
     const char** error_message
 );
 
+/* Gradient of the pair geometry: given dE/d(distances) and dE/d(vectors) of some scalar E for the rows of a list,
+ * ADD dE/d(points) and dE/d(box) to `points_grad` and `box_grad` (the caller zeroes them, or accumulates):
+ *     g_k = vectors_grad[k] + distances_grad[k] * vectors[k] / distances[k]
+ *     points_grad[j_k] += g_k;   points_grad[i_k] -= g_k;   box_grad[a][b] += shifts[k][a] * g_k[b]
+ * This is what the reference's TorchScript class does with tensor operations in its backward step
+ * (vesin-torch/src/vesin_torch.cpp:437-468); here it is one kernel. All arrays are device memory of GPU
+ * `device.device_id`. `distances_grad` or `vectors_grad` may be NULL (taken as zero), `points_grad` or `box_grad`
+ * may be NULL (not wanted); `shifts` is only read for `box_grad`, `distances` and `vectors` only for
+ * `distances_grad`. Sums are accumulated with floating-point atomics: their last bits depend on the order of
+ * arrival. Work is issued on the null stream and the call returns after it completed. */
+int VESIN_API vesin_hip_pairs_backward(
+    const size_t (*pairs)[2],
+    const int32_t (*shifts)[3],
+    const double* distances,
+    const double (*vectors)[3],
+    size_t n_pairs,
+    const double* distances_grad,
+    const double (*vectors_grad)[3],
+    size_t n_points,
+    struct VesinDevice device,
+    double (*points_grad)[3],
+    double (*box_grad)[3],
+    const char** error_message
+);
+
 void VESIN_API vesin_hip_enable_timings(int enabled);
 int VESIN_API vesin_hip_last_timings(const struct VesinNeighborList* neighbors, struct VesinHipTimings* timings);
 

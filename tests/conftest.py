@@ -23,5 +23,7 @@ def _built_libraries():
 
     if not os.path.exists(_build.LIB_PATH):
         _build.build()
+    if not os.path.exists(_build.TORCH_LIB_PATH):
+        _build.build_torch()
     if not os.path.exists(oracle.ORACLE_LIB):
         oracle.build()

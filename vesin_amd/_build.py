@@ -30,6 +30,45 @@ FLAGS = [
 ]
 
 
+TORCH_SOURCE = os.path.join(CSRC, "torch", "neighbor_list_class.cpp")
+TORCH_LIB_PATH = os.path.join(LIB_DIR, "libvesin_torch.so")
+
+
+def build_torch(verbose=False):
+    """Compile the TorchScript class (vesin_amd/lib/libvesin_torch.so) against the installed PyTorch and against
+    libvesin.so, which must have been built before. Host code only: the kernels are all in libvesin.so."""
+    import torch
+    from torch.utils import cpp_extension
+
+    compiler = os.environ.get("CXX", "g++")
+    command = [
+        compiler,
+        "-O2",
+        "-std=c++17",
+        "-fPIC",
+        "-shared",
+        "-fvisibility=hidden",
+        f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+        "-D__HIP_PLATFORM_AMD__",
+        "-DUSE_ROCM",
+        "-DVESIN_SHARED",
+        "-I" + os.path.join(ROOT, "include"),
+        "-I/opt/rocm/include",
+    ]
+    command += ["-I" + path for path in cpp_extension.include_paths()]
+    command += [TORCH_SOURCE, "-o", TORCH_LIB_PATH]
+    # libvesin.so is found next to this library; PyTorch's libraries are in the process before this one is loaded
+    command += ["-L" + LIB_DIR, "-lvesin", "-Wl,-rpath,$ORIGIN"]
+    command += ["-L" + path for path in cpp_extension.library_paths()]
+    command += ["-ltorch", "-ltorch_cpu", "-lc10", "-ltorch_hip", "-lc10_hip"]
+    result = subprocess.run(command, capture_output=True, text=True)
+    if result.returncode != 0:
+        raise RuntimeError(f"{compiler} failed:\n" + result.stdout + result.stderr)
+    if verbose:
+        print(result.stderr)
+    return TORCH_LIB_PATH
+
+
 def build(verbose=False):
     """Compile the library in-tree (vesin_amd/lib/libvesin.so). Always recompiles."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -49,3 +88,4 @@ def build(verbose=False):
 
 if __name__ == "__main__":
     print(build(verbose=True))
+    print(build_torch(verbose=True))

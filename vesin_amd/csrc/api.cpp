@@ -172,6 +172,45 @@ extern "C" int vesin_hip_neighbors_batch(
     return EXIT_SUCCESS;
 }
 
+extern "C" int vesin_hip_pairs_backward(
+    const size_t (*pairs)[2],
+    const int32_t (*shifts)[3],
+    const double* distances,
+    const double (*vectors)[3],
+    size_t n_pairs,
+    const double* distances_grad,
+    const double (*vectors_grad)[3],
+    size_t n_points,
+    VesinDevice device,
+    double (*points_grad)[3],
+    double (*box_grad)[3],
+    const char** error_message
+) {
+    if (error_message == nullptr) {
+        return EXIT_FAILURE;
+    }
+    if (device.type != VesinCUDA) {
+        return fail(error_message, "the gradient is only computed on a GPU device (VesinCUDA, i.e. HIP on ROCm)");
+    }
+    try {
+        vesin_hip::pairs_backward(
+            pairs, shifts, distances, vectors, n_pairs, distances_grad, vectors_grad, n_points, device.device_id,
+            points_grad, box_grad
+        );
+    } catch (const std::bad_alloc&) {
+        LAST_ERROR = "failed to allocate memory";
+        *error_message = LAST_ERROR.c_str();
+        return EXIT_FAILURE;
+    } catch (const std::exception& e) {
+        LAST_ERROR = e.what();
+        *error_message = LAST_ERROR.c_str();
+        return EXIT_FAILURE;
+    } catch (...) {
+        return fail(error_message, "fatal error: unknown type thrown as exception");
+    }
+    return EXIT_SUCCESS;
+}
+
 extern "C" void vesin_free(VesinNeighborList* neighbors) {
     if (neighbors == nullptr) {
         return;

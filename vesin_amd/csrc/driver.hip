@@ -20,6 +20,7 @@
 #include <string>
 #include <vector>
 
+#include "backward.cuh"
 #include "cells.cuh"
 #include "device_common.cuh"
 #include "driver.hpp"
@@ -1166,6 +1167,79 @@ void free_neighbors(VesinNeighborList& neighbors) {
     free_outputs(neighbors);
     delete static_cast<HipExtras*>(neighbors.opaque);
     neighbors.opaque = nullptr;
+}
+
+void pairs_backward(
+    const size_t (*pairs)[2],
+    const int32_t (*shifts)[3],
+    const double* distances,
+    const double (*vectors)[3],
+    size_t n_pairs,
+    const double* distances_grad,
+    const double (*vectors_grad)[3],
+    size_t n_points,
+    int device_id,
+    double (*points_grad)[3],
+    double (*box_grad)[3]
+) {
+    if (n_pairs == 0 || (points_grad == nullptr && box_grad == nullptr)) {
+        return;
+    }
+    if (distances_grad == nullptr && vectors_grad == nullptr) {
+        return;
+    }
+    if (pairs == nullptr) {
+        throw std::runtime_error("`pairs` can not be a NULL pointer");
+    }
+    if (distances_grad != nullptr && (distances == nullptr || vectors == nullptr)) {
+        throw std::runtime_error("the gradient of distances needs both `distances` and `vectors`");
+    }
+    if (box_grad != nullptr && shifts == nullptr) {
+        throw std::runtime_error("the gradient of the box needs `shifts`");
+    }
+    const void* on_device[] = {pairs, shifts, distances, vectors, distances_grad, vectors_grad, points_grad, box_grad};
+    for (const void* pointer : on_device) {
+        if (pointer != nullptr && device_of(pointer) != device_id) {
+            throw std::runtime_error("every array of the gradient must be memory of the device it is computed on");
+        }
+    }
+
+    const DeviceGuard guard(device_id);
+    // one flag per host thread, in pinned memory every device can write to
+    thread_local uint32_t* bad_index = nullptr;
+    if (bad_index == nullptr) {
+        HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&bad_index), sizeof(uint32_t), hipHostMallocPortable));
+    }
+    *bad_index = 0;
+
+    BackwardArgs args;
+    args.pairs = pairs;
+    args.shifts = box_grad != nullptr ? shifts : nullptr;
+    args.distances = distances;
+    args.vectors = vectors;
+    args.distances_grad = distances_grad;
+    args.vectors_grad = vectors_grad;
+    args.n_pairs = n_pairs;
+    args.n_points = n_points;
+    args.points_grad = reinterpret_cast<double*>(points_grad);
+    args.box_grad = reinterpret_cast<double*>(box_grad);
+    args.bad_index = bad_index;
+
+    if (n_points > 0xFFFFFFF0ull) {
+        throw std::runtime_error("too many points: the GPU path indexes points with 32 bits");
+    }
+    const size_t wanted = (n_pairs + BACKWARD_ROWS_PER_BLOCK - 1) / BACKWARD_ROWS_PER_BLOCK;
+    if (wanted > 0x7FFFFFFFull) {
+        throw std::runtime_error("too many pairs for one launch");
+    }
+    const unsigned blocks = static_cast<unsigned>(wanted);
+    hipStream_t stream = nullptr;
+    hipLaunchKernelGGL(pairs_backward_kernel, dim3(blocks), dim3(BACKWARD_THREADS), 0, stream, args);
+    HIP_CHECK(hipGetLastError());
+    HIP_CHECK(hipStreamSynchronize(stream));
+    if (*bad_index != 0) {
+        throw std::runtime_error("`pairs` names a point beyond `n_points`");
+    }
 }
 
 bool last_timings(const VesinNeighborList& neighbors, VesinHipTimings& timings) {

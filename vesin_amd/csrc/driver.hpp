@@ -32,6 +32,23 @@ void neighbors_batch(
     size_t* first_pair
 );
 
+/// Adds the gradient of a scalar with respect to points and box, given its gradient with respect to the distances
+/// and vectors of the rows. All arrays are device memory of GPU `device_id`; `points_grad` ([n_points][3]) and
+/// `box_grad` ([3][3]) are accumulated into. Returns after the work completed.
+void pairs_backward(
+    const size_t (*pairs)[2],
+    const int32_t (*shifts)[3],
+    const double* distances,
+    const double (*vectors)[3],
+    size_t n_pairs,
+    const double* distances_grad,
+    const double (*vectors_grad)[3],
+    size_t n_points,
+    int device_id,
+    double (*points_grad)[3],
+    double (*box_grad)[3]
+);
+
 /// Free the outputs and the private state of a GPU list (does not zero the struct).
 void free_neighbors(VesinNeighborList& neighbors);
 
