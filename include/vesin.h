@@ -123,6 +123,25 @@ struct VesinHipTimings {
     uint64_t candidates;/* reserved, 0 */
 };
 
+/* vesin_neighbors on a stream of the caller's: the work is issued on `stream` (a hipStream_t of GPU
+ * `device.device_id`, passed as void*; NULL is the null stream) and the call returns once that stream has
+ * completed it, so the outputs and `length` are final on return. The kernels are ordered after whatever the
+ * caller queued on `stream` before (no synchronisation is needed to hand over inputs produced there) and other
+ * streams of the device are neither waited for nor held up, as they are by work on the null stream. A list must
+ * not be used by two calls at once. The first call of a list and calls whose rows outgrow its arrays allocate
+ * device memory, which synchronises the device. */
+int VESIN_API vesin_hip_neighbors_on_stream(
+    const double (*points)[3],
+    size_t n_points,
+    const double box[3][3],
+    const bool periodic[3],
+    struct VesinDevice device,
+    struct VesinOptions options,
+    struct VesinNeighborList* neighbors,
+    void* stream,
+    const char** error_message
+);
+
 /* Neighbor lists of many systems that share the options, computed by one sequence of launches (thousands of small
  * systems cost about as much as one large one with as many points, instead of thousands of calls). Per system the
  * rows are exactly those of vesin_neighbors on that system alone; only their order may differ.
@@ -161,7 +180,8 @@ int VESIN_API vesin_hip_neighbors_batch(
  * `device.device_id`. `distances_grad` or `vectors_grad` may be NULL (taken as zero), `points_grad` or `box_grad`
  * may be NULL (not wanted); `shifts` is only read for `box_grad`, `distances` and `vectors` only for
  * `distances_grad`. Sums are accumulated with floating-point atomics: their last bits depend on the order of
- * arrival. Work is issued on the null stream and the call returns after it completed. */
+ * arrival. Work is issued on `stream` (a hipStream_t as void*, NULL for the null stream) and the call returns
+ * after it completed. */
 int VESIN_API vesin_hip_pairs_backward(
     const size_t (*pairs)[2],
     const int32_t (*shifts)[3],
@@ -174,6 +194,7 @@ int VESIN_API vesin_hip_pairs_backward(
     struct VesinDevice device,
     double (*points_grad)[3],
     double (*box_grad)[3],
+    void* stream,
     const char** error_message
 );
 

@@ -249,7 +249,7 @@ def test_backward_with_rows_in_no_order(n_points):
     status = lib.vesin_hip_pairs_backward(
         pairs.data_ptr(), shifts.data_ptr(), distances.data_ptr(), vectors.data_ptr(), n_pairs,
         distances_grad.data_ptr(), vectors_grad.data_ptr(), n_points, VesinDevice(VesinCUDA, 0),
-        points_grad.data_ptr(), box_grad.data_ptr(), ctypes.byref(message),
+        points_grad.data_ptr(), box_grad.data_ptr(), None, ctypes.byref(message),
     )
     assert status == 0, message.value
     expected_points, expected_box = _backward_with_tensor_operations(
@@ -273,7 +273,7 @@ def test_backward_refuses_rows_of_another_system():
     message = ctypes.c_char_p()
     status = lib.vesin_hip_pairs_backward(
         pairs.data_ptr(), None, None, None, 2, None, vectors_grad.data_ptr(), 2, VesinDevice(VesinCUDA, 0),
-        points_grad.data_ptr(), None, ctypes.byref(message),
+        points_grad.data_ptr(), None, None, ctypes.byref(message),
     )
     assert status == 1
     assert message.value == b"`pairs` names a point beyond `n_points`"

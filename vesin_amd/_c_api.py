@@ -115,6 +115,19 @@ def get_library():
             VesinDevice,
             ctypes.c_void_p,
             ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.POINTER(ctypes.c_char_p),
+        ]
+        lib.vesin_hip_neighbors_on_stream.restype = ctypes.c_int
+        lib.vesin_hip_neighbors_on_stream.argtypes = [
+            ctypes.c_void_p,
+            ctypes.c_size_t,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            VesinDevice,
+            VesinOptions,
+            ctypes.POINTER(VesinNeighborList),
+            ctypes.c_void_p,
             ctypes.POINTER(ctypes.c_char_p),
         ]
         lib.vesin_hip_enable_timings.restype = None

@@ -22,7 +22,7 @@ static int fail(const char** error_message, const char* text) {
     return EXIT_FAILURE;
 }
 
-extern "C" int vesin_neighbors(
+static int neighbors_on(
     const double (*points)[3],
     size_t n_points,
     const double box[3][3],
@@ -30,6 +30,7 @@ extern "C" int vesin_neighbors(
     VesinDevice device,
     VesinOptions options,
     VesinNeighborList* neighbors,
+    void* stream,
     const char** error_message
 ) {
     if (error_message == nullptr) {
@@ -76,7 +77,7 @@ extern "C" int vesin_neighbors(
             if (neighbors->device.type == VesinUnknownDevice) {
                 neighbors->device = device;
             }
-            vesin_hip::neighbors(points, n_points, box, periodic, options, *neighbors);
+            vesin_hip::neighbors(points, n_points, box, periodic, options, *neighbors, stream);
         } else if (device.type == VesinCPU) {
             throw std::runtime_error(
                 "this library only implements GPU devices (VesinCUDA, i.e. HIP on ROCm); there is no CPU engine in it"
@@ -96,6 +97,33 @@ extern "C" int vesin_neighbors(
         return fail(error_message, "fatal error: unknown type thrown as exception");
     }
     return EXIT_SUCCESS;
+}
+
+extern "C" int vesin_neighbors(
+    const double (*points)[3],
+    size_t n_points,
+    const double box[3][3],
+    const bool periodic[3],
+    VesinDevice device,
+    VesinOptions options,
+    VesinNeighborList* neighbors,
+    const char** error_message
+) {
+    return neighbors_on(points, n_points, box, periodic, device, options, neighbors, nullptr, error_message);
+}
+
+extern "C" int vesin_hip_neighbors_on_stream(
+    const double (*points)[3],
+    size_t n_points,
+    const double box[3][3],
+    const bool periodic[3],
+    VesinDevice device,
+    VesinOptions options,
+    VesinNeighborList* neighbors,
+    void* stream,
+    const char** error_message
+) {
+    return neighbors_on(points, n_points, box, periodic, device, options, neighbors, stream, error_message);
 }
 
 extern "C" int vesin_hip_neighbors_batch(
@@ -184,6 +212,7 @@ extern "C" int vesin_hip_pairs_backward(
     VesinDevice device,
     double (*points_grad)[3],
     double (*box_grad)[3],
+    void* stream,
     const char** error_message
 ) {
     if (error_message == nullptr) {
@@ -195,7 +224,7 @@ extern "C" int vesin_hip_pairs_backward(
     try {
         vesin_hip::pairs_backward(
             pairs, shifts, distances, vectors, n_pairs, distances_grad, vectors_grad, n_points, device.device_id,
-            points_grad, box_grad
+            points_grad, box_grad, stream
         );
     } catch (const std::bad_alloc&) {
         LAST_ERROR = "failed to allocate memory";

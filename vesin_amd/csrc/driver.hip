@@ -328,7 +328,7 @@ void non_finite_error(const double (*points)[3], unsigned int flat) {
 
 bool compute(
     const double (*points)[3], size_t n_points, const double box[3][3], const bool periodic[3], VesinOptions options,
-    VesinNeighborList& neighbors, HipExtras& extras, bool speculate
+    VesinNeighborList& neighbors, HipExtras& extras, bool speculate, hipStream_t stream
 );
 
 } // namespace
@@ -339,8 +339,11 @@ void neighbors(
     const double box[3][3],
     const bool periodic[3],
     VesinOptions options,
-    VesinNeighborList& neighbors
+    VesinNeighborList& neighbors,
+    void* caller_stream
 ) {
+    // the null stream when the caller names none, like the reference (vesin/src/vesin_cuda.cpp:798)
+    hipStream_t stream = static_cast<hipStream_t>(caller_stream);
     const int device_id = neighbors.device.device_id;
     int device_count = 0;
     if (hipGetDeviceCount(&device_count) != hipSuccess || device_count == 0) {
@@ -393,7 +396,7 @@ void neighbors(
         bool failed = false;
         std::exception_ptr failure;
         try {
-            box_was_right = compute(points, n_points, box, periodic, options, neighbors, extras, true);
+            box_was_right = compute(points, n_points, box, periodic, options, neighbors, extras, true, stream);
         } catch (...) {
             failed = true;
             failure = std::current_exception();
@@ -401,10 +404,10 @@ void neighbors(
         if (failed) {
             // the error may be a consequence of the wrong box: fetch the one of this call and find out
             hipLaunchKernelGGL(
-                fetch_box, dim3(1), dim3(64), 0, nullptr,
+                fetch_box, dim3(1), dim3(64), 0, stream,
                 reinterpret_cast<const double*>(box), periodic, extras.h_small, extras.d_status
             );
-            HIP_CHECK(hipStreamSynchronize(nullptr));
+            HIP_CHECK(hipStreamSynchronize(stream));
             box_was_right = std::memcmp(extras.h_small, extras.last_box, BOX_BYTES) == 0;
             if (box_was_right) {
                 std::rethrow_exception(failure);
@@ -415,7 +418,7 @@ void neighbors(
         }
         extras.box_rest = BOX_REST;
     }
-    (void)compute(points, n_points, box, periodic, options, neighbors, extras, false);
+    (void)compute(points, n_points, box, periodic, options, neighbors, extras, false, stream);
 }
 
 namespace {
@@ -428,10 +431,10 @@ bool compute(
     VesinOptions options,
     VesinNeighborList& neighbors,
     HipExtras& extras,
-    bool speculate
+    bool speculate,
+    hipStream_t stream
 ) {
     const size_t pair_limit = pairs_per_point_limit();
-    hipStream_t stream = nullptr; // the null stream, like the reference (vesin/src/vesin_cuda.cpp:798)
 
     const bool timed = TIMINGS_ENABLED.load();
     if (timed && !extras.have_events) {
@@ -1180,7 +1183,8 @@ void pairs_backward(
     size_t n_points,
     int device_id,
     double (*points_grad)[3],
-    double (*box_grad)[3]
+    double (*box_grad)[3],
+    void* caller_stream
 ) {
     if (n_pairs == 0 || (points_grad == nullptr && box_grad == nullptr)) {
         return;
@@ -1233,7 +1237,7 @@ void pairs_backward(
         throw std::runtime_error("too many pairs for one launch");
     }
     const unsigned blocks = static_cast<unsigned>(wanted);
-    hipStream_t stream = nullptr;
+    hipStream_t stream = static_cast<hipStream_t>(caller_stream);
     hipLaunchKernelGGL(pairs_backward_kernel, dim3(blocks), dim3(BACKWARD_THREADS), 0, stream, args);
     HIP_CHECK(hipGetLastError());
     HIP_CHECK(hipStreamSynchronize(stream));

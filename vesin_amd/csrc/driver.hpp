@@ -6,7 +6,8 @@
 
 namespace vesin_hip {
 
-/// Compute the list on GPU `neighbors.device.device_id`. All three input pointers are device memory.
+/// Compute the list on GPU `neighbors.device.device_id`. All three input pointers are device memory. The work is
+/// issued on `stream` (a hipStream_t of that device; nullptr is the null stream) and has completed on return.
 /// Throws std::runtime_error / std::bad_alloc; never leaves HIP work in flight.
 void neighbors(
     const double (*points)[3],
@@ -14,7 +15,8 @@ void neighbors(
     const double box[3][3],
     const bool periodic[3],
     VesinOptions options,
-    VesinNeighborList& neighbors
+    VesinNeighborList& neighbors,
+    void* stream
 );
 
 /// The lists of many (fully periodic) systems in one sequence of launches. `points`, `boxes`, `periodic` are device
@@ -34,7 +36,8 @@ void neighbors_batch(
 
 /// Adds the gradient of a scalar with respect to points and box, given its gradient with respect to the distances
 /// and vectors of the rows. All arrays are device memory of GPU `device_id`; `points_grad` ([n_points][3]) and
-/// `box_grad` ([3][3]) are accumulated into. Returns after the work completed.
+/// `box_grad` ([3][3]) are accumulated into. Runs on `stream` (nullptr: the null stream) and returns after the work
+/// completed.
 void pairs_backward(
     const size_t (*pairs)[2],
     const int32_t (*shifts)[3],
@@ -46,7 +49,8 @@ void pairs_backward(
     size_t n_points,
     int device_id,
     double (*points_grad)[3],
-    double (*box_grad)[3]
+    double (*box_grad)[3],
+    void* stream
 );
 
 /// Free the outputs and the private state of a GPU list (does not zero the struct).

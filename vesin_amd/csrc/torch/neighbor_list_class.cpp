@@ -5,8 +5,8 @@
 // exported model that holds the reference's class loads this one instead. Differences, all on the device side:
 //   - pairs are handed out as int64 views of the size_t arrays the kernels wrote (every index is below 2^63, so
 //     the bits are the same): no conversion pass over 16 bytes per pair (the reference converts, :225-226);
-//   - a caller on a non-default stream is waited for before the library (which works on the null stream) reads
-//     its tensors.
+//   - the kernels run on the caller's current stream (vesin_hip_neighbors_on_stream), ordered after whatever
+//     produced the inputs there, instead of on the null stream.
 // The gradient of distances and vectors with respect to points and box (reference :403-479) is one HIP kernel
 // of the library (vesin_hip_pairs_backward) instead of a chain of tensor operations.
 
@@ -98,7 +98,6 @@ public:
             }
             if (n_pairs > 0 && (distances_grad.defined() || vectors_grad.defined())) {
                 TORCH_CHECK(vectors.is_cuda(), "the gradient of a neighbor list is computed on the GPU only");
-                wait_for_caller(vectors.device());
                 const char* error_message = nullptr;
                 const auto status = vesin_hip_pairs_backward(
                     reinterpret_cast<const size_t (*)[2]>(pairs.data_ptr<int64_t>()),
@@ -112,6 +111,7 @@ public:
                     VesinDevice{VesinCUDA, static_cast<int>(vectors.device().index())},
                     want_points ? reinterpret_cast<double (*)[3]>(points_grad.data_ptr<double>()) : nullptr,
                     want_box ? reinterpret_cast<double (*)[3]>(box_grad.data_ptr<double>()) : nullptr,
+                    current_stream(vectors.device()),
                     &error_message
                 );
                 if (status != EXIT_SUCCESS) {
@@ -122,12 +122,9 @@ public:
         return {points_grad, box_grad, torch::Tensor(), torch::Tensor(), torch::Tensor(), torch::Tensor(), torch::Tensor()};
     }
 
-    /// The library works on the null stream: work the caller queued on another stream has to be done first.
-    static void wait_for_caller(const torch::Device& device) {
-        auto stream = c10::hip::getCurrentHIPStream(device.index());
-        if (stream != c10::hip::getDefaultHIPStream(device.index())) {
-            stream.synchronize();
-        }
+    /// The stream PyTorch queues the caller's work on: the library's kernels go there too.
+    static void* current_stream(const torch::Device& device) {
+        return static_cast<void*>(c10::hip::getCurrentHIPStream(device.index()).stream());
     }
 };
 
@@ -235,12 +232,8 @@ public:
 
         auto points_data = points.detach().contiguous();
         auto box_data = box.detach().contiguous();
-        if (points.is_cuda()) {
-            PairGeometry::wait_for_caller(points.device());
-        }
-
         const char* error_message = nullptr;
-        const auto status = vesin_neighbors(
+        const auto status = vesin_hip_neighbors_on_stream(
             reinterpret_cast<const double (*)[3]>(points_data.data_ptr<double>()),
             static_cast<size_t>(points_data.size(0)),
             reinterpret_cast<const double (*)[3]>(box_data.data_ptr<double>()),
@@ -248,6 +241,7 @@ public:
             device,
             options,
             &list_,
+            points.is_cuda() ? PairGeometry::current_stream(points.device()) : nullptr,
             &error_message
         );
         if (status != EXIT_SUCCESS) {
