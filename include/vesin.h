@@ -47,7 +47,7 @@ struct VesinOptions {
     bool return_shifts;        /* fill VesinNeighborList::shifts */
     bool return_distances;     /* fill VesinNeighborList::distances */
     bool return_vectors;       /* fill VesinNeighborList::vectors */
-    double skin;               /* Verlet skin; only 0 is supported by this library */
+    double skin;               /* Verlet skin: > 0 keeps candidates at cutoff + skin between calls */
 };
 
 enum VesinDeviceKind {

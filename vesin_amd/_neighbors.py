@@ -69,7 +69,8 @@ class NeighborList:
         :param full_list: return each pair twice (``i-j`` and ``j-i``) or only once
         :param sorted: order the pairs by ``i`` (this implementation orders by ``(i, j, shift)``)
         :param algorithm: ``"auto"``, ``"brute_force"`` or ``"cell_list"``
-        :param skin: Verlet skin; only ``0`` is supported
+        :param skin: Verlet skin: with a positive value, candidates computed at ``cutoff + skin`` are kept and
+            filtered at the cutoff while no point moved further than half of it; the result is that of ``skin=0``
         :param n_threads: accepted for compatibility (must be ``>= 0``); the GPU path does not use it
         :param device: GPU used for inputs that are not already torch GPU tensors
         """

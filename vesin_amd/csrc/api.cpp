@@ -52,8 +52,8 @@ static int neighbors_on(
         return fail(error_message, "cutoff is too small");
     }
     if (!std::isfinite(options.skin) || options.skin < 0.0) {
-        // the reference sets this message without returning (vesin/src/vesin.cpp:80-82); a caching skin is not
-        // available here at all, so this is an error
+        // the reference sets this message without returning (vesin/src/vesin.cpp:80-82) and goes on with the
+        // unusable value; here it is an error
         return fail(error_message, "skin must be a finite, non-negative number");
     }
     if (options.n_threads < 0) {
@@ -68,9 +68,6 @@ static int neighbors_on(
 
     try {
         if (device.type == VesinCUDA) {
-            if (options.skin > 0.0) {
-                throw std::runtime_error("a non-zero `skin` (Verlet caching) is not supported by the HIP path");
-            }
             if (periodic == nullptr) {
                 throw std::runtime_error("`periodic` can not be a NULL pointer");
             }
@@ -180,7 +177,7 @@ extern "C" int vesin_hip_neighbors_batch(
 
     try {
         if (options.skin > 0.0) {
-            throw std::runtime_error("a non-zero `skin` (Verlet caching) is not supported by the HIP path");
+            throw std::runtime_error("a non-zero `skin` (Verlet caching) is not available for a batch of systems");
         }
         if (neighbors->device.type == VesinUnknownDevice) {
             neighbors->device = device;

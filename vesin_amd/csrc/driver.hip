@@ -17,6 +17,7 @@
 #include <atomic>
 #include <exception>
 #include <stdexcept>
+#include <memory>
 #include <string>
 #include <vector>
 
@@ -29,6 +30,7 @@
 #include "scan.cuh"
 #include "search.cuh"
 #include "sort.cuh"
+#include "verlet.cuh"
 
 namespace vesin_hip {
 
@@ -125,11 +127,57 @@ struct Carver {
     }
 };
 
+/// Candidates beyond which a cached list is not worth filtering: the direct search writes its rows at more than
+/// half the memory bandwidth, and a filter has to read every candidate on top of writing the same rows. Measured
+/// on jittered diamond (cutoff 5, skin 0.5): the filter takes 0.038 ms against 0.077 ms at 0.2 M candidates,
+/// breaks even near 1.6 M and takes twice the direct search's time at 15 M.
+constexpr size_t VERLET_MAX_CANDIDATES = size_t(1) << 20;
+
 constexpr int SINGLE_PASS_REST = 64;
 constexpr int BOX_REST = 32;
 constexpr size_t BOX_BYTES = 75; // 9 doubles and 3 flags, as fetch_box lays them out
 
 enum Stage { T_START = 0, T_CELLS, T_COUNT, T_SCAN, T_WRITE_BEGIN, T_WRITE, T_SORT, T_STAGES };
+
+/// Candidate list of a Verlet-cached calculation (options.skin > 0) and what it was built from; the counterpart
+/// of the reference's VerletList / VerletCache (vesin/src/verlet.hpp:19-95, vesin/src/verlet_cuda.hpp).
+struct VerletCache {
+    VesinNeighborList candidates = VesinNeighborList(); // full lists of this library, with a private state of its own
+    double* ref_points = nullptr;                       // device: the points the candidates were built from
+    size_t ref_capacity = 0;
+    size_t n_ref = 0;
+    VerletReference* reference = nullptr; // device: box and periodicity of that call
+    VerletWork* work = nullptr;           // device
+    VerletStatus* status = nullptr;       // pinned
+    VesinOptions options = {};
+    bool valid = false;
+    /// Lists too long for a filter to pay are searched directly on every call (see verlet_neighbors); the
+    /// estimate is revised with every call's row count.
+    bool direct = false;
+    size_t direct_n_points = 0;
+
+    VerletCache() = default;
+    VerletCache(const VerletCache&) = delete;
+    VerletCache& operator=(const VerletCache&) = delete;
+
+    ~VerletCache() {
+        if (candidates.device.type == VesinCUDA) {
+            free_neighbors(candidates);
+        }
+        if (ref_points != nullptr) {
+            (void)hipFree(ref_points);
+        }
+        if (reference != nullptr) {
+            (void)hipFree(reference);
+        }
+        if (work != nullptr) {
+            (void)hipFree(work);
+        }
+        if (status != nullptr) {
+            (void)hipHostFree(status);
+        }
+    }
+};
 
 /// Private state of one VesinNeighborList (VesinNeighborList::opaque).
 struct HipExtras {
@@ -151,8 +199,10 @@ struct HipExtras {
     bool have_events = false;
     bool timings_valid = false;
     VesinHipTimings timings = {};
+    VerletCache* verlet = nullptr;    // only while the caller asks for a skin
 
     ~HipExtras() {
+        delete verlet;
         work.release();
         sort_work.release();
         if (d_status != nullptr) {
@@ -283,6 +333,32 @@ void size_outputs(VesinNeighborList& neighbors, HipExtras& extras, size_t rows, 
     }
 }
 
+/// Scratch rows for `rows` unsorted rows (shifts always present: they are part of the sort key) and the workspace
+/// of the radix sort, from the list's sort arena; the sort's final gather fills the caller's arrays.
+void carve_sort_space(
+    HipExtras& extras, size_t rows, const VesinOptions& options, SearchOutputs& unsorted, SortWorkspace& space
+) {
+    const size_t table_entries = static_cast<size_t>(RADIX) * sort_blocks(rows);
+    auto carve = [&](Carver& c) {
+        unsorted.pairs = c.take<unsigned long long>(2 * rows);
+        unsorted.shifts = c.take<int32_t>(3 * rows);
+        unsorted.distances = options.return_distances ? c.take<double>(rows) : nullptr;
+        unsorted.vectors = options.return_vectors ? c.take<double>(3 * rows) : nullptr;
+        for (int b = 0; b < 2; b++) {
+            space.keys[b] = c.take<uint64_t>(rows);
+            space.rows[b] = c.take<uint32_t>(rows);
+        }
+        space.table = c.take<uint32_t>(table_entries);
+        space.table_scan = c.take<uint64_t>(table_entries + 1);
+        space.scan_scratch = c.take<uint64_t>(scan_scratch_elements(table_entries));
+    };
+    Carver measure(nullptr);
+    carve(measure);
+    extras.sort_work.reserve(measure.used);
+    Carver carver(extras.sort_work.ptr);
+    carve(carver);
+}
+
 /// Optional user-imposed limit on pairs per point, kept for callers that rely on the reference's environment
 /// variable and its messages (vesin/src/vesin_cuda.cpp:871-884, :911-918). 0 = no limit.
 size_t pairs_per_point_limit() {
@@ -329,6 +405,16 @@ void non_finite_error(const double (*points)[3], unsigned int flat) {
 bool compute(
     const double (*points)[3], size_t n_points, const double box[3][3], const bool periodic[3], VesinOptions options,
     VesinNeighborList& neighbors, HipExtras& extras, bool speculate, hipStream_t stream
+);
+
+void verlet_neighbors(
+    const double (*points)[3], size_t n_points, const double box[3][3], const bool periodic[3], VesinOptions options,
+    VesinNeighborList& neighbors, HipExtras& extras, hipStream_t stream
+);
+
+void direct_neighbors(
+    const double (*points)[3], size_t n_points, const double box[3][3], const bool periodic[3], VesinOptions options,
+    VesinNeighborList& neighbors, HipExtras& extras, hipStream_t stream
 );
 
 } // namespace
@@ -384,6 +470,25 @@ void neighbors(
     HipExtras& extras = extras_of(neighbors);
     extras.timings_valid = false;
 
+    if (options.skin > 0.0) {
+        verlet_neighbors(points, n_points, box, periodic, options, neighbors, extras, stream);
+        return;
+    }
+    if (extras.verlet != nullptr) {
+        // no skin any more: the cache goes, like in the reference (vesin/src/cpu_cell_list.cpp:235-238)
+        delete extras.verlet;
+        extras.verlet = nullptr;
+    }
+    direct_neighbors(points, n_points, box, periodic, options, neighbors, extras, stream);
+}
+
+namespace {
+
+/// The search itself (no caching), on a list whose inputs were checked.
+void direct_neighbors(
+    const double (*points)[3], size_t n_points, const double box[3][3], const bool periodic[3], VesinOptions options,
+    VesinNeighborList& neighbors, HipExtras& extras, hipStream_t stream
+) {
     // The grid is picked on the host from the box, which lives on the device: reading it costs a round trip before
     // anything else can be launched. A box that did not change over the last calls is assumed not to have changed
     // now either: the call runs with the remembered one and checks the assumption at its last synchronisation.
@@ -420,8 +525,6 @@ void neighbors(
     }
     (void)compute(points, n_points, box, periodic, options, neighbors, extras, false, stream);
 }
-
-namespace {
 
 bool compute(
     const double (*points)[3],
@@ -816,27 +919,7 @@ bool compute(
     SortWorkspace sort_space = {};
     sort_space.host_ranges = extras.h_shift_ranges;
     if (sorting) {
-        // the write pass goes to scratch rows (shifts always present: they are part of the sort key); the sort's
-        // final gather fills the caller's arrays
-        const size_t table_entries = static_cast<size_t>(RADIX) * sort_blocks(total);
-        auto carve_sort = [&](Carver& c) {
-            unsorted.pairs = c.take<unsigned long long>(2 * total);
-            unsorted.shifts = c.take<int32_t>(3 * total);
-            unsorted.distances = options.return_distances ? c.take<double>(total) : nullptr;
-            unsorted.vectors = options.return_vectors ? c.take<double>(3 * total) : nullptr;
-            for (int b = 0; b < 2; b++) {
-                sort_space.keys[b] = c.take<uint64_t>(total);
-                sort_space.rows[b] = c.take<uint32_t>(total);
-            }
-            sort_space.table = c.take<uint32_t>(table_entries);
-            sort_space.table_scan = c.take<uint64_t>(table_entries + 1);
-            sort_space.scan_scratch = c.take<uint64_t>(scan_scratch_elements(table_entries));
-        };
-        Carver measure_sort(nullptr);
-        carve_sort(measure_sort);
-        extras.sort_work.reserve(measure_sort.used);
-        Carver sort_carver(extras.sort_work.ptr);
-        carve_sort(sort_carver);
+        carve_sort_space(extras, total, options, unsorted, sort_space);
     }
 
     if (!speculative || !fits) {
@@ -877,6 +960,201 @@ bool compute(
 
 
 namespace {
+
+/// options.skin > 0: filter the cached candidates, after rebuilding them when they no longer cover the points
+/// (reference: vesin/src/cpu_cell_list.cpp:222-234, vesin/src/verlet.cpp). In the steady state a call is three
+/// launches (check, filter, publish) and one synchronisation; the filter writes straight into the arrays the list
+/// kept, and is repeated when they turn out too small or when the check asks for new candidates.
+void verlet_neighbors(
+    const double (*points)[3], size_t n_points, const double box[3][3], const bool periodic[3], VesinOptions options,
+    VesinNeighborList& neighbors, HipExtras& extras, hipStream_t stream
+) {
+    if (extras.verlet == nullptr) {
+        auto cache = std::make_unique<VerletCache>();
+        HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&cache->reference), sizeof(VerletReference)));
+        HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&cache->work), sizeof(VerletWork)));
+        HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&cache->status), sizeof(VerletStatus), hipHostMallocDefault));
+        extras.verlet = cache.release();
+    }
+    VerletCache& cache = *extras.verlet;
+    const size_t pair_limit = pairs_per_point_limit();
+
+    // same triggers as the reference (vesin/src/verlet.cpp:48-54, :65-71)
+    const bool options_changed = cache.options.cutoff != options.cutoff || cache.options.skin != options.skin ||
+                                 cache.options.full != options.full;
+    bool fresh = false;
+    auto rebuild = [&]() {
+        cache.valid = false;
+        VesinOptions build = {};
+        build.cutoff = options.cutoff + options.skin;
+        build.full = options.full;
+        build.sorted = false;
+        build.algorithm = VesinCellList;
+        build.n_threads = options.n_threads;
+        build.return_shifts = true;
+        build.return_distances = false;
+        build.return_vectors = false;
+        build.skin = 0.0;
+        cache.candidates.device = neighbors.device;
+        vesin_hip::neighbors(points, n_points, box, periodic, build, cache.candidates, stream);
+
+        if (cache.ref_capacity < n_points) {
+            if (cache.ref_points != nullptr) {
+                (void)hipFree(cache.ref_points);
+                cache.ref_points = nullptr;
+                cache.ref_capacity = 0;
+            }
+            const size_t capacity = n_points + n_points / 8 + 64;
+            HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&cache.ref_points), capacity * 3 * sizeof(double)));
+            cache.ref_capacity = capacity;
+        }
+        if (n_points > 0) {
+            HIP_CHECK(hipMemcpyAsync(
+                cache.ref_points, points, n_points * 3 * sizeof(double), hipMemcpyDeviceToDevice, stream
+            ));
+        }
+        hipLaunchKernelGGL(
+            verlet_store_reference, dim3(1), dim3(64), 0, stream, reinterpret_cast<const double*>(box), periodic,
+            cache.reference
+        );
+        cache.options = options;
+        cache.n_ref = n_points;
+        cache.valid = true;
+        fresh = true;
+    };
+    // VESIN_HIP_VERLET=cache / direct takes the choice between filtering and searching away from the estimate
+    const char* forced = std::getenv("VESIN_HIP_VERLET");
+    const bool force_cache = forced != nullptr && std::strcmp(forced, "cache") == 0;
+    const bool force_direct = forced != nullptr && std::strcmp(forced, "direct") == 0;
+    auto too_long_for_a_filter = [&](size_t rows) {
+        const double ratio = (options.cutoff + options.skin) / options.cutoff;
+        const double candidates = static_cast<double>(rows) * ratio * ratio * ratio;
+        return force_direct || (!force_cache && candidates > static_cast<double>(VERLET_MAX_CANDIDATES));
+    };
+    if (options_changed || cache.direct_n_points != n_points) {
+        cache.direct = false;
+    }
+    if (!cache.valid || options_changed || cache.n_ref != n_points || cache.direct) {
+        // Without usable candidates this call is a direct search, whose rows are the answer. Its row count says
+        // how many candidates there would be: few enough, and they are computed now for the next calls to filter.
+        VesinOptions plain = options;
+        plain.skin = 0.0;
+        direct_neighbors(points, n_points, box, periodic, plain, neighbors, extras, stream);
+        cache.direct = too_long_for_a_filter(neighbors.length);
+        cache.direct_n_points = n_points;
+        if (cache.direct) {
+            if (cache.valid) {
+                // the candidates of a smaller past are of no use any more
+                free_neighbors(cache.candidates);
+                cache.candidates = VesinNeighborList();
+                cache.valid = false;
+            }
+        } else {
+            rebuild();
+        }
+        return;
+    }
+
+    SortWorkspace sort_space = {};
+    sort_space.host_ranges = extras.h_shift_ranges;
+    size_t total = 0;
+    bool through_scratch = options.sorted;
+    for (int attempt = 0;; attempt++) {
+        if (attempt > 4) {
+            throw std::runtime_error("internal error: the Verlet filter did not settle");
+        }
+        const size_t n_candidates = cache.candidates.length;
+        SearchOutputs out;
+        size_t capacity = 0;
+        if (through_scratch) {
+            // the rows are sorted afterwards: they go to scratch rows, of which there are at most as many as
+            // candidates
+            carve_sort_space(extras, std::max<size_t>(n_candidates, 1), options, out, sort_space);
+            capacity = n_candidates;
+        } else {
+            size_outputs(neighbors, extras, 0, options);
+            out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
+            out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
+            out.distances = neighbors.distances;
+            out.vectors = reinterpret_cast<double*>(neighbors.vectors);
+            capacity = extras.capacity;
+        }
+
+        cache.status->rebuild = 0;
+        cache.status->total_rows = 0;
+        const unsigned check_blocks = static_cast<unsigned>(std::max<size_t>((n_points + VERLET_BLOCK - 1) / VERLET_BLOCK, 1));
+        hipLaunchKernelGGL(
+            verlet_check_kernel, dim3(check_blocks), dim3(VERLET_BLOCK), 0, stream,
+            reinterpret_cast<const double*>(points), cache.ref_points, n_points, reinterpret_cast<const double*>(box),
+            periodic, cache.reference, options.skin, cache.status, cache.work
+        );
+        if (n_candidates > 0) {
+            VerletFilterArgs fargs;
+            fargs.candidate_pairs = reinterpret_cast<const unsigned long long*>(cache.candidates.pairs);
+            fargs.candidate_shifts = reinterpret_cast<const int32_t*>(cache.candidates.shifts);
+            fargs.n_candidates = n_candidates;
+            fargs.points = reinterpret_cast<const double*>(points);
+            fargs.work = cache.work;
+            fargs.cutoff_sq = options.cutoff * options.cutoff;
+            fargs.out = out;
+            fargs.capacity = capacity;
+            const size_t chunks = (n_candidates + VERLET_CHUNK - 1) / VERLET_CHUNK;
+            const size_t wanted = (chunks + VERLET_WAVES - 1) / VERLET_WAVES;
+            const unsigned blocks = static_cast<unsigned>(std::min<size_t>(wanted, 256 * 64));
+            hipLaunchKernelGGL(verlet_filter_kernel, dim3(blocks), dim3(VERLET_BLOCK), 0, stream, fargs);
+        }
+        hipLaunchKernelGGL(verlet_publish, dim3(1), dim3(1), 0, stream, cache.work, cache.status);
+        HIP_CHECK(hipStreamSynchronize(stream));
+        HIP_CHECK(hipGetLastError());
+
+        if (cache.status->rebuild != 0) {
+            if (fresh) {
+                throw std::runtime_error("internal error: fresh Verlet candidates do not cover their own points");
+            }
+            rebuild();
+            continue;
+        }
+        total = cache.status->total_rows;
+        if (pair_limit != 0 && total > n_points * pair_limit) {
+            throw std::runtime_error(
+                "The number of neighbor pairs exceeds the maximum capacity of " + std::to_string(n_points * pair_limit) +
+                " (max_pairs_per_point=" + std::to_string(pair_limit) + "; n_points=" + std::to_string(n_points) + "). " +
+                "Consider reducing the cutoff distance, or explicitly setting " +
+                "VESIN_CUDA_MAX_PAIRS_PER_POINT as an environment variable."
+            );
+        }
+        if (through_scratch) {
+            size_outputs(neighbors, extras, total, options);
+            if (total <= 1) {
+                // nothing to sort: the one row is produced again, in place
+                if (total == 0) {
+                    break;
+                }
+                through_scratch = false;
+                continue;
+            }
+            SearchOutputs final_out;
+            final_out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
+            final_out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
+            final_out.distances = neighbors.distances;
+            final_out.vectors = reinterpret_cast<double*>(neighbors.vectors);
+            sort_pairs(out, final_out, total, n_points, sort_space, stream);
+            HIP_CHECK(hipStreamSynchronize(stream));
+            HIP_CHECK(hipGetLastError());
+            break;
+        }
+        if (total > extras.capacity) {
+            size_outputs(neighbors, extras, total, options);
+            continue;
+        }
+        break;
+    }
+    neighbors.length = total;
+    if (too_long_for_a_filter(total)) {
+        cache.direct = true;
+        cache.direct_n_points = n_points;
+    }
+}
 
 /// first_pair[s] = first output row of system s (offsets are kept per tile-major work item), first_pair[n] = total.
 __global__ void system_rows_kernel(
