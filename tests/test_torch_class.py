@@ -199,7 +199,7 @@ def _backward_with_tensor_operations(pairs, shifts, distances, vectors, distance
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("sorted_rows", [True, False])
-@pytest.mark.parametrize("n_cells", [2, 12])
+@pytest.mark.parametrize("n_cells", [2, 12, 30])
 def test_backward_kernel_equals_tensor_operations(sorted_rows, n_cells):
     """An energy that uses both distances and vectors, on a jittered diamond crystal: forces and box gradient
     from the kernel against the reference's formulas evaluated with tensor operations. Sums of about a hundred
