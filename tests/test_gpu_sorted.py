@@ -1,0 +1,117 @@
+"""sorted=True: the search that produces the rows in order, the cases it leaves to the radix sort, and the radix
+sort itself (VESIN_HIP_SORT=radix) give the same list, in the order (i, j, S) of the canonicalised oracle."""
+
+import numpy as np
+import pytest
+
+import oracle
+from vesin_amd import NeighborList, configs
+
+pytestmark = pytest.mark.gpu
+
+
+def _sorted_list(points, box, periodic, cutoff, full, quantities="PSdD"):
+    import torch
+
+    calculator = NeighborList(cutoff=cutoff, full_list=full, sorted=True)
+    outputs = calculator.compute(
+        torch.tensor(np.ascontiguousarray(points), device="cuda:0"),
+        torch.tensor(np.ascontiguousarray(box), device="cuda:0"),
+        periodic,
+        quantities,
+    )
+    names = {"P": "pairs", "S": "shifts", "d": "distances", "D": "vectors"}
+    return {names[q]: out.cpu().numpy() for q, out in zip(quantities, outputs)}
+
+
+def _check(points, box, periodic, cutoff, full, capfd, monkeypatch, expect):
+    """`expect`: "used" / "left to the radix sort" for what the in-order search must report, None when it must
+    not even be tried."""
+    flags = [bool(periodic)] * 3 if isinstance(periodic, (bool, np.bool_)) else [bool(p) for p in periodic]
+    expected = oracle.canonicalize(oracle.neighbors(points, box, flags, cutoff, full, False, "ijSdD"))
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    for mode in ("default", "radix"):
+        if mode == "radix":
+            monkeypatch.setenv("VESIN_HIP_SORT", "radix")
+        else:
+            monkeypatch.delenv("VESIN_HIP_SORT", raising=False)
+        capfd.readouterr()
+        result = _sorted_list(points, box, periodic, cutoff, full)
+        err = capfd.readouterr().err
+        lines = [line for line in err.splitlines() if line.startswith("in-order search:")]
+        if mode == "radix" or expect is None:
+            assert not lines, err
+        else:
+            assert lines and all(line.endswith(expect) for line in lines), err
+        assert result["pairs"].shape == expected["pairs"].shape, mode
+        for key in result:
+            assert np.array_equal(result[key], expected[key]), (mode, key)
+
+
+@pytest.mark.parametrize("full", [True, False])
+@pytest.mark.parametrize(
+    "replicas,expect",
+    [
+        # one conventional cell with cutoff 5 needs two images per direction: 125 cells, more than that search holds
+        (1, None),
+        (3, "used"),
+        # 4 cells of 6.2 A per direction: 43 atoms per cell, 1175 candidates per tile
+        (7, "left to the radix sort"),
+        (8, "used"),
+    ],
+)
+def test_crystal(full, replicas, expect, capfd, monkeypatch):
+    points, box, periodic = configs.diamond(replicas, seed=replicas)
+    _check(points, box, True, 5.0, full, capfd, monkeypatch, expect)
+
+
+@pytest.mark.parametrize("full", [True, False])
+def test_small_box_with_self_images(full, capfd, monkeypatch):
+    """Box barely wider than the cutoff: a single cell whose stencil is the 27 images; every point pairs with its
+    own images, which the half list keeps under the reference's rule."""
+    rng = np.random.default_rng(17)
+    box = np.array([[3.2, 0.0, 0.0], [0.4, 3.1, 0.0], [-0.3, 0.2, 3.3]])
+    points = rng.random((7, 3)) @ box
+    _check(points, box, True, 3.0, full, capfd, monkeypatch, "used")
+
+
+@pytest.mark.parametrize("periodic", [(True, True, False), (False, False, False), (True, False, True)])
+@pytest.mark.parametrize("full", [True, False])
+def test_mixed_periodicity_and_points_outside_of_the_box(periodic, full, capfd, monkeypatch):
+    rng = np.random.default_rng(23)
+    box = np.diag([11.0, 12.0, 13.0])
+    points = rng.uniform(-6.0, 18.0, size=(900, 3))  # many are wrapped by a box vector or two
+    _check(points, box, periodic, 3.0, full, capfd, monkeypatch, "used")
+
+
+def test_rows_of_one_point_beyond_the_ranking(capfd, monkeypatch):
+    """400 points within a ball of radius 1.2: every point has 399 rows, more than are ranked in one go."""
+    rng = np.random.default_rng(29)
+    directions = rng.normal(size=(400, 3))
+    points = 1.2 * directions / np.linalg.norm(directions, axis=1)[:, None] * rng.random((400, 1)) ** (1 / 3) + 10.0
+    _check(points, np.diag([20.0, 20.0, 20.0]), True, 3.0, True, capfd, monkeypatch, "left to the radix sort")
+
+
+def test_candidates_of_one_tile_beyond_the_registers(capfd, monkeypatch):
+    """A dense liquid: 148 points per cell, 4000 candidates around every tile."""
+    rng = np.random.default_rng(31)
+    points = rng.random((4000, 3)) * np.array([9.0, 9.0, 9.0])
+    _check(points, np.diag([9.0, 9.0, 9.0]), True, 3.0, False, capfd, monkeypatch, "left to the radix sort")
+
+
+def test_points_many_boxes_away(capfd, monkeypatch):
+    """Wraps of several hundred box vectors do not fit the packed shifts of that search."""
+    rng = np.random.default_rng(37)
+    box = np.diag([4.0, 4.0, 4.0])
+    points = rng.random((60, 3)) * 4.0
+    points[::2] += np.array([1600.0, -1200.0, 0.0])
+    _check(points, box, True, 2.0, True, capfd, monkeypatch, "left to the radix sort")
+
+
+@pytest.mark.parametrize("n_points", [1, 2, 5, 33, 70])
+def test_few_points(n_points, capfd, monkeypatch):
+    rng = np.random.default_rng(n_points)
+    box = np.diag([6.0, 7.0, 8.0])
+    points = rng.random((n_points, 3)) @ box
+    _check(points, box, True, 2.9, True, capfd, monkeypatch, "used")
+    _check(points, box, False, 2.9, False, capfd, monkeypatch, "used")

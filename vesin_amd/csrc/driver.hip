@@ -27,6 +27,7 @@
 #include "driver.hpp"
 #include "fused.cuh"
 #include "geometry.hpp"
+#include "ordered.cuh"
 #include "scan.cuh"
 #include "search.cuh"
 #include "sort.cuh"
@@ -61,7 +62,32 @@ static bool two_pass_only() {
     return text != nullptr && std::strcmp(text, "two-pass") == 0;
 }
 
+/// VESIN_HIP_SORT=radix keeps sorted lists on the unsorted search followed by the radix sort (for comparisons and
+/// tests) instead of the search that produces them in order.
+static bool radix_sort_only() {
+    const char* text = std::getenv("VESIN_HIP_SORT");
+    return text != nullptr && std::strcmp(text, "radix") == 0;
+}
+
 namespace {
+
+/// What the counting pass of the in-order search reports (pinned host memory).
+struct OrderedHostStatus {
+    OrderedStatus found;
+    unsigned long long total_rows;
+    unsigned int first_bad_coordinate;
+    unsigned int padding;
+};
+
+__global__ void publish_ordered_status(
+    const OrderedStatus* found, const uint64_t* total, const DeviceStatus* status, OrderedHostStatus* host
+) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        host->found = *found;
+        host->total_rows = *total;
+        host->first_bad_coordinate = status->first_bad_coordinate;
+    }
+}
 
 /// Makes `device` current for a scope and gives the caller's device back afterwards.
 struct DeviceGuard {
@@ -190,6 +216,7 @@ struct HipExtras {
     BlockBounds* h_bounds = nullptr;  // pinned: one slot per workgroup of the bounding pass
     FusedStatus* h_fused = nullptr;   // pinned
     ShiftRange* h_shift_ranges = nullptr; // pinned: one slot per workgroup of the sort's range pass
+    OrderedHostStatus* h_ordered = nullptr; // pinned
     size_t capacity = 0;              // rows every allocated output array can hold
     unsigned char last_box[BOX_BYTES] = {}; // box and periodicity of the last call that read them
     bool have_last_box = false;
@@ -223,6 +250,9 @@ struct HipExtras {
         if (h_shift_ranges != nullptr) {
             (void)hipHostFree(h_shift_ranges);
         }
+        if (h_ordered != nullptr) {
+            (void)hipHostFree(h_ordered);
+        }
         if (have_events) {
             for (auto& event : events) {
                 (void)hipEventDestroy(event);
@@ -246,6 +276,7 @@ HipExtras& extras_of(VesinNeighborList& neighbors) {
         HIP_CHECK(hipHostMalloc(
             reinterpret_cast<void**>(&extras->h_shift_ranges), SHIFT_RANGE_BLOCKS * sizeof(ShiftRange), hipHostMallocDefault
         ));
+        HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&extras->h_ordered), sizeof(OrderedHostStatus), hipHostMallocDefault));
     }
     return *static_cast<HipExtras*>(neighbors.opaque);
 }
@@ -693,7 +724,16 @@ bool compute(
     uint32_t* counts = nullptr;
     uint64_t* offsets = nullptr;
     uint64_t* scan_scratch = nullptr;
-    const size_t scratch_elements = std::max(scan_scratch_elements(n_cells), scan_scratch_elements(n_slots));
+    // the search that produces a sorted list in order covers stencils that fit its tables
+    const size_t full_stencil = static_cast<size_t>(2 * grid.s[0] + 1) * (2 * grid.s[1] + 1) * (2 * grid.s[2] + 1);
+    const bool try_in_order = options.sorted && full_stencil <= MAX_ENTRIES && !radix_sort_only();
+    OrderedStatus* ordered_status = nullptr;
+    uint32_t* rows_of_point = nullptr;
+    uint64_t* first_row_of_point = nullptr;
+    const size_t scratch_elements = std::max(
+        std::max(scan_scratch_elements(n_cells), scan_scratch_elements(n_slots)),
+        try_in_order ? scan_scratch_elements(n_points) : 0
+    );
 
     auto carve = [&](Carver& carver) {
         // adjacent, so that one fill clears the histogram, the tiles' flags and the state of the single-pass search
@@ -703,6 +743,7 @@ bool compute(
         chain.groups = carver.take<uint64_t>(chain_groups);
         chain.bases = carver.take<uint64_t>(chain_groups);
         fused_status = carver.take<FusedStatus>(1);
+        ordered_status = carver.take<OrderedStatus>(1);
         cell_scan = carver.take<uint64_t>(n_cells + 1);
         if (!single_cell) {
             cell_of = carver.take<uint32_t>(n_points);
@@ -720,6 +761,10 @@ bool compute(
         counts = carver.take<uint32_t>(n_slots);
         offsets = carver.take<uint64_t>(n_slots + 1);
         scan_scratch = carver.take<uint64_t>(scratch_elements);
+        if (try_in_order) {
+            rows_of_point = carver.take<uint32_t>(n_points);
+            first_row_of_point = carver.take<uint64_t>(n_points + 1);
+        }
     };
     Carver measure(nullptr);
     carve(measure);
@@ -732,7 +777,7 @@ bool compute(
     const auto* flat_points = reinterpret_cast<const double*>(points);
     {
         // every piece of the work buffer is padded to 256 bytes: clearing whole 16-byte blocks stays inside
-        const size_t to_clear = reinterpret_cast<char*>(fused_status + 1) - reinterpret_cast<char*>(cell_counts);
+        const size_t to_clear = reinterpret_cast<char*>(ordered_status + 1) - reinterpret_cast<char*>(cell_counts);
         const size_t blocks16 = (to_clear + 15) / 16;
         const uint32_t fill_blocks = static_cast<uint32_t>(std::min<size_t>(1024, (blocks16 + BLOCK - 1) / BLOCK));
         hipLaunchKernelGGL(
@@ -881,6 +926,86 @@ bool compute(
             // the shape of this system is not the single-pass kernel's: leave it alone for a while
             extras.single_pass_rest = SINGLE_PASS_REST;
         }
+    }
+
+    // ---- a sorted list straight from the search, when the system has the shape that search covers
+    if (try_in_order && n_points > 0) {
+        OrderedArgs oargs = {};
+        oargs.sorted = sorted;
+        oargs.cell_scan = cell_scan;
+        oargs.tiles = tiles;
+        // small systems: the points of a tile are dealt to several waves, about 2048 in all
+        uint32_t points_per_item = TILE_POINTS;
+        while (points_per_item > 1 && tiles_bound * (TILE_POINTS / points_per_item) < 2048) {
+            points_per_item /= 2;
+        }
+        oargs.points_per_item = points_per_item;
+        oargs.items_per_tile = TILE_POINTS / points_per_item;
+        oargs.rows_of_point = rows_of_point;
+        oargs.first_row = first_row_of_point;
+        oargs.status = ordered_status;
+        const uint32_t blocks =
+            static_cast<uint32_t>((tiles_bound * oargs.items_per_tile + ORDERED_WAVES - 1) / ORDERED_WAVES);
+        if (options.full) {
+            hipLaunchKernelGGL((ordered_search_kernel<false, true>), dim3(blocks), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
+        } else {
+            hipLaunchKernelGGL((ordered_search_kernel<false, false>), dim3(blocks), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
+        }
+        mark(T_COUNT);
+        exclusive_scan<SCAN_U32>(rows_of_point, n_points, first_row_of_point, scan_scratch, stream);
+        mark(T_SCAN);
+        hipLaunchKernelGGL(
+            publish_ordered_status, dim3(1), dim3(1), 0, stream,
+            ordered_status, first_row_of_point + n_points, extras.d_status, extras.h_ordered
+        );
+        HIP_CHECK(hipStreamSynchronize(stream));
+        if (!box_was_right()) {
+            return false;
+        }
+        const OrderedHostStatus found = *extras.h_ordered;
+        if (found.first_bad_coordinate != 0xFFFFFFFFu) {
+            non_finite_error(points, found.first_bad_coordinate);
+        }
+        const bool suitable = found.found.max_rows <= ORDERED_MAX_ROWS &&
+                              found.found.max_candidates <= ORDERED_CANDIDATES && found.found.unsuitable == 0;
+        if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
+            std::fprintf(
+                stderr,
+                "in-order search: rows %llu, most rows of a point %u, most candidates of a tile %u, unsuitable %u: %s\n",
+                found.total_rows, found.found.max_rows, found.found.max_candidates, found.found.unsuitable,
+                suitable ? "used" : "left to the radix sort"
+            );
+        }
+        if (suitable) {
+            const size_t total = found.total_rows;
+            check_pair_limit(total);
+            size_outputs(neighbors, extras, total, options);
+            oargs.out = outputs_of();
+            mark(T_WRITE_BEGIN);
+            if (total > 0) {
+                if (options.full) {
+                    hipLaunchKernelGGL((ordered_search_kernel<true, true>), dim3(blocks), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
+                } else {
+                    hipLaunchKernelGGL((ordered_search_kernel<true, false>), dim3(blocks), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
+                }
+            }
+            mark(T_WRITE);
+            mark(T_SORT);
+            HIP_CHECK(hipStreamSynchronize(stream));
+            HIP_CHECK(hipGetLastError());
+            neighbors.length = total;
+            if (timed) {
+                extras.timings = {};
+                extras.timings.total = elapsed(T_START, T_SORT);
+                extras.timings.cell_build = elapsed(T_START, T_CELLS);
+                extras.timings.count = elapsed(T_CELLS, T_COUNT);
+                extras.timings.scan = elapsed(T_COUNT, T_SCAN);
+                extras.timings.write = elapsed(T_WRITE_BEGIN, T_WRITE);
+                extras.timings_valid = true;
+            }
+            return true;
+        }
+        // rows per point, candidates per tile or shifts beyond what that search handles: the general way below
     }
 
     // ---- pass 1: count
