@@ -80,7 +80,7 @@ def test_ordered_rows_are_the_same_on_every_run(timings, monkeypatch, full):
 def test_ordered_rows_with_crowded_tiles_and_growth(timings, monkeypatch):
     monkeypatch.setenv("VESIN_HIP_ROWS", "ordered")
     rng = np.random.default_rng(22)
-    points = np.concatenate([rng.random((3000, 3)) * 30.0, rng.random((1200, 3)) * 2.5 + 10.0])
+    points = np.concatenate([rng.random((3000, 3)) * 30.0, rng.random((3000, 3)) * 2.5 + 10.0])
     box = np.eye(3) * 30.0
     expected = oracle.neighbors(points, box, True, 2.5, True, False, "ijSdD")
     calculator = NeighborList(cutoff=2.5, full_list=True)
@@ -121,18 +121,22 @@ def test_rows_that_do_not_fit_fall_back(timings):
     assert_same_list(shrunk, oracle.neighbors(*small[:3], 5.0, True, False, "ijSdD"), what="shrunk")
 
 
-def test_crowded_tiles_are_left_to_the_write_pass(timings):
-    # a dense blob inside a sparse gas: tiles of the blob see more candidates than the single pass keeps columns
-    # for; they are counted and placed by it and written by the write pass
+def test_crowded_tiles_are_left_to_the_write_pass(timings, capfd, monkeypatch):
+    # a dense blob inside a sparse gas: tiles of the blob see more candidates (2048) than the single pass keeps
+    # columns for; they are counted and placed by it and written by the write pass
     rng = np.random.default_rng(21)
     gas = rng.random((4000, 3)) * 40.0
-    blob = rng.random((1500, 3)) * 3.0 + 18.0
+    blob = rng.random((4000, 3)) * 3.0 + 18.0
     points = np.concatenate([gas, blob])
     box = np.eye(3) * 40.0
     expected = oracle.neighbors(points, box, True, 2.5, True, False, "ijSdD")
     calculator = NeighborList(cutoff=2.5, full_list=True)
     first = call(calculator, points, box, True)
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    capfd.readouterr()
     second = call(calculator, points, box, True)
+    report = [line for line in capfd.readouterr().err.splitlines() if line.startswith("single pass:")]
+    assert report and " deferred 0 " not in report[-1], report
     assert used_single_pass(calculator)
     assert_same_list(first, expected, what="two-pass")
     assert_same_list(second, expected, what="single pass with deferred tiles")

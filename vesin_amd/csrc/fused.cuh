@@ -30,7 +30,7 @@
 
 namespace vesin_hip {
 
-constexpr int FUSED_UNITS = 8;          // 64-candidate units of one work item whose columns stay in registers
+constexpr int FUSED_UNITS = 32;         // 64-candidate units of one work item whose columns stay in registers
 constexpr int FUSED_SLOTS = 2 * WAVE;   // candidate records in LDS: two units, so that tickets survive a unit change
 constexpr int32_t PACKED_SHIFT_LIMIT = 500;
 constexpr uint32_t CHAIN_SPIN_LIMIT = 1u << 18;
