@@ -56,6 +56,41 @@ def test_random_systems_on_one_reused_list(seed, full):
             assert_same_list(actual, expected, what=f"seed {seed} step {step} repeat {repeat} n={len(points)} periodic={periodic}")
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_random_options_and_moves_on_one_reused_list(seed):
+    """Sorted or not, half or full, with or without a skin; a system is followed for a few small moves (which the
+    Verlet filter and the remembered box meet) before the next one replaces it."""
+    import torch
+
+    rng = np.random.default_rng(50_000 + seed)
+    cutoff = float(rng.choice([1.1, 1.5, 2.5, 3.7]))
+    full = bool(rng.integers(0, 2))
+    is_sorted = bool(rng.integers(0, 2))
+    skin = float(rng.choice([0.0, 0.0, 0.3, 0.9]))
+    calculator = NeighborList(cutoff=cutoff, full_list=full, sorted=is_sorted, skin=skin)
+    points = None
+    for step in range(8):
+        if points is None or rng.random() < 0.5:
+            points, box, periodic = random_system(rng)
+        else:
+            points = points + rng.normal(scale=rng.choice([0.01, 0.1, 0.6]), size=points.shape)
+            if rng.random() < 0.3:
+                box = box + rng.normal(scale=0.02, size=(3, 3)) * (np.abs(box) > 0)
+        expected = oracle.neighbors(points, box, periodic, cutoff, full, False, "ijSdD")
+        outputs = calculator.compute(
+            torch.as_tensor(points, device="cuda:0"), torch.as_tensor(box, device="cuda:0"), periodic, "PSdD"
+        )
+        actual = {NAMES[q]: t.cpu().numpy() for q, t in zip("PSdD", outputs)}
+        what = f"seed {seed} step {step} n={len(points)} sorted={is_sorted} skin={skin} periodic={periodic}"
+        if is_sorted:
+            in_order = oracle.canonicalize(expected)
+            assert actual["pairs"].shape == in_order["pairs"].shape, what
+            for key in actual:
+                assert np.array_equal(actual[key], in_order[key]), (what, key)
+        else:
+            assert_same_list(actual, expected, what=what)
+
+
 def test_random_batches():
     import torch
 
