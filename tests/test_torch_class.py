@@ -260,6 +260,32 @@ def test_backward_with_rows_in_no_order(n_points):
 
 
 @pytest.mark.gpu
+def test_backward_after_the_calculator_moved_on():
+    """With gradients the outputs are copies even when views were asked for: a later calculation on the same
+    calculator must not change what the backward step of an earlier one reads."""
+    from vesin_amd import configs
+
+    calculator = NeighborList(cutoff=4.0, full_list=True, sorted=True)
+    first, box, _ = configs.diamond(3, seed=1)
+    first = torch.tensor(first, device="cuda:0", requires_grad=True)
+    box = torch.tensor(box, device="cuda:0")
+    P, d, D = calculator.compute(first, box, True, "PdD", copy=False)
+    kept = (P.clone(), d.detach().clone(), D.detach().clone())
+    energy = (d**2).sum() + D[:, 0].sum()
+
+    other, other_box, _ = configs.diamond(4, seed=2)
+    calculator.compute(torch.tensor(other, device="cuda:0"), torch.tensor(other_box, device="cuda:0"), True, "PdD", copy=False)
+
+    (points_grad,) = torch.autograd.grad(energy, (first,))
+    distances_grad = 2.0 * kept[1]
+    vectors_grad = torch.zeros_like(kept[2])
+    vectors_grad[:, 0] = 1.0
+    shifts = torch.zeros((len(kept[0]), 3), dtype=torch.int32, device="cuda:0")
+    expected, _ = _backward_with_tensor_operations(kept[0], shifts, kept[1], kept[2], distances_grad, vectors_grad, len(first))
+    assert float((points_grad - expected).abs().max()) <= 1e-12 * float(expected.abs().max())
+
+
+@pytest.mark.gpu
 def test_backward_refuses_rows_of_another_system():
     """The entry point checks the indices it is given instead of writing outside `points_grad`."""
     import ctypes

@@ -251,12 +251,14 @@ public:
         static_assert(sizeof(size_t) == sizeof(int64_t), "pairs are handed out as 64-bit integers");
         const auto length = static_cast<int64_t>(list_.length);
         const auto on_device = torch::TensorOptions().device(points.device());
+        // what the backward step will read must outlive the next calculation on this list: never a view then
+        const bool own_copy = copy || through_autograd;
         const auto wrap = [&](void* data, std::vector<int64_t> shape, torch::ScalarType dtype) {
             if (length == 0 || data == nullptr) {
                 return torch::empty(shape, on_device.dtype(dtype));
             }
             auto view = torch::from_blob(data, shape, on_device.dtype(dtype));
-            return copy ? view.clone() : view;
+            return own_copy ? view.clone() : view;
         };
 
         auto pairs = wrap(list_.pairs, {length, 2}, torch::kInt64);
