@@ -150,7 +150,8 @@ int VESIN_API vesin_hip_neighbors_on_stream(
  *   first_point  host, n_systems + 1 entries: first_point[s] is the index in `points` of the first point of system
  *                s, first_point[n_systems] the total number of points
  *   boxes        device: n_systems boxes (3x3 each, rows = box vectors)
- *   periodic     device: n_systems x 3 flags; every system must be periodic in all three directions
+ *   periodic     device: n_systems x 3 flags, per system and direction (a free molecule has none set and its box
+ *                is not read, like in vesin_neighbors)
  *   neighbors    receives all rows, system after system; the indices in `pairs` count from the first point of the
  *                row's system. Same ownership rules as for vesin_neighbors; the same struct may be used with both.
  *   first_pair   host, n_systems + 1 entries, filled on success: rows [first_pair[s], first_pair[s + 1]) belong to

@@ -65,6 +65,56 @@ def test_systems_of_different_sizes_and_shapes():
             assert_same_list(lists[s], expected, what=f"system {s} full={full}")
 
 
+@pytest.mark.parametrize("full", [True, False], ids=["full", "half"])
+def test_molecules_slabs_and_crystals_in_one_batch(full):
+    """Per-system periodicity: free molecules (box ignored, even all zeros), slabs, wires and crystals side by side,
+    every one with the rows of a call on it alone."""
+    rng = np.random.default_rng(41)
+    all_points, all_boxes, all_flags = [], [], []
+    for n, flags in (
+        (5, (False, False, False)),
+        (180, (False, False, False)),
+        (64, (True, True, True)),
+        (300, (True, True, False)),
+        (1, (False, False, False)),
+        (90, (False, True, False)),
+        (0, (False, False, False)),
+        (1200, (False, False, False)),
+        (400, (True, False, True)),
+    ):
+        edge = 7.0 + 3.0 * rng.random()
+        box = np.eye(3) * edge + 0.4 * rng.normal(size=(3, 3))
+        points = rng.random((n, 3)) @ box * rng.choice([0.6, 1.0, 1.7])
+        if not any(flags) and n == 180:
+            box = np.zeros((3, 3))  # free molecules need no box at all
+        all_points.append(points)
+        all_boxes.append(box)
+        all_flags.append(flags)
+    calculator = NeighborList(cutoff=3.1, full_list=full)
+    lists = run_batch(calculator, all_points, all_boxes, periodic=np.array(all_flags))
+    for s, (points, box, flags) in enumerate(zip(all_points, all_boxes, all_flags)):
+        expected = oracle.neighbors(points, box, list(flags), 3.1, full, False, "ijSdD")
+        assert_same_list(lists[s], expected, what=f"system {s} periodic={flags}")
+
+
+def test_many_free_molecules():
+    """2000 molecules of 3 to 40 atoms: the case a batch is for."""
+    rng = np.random.default_rng(43)
+    all_points = [rng.normal(scale=2.0, size=(int(rng.integers(3, 41)), 3)) + rng.uniform(-50, 50, size=3) for _ in range(2000)]
+    all_boxes = [np.zeros((3, 3))] * len(all_points)
+    calculator = NeighborList(cutoff=2.4, full_list=True)
+    lists = run_batch(calculator, all_points, all_boxes, periodic=False)
+    for s in range(0, len(all_points), 37):
+        expected = oracle.neighbors(all_points[s], all_boxes[s], [False] * 3, 2.4, True, False, "ijSdD")
+        assert_same_list(lists[s], expected, what=f"molecule {s}")
+    total = sum(len(rows["pairs"]) for rows in lists)
+    brute = 0
+    for points in all_points:
+        d = np.linalg.norm(points[:, None, :] - points[None, :, :], axis=-1)
+        brute += int((d < 2.4).sum()) - len(points)
+    assert abs(total - brute) <= 2  # pairs at the cutoff to the last bit aside
+
+
 def test_batch_of_one_equals_the_single_call():
     points, box, periodic, _ = configs.config1(8)
     calculator = NeighborList(cutoff=5.0, full_list=True)
@@ -87,9 +137,11 @@ def test_batch_errors():
     boxes = torch.as_tensor(box[None], device="cuda:0")
     with pytest.raises(RuntimeError, match="sorted output is not available for a batch"):
         NeighborList(cutoff=5.0, full_list=True, sorted=True).compute_batch(device_points, [0, len(points)], boxes)
-    with pytest.raises(RuntimeError, match="not periodic in all directions"):
+    with pytest.raises(RuntimeError, match="non-finite coordinate along axis 1"):
         flags = torch.as_tensor([[True, False, True]], device="cuda:0")
-        NeighborList(cutoff=5.0, full_list=True).compute_batch(device_points, [0, len(points)], boxes, flags)
+        broken = device_points.clone()
+        broken[5, 1] = float("nan")
+        NeighborList(cutoff=5.0, full_list=True).compute_batch(broken, [0, len(points)], boxes, flags)
     with pytest.raises(RuntimeError, match="must not decrease"):
         NeighborList(cutoff=5.0, full_list=True).compute_batch(device_points, [0, 70, len(points)], torch.cat([boxes, boxes]))
     singular = boxes.clone()

@@ -268,11 +268,11 @@ class NeighborList:
         return tuple(data)
 
     def compute_batch(self, points, first_point, boxes, periodic=True, quantities: str = "ij", copy: bool = True):
-        """Neighbor lists of many fully periodic systems in one go (``vesin_hip_neighbors_batch``).
+        """Neighbor lists of many systems in one go (``vesin_hip_neighbors_batch``).
 
         ``points``: (N, 3) GPU tensor with the systems one after the other; ``first_point``: n_systems + 1 integers,
-        where each system starts; ``boxes``: (n_systems, 3, 3) GPU tensor; ``periodic``: ``True`` or an
-        (n_systems, 3) boolean tensor. Returns ``(outputs, first_pair)``: the requested quantities for all systems
+        where each system starts; ``boxes``: (n_systems, 3, 3) GPU tensor; ``periodic``: one flag for everything, or an
+        (n_systems, 3) boolean tensor (free molecules, slabs and crystals can share a batch). Returns ``(outputs, first_pair)``: the requested quantities for all systems
         (indices count inside each system) and the n_systems + 1 row offsets of the systems as a numpy array.
         """
         import torch

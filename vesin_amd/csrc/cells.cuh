@@ -363,6 +363,61 @@ __global__ __launch_bounds__(BLOCK) void place_points(
     }
 }
 
+/// Bounding pass of a batch: one wave per system finds the extrema of the fractional coordinates of its points
+/// (with that system's inverse box, which is all `grids` needs to hold at this point) and the first non-finite
+/// coordinate. Only launched when some system has a non-periodic direction.
+__global__ __launch_bounds__(BLOCK) void bounding_batch_kernel(
+    const double* __restrict__ points, const GridParams* __restrict__ grids, const uint32_t* __restrict__ first_point,
+    uint32_t n_systems, BlockBounds* __restrict__ bounds
+) {
+    const uint32_t system = blockIdx.x * WAVES_PER_BLOCK + threadIdx.x / WAVE;
+    if (system >= n_systems) {
+        return;
+    }
+    const GridParams& g = grids[system];
+    double lo[3] = {INFINITY, INFINITY, INFINITY};
+    double hi[3] = {-INFINITY, -INFINITY, -INFINITY};
+    unsigned int bad = 0xFFFFFFFFu;
+    const uint32_t end = first_point[system + 1];
+    for (uint32_t i = first_point[system] + lane_id(); i < end; i += WAVE) {
+        const double x = points[3 * static_cast<size_t>(i) + 0];
+        const double y = points[3 * static_cast<size_t>(i) + 1];
+        const double z = points[3 * static_cast<size_t>(i) + 2];
+        unsigned int axis;
+        if (!all_finite(x, y, z, axis)) {
+            bad = min(bad, 3u * i + axis);
+            continue;
+        }
+        double f[3];
+        fractional(g, x, y, z, f);
+#pragma unroll
+        for (int d = 0; d < 3; d++) {
+            lo[d] = fmin(lo[d], f[d]);
+            hi[d] = fmax(hi[d], f[d]);
+        }
+    }
+#pragma unroll
+    for (int offset = WAVE / 2; offset > 0; offset >>= 1) {
+#pragma unroll
+        for (int d = 0; d < 3; d++) {
+            lo[d] = fmin(lo[d], __shfl_xor(lo[d], offset));
+            hi[d] = fmax(hi[d], __shfl_xor(hi[d], offset));
+        }
+        bad = min(bad, static_cast<unsigned int>(__shfl_xor(static_cast<int>(bad), offset)));
+    }
+    if (lane_id() == 0) {
+        BlockBounds all;
+#pragma unroll
+        for (int d = 0; d < 3; d++) {
+            all.lo[d] = lo[d];
+            all.hi[d] = hi[d];
+        }
+        all.first_bad_coordinate = bad;
+        all.padding = 0;
+        bounds[system] = all;
+    }
+}
+
 /// assign_cells for many systems at once: every point looks up its system (binary search in `first_point`), uses
 /// that system's grid, and counts itself in the system's range of cells.
 __global__ __launch_bounds__(BLOCK) void assign_cells_batch(

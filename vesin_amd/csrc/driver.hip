@@ -1381,27 +1381,18 @@ void neighbors_batch(
     HIP_CHECK(hipMemcpy(host_periodic.data(), periodic, host_periodic.size(), hipMemcpyDeviceToHost));
 
     std::vector<GridParams> grids(n_systems);
+    std::vector<HostBox> host_grids_box(n_systems);
     std::vector<uint32_t> cell_base_host(n_systems + 1);
     std::vector<uint32_t> first_point_host(n_systems + 1);
-    uint64_t total_cells = 0;
-    const double zeros[3] = {0.0, 0.0, 0.0};
+    bool any_open_direction = false;
     for (size_t s = 0; s < n_systems; s++) {
         bool flags[3];
         for (int d = 0; d < 3; d++) {
             flags[d] = host_periodic[3 * s + d] != 0;
-        }
-        if (!(flags[0] && flags[1] && flags[2])) {
-            throw std::runtime_error(
-                "system " + std::to_string(s) + " is not periodic in all directions: a batch only takes fully periodic systems"
-            );
+            any_open_direction = any_open_direction || !flags[d];
         }
         const HostBox hbox = normalise_box(&host_boxes[9 * s], flags);
-        const size_t n_here = first_point[s + 1] - first_point[s];
-        bool single_cell = options.algorithm == VesinBruteForce;
-        HostGrid grid = choose_grid(hbox, options.cutoff, n_here, zeros, zeros, single_cell);
-        if (options.algorithm == VesinAutoAlgorithm && !single_cell && (grid.n_cells == 1 || n_here < 32)) {
-            grid = choose_grid(hbox, options.cutoff, n_here, zeros, zeros, true);
-        }
+        host_grids_box[s] = hbox;
         GridParams& g = grids[s];
         std::memset(&g, 0, sizeof(g));
         for (int d = 0; d < 3; d++) {
@@ -1409,7 +1400,58 @@ void neighbors_batch(
                 g.H[3 * d + e] = hbox.H[d][e];
                 g.Hinv[3 * d + e] = hbox.Hinv[d][e];
             }
-            g.periodic[d] = 1;
+            g.periodic[d] = flags[d] ? 1 : 0;
+        }
+        first_point_host[s] = static_cast<uint32_t>(first_point[s]);
+    }
+    first_point_host[n_systems] = static_cast<uint32_t>(n_points);
+
+    // ---- systems with a non-periodic direction need the extent of their points along it (reference:
+    // BoundingBox::make_bounding_for, vesin/src/types.hpp:159-200): one wave per system finds it
+    std::vector<BlockBounds> bounds;
+    if (any_open_direction && n_points > 0) {
+        const size_t grids_bytes = (n_systems * sizeof(GridParams) + 255) & ~size_t(255);
+        const size_t firsts_bytes = ((n_systems + 1) * sizeof(uint32_t) + 255) & ~size_t(255);
+        extras.sort_work.reserve(grids_bytes + firsts_bytes + n_systems * sizeof(BlockBounds));
+        char* base = static_cast<char*>(extras.sort_work.ptr);
+        auto* early_grids = reinterpret_cast<GridParams*>(base);
+        auto* early_firsts = reinterpret_cast<uint32_t*>(base + grids_bytes);
+        auto* d_bounds = reinterpret_cast<BlockBounds*>(base + grids_bytes + firsts_bytes);
+        HIP_CHECK(hipMemcpyAsync(early_grids, grids.data(), n_systems * sizeof(GridParams), hipMemcpyHostToDevice, stream));
+        HIP_CHECK(hipMemcpyAsync(
+            early_firsts, first_point_host.data(), (n_systems + 1) * sizeof(uint32_t), hipMemcpyHostToDevice, stream
+        ));
+        const uint32_t blocks = static_cast<uint32_t>((n_systems + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK);
+        hipLaunchKernelGGL(
+            bounding_batch_kernel, dim3(blocks), dim3(BLOCK), 0, stream,
+            reinterpret_cast<const double*>(points), early_grids, early_firsts, static_cast<uint32_t>(n_systems), d_bounds
+        );
+        bounds.resize(n_systems);
+        HIP_CHECK(hipMemcpyAsync(bounds.data(), d_bounds, n_systems * sizeof(BlockBounds), hipMemcpyDeviceToHost, stream));
+        HIP_CHECK(hipStreamSynchronize(stream));
+        unsigned int bad = 0xFFFFFFFFu;
+        for (const BlockBounds& found : bounds) {
+            bad = std::min(bad, found.first_bad_coordinate);
+        }
+        if (bad != 0xFFFFFFFFu) {
+            non_finite_error(points, bad);
+        }
+    }
+
+    uint64_t total_cells = 0;
+    const double zeros[3] = {0.0, 0.0, 0.0};
+    for (size_t s = 0; s < n_systems; s++) {
+        const HostBox& hbox = host_grids_box[s];
+        const size_t n_here = first_point[s + 1] - first_point[s];
+        const double* lo = bounds.empty() ? zeros : bounds[s].lo;
+        const double* hi = bounds.empty() ? zeros : bounds[s].hi;
+        bool single_cell = options.algorithm == VesinBruteForce;
+        HostGrid grid = choose_grid(hbox, options.cutoff, n_here, lo, hi, single_cell);
+        if (options.algorithm == VesinAutoAlgorithm && !single_cell && (grid.n_cells == 1 || n_here < 32)) {
+            grid = choose_grid(hbox, options.cutoff, n_here, lo, hi, true);
+        }
+        GridParams& g = grids[s];
+        for (int d = 0; d < 3; d++) {
             g.n[d] = grid.n[d];
             g.s[d] = grid.s[d];
             g.np_min[d] = grid.np_min[d];
@@ -1419,14 +1461,12 @@ void neighbors_batch(
         g.n_points = static_cast<uint32_t>(n_here);
         g.n_cells = static_cast<uint32_t>(grid.n_cells);
         cell_base_host[s] = static_cast<uint32_t>(total_cells);
-        first_point_host[s] = static_cast<uint32_t>(first_point[s]);
         total_cells += grid.n_cells;
         if (total_cells >= 0xFFFFFFF0ull) {
             throw std::runtime_error("too many cells in this batch");
         }
     }
     cell_base_host[n_systems] = static_cast<uint32_t>(total_cells);
-    first_point_host[n_systems] = static_cast<uint32_t>(n_points);
 
     if (n_points == 0) {
         size_outputs(neighbors, extras, 0, options);

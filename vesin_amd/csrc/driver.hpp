@@ -19,7 +19,7 @@ void neighbors(
     void* stream
 );
 
-/// The lists of many (fully periodic) systems in one sequence of launches. `points`, `boxes`, `periodic` are device
+/// The lists of many systems in one sequence of launches. `points`, `boxes`, `periodic` are device
 /// memory holding the systems one after the other; `first_point` (host, n_systems + 1 entries) says where each
 /// system starts. Rows come out system after system with indices counted inside each system; `first_pair` (host,
 /// n_systems + 1 entries) receives where each system's rows start.
