@@ -20,14 +20,24 @@ def run_batch(calculator, all_points, all_boxes, letters="PSdD", periodic=True):
     first_point = np.cumsum([0] + [len(p) for p in all_points])
     points = torch.as_tensor(np.concatenate(all_points).astype(np.float64), device="cuda:0")
     boxes = torch.as_tensor(np.stack(all_boxes).astype(np.float64), device="cuda:0")
-    outputs, first_pair = calculator.compute_batch(points, first_point, boxes, periodic, letters)
-    whole = {NAMES[q]: out.cpu().numpy() for q, out in zip(letters, outputs)}
-    per_system = []
-    for s in range(len(all_points)):
-        rows = slice(int(first_pair[s]), int(first_pair[s + 1]))
-        per_system.append({key: value[rows] for key, value in whole.items()})
-    assert first_pair[0] == 0 and first_pair[-1] == len(whole["pairs"])
-    return per_system
+    # the first call of a list sizes its arrays with the two passes, the second goes through the single-pass
+    # search: both must give the same rows per system
+    results = []
+    for _ in range(2):
+        outputs, first_pair = calculator.compute_batch(points, first_point, boxes, periodic, letters)
+        whole = {NAMES[q]: out.cpu().numpy() for q, out in zip(letters, outputs)}
+        per_system = []
+        for s in range(len(all_points)):
+            rows = slice(int(first_pair[s]), int(first_pair[s + 1]))
+            per_system.append({key: value[rows] for key, value in whole.items()})
+        assert first_pair[0] == 0 and first_pair[-1] == len(whole["pairs"])
+        results.append(per_system)
+    first, second = results
+    for s, (a, b) in enumerate(zip(first, second)):
+        assert len(a["pairs"]) == len(b["pairs"]), f"system {s}: the second call has other rows than the first"
+        if "shifts" in a and "distances" in a and "vectors" in a:
+            assert_same_list(b, a, what=f"system {s}, second call against the first")
+    return second
 
 
 @pytest.mark.parametrize("full", [True, False], ids=["full", "half"])
@@ -113,6 +123,49 @@ def test_many_free_molecules():
         d = np.linalg.norm(points[:, None, :] - points[None, :, :], axis=-1)
         brute += int((d < 2.4).sum()) - len(points)
     assert abs(total - brute) <= 2  # pairs at the cutoff to the last bit aside
+
+
+def test_single_pass_on_a_reused_list_and_its_fallbacks(capfd, monkeypatch):
+    """A list that served a batch goes through the single-pass search on the next one; a larger batch that does
+    not fit its arrays, or VESIN_HIP_SEARCH=two-pass, starts over with the two passes."""
+    import torch
+
+    def batch(replicas):
+        chosen = [configs.config3(r) for r in replicas]
+        first_point = np.cumsum([0] + [len(c[0]) for c in chosen])
+        points = torch.as_tensor(np.concatenate([c[0] for c in chosen]), device="cuda:0")
+        boxes = torch.as_tensor(np.stack([c[1] for c in chosen]), device="cuda:0")
+        return chosen, points, first_point, boxes
+
+    def report():
+        return [line for line in capfd.readouterr().err.splitlines() if line.startswith("single pass (batch):")]
+
+    def check(chosen, outputs, first_pair):
+        whole = {NAMES[q]: out.cpu().numpy() for q, out in zip("PSdD", outputs)}
+        for s in (0, len(chosen) - 1):
+            rows = slice(int(first_pair[s]), int(first_pair[s + 1]))
+            expected = oracle.neighbors(chosen[s][0], chosen[s][1], chosen[s][2], 10.0, True, False, "ijSdD")
+            assert_same_list({key: value[rows] for key, value in whole.items()}, expected, what=f"system {s}")
+
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    calculator = NeighborList(cutoff=10.0, full_list=True)
+    small = batch(range(6))
+    large = batch(range(6, 30))
+    capfd.readouterr()
+    check(small[0], *calculator.compute_batch(small[1], small[2], small[3], True, "PSdD"))
+    assert not report()  # first call: nothing to write into yet
+    check(small[0], *calculator.compute_batch(small[1], small[2], small[3], True, "PSdD"))
+    lines = report()
+    assert lines and " deferred 0 overflow 0 timeout 0" in lines[-1] and " general 0 " in lines[-1], lines
+    check(large[0], *calculator.compute_batch(large[1], large[2], large[3], True, "PSdD"))
+    lines = report()
+    assert lines and " overflow 0 " not in lines[-1], lines  # four times the rows: did not fit, two passes
+    check(large[0], *calculator.compute_batch(large[1], large[2], large[3], True, "PSdD"))
+    lines = report()
+    assert lines and " overflow 0 " in lines[-1], lines
+    monkeypatch.setenv("VESIN_HIP_SEARCH", "two-pass")
+    check(small[0], *calculator.compute_batch(small[1], small[2], small[3], True, "PSdD"))
+    assert not report()
 
 
 def test_batch_of_one_equals_the_single_call():

@@ -1290,14 +1290,16 @@ void verlet_neighbors(
 /// first_pair[s] = first output row of system s (offsets are kept per tile-major work item), first_pair[n] = total.
 __global__ void system_rows_kernel(
     const uint64_t* __restrict__ cell_scan, const uint32_t* __restrict__ cell_base, const uint64_t* __restrict__ offsets,
-    uint32_t n_systems, uint32_t n_slices, uint32_t n_slots, unsigned long long* __restrict__ first_pair
+    uint32_t n_systems, uint32_t n_slices, uint32_t n_slots, const FusedStatus* __restrict__ single_pass,
+    unsigned long long* __restrict__ first_pair
 ) {
     const uint32_t s = blockIdx.x * BLOCK + threadIdx.x;
     if (s > n_systems) {
         return;
     }
     if (s == n_systems) {
-        first_pair[s] = offsets[n_slots];
+        // after the single-pass search `offsets` holds the first row of every work item, the total is in its status
+        first_pair[s] = single_pass != nullptr ? single_pass->total_rows : offsets[n_slots];
         return;
     }
     const uint32_t first_tile = static_cast<uint32_t>(cell_scan[cell_base[s]] >> 32);
@@ -1485,7 +1487,26 @@ void neighbors_batch(
     if (tiles_bound < 8192) {
         n_slices = static_cast<uint32_t>(std::min<size_t>(256, (8192 + tiles_bound - 1) / tiles_bound));
     }
+    // the single-pass search keeps the hit columns of FUSED_UNITS units per work item: enough slices for the
+    // system with the most candidates per tile (estimated from its mean occupation)
+    {
+        double most_units = 1.0;
+        for (size_t s = 0; s < n_systems; s++) {
+            const GridParams& g = grids[s];
+            const double entries = 0.5 * ((2.0 * g.s[0] + 1.0) * (2.0 * g.s[1] + 1.0) * (2.0 * g.s[2] + 1.0) + 1.0);
+            const double per_cell = std::max(1.0, static_cast<double>(g.n_points) / std::max(1u, g.n_cells));
+            most_units = std::max(most_units, std::ceil(entries * per_cell / WAVE));
+        }
+        const double wanted = std::ceil(most_units / FUSED_UNITS);
+        if (wanted > n_slices) {
+            n_slices = static_cast<uint32_t>(std::min(256.0, wanted));
+        }
+    }
     const size_t n_slots = tiles_bound * n_slices;
+    const size_t search_workgroups = (n_slots + SEARCH_WAVES - 1) / SEARCH_WAVES;
+    const size_t chain_groups = (search_workgroups + CHAIN_GROUP - 1) / CHAIN_GROUP;
+    Chain chain = {};
+    FusedStatus* fused_status = nullptr;
 
     uint32_t* cell_counts = nullptr;
     Tile* tiles = nullptr;
@@ -1504,8 +1525,13 @@ void neighbors_batch(
     unsigned long long* d_first_pair = nullptr;
     const size_t scratch_elements = std::max(scan_scratch_elements(total_cells), scan_scratch_elements(n_slots));
     auto carve = [&](Carver& carver) {
+        // adjacent, so that one fill clears the histogram, the tiles' flags and the state of the single-pass search
         cell_counts = carver.take<uint32_t>(total_cells);
         tiles = carver.take<Tile>(tiles_bound);
+        chain.blocks = carver.take<uint64_t>(search_workgroups);
+        chain.groups = carver.take<uint64_t>(chain_groups);
+        chain.bases = carver.take<uint64_t>(chain_groups);
+        fused_status = carver.take<FusedStatus>(1);
         cell_scan = carver.take<uint64_t>(total_cells + 1);
         cell_of = carver.take<uint32_t>(n_points);
         slot_of = carver.take<uint32_t>(n_points);
@@ -1548,7 +1574,7 @@ void neighbors_batch(
         reinterpret_cast<const double*>(boxes), reinterpret_cast<const bool*>(periodic), extras.h_small, extras.d_status
     );
     {
-        const size_t to_clear = reinterpret_cast<char*>(tiles + tiles_bound) - reinterpret_cast<char*>(cell_counts);
+        const size_t to_clear = reinterpret_cast<char*>(fused_status + 1) - reinterpret_cast<char*>(cell_counts);
         HIP_CHECK(hipMemsetAsync(cell_counts, 0, to_clear, stream));
         HIP_CHECK(hipMemsetAsync(counts, 0, n_slots * sizeof(uint32_t), stream));
     }
@@ -1576,6 +1602,66 @@ void neighbors_batch(
     args.grids = d_grids;
     args.cell_base = d_cell_base;
     args.total_cells = static_cast<uint32_t>(total_cells);
+    const uint32_t system_blocks = static_cast<uint32_t>((n_systems + 1 + BLOCK - 1) / BLOCK);
+    static_assert(sizeof(size_t) == sizeof(unsigned long long), "size_t is 64 bits wide here");
+
+    // ---- a list that has arrays from earlier calls: single-pass search straight into them, rows in work-item order
+    // (the rows of a system stay together). Whatever does not fit its shape starts over with the two passes below.
+    if (extras.capacity > 0 && !two_pass_only()) {
+        size_outputs(neighbors, extras, 0, options);
+        FusedArgs fargs = {};
+        fargs.search = args;
+        fargs.search.out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
+        fargs.search.out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
+        fargs.search.out.distances = neighbors.distances;
+        fargs.search.out.vectors = reinterpret_cast<double*>(neighbors.vectors);
+        fargs.search.capacity = extras.capacity;
+        fargs.chain = chain;
+        fargs.first_rows = offsets;
+        fargs.status = fused_status;
+        const uint32_t blocks = static_cast<uint32_t>(search_workgroups);
+        if (options.full) {
+            hipLaunchKernelGGL(
+                (fused_search_kernel<true, true, true>), dim3(blocks), dim3(SEARCH_BLOCK), 0, stream, fargs, GridParams{}
+            );
+        } else {
+            hipLaunchKernelGGL(
+                (fused_search_kernel<false, true, true>), dim3(blocks), dim3(SEARCH_BLOCK), 0, stream, fargs, GridParams{}
+            );
+        }
+        hipLaunchKernelGGL(publish_fused_status, dim3(1), dim3(1), 0, stream, extras.d_status, fused_status, extras.h_fused);
+        hipLaunchKernelGGL(
+            system_rows_kernel, dim3(system_blocks), dim3(BLOCK), 0, stream,
+            cell_scan, d_cell_base, offsets, static_cast<uint32_t>(n_systems), n_slices, static_cast<uint32_t>(n_slots),
+            fused_status, d_first_pair
+        );
+        HIP_CHECK(hipMemcpyAsync(first_pair, d_first_pair, (n_systems + 1) * sizeof(size_t), hipMemcpyDeviceToHost, stream));
+        HIP_CHECK(hipStreamSynchronize(stream));
+        const FusedStatus result = *extras.h_fused;
+        if (result.first_bad_coordinate != 0xFFFFFFFFu) {
+            non_finite_error(points, result.first_bad_coordinate);
+        }
+        if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
+            std::fprintf(
+                stderr, "single pass (batch): rows %llu general %u deferred %u overflow %u timeout %u (slices %u)\n",
+                result.total_rows, result.general, result.deferred, result.overflow, result.chain_timeout, n_slices
+            );
+        }
+        if (result.general == 0 && result.deferred == 0 && result.overflow == 0 && result.chain_timeout == 0) {
+            if (pair_limit != 0 && result.total_rows > n_points * pair_limit) {
+                throw std::runtime_error(
+                    "The number of neighbor pairs exceeds the maximum capacity of " + std::to_string(n_points * pair_limit) +
+                    " (max_pairs_per_point=" + std::to_string(pair_limit) + "; n_points=" + std::to_string(n_points) + "). " +
+                    "Consider reducing the cutoff distance, or explicitly setting " +
+                    "VESIN_CUDA_MAX_PAIRS_PER_POINT as an environment variable."
+                );
+            }
+            HIP_CHECK(hipGetLastError());
+            neighbors.length = result.total_rows;
+            return;
+        }
+    }
+
     launch_search_batch<false>(options.full, args, stream);
     exclusive_scan<SCAN_U32>(counts, n_slots, offsets, scan_scratch, stream);
     hipLaunchKernelGGL(publish_status, dim3(1), dim3(1), 0, stream, extras.d_status, offsets + n_slots, extras.h_status);
@@ -1602,12 +1688,11 @@ void neighbors_batch(
     if (total > 0) {
         launch_search_batch<true>(options.full, args, stream);
     }
-    const uint32_t system_blocks = static_cast<uint32_t>((n_systems + 1 + BLOCK - 1) / BLOCK);
     hipLaunchKernelGGL(
         system_rows_kernel, dim3(system_blocks), dim3(BLOCK), 0, stream,
-        cell_scan, d_cell_base, offsets, static_cast<uint32_t>(n_systems), n_slices, static_cast<uint32_t>(n_slots), d_first_pair
+        cell_scan, d_cell_base, offsets, static_cast<uint32_t>(n_systems), n_slices, static_cast<uint32_t>(n_slots),
+        static_cast<const FusedStatus*>(nullptr), d_first_pair
     );
-    static_assert(sizeof(size_t) == sizeof(unsigned long long), "size_t is 64 bits wide here");
     HIP_CHECK(hipMemcpyAsync(first_pair, d_first_pair, (n_systems + 1) * sizeof(size_t), hipMemcpyDeviceToHost, stream));
     HIP_CHECK(hipStreamSynchronize(stream));
     HIP_CHECK(hipGetLastError());

@@ -456,15 +456,21 @@ __device__ __forceinline__ uint64_t chain_position(
 /// run (the waves of a workgroup meet twice: to add up their rows, and to learn their place from the chain).
 /// Otherwise the waves never wait for one another and the rows come out in order of arrival, which varies from run
 /// to run like the order of the reference's GPU kernels (vesin/src/cuda/cell_list.cu:664, an atomic per pair there).
-template <bool FULL, bool ORDERED>
-__global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fargs, GridParams g) {
+/// BATCH: many systems in one launch (see search_kernel_batch): the grid is the one of the tile's system, tiles are
+/// taken in their order (systems stay together) and every work item reports its first row, from which the host
+/// learns where each system's rows start. Only used with ORDERED.
+template <bool FULL, bool ORDERED, bool BATCH = false>
+__global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fargs, GridParams single_grid) {
     constexpr int R = 2;
     __shared__ FusedShared shared;
     const SearchArgs& args = fargs.search;
     const int lane = lane_id();
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     FusedWaveShared& sh = shared.wave[wave];
-    const uint32_t n_tiles = static_cast<uint32_t>(args.cell_scan[g.n_cells] >> 32);
+    GridParams batch_grid;
+    const GridParams& g = BATCH ? batch_grid : single_grid;
+    const uint32_t n_tiles =
+        static_cast<uint32_t>(args.cell_scan[BATCH ? args.total_cells : single_grid.n_cells] >> 32);
     const uint32_t work = blockIdx.x * SEARCH_WAVES + wave;
     const SortedPoints& sorted = args.sorted;
 
@@ -492,19 +498,27 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fa
     if (work < args.n_work) {
         const uint32_t slice = work % args.n_slices;
         const uint32_t slot = work / args.n_slices;
-        const uint32_t per_xcd = (n_tiles + N_XCD - 1) / N_XCD;
-        const uint32_t xcd = (slot / SEARCH_WAVES) % N_XCD;
-        const uint32_t within = (slot / (SEARCH_WAVES * N_XCD)) * SEARCH_WAVES + slot % SEARCH_WAVES;
+        const uint32_t per_xcd = BATCH ? n_tiles : (n_tiles + N_XCD - 1) / N_XCD;
+        const uint32_t xcd = BATCH ? 0 : (slot / SEARCH_WAVES) % N_XCD;
+        const uint32_t within = BATCH ? slot : (slot / (SEARCH_WAVES * N_XCD)) * SEARCH_WAVES + slot % SEARCH_WAVES;
         const uint32_t tile_id = xcd * per_xcd + within;
 
         if (within < per_xcd && tile_id < n_tiles) {
             const Tile tile = args.tiles[tile_id];
             item.n_i = tile.count;
             item.first_i = tile.first;
-            item.tile_wrapped = tile.wrapped != 0;
-            const int32_t cx = tile.cell % g.n[0];
-            const int32_t cy = (tile.cell / g.n[0]) % g.n[1];
-            const int32_t cz = tile.cell / (g.n[0] * g.n[1]);
+            item.tile_wrapped = (tile.wrapped & 1u) != 0;
+            uint32_t first_cell = 0;
+            if (BATCH) {
+                const uint32_t system = tile_system(tile);
+                batch_grid = args.grids[system];
+                first_cell = args.cell_base[system];
+            }
+            const uint64_t* __restrict__ cell_scan = args.cell_scan + first_cell;
+            const uint32_t local_cell = tile.cell - first_cell;
+            const int32_t cx = local_cell % g.n[0];
+            const int32_t cy = (local_cell / g.n[0]) % g.n[1];
+            const int32_t cz = local_cell / (g.n[0] * g.n[1]);
 
             const int32_t span_y = 2 * g.s[1] + 1;
             const int32_t span_z = 2 * g.s[2] + 1;
@@ -526,7 +540,7 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fa
                     sh.tile_wz[lane] = sorted.wz[at];
                 }
                 item.n_batch = n_entries;
-                fill_stencil_tables(sh, lane, centre, n_entries, cx, cy, cz, span_y, span_z, g, args.cell_scan);
+                fill_stencil_tables(sh, lane, centre, n_entries, cx, cy, cz, span_y, span_z, g, cell_scan);
                 item.n_candidates = __builtin_amdgcn_readfirstlane(sh.n_candidates);
 
                 const uint32_t n_groups = (item.n_candidates + WAVE * R - 1) / (WAVE * R);
@@ -662,6 +676,9 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fa
     }
     const bool leave_to_write_pass = item.valid && item.deferred && item.hits != 0 && writable;
     if (work < args.n_work && lane == 0) {
+        if (BATCH) {
+            fargs.first_rows[work] = first_row;
+        }
         args.counts[work] = leave_to_write_pass ? 1u : 0u;
         if (leave_to_write_pass) {
             fargs.first_rows[work] = first_row;
