@@ -228,3 +228,48 @@ def test_stencils_larger_than_the_single_pass_tables(timings):
     for repeat in range(3):
         assert_same_list(call(calculator, points, box, True), expected, what=f"call {repeat + 1}")
         assert not used_single_pass(calculator)
+
+
+def _single_pass_reports(capfd):
+    return [line for line in capfd.readouterr().err.splitlines() if line.startswith("single pass:")]
+
+
+@pytest.mark.parametrize("full", [True, False], ids=["full", "half"])
+def test_one_pass_cell_build(full, capfd, monkeypatch):
+    """Large systems with cells of ordinary occupation (here 64,000 atoms, 23 per cell) build their cells in one
+    pass, every cell owning 32 slots; VESIN_HIP_CELLS=packed keeps the counting sort. Same rows either way, also
+    with points that were moved out of the box by whole box vectors."""
+    points, box, periodic, _ = configs.config1(20)
+    rng = np.random.default_rng(3)
+    points = points + rng.integers(-1, 2, size=points.shape) @ box * (rng.random((len(points), 1)) < 0.05)
+    expected = oracle.neighbors(points, box, periodic, 5.0, full, False, "ijSdD")
+    calculator = NeighborList(cutoff=5.0, full_list=full)
+    call(calculator, points, box, periodic)
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    capfd.readouterr()
+    assert_same_list(call(calculator, points, box, periodic), expected, what="one-pass cell build")
+    reports = _single_pass_reports(capfd)
+    assert reports and "one-pass cell build, crowded 0)" in reports[-1], reports
+    monkeypatch.setenv("VESIN_HIP_CELLS", "packed")
+    assert_same_list(call(calculator, points, box, periodic), expected, what="packed cells")
+    reports = _single_pass_reports(capfd)
+    assert reports and "packed cells" in reports[-1], reports
+
+
+def test_one_pass_cell_build_with_a_cell_too_full(capfd, monkeypatch):
+    """One cell holds more points than it has slots: the call's result comes from the packed layout and the two
+    passes, and the list stays away from the one-pass build afterwards."""
+    points, box, periodic, _ = configs.config1(20)
+    rng = np.random.default_rng(4)
+    points[:40] = points[0] + 0.3 * rng.random((40, 3))
+    expected = oracle.neighbors(points, box, periodic, 5.0, True, False, "ijSdD")
+    calculator = NeighborList(cutoff=5.0, full_list=True)
+    call(calculator, points, box, periodic)
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    capfd.readouterr()
+    assert_same_list(call(calculator, points, box, periodic), expected, what="after the overflow")
+    reports = _single_pass_reports(capfd)
+    assert reports and "one-pass cell build, crowded" in reports[-1] and "crowded 0)" not in reports[-1], reports
+    assert_same_list(call(calculator, points, box, periodic), expected, what="next call")
+    reports = _single_pass_reports(capfd)
+    assert reports and "packed cells" in reports[-1], reports

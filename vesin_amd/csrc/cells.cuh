@@ -21,7 +21,7 @@ struct FusedStatus {
     unsigned int overflow;         // workgroups whose rows did not fit the output arrays
     unsigned int chain_timeout;    // waves that gave up waiting for an earlier workgroup
     unsigned int first_bad_coordinate;
-    unsigned int padding;
+    unsigned int crowded_cells;    // fixed-capacity layout: points that found their cell full (the result is void)
 };
 
 /// Cell-sorted copy of the points, one array per component: 64 consecutive candidates load coalesced, and four
@@ -52,6 +52,7 @@ __global__ void fetch_box(
     } else if (t == 12) {
         status->total_pairs = 0;
         status->first_bad_coordinate = 0xFFFFFFFFu;
+        status->crowded_cells = 0;
     }
 }
 
@@ -71,6 +72,7 @@ __global__ __launch_bounds__(BLOCK) void clear_and_fetch(
         } else if (t == 12) {
             status->total_pairs = 0;
             status->first_bad_coordinate = 0xFFFFFFFFu;
+            status->crowded_cells = 0;
         }
     }
     const uint4 zero = {0u, 0u, 0u, 0u};
@@ -94,6 +96,7 @@ __global__ void publish_fused_status(const DeviceStatus* status, const FusedStat
     if (threadIdx.x == 0 && blockIdx.x == 0) {
         FusedStatus copy = *fused;
         copy.first_bad_coordinate = status->first_bad_coordinate;
+        copy.crowded_cells = status->crowded_cells;
         *host_fused = copy;
     }
 }
@@ -278,6 +281,79 @@ __global__ __launch_bounds__(BLOCK) void assign_cells(
             wrap_of[3 * static_cast<size_t>(i) + 1] = wrap[1];
             wrap_of[3 * static_cast<size_t>(i) + 2] = wrap[2];
         }
+    }
+}
+
+/// Cell build in one pass, for the single-pass search: every cell owns `capacity` slots of the cell-sorted arrays
+/// (cell c: slots c * capacity ...), a point takes the slot the histogram atomic hands out and is written there at
+/// once. No scan, no second pass over the points; the search reads a cell's points as (c * capacity, count[c]).
+/// A point that finds its cell full is counted in `status->crowded_cells` and dropped: the host then builds the
+/// packed layout instead. `wrapped[c * capacity / TILE_POINTS + k]` is set when tile k of cell c holds a point
+/// that was moved by a box vector. Lanes of a wave in the same cell share one atomic, like in assign_cells.
+__global__ __launch_bounds__(BLOCK) void place_direct(
+    const double* __restrict__ points, GridParams g, uint32_t capacity, uint32_t* __restrict__ cell_counts,
+    uint32_t* __restrict__ wrapped, SortedPoints sorted, DeviceStatus* status
+) {
+    const uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
+    const bool active = i < g.n_points;
+    const int lane = lane_id();
+
+    int32_t cell[3] = {0, 0, 0};
+    int32_t wrap[3] = {0, 0, 0};
+    double x = 0.0, y = 0.0, z = 0.0;
+    if (active) {
+        x = points[3 * static_cast<size_t>(i) + 0];
+        y = points[3 * static_cast<size_t>(i) + 1];
+        z = points[3 * static_cast<size_t>(i) + 2];
+        unsigned int axis;
+        if (all_finite(x, y, z, axis)) {
+            locate(g, x, y, z, cell, wrap);
+        } else {
+            atomicMin(&status->first_bad_coordinate, 3u * i + axis);
+        }
+    }
+    const uint32_t linear = (static_cast<uint32_t>(cell[2]) * g.n[1] + cell[1]) * g.n[0] + cell[0];
+
+    uint64_t group = 1ull << lane; // lanes left over after the rounds stand alone
+    bool pending = active;
+    for (int round = 0; round < ASSIGN_ROUNDS; round++) {
+        const uint64_t remaining = __ballot(pending);
+        if (remaining == 0) {
+            break;
+        }
+        const int leader = __ffsll(static_cast<unsigned long long>(remaining)) - 1;
+        const uint32_t leader_cell = read_lane(linear, leader);
+        const bool same = pending && linear == leader_cell;
+        const uint64_t members = __ballot(same);
+        if (same) {
+            group = members;
+            pending = false;
+        }
+    }
+    const int first = __ffsll(static_cast<unsigned long long>(group)) - 1;
+    uint32_t base = 0;
+    if (active && lane == first) {
+        base = atomicAdd(&cell_counts[linear], static_cast<uint32_t>(__popcll(group)));
+    }
+    base = static_cast<uint32_t>(__shfl(static_cast<int>(base), first));
+    if (!active) {
+        return;
+    }
+    const uint32_t k = base + rank_in_mask(group);
+    if (k >= capacity) {
+        atomicAdd(&status->crowded_cells, 1u);
+        return;
+    }
+    const size_t to = static_cast<size_t>(linear) * capacity + k;
+    sorted.index[to] = i;
+    sorted.x[to] = x;
+    sorted.y[to] = y;
+    sorted.z[to] = z;
+    sorted.wx[to] = wrap[0];
+    sorted.wy[to] = wrap[1];
+    sorted.wz[to] = wrap[2];
+    if ((wrap[0] | wrap[1] | wrap[2]) != 0) {
+        atomicOr(&wrapped[(linear * capacity + k) / TILE_POINTS], 1u);
     }
 }
 

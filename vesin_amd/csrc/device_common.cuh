@@ -44,7 +44,7 @@ struct Tile {
 struct DeviceStatus {
     unsigned long long total_pairs;
     unsigned int first_bad_coordinate; // 3 * point + axis of the first non-finite coordinate, or 0xFFFFFFFF
-    unsigned int padding;
+    unsigned int crowded_cells;        // fixed-capacity layout: points that found their cell full
 };
 
 /// What one workgroup of the bounding pass reports (to pinned host memory; the host folds the workgroups).

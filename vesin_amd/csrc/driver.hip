@@ -62,6 +62,13 @@ static bool two_pass_only() {
     return text != nullptr && std::strcmp(text, "two-pass") == 0;
 }
 
+/// VESIN_HIP_CELLS=packed keeps every call on the counting-sort cell build (for comparisons and tests) instead of
+/// the one-pass build with a fixed number of slots per cell that the single-pass search can read.
+static bool packed_cells_only() {
+    const char* text = std::getenv("VESIN_HIP_CELLS");
+    return text != nullptr && std::strcmp(text, "packed") == 0;
+}
+
 /// VESIN_HIP_SORT=radix keeps sorted lists on the unsorted search followed by the radix sort (for comparisons and
 /// tests) instead of the search that produces them in order.
 static bool radix_sort_only() {
@@ -159,6 +166,14 @@ struct Carver {
 /// breaks even near 1.6 M and takes twice the direct search's time at 15 M.
 constexpr size_t VERLET_MAX_CANDIDATES = size_t(1) << 20;
 
+/// One-pass cell build: slots per cell (one tile: with two the search has as many empty tiles as full ones and
+/// loses more than the build gains) and the mean occupations between which it is tried. A cell that overflows voids
+/// the call's result (the packed build and the two passes start over) and the list stays away from it for long.
+constexpr uint32_t DIRECT_CAPACITY = TILE_POINTS;
+constexpr double DIRECT_MEAN_MIN = 10.0;
+constexpr double DIRECT_MEAN_MAX = 24.0;
+constexpr int DIRECT_REST = 1024;
+
 constexpr int SINGLE_PASS_REST = 64;
 constexpr int BOX_REST = 32;
 constexpr size_t BOX_BYTES = 75; // 9 doubles and 3 flags, as fetch_box lays them out
@@ -222,6 +237,7 @@ struct HipExtras {
     bool have_last_box = false;
     int box_rest = 0;                 // calls left before a changing box is assumed constant again
     int single_pass_rest = 0;         // calls left before the single-pass search is tried again after it did not fit
+    int direct_rest = 0;              // calls left before the one-pass cell build is tried again after a cell overflowed
     hipEvent_t events[T_STAGES] = {};
     bool have_events = false;
     bool timings_valid = false;
@@ -724,6 +740,30 @@ bool compute(
     uint32_t* counts = nullptr;
     uint64_t* offsets = nullptr;
     uint64_t* scan_scratch = nullptr;
+
+    // The single-pass search writes straight into the arrays kept from earlier calls. It does not cover every shape
+    // of problem and the rows may not fit: in both cases nothing is lost but time, the two passes start over.
+    bool try_single_pass = !options.sorted && extras.capacity > 0 && !two_pass_only();
+    if (try_single_pass && extras.single_pass_rest > 0) {
+        extras.single_pass_rest -= 1;
+        try_single_pass = false;
+    }
+    // Large systems with cells of ordinary occupation: the cells are built in one pass over the points, every cell
+    // owning DIRECT_CAPACITY slots (place_direct); only the single-pass search reads that layout.
+    bool direct_cells = try_single_pass && !single_cell && n_slices == 1 && !ordered_rows() && !packed_cells_only() &&
+                        static_cast<double>(n_points) <= DIRECT_MEAN_MAX * static_cast<double>(n_cells) &&
+                        static_cast<double>(n_points) >= DIRECT_MEAN_MIN * static_cast<double>(n_cells) &&
+                        n_cells * DIRECT_CAPACITY < 0xFFFFFF00ull;
+    if (direct_cells && extras.direct_rest > 0) {
+        extras.direct_rest -= 1;
+        direct_cells = false;
+    }
+    constexpr size_t direct_tiles_per_cell = DIRECT_CAPACITY / TILE_POINTS;
+    const size_t direct_slots =
+        direct_cells ? (n_cells * direct_tiles_per_cell + slot_multiple - 1) / slot_multiple * slot_multiple : 0;
+    const size_t sorted_slots = direct_cells ? std::max<size_t>(n_points, n_cells * DIRECT_CAPACITY) : n_points;
+    uint32_t* direct_wrapped = nullptr;
+
     // the search that produces a sorted list in order covers stencils that fit its tables
     const size_t full_stencil = static_cast<size_t>(2 * grid.s[0] + 1) * (2 * grid.s[1] + 1) * (2 * grid.s[2] + 1);
     const bool try_in_order = options.sorted && full_stencil <= MAX_ENTRIES && !radix_sort_only();
@@ -742,6 +782,7 @@ bool compute(
         chain.blocks = carver.take<uint64_t>(search_workgroups);
         chain.groups = carver.take<uint64_t>(chain_groups);
         chain.bases = carver.take<uint64_t>(chain_groups);
+        direct_wrapped = carver.take<uint32_t>(direct_slots);
         fused_status = carver.take<FusedStatus>(1);
         ordered_status = carver.take<OrderedStatus>(1);
         cell_scan = carver.take<uint64_t>(n_cells + 1);
@@ -751,15 +792,15 @@ bool compute(
             wrap_of = carver.take<int32_t>(3 * n_points);
             provisional = carver.take<uint32_t>(n_points);
         }
-        sorted.x = carver.take<double>(n_points + SORTED_PADDING);
-        sorted.y = carver.take<double>(n_points + SORTED_PADDING);
-        sorted.z = carver.take<double>(n_points + SORTED_PADDING);
-        sorted.index = carver.take<uint32_t>(n_points + SORTED_PADDING);
-        sorted.wx = carver.take<int32_t>(n_points);
-        sorted.wy = carver.take<int32_t>(n_points);
-        sorted.wz = carver.take<int32_t>(n_points);
-        counts = carver.take<uint32_t>(n_slots);
-        offsets = carver.take<uint64_t>(n_slots + 1);
+        sorted.x = carver.take<double>(sorted_slots + SORTED_PADDING);
+        sorted.y = carver.take<double>(sorted_slots + SORTED_PADDING);
+        sorted.z = carver.take<double>(sorted_slots + SORTED_PADDING);
+        sorted.index = carver.take<uint32_t>(sorted_slots + SORTED_PADDING);
+        sorted.wx = carver.take<int32_t>(sorted_slots);
+        sorted.wy = carver.take<int32_t>(sorted_slots);
+        sorted.wz = carver.take<int32_t>(sorted_slots);
+        counts = carver.take<uint32_t>(std::max(n_slots, direct_slots));
+        offsets = carver.take<uint64_t>(std::max(n_slots, direct_slots) + 1);
         scan_scratch = carver.take<uint64_t>(scratch_elements);
         if (try_in_order) {
             rows_of_point = carver.take<uint32_t>(n_points);
@@ -775,7 +816,7 @@ bool compute(
     // ---- cell list
     const uint32_t point_blocks = static_cast<uint32_t>((n_points + BLOCK - 1) / BLOCK);
     const auto* flat_points = reinterpret_cast<const double*>(points);
-    {
+    auto clear_work_state = [&]() {
         // every piece of the work buffer is padded to 256 bytes: clearing whole 16-byte blocks stays inside
         const size_t to_clear = reinterpret_cast<char*>(ordered_status + 1) - reinterpret_cast<char*>(cell_counts);
         const size_t blocks16 = (to_clear + 15) / 16;
@@ -786,13 +827,16 @@ bool compute(
             fetched ? static_cast<const double*>(nullptr) : reinterpret_cast<const double*>(box), periodic,
             extras.h_small, extras.d_status
         );
-    }
-    if (single_cell) {
-        hipLaunchKernelGGL(
-            prepare_single_cell, dim3(point_blocks), dim3(BLOCK), 0, stream,
-            flat_points, g, sorted, tiles, cell_scan, extras.d_status
-        );
-    } else {
+        fetched = true;
+    };
+    auto build_packed_cells = [&]() {
+        if (single_cell) {
+            hipLaunchKernelGGL(
+                prepare_single_cell, dim3(point_blocks), dim3(BLOCK), 0, stream,
+                flat_points, g, sorted, tiles, cell_scan, extras.d_status
+            );
+            return;
+        }
         const bool ordered = ordered_rows();
         hipLaunchKernelGGL(
             assign_cells, dim3(point_blocks), dim3(BLOCK), 0, stream,
@@ -818,6 +862,15 @@ bool compute(
                 static_cast<const uint32_t*>(nullptr), static_cast<const uint32_t*>(nullptr)
             );
         }
+    };
+    clear_work_state();
+    if (direct_cells) {
+        hipLaunchKernelGGL(
+            place_direct, dim3(point_blocks), dim3(BLOCK), 0, stream,
+            flat_points, g, DIRECT_CAPACITY, cell_counts, direct_wrapped, sorted, extras.d_status
+        );
+    } else {
+        build_packed_cells();
     }
     mark(T_CELLS);
 
@@ -854,13 +907,7 @@ bool compute(
         return ms;
     };
 
-    // ---- single-pass search straight into the arrays kept from earlier calls. It does not cover every shape of
-    // problem and the rows may not fit: in both cases nothing is lost but time, the two passes below start over.
-    bool try_single_pass = !options.sorted && extras.capacity > 0 && !two_pass_only();
-    if (try_single_pass && extras.single_pass_rest > 0) {
-        extras.single_pass_rest -= 1;
-        try_single_pass = false;
-    }
+    // ---- single-pass search straight into the arrays kept from earlier calls
     if (try_single_pass) {
         size_outputs(neighbors, extras, 0, options);
         FusedArgs fargs = {};
@@ -870,7 +917,14 @@ bool compute(
         fargs.chain = chain;
         fargs.first_rows = offsets;
         fargs.status = fused_status;
-        const uint32_t blocks = static_cast<uint32_t>(search_workgroups);
+        uint32_t blocks = static_cast<uint32_t>(search_workgroups);
+        if (direct_cells) {
+            fargs.search.direct_capacity = DIRECT_CAPACITY;
+            fargs.search.direct_counts = cell_counts;
+            fargs.search.direct_wrapped = direct_wrapped;
+            fargs.search.n_work = static_cast<uint32_t>(direct_slots);
+            blocks = static_cast<uint32_t>(direct_slots / SEARCH_WAVES);
+        }
         const bool ordered = ordered_rows();
         auto kernel = options.full ? (ordered ? fused_search_kernel<true, true> : fused_search_kernel<true, false>)
                                    : (ordered ? fused_search_kernel<false, true> : fused_search_kernel<false, false>);
@@ -887,15 +941,18 @@ bool compute(
         }
         if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
             std::fprintf(
-                stderr, "single pass: rows %llu general %u deferred %u overflow %u timeout %u (cells %u %u %u, capacity %zu)\n",
+                stderr,
+                "single pass: rows %llu general %u deferred %u overflow %u timeout %u (cells %u %u %u, capacity %zu, %s%u)\n",
                 result.total_rows, result.general, result.deferred, result.overflow, result.chain_timeout, g.n[0], g.n[1], g.n[2],
-                extras.capacity
+                extras.capacity, direct_cells ? "one-pass cell build, crowded " : "packed cells, crowded ", result.crowded_cells
             );
         }
         if (result.chain_timeout != 0) {
             throw std::runtime_error("internal error: the single-pass search gave up waiting for an earlier workgroup");
         }
-        if (result.general == 0 && result.overflow == 0) {
+        // the one-pass cell build is void when a cell overflowed, and the write pass cannot read its layout
+        const bool cells_ok = !direct_cells || (result.crowded_cells == 0 && result.deferred == 0);
+        if (result.general == 0 && result.overflow == 0 && cells_ok) {
             check_pair_limit(result.total_rows);
             if (result.deferred != 0) {
                 // work items too large for the single pass: their rows are counted and placed, the write pass of
@@ -925,6 +982,14 @@ bool compute(
         if (result.general != 0) {
             // the shape of this system is not the single-pass kernel's: leave it alone for a while
             extras.single_pass_rest = SINGLE_PASS_REST;
+        }
+        if (direct_cells) {
+            // everything below reads the packed layout: build it now
+            if (!cells_ok) {
+                extras.direct_rest = DIRECT_REST;
+            }
+            clear_work_state();
+            build_packed_cells();
         }
     }
 

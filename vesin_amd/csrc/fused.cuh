@@ -469,8 +469,13 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fa
     FusedWaveShared& sh = shared.wave[wave];
     GridParams batch_grid;
     const GridParams& g = BATCH ? batch_grid : single_grid;
+    // fixed-capacity layout (never in a batch): every cell has the same number of tiles, some of them empty
+    const uint32_t direct_capacity = BATCH ? 0 : args.direct_capacity;
+    const uint32_t direct_tiles = direct_capacity / TILE_POINTS;
     const uint32_t n_tiles =
-        static_cast<uint32_t>(args.cell_scan[BATCH ? args.total_cells : single_grid.n_cells] >> 32);
+        direct_capacity != 0
+            ? single_grid.n_cells * direct_tiles
+            : static_cast<uint32_t>(args.cell_scan[BATCH ? args.total_cells : single_grid.n_cells] >> 32);
     const uint32_t work = blockIdx.x * SEARCH_WAVES + wave;
     const SortedPoints& sorted = args.sorted;
 
@@ -503,8 +508,21 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fa
         const uint32_t within = BATCH ? slot : (slot / (SEARCH_WAVES * N_XCD)) * SEARCH_WAVES + slot % SEARCH_WAVES;
         const uint32_t tile_id = xcd * per_xcd + within;
 
+        Tile tile = {};
         if (within < per_xcd && tile_id < n_tiles) {
-            const Tile tile = args.tiles[tile_id];
+            if (direct_capacity != 0) {
+                const uint32_t cell = tile_id / direct_tiles;
+                const uint32_t k = tile_id % direct_tiles;
+                const uint32_t in_cell = min(args.direct_counts[cell], direct_capacity);
+                tile.cell = cell;
+                tile.first = cell * direct_capacity + k * TILE_POINTS;
+                tile.count = in_cell > k * TILE_POINTS ? min(static_cast<uint32_t>(TILE_POINTS), in_cell - k * TILE_POINTS) : 0;
+                tile.wrapped = args.direct_wrapped[tile_id];
+            } else {
+                tile = args.tiles[tile_id];
+            }
+        }
+        if (tile.count != 0) {
             item.n_i = tile.count;
             item.first_i = tile.first;
             item.tile_wrapped = (tile.wrapped & 1u) != 0;
@@ -540,7 +558,9 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fa
                     sh.tile_wz[lane] = sorted.wz[at];
                 }
                 item.n_batch = n_entries;
-                fill_stencil_tables(sh, lane, centre, n_entries, cx, cy, cz, span_y, span_z, g, cell_scan);
+                fill_stencil_tables(
+                    sh, lane, centre, n_entries, cx, cy, cz, span_y, span_z, g, cell_scan, args.direct_counts, direct_capacity
+                );
                 item.n_candidates = __builtin_amdgcn_readfirstlane(sh.n_candidates);
 
                 const uint32_t n_groups = (item.n_candidates + WAVE * R - 1) / (WAVE * R);

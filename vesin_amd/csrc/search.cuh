@@ -73,6 +73,10 @@ struct SearchArgs {
                                // N_XCD * SEARCH_WAVES and at least the number of tiles
     uint64_t capacity;         // WRITE: rows the output arrays hold; a launch that would overflow writes nothing
     const uint32_t* only;      // WRITE: when not null, only work items with a non-zero entry are processed
+    // fixed-capacity layout of the cells (place_direct), understood by the single-pass search only; 0 otherwise
+    uint32_t direct_capacity;  // slots per cell, a multiple of TILE_POINTS
+    const uint32_t* direct_counts;  // points of every cell
+    const uint32_t* direct_wrapped; // per tile: holds a point that was moved by a box vector
     // many systems in one launch (batched entry point); null / zero otherwise
     const GridParams* grids;   // one per system
     const uint32_t* cell_base; // first cell of every system in the concatenated grids, n_systems + 1 entries
@@ -169,7 +173,8 @@ __device__ __forceinline__ void wave_sync() {
 /// offsets run dx major, dz minor.
 __device__ __forceinline__ void fill_stencil_tables(
     SearchTables& sh, int lane, uint32_t first_linear, uint32_t n_batch, int32_t cx, int32_t cy, int32_t cz,
-    int32_t span_y, int32_t span_z, const GridParams& g, const uint64_t* __restrict__ cell_scan
+    int32_t span_y, int32_t span_z, const GridParams& g, const uint64_t* __restrict__ cell_scan,
+    const uint32_t* __restrict__ direct_counts = nullptr, uint32_t direct_capacity = 0
 ) {
     const uint32_t centre = static_cast<uint32_t>(2 * g.s[0] + 1) * span_y * span_z / 2;
     for (uint32_t e = lane; e < n_batch; e += WAVE) {
@@ -220,8 +225,13 @@ __device__ __forceinline__ void fill_stencil_tables(
         int32_t packed = 0;
         if (valid) {
             uint32_t neighbour = (static_cast<uint32_t>(cell[2]) * g.n[1] + cell[1]) * g.n[0] + cell[0];
-            start = static_cast<uint32_t>(cell_scan[neighbour]);
-            count = static_cast<uint32_t>(cell_scan[neighbour + 1]) - start;
+            if (direct_capacity != 0) {
+                start = neighbour * direct_capacity;
+                count = min(direct_counts[neighbour], direct_capacity);
+            } else {
+                start = static_cast<uint32_t>(cell_scan[neighbour]);
+                count = static_cast<uint32_t>(cell_scan[neighbour + 1]) - start;
+            }
             packed = pack_shift(q[0], q[1], q[2]);
             if (linear == centre) {
                 packed |= 1 << 30;
