@@ -748,9 +748,9 @@ bool compute(
         extras.single_pass_rest -= 1;
         try_single_pass = false;
     }
-    // Large systems with cells of ordinary occupation: the cells are built in one pass over the points, every cell
-    // owning DIRECT_CAPACITY slots (place_direct); only the single-pass search reads that layout.
-    bool direct_cells = try_single_pass && !single_cell && n_slices == 1 && !ordered_rows() && !packed_cells_only() &&
+    // Cells of ordinary occupation: the cells are built in one pass over the points, every cell owning
+    // DIRECT_CAPACITY slots (place_direct); only the single-pass search reads that layout.
+    bool direct_cells = try_single_pass && !single_cell && !ordered_rows() && !packed_cells_only() &&
                         static_cast<double>(n_points) <= DIRECT_MEAN_MAX * static_cast<double>(n_cells) &&
                         static_cast<double>(n_points) >= DIRECT_MEAN_MIN * static_cast<double>(n_cells) &&
                         n_cells * DIRECT_CAPACITY < 0xFFFFFF00ull;
@@ -799,8 +799,8 @@ bool compute(
         sorted.wx = carver.take<int32_t>(sorted_slots);
         sorted.wy = carver.take<int32_t>(sorted_slots);
         sorted.wz = carver.take<int32_t>(sorted_slots);
-        counts = carver.take<uint32_t>(std::max(n_slots, direct_slots));
-        offsets = carver.take<uint64_t>(std::max(n_slots, direct_slots) + 1);
+        counts = carver.take<uint32_t>(std::max(n_slots, direct_slots * n_slices));
+        offsets = carver.take<uint64_t>(std::max(n_slots, direct_slots * n_slices) + 1);
         scan_scratch = carver.take<uint64_t>(scratch_elements);
         if (try_in_order) {
             rows_of_point = carver.take<uint32_t>(n_points);
@@ -922,8 +922,8 @@ bool compute(
             fargs.search.direct_capacity = DIRECT_CAPACITY;
             fargs.search.direct_counts = cell_counts;
             fargs.search.direct_wrapped = direct_wrapped;
-            fargs.search.n_work = static_cast<uint32_t>(direct_slots);
-            blocks = static_cast<uint32_t>(direct_slots / SEARCH_WAVES);
+            fargs.search.n_work = static_cast<uint32_t>(direct_slots * n_slices);
+            blocks = static_cast<uint32_t>(direct_slots * n_slices / SEARCH_WAVES);
         }
         const bool ordered = ordered_rows();
         auto kernel = options.full ? (ordered ? fused_search_kernel<true, true> : fused_search_kernel<true, false>)
