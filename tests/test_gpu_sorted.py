@@ -115,3 +115,25 @@ def test_few_points(n_points, capfd, monkeypatch):
     points = rng.random((n_points, 3)) @ box
     _check(points, box, True, 2.9, True, capfd, monkeypatch, "used")
     _check(points, box, False, 2.9, False, capfd, monkeypatch, "used")
+
+
+def test_a_system_that_search_does_not_cover_is_not_asked_again(capfd, monkeypatch):
+    import torch
+
+    rng = np.random.default_rng(31)
+    points = rng.random((4000, 3)) * 9.0
+    box = np.diag([9.0, 9.0, 9.0])
+    expected = oracle.canonicalize(oracle.neighbors(points, box, [True] * 3, 3.0, False, False, "ijSdD"))
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    calculator = NeighborList(cutoff=3.0, full_list=False, sorted=True)
+    device_points = torch.tensor(points, device="cuda:0")
+    device_box = torch.tensor(box, device="cuda:0")
+    tried = []
+    for _ in range(3):
+        capfd.readouterr()
+        P, S, d = calculator.compute(device_points, device_box, True, "PSd")
+        tried.append(any(line.startswith("in-order search:") for line in capfd.readouterr().err.splitlines()))
+        assert np.array_equal(P.cpu().numpy(), expected["pairs"])
+        assert np.array_equal(S.cpu().numpy(), expected["shifts"])
+        assert np.array_equal(d.cpu().numpy(), expected["distances"])
+    assert tried == [True, False, False]

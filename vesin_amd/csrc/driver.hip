@@ -238,6 +238,7 @@ struct HipExtras {
     int box_rest = 0;                 // calls left before a changing box is assumed constant again
     int single_pass_rest = 0;         // calls left before the single-pass search is tried again after it did not fit
     int direct_rest = 0;              // calls left before the one-pass cell build is tried again after a cell overflowed
+    int in_order_rest = 0;            // calls left before the in-order search is tried again on a system it did not cover
     hipEvent_t events[T_STAGES] = {};
     bool have_events = false;
     bool timings_valid = false;
@@ -766,7 +767,11 @@ bool compute(
 
     // the search that produces a sorted list in order covers stencils that fit its tables
     const size_t full_stencil = static_cast<size_t>(2 * grid.s[0] + 1) * (2 * grid.s[1] + 1) * (2 * grid.s[2] + 1);
-    const bool try_in_order = options.sorted && full_stencil <= MAX_ENTRIES && !radix_sort_only();
+    bool try_in_order = options.sorted && full_stencil <= MAX_ENTRIES && !radix_sort_only();
+    if (try_in_order && extras.in_order_rest > 0) {
+        extras.in_order_rest -= 1;
+        try_in_order = false;
+    }
     OrderedStatus* ordered_status = nullptr;
     uint32_t* rows_of_point = nullptr;
     uint64_t* first_row_of_point = nullptr;
@@ -1070,7 +1075,9 @@ bool compute(
             }
             return true;
         }
-        // rows per point, candidates per tile or shifts beyond what that search handles: the general way below
+        // rows per point, candidates per tile or shifts beyond what that search handles: the general way below,
+        // and for a while without asking again
+        extras.in_order_rest = SINGLE_PASS_REST;
     }
 
     // ---- pass 1: count

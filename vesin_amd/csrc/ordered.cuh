@@ -60,7 +60,8 @@ struct OrderedWaveShared: SearchTables {
     double tile_x[TILE_POINTS], tile_y[TILE_POINTS], tile_z[TILE_POINTS];
     int32_t tile_wx[TILE_POINTS], tile_wy[TILE_POINTS], tile_wz[TILE_POINTS];
     uint64_t tile_row[TILE_POINTS];   // WRITE: first output row of each point
-    uint64_t keys[ORDERED_MAX_ROWS];  // WRITE: (second point << 32) | biased shift, rows of one point
+    // WRITE: (second point << 32) | biased shift, rows of one point; read four at a time, hence the padding
+    __attribute__((aligned(16))) uint64_t keys[ORDERED_MAX_ROWS + 4];
     uint32_t key_at[ORDERED_MAX_ROWS];// WRITE: position of the second point in the cell-sorted arrays
 };
 
@@ -333,6 +334,9 @@ __global__ __launch_bounds__(ORDERED_BLOCK) void ordered_search_kernel(OrderedAr
         if (n_rows == 0) {
             continue;
         }
+        if (lane < 4) {
+            sh.keys[n_rows + lane] = ~0ull; // larger than any key: the ranking reads whole groups of four
+        }
         wave_sync();
 
         const double xi = sh.tile_x[p];
@@ -350,8 +354,12 @@ __global__ __launch_bounds__(ORDERED_BLOCK) void ordered_search_kernel(OrderedAr
             const double yj = sorted.y[at];
             const double zj = sorted.z[at];
             uint32_t rank = 0;
-            for (uint32_t other = 0; other < n_rows; other++) {
-                rank += sh.keys[other] < key ? 1u : 0u;
+            for (uint32_t other = 0; other < n_rows; other += 4) {
+                // every lane reads the same 32 bytes: two LDS broadcasts for four comparisons
+                const ulonglong2 first_two = *reinterpret_cast<const ulonglong2*>(&sh.keys[other]);
+                const ulonglong2 next_two = *reinterpret_cast<const ulonglong2*>(&sh.keys[other + 2]);
+                rank += (first_two.x < key ? 1u : 0u) + (first_two.y < key ? 1u : 0u);
+                rank += (next_two.x < key ? 1u : 0u) + (next_two.y < key ? 1u : 0u);
             }
             if (active) {
                 const uint32_t oj = static_cast<uint32_t>(key >> 32);
