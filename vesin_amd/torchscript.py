@@ -35,16 +35,9 @@ load_torch_library()
 
 
 class NeighborList:
-    """A neighbor list calculator that can be used with TorchScript."""
+    """Calculator usable from TorchScript code; thin front of ``torch.classes.vesin._NeighborList``."""
 
-    def __init__(
-        self,
-        cutoff: float,
-        full_list: bool,
-        sorted: bool = False,
-        algorithm: str = "auto",
-        n_threads: int = 0,
-    ):
+    def __init__(self, cutoff: float, full_list: bool, sorted: bool = False, algorithm: str = "auto", n_threads: int = 0):
         """
         :param cutoff: spherical cutoff
         :param full_list: return every pair twice (``i-j`` and ``j-i``) or once
@@ -53,17 +46,9 @@ class NeighborList:
             covers every case on the GPU
         :param n_threads: accepted for compatibility, must be zero or positive
         """
-        n_threads = int(n_threads)
-        if n_threads < 0:
+        if int(n_threads) < 0:
             raise ValueError("n_threads must be zero or a positive integer")
-
-        self._c = torch.classes.vesin._NeighborList(
-            cutoff=cutoff,
-            full_list=full_list,
-            sorted=sorted,
-            algorithm=algorithm,
-            n_threads=n_threads,
-        )
+        self._c = torch.classes.vesin._NeighborList(cutoff, full_list, sorted, algorithm, int(n_threads))
 
     def compute(
         self,
@@ -76,29 +61,21 @@ class NeighborList:
         """
         Neighbor list of ``points`` in ``box``; ``quantities`` is any combination of ``i``, ``j``, ``P`` (both
         indices), ``S`` (shifts), ``d`` (distances), ``D`` (vectors). With ``copy=False`` the tensors are views of
-        memory the calculator owns, valid until its next calculation.
+        memory the calculator owns, valid until its next calculation (outputs that carry gradients are always
+        copies). The library computes in float64: other floating-point inputs are converted on the way in, and
+        distances and vectors come back in the dtype of ``points``.
         """
-        if isinstance(periodic, bool):
-            periodic = torch.as_tensor(periodic)
+        dtype = points.dtype
+        if box.dtype != dtype:
+            raise RuntimeError(f"`points` and `box` must have the same dtype, got {points.dtype} and {box.dtype}")
+        flags = torch.as_tensor(periodic) if isinstance(periodic, bool) else periodic
 
-        initial_dtype = points.dtype
-        if box.dtype != initial_dtype:
-            raise RuntimeError(
-                f"`points` and `box` must have the same dtype, got {points.dtype} and {box.dtype}"
-            )
-
-        results = self._c.compute(
-            points=points.to(torch.float64),
-            box=box.to(torch.float64),
-            periodic=periodic,
-            quantities=quantities,
-            copy=copy,
-        )
-
-        converted: List[torch.Tensor] = []
-        for index, result in enumerate(results):
-            letter = quantities[index]
-            if letter == "d" or letter == "D":
-                result = result.to(initial_dtype)
-            converted.append(result)
-        return converted
+        outputs = self._c.compute(points.to(torch.float64), box.to(torch.float64), flags, quantities, copy)
+        if dtype == torch.float64:
+            return outputs
+        back: List[torch.Tensor] = []
+        for position in range(len(outputs)):
+            letter = quantities[position]
+            tensor = outputs[position]
+            back.append(tensor.to(dtype) if letter in ("d", "D") else tensor)
+        return back
