@@ -232,6 +232,53 @@ __global__ __launch_bounds__(ORDERED_BLOCK) void ordered_search_kernel(OrderedAr
         return; // the host does not use this path for such a tile: nothing to count, nothing may be written
     }
 
+    if constexpr (!WRITE) {
+        // ---- COUNT: nothing is kept but the number of rows of every point (lane p adds up the hits of point p):
+        // a plain loop over the pairs of units, small code
+        uint32_t own_rows = 0;
+        for (uint32_t unit0 = 0; unit0 < n_units; unit0 += R) {
+            uint32_t column[R], at[R], original[R];
+            int32_t packed_b[R];
+            if (tile_wrapped) {
+                ordered_sweep_pair<FULL, true>(
+                    sh, sorted, g, unit0, n_stencil, n_candidates, first_i, n_i, lane, column, at, original, packed_b,
+                    out_of_range
+                );
+            } else {
+                ordered_sweep_pair<FULL, false>(
+                    sh, sorted, g, unit0, n_stencil, n_candidates, first_i, n_i, lane, column, at, original, packed_b,
+                    out_of_range
+                );
+            }
+            for (uint32_t p = 0; p < n_i; p++) {
+                const uint32_t bit = n_i - 1 - p;
+                uint32_t rows = 0;
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    rows += __popcll(__ballot(((column[r] >> bit) & 1u) != 0));
+                }
+                if (static_cast<uint32_t>(lane) == p) {
+                    own_rows += rows;
+                }
+            }
+        }
+        if (static_cast<uint32_t>(lane) < n_i) {
+            args.rows_of_point[sh.tile_index[lane]] = own_rows;
+        }
+        uint32_t most = own_rows;
+#pragma unroll
+        for (int offset = 32; offset > 0; offset >>= 1) {
+            most = max(most, static_cast<uint32_t>(__shfl_xor(static_cast<int>(most), offset, WAVE)));
+        }
+        if (lane == 0) {
+            atomicMax(&args.status->max_rows, most);
+        }
+        if (__ballot(out_of_range) != 0 && lane == 0) {
+            atomicAdd(&args.status->unsuitable, 1u);
+        }
+        return;
+    }
+
     // ---- sweep: per candidate (registers of its lane, indexed by unit) the hit column against this item's points
     uint32_t columns[ORDERED_UNITS];
     uint32_t cand_at[ORDERED_UNITS];
@@ -270,39 +317,6 @@ __global__ __launch_bounds__(ORDERED_BLOCK) void ordered_search_kernel(OrderedAr
                 }
             }
         }
-    }
-
-    if (!WRITE) {
-        // rows of every point of the item: lane p adds up the bits of point p over all candidates
-        uint32_t own_rows = 0;
-        for (uint32_t p = 0; p < n_i; p++) {
-            const uint32_t bit = n_i - 1 - p;
-            uint32_t rows = 0;
-#pragma unroll
-            for (int u = 0; u < ORDERED_UNITS; u++) {
-                if (static_cast<uint32_t>(u) < n_units) {
-                    rows += __popcll(__ballot(((columns[u] >> bit) & 1u) != 0));
-                }
-            }
-            if (static_cast<uint32_t>(lane) == p) {
-                own_rows = rows;
-            }
-        }
-        if (static_cast<uint32_t>(lane) < n_i) {
-            args.rows_of_point[sh.tile_index[lane]] = own_rows;
-        }
-        uint32_t most = own_rows;
-#pragma unroll
-        for (int offset = 32; offset > 0; offset >>= 1) {
-            most = max(most, static_cast<uint32_t>(__shfl_xor(static_cast<int>(most), offset, WAVE)));
-        }
-        if (lane == 0) {
-            atomicMax(&args.status->max_rows, most);
-        }
-        if (__ballot(out_of_range) != 0 && lane == 0) {
-            atomicAdd(&args.status->unsuitable, 1u);
-        }
-        return;
     }
 
     // ---- WRITE: point by point, collect the hits, rank them, store the rows
