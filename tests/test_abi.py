@@ -122,3 +122,69 @@ def test_free_accepts_null_and_zeroed_lists():
     neighbors = _c_api.VesinNeighborList()
     lib.vesin_free(ctypes.byref(neighbors))
     assert neighbors.length == 0 and neighbors.pairs is None
+
+
+def test_validation_of_the_additions():
+    """The entry points this library adds check their arguments like vesin_neighbors does, before any GPU work."""
+    lib = _c_api.get_library()
+    dummy = (ctypes.c_double * 16)()
+    address = ctypes.addressof(dummy)
+    gpu = _c_api.VesinDevice(_c_api.VesinCUDA, 0)
+    cpu = _c_api.VesinDevice(_c_api.VesinCPU, 0)
+    options = _c_api.VesinOptions()
+    options.cutoff = 1.0
+
+    def text(message):
+        return message.value.decode() if message.value else None
+
+    # the calculation on a stream: same checks, same texts
+    neighbors = _c_api.VesinNeighborList()
+    message = ctypes.c_char_p()
+    status = lib.vesin_hip_neighbors_on_stream(
+        None, 1, address, address, gpu, options, ctypes.byref(neighbors), None, ctypes.byref(message)
+    )
+    assert (status, text(message)) == (1, "`points` can not be a NULL pointer")
+    bad = _c_api.VesinOptions()
+    bad.cutoff = -2.0
+    message = ctypes.c_char_p()
+    status = lib.vesin_hip_neighbors_on_stream(
+        address, 1, address, address, gpu, bad, ctypes.byref(neighbors), None, ctypes.byref(message)
+    )
+    assert (status, text(message)) == (1, "cutoff must be a finite, positive number")
+    assert lib.vesin_hip_neighbors_on_stream(address, 1, address, address, gpu, options, ctypes.byref(neighbors), None, None) == 1
+
+    # the gradient
+    message = ctypes.c_char_p()
+    status = lib.vesin_hip_pairs_backward(
+        address, None, None, None, 1, None, address, 1, cpu, address, None, None, ctypes.byref(message)
+    )
+    assert status == 1 and "only computed on a GPU device" in text(message)
+    message = ctypes.c_char_p()
+    status = lib.vesin_hip_pairs_backward(
+        address, None, None, None, 0, None, address, 1, gpu, address, None, None, ctypes.byref(message)
+    )
+    assert (status, text(message)) == (0, None)  # no rows: nothing to do, no device needed
+    assert lib.vesin_hip_pairs_backward(address, None, None, None, 1, None, address, 1, gpu, address, None, None, None) == 1
+
+    # the batch
+    first_point = (ctypes.c_size_t * 2)(0, 1)
+    first_pair = (ctypes.c_size_t * 2)()
+    message = ctypes.c_char_p()
+    status = lib.vesin_hip_neighbors_batch(
+        address, None, 1, address, address, gpu, options, ctypes.byref(neighbors), first_pair, ctypes.byref(message)
+    )
+    assert (status, text(message)) == (1, "`first_point` can not be a NULL pointer")
+    message = ctypes.c_char_p()
+    status = lib.vesin_hip_neighbors_batch(
+        address, first_point, 1, address, address, cpu, options, ctypes.byref(neighbors), first_pair, ctypes.byref(message)
+    )
+    assert status == 1 and "only computed on a GPU device" in text(message)
+    with_skin = _c_api.VesinOptions()
+    with_skin.cutoff = 1.0
+    with_skin.skin = 0.2
+    message = ctypes.c_char_p()
+    status = lib.vesin_hip_neighbors_batch(
+        address, first_point, 1, address, address, gpu, with_skin, ctypes.byref(neighbors), first_pair, ctypes.byref(message)
+    )
+    assert status == 1 and "not available for a batch" in text(message)
+    lib.vesin_free(ctypes.byref(neighbors))
