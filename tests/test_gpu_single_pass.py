@@ -273,3 +273,23 @@ def test_one_pass_cell_build_with_a_cell_too_full(capfd, monkeypatch):
     assert_same_list(call(calculator, points, box, periodic), expected, what="next call")
     reports = _single_pass_reports(capfd)
     assert reports and "packed cells" in reports[-1], reports
+
+
+@pytest.mark.parametrize("n_points", [1, 31, 33, 700, 2048, 2049])
+@pytest.mark.parametrize("periodic", [(True, True, True), (True, False, True)])
+def test_cell_build_of_small_systems(n_points, periodic, monkeypatch):
+    """Up to 2048 points the packed cell build is one launch of one workgroup (above, and with
+    VESIN_HIP_CELLS=packed, the four launches): same rows, first call and reused list, points outside the box
+    included."""
+    rng = np.random.default_rng(n_points)
+    box = np.array([[13.0, 0.0, 0.0], [1.5, 12.0, 0.0], [-1.0, 0.8, 14.0]])
+    points = rng.random((n_points, 3)) @ box + (rng.integers(-1, 2, size=(n_points, 3)) * (rng.random((n_points, 1)) < 0.2)) @ box
+    expected = oracle.neighbors(points, box, list(periodic), 3.0, True, False, "ijSdD")
+    for mode in ("default", "packed"):
+        if mode == "packed":
+            monkeypatch.setenv("VESIN_HIP_CELLS", "packed")
+        else:
+            monkeypatch.delenv("VESIN_HIP_CELLS", raising=False)
+        calculator = NeighborList(cutoff=3.0, full_list=True)
+        for repeat in range(3):
+            assert_same_list(call(calculator, points, box, list(periodic)), expected, what=f"{mode} call {repeat}")

@@ -598,6 +598,143 @@ __global__ __launch_bounds__(BLOCK) void gather_points(
     }
 }
 
+/// The whole cell build of a small system in one launch of one workgroup, so that a call is three launches instead
+/// of seven: clears the work state (`clear`, whole 16-byte blocks), fetches the box when `box` is not null, then
+/// histogram (LDS atomics), scan of points and tiles per cell, and placement into the packed layout with its tile
+/// list - what clear_and_fetch, assign_cells, the scan and place_points do for systems of any size. The slot of a
+/// point inside its cell is the one the atomic handed out, as with place_points.
+constexpr uint32_t SMALL_BUILD_THREADS = 1024;
+constexpr uint32_t SMALL_BUILD_POINTS = 2 * SMALL_BUILD_THREADS; // points and cells one workgroup takes (beyond
+                                                                 // about 2500 points the four launches win)
+constexpr uint32_t SMALL_BUILD_PER_THREAD = SMALL_BUILD_POINTS / SMALL_BUILD_THREADS;
+
+__global__ __launch_bounds__(SMALL_BUILD_THREADS) void build_cells_small(
+    const double* __restrict__ points, GridParams g, uint4* __restrict__ clear, size_t clear_blocks16,
+    const double* __restrict__ box, const bool* __restrict__ periodic, unsigned char* host_small,
+    SortedPoints sorted, Tile* __restrict__ tiles, uint64_t* __restrict__ cell_scan, DeviceStatus* status
+) {
+    __shared__ uint32_t cell_count[SMALL_BUILD_POINTS];
+    __shared__ uint64_t cell_first[SMALL_BUILD_POINTS]; // points before the cell | tiles before it << 32
+    __shared__ uint64_t wave_totals[SMALL_BUILD_THREADS / WAVE];
+    const uint32_t t = threadIdx.x;
+    const int lane = lane_id();
+    const uint32_t wave = t / WAVE;
+
+    if (box != nullptr) {
+        if (t < 9) {
+            reinterpret_cast<double*>(host_small)[t] = box[t];
+        } else if (t < 12) {
+            host_small[72 + (t - 9)] = periodic[t - 9] ? 1 : 0;
+        } else if (t == 12) {
+            status->total_pairs = 0;
+            status->first_bad_coordinate = 0xFFFFFFFFu;
+            status->crowded_cells = 0;
+        }
+    }
+    const uint4 zero = {0u, 0u, 0u, 0u};
+    for (size_t k = t; k < clear_blocks16; k += SMALL_BUILD_THREADS) {
+        clear[k] = zero;
+    }
+    for (uint32_t c = t; c < g.n_cells; c += SMALL_BUILD_THREADS) {
+        cell_count[c] = 0;
+    }
+    __syncthreads();
+
+    // ---- histogram: the slot inside the cell comes back from the LDS atomic
+    double x[SMALL_BUILD_PER_THREAD], y[SMALL_BUILD_PER_THREAD], z[SMALL_BUILD_PER_THREAD];
+    uint32_t cell_of[SMALL_BUILD_PER_THREAD], slot_of[SMALL_BUILD_PER_THREAD];
+    int32_t wx[SMALL_BUILD_PER_THREAD], wy[SMALL_BUILD_PER_THREAD], wz[SMALL_BUILD_PER_THREAD];
+#pragma unroll
+    for (uint32_t k = 0; k < SMALL_BUILD_PER_THREAD; k++) {
+        const uint32_t i = k * SMALL_BUILD_THREADS + t;
+        cell_of[k] = 0;
+        slot_of[k] = 0;
+        wx[k] = wy[k] = wz[k] = 0;
+        x[k] = y[k] = z[k] = 0.0;
+        if (i < g.n_points) {
+            x[k] = points[3 * static_cast<size_t>(i) + 0];
+            y[k] = points[3 * static_cast<size_t>(i) + 1];
+            z[k] = points[3 * static_cast<size_t>(i) + 2];
+            int32_t where[3] = {0, 0, 0};
+            int32_t wrap[3] = {0, 0, 0};
+            unsigned int axis;
+            if (all_finite(x[k], y[k], z[k], axis)) {
+                locate(g, x[k], y[k], z[k], where, wrap);
+            } else {
+                atomicMin(&status->first_bad_coordinate, 3u * i + axis);
+            }
+            cell_of[k] = (static_cast<uint32_t>(where[2]) * g.n[1] + where[1]) * g.n[0] + where[0];
+            wx[k] = wrap[0];
+            wy[k] = wrap[1];
+            wz[k] = wrap[2];
+            slot_of[k] = atomicAdd(&cell_count[cell_of[k]], 1u);
+        }
+    }
+    __syncthreads();
+
+    // ---- exclusive scan over the cells of (points, tiles), both in one 64-bit word
+    uint64_t mine[SMALL_BUILD_PER_THREAD];
+    uint64_t own_total = 0;
+#pragma unroll
+    for (uint32_t k = 0; k < SMALL_BUILD_PER_THREAD; k++) {
+        const uint32_t c = t * SMALL_BUILD_PER_THREAD + k;
+        const uint32_t count = c < g.n_cells ? cell_count[c] : 0;
+        const uint64_t n_tiles = (count + TILE_POINTS - 1) / TILE_POINTS;
+        mine[k] = own_total;
+        own_total += static_cast<uint64_t>(count) | (n_tiles << 32);
+    }
+    const uint64_t inclusive = wave_inclusive_scan(own_total);
+    if (lane == WAVE - 1) {
+        wave_totals[wave] = inclusive;
+    }
+    __syncthreads();
+    uint64_t before = inclusive - own_total;
+    for (uint32_t w = 0; w < wave; w++) {
+        before += wave_totals[w];
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < SMALL_BUILD_PER_THREAD; k++) {
+        const uint32_t c = t * SMALL_BUILD_PER_THREAD + k;
+        if (c < g.n_cells) {
+            cell_first[c] = before + mine[k];
+            cell_scan[c] = before + mine[k];
+        }
+    }
+    if (t == SMALL_BUILD_THREADS - 1) {
+        cell_scan[g.n_cells] = before + own_total;
+    }
+    __syncthreads();
+
+    // ---- placement and tile list
+#pragma unroll
+    for (uint32_t k = 0; k < SMALL_BUILD_PER_THREAD; k++) {
+        const uint32_t i = k * SMALL_BUILD_THREADS + t;
+        if (i < g.n_points) {
+            const uint64_t here = cell_first[cell_of[k]];
+            const uint32_t start = static_cast<uint32_t>(here);
+            const uint32_t first_tile = static_cast<uint32_t>(here >> 32);
+            const uint32_t count = cell_count[cell_of[k]];
+            const uint32_t to = start + slot_of[k];
+            sorted.index[to] = i;
+            sorted.x[to] = x[k];
+            sorted.y[to] = y[k];
+            sorted.z[to] = z[k];
+            sorted.wx[to] = wx[k];
+            sorted.wy[to] = wy[k];
+            sorted.wz[to] = wz[k];
+            Tile* tile = &tiles[first_tile + slot_of[k] / TILE_POINTS];
+            if ((wx[k] | wy[k] | wz[k]) != 0) {
+                atomicOr(&tile->wrapped, 1u);
+            }
+            if (slot_of[k] % TILE_POINTS == 0) {
+                tile->cell = cell_of[k];
+                tile->first = to;
+                tile->count = min(TILE_POINTS, count - slot_of[k]);
+            }
+        }
+    }
+}
+
 /// The single-cell layout used by the brute-force / multi-image path: points keep their order, the one cell
 /// holds all of them, tiles are consecutive blocks of 64 points. Also performs the non-finite check.
 __global__ __launch_bounds__(BLOCK) void prepare_single_cell(

@@ -759,6 +759,12 @@ bool compute(
         extras.direct_rest -= 1;
         direct_cells = false;
     }
+    // small systems: the whole packed cell build, clearing and box fetch included, is one launch of one workgroup
+    const bool small_build = !single_cell && !ordered_rows() && n_points <= SMALL_BUILD_POINTS &&
+                             n_cells <= SMALL_BUILD_POINTS && std::getenv("VESIN_HIP_CELLS") == nullptr;
+    if (small_build) {
+        direct_cells = false;
+    }
     constexpr size_t direct_tiles_per_cell = DIRECT_CAPACITY / TILE_POINTS;
     const size_t direct_slots =
         direct_cells ? (n_cells * direct_tiles_per_cell + slot_multiple - 1) / slot_multiple * slot_multiple : 0;
@@ -868,13 +874,23 @@ bool compute(
             );
         }
     };
-    clear_work_state();
-    if (direct_cells) {
+    if (small_build) {
+        const size_t to_clear = reinterpret_cast<char*>(ordered_status + 1) - reinterpret_cast<char*>(cell_counts);
+        hipLaunchKernelGGL(
+            build_cells_small, dim3(1), dim3(SMALL_BUILD_THREADS), 0, stream,
+            flat_points, g, reinterpret_cast<uint4*>(cell_counts), (to_clear + 15) / 16,
+            fetched ? static_cast<const double*>(nullptr) : reinterpret_cast<const double*>(box), periodic,
+            extras.h_small, sorted, tiles, cell_scan, extras.d_status
+        );
+        fetched = true;
+    } else if (direct_cells) {
+        clear_work_state();
         hipLaunchKernelGGL(
             place_direct, dim3(point_blocks), dim3(BLOCK), 0, stream,
             flat_points, g, DIRECT_CAPACITY, cell_counts, direct_wrapped, sorted, extras.d_status
         );
     } else {
+        clear_work_state();
         build_packed_cells();
     }
     mark(T_CELLS);
