@@ -737,10 +737,36 @@ __global__ __launch_bounds__(SMALL_BUILD_THREADS) void build_cells_small(
 
 /// The single-cell layout used by the brute-force / multi-image path: points keep their order, the one cell
 /// holds all of them, tiles are consecutive blocks of 64 points. Also performs the non-finite check.
+/// When `clear` is given (launches of a single workgroup only), it also clears that part of the work state (the
+/// state of the search kernels: the tile list is written here in full and needs no clearing), fetches the box and
+/// resets the status like fetch_box does: a call on this layout then starts with one launch instead of two.
 __global__ __launch_bounds__(BLOCK) void prepare_single_cell(
     const double* __restrict__ points, GridParams g, SortedPoints sorted, Tile* __restrict__ tiles,
-    uint64_t* __restrict__ cell_scan, DeviceStatus* status
+    uint64_t* __restrict__ cell_scan, DeviceStatus* status, uint4* __restrict__ clear = nullptr,
+    size_t clear_blocks16 = 0, const double* __restrict__ box = nullptr, const bool* __restrict__ periodic = nullptr,
+    unsigned char* host_small = nullptr
 ) {
+    if (blockIdx.x == 0) {
+        const int t = threadIdx.x;
+        if (box != nullptr) {
+            if (t < 9) {
+                reinterpret_cast<double*>(host_small)[t] = box[t];
+            } else if (t < 12) {
+                host_small[72 + (t - 9)] = periodic[t - 9] ? 1 : 0;
+            } else if (t == 12) {
+                status->total_pairs = 0;
+                status->first_bad_coordinate = 0xFFFFFFFFu;
+                status->crowded_cells = 0;
+            }
+        }
+        const uint4 zero = {0u, 0u, 0u, 0u};
+        for (size_t k = t; k < clear_blocks16; k += BLOCK) {
+            clear[k] = zero;
+        }
+        if (clear != nullptr) {
+            __syncthreads(); // the status is reset before any thread reports into it: one workgroup only
+        }
+    }
     uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
     const uint32_t n_tiles = (g.n_points + TILE_POINTS - 1) / TILE_POINTS;
     if (i == 0) {

@@ -883,6 +883,16 @@ bool compute(
             extras.h_small, sorted, tiles, cell_scan, extras.d_status
         );
         fetched = true;
+    } else if (single_cell && point_blocks == 1) {
+        // the single cell of a small system: one launch prepares it, clears the state of the search and fetches the box
+        char* first = reinterpret_cast<char*>(chain.blocks);
+        const size_t to_clear = reinterpret_cast<char*>(ordered_status + 1) - first;
+        hipLaunchKernelGGL(
+            prepare_single_cell, dim3(1), dim3(BLOCK), 0, stream,
+            flat_points, g, sorted, tiles, cell_scan, extras.d_status, reinterpret_cast<uint4*>(first), (to_clear + 15) / 16,
+            fetched ? static_cast<const double*>(nullptr) : reinterpret_cast<const double*>(box), periodic, extras.h_small
+        );
+        fetched = true;
     } else if (direct_cells) {
         clear_work_state();
         hipLaunchKernelGGL(
