@@ -1,0 +1,185 @@
+"""The Python adapters around ``NeighborList``: the ASE calling convention (python/vesin/vesin/_ase.py:9-55, tested
+by the reference in python/vesin/tests/test_numpy.py:88-141) and device arrays of libraries other than torch
+(python/vesin/vesin/_neighbors.py:173-183,436-452, tested in python/vesin/tests/test_cupy.py).
+
+Neither ase nor cupy is installed here, so both are driven through stand-ins that offer exactly what the adapters
+read: an ``Atoms`` with ``positions`` / ``cell`` / ``pbc``, and an array library whose arrays have a
+``__cuda_array_interface__`` and a ``device.id`` and whose ``asarray`` takes objects with that interface, like
+cupy's. What the real packages would add on top of that is not covered.
+"""
+
+import sys
+import types
+
+import numpy as np
+import pytest
+
+import oracle
+from _helpers import assert_same_list
+from golden import systems
+
+import vesin_amd
+from vesin_amd import _ase
+
+
+class Atoms:
+    def __init__(self, positions, cell, pbc):
+        self.positions = np.asarray(positions, dtype=np.float64)
+        self.cell = np.asarray(cell, dtype=np.float64)
+        self.pbc = np.array([pbc] * 3 if isinstance(pbc, bool) else pbc, dtype=np.bool_)
+
+
+@pytest.fixture
+def with_ase(monkeypatch):
+    monkeypatch.setattr(_ase, "ase", types.SimpleNamespace(Atoms=Atoms))
+
+
+def test_ase_wrapper_needs_ase(monkeypatch):
+    monkeypatch.setattr(_ase, "ase", None)
+    with pytest.raises(ImportError, match="could not import ase"):
+        vesin_amd.ase_neighbor_list("ij", Atoms(np.zeros((1, 3)), np.eye(3), True), cutoff=1.0)
+
+
+def test_ase_wrapper_refusals(with_ase):
+    atoms = Atoms(np.zeros((1, 3)), np.eye(3), True)
+    with pytest.raises(ValueError, match="self_interaction=True is not implemented"):
+        vesin_amd.ase_neighbor_list("ij", atoms, cutoff=1.0, self_interaction=True)
+    with pytest.raises(ValueError, match="only a single float cutoff is supported"):
+        vesin_amd.ase_neighbor_list("ij", atoms, cutoff={("H", "H"): 1.0})
+    with pytest.raises(TypeError, match="`a` should be ase.Atoms"):
+        vesin_amd.ase_neighbor_list("ij", object(), cutoff=1.0)
+
+
+@pytest.mark.gpu
+def test_ase_wrapper_integer_cutoff(with_ase):
+    # python/vesin/tests/test_numpy.py:131-141
+    atoms = Atoms([[0.0, 0.0, 0.0], [0.5, 0.0, 0.0]], 2.0 * np.eye(3), False)
+    i, j = vesin_amd.ase_neighbor_list("ij", atoms, cutoff=1)
+    assert isinstance(i, np.ndarray) and isinstance(j, np.ndarray)
+    assert i.tolist() == [0, 1]
+    assert j.tolist() == [1, 0]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["slab", "diamond", "naphthalene", "water"])
+def test_ase_wrapper_gives_the_full_list_ordered_by_i(with_ase, name):
+    points, box, periodic = systems.read_xyz(name)
+    atoms = Atoms(points, box, periodic)
+    i, j, S, D, d = vesin_amd.ase_neighbor_list("ijSDd", atoms, cutoff=5.0)
+    assert np.all(np.diff(i.astype(np.int64)) >= 0)
+    expected = oracle.neighbors(points, box, periodic, 5.0, full=True, sorted=True)
+    actual = {"pairs": np.stack([i, j], axis=1), "shifts": S, "distances": d, "vectors": D}
+    assert_same_list(actual, expected, what=name)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# a device-array library with the surface of cupy that the adapter uses
+
+
+class _Device:
+    def __init__(self, index):
+        self.id = index
+
+
+class StandInArray:
+    """Holds a torch GPU tensor and shows it through ``__cuda_array_interface__`` only."""
+
+    def __init__(self, tensor, owner=None):
+        self._tensor = tensor
+        self._owner = owner
+        self.device = _Device(tensor.device.index)
+        self.shape = tuple(tensor.shape)
+
+    @property
+    def __cuda_array_interface__(self):
+        typestr = {"torch.float64": "<f8", "torch.float32": "<f4", "torch.int32": "<i4", "torch.uint64": "<u8",
+                   "torch.bool": "|b1", "torch.int64": "<i8"}[str(self._tensor.dtype)]
+        itemsize = self._tensor.element_size()
+        contiguous = self._tensor.is_contiguous()
+        return {
+            "shape": tuple(self._tensor.shape),
+            "typestr": typestr,
+            "data": (self._tensor.data_ptr() if self._tensor.numel() else 0, False),
+            "version": 2,
+            "strides": None if contiguous else tuple(s * itemsize for s in self._tensor.stride()),
+        }
+
+    def get(self):
+        return self._tensor.cpu().numpy()
+
+    @property
+    def pointer(self):
+        return self._tensor.data_ptr()
+
+
+@pytest.fixture
+def standin_library(monkeypatch):
+    import torch
+
+    module = types.ModuleType("standin_arrays")
+
+    def asarray(obj):
+        interface = obj.__cuda_array_interface__
+        if 0 in interface["shape"]:
+            dtype = {"<u8": torch.uint64, "<i4": torch.int32, "<f8": torch.float64, "<f4": torch.float32}
+            return StandInArray(torch.empty(interface["shape"], dtype=dtype[interface["typestr"]], device="cuda:0"))
+        return StandInArray(torch.as_tensor(obj, device="cuda:0"), owner=obj)
+
+    module.asarray = asarray
+    module.ndarray = StandInArray
+    monkeypatch.setitem(sys.modules, "standin_arrays", module)
+    monkeypatch.setattr(StandInArray, "__module__", "standin_arrays.core")
+    return module
+
+
+def on_device(array, dtype=np.float64):
+    import torch
+
+    return StandInArray(torch.as_tensor(np.ascontiguousarray(array, dtype=dtype), device="cuda:0"))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("copy", [True, False])
+def test_device_arrays_of_another_library(standin_library, copy):
+    points, box, periodic = systems.diamond_crystal()
+    calculator = vesin_amd.NeighborList(cutoff=3.5, full_list=False)
+    for _ in range(2):
+        outputs = calculator.compute(on_device(points), on_device(box), periodic, "PijSdD", copy=copy)
+        assert all(isinstance(out, StandInArray) for out in outputs)
+        P, i, j, S, d, D = (out.get() for out in outputs)
+        assert P.dtype == np.uint64 and S.dtype == np.int32 and d.dtype == np.float64 and D.dtype == np.float64
+        assert np.array_equal(P[:, 0], i) and np.array_equal(P[:, 1], j)
+        expected = oracle.neighbors(points, box, periodic, 3.5, full=False)
+        assert_same_list({"pairs": P, "shifts": S, "distances": d, "vectors": D}, expected)
+        # views are the calculator's own arrays, copies are not
+        assert (outputs[0].pointer == calculator._neighbors.pairs) == (not copy)
+        assert (outputs[4].pointer == calculator._neighbors.distances) == (not copy)
+
+
+@pytest.mark.gpu
+def test_device_arrays_box_and_flags_may_live_anywhere(standin_library):
+    points, box, periodic = systems.graphene_sheet()
+    calculator = vesin_amd.NeighborList(cutoff=3.0, full_list=True, sorted=True)
+    expected = oracle.neighbors(points, box, periodic, 3.0, full=True, sorted=True, quantities="ijS")
+    for device_box in (box, box.tolist(), on_device(box)):
+        for flags in (periodic, list(periodic), on_device(periodic, np.bool_)):
+            P, S = calculator.compute(on_device(points), device_box, flags, "PS")
+            assert_same_list({"pairs": P.get(), "shifts": S.get()}, expected, ordered=True)
+
+
+@pytest.mark.gpu
+def test_device_arrays_dtypes_and_empty_results(standin_library):
+    # python/vesin/tests/test_cupy.py: float32 in, float32 out; nothing within the cutoff gives shaped empty arrays
+    points = np.array([[0.0, 0.0, 0.0], [0.0, 0.0, 2.0]])
+    box = np.zeros((3, 3))
+    calculator = vesin_amd.NeighborList(cutoff=2.5, full_list=True)
+    i, d, D = calculator.compute(on_device(points, np.float32), on_device(box, np.float32), False, "idD")
+    assert d.get().dtype == np.float32 and D.get().dtype == np.float32
+    assert sorted(i.get().tolist()) == [0, 1] and np.allclose(d.get(), 2.0)
+
+    calculator = vesin_amd.NeighborList(cutoff=0.5, full_list=True)
+    P, S, d, D = calculator.compute(on_device(points), on_device(box), False, "PSdD")
+    assert P.shape == (0, 2) and S.shape == (0, 3) and d.shape == (0,) and D.shape == (0, 3)
+
+    with pytest.raises(RuntimeError, match="must have the same dtype"):
+        calculator.compute(on_device(points, np.float32), on_device(box), False, "ij")

@@ -6,6 +6,10 @@ The calculation always runs on a GPU through ``vesin_neighbors`` with ``device =
 
 * torch tensors on a ``cuda`` device (what PyTorch-ROCm calls a HIP GPU) are used in place, and the results are
   torch tensors on the same device (zero-copy views of the library's buffers when ``copy=False``);
+* device arrays of other libraries (cupy on ROCm, numba: anything that is not a torch tensor and has a
+  ``__cuda_array_interface__``; the reference takes ``cupy.ndarray`` at python/vesin/vesin/_neighbors.py:173-183,
+  436-452) are used in place too, and the results are arrays of the same library, made by its ``asarray`` from
+  objects with that interface (views of the library's buffers when ``copy=False``);
 * numpy arrays (or anything numpy can convert) are uploaded to ``device`` (default ``cuda:0``) and the results come
   back as numpy arrays.
 
@@ -38,17 +42,50 @@ _ALGORITHMS = {
 
 
 class _DeviceView:
-    """Expose a raw device pointer through ``__cuda_array_interface__`` so torch can wrap it without a copy."""
+    """Expose a raw device pointer through ``__cuda_array_interface__`` so torch (or any array library that reads
+    the interface) can wrap it without a copy. ``owner`` is kept alive as long as the view."""
 
-    def __init__(self, pointer, shape, typestr, owner):
+    def __init__(self, pointer, shape, typestr, owner, strides=None):
         self._owner = owner
         self.__cuda_array_interface__ = {
             "shape": tuple(shape),
             "typestr": typestr,
             "data": (int(pointer), False),
             "version": 2,
-            "strides": None,
+            "strides": strides,
         }
+
+
+_TYPESTR = {"torch.uint64": "<u8", "torch.int32": "<i4", "torch.float64": "<f8", "torch.float32": "<f4",
+            "torch.float16": "<f2"}
+
+
+def _export(tensor, namespace):
+    """Hand a torch GPU tensor to another array library: ``namespace.asarray`` of a view of the same memory."""
+    itemsize = tensor.element_size()
+    strides = None if tensor.is_contiguous() else tuple(stride * itemsize for stride in tensor.stride())
+    pointer = tensor.data_ptr() if tensor.numel() > 0 else 0
+    return namespace.asarray(_DeviceView(pointer, tensor.shape, _TYPESTR[str(tensor.dtype)], tensor, strides))
+
+
+def _namespace_of(array):
+    """The top-level module of the library an array comes from (``cupy`` for a ``cupy.ndarray``)."""
+    import importlib
+
+    namespace = importlib.import_module(type(array).__module__.split(".")[0])
+    if not hasattr(namespace, "asarray"):
+        raise TypeError(f"can not return results as {type(array)}: its module `{namespace.__name__}` has no `asarray`")
+    return namespace
+
+
+def _device_index_of(array, default):
+    """GPU index of a device array: ``array.device.id`` (cupy), ``array.device.index``, else ``default``."""
+    device = getattr(array, "device", None)
+    for name in ("id", "index"):
+        index = getattr(device, name, None)
+        if isinstance(index, int):
+            return index
+    return default
 
 
 class NeighborList:
@@ -126,6 +163,19 @@ class NeighborList:
                 "this implementation only computes on GPU tensors; move `points` to a cuda (HIP) device"
             )
         device = points.device if is_torch else torch.device(self.device)
+        namespace = None
+        if not is_torch and hasattr(points, "__cuda_array_interface__"):
+            # a device array of another library: used in place, results go back through its own `asarray`
+            namespace = _namespace_of(points)
+            device = torch.device("cuda", _device_index_of(points, device.index if device.index is not None else 0))
+            points = torch.as_tensor(points, device=device)
+            if hasattr(box, "__cuda_array_interface__"):
+                box = torch.as_tensor(box, device=device)
+            else:
+                box = torch.from_numpy(np.ascontiguousarray(np.asarray(box))).to(device=device)
+            if hasattr(periodic, "__cuda_array_interface__"):
+                periodic = torch.as_tensor(periodic, device=device)
+            is_torch = True
 
         if isinstance(periodic, (bool, np.bool_)):
             periodic = [bool(periodic)] * 3
@@ -140,7 +190,10 @@ class NeighborList:
             if points.requires_grad or box.requires_grad:
                 raise RuntimeError("NeighborList.compute does not support autograd for torch tensors")
             float_dtype = initial_dtype if initial_dtype.is_floating_point else torch.float64
-            to_result = lambda t: t  # noqa: E731
+            if namespace is None:
+                to_result = lambda t: t  # noqa: E731
+            else:
+                to_result = lambda t: _export(t, namespace)  # noqa: E731
         else:
             points = np.asarray(points)
             box = np.asarray(box)
