@@ -137,3 +137,95 @@ def test_a_system_that_search_does_not_cover_is_not_asked_again(capfd, monkeypat
         assert np.array_equal(S.cpu().numpy(), expected["shifts"])
         assert np.array_equal(d.cpu().numpy(), expected["distances"])
     assert tried == [True, False, False]
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Systems with enough tiles for the candidates of every tile to be put in order once (ordered_sort_kernel): the
+# order of the input decides how (a window of original indices counted through a bit set, or buckets).
+
+
+def _lattice(nx, ny, nz, seed, a=3.567):
+    """Jittered diamond, atoms numbered cell by cell with x changing slowest: what a crystal builder hands over."""
+    basis = np.array([[0, 0, 0], [0, 2, 2], [2, 0, 2], [2, 2, 0], [1, 1, 1], [1, 3, 3], [3, 1, 3], [3, 3, 1]]) / 4.0
+    cells = np.stack(np.meshgrid(np.arange(nx), np.arange(ny), np.arange(nz), indexing="ij"), axis=-1).reshape(-1, 3)
+    points = (cells[:, None, :] + basis[None, :, :]).reshape(-1, 3) * a
+    points += np.random.default_rng(seed).normal(scale=0.05, size=points.shape)
+    return points, np.diag([nx * a, ny * a, nz * a])
+
+
+def _modes(err):
+    import re
+
+    found = re.findall(r"of (\d+) tiles ordered by window and of (\d+) by buckets", err)
+    assert found, err
+    return int(found[-1][0]), int(found[-1][1])
+
+
+def _check_order_once(points, box, periodic, cutoff, full, capfd, monkeypatch):
+    expected = oracle.canonicalize(oracle.neighbors(points, box, periodic, cutoff, full, False, "ijSdD"))
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    capfd.readouterr()
+    result = _sorted_list(points, box, periodic, cutoff, full)
+    err = capfd.readouterr().err
+    assert any(line.startswith("in-order search:") and line.endswith("used") for line in err.splitlines()), err
+    assert result["pairs"].shape == expected["pairs"].shape
+    for key in result:
+        assert np.array_equal(result[key], expected[key]), key
+    return _modes(err)
+
+
+@pytest.mark.parametrize("full", [True, False])
+def test_lattice_order_in_one_round_of_the_window(full, capfd, monkeypatch):
+    # 110,592 atoms: any tile sees a range of original indices well below 65,536
+    points, box = _lattice(24, 24, 24, seed=1)
+    windowed, bucketed = _check_order_once(points, box, [True] * 3, 5.0, full, capfd, monkeypatch)
+    assert windowed > 2048 and bucketed == 0
+
+
+def test_lattice_order_in_several_rounds_and_around_the_end(capfd, monkeypatch):
+    # 12 x 48 x 48 cells, 221,184 atoms: three search cells of x are 5 or 6 of the 12 lattice cells, about 100,000
+    # indices; at the two ends of x the neighbourhood continues at the other end of the numbering
+    points, box = _lattice(12, 48, 48, seed=2)
+    windowed, bucketed = _check_order_once(points, box, [True] * 3, 5.0, True, capfd, monkeypatch)
+    assert windowed > 2048 and bucketed == 0
+
+
+def test_lattice_order_too_wide_for_the_window(capfd, monkeypatch):
+    # 6 x 96 x 96 cells, 442,368 atoms: four search cells along x, three of them in every stencil, so a tile sees
+    # dense runs of indices spread over two thirds of the numbering or more, whichever way around: beyond 262,144
+    points, box = _lattice(6, 96, 96, seed=3)
+    windowed, bucketed = _check_order_once(points, box, [True] * 3, 5.0, True, capfd, monkeypatch)
+    assert bucketed > 2048
+
+
+@pytest.mark.parametrize("full", [True, False])
+def test_no_order_in_the_input(full, capfd, monkeypatch):
+    # 373,248 atoms: more than the window holds, and every tile sees indices from all over
+    points, box = _lattice(36, 36, 36, seed=4)
+    points = points[np.random.default_rng(5).permutation(len(points))]
+    windowed, bucketed = _check_order_once(points, box, [True] * 3, 5.0, full, capfd, monkeypatch)
+    assert bucketed > 2048 and windowed == 0
+
+
+def test_no_order_in_an_input_the_window_holds(capfd, monkeypatch):
+    points, box = _lattice(30, 30, 30, seed=9)
+    points = points[np.random.default_rng(10).permutation(len(points))]
+    windowed, bucketed = _check_order_once(points, box, [True] * 3, 5.0, True, capfd, monkeypatch)
+    assert windowed > 2048 and bucketed == 0
+
+
+@pytest.mark.parametrize("shuffle", [False, True])
+def test_two_images_of_a_point_among_the_candidates(shuffle, capfd, monkeypatch):
+    # two search cells along x: the stencil reaches the same cell from both sides, a tile sees points twice, with
+    # different shifts; only the buckets tell such candidates apart
+    points, box = _lattice(3, 70, 70, seed=6)
+    if shuffle:
+        points = points[np.random.default_rng(7).permutation(len(points))]
+    windowed, bucketed = _check_order_once(points, box, [True] * 3, 5.0, True, capfd, monkeypatch)
+    assert bucketed > 2048 and windowed == 0
+
+
+def test_slab_with_free_directions(capfd, monkeypatch):
+    points, box = _lattice(40, 40, 6, seed=8)
+    windowed, bucketed = _check_order_once(points, box, [True, True, False], 5.0, False, capfd, monkeypatch)
+    assert windowed + bucketed > 2048

@@ -781,6 +781,16 @@ bool compute(
     OrderedStatus* ordered_status = nullptr;
     uint32_t* rows_of_point = nullptr;
     uint64_t* first_row_of_point = nullptr;
+    uint32_t* hit_columns = nullptr;
+    uint16_t* candidate_order = nullptr;
+    // small systems: the points of a tile are dealt to several waves, about 2048 in all
+    uint32_t ordered_points_per_item = TILE_POINTS;
+    while (ordered_points_per_item > 1 && tiles_bound * (TILE_POINTS / ordered_points_per_item) < 2048) {
+        ordered_points_per_item /= 2;
+    }
+    const uint32_t ordered_items_per_tile = TILE_POINTS / ordered_points_per_item;
+    const uint32_t ordered_blocks =
+        static_cast<uint32_t>((tiles_bound * ordered_items_per_tile + ORDERED_WAVES - 1) / ORDERED_WAVES);
     const size_t scratch_elements = std::max(
         std::max(scan_scratch_elements(n_cells), scan_scratch_elements(n_slots)),
         try_in_order ? scan_scratch_elements(n_points) : 0
@@ -816,6 +826,10 @@ bool compute(
         if (try_in_order) {
             rows_of_point = carver.take<uint32_t>(n_points);
             first_row_of_point = carver.take<uint64_t>(n_points + 1);
+            hit_columns = carver.take<uint32_t>(static_cast<size_t>(ordered_blocks) * ORDERED_WAVES * ORDERED_UNITS * WAVE);
+            if (ordered_items_per_tile == 1) {
+                candidate_order = carver.take<uint16_t>(tiles_bound * ORDERED_CANDIDATES);
+            }
         }
     };
     Carver measure(nullptr);
@@ -1030,22 +1044,28 @@ bool compute(
         oargs.sorted = sorted;
         oargs.cell_scan = cell_scan;
         oargs.tiles = tiles;
-        // small systems: the points of a tile are dealt to several waves, about 2048 in all
-        uint32_t points_per_item = TILE_POINTS;
-        while (points_per_item > 1 && tiles_bound * (TILE_POINTS / points_per_item) < 2048) {
-            points_per_item /= 2;
-        }
-        oargs.points_per_item = points_per_item;
-        oargs.items_per_tile = TILE_POINTS / points_per_item;
+        oargs.points_per_item = ordered_points_per_item;
+        oargs.items_per_tile = ordered_items_per_tile;
         oargs.rows_of_point = rows_of_point;
+        oargs.columns = hit_columns;
+        oargs.order = candidate_order;
         oargs.first_row = first_row_of_point;
         oargs.status = ordered_status;
-        const uint32_t blocks =
-            static_cast<uint32_t>((tiles_bound * oargs.items_per_tile + ORDERED_WAVES - 1) / ORDERED_WAVES);
+        const uint32_t blocks = ordered_blocks;
         if (options.full) {
             hipLaunchKernelGGL((ordered_search_kernel<false, true>), dim3(blocks), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
         } else {
             hipLaunchKernelGGL((ordered_search_kernel<false, false>), dim3(blocks), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
+        }
+        // The order of every tile's candidates, for the writing pass (wasted when the counting pass finds the
+        // system unsuitable, which the host only knows after both). Small systems do without: one more launch
+        // costs them more than ranking the rows of every point does.
+        const bool presorted = ordered_items_per_tile == 1;
+        if (presorted) {
+            hipLaunchKernelGGL(
+                ordered_sort_kernel, dim3(static_cast<uint32_t>((tiles_bound + ORDER_WAVES - 1) / ORDER_WAVES)),
+                dim3(ORDER_BLOCK), 0, stream, oargs, g
+            );
         }
         mark(T_COUNT);
         exclusive_scan<SCAN_U32>(rows_of_point, n_points, first_row_of_point, scan_scratch, stream);
@@ -1067,9 +1087,10 @@ bool compute(
         if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
             std::fprintf(
                 stderr,
-                "in-order search: rows %llu, most rows of a point %u, most candidates of a tile %u, unsuitable %u: %s\n",
+                "in-order search: rows %llu, most rows of a point %u, most candidates of a tile %u, unsuitable %u, "
+                "candidates of %u tiles ordered by window and of %u by buckets: %s\n",
                 found.total_rows, found.found.max_rows, found.found.max_candidates, found.found.unsuitable,
-                suitable ? "used" : "left to the radix sort"
+                found.found.windowed, found.found.bucketed, suitable ? "used" : "left to the radix sort"
             );
         }
         if (suitable) {
@@ -1079,11 +1100,9 @@ bool compute(
             oargs.out = outputs_of();
             mark(T_WRITE_BEGIN);
             if (total > 0) {
-                if (options.full) {
-                    hipLaunchKernelGGL((ordered_search_kernel<true, true>), dim3(blocks), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
-                } else {
-                    hipLaunchKernelGGL((ordered_search_kernel<true, false>), dim3(blocks), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
-                }
+                auto kernel = presorted ? (options.full ? ordered_search_kernel<true, true, true> : ordered_search_kernel<true, false, true>)
+                                        : (options.full ? ordered_search_kernel<true, true, false> : ordered_search_kernel<true, false, false>);
+                hipLaunchKernelGGL(kernel, dim3(blocks), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
             }
             mark(T_WRITE);
             mark(T_SORT);

@@ -6,11 +6,17 @@
 // the whole (2s+1)^3 stencil, so every row (i, j, S) is found by the tile that holds i and by no other (a half
 // list keeps i < j, or the self-image the reference's rule keeps, vesin/src/cpu_cell_list.cpp:101-133: the other
 // orientation is found, and dropped, by the tile of j). Twice the distance tests of the other kernels, but then
-//   COUNT  knows the number of rows of each of its points (one store per point, indexed by original index),
+//   COUNT  knows the number of rows of each of its points (one store per point, indexed by original index) and
+//          leaves the hit column of every candidate in memory,
 //   a scan over the points in original order gives every point its place in the output,
-//   WRITE  keeps one hit column per candidate lane, then, point by point, collects the point's hits as 64-bit
-//          keys (second point, biased shift) in LDS, ranks them (each lane counts the smaller keys: at most 256
-//          keys, read as LDS broadcasts) and stores the row of rank r at the point's place + r.
+//   SORT   orders the candidates of every tile by (second point, shift without the wrap of the first point). All
+//          points of a tile share that order: the wrap of the first point adds the same constant to the shift of
+//          every one of its rows. One small sort per tile replaces a sort of the rows of every point,
+//   WRITE  takes the candidates in that order, one per lane and unit, with their hit columns; point by point the
+//          hits of the lanes, taken in lane order, are the rows in final order: they are compacted through LDS and
+//          stored as runs of consecutive rows.
+// Small systems (several waves per tile) skip SORT: their WRITE takes the candidates in table order and ranks the
+// rows of every point by comparing all its keys (at most 256, read as LDS broadcasts).
 // Rows per point beyond 256, candidates per tile beyond 1024, stencils beyond 64 cells or shifts and wraps beyond
 // +-255 are reported in the status and the host falls back to the unsorted search followed by the radix sort.
 //
@@ -38,7 +44,9 @@ struct OrderedStatus {
     unsigned int max_rows;       // largest number of rows of one point
     unsigned int max_candidates; // largest number of candidates of one tile
     unsigned int unsuitable;     // tiles with a shift outside of the key's range
-    unsigned int padding;
+    unsigned int windowed;       // tiles whose candidates were ordered through the bit set
+    unsigned int bucketed;       // tiles whose candidates were ordered through buckets
+    unsigned int padding[3];
 };
 
 struct OrderedArgs {
@@ -48,6 +56,8 @@ struct OrderedArgs {
     uint32_t points_per_item;   // a tile's points are dealt to ceil(TILE_POINTS / points_per_item) waves
     uint32_t items_per_tile;
     uint32_t* rows_of_point;    // COUNT: [n_points], by original index
+    uint32_t* columns;          // COUNT -> WRITE: hit columns, [work item][ORDERED_UNITS][64], candidates in table order
+    uint16_t* order;            // SORT -> WRITE: [tile][ORDERED_CANDIDATES], candidate number at each place of the order
     const uint64_t* first_row;  // WRITE: [n_points + 1], exclusive scan of rows_of_point
     OrderedStatus* status;
     SearchOutputs out;
@@ -60,9 +70,10 @@ struct OrderedWaveShared: SearchTables {
     double tile_x[TILE_POINTS], tile_y[TILE_POINTS], tile_z[TILE_POINTS];
     int32_t tile_wx[TILE_POINTS], tile_wy[TILE_POINTS], tile_wz[TILE_POINTS];
     uint64_t tile_row[TILE_POINTS];   // WRITE: first output row of each point
-    // WRITE: (second point << 32) | biased shift, rows of one point; read four at a time, hence the padding
+    // WRITE: the rows of one point: (second point << 32) | biased shift, and the position of the second point in
+    // the cell-sorted arrays; read four at a time when they are ranked, hence the padding
     __attribute__((aligned(16))) uint64_t keys[ORDERED_MAX_ROWS + 4];
-    uint32_t key_at[ORDERED_MAX_ROWS];// WRITE: position of the second point in the cell-sorted arrays
+    uint32_t key_at[ORDERED_MAX_ROWS];
 };
 
 struct OrderedShared {
@@ -79,16 +90,16 @@ __device__ __forceinline__ bool beyond(int32_t a, int32_t b, int32_t c, int32_t 
 }
 
 /// Two units of candidates (numbers unit0 * 64 ... + 127 of the tables) against the item's points: hit columns
-/// (the item's first point in the highest bit used) and what the writing pass needs to know about each candidate.
+/// (the item's first point in the highest bit used).
 template <bool FULL, bool WRAPPED>
 __device__ __forceinline__ void ordered_sweep_pair(
     const OrderedWaveShared& sh, const SortedPoints& sorted, const GridParams& g, uint32_t unit0, uint32_t n_stencil,
-    uint32_t n_candidates, uint32_t first_i, uint32_t n_i, int lane, uint32_t (&column)[ORDERED_R],
-    uint32_t (&at)[ORDERED_R], uint32_t (&original)[ORDERED_R], int32_t (&packed_b)[ORDERED_R], bool& out_of_range
+    uint32_t n_candidates, uint32_t first_i, uint32_t n_i, int lane, uint32_t (&column)[ORDERED_R], bool& out_of_range
 ) {
     constexpr int R = ORDERED_R;
     SweepCandidates<R> c;
     int32_t packed_q[R];
+    uint32_t at[R], original[R];
     bool any_shift = false;
 #pragma unroll
     for (int r = 0; r < R; r++) {
@@ -116,7 +127,6 @@ __device__ __forceinline__ void ordered_sweep_pair(
             c.shift[r] = pack_shift(bx, by, bz);
             out_of_range = out_of_range || beyond(bx, by, bz, ORDERED_SHIFT_LIMIT);
         }
-        packed_b[r] = c.shift[r];
         any_shift = any_shift || (__ballot((bx | by | bz) != 0) != 0);
         if (!WRAPPED && any_shift) {
             shift_vector(g, bx, by, bz, c.tx[r], c.ty[r], c.tz[r]);
@@ -158,7 +168,10 @@ __device__ __forceinline__ void ordered_sweep_pair(
     }
 }
 
-template <bool WRITE, bool FULL>
+/// PRESORTED (WRITE only): the candidates are taken in the order ordered_sort_kernel left for the tile, and the hits
+/// of a point in lane order are its rows in final order. Otherwise (small systems, where one more launch costs more
+/// than it saves) candidates come in table order and the rows of every point are ranked by comparing all its keys.
+template <bool WRITE, bool FULL, bool PRESORTED = false>
 __global__ __launch_bounds__(ORDERED_BLOCK) void ordered_search_kernel(OrderedArgs args, GridParams g) {
     constexpr int R = ORDERED_R;
     __shared__ OrderedShared shared;
@@ -232,23 +245,27 @@ __global__ __launch_bounds__(ORDERED_BLOCK) void ordered_search_kernel(OrderedAr
         return; // the host does not use this path for such a tile: nothing to count, nothing may be written
     }
 
+    uint32_t* item_columns = args.columns + static_cast<size_t>(work) * (ORDERED_UNITS * WAVE);
     if constexpr (!WRITE) {
-        // ---- COUNT: nothing is kept but the number of rows of every point (lane p adds up the hits of point p):
-        // a plain loop over the pairs of units, small code
+        // ---- COUNT: the number of rows of every point (lane p adds up the hits of point p) and, for the writing
+        // pass, the hit column of every candidate: a plain loop over the pairs of units, small code
         uint32_t own_rows = 0;
         for (uint32_t unit0 = 0; unit0 < n_units; unit0 += R) {
-            uint32_t column[R], at[R], original[R];
-            int32_t packed_b[R];
+            uint32_t column[R];
             if (tile_wrapped) {
                 ordered_sweep_pair<FULL, true>(
-                    sh, sorted, g, unit0, n_stencil, n_candidates, first_i, n_i, lane, column, at, original, packed_b,
-                    out_of_range
+                    sh, sorted, g, unit0, n_stencil, n_candidates, first_i, n_i, lane, column, out_of_range
                 );
             } else {
                 ordered_sweep_pair<FULL, false>(
-                    sh, sorted, g, unit0, n_stencil, n_candidates, first_i, n_i, lane, column, at, original, packed_b,
-                    out_of_range
+                    sh, sorted, g, unit0, n_stencil, n_candidates, first_i, n_i, lane, column, out_of_range
                 );
+            }
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                if (unit0 + r < n_units) {
+                    __builtin_nontemporal_store(column[r], &item_columns[(unit0 + r) * WAVE + lane]);
+                }
             }
             for (uint32_t p = 0; p < n_i; p++) {
                 const uint32_t bit = n_i - 1 - p;
@@ -279,76 +296,59 @@ __global__ __launch_bounds__(ORDERED_BLOCK) void ordered_search_kernel(OrderedAr
         return;
     }
 
-    // ---- sweep: per candidate (registers of its lane, indexed by unit) the hit column against this item's points
+    // ---- per place of the tile's order (registers of its lane, indexed by unit): the candidate there, the hit
+    // column the counting pass found for it against this item's points, its original index and its shift (biased,
+    // without the wrap of the first point: that one is added per point, field by field in one integer addition)
+    const uint16_t* tile_order = args.order + static_cast<size_t>(tile_id) * ORDERED_CANDIDATES;
     uint32_t columns[ORDERED_UNITS];
     uint32_t cand_at[ORDERED_UNITS];
     uint32_t cand_index[ORDERED_UNITS];
-    int32_t cand_shift[ORDERED_UNITS];
+    uint32_t cand_biased[ORDERED_UNITS];
 #pragma unroll
     for (int u = 0; u < ORDERED_UNITS; u++) {
         columns[u] = 0;
         cand_at[u] = 0;
         cand_index[u] = 0;
-        cand_shift[u] = 0;
-    }
-#pragma unroll
-    for (int pair = 0; pair < ORDERED_UNITS / R; pair++) {
-        if (static_cast<uint32_t>(pair * R) < n_units) {
-            uint32_t column[R], at[R], original[R];
-            int32_t packed_b[R];
-            if (tile_wrapped) {
-                ordered_sweep_pair<FULL, true>(
-                    sh, sorted, g, pair * R, n_stencil, n_candidates, first_i, n_i, lane, column, at, original, packed_b,
-                    out_of_range
-                );
-            } else {
-                ordered_sweep_pair<FULL, false>(
-                    sh, sorted, g, pair * R, n_stencil, n_candidates, first_i, n_i, lane, column, at, original, packed_b,
-                    out_of_range
-                );
-            }
-#pragma unroll
-            for (int r = 0; r < R; r++) {
-                columns[pair * R + r] = column[r];
-                if (WRITE) {
-                    cand_at[pair * R + r] = at[r];
-                    cand_index[pair * R + r] = original[r];
-                    cand_shift[pair * R + r] = packed_b[r];
-                }
-            }
+        cand_biased[u] = 0;
+        const uint32_t place = u * WAVE + lane;
+        if (static_cast<uint32_t>(u) < n_units && place < n_candidates) {
+            const uint32_t k = PRESORTED ? min(static_cast<uint32_t>(tile_order[place]), n_candidates - 1) : place;
+            columns[u] = __builtin_nontemporal_load(&item_columns[k]);
+            int32_t packed_q;
+            locate_candidate(sh, n_stencil, k, cand_at[u], packed_q);
+            int32_t qx, qy, qz;
+            unpack_shift(packed_q, qx, qy, qz);
+            cand_index[u] = sorted.index[cand_at[u]];
+            cand_biased[u] = biased_shift(qx - sorted.wx[cand_at[u]], qy - sorted.wy[cand_at[u]], qz - sorted.wz[cand_at[u]]);
         }
     }
 
-    // ---- WRITE: point by point, collect the hits, rank them, store the rows
+    // ---- WRITE: point by point, collect the hits in lane order, rank them where that is not their final order,
+    // store the rows
     wave_sync();
     for (uint32_t p = 0; p < n_i; p++) {
         const uint32_t bit = n_i - 1 - p;
-        const int32_t wix = sh.tile_wx[p];
-        const int32_t wiy = sh.tile_wy[p];
-        const int32_t wiz = sh.tile_wz[p];
+        // every field of the sum stays inside its ten bits (operands within +-255), so the fields add independently
+        const uint32_t wrap_i = (static_cast<uint32_t>(sh.tile_wx[p]) << 20) + (static_cast<uint32_t>(sh.tile_wy[p]) << 10) +
+                                static_cast<uint32_t>(sh.tile_wz[p]);
         uint32_t n_rows = 0;
 #pragma unroll
         for (int u = 0; u < ORDERED_UNITS; u++) {
             if (static_cast<uint32_t>(u) < n_units) {
                 const bool hit = ((columns[u] >> bit) & 1u) != 0;
                 const uint64_t mask = __ballot(hit);
-                if (mask != 0) {
-                    if (hit) {
-                        int32_t bx, by, bz;
-                        unpack_shift(cand_shift[u], bx, by, bz);
-                        const uint32_t slot = n_rows + rank_in_mask(mask);
-                        sh.keys[slot] = (static_cast<uint64_t>(cand_index[u]) << 32) |
-                                        biased_shift(bx + wix, by + wiy, bz + wiz);
-                        sh.key_at[slot] = cand_at[u];
-                    }
-                    n_rows += __popcll(mask);
+                if (hit) {
+                    const uint32_t slot = n_rows + rank_in_mask(mask);
+                    sh.keys[slot] = (static_cast<uint64_t>(cand_index[u]) << 32) | (cand_biased[u] + wrap_i);
+                    sh.key_at[slot] = cand_at[u];
                 }
+                n_rows += __popcll(mask);
             }
         }
         if (n_rows == 0) {
             continue;
         }
-        if (lane < 4) {
+        if (!PRESORTED && lane < 4) {
             sh.keys[n_rows + lane] = ~0ull; // larger than any key: the ranking reads whole groups of four
         }
         wave_sync();
@@ -367,13 +367,16 @@ __global__ __launch_bounds__(ORDERED_BLOCK) void ordered_search_kernel(OrderedAr
             const double xj = sorted.x[at];
             const double yj = sorted.y[at];
             const double zj = sorted.z[at];
-            uint32_t rank = 0;
-            for (uint32_t other = 0; other < n_rows; other += 4) {
-                // every lane reads the same 32 bytes: two LDS broadcasts for four comparisons
-                const ulonglong2 first_two = *reinterpret_cast<const ulonglong2*>(&sh.keys[other]);
-                const ulonglong2 next_two = *reinterpret_cast<const ulonglong2*>(&sh.keys[other + 2]);
-                rank += (first_two.x < key ? 1u : 0u) + (first_two.y < key ? 1u : 0u);
-                rank += (next_two.x < key ? 1u : 0u) + (next_two.y < key ? 1u : 0u);
+            uint32_t rank = e;
+            if (!PRESORTED) {
+                rank = 0;
+                for (uint32_t other = 0; other < n_rows; other += 4) {
+                    // every lane reads the same 32 bytes: two LDS broadcasts for four comparisons
+                    const ulonglong2 first_two = *reinterpret_cast<const ulonglong2*>(&sh.keys[other]);
+                    const ulonglong2 next_two = *reinterpret_cast<const ulonglong2*>(&sh.keys[other + 2]);
+                    rank += (first_two.x < key ? 1u : 0u) + (first_two.y < key ? 1u : 0u);
+                    rank += (next_two.x < key ? 1u : 0u) + (next_two.y < key ? 1u : 0u);
+                }
             }
             if (active) {
                 const uint32_t oj = static_cast<uint32_t>(key >> 32);
@@ -386,25 +389,301 @@ __global__ __launch_bounds__(ORDERED_BLOCK) void ordered_search_kernel(OrderedAr
                 const double vx = (xj - xi) + tx;
                 const double vy = (yj - yi) + ty;
                 const double vz = (zj - zi) + tz;
+                // PRESORTED: consecutive lanes, consecutive rows
                 const uint64_t row = first_row + rank;
-                args.out.pairs[2 * row + 0] = oi;
-                args.out.pairs[2 * row + 1] = oj;
+                stream_store(args.out.pairs + 2 * row, PairRow{oi, oj});
                 if (args.out.shifts != nullptr) {
-                    args.out.shifts[3 * row + 0] = sx;
-                    args.out.shifts[3 * row + 1] = sy;
-                    args.out.shifts[3 * row + 2] = sz;
+                    stream_store(args.out.shifts + 3 * row, ShiftRow{sx, sy, sz});
                 }
                 if (args.out.distances != nullptr) {
-                    args.out.distances[row] = sqrt(vx * vx + vy * vy + vz * vz);
+                    stream_store(args.out.distances + row, sqrt(vx * vx + vy * vy + vz * vz));
                 }
                 if (args.out.vectors != nullptr) {
-                    args.out.vectors[3 * row + 0] = vx;
-                    args.out.vectors[3 * row + 1] = vy;
-                    args.out.vectors[3 * row + 2] = vz;
+                    stream_store(args.out.vectors + 3 * row, VectorHead{vx, vy});
+                    stream_store(args.out.vectors + 3 * row + 2, vz);
                 }
             }
         }
         wave_sync(); // the keys are about to be overwritten by the next point's
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// SORT: the order of a tile's candidates
+
+constexpr int ORDER_WAVES = 4;
+constexpr int ORDER_BLOCK = ORDER_WAVES * WAVE;
+constexpr uint32_t ORDER_BUCKETS = 4 * WAVE;
+constexpr uint32_t ORDER_BITS = 64 * 1024;        // original indices the bit set covers at a time
+constexpr uint32_t ORDER_WORDS = ORDER_BITS / 32;
+constexpr uint32_t ORDER_ROUNDS = 4;              // the window of indices ranked through the bit set: that many times ORDER_BITS
+
+/// LDS of one wave, used in one of two ways.
+union OrderScratch {
+    struct {
+        uint32_t index_of[ORDERED_CANDIDATES];      // original index by candidate number
+        uint32_t grouped_index[ORDERED_CANDIDATES]; // original indices grouped by bucket
+        uint16_t grouped[ORDERED_CANDIDATES];       // candidate numbers, same grouping
+        uint32_t bucket_end[ORDER_BUCKETS];         // counts, then where the next key of the bucket goes, at last its end
+    } buckets;
+    struct {
+        __attribute__((aligned(16))) uint32_t present[ORDER_WORDS]; // one bit per original index of the window
+        uint16_t before[ORDER_WORDS / 4];                           // bits set before each group of four words
+        uint16_t offset[ORDERED_CANDIDATES];                        // by candidate number: its bit ...
+        uint8_t round_of[ORDERED_CANDIDATES];                       // ... in the round that covers its index
+    } bits;
+};
+
+struct OrderWaveShared: SearchTables {
+    OrderScratch scratch;
+};
+
+struct OrderShared {
+    OrderWaveShared wave[ORDER_WAVES];
+};
+
+/// One wave per tile: writes, for every place of the order of the tile's candidates by (original index, shift less
+/// the wrap of the first point), the number of the candidate in the stencil tables.
+///
+/// When the original indices the tile sees fit a window of ORDER_ROUNDS x ORDER_BITS and no point is seen twice (as
+/// two images), the place of a candidate is the number of smaller indices present: one bit per index, counted with
+/// prefix sums, ORDER_BITS indices at a time.
+/// That is the case of inputs ordered like the lattice they were built from, where the candidates come as runs of
+/// consecutive indices; the window may wrap around from the last index to the first, as the neighbourhood of a tile
+/// at the edge of a periodic box does. Otherwise the range is cut into 256 buckets, monotonic in the index, and a
+/// key is only compared with the keys of its own bucket: few when the indices are spread evenly, as they are in
+/// inputs without any order. Loops over the units are kept rolled: this kernel is small work, it should be small
+/// code.
+__global__ __launch_bounds__(ORDER_BLOCK) void ordered_sort_kernel(OrderedArgs args, GridParams g) {
+    __shared__ OrderShared shared;
+    const int lane = lane_id();
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    OrderWaveShared& sh = shared.wave[wave];
+    const uint32_t n_tiles = static_cast<uint32_t>(args.cell_scan[g.n_cells] >> 32);
+    const uint32_t tile_id = blockIdx.x * ORDER_WAVES + wave;
+    if (tile_id >= n_tiles) {
+        return;
+    }
+    const SortedPoints& sorted = args.sorted;
+    const Tile tile = args.tiles[tile_id];
+    const int32_t cx = tile.cell % g.n[0];
+    const int32_t cy = (tile.cell / g.n[0]) % g.n[1];
+    const int32_t cz = tile.cell / (g.n[0] * g.n[1]);
+    const int32_t span_y = 2 * g.s[1] + 1;
+    const int32_t span_z = 2 * g.s[2] + 1;
+    const uint32_t n_stencil = static_cast<uint32_t>(2 * g.s[0] + 1) * span_y * span_z;
+    if (n_stencil > MAX_ENTRIES) {
+        return;
+    }
+    fill_stencil_tables(sh, lane, 0, n_stencil, cx, cy, cz, span_y, span_z, g, args.cell_scan);
+    const uint32_t n_candidates = __builtin_amdgcn_readfirstlane(sh.n_candidates);
+    if (n_candidates > ORDERED_CANDIDATES || n_candidates == 0) {
+        return; // the writing pass is not launched when a tile has too many
+    }
+    uint16_t* tile_order = args.order + static_cast<size_t>(tile_id) * ORDERED_CANDIDATES;
+
+    // the range of original indices, and the same for each half of the index space
+    const uint32_t half = g.n_points / 2;
+    uint32_t lowest = 0xFFFFFFFFu;
+    uint32_t highest = 0;
+    uint32_t upper_lowest = 0xFFFFFFFFu;
+    uint32_t lower_highest = 0;
+#pragma unroll 4
+    for (uint32_t k = lane; k < n_candidates; k += WAVE) {
+        uint32_t at;
+        int32_t packed_q;
+        locate_candidate(sh, n_stencil, k, at, packed_q);
+        const uint32_t index = sorted.index[at];
+        lowest = min(lowest, index);
+        highest = max(highest, index);
+        if (index >= half) {
+            upper_lowest = min(upper_lowest, index);
+        } else {
+            lower_highest = max(lower_highest, index);
+        }
+    }
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) {
+        lowest = min(lowest, static_cast<uint32_t>(__shfl_xor(static_cast<int>(lowest), offset, WAVE)));
+        highest = max(highest, static_cast<uint32_t>(__shfl_xor(static_cast<int>(highest), offset, WAVE)));
+        upper_lowest = min(upper_lowest, static_cast<uint32_t>(__shfl_xor(static_cast<int>(upper_lowest), offset, WAVE)));
+        lower_highest = max(lower_highest, static_cast<uint32_t>(__shfl_xor(static_cast<int>(lower_highest), offset, WAVE)));
+    }
+    lowest = uniform(lowest);
+    highest = uniform(highest);
+    upper_lowest = uniform(upper_lowest);
+    lower_highest = uniform(lower_highest);
+
+    // The window: from `origin` on, ORDER_ROUNDS x ORDER_BITS indices, continuing at index 0 after the last one.
+    // Either the whole range fits, or the indices of the upper half followed by those of the lower half do.
+    constexpr uint32_t WINDOW = ORDER_ROUNDS * ORDER_BITS;
+    uint32_t origin = lowest;
+    uint32_t last = highest - lowest; // of the window
+    if (last >= WINDOW && upper_lowest != 0xFFFFFFFFu && lowest < half &&
+        static_cast<uint64_t>(g.n_points - upper_lowest) + lower_highest < WINDOW) {
+        origin = upper_lowest;
+        last = (g.n_points - upper_lowest) + lower_highest;
+    }
+    bool window = last < WINDOW;
+    // a point can only be seen twice when the stencil wraps around the box along some direction
+    for (int d = 0; d < 3; d++) {
+        window = window && !(g.periodic[d] && g.n[d] < 2 * g.s[d] + 1);
+    }
+    if (lane == 0) {
+        atomicAdd(window ? &args.status->windowed : &args.status->bucketed, 1u);
+    }
+    if (window) {
+        auto& bits = sh.scratch.bits;
+        uint32_t wrapped_around = 0; // candidates below the origin: first in the order, last in the window
+#pragma unroll 4
+        for (uint32_t k = lane; k < n_candidates; k += WAVE) {
+            uint32_t at;
+            int32_t packed_q;
+            locate_candidate(sh, n_stencil, k, at, packed_q);
+            const uint32_t index = sorted.index[at];
+            const uint32_t offset = index >= origin ? index - origin : (g.n_points - origin) + index;
+            wrapped_around += index < origin ? 1u : 0u;
+            bits.offset[k] = static_cast<uint16_t>(offset % ORDER_BITS);
+            bits.round_of[k] = static_cast<uint8_t>(offset / ORDER_BITS);
+        }
+#pragma unroll
+        for (int offset = 32; offset > 0; offset >>= 1) {
+            wrapped_around += static_cast<uint32_t>(__shfl_xor(static_cast<int>(wrapped_around), offset, WAVE));
+        }
+        const uint32_t in_window_first = n_candidates - wrapped_around; // candidates at or above the origin
+        uint32_t carried = 0;                                           // candidates of the rounds before
+        for (uint32_t round = 0; round <= last / ORDER_BITS; round++) {
+            const uint32_t n_groups = (round < last / ORDER_BITS ? ORDER_BITS - 1 : last % ORDER_BITS) / 128 + 1;
+            wave_sync();
+            for (uint32_t group = lane; group < n_groups; group += WAVE) {
+                *reinterpret_cast<uint4*>(&bits.present[4 * group]) = uint4{0u, 0u, 0u, 0u};
+            }
+            wave_sync();
+#pragma unroll 4
+            for (uint32_t k = lane; k < n_candidates; k += WAVE) {
+                if (bits.round_of[k] == round) {
+                    const uint32_t offset = bits.offset[k];
+                    atomicOr(&bits.present[offset / 32], 1u << (offset % 32));
+                }
+            }
+            wave_sync();
+            const uint32_t carried_in = carried;
+            for (uint32_t group0 = 0; group0 < n_groups; group0 += WAVE) {
+                const uint32_t group = group0 + lane;
+                uint32_t here = 0;
+                if (group < n_groups) {
+                    const uint4 words = *reinterpret_cast<const uint4*>(&bits.present[4 * group]);
+                    here = __popc(words.x) + __popc(words.y) + __popc(words.z) + __popc(words.w);
+                }
+                const uint32_t through = wave_inclusive_scan(here);
+                if (group < n_groups) {
+                    bits.before[group] = static_cast<uint16_t>(carried + through - here);
+                }
+                carried += read_lane(through, WAVE - 1);
+            }
+            wave_sync();
+            if (carried == carried_in) {
+                continue; // no candidate in this stretch of the window
+            }
+#pragma unroll 4
+            for (uint32_t k = lane; k < n_candidates; k += WAVE) {
+                if (bits.round_of[k] == round) {
+                    const uint32_t offset = bits.offset[k];
+                    const uint32_t word = offset / 32;
+                    const uint4 words = *reinterpret_cast<const uint4*>(&bits.present[word & ~3u]);
+                    uint32_t place = bits.before[word / 4];
+                    place += (word % 4 > 0) ? __popc(words.x) : 0;
+                    place += (word % 4 > 1) ? __popc(words.y) : 0;
+                    place += (word % 4 > 2) ? __popc(words.z) : 0;
+                    const uint32_t own = word % 4 == 0 ? words.x : word % 4 == 1 ? words.y : word % 4 == 2 ? words.z : words.w;
+                    place += __popc(own & ((1u << (offset % 32)) - 1u));
+                    // the window's order starts at the origin, the order of the indices with those that wrapped around
+                    place = place >= in_window_first ? place - in_window_first : place + wrapped_around;
+                    tile_order[min(place, ORDERED_CANDIDATES - 1)] = static_cast<uint16_t>(k);
+                }
+            }
+        }
+        return;
+    }
+
+    auto& buckets = sh.scratch.buckets;
+    const float per_index = static_cast<float>(ORDER_BUCKETS) / (static_cast<float>(highest - lowest) + 1.0f);
+    auto bucket_of = [&](uint32_t index) {
+        return min(ORDER_BUCKETS - 1, static_cast<uint32_t>(static_cast<float>(index - lowest) * per_index));
+    };
+    // the shift of a candidate, as it is ordered: only ever needed to tell two images of one point apart
+    auto biased_of = [&](uint32_t k) {
+        uint32_t at;
+        int32_t packed_q;
+        locate_candidate(sh, n_stencil, k, at, packed_q);
+        int32_t qx, qy, qz;
+        unpack_shift(packed_q, qx, qy, qz);
+        // shifts beyond the key's fields make the counting pass call the whole search off: only memory safety
+        // matters for them here
+        return biased_shift(qx - sorted.wx[at], qy - sorted.wy[at], qz - sorted.wz[at]);
+    };
+#pragma unroll
+    for (uint32_t b = 0; b < ORDER_BUCKETS / WAVE; b++) {
+        buckets.bucket_end[b * WAVE + lane] = 0;
+    }
+    wave_sync();
+#pragma unroll 4
+    for (uint32_t k = lane; k < n_candidates; k += WAVE) {
+        uint32_t at;
+        int32_t packed_q;
+        locate_candidate(sh, n_stencil, k, at, packed_q);
+        const uint32_t index = sorted.index[at];
+        buckets.index_of[k] = index;
+        atomicAdd(&buckets.bucket_end[bucket_of(index)], 1u);
+    }
+    wave_sync();
+    // lane l owns buckets 4l .. 4l+3
+    uint32_t in_bucket[ORDER_BUCKETS / WAVE];
+    uint32_t mine = 0;
+#pragma unroll
+    for (uint32_t b = 0; b < ORDER_BUCKETS / WAVE; b++) {
+        in_bucket[b] = buckets.bucket_end[(ORDER_BUCKETS / WAVE) * lane + b];
+        mine += in_bucket[b];
+    }
+    uint32_t before = wave_inclusive_scan(mine) - mine;
+#pragma unroll
+    for (uint32_t b = 0; b < ORDER_BUCKETS / WAVE; b++) {
+        buckets.bucket_end[(ORDER_BUCKETS / WAVE) * lane + b] = before;
+        before += in_bucket[b];
+    }
+    wave_sync();
+#pragma unroll 4
+    for (uint32_t k = lane; k < n_candidates; k += WAVE) {
+        const uint32_t index = buckets.index_of[k];
+        const uint32_t slot = min(atomicAdd(&buckets.bucket_end[bucket_of(index)], 1u), ORDERED_CANDIDATES - 1);
+        buckets.grouped_index[slot] = index;
+        buckets.grouped[slot] = static_cast<uint16_t>(k);
+    }
+    wave_sync();
+    // every bucket now ends where the next one starts
+#pragma unroll 2
+    for (uint32_t slot = lane; slot < n_candidates; slot += WAVE) {
+        const uint32_t index = buckets.grouped_index[slot];
+        const uint32_t k = buckets.grouped[slot];
+        const uint32_t bucket = bucket_of(index);
+        const uint32_t first = bucket == 0 ? 0u : min(buckets.bucket_end[bucket - 1], ORDERED_CANDIDATES);
+        const uint32_t end = min(buckets.bucket_end[bucket], ORDERED_CANDIDATES);
+        uint32_t place = first;
+        bool twice = false;
+        for (uint32_t other = first; other < end; other++) {
+            const uint32_t theirs = buckets.grouped_index[other];
+            place += theirs < index ? 1u : 0u;
+            twice = twice || (theirs == index && other != slot);
+        }
+        if (twice) {
+            const uint32_t own = biased_of(k);
+            for (uint32_t other = first; other < end; other++) {
+                if (buckets.grouped_index[other] == index && other != slot) {
+                    place += biased_of(buckets.grouped[other]) < own ? 1u : 0u;
+                }
+            }
+        }
+        tile_order[min(place, ORDERED_CANDIDATES - 1)] = static_cast<uint16_t>(k);
     }
 }
 
