@@ -172,6 +172,24 @@ int VESIN_API vesin_hip_neighbors_batch(
     const char** error_message
 );
 
+/* vesin_hip_neighbors_batch with its GPU work (kernels and the small copies to and from the host) on the HIP
+ * stream `stream` (a hipStream_t; NULL is the null stream) of the list's device, like
+ * vesin_hip_neighbors_on_stream: everything queued on that stream before the call is seen, the results are complete
+ * on return, other streams are neither waited for nor held up. No counterpart in the reference. */
+int VESIN_API vesin_hip_neighbors_batch_on_stream(
+    const double (*points)[3],
+    const size_t* first_point,
+    size_t n_systems,
+    const double (*boxes)[3][3],
+    const bool (*periodic)[3],
+    struct VesinDevice device,
+    struct VesinOptions options,
+    struct VesinNeighborList* neighbors,
+    size_t* first_pair,
+    void* stream,
+    const char** error_message
+);
+
 /* Gradient of the pair geometry: given dE/d(distances) and dE/d(vectors) of some scalar E for the rows of a list,
  * ADD dE/d(points) and dE/d(box) to `points_grad` and `box_grad` (the caller zeroes them, or accumulates):
  *     g_k = vectors_grad[k] + distances_grad[k] * vectors[k] / distances[k]

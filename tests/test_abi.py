@@ -179,6 +179,11 @@ def test_validation_of_the_additions():
         address, first_point, 1, address, address, cpu, options, ctypes.byref(neighbors), first_pair, ctypes.byref(message)
     )
     assert status == 1 and "only computed on a GPU device" in text(message)
+    message = ctypes.c_char_p()
+    status = lib.vesin_hip_neighbors_batch_on_stream(
+        address, first_point, 1, address, address, gpu, options, ctypes.byref(neighbors), None, None, ctypes.byref(message)
+    )
+    assert (status, text(message)) == (1, "`first_pair` can not be a NULL pointer")
     with_skin = _c_api.VesinOptions()
     with_skin.cutoff = 1.0
     with_skin.skin = 0.2

@@ -1,5 +1,6 @@
-"""vesin_hip_neighbors_on_stream: the same calculation issued on a stream of the caller's instead of the null
-stream (the reference works on the null stream only, vesin/src/vesin_cuda.cpp:793-803)."""
+"""vesin_hip_neighbors_on_stream and vesin_hip_neighbors_batch_on_stream: the same calculations issued on a stream
+of the caller's instead of the null stream (the reference works on the null stream only,
+vesin/src/vesin_cuda.cpp:793-803)."""
 
 import ctypes
 import threading
@@ -135,5 +136,56 @@ def test_null_stream_handle_is_the_plain_call():
         result = _to_host(neighbors)
         for key in ("pairs", "shifts", "distances", "vectors"):
             assert np.array_equal(result[key], expected[key]), key
+    finally:
+        lib.vesin_free(ctypes.byref(neighbors))
+
+
+def test_batch_with_inputs_produced_on_the_same_stream():
+    import torch
+
+    lib = get_library()
+    rng = np.random.default_rng(33)
+    systems = []
+    for s in range(40):
+        n = int(rng.integers(1, 90))
+        box = np.diag(rng.uniform(6.0, 12.0, size=3)) + rng.uniform(-0.5, 0.5, size=(3, 3))
+        flags = [True, True, True] if s % 3 else [bool(f) for f in rng.integers(0, 2, size=3)]
+        systems.append((rng.random((n, 3)) @ box, box, flags))
+    first_point = np.zeros(len(systems) + 1, dtype=np.uint64)
+    first_point[1:] = np.cumsum([len(p) for p, _, _ in systems])
+    host_points = torch.tensor(np.concatenate([p for p, _, _ in systems])).pin_memory()
+    host_boxes = torch.tensor(np.stack([b for _, b, _ in systems])).pin_memory()
+    host_flags = torch.tensor(np.array([f for _, _, f in systems], dtype=np.bool_)).pin_memory()
+    expected = [oracle.canonicalize(oracle.neighbors(p, b, f, 4.0, False, False, "ijSdD")) for p, b, f in systems]
+    torch.cuda.synchronize()
+
+    options = _options(4.0, full=False, sorted=False)
+    stream = torch.cuda.Stream()
+    neighbors = VesinNeighborList()
+    first_pair = np.zeros(len(systems) + 1, dtype=np.uint64)
+    try:
+        for _ in range(3):  # two passes first, then the single pass into the arrays that are kept
+            with torch.cuda.stream(stream):
+                filler = torch.zeros((4096, 4096), device="cuda:0")
+                for _ in range(20):
+                    filler = filler * 1.0001 + 1.0
+                device_points = host_points.to("cuda:0", non_blocking=True) + 0.0
+                device_boxes = host_boxes.to("cuda:0", non_blocking=True) + 0.0
+                device_flags = host_flags.to("cuda:0", non_blocking=True).clone()
+            message = ctypes.c_char_p()
+            status = lib.vesin_hip_neighbors_batch_on_stream(
+                device_points.data_ptr(), first_point.ctypes.data_as(ctypes.POINTER(ctypes.c_size_t)), len(systems),
+                device_boxes.data_ptr(), device_flags.data_ptr(), VesinDevice(VesinCUDA, 0), options,
+                ctypes.byref(neighbors), first_pair.ctypes.data_as(ctypes.POINTER(ctypes.c_size_t)), stream.cuda_stream,
+                ctypes.byref(message),
+            )
+            assert status == 0, message.value
+            result = _to_host(neighbors)
+            assert first_pair[-1] == neighbors.length
+            for s, want in enumerate(expected):
+                rows = slice(int(first_pair[s]), int(first_pair[s + 1]))
+                got = oracle.canonicalize({key: value[rows] for key, value in result.items()})
+                for key in ("pairs", "shifts", "distances", "vectors"):
+                    assert np.array_equal(got[key], want[key]), (s, key)
     finally:
         lib.vesin_free(ctypes.byref(neighbors))

@@ -102,6 +102,20 @@ def get_library():
             ctypes.POINTER(ctypes.c_size_t),
             ctypes.POINTER(ctypes.c_char_p),
         ]
+        lib.vesin_hip_neighbors_batch_on_stream.restype = ctypes.c_int
+        lib.vesin_hip_neighbors_batch_on_stream.argtypes = [
+            ctypes.c_void_p,
+            ctypes.POINTER(ctypes.c_size_t),
+            ctypes.c_size_t,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            VesinDevice,
+            VesinOptions,
+            ctypes.POINTER(VesinNeighborList),
+            ctypes.POINTER(ctypes.c_size_t),
+            ctypes.c_void_p,
+            ctypes.POINTER(ctypes.c_char_p),
+        ]
         lib.vesin_hip_pairs_backward.restype = ctypes.c_int
         lib.vesin_hip_pairs_backward.argtypes = [
             ctypes.c_void_p,

@@ -123,7 +123,7 @@ extern "C" int vesin_hip_neighbors_on_stream(
     return neighbors_on(points, n_points, box, periodic, device, options, neighbors, stream, error_message);
 }
 
-extern "C" int vesin_hip_neighbors_batch(
+static int neighbors_batch_on(
     const double (*points)[3],
     const size_t* first_point,
     size_t n_systems,
@@ -133,6 +133,7 @@ extern "C" int vesin_hip_neighbors_batch(
     VesinOptions options,
     VesinNeighborList* neighbors,
     size_t* first_pair,
+    void* stream,
     const char** error_message
 ) {
     if (error_message == nullptr) {
@@ -182,7 +183,7 @@ extern "C" int vesin_hip_neighbors_batch(
         if (neighbors->device.type == VesinUnknownDevice) {
             neighbors->device = device;
         }
-        vesin_hip::neighbors_batch(points, first_point, n_systems, boxes, periodic, options, *neighbors, first_pair);
+        vesin_hip::neighbors_batch(points, first_point, n_systems, boxes, periodic, options, *neighbors, first_pair, stream);
     } catch (const std::bad_alloc&) {
         LAST_ERROR = "failed to allocate memory";
         *error_message = LAST_ERROR.c_str();
@@ -195,6 +196,41 @@ extern "C" int vesin_hip_neighbors_batch(
         return fail(error_message, "fatal error: unknown type thrown as exception");
     }
     return EXIT_SUCCESS;
+}
+
+extern "C" int vesin_hip_neighbors_batch(
+    const double (*points)[3],
+    const size_t* first_point,
+    size_t n_systems,
+    const double (*boxes)[3][3],
+    const bool (*periodic)[3],
+    VesinDevice device,
+    VesinOptions options,
+    VesinNeighborList* neighbors,
+    size_t* first_pair,
+    const char** error_message
+) {
+    return neighbors_batch_on(
+        points, first_point, n_systems, boxes, periodic, device, options, neighbors, first_pair, nullptr, error_message
+    );
+}
+
+extern "C" int vesin_hip_neighbors_batch_on_stream(
+    const double (*points)[3],
+    const size_t* first_point,
+    size_t n_systems,
+    const double (*boxes)[3][3],
+    const bool (*periodic)[3],
+    VesinDevice device,
+    VesinOptions options,
+    VesinNeighborList* neighbors,
+    size_t* first_pair,
+    void* stream,
+    const char** error_message
+) {
+    return neighbors_batch_on(
+        points, first_point, n_systems, boxes, periodic, device, options, neighbors, first_pair, stream, error_message
+    );
 }
 
 extern "C" int vesin_hip_pairs_backward(

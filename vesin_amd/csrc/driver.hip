@@ -1447,7 +1447,8 @@ void neighbors_batch(
     const bool (*periodic)[3],
     VesinOptions options,
     VesinNeighborList& neighbors,
-    size_t* first_pair
+    size_t* first_pair,
+    void* caller_stream
 ) {
     const int device_id = neighbors.device.device_id;
     int device_count = 0;
@@ -1490,14 +1491,15 @@ void neighbors_batch(
     HipExtras& extras = extras_of(neighbors);
     extras.timings_valid = false;
     extras.have_last_box = false; // the work buffers of the single-system path are about to be reused
-    hipStream_t stream = nullptr;
+    hipStream_t stream = static_cast<hipStream_t>(caller_stream);
     const size_t pair_limit = pairs_per_point_limit();
 
     // ---- every system's box comes to the host: the grids are picked there
     std::vector<double> host_boxes(9 * n_systems);
     std::vector<unsigned char> host_periodic(3 * n_systems);
-    HIP_CHECK(hipMemcpy(host_boxes.data(), boxes, host_boxes.size() * sizeof(double), hipMemcpyDeviceToHost));
-    HIP_CHECK(hipMemcpy(host_periodic.data(), periodic, host_periodic.size(), hipMemcpyDeviceToHost));
+    HIP_CHECK(hipMemcpyAsync(host_boxes.data(), boxes, host_boxes.size() * sizeof(double), hipMemcpyDeviceToHost, stream));
+    HIP_CHECK(hipMemcpyAsync(host_periodic.data(), periodic, host_periodic.size(), hipMemcpyDeviceToHost, stream));
+    HIP_CHECK(hipStreamSynchronize(stream));
 
     std::vector<GridParams> grids(n_systems);
     std::vector<HostBox> host_grids_box(n_systems);

@@ -31,7 +31,8 @@ void neighbors_batch(
     const bool (*periodic)[3],
     VesinOptions options,
     VesinNeighborList& neighbors,
-    size_t* first_pair
+    size_t* first_pair,
+    void* stream
 );
 
 /// Adds the gradient of a scalar with respect to points and box, given its gradient with respect to the distances
