@@ -1051,6 +1051,7 @@ bool compute(
         oargs.order = candidate_order;
         oargs.first_row = first_row_of_point;
         oargs.status = ordered_status;
+        oargs.report_order = std::getenv("VESIN_HIP_DEBUG") != nullptr ? 1u : 0u;
         const uint32_t blocks = ordered_blocks;
         if (options.full) {
             hipLaunchKernelGGL((ordered_search_kernel<false, true>), dim3(blocks), dim3(ORDERED_BLOCK), 0, stream, oargs, g);

@@ -60,6 +60,7 @@ struct OrderedArgs {
     uint16_t* order;            // SORT -> WRITE: [tile][ORDERED_CANDIDATES], candidate number at each place of the order
     const uint64_t* first_row;  // WRITE: [n_points + 1], exclusive scan of rows_of_point
     OrderedStatus* status;
+    uint32_t report_order;      // SORT: count the tiles ordered either way (an atomic per tile on one word: for tests)
     SearchOutputs out;
 };
 
@@ -89,12 +90,74 @@ __device__ __forceinline__ bool beyond(int32_t a, int32_t b, int32_t c, int32_t 
     return a > limit || a < -limit || b > limit || b < -limit || c > limit || c < -limit;
 }
 
+/// Original indices of four consecutive cell-sorted points in scalar registers (wave-uniform address; reading
+/// past the end of a tile is harmless: the arrays are padded).
+__device__ __forceinline__ uint4 load_four_indices(const uint32_t* index) {
+    uint4 four;
+    asm volatile("s_load_dwordx4 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=&s"(four) : "s"(index));
+    return four;
+}
+
+/// sweep_columns for the counting pass of the in-order search, for a tile without wrapped points: what the
+/// distance test does not decide is decided per test as well, and the rows of every point are counted on the way.
+///   - candidate lanes whose `c.position` is the position of the point under test sit out: a point is no
+///     neighbour of itself, and a half list keeps a point with its own image under the rule of the reference only;
+///   - a half list keeps the orientation whose first index is the smaller one (!FULL);
+///   - lane p of `rows` adds up the hits of the item's point p (a scalar population count per test).
+template <int R, bool SHIFTED, bool FULL>
+__device__ __forceinline__ void sweep_and_count(
+    const SortedPoints& sorted, uint32_t first, uint32_t count, const SweepCandidates<R>& c, double cutoff2,
+    const uint32_t (&original)[R], int lane, uint32_t (&column)[R], uint32_t& rows
+) {
+    for (uint32_t i0 = 0; i0 < count; i0 += POINTS_PER_LOAD) {
+        const uint32_t at = first + i0;
+        const FourPoints p = load_four_points(sorted.x + at, sorted.y + at, sorted.z + at);
+        uint4 indices = uint4{0u, 0u, 0u, 0u};
+        if (!FULL) {
+            indices = load_four_indices(sorted.index + at);
+        }
+#pragma unroll
+        for (int u = 0; u < POINTS_PER_LOAD; u++) {
+            if (u > 0 && i0 + u >= count) {
+                break;
+            }
+            const double xi = words_to_double(p.x[2 * u], p.x[2 * u + 1]);
+            const double yi = words_to_double(p.y[2 * u], p.y[2 * u + 1]);
+            const double zi = words_to_double(p.z[2 * u], p.z[2 * u + 1]);
+            const uint32_t index_i = u == 0 ? indices.x : u == 1 ? indices.y : u == 2 ? indices.z : indices.w;
+            uint32_t found = 0;
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                double vx = c.x[r] - xi;
+                double vy = c.y[r] - yi;
+                double vz = c.z[r] - zi;
+                if (SHIFTED) {
+                    vx += c.tx[r];
+                    vy += c.ty[r];
+                    vz += c.tz[r];
+                }
+                const double d2 = vx * vx + vy * vy + vz * vz;
+                uint64_t mask = __ballot(d2 < cutoff2) & __ballot(c.position[r] != at + u);
+                if (!FULL) {
+                    mask &= __ballot(index_i <= original[r]);
+                }
+                found += __popcll(mask);
+                column[r] = shift_in(column[r], mask);
+            }
+            if (static_cast<uint32_t>(lane) == i0 + u) {
+                rows += found;
+            }
+        }
+    }
+}
+
 /// Two units of candidates (numbers unit0 * 64 ... + 127 of the tables) against the item's points: hit columns
-/// (the item's first point in the highest bit used).
+/// (the item's first point in the highest bit used); lane p of `rows` adds up the hits of the item's point p.
 template <bool FULL, bool WRAPPED>
 __device__ __forceinline__ void ordered_sweep_pair(
     const OrderedWaveShared& sh, const SortedPoints& sorted, const GridParams& g, uint32_t unit0, uint32_t n_stencil,
-    uint32_t n_candidates, uint32_t first_i, uint32_t n_i, int lane, uint32_t (&column)[ORDERED_R], bool& out_of_range
+    uint32_t n_candidates, uint32_t first_i, uint32_t n_i, int lane, uint32_t (&column)[ORDERED_R], uint32_t& rows,
+    bool& out_of_range
 ) {
     constexpr int R = ORDERED_R;
     SweepCandidates<R> c;
@@ -107,7 +170,9 @@ __device__ __forceinline__ void ordered_sweep_pair(
         c.x[r] = c.y[r] = c.z[r] = __builtin_nan("");
         c.tx[r] = c.ty[r] = c.tz[r] = 0.0;
         c.shift[r] = 0;
-        c.position[r] = 0xFFFFFFFFu; // no candidate is left to another tile: the whole stencil is this tile's
+        // sweep_columns_wrapped: no candidate is left to another tile, the whole stencil is this tile's;
+        // sweep_and_count: the position of the candidate when it must not pair with itself
+        c.position[r] = 0xFFFFFFFFu;
         column[r] = 0;
         at[r] = 0xFFFFFFFFu;
         original[r] = 0;
@@ -126,6 +191,13 @@ __device__ __forceinline__ void ordered_sweep_pair(
             bz = qz - sorted.wz[at[r]];
             c.shift[r] = pack_shift(bx, by, bz);
             out_of_range = out_of_range || beyond(bx, by, bz, ORDERED_SHIFT_LIMIT);
+            if (!WRAPPED) {
+                // a point is no neighbour of itself (of its images it is: the unshifted entry of the tile's own
+                // cell is meant); a half list keeps a point with its own image under the rule of the reference
+                // (the total shift of such a pair is the cell shift)
+                const bool never_with_itself = (qx | qy | qz) == 0 || (!FULL && !half_keeps_self_image(qx, qy, qz));
+                c.position[r] = never_with_itself ? at[r] : 0xFFFFFFFFu;
+            }
         }
         any_shift = any_shift || (__ballot((bx | by | bz) != 0) != 0);
         if (!WRAPPED && any_shift) {
@@ -133,14 +205,16 @@ __device__ __forceinline__ void ordered_sweep_pair(
         }
     }
 
-    if (WRAPPED) {
-        (void)sweep_columns_wrapped<R>(sorted, first_i, n_i, c, g, column);
-    } else if (any_shift) {
-        (void)sweep_columns<R, true, false>(sorted, first_i, n_i, c, g.cutoff2, column);
-    } else {
-        (void)sweep_columns<R, false, false>(sorted, first_i, n_i, c, g.cutoff2, column);
+    if (!WRAPPED) {
+        if (any_shift) {
+            sweep_and_count<R, true, FULL>(sorted, first_i, n_i, c, g.cutoff2, original, lane, column, rows);
+        } else {
+            sweep_and_count<R, false, FULL>(sorted, first_i, n_i, c, g.cutoff2, original, lane, column, rows);
+        }
+        return;
     }
 
+    (void)sweep_columns_wrapped<R>(sorted, first_i, n_i, c, g, column);
     // what the distance test alone does not decide
 #pragma unroll
     for (int r = 0; r < R; r++) {
@@ -164,6 +238,17 @@ __device__ __forceinline__ void ordered_sweep_pair(
             if (is_own && !half_keeps_self_image(qx, qy, qz)) {
                 column[r] &= ~own_bit;
             }
+        }
+    }
+    for (uint32_t p = 0; p < n_i; p++) {
+        const uint32_t bit = n_i - 1 - p;
+        uint32_t found = 0;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            found += __popcll(__ballot(((column[r] >> bit) & 1u) != 0));
+        }
+        if (static_cast<uint32_t>(lane) == p) {
+            rows += found;
         }
     }
 }
@@ -237,7 +322,8 @@ __global__ __launch_bounds__(ORDERED_BLOCK) void ordered_search_kernel(OrderedAr
     const uint32_t n_units = (n_candidates + WAVE - 1) / WAVE;
 
     if (!WRITE) {
-        if (lane == 0 && item == 0) {
+        // thousands of waves report to the same words: an atomic only where it would change something
+        if (lane == 0 && item == 0 && n_candidates > __atomic_load_n(&args.status->max_candidates, __ATOMIC_RELAXED)) {
             atomicMax(&args.status->max_candidates, n_candidates);
         }
     }
@@ -254,28 +340,17 @@ __global__ __launch_bounds__(ORDERED_BLOCK) void ordered_search_kernel(OrderedAr
             uint32_t column[R];
             if (tile_wrapped) {
                 ordered_sweep_pair<FULL, true>(
-                    sh, sorted, g, unit0, n_stencil, n_candidates, first_i, n_i, lane, column, out_of_range
+                    sh, sorted, g, unit0, n_stencil, n_candidates, first_i, n_i, lane, column, own_rows, out_of_range
                 );
             } else {
                 ordered_sweep_pair<FULL, false>(
-                    sh, sorted, g, unit0, n_stencil, n_candidates, first_i, n_i, lane, column, out_of_range
+                    sh, sorted, g, unit0, n_stencil, n_candidates, first_i, n_i, lane, column, own_rows, out_of_range
                 );
             }
 #pragma unroll
             for (int r = 0; r < R; r++) {
                 if (unit0 + r < n_units) {
                     __builtin_nontemporal_store(column[r], &item_columns[(unit0 + r) * WAVE + lane]);
-                }
-            }
-            for (uint32_t p = 0; p < n_i; p++) {
-                const uint32_t bit = n_i - 1 - p;
-                uint32_t rows = 0;
-#pragma unroll
-                for (int r = 0; r < R; r++) {
-                    rows += __popcll(__ballot(((column[r] >> bit) & 1u) != 0));
-                }
-                if (static_cast<uint32_t>(lane) == p) {
-                    own_rows += rows;
                 }
             }
         }
@@ -287,7 +362,7 @@ __global__ __launch_bounds__(ORDERED_BLOCK) void ordered_search_kernel(OrderedAr
         for (int offset = 32; offset > 0; offset >>= 1) {
             most = max(most, static_cast<uint32_t>(__shfl_xor(static_cast<int>(most), offset, WAVE)));
         }
-        if (lane == 0) {
+        if (lane == 0 && most > __atomic_load_n(&args.status->max_rows, __ATOMIC_RELAXED)) {
             atomicMax(&args.status->max_rows, most);
         }
         if (__ballot(out_of_range) != 0 && lane == 0) {
@@ -529,7 +604,7 @@ __global__ __launch_bounds__(ORDER_BLOCK) void ordered_sort_kernel(OrderedArgs a
     for (int d = 0; d < 3; d++) {
         window = window && !(g.periodic[d] && g.n[d] < 2 * g.s[d] + 1);
     }
-    if (lane == 0) {
+    if (args.report_order != 0 && lane == 0) {
         atomicAdd(window ? &args.status->windowed : &args.status->bucketed, 1u);
     }
     if (window) {
