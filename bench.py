@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0
 
 # HBM bytes moved by ONE launch of the single-pass search kernel on this workload, from rocprofv3 --pmc FETCH_SIZE
 # and WRITE_SIZE runs scaled by a device copy of known size (profiles/fused_search_config1_pmc.txt):
-# 96.1 MB fetched + 3217.7 MB written. Only meaningful for the default 1M-atom workload.
+# 171.1 MB fetched + 3214.8 MB written. Only meaningful for the default 1M-atom workload.
 SEARCH_KERNEL_TRAFFIC_BYTES = 3_385_800_000
 
 
