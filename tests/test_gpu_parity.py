@@ -92,6 +92,39 @@ def test_points_far_outside_the_box():
         assert_same_list(actual, expected, ordered=True, what=algorithm)
 
 
+@pytest.mark.parametrize("shape", ["orthorhombic", "rotated", "sheared", "slab", "flat-cells"])
+@pytest.mark.parametrize("full", [True, False])
+def test_stencils_of_several_cells_per_direction(shape, full):
+    # Boxes much narrower than the cutoff: stencils of radius 2 to 5, different per direction. In a box of
+    # orthogonal vectors the entries at the corners of the stencil cannot hold a neighbour and are dropped; a pair
+    # dropped with them would be missing here. "sheared" has no such shortcut, "rotated" has it although no
+    # component of its matrix is zero, "slab" mixes it with an open direction, "flat-cells" has several cells along
+    # the long direction and images along the short ones. Points lie in and around the box.
+    rng = np.random.default_rng(77)
+    box = np.diag([3.1, 4.3, 5.7])
+    periodic = [True, True, True]
+    n_points = 40
+    if shape == "rotated":
+        q, _ = np.linalg.qr(rng.normal(size=(3, 3)))
+        box = box @ q
+    elif shape == "sheared":
+        box[1, 0] = 0.9
+        box[2, 1] = -1.3
+    elif shape == "slab":
+        periodic = [True, False, True]
+    elif shape == "flat-cells":
+        box = np.diag([3.1, 4.3, 61.0])
+        n_points = 300
+    points = (rng.random((n_points, 3)) * 1.6 - 0.3) @ box
+    for cutoff in (6.0, 9.5):
+        expected = oracle.neighbors(points, box, periodic, cutoff, full, False, "ijSdD")
+        for algorithm in ("cell_list", "brute_force"):
+            actual = gpu_neighbors(points, box, periodic, cutoff, full, False, "ijSdD", algorithm)
+            assert_same_list(actual, expected, what=f"{shape} rc={cutoff} {algorithm}")
+            ordered = gpu_neighbors(points, box, periodic, cutoff, full, True, "ijSdD", algorithm)
+            assert_same_list(ordered, expected, ordered=True, what=f"{shape} rc={cutoff} {algorithm} sorted")
+
+
 def test_coincident_points_are_neighbours():
     # the CPU engine keeps distinct points at zero distance (the reference's CUDA kernel drops them,
     # vesin/src/cuda/cell_list.cu:631); this path follows the CPU

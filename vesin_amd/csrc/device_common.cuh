@@ -30,6 +30,13 @@ struct GridParams {
     int32_t periodic[3];
     uint32_t n_points;
     uint32_t n_cells;
+    // Stencil entries that cannot hold a neighbour (stencils of radius two and more in a box of orthogonal vectors:
+    // the corners of the cube of cells lie outside the cutoff sphere). prune_width2[d] = squared width of a cell
+    // along d; an entry whose cells are at least `gap` whole cells away along d is dropped when the sum over d of
+    // gap^2 * prune_width2[d] exceeds prune_limit. prune = 0: nothing is dropped.
+    double prune_width2[3];
+    double prune_limit;
+    int32_t prune;
 };
 
 /// One row of TILE_POINTS i-points (or fewer) that one wave searches for.

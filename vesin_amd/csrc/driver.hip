@@ -62,6 +62,13 @@ static bool two_pass_only() {
     return text != nullptr && std::strcmp(text, "two-pass") == 0;
 }
 
+/// VESIN_HIP_STENCIL=full searches every cell of a stencil, also those that cannot hold a neighbour (for comparisons
+/// and tests).
+static bool full_stencil_only() {
+    const char* text = std::getenv("VESIN_HIP_STENCIL");
+    return text != nullptr && std::strcmp(text, "full") == 0;
+}
+
 /// VESIN_HIP_CELLS=packed keeps every call on the counting-sort cell build (for comparisons and tests) instead of
 /// the one-pass build with a fixed number of slots per cell that the single-pass search can read.
 static bool packed_cells_only() {
@@ -705,6 +712,10 @@ bool compute(
         g.np_scale[d] = grid.np_scale[d];
     }
     g.n_cells = static_cast<uint32_t>(grid.n_cells);
+    choose_pruning(hbox, grid, options.cutoff, g);
+    if (full_stencil_only()) {
+        g.prune = 0;
+    }
 
     // ---- carve the work buffers
     const size_t n_cells = grid.n_cells;
@@ -1582,6 +1593,10 @@ void neighbors_batch(
         g.cutoff2 = options.cutoff * options.cutoff;
         g.n_points = static_cast<uint32_t>(n_here);
         g.n_cells = static_cast<uint32_t>(grid.n_cells);
+        choose_pruning(hbox, grid, options.cutoff, g);
+        if (full_stencil_only()) {
+            g.prune = 0;
+        }
         cell_base_host[s] = static_cast<uint32_t>(total_cells);
         total_cells += grid.n_cells;
         if (total_cells >= 0xFFFFFFF0ull) {

@@ -225,6 +225,41 @@ inline HostGrid choose_grid(
     return grid;
 }
 
+/// Which stencil entries can be dropped (see GridParams::prune): only decided for boxes whose vectors are orthogonal
+/// to each other (to 1e-12 of their lengths), where distances along the three directions add up in squares, and only
+/// when some direction has a stencil radius of two or more: with radius one every cell of the stencil touches the
+/// centre cell. Two points in cells `k` apart along a direction are more than (k - 1) * width apart along it.
+template <typename Grid>
+inline void choose_pruning(const HostBox& box, const HostGrid& grid, double cutoff, Grid& g) {
+    using namespace detail;
+    g.prune = 0;
+    g.prune_limit = cutoff * cutoff * CELL_MARGIN * CELL_MARGIN;
+    for (int d = 0; d < 3; d++) {
+        g.prune_width2[d] = 0.0;
+    }
+    if (grid.s[0] < 2 && grid.s[1] < 2 && grid.s[2] < 2) {
+        return;
+    }
+    const V3 rows[3] = {get_row(box.H, 0), get_row(box.H, 1), get_row(box.H, 2)};
+    for (int d = 0; d < 3; d++) {
+        const V3 a = rows[d];
+        const V3 b = rows[(d + 1) % 3];
+        const double lengths = std::sqrt(dot(a, a) * dot(b, b));
+        if (!(std::abs(dot(a, b)) <= 1e-12 * lengths)) {
+            return;
+        }
+    }
+    for (int d = 0; d < 3; d++) {
+        const double extent = box.periodic[d] ? box.face[d] : 1.0 / grid.np_scale[d];
+        const double width = extent / static_cast<double>(grid.n[d]);
+        if (!(width > 0.0) || !std::isfinite(width)) {
+            return;
+        }
+        g.prune_width2[d] = width * width;
+    }
+    g.prune = 1;
+}
+
 } // namespace vesin_hip
 
 #endif

@@ -220,6 +220,19 @@ __device__ __forceinline__ void fill_stencil_tables(
                 valid = false;
             }
         }
+        if (g.prune != 0) {
+            // Points lie inside their cells, so two points whose cells are |d| cells apart along a direction are
+            // more than |d| - 1 cell widths apart along it. A millionth of a cell is left for the rounding of the
+            // fractional coordinates that put the points into their cells.
+            const double gx = fmax(static_cast<double>(abs(dx) - 1) - 1e-6, 0.0);
+            const double gy = fmax(static_cast<double>(abs(dy) - 1) - 1e-6, 0.0);
+            const double gz = fmax(static_cast<double>(abs(dz) - 1) - 1e-6, 0.0);
+            const double apart2 =
+                gx * gx * g.prune_width2[0] + gy * gy * g.prune_width2[1] + gz * gz * g.prune_width2[2];
+            if (apart2 > g.prune_limit) {
+                valid = false;
+            }
+        }
         uint32_t start = 0;
         uint32_t count = 0;
         int32_t packed = 0;
