@@ -168,6 +168,63 @@ def test_single_pass_on_a_reused_list_and_its_fallbacks(capfd, monkeypatch):
     assert not report()
 
 
+def test_what_the_host_keeps_between_batches_follows_the_inputs():
+    # One list, many batches: the host keeps the grids it derived from the boxes while boxes, flags and division
+    # into systems stay what they were. Every change of one of them, and of the points alone, must show in the rows.
+    import torch
+
+    rng = np.random.default_rng(91)
+
+    def batch(n_systems, edge, sizes):
+        boxes = [np.diag(edge + rng.random(3)) for _ in range(n_systems)]
+        points = [rng.random((n, 3)) @ box for n, box in zip(sizes, boxes)]
+        return points, boxes
+
+    def check(calculator, points, boxes, periodic, cutoff, what):
+        first_point = np.cumsum([0] + [len(p) for p in points])
+        outputs, first_pair = calculator.compute_batch(
+            torch.as_tensor(np.concatenate(points), device="cuda:0"), first_point,
+            torch.as_tensor(np.stack(boxes), device="cuda:0"), periodic, "PSdD",
+        )
+        whole = {NAMES[q]: out.cpu().numpy() for q, out in zip("PSdD", outputs)}
+        flags = np.broadcast_to(np.asarray(periodic, dtype=bool), (len(points), 3)) if not isinstance(periodic, bool) else None
+        for s, (p, box) in enumerate(zip(points, boxes)):
+            rows = slice(int(first_pair[s]), int(first_pair[s + 1]))
+            per = periodic if flags is None else [bool(f) for f in flags[s]]
+            expected = oracle.neighbors(p, box, per, cutoff, True, False, "ijSdD")
+            assert_same_list({k: v[rows] for k, v in whole.items()}, expected, what=f"{what}, system {s}")
+
+    sizes = [40, 25, 60, 33, 48]
+    points, boxes = batch(5, 6.0, sizes)
+    calculator = NeighborList(cutoff=4.0, full_list=True)
+    check(calculator, points, boxes, True, 4.0, "first batch")
+    check(calculator, points, boxes, True, 4.0, "the same batch again")
+    # a call on one system uses the same work buffer its own way
+    single = calculator.compute(
+        torch.as_tensor(points[2], device="cuda:0"), torch.as_tensor(boxes[2], device="cuda:0"), True, "PSdD"
+    )
+    assert_same_list(
+        {NAMES[q]: out.cpu().numpy() for q, out in zip("PSdD", single)},
+        oracle.neighbors(points[2], boxes[2], True, 4.0, True, False, "ijSdD"), what="one system between two batches",
+    )
+    check(calculator, points, boxes, True, 4.0, "the same batch after a call on one system")
+    moved = [p + 0.3 * rng.normal(size=p.shape) for p in points]
+    check(calculator, moved, boxes, True, 4.0, "same boxes, moved points")
+    other_boxes = [box.copy() for box in boxes]
+    other_boxes[3] = np.diag([9.0, 5.5, 7.0])
+    check(calculator, moved, other_boxes, True, 4.0, "one box changed")
+    regrouped = [moved[0][:30], np.concatenate([moved[0][30:], moved[1]]), moved[2], moved[3], moved[4]]
+    check(calculator, regrouped, other_boxes, True, 4.0, "same boxes, other division into systems")
+    slab = np.array([[True, True, True]] * 4 + [[True, True, False]])
+    check(calculator, regrouped, other_boxes, slab, 4.0, "one system opened along z")
+    check(calculator, [p * 1.0 for p in regrouped], other_boxes, slab, 4.0, "open direction: never kept")
+    check(calculator, regrouped, other_boxes, True, 4.0, "closed again")
+    wider = NeighborList(cutoff=4.0, full_list=True)
+    check(wider, points, boxes, True, 4.0, "another list, first cutoff")
+    wider.cutoff = 7.5
+    check(wider, points, boxes, True, 7.5, "same list and boxes, larger cutoff")
+
+
 def test_batch_of_one_equals_the_single_call():
     points, box, periodic, _ = configs.config1(8)
     calculator = NeighborList(cutoff=5.0, full_list=True)

@@ -132,6 +132,7 @@ struct DeviceGuard {
 struct DeviceBuffer {
     void* ptr = nullptr;
     size_t bytes = 0;
+    uint64_t generation = 0; // counts the allocations: what was written into an earlier one is gone
 
     void reserve(size_t wanted) {
         if (wanted <= bytes) {
@@ -141,6 +142,7 @@ struct DeviceBuffer {
         size_t padded = wanted + wanted / 4;
         HIP_CHECK(hipMalloc(&ptr, padded));
         bytes = padded;
+        generation += 1;
     }
 
     void release() {
@@ -228,8 +230,36 @@ struct VerletCache {
 };
 
 /// Private state of one VesinNeighborList (VesinNeighborList::opaque).
+/// What the host derives from the boxes of a batch of systems, kept between calls: a batch whose boxes, flags and
+/// division into systems are those of the call before (a trajectory at constant volume, the same set of structures
+/// evaluated again) starts its kernels without the host going over the systems one by one again.
+struct BatchSetup {
+    bool valid = false;
+    bool any_open_direction = false;
+    double cutoff = 0.0;
+    int algorithm = 0;
+    std::vector<double> boxes;              // 9 per system, as the caller gave them
+    std::vector<unsigned char> periodic;    // 3 per system
+    std::vector<double> incoming_boxes;     // where a call's boxes land before they are compared
+    std::vector<unsigned char> incoming_periodic;
+    std::vector<size_t> first_point;
+    std::vector<HostBox> host_boxes;        // normalised
+    std::vector<GridParams> grids;
+    std::vector<uint32_t> cell_base;
+    std::vector<uint32_t> first_point32;
+    uint64_t total_cells = 0;
+    // where the last batch left grids, first points and first cells in the work buffer; a call on a single system
+    // carves the same buffer its own way and clears the flag
+    bool on_device = false;
+    const void* d_grids = nullptr;
+    const void* d_first_point = nullptr;
+    const void* d_cell_base = nullptr;
+    uint64_t work_generation = 0;
+};
+
 struct HipExtras {
     int device_id = 0;
+    BatchSetup batch;
     DeviceBuffer work;
     DeviceBuffer sort_work;
     DeviceStatus* d_status = nullptr;
@@ -848,6 +878,7 @@ bool compute(
     extras.work.reserve(measure.used);
     Carver carver(extras.work.ptr);
     carve(carver);
+    extras.batch.on_device = false; // what a batch left in this buffer is about to be overwritten
 
     // ---- cell list
     const uint32_t point_blocks = static_cast<uint32_t>((n_points + BLOCK - 1) / BLOCK);
@@ -1507,103 +1538,143 @@ void neighbors_batch(
     const size_t pair_limit = pairs_per_point_limit();
 
     // ---- every system's box comes to the host: the grids are picked there
-    std::vector<double> host_boxes(9 * n_systems);
-    std::vector<unsigned char> host_periodic(3 * n_systems);
-    HIP_CHECK(hipMemcpyAsync(host_boxes.data(), boxes, host_boxes.size() * sizeof(double), hipMemcpyDeviceToHost, stream));
-    HIP_CHECK(hipMemcpyAsync(host_periodic.data(), periodic, host_periodic.size(), hipMemcpyDeviceToHost, stream));
+    BatchSetup& setup = extras.batch;
+    setup.incoming_boxes.resize(9 * n_systems);
+    setup.incoming_periodic.resize(3 * n_systems);
+    HIP_CHECK(hipMemcpyAsync(
+        setup.incoming_boxes.data(), boxes, setup.incoming_boxes.size() * sizeof(double), hipMemcpyDeviceToHost, stream
+    ));
+    HIP_CHECK(hipMemcpyAsync(
+        setup.incoming_periodic.data(), periodic, setup.incoming_periodic.size(), hipMemcpyDeviceToHost, stream
+    ));
     HIP_CHECK(hipStreamSynchronize(stream));
 
-    std::vector<GridParams> grids(n_systems);
-    std::vector<HostBox> host_grids_box(n_systems);
-    std::vector<uint32_t> cell_base_host(n_systems + 1);
-    std::vector<uint32_t> first_point_host(n_systems + 1);
-    bool any_open_direction = false;
-    for (size_t s = 0; s < n_systems; s++) {
-        bool flags[3];
-        for (int d = 0; d < 3; d++) {
-            flags[d] = host_periodic[3 * s + d] != 0;
-            any_open_direction = any_open_direction || !flags[d];
-        }
-        const HostBox hbox = normalise_box(&host_boxes[9 * s], flags);
-        host_grids_box[s] = hbox;
-        GridParams& g = grids[s];
-        std::memset(&g, 0, sizeof(g));
-        for (int d = 0; d < 3; d++) {
-            for (int e = 0; e < 3; e++) {
-                g.H[3 * d + e] = hbox.H[d][e];
-                g.Hinv[3 * d + e] = hbox.Hinv[d][e];
+    // The grids follow from the boxes, the flags, the division into systems, the cutoff and the algorithm alone,
+    // unless some direction is open: then they also follow the points. Same inputs as the call before: same grids.
+    const bool same_setup =
+        setup.valid && !setup.any_open_direction && setup.cutoff == options.cutoff &&
+        setup.algorithm == static_cast<int>(options.algorithm) && setup.first_point.size() == n_systems + 1 &&
+        std::memcmp(setup.first_point.data(), first_point, (n_systems + 1) * sizeof(size_t)) == 0 &&
+        setup.boxes.size() == setup.incoming_boxes.size() &&
+        std::memcmp(setup.boxes.data(), setup.incoming_boxes.data(), setup.boxes.size() * sizeof(double)) == 0 &&
+        std::memcmp(setup.periodic.data(), setup.incoming_periodic.data(), setup.periodic.size()) == 0;
+
+    std::vector<GridParams>& grids = setup.grids;
+    std::vector<uint32_t>& cell_base_host = setup.cell_base;
+    std::vector<uint32_t>& first_point_host = setup.first_point32;
+    if (!same_setup) {
+        setup.valid = false;
+        setup.on_device = false;
+        setup.boxes.swap(setup.incoming_boxes);
+        setup.periodic.swap(setup.incoming_periodic);
+        setup.first_point.assign(first_point, first_point + n_systems + 1);
+        setup.cutoff = options.cutoff;
+        setup.algorithm = static_cast<int>(options.algorithm);
+        const std::vector<double>& host_boxes = setup.boxes;
+        const std::vector<unsigned char>& host_periodic = setup.periodic;
+
+        grids.resize(n_systems);
+        std::vector<HostBox>& host_grids_box = setup.host_boxes;
+        host_grids_box.resize(n_systems);
+        cell_base_host.resize(n_systems + 1);
+        first_point_host.resize(n_systems + 1);
+        bool any_open_direction = false;
+        for (size_t s = 0; s < n_systems; s++) {
+            bool flags[3];
+            for (int d = 0; d < 3; d++) {
+                flags[d] = host_periodic[3 * s + d] != 0;
+                any_open_direction = any_open_direction || !flags[d];
             }
-            g.periodic[d] = flags[d] ? 1 : 0;
+            const HostBox hbox = normalise_box(&host_boxes[9 * s], flags);
+            host_grids_box[s] = hbox;
+            GridParams& g = grids[s];
+            std::memset(&g, 0, sizeof(g));
+            for (int d = 0; d < 3; d++) {
+                for (int e = 0; e < 3; e++) {
+                    g.H[3 * d + e] = hbox.H[d][e];
+                    g.Hinv[3 * d + e] = hbox.Hinv[d][e];
+                }
+                g.periodic[d] = flags[d] ? 1 : 0;
+            }
+            first_point_host[s] = static_cast<uint32_t>(first_point[s]);
         }
-        first_point_host[s] = static_cast<uint32_t>(first_point[s]);
-    }
-    first_point_host[n_systems] = static_cast<uint32_t>(n_points);
+        first_point_host[n_systems] = static_cast<uint32_t>(n_points);
+        setup.any_open_direction = any_open_direction;
 
-    // ---- systems with a non-periodic direction need the extent of their points along it (reference:
-    // BoundingBox::make_bounding_for, vesin/src/types.hpp:159-200): one wave per system finds it
-    std::vector<BlockBounds> bounds;
-    if (any_open_direction && n_points > 0) {
-        const size_t grids_bytes = (n_systems * sizeof(GridParams) + 255) & ~size_t(255);
-        const size_t firsts_bytes = ((n_systems + 1) * sizeof(uint32_t) + 255) & ~size_t(255);
-        extras.sort_work.reserve(grids_bytes + firsts_bytes + n_systems * sizeof(BlockBounds));
-        char* base = static_cast<char*>(extras.sort_work.ptr);
-        auto* early_grids = reinterpret_cast<GridParams*>(base);
-        auto* early_firsts = reinterpret_cast<uint32_t*>(base + grids_bytes);
-        auto* d_bounds = reinterpret_cast<BlockBounds*>(base + grids_bytes + firsts_bytes);
-        HIP_CHECK(hipMemcpyAsync(early_grids, grids.data(), n_systems * sizeof(GridParams), hipMemcpyHostToDevice, stream));
-        HIP_CHECK(hipMemcpyAsync(
-            early_firsts, first_point_host.data(), (n_systems + 1) * sizeof(uint32_t), hipMemcpyHostToDevice, stream
-        ));
-        const uint32_t blocks = static_cast<uint32_t>((n_systems + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK);
-        hipLaunchKernelGGL(
-            bounding_batch_kernel, dim3(blocks), dim3(BLOCK), 0, stream,
-            reinterpret_cast<const double*>(points), early_grids, early_firsts, static_cast<uint32_t>(n_systems), d_bounds
-        );
-        bounds.resize(n_systems);
-        HIP_CHECK(hipMemcpyAsync(bounds.data(), d_bounds, n_systems * sizeof(BlockBounds), hipMemcpyDeviceToHost, stream));
-        HIP_CHECK(hipStreamSynchronize(stream));
-        unsigned int bad = 0xFFFFFFFFu;
-        for (const BlockBounds& found : bounds) {
-            bad = std::min(bad, found.first_bad_coordinate);
+        // ---- systems with a non-periodic direction need the extent of their points along it (reference:
+        // BoundingBox::make_bounding_for, vesin/src/types.hpp:159-200): one wave per system finds it
+        std::vector<BlockBounds> bounds;
+        if (any_open_direction && n_points > 0) {
+            const size_t grids_bytes = (n_systems * sizeof(GridParams) + 255) & ~size_t(255);
+            const size_t firsts_bytes = ((n_systems + 1) * sizeof(uint32_t) + 255) & ~size_t(255);
+            extras.sort_work.reserve(grids_bytes + firsts_bytes + n_systems * sizeof(BlockBounds));
+            char* base = static_cast<char*>(extras.sort_work.ptr);
+            auto* early_grids = reinterpret_cast<GridParams*>(base);
+            auto* early_firsts = reinterpret_cast<uint32_t*>(base + grids_bytes);
+            auto* d_bounds = reinterpret_cast<BlockBounds*>(base + grids_bytes + firsts_bytes);
+            HIP_CHECK(hipMemcpyAsync(
+                early_grids, grids.data(), n_systems * sizeof(GridParams), hipMemcpyHostToDevice, stream
+            ));
+            HIP_CHECK(hipMemcpyAsync(
+                early_firsts, first_point_host.data(), (n_systems + 1) * sizeof(uint32_t), hipMemcpyHostToDevice, stream
+            ));
+            const uint32_t blocks = static_cast<uint32_t>((n_systems + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK);
+            hipLaunchKernelGGL(
+                bounding_batch_kernel, dim3(blocks), dim3(BLOCK), 0, stream,
+                reinterpret_cast<const double*>(points), early_grids, early_firsts, static_cast<uint32_t>(n_systems),
+                d_bounds
+            );
+            bounds.resize(n_systems);
+            HIP_CHECK(hipMemcpyAsync(
+                bounds.data(), d_bounds, n_systems * sizeof(BlockBounds), hipMemcpyDeviceToHost, stream
+            ));
+            HIP_CHECK(hipStreamSynchronize(stream));
+            unsigned int bad = 0xFFFFFFFFu;
+            for (const BlockBounds& found : bounds) {
+                bad = std::min(bad, found.first_bad_coordinate);
+            }
+            if (bad != 0xFFFFFFFFu) {
+                non_finite_error(points, bad);
+            }
         }
-        if (bad != 0xFFFFFFFFu) {
-            non_finite_error(points, bad);
-        }
-    }
 
-    uint64_t total_cells = 0;
-    const double zeros[3] = {0.0, 0.0, 0.0};
-    for (size_t s = 0; s < n_systems; s++) {
-        const HostBox& hbox = host_grids_box[s];
-        const size_t n_here = first_point[s + 1] - first_point[s];
-        const double* lo = bounds.empty() ? zeros : bounds[s].lo;
-        const double* hi = bounds.empty() ? zeros : bounds[s].hi;
-        bool single_cell = options.algorithm == VesinBruteForce;
-        HostGrid grid = choose_grid(hbox, options.cutoff, n_here, lo, hi, single_cell);
-        if (options.algorithm == VesinAutoAlgorithm && !single_cell && (grid.n_cells == 1 || n_here < 32)) {
-            grid = choose_grid(hbox, options.cutoff, n_here, lo, hi, true);
+        uint64_t cells_so_far = 0;
+        const double zeros[3] = {0.0, 0.0, 0.0};
+        for (size_t s = 0; s < n_systems; s++) {
+            const HostBox& hbox = host_grids_box[s];
+            const size_t n_here = first_point[s + 1] - first_point[s];
+            const double* lo = bounds.empty() ? zeros : bounds[s].lo;
+            const double* hi = bounds.empty() ? zeros : bounds[s].hi;
+            bool single_cell = options.algorithm == VesinBruteForce;
+            HostGrid grid = choose_grid(hbox, options.cutoff, n_here, lo, hi, single_cell);
+            if (options.algorithm == VesinAutoAlgorithm && !single_cell && (grid.n_cells == 1 || n_here < 32)) {
+                grid = choose_grid(hbox, options.cutoff, n_here, lo, hi, true);
+            }
+            GridParams& g = grids[s];
+            for (int d = 0; d < 3; d++) {
+                g.n[d] = grid.n[d];
+                g.s[d] = grid.s[d];
+                g.np_min[d] = grid.np_min[d];
+                g.np_scale[d] = grid.np_scale[d];
+            }
+            g.cutoff2 = options.cutoff * options.cutoff;
+            g.n_points = static_cast<uint32_t>(n_here);
+            g.n_cells = static_cast<uint32_t>(grid.n_cells);
+            choose_pruning(hbox, grid, options.cutoff, g);
+            if (full_stencil_only()) {
+                g.prune = 0;
+            }
+            cell_base_host[s] = static_cast<uint32_t>(cells_so_far);
+            cells_so_far += grid.n_cells;
+            if (cells_so_far >= 0xFFFFFFF0ull) {
+                throw std::runtime_error("too many cells in this batch");
+            }
         }
-        GridParams& g = grids[s];
-        for (int d = 0; d < 3; d++) {
-            g.n[d] = grid.n[d];
-            g.s[d] = grid.s[d];
-            g.np_min[d] = grid.np_min[d];
-            g.np_scale[d] = grid.np_scale[d];
-        }
-        g.cutoff2 = options.cutoff * options.cutoff;
-        g.n_points = static_cast<uint32_t>(n_here);
-        g.n_cells = static_cast<uint32_t>(grid.n_cells);
-        choose_pruning(hbox, grid, options.cutoff, g);
-        if (full_stencil_only()) {
-            g.prune = 0;
-        }
-        cell_base_host[s] = static_cast<uint32_t>(total_cells);
-        total_cells += grid.n_cells;
-        if (total_cells >= 0xFFFFFFF0ull) {
-            throw std::runtime_error("too many cells in this batch");
-        }
+        cell_base_host[n_systems] = static_cast<uint32_t>(cells_so_far);
+        setup.total_cells = cells_so_far;
+        setup.valid = true;
     }
-    cell_base_host[n_systems] = static_cast<uint32_t>(total_cells);
+    const uint64_t total_cells = setup.total_cells;
 
     if (n_points == 0) {
         size_outputs(neighbors, extras, 0, options);
@@ -1636,6 +1707,9 @@ void neighbors_batch(
         if (wanted > n_slices) {
             n_slices = static_cast<uint32_t>(std::min(256.0, wanted));
         }
+    }
+    if (const char* text = std::getenv("VESIN_HIP_EXPERIMENT_SLICES")) {
+        n_slices = static_cast<uint32_t>(std::atoi(text));
     }
     const size_t n_slots = tiles_bound * n_slices;
     const size_t search_workgroups = (n_slots + SEARCH_WAVES - 1) / SEARCH_WAVES;
@@ -1693,13 +1767,24 @@ void neighbors_batch(
     Carver carver(extras.work.ptr);
     carve(carver);
 
-    HIP_CHECK(hipMemcpyAsync(d_grids, grids.data(), n_systems * sizeof(GridParams), hipMemcpyHostToDevice, stream));
-    HIP_CHECK(hipMemcpyAsync(
-        d_first_point, first_point_host.data(), (n_systems + 1) * sizeof(uint32_t), hipMemcpyHostToDevice, stream
-    ));
-    HIP_CHECK(hipMemcpyAsync(
-        d_cell_base, cell_base_host.data(), (n_systems + 1) * sizeof(uint32_t), hipMemcpyHostToDevice, stream
-    ));
+    const bool already_there = same_setup && setup.on_device && setup.work_generation == extras.work.generation &&
+                               setup.d_grids == d_grids &&
+                               setup.d_first_point == d_first_point && setup.d_cell_base == d_cell_base;
+    if (!already_there) {
+        setup.on_device = false;
+        HIP_CHECK(hipMemcpyAsync(d_grids, grids.data(), n_systems * sizeof(GridParams), hipMemcpyHostToDevice, stream));
+        HIP_CHECK(hipMemcpyAsync(
+            d_first_point, first_point_host.data(), (n_systems + 1) * sizeof(uint32_t), hipMemcpyHostToDevice, stream
+        ));
+        HIP_CHECK(hipMemcpyAsync(
+            d_cell_base, cell_base_host.data(), (n_systems + 1) * sizeof(uint32_t), hipMemcpyHostToDevice, stream
+        ));
+        setup.d_grids = d_grids;
+        setup.d_first_point = d_first_point;
+        setup.d_cell_base = d_cell_base;
+        setup.work_generation = extras.work.generation;
+        setup.on_device = true;
+    }
 
     // ---- cell lists of all systems, in one sequence of launches
     const uint32_t point_blocks = static_cast<uint32_t>((n_points + BLOCK - 1) / BLOCK);

@@ -166,6 +166,8 @@ __device__ __forceinline__ uint32_t sweep_columns(
 }
 
 /// Variant for a tile holding points that were wrapped into the box: the shift of a pair depends on both points.
+/// Only the wrapped points of the tile (usually a few) pay for it: against a point that was not moved the shift is
+/// the candidate's own, whose vector `c.tx/ty/tz` holds (zero for a candidate without shift).
 template <int R>
 __device__ __forceinline__ uint32_t sweep_columns_wrapped(
     const SortedPoints& sorted, uint32_t first_i, uint32_t n_i, const SweepCandidates<R>& c, const GridParams& g,
@@ -177,15 +179,20 @@ __device__ __forceinline__ uint32_t sweep_columns_wrapped(
         const double xi = sorted.x[at];
         const double yi = sorted.y[at];
         const double zi = sorted.z[at];
-        const int32_t wix = sorted.wx[at];
-        const int32_t wiy = sorted.wy[at];
-        const int32_t wiz = sorted.wz[at];
+        const int32_t wix = static_cast<int32_t>(uniform(static_cast<uint32_t>(sorted.wx[at])));
+        const int32_t wiy = static_cast<int32_t>(uniform(static_cast<uint32_t>(sorted.wy[at])));
+        const int32_t wiz = static_cast<int32_t>(uniform(static_cast<uint32_t>(sorted.wz[at])));
+        const bool moved = (wix | wiy | wiz) != 0;
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            int32_t bx, by, bz;
-            unpack_shift(c.shift[r], bx, by, bz);
-            double tx, ty, tz;
-            shift_vector(g, bx + wix, by + wiy, bz + wiz, tx, ty, tz);
+            double tx = c.tx[r];
+            double ty = c.ty[r];
+            double tz = c.tz[r];
+            if (moved) {
+                int32_t bx, by, bz;
+                unpack_shift(c.shift[r], bx, by, bz);
+                shift_vector(g, bx + wix, by + wiy, bz + wiz, tx, ty, tz);
+            }
             const double vx = (c.x[r] - xi) + tx;
             const double vy = (c.y[r] - yi) + ty;
             const double vz = (c.z[r] - zi) + tz;

@@ -200,7 +200,8 @@ __device__ __forceinline__ void ordered_sweep_pair(
             }
         }
         any_shift = any_shift || (__ballot((bx | by | bz) != 0) != 0);
-        if (!WRAPPED && any_shift) {
+        if (any_shift) {
+            // also read by the sweep of a tile with wrapped points, for its points that were not moved
             shift_vector(g, bx, by, bz, c.tx[r], c.ty[r], c.tz[r]);
         }
     }

@@ -527,7 +527,8 @@ __device__ __forceinline__ void sweep_unwrapped(
     }
 }
 
-/// General variant: the tile holds wrapped points, so the shift depends on both points of a pair.
+/// General variant: the tile holds wrapped points, so the shift depends on both points of a pair. Against a point
+/// that was not moved itself the shift is the candidate's own, whose vector the candidates carry.
 template <bool WRITE, bool FULL, int R, typename Shared>
 __device__ __forceinline__ void sweep_wrapped(
     const SortedPoints& sorted, uint32_t first_i, uint32_t n_i,
@@ -539,13 +540,18 @@ __device__ __forceinline__ void sweep_wrapped(
         const double xi = sorted.x[at];
         const double yi = sorted.y[at];
         const double zi = sorted.z[at];
-        const int32_t wix = sorted.wx[at];
-        const int32_t wiy = sorted.wy[at];
-        const int32_t wiz = sorted.wz[at];
+        const int32_t wix = static_cast<int32_t>(uniform(static_cast<uint32_t>(sorted.wx[at])));
+        const int32_t wiy = static_cast<int32_t>(uniform(static_cast<uint32_t>(sorted.wy[at])));
+        const int32_t wiz = static_cast<int32_t>(uniform(static_cast<uint32_t>(sorted.wz[at])));
+        const bool moved = (wix | wiy | wiz) != 0;
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            double tx, ty, tz;
-            shift_vector(g, c.bx[r] + wix, c.by[r] + wiy, c.bz[r] + wiz, tx, ty, tz);
+            double tx = c.tx[r];
+            double ty = c.ty[r];
+            double tz = c.tz[r];
+            if (moved) {
+                shift_vector(g, c.bx[r] + wix, c.by[r] + wiy, c.bz[r] + wiz, tx, ty, tz);
+            }
             const double vx = (c.x[r] - xi) + tx;
             const double vy = (c.y[r] - yi) + ty;
             const double vz = (c.z[r] - zi) + tz;
