@@ -340,7 +340,13 @@ class NeighborList:
         if tuple(boxes.shape) != (n_systems, 3, 3):
             raise ValueError("`boxes` must hold one 3x3 matrix per system")
         if isinstance(periodic, (bool, np.bool_)):
-            periodic = torch.full((n_systems, 3), bool(periodic), dtype=torch.bool, device=device)
+            # one flag for everything: the tensor of flags is kept for the next batch of this size
+            key = (n_systems, bool(periodic), str(device))
+            kept = getattr(self, "_batch_flags", None)
+            if kept is None or kept[0] != key:
+                kept = (key, torch.full((n_systems, 3), bool(periodic), dtype=torch.bool, device=device))
+                self._batch_flags = kept
+            periodic = kept[1]
         else:
             periodic = torch.as_tensor(periodic).to(device=device, dtype=torch.bool).contiguous()
         if tuple(periodic.shape) != (n_systems, 3):

@@ -495,7 +495,8 @@ __global__ __launch_bounds__(BLOCK) void bounding_batch_kernel(
 }
 
 /// assign_cells for many systems at once: every point looks up its system (binary search in `first_point`), uses
-/// that system's grid, and counts itself in the system's range of cells.
+/// that system's grid, and counts itself in the system's range of cells. Lanes of a wave in the same cell share one
+/// atomic, like in assign_cells: small systems put a whole wave into one cell.
 __global__ __launch_bounds__(BLOCK) void assign_cells_batch(
     const double* __restrict__ points, uint32_t n_points, const GridParams* __restrict__ grids,
     const uint32_t* __restrict__ first_point, const uint32_t* __restrict__ cell_base, uint32_t n_systems,
@@ -503,42 +504,71 @@ __global__ __launch_bounds__(BLOCK) void assign_cells_batch(
     uint32_t* __restrict__ system_of, uint32_t* __restrict__ cell_counts, DeviceStatus* status
 ) {
     const uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
-    if (i >= n_points) {
-        return;
-    }
-    // largest s with first_point[s] <= i
-    uint32_t lo = 0;
-    uint32_t hi = n_systems;
-    while (hi - lo > 1) {
-        const uint32_t mid = (lo + hi) >> 1;
-        if (first_point[mid] <= i) {
-            lo = mid;
+    const bool active = i < n_points;
+    const int lane = lane_id();
+
+    uint32_t system = 0;
+    uint32_t linear = 0;
+    int32_t wrap[3] = {0, 0, 0};
+    if (active) {
+        // largest s with first_point[s] <= i
+        uint32_t lo = 0;
+        uint32_t hi = n_systems;
+        while (hi - lo > 1) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (first_point[mid] <= i) {
+                lo = mid;
+            } else {
+                hi = mid;
+            }
+        }
+        system = lo;
+        const GridParams& g = grids[system];
+
+        const double x = points[3 * static_cast<size_t>(i) + 0];
+        const double y = points[3 * static_cast<size_t>(i) + 1];
+        const double z = points[3 * static_cast<size_t>(i) + 2];
+        int32_t cell[3] = {0, 0, 0};
+        unsigned int axis;
+        if (all_finite(x, y, z, axis)) {
+            locate(g, x, y, z, cell, wrap);
         } else {
-            hi = mid;
+            atomicMin(&status->first_bad_coordinate, 3u * i + axis);
+        }
+        linear = cell_base[system] + (static_cast<uint32_t>(cell[2]) * g.n[1] + cell[1]) * g.n[0] + cell[0];
+    }
+
+    uint64_t group = 1ull << lane; // lanes left over after the rounds stand alone
+    bool pending = active;
+    for (int round = 0; round < ASSIGN_ROUNDS; round++) {
+        const uint64_t remaining = __ballot(pending);
+        if (remaining == 0) {
+            break;
+        }
+        const int leader = __ffsll(static_cast<unsigned long long>(remaining)) - 1;
+        const uint32_t leader_cell = read_lane(linear, leader);
+        const bool same = pending && linear == leader_cell;
+        const uint64_t members = __ballot(same);
+        if (same) {
+            group = members;
+            pending = false;
         }
     }
-    const uint32_t system = lo;
-    const GridParams& g = grids[system];
 
-    const double x = points[3 * static_cast<size_t>(i) + 0];
-    const double y = points[3 * static_cast<size_t>(i) + 1];
-    const double z = points[3 * static_cast<size_t>(i) + 2];
-    int32_t cell[3] = {0, 0, 0};
-    int32_t wrap[3] = {0, 0, 0};
-    unsigned int axis;
-    if (all_finite(x, y, z, axis)) {
-        locate(g, x, y, z, cell, wrap);
-    } else {
-        atomicMin(&status->first_bad_coordinate, 3u * i + axis);
+    const int first = __ffsll(static_cast<unsigned long long>(group)) - 1;
+    uint32_t base = 0;
+    if (active && lane == first) {
+        base = atomicAdd(&cell_counts[linear], static_cast<uint32_t>(__popcll(group)));
     }
-    const uint32_t linear =
-        cell_base[system] + (static_cast<uint32_t>(cell[2]) * g.n[1] + cell[1]) * g.n[0] + cell[0];
-    cell_of[i] = linear;
-    slot_of[i] = atomicAdd(&cell_counts[linear], 1u);
-    system_of[i] = system;
-    wrap_of[3 * static_cast<size_t>(i) + 0] = wrap[0];
-    wrap_of[3 * static_cast<size_t>(i) + 1] = wrap[1];
-    wrap_of[3 * static_cast<size_t>(i) + 2] = wrap[2];
+    base = static_cast<uint32_t>(__shfl(static_cast<int>(base), first));
+    if (active) {
+        cell_of[i] = linear;
+        slot_of[i] = base + rank_in_mask(group);
+        system_of[i] = system;
+        wrap_of[3 * static_cast<size_t>(i) + 0] = wrap[0];
+        wrap_of[3 * static_cast<size_t>(i) + 1] = wrap[1];
+        wrap_of[3 * static_cast<size_t>(i) + 2] = wrap[2];
+    }
 }
 
 constexpr uint32_t CANONICAL_LIMIT = 4096;
