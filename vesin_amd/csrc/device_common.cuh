@@ -30,11 +30,15 @@ struct GridParams {
     int32_t periodic[3];
     uint32_t n_points;
     uint32_t n_cells;
-    // Stencil entries that cannot hold a neighbour (stencils of radius two and more in a box of orthogonal vectors:
-    // the corners of the cube of cells lie outside the cutoff sphere). prune_width2[d] = squared width of a cell
-    // along d; an entry whose cells are at least `gap` whole cells away along d is dropped when the sum over d of
-    // gap^2 * prune_width2[d] exceeds prune_limit. prune = 0: nothing is dropped.
-    double prune_width2[3];
+    // Stencil entries that cannot hold a neighbour (stencils of radius two and more: the corners of the block of
+    // cells lie outside the cutoff sphere). With the edge vectors of a cell written in an orthonormal frame whose
+    // first axis lies along the first edge and whose second lies in the plane of the first two (prune_edges: x of
+    // the three edges, y of the second and third, z of the third), two points in cells (dx, dy, dz) apart differ
+    // along each axis by at least |what the whole cells contribute| - prune_slack (the most that the places of the
+    // two points inside their cells can take back). An entry is dropped when the squares of these three lower
+    // bounds add up to more than prune_limit. prune = 0: nothing is dropped.
+    double prune_edges[6];
+    double prune_slack[3];
     double prune_limit;
     int32_t prune;
 };

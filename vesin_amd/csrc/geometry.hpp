@@ -225,38 +225,61 @@ inline HostGrid choose_grid(
     return grid;
 }
 
-/// Which stencil entries can be dropped (see GridParams::prune): only decided for boxes whose vectors are orthogonal
-/// to each other (to 1e-12 of their lengths), where distances along the three directions add up in squares, and only
-/// when some direction has a stencil radius of two or more: with radius one every cell of the stencil touches the
-/// centre cell. Two points in cells `k` apart along a direction are more than (k - 1) * width apart along it.
+/// Which stencil entries can be dropped (see GridParams::prune_edges). Only when some direction has a stencil radius
+/// of two or more: with radius one every cell of the stencil touches the centre cell. The slack carries a millionth
+/// of a cell for the rounding of the fractional coordinates that put the points into their cells.
 template <typename Grid>
 inline void choose_pruning(const HostBox& box, const HostGrid& grid, double cutoff, Grid& g) {
     using namespace detail;
     g.prune = 0;
     g.prune_limit = cutoff * cutoff * CELL_MARGIN * CELL_MARGIN;
+    for (int k = 0; k < 6; k++) {
+        g.prune_edges[k] = 0.0;
+    }
     for (int d = 0; d < 3; d++) {
-        g.prune_width2[d] = 0.0;
+        g.prune_slack[d] = 0.0;
     }
     if (grid.s[0] < 2 && grid.s[1] < 2 && grid.s[2] < 2) {
         return;
     }
-    const V3 rows[3] = {get_row(box.H, 0), get_row(box.H, 1), get_row(box.H, 2)};
+    // edge vectors of one cell: a non-periodic row of the box is a unit vector, its cells divide the extent of the
+    // points along it
+    V3 edge[3];
     for (int d = 0; d < 3; d++) {
-        const V3 a = rows[d];
-        const V3 b = rows[(d + 1) % 3];
-        const double lengths = std::sqrt(dot(a, a) * dot(b, b));
-        if (!(std::abs(dot(a, b)) <= 1e-12 * lengths)) {
-            return;
-        }
+        const double scale = (box.periodic[d] ? 1.0 : 1.0 / grid.np_scale[d]) / static_cast<double>(grid.n[d]);
+        const V3 row = get_row(box.H, d);
+        edge[d] = V3{row.x * scale, row.y * scale, row.z * scale};
     }
-    for (int d = 0; d < 3; d++) {
-        const double extent = box.periodic[d] ? box.face[d] : 1.0 / grid.np_scale[d];
-        const double width = extent / static_cast<double>(grid.n[d]);
-        if (!(width > 0.0) || !std::isfinite(width)) {
-            return;
-        }
-        g.prune_width2[d] = width * width;
+    // orthonormal frame by Gram-Schmidt: q0 along edge 0, q1 in the plane of edges 0 and 1
+    const double l00 = std::sqrt(dot(edge[0], edge[0]));
+    if (!(l00 > 0.0) || !std::isfinite(l00)) {
+        return;
     }
+    const V3 q0 = V3{edge[0].x / l00, edge[0].y / l00, edge[0].z / l00};
+    const double l10 = dot(edge[1], q0);
+    const V3 rest1 = V3{edge[1].x - l10 * q0.x, edge[1].y - l10 * q0.y, edge[1].z - l10 * q0.z};
+    const double l11 = std::sqrt(dot(rest1, rest1));
+    if (!(l11 > 1e-9 * l00) || !std::isfinite(l11)) {
+        return;
+    }
+    const V3 q1 = V3{rest1.x / l11, rest1.y / l11, rest1.z / l11};
+    const double l20 = dot(edge[2], q0);
+    const double l21 = dot(edge[2], q1);
+    const V3 q2 = cross(q0, q1);
+    const double l22 = dot(edge[2], q2);
+    if (!(std::abs(l22) > 1e-9 * l00) || !std::isfinite(l22)) {
+        return;
+    }
+    const double margin = 1.0 + 1e-6;
+    g.prune_edges[0] = l00;
+    g.prune_edges[1] = l10;
+    g.prune_edges[2] = l20;
+    g.prune_edges[3] = l11;
+    g.prune_edges[4] = l21;
+    g.prune_edges[5] = l22;
+    g.prune_slack[0] = (std::abs(l00) + std::abs(l10) + std::abs(l20)) * margin;
+    g.prune_slack[1] = (std::abs(l11) + std::abs(l21)) * margin;
+    g.prune_slack[2] = std::abs(l22) * margin;
     g.prune = 1;
 }
 

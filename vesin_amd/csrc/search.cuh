@@ -221,15 +221,15 @@ __device__ __forceinline__ void fill_stencil_tables(
             }
         }
         if (g.prune != 0) {
-            // Points lie inside their cells, so two points whose cells are |d| cells apart along a direction are
-            // more than |d| - 1 cell widths apart along it. A millionth of a cell is left for the rounding of the
-            // fractional coordinates that put the points into their cells.
-            const double gx = fmax(static_cast<double>(abs(dx) - 1) - 1e-6, 0.0);
-            const double gy = fmax(static_cast<double>(abs(dy) - 1) - 1e-6, 0.0);
-            const double gz = fmax(static_cast<double>(abs(dz) - 1) - 1e-6, 0.0);
-            const double apart2 =
-                gx * gx * g.prune_width2[0] + gy * gy * g.prune_width2[1] + gz * gz * g.prune_width2[2];
-            if (apart2 > g.prune_limit) {
+            // points lie inside their cells: see GridParams::prune_edges
+            const double fx = static_cast<double>(dx);
+            const double fy = static_cast<double>(dy);
+            const double fz = static_cast<double>(dz);
+            const double ax =
+                fmax(fabs(fx * g.prune_edges[0] + fy * g.prune_edges[1] + fz * g.prune_edges[2]) - g.prune_slack[0], 0.0);
+            const double ay = fmax(fabs(fy * g.prune_edges[3] + fz * g.prune_edges[4]) - g.prune_slack[1], 0.0);
+            const double az = fmax(fabs(fz * g.prune_edges[5]) - g.prune_slack[2], 0.0);
+            if (ax * ax + ay * ay + az * az > g.prune_limit) {
                 valid = false;
             }
         }
