@@ -142,6 +142,39 @@ def test_crowded_tiles_are_left_to_the_write_pass(timings, capfd, monkeypatch):
     assert_same_list(second, expected, what="single pass with deferred tiles")
 
 
+def test_stencil_corners_are_dropped_and_the_switch_keeps_them(capfd, monkeypatch):
+    # 64 atoms in a 7.134 A cube, cutoff 10 A: 5^3 = 125 images, of which those with two components of +-2 are more
+    # than sqrt(2) * 7.134 A > 10 A away from the box: 81 stay (27 without a 2, 54 with one). A sheared box of the
+    # same volume drops fewer. VESIN_HIP_STENCIL=full keeps all of them; the rows are the same either way.
+    points, box, periodic, options = configs.config3(5)
+    sheared = box.copy()
+    sheared[1, 0] = 2.0
+    sheared[2, 1] = -1.5
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    for matrix, kept in ((box, "81 of 125"), (sheared, None)):
+        expected = oracle.neighbors(points, matrix, periodic, options["cutoff"], True, False, "ijSdD")
+        for switch in (None, "full"):
+            if switch is None:
+                monkeypatch.delenv("VESIN_HIP_STENCIL", raising=False)
+            else:
+                monkeypatch.setenv("VESIN_HIP_STENCIL", switch)
+            calculator = NeighborList(cutoff=options["cutoff"], full_list=True)
+            call(calculator, points, matrix, periodic)
+            capfd.readouterr()
+            again = call(calculator, points, matrix, periodic)
+            report = [line for line in capfd.readouterr().err.splitlines() if line.startswith("single pass:")]
+            assert report, "the second call of a list goes through the single-pass search"
+            stencil = report[-1].split("stencil ")[1].rstrip(")")
+            if switch == "full":
+                assert stencil == "125 of 125", report[-1]
+            elif kept is not None:
+                assert stencil == kept, report[-1]
+            else:
+                n_kept = int(stencil.split(" of ")[0])
+                assert 81 <= n_kept < 125, report[-1]
+            assert_same_list(again, expected, what=f"stencil {stencil}")
+
+
 def test_shifts_beyond_the_packing_fall_back():
     # points thousands of boxes away: their shifts do not fit the 10-bit fields of the single pass
     rng = np.random.default_rng(6)
@@ -249,7 +282,7 @@ def test_one_pass_cell_build(full, capfd, monkeypatch):
     capfd.readouterr()
     assert_same_list(call(calculator, points, box, periodic), expected, what="one-pass cell build")
     reports = _single_pass_reports(capfd)
-    assert reports and "one-pass cell build, crowded 0)" in reports[-1], reports
+    assert reports and "one-pass cell build, crowded 0," in reports[-1], reports
     monkeypatch.setenv("VESIN_HIP_CELLS", "packed")
     assert_same_list(call(calculator, points, box, periodic), expected, what="packed cells")
     reports = _single_pass_reports(capfd)
@@ -269,7 +302,7 @@ def test_one_pass_cell_build_with_a_cell_too_full(capfd, monkeypatch):
     capfd.readouterr()
     assert_same_list(call(calculator, points, box, periodic), expected, what="after the overflow")
     reports = _single_pass_reports(capfd)
-    assert reports and "one-pass cell build, crowded" in reports[-1] and "crowded 0)" not in reports[-1], reports
+    assert reports and "one-pass cell build, crowded" in reports[-1] and "crowded 0," not in reports[-1], reports
     assert_same_list(call(calculator, points, box, periodic), expected, what="next call")
     reports = _single_pass_reports(capfd)
     assert reports and "packed cells" in reports[-1], reports

@@ -1027,11 +1027,23 @@ bool compute(
             non_finite_error(points, result.first_bad_coordinate);
         }
         if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
+            uint32_t stencil_cells = 0;
+            uint32_t stencil_kept = 0;
+            for (int32_t dx = -g.s[0]; dx <= g.s[0]; dx++) {
+                for (int32_t dy = -g.s[1]; dy <= g.s[1]; dy++) {
+                    for (int32_t dz = -g.s[2]; dz <= g.s[2]; dz++) {
+                        stencil_cells += 1;
+                        stencil_kept += stencil_entry_too_far(g, dx, dy, dz) ? 0 : 1;
+                    }
+                }
+            }
             std::fprintf(
                 stderr,
-                "single pass: rows %llu general %u deferred %u overflow %u timeout %u (cells %u %u %u, capacity %zu, %s%u)\n",
+                "single pass: rows %llu general %u deferred %u overflow %u timeout %u (cells %u %u %u, capacity %zu, %s%u, "
+                "stencil %u of %u)\n",
                 result.total_rows, result.general, result.deferred, result.overflow, result.chain_timeout, g.n[0], g.n[1], g.n[2],
-                extras.capacity, direct_cells ? "one-pass cell build, crowded " : "packed cells, crowded ", result.crowded_cells
+                extras.capacity, direct_cells ? "one-pass cell build, crowded " : "packed cells, crowded ", result.crowded_cells,
+                stencil_kept, stencil_cells
             );
         }
         if (result.chain_timeout != 0) {

@@ -220,18 +220,9 @@ __device__ __forceinline__ void fill_stencil_tables(
                 valid = false;
             }
         }
-        if (g.prune != 0) {
-            // points lie inside their cells: see GridParams::prune_edges
-            const double fx = static_cast<double>(dx);
-            const double fy = static_cast<double>(dy);
-            const double fz = static_cast<double>(dz);
-            const double ax =
-                fmax(fabs(fx * g.prune_edges[0] + fy * g.prune_edges[1] + fz * g.prune_edges[2]) - g.prune_slack[0], 0.0);
-            const double ay = fmax(fabs(fy * g.prune_edges[3] + fz * g.prune_edges[4]) - g.prune_slack[1], 0.0);
-            const double az = fmax(fabs(fz * g.prune_edges[5]) - g.prune_slack[2], 0.0);
-            if (ax * ax + ay * ay + az * az > g.prune_limit) {
-                valid = false;
-            }
+        if (stencil_entry_too_far(g, dx, dy, dz)) {
+            // points lie inside their cells: no pair between these two cells is within the cutoff
+            valid = false;
         }
         uint32_t start = 0;
         uint32_t count = 0;
