@@ -136,7 +136,7 @@ def test_coincident_points_are_neighbours():
 
 
 def test_heavy_cell_and_many_tiles():
-    # 3000 points inside one cutoff-sized cell: tiles of 64, canonical ordering of a crowded cell
+    # 3000 points inside one cutoff-sized cell: many tiles, canonical ordering of a crowded cell
     rng = np.random.default_rng(8)
     points = rng.random((3000, 3)) * 2.0 + 20.0
     box = np.eye(3) * 60.0

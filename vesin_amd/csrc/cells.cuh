@@ -575,7 +575,7 @@ constexpr uint32_t CANONICAL_LIMIT = 4096;
 
 /// One thread per slot of the counting sort. The atomics of assign_cells leave the points of a cell in arbitrary
 /// order; here every point is ranked by original index among the points of its cell (so the whole pipeline is
-/// deterministic), gathered into the structure-of-arrays layout, and the first point of every run of 64 appends
+/// deterministic), gathered into the structure-of-arrays layout, and the first point of every run of 32 appends
 /// the tile to the tile list. Work is proportional to the number of points, whatever the number of empty cells.
 /// `tiles[].wrapped` must be zero on entry: points moved by a box vector set it with an atomic.
 __global__ __launch_bounds__(BLOCK) void gather_points(
@@ -766,7 +766,7 @@ __global__ __launch_bounds__(SMALL_BUILD_THREADS) void build_cells_small(
 }
 
 /// The single-cell layout used by the brute-force / multi-image path: points keep their order, the one cell
-/// holds all of them, tiles are consecutive blocks of 64 points. Also performs the non-finite check.
+/// holds all of them, tiles are consecutive blocks of 32 points. Also performs the non-finite check.
 /// When `clear` is given (launches of a single workgroup only), it also clears that part of the work state (the
 /// state of the search kernels: the tile list is written here in full and needs no clearing), fetches the box and
 /// resets the status like fetch_box does: a call on this layout then starts with one launch instead of two.

@@ -1,6 +1,6 @@
 // Stencil search over the cell grid: the kernel that decides pair membership and produces the output arrays.
 //
-// One wave owns one tile = up to 64 points `i` of one cell. The candidates `j` are the points of the cells in
+// One wave owns one tile = up to 32 points `i` of one cell. The candidates `j` are the points of the cells in
 // the upper half of the (2s+1)^3 stencil around that cell (offsets that are lexicographically positive, plus the
 // cell itself restricted to later points), periodic images included: every unordered pair {(i, j, S), (j, i, -S)}
 // is tested exactly once, by the tile of one of its two points, and both rows are produced from that one test.
