@@ -62,6 +62,23 @@ static bool two_pass_only() {
     return text != nullptr && std::strcmp(text, "two-pass") == 0;
 }
 
+/// Cells of the upper half of the stencil (the centre cell and what follows it in the kernels' order) that can hold
+/// a neighbour: what a tile's candidates are drawn from.
+static double upper_stencil_cells(const GridParams& g) {
+    if (g.prune == 0) {
+        return 0.5 * ((2.0 * g.s[0] + 1.0) * (2.0 * g.s[1] + 1.0) * (2.0 * g.s[2] + 1.0) + 1.0);
+    }
+    uint32_t kept = 0;
+    for (int32_t dx = 0; dx <= g.s[0]; dx++) {
+        for (int32_t dy = (dx == 0 ? 0 : -g.s[1]); dy <= g.s[1]; dy++) {
+            for (int32_t dz = (dx == 0 && dy == 0 ? 0 : -g.s[2]); dz <= g.s[2]; dz++) {
+                kept += stencil_entry_too_far(g, dx, dy, dz) ? 0 : 1;
+            }
+        }
+    }
+    return static_cast<double>(kept);
+}
+
 /// VESIN_HIP_STENCIL=full searches every cell of a stencil, also those that cannot hold a neighbour (for comparisons
 /// and tests).
 static bool full_stencil_only() {
@@ -248,6 +265,7 @@ struct BatchSetup {
     std::vector<uint32_t> cell_base;
     std::vector<uint32_t> first_point32;
     uint64_t total_cells = 0;
+    double most_units = 1.0;
     // where the last batch left grids, first points and first cells in the work buffer; a call on a single system
     // carves the same buffer its own way and clears the flag
     bool on_device = false;
@@ -758,7 +776,7 @@ bool compute(
     // only add to the time (measured: 216 atoms take 43 us with 256 slices per tile, 25 us with 8).
     uint32_t n_slices = 1;
     if (tiles_bound < 4096) {
-        const double entries = 0.5 * ((2.0 * grid.s[0] + 1.0) * (2.0 * grid.s[1] + 1.0) * (2.0 * grid.s[2] + 1.0) + 1.0);
+        const double entries = upper_stencil_cells(g);
         const double per_cell = std::max(1.0, static_cast<double>(n_points) / static_cast<double>(n_cells));
         const double units = std::ceil(entries * per_cell / WAVE);
         const double wanted = std::min(units, std::floor(4096.0 / static_cast<double>(tiles_bound)));
@@ -1651,6 +1669,7 @@ void neighbors_batch(
         }
 
         uint64_t cells_so_far = 0;
+        double most_units = 1.0; // candidates per tile, in units of 64, of the system with the most (estimate)
         const double zeros[3] = {0.0, 0.0, 0.0};
         for (size_t s = 0; s < n_systems; s++) {
             const HostBox& hbox = host_grids_box[s];
@@ -1676,6 +1695,8 @@ void neighbors_batch(
             if (full_stencil_only()) {
                 g.prune = 0;
             }
+            const double per_cell = std::max(1.0, static_cast<double>(g.n_points) / std::max(1u, g.n_cells));
+            most_units = std::max(most_units, std::ceil(upper_stencil_cells(g) * per_cell / WAVE));
             cell_base_host[s] = static_cast<uint32_t>(cells_so_far);
             cells_so_far += grid.n_cells;
             if (cells_so_far >= 0xFFFFFFF0ull) {
@@ -1684,6 +1705,7 @@ void neighbors_batch(
         }
         cell_base_host[n_systems] = static_cast<uint32_t>(cells_so_far);
         setup.total_cells = cells_so_far;
+        setup.most_units = most_units;
         setup.valid = true;
     }
     const uint64_t total_cells = setup.total_cells;
@@ -1708,20 +1730,10 @@ void neighbors_batch(
     // the single-pass search keeps the hit columns of FUSED_UNITS units per work item: enough slices for the
     // system with the most candidates per tile (estimated from its mean occupation)
     {
-        double most_units = 1.0;
-        for (size_t s = 0; s < n_systems; s++) {
-            const GridParams& g = grids[s];
-            const double entries = 0.5 * ((2.0 * g.s[0] + 1.0) * (2.0 * g.s[1] + 1.0) * (2.0 * g.s[2] + 1.0) + 1.0);
-            const double per_cell = std::max(1.0, static_cast<double>(g.n_points) / std::max(1u, g.n_cells));
-            most_units = std::max(most_units, std::ceil(entries * per_cell / WAVE));
-        }
-        const double wanted = std::ceil(most_units / FUSED_UNITS);
+        const double wanted = std::ceil(setup.most_units / FUSED_UNITS);
         if (wanted > n_slices) {
             n_slices = static_cast<uint32_t>(std::min(256.0, wanted));
         }
-    }
-    if (const char* text = std::getenv("VESIN_HIP_EXPERIMENT_SLICES")) {
-        n_slices = static_cast<uint32_t>(std::atoi(text));
     }
     const size_t n_slots = tiles_bound * n_slices;
     const size_t search_workgroups = (n_slots + SEARCH_WAVES - 1) / SEARCH_WAVES;
