@@ -255,6 +255,7 @@ struct BatchSetup {
     bool any_open_direction = false;
     double cutoff = 0.0;
     int algorithm = 0;
+    bool full_stencil = false;              // VESIN_HIP_STENCIL=full was set
     std::vector<double> boxes;              // 9 per system, as the caller gave them
     std::vector<unsigned char> periodic;    // 3 per system
     std::vector<double> incoming_boxes;     // where a call's boxes land before they are compared
@@ -1583,7 +1584,8 @@ void neighbors_batch(
     // unless some direction is open: then they also follow the points. Same inputs as the call before: same grids.
     const bool same_setup =
         setup.valid && !setup.any_open_direction && setup.cutoff == options.cutoff &&
-        setup.algorithm == static_cast<int>(options.algorithm) && setup.first_point.size() == n_systems + 1 &&
+        setup.algorithm == static_cast<int>(options.algorithm) && setup.full_stencil == full_stencil_only() &&
+        setup.first_point.size() == n_systems + 1 &&
         std::memcmp(setup.first_point.data(), first_point, (n_systems + 1) * sizeof(size_t)) == 0 &&
         setup.boxes.size() == setup.incoming_boxes.size() &&
         std::memcmp(setup.boxes.data(), setup.incoming_boxes.data(), setup.boxes.size() * sizeof(double)) == 0 &&
@@ -1600,6 +1602,7 @@ void neighbors_batch(
         setup.first_point.assign(first_point, first_point + n_systems + 1);
         setup.cutoff = options.cutoff;
         setup.algorithm = static_cast<int>(options.algorithm);
+        setup.full_stencil = full_stencil_only();
         const std::vector<double>& host_boxes = setup.boxes;
         const std::vector<unsigned char>& host_periodic = setup.periodic;
 
