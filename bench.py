@@ -4,12 +4,16 @@ One "step" is one ``vesin_neighbors`` call (the whole job: cell list, single-pas
 kept from its first call, final device sync) on the 1,000,000-atom jittered diamond configuration, cutoff 5 A, full list, unsorted, returning i, j, S, d,
 with the inputs already resident in HBM. Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-other-configs]
 
 The line carries, next to the throughput:
 * ``roofline``: the dominant kernel (the single-pass search, fused_search_kernel) against the 8 TB/s HBM peak, from its
   algorithmic bytes (24 B per point read + 36 B per pair written) and its launch duration measured with HIP events
   on the stream it runs on (``vesin_hip_last_timings``);
+* ``other_configs``: steady-state time per call, pairs per second and fraction of the HBM peak (algorithmic bytes over
+  the whole call) of the other configurations of the baseline, measured after the timed region: the 216-atom sorted
+  case, the triclinic sorted half list, the batch of 4096 small cells, the clustered system without and with periodic
+  directions. They are parity cases (tests/test_gpu_parity.py), timed here for the record;
 * ``cpu_baseline``: the reference's CPU path (the compiled reference in oracle/_ref when present, otherwise the C
   restatement in oracle/) timed in the same run on the host cores.
 """
@@ -39,6 +43,7 @@ def main():
     parser.add_argument("--warmup", type=int, default=10)
     parser.add_argument("--replicas", type=int, default=50, help="diamond cells per edge (50 = the 1M-atom workload)")
     parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--no-other-configs", action="store_true", help="only the headline workload (profiling runs)")
     args = parser.parse_args()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -152,10 +157,78 @@ def main():
         "device_fill_GBs": round(fill_gbs, 1),
     }
 
+    if not args.no_other_configs:
+        del outputs, calculator, d_points
+        result["other_configs"] = other_configs(np, torch)
+
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(points, box, periodic, options, n_pairs, np)
 
     print(json.dumps(result))
+
+
+def other_configs(np, torch):
+    """Steady-state figures of the baseline's other configurations: wall clock around the blocking call, inputs in
+    HBM, median of 10 calls after the list's first call and 3 more."""
+    from vesin_amd import NeighborList, configs
+
+    def timed(call):
+        rows = call()
+        for _ in range(3):
+            call()
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(10):
+            start = time.perf_counter()
+            call()
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - start) * 1e3)
+        return rows, float(np.median(times))
+
+    def entry(name, n_points, rows, ms, quantities):
+        algorithmic = configs.algorithmic_bytes(n_points, rows, quantities)
+        return {
+            "config": name,
+            "n_points": n_points,
+            "n_pairs": rows,
+            "ms_per_call": round(ms, 4),
+            "pairs_per_second": rows / (ms * 1e-3),
+            "algorithmic_bytes": algorithmic,
+            "hbm_frac": round(algorithmic / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        }
+
+    results = []
+    single = [
+        ("config0: 216 atoms, cutoff 5 A, full, sorted, i j S d", configs.config0()),
+        ("config2: 100000 atoms, triclinic, cutoff 6 A, half, sorted, i j S d D", configs.config2()),
+        ("config4a: 500000 clustered atoms, no periodic direction, cutoff 4.5 A, full, i j d",
+         configs.config4(periodic=(False, False, False))),
+        ("config4b: the same atoms, periodic (T, T, F)", configs.config4(periodic=(True, True, False))),
+    ]
+    for name, (points, box, periodic, options) in single:
+        d_points = torch.as_tensor(points, device="cuda:0")
+        d_box = torch.as_tensor(box, device="cuda:0")
+        calculator = NeighborList(cutoff=options["cutoff"], full_list=options["full_list"], sorted=options["sorted"])
+        quantities = options["quantities"]
+        rows, ms = timed(lambda: int(calculator.compute(d_points, d_box, periodic, quantities, copy=False)[0].shape[0]))
+        results.append(entry(name, len(points), rows, ms, quantities))
+        del calculator, d_points
+
+    replicas = [configs.config3(r) for r in range(4096)]
+    options = replicas[0][3]
+    first_point = np.cumsum([0] + [len(r[0]) for r in replicas])
+    d_points = torch.as_tensor(np.concatenate([r[0] for r in replicas]), device="cuda:0")
+    d_boxes = torch.as_tensor(np.stack([r[1] for r in replicas]), device="cuda:0")
+    calculator = NeighborList(cutoff=options["cutoff"], full_list=options["full_list"])
+    letters = "P" + options["quantities"].replace("i", "").replace("j", "")
+    rows, ms = timed(
+        lambda: int(calculator.compute_batch(d_points, first_point, d_boxes, True, letters, copy=False)[0][0].shape[0])
+    )
+    results.insert(2, entry(
+        "config3: 4096 replicas of 64 atoms, box 7.134 A, cutoff 10 A, full, i j S d, one batched call",
+        int(first_point[-1]), rows, ms, options["quantities"],
+    ))
+    return results
 
 
 def cpu_baseline(points, box, periodic, options, n_pairs, np):
