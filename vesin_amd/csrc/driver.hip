@@ -1144,6 +1144,26 @@ bool compute(
         mark(T_COUNT);
         exclusive_scan<SCAN_U32>(rows_of_point, n_points, first_row_of_point, scan_scratch, stream);
         mark(T_SCAN);
+        auto launch_write = [&]() {
+            auto kernel = presorted ? (options.full ? ordered_search_kernel<true, true, true> : ordered_search_kernel<true, false, true>)
+                                    : (options.full ? ordered_search_kernel<true, true, false> : ordered_search_kernel<true, false, false>);
+            hipLaunchKernelGGL(kernel, dim3(blocks), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
+        };
+        // A list that has arrays from earlier calls writes into them without waiting for the host to learn what the
+        // counting pass found: the launch checks on the device that the system suits this search and that the rows
+        // fit, and writes nothing otherwise. One round trip to the host instead of two.
+        const bool early_write = extras.capacity > 0;
+        size_t early_capacity = 0;
+        if (early_write) {
+            size_outputs(neighbors, extras, 0, options);
+            early_capacity = extras.capacity;
+            oargs.out = outputs_of();
+            oargs.capacity = early_capacity;
+            oargs.guarded = 1;
+            mark(T_WRITE_BEGIN);
+            launch_write();
+            mark(T_WRITE);
+        }
         hipLaunchKernelGGL(
             publish_ordered_status, dim3(1), dim3(1), 0, stream,
             ordered_status, first_row_of_point + n_points, extras.d_status, extras.h_ordered
@@ -1170,17 +1190,24 @@ bool compute(
         if (suitable) {
             const size_t total = found.total_rows;
             check_pair_limit(total);
-            size_outputs(neighbors, extras, total, options);
-            oargs.out = outputs_of();
-            mark(T_WRITE_BEGIN);
-            if (total > 0) {
-                auto kernel = presorted ? (options.full ? ordered_search_kernel<true, true, true> : ordered_search_kernel<true, false, true>)
-                                        : (options.full ? ordered_search_kernel<true, true, false> : ordered_search_kernel<true, false, false>);
-                hipLaunchKernelGGL(kernel, dim3(blocks), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
+            if (!(early_write && total <= early_capacity)) {
+                // first call of the list, or more rows than its arrays hold
+                size_outputs(neighbors, extras, total, options);
+                oargs.out = outputs_of();
+                oargs.guarded = 0;
+                mark(T_WRITE_BEGIN);
+                if (total > 0) {
+                    launch_write();
+                }
+                mark(T_WRITE);
+                mark(T_SORT);
+                HIP_CHECK(hipStreamSynchronize(stream));
+            } else {
+                mark(T_SORT);
+                if (timed) {
+                    HIP_CHECK(hipStreamSynchronize(stream));
+                }
             }
-            mark(T_WRITE);
-            mark(T_SORT);
-            HIP_CHECK(hipStreamSynchronize(stream));
             HIP_CHECK(hipGetLastError());
             neighbors.length = total;
             if (timed) {

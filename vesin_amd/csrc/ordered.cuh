@@ -61,6 +61,9 @@ struct OrderedArgs {
     const uint64_t* first_row;  // WRITE: [n_points + 1], exclusive scan of rows_of_point
     OrderedStatus* status;
     uint32_t report_order;      // SORT: count the tiles ordered either way (an atomic per tile on one word: for tests)
+    uint32_t guarded;           // WRITE launched before the host has seen what COUNT found: write nothing unless the
+                                // system suits this search and the rows fit the `capacity` of the arrays
+    uint64_t capacity;
     SearchOutputs out;
 };
 
@@ -264,6 +267,14 @@ __global__ __launch_bounds__(ORDERED_BLOCK) void ordered_search_kernel(OrderedAr
     const int lane = lane_id();
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     OrderedWaveShared& sh = shared.wave[wave];
+    if (WRITE && args.guarded != 0) {
+        const OrderedStatus found = *args.status;
+        const bool suitable = found.max_rows <= ORDERED_MAX_ROWS && found.max_candidates <= ORDERED_CANDIDATES &&
+                              found.unsuitable == 0 && args.first_row[g.n_points] <= args.capacity;
+        if (!suitable) {
+            return;
+        }
+    }
     const uint32_t n_tiles = static_cast<uint32_t>(args.cell_scan[g.n_cells] >> 32);
     const uint32_t work = blockIdx.x * ORDERED_WAVES + wave;
     const uint32_t slot = work / args.items_per_tile;
