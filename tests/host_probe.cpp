@@ -34,3 +34,50 @@ extern "C" int probe_grid(
     }
     return 0;
 }
+
+// The fields choose_pruning fills, without the rest of the kernels' grid description.
+struct ProbePruning {
+    double prune_edges[6];
+    double prune_slack[3];
+    double prune_limit;
+    int prune;
+};
+
+/// Grid and pruning of a system; `dropped[((dx + s0) * (2 s1 + 1) + (dy + s1)) * (2 s2 + 1) + (dz + s2)]` tells
+/// whether the stencil entry (dx, dy, dz) is dropped (room for `n_dropped` entries). Also returns the edge vectors of
+/// one cell (rows of `cell`), which the caller needs to check the decision.
+extern "C" int probe_pruning(
+    const double box[9], const unsigned char periodic[3], double cutoff, size_t n_points,
+    const double lo[3], const double hi[3], int single_cell, int n[3], int s[3], double cell[9],
+    unsigned char* dropped, size_t n_dropped
+) {
+    bool flags[3] = {periodic[0] != 0, periodic[1] != 0, periodic[2] != 0};
+    try {
+        auto hbox = vesin_hip::normalise_box(box, flags);
+        auto grid = vesin_hip::choose_grid(hbox, cutoff, n_points, lo, hi, single_cell != 0);
+        ProbePruning g;
+        vesin_hip::choose_pruning(hbox, grid, cutoff, g);
+        size_t at = 0;
+        for (int d = 0; d < 3; d++) {
+            n[d] = grid.n[d];
+            s[d] = grid.s[d];
+            const double scale = (flags[d] ? 1.0 : 1.0 / grid.np_scale[d]) / grid.n[d];
+            for (int e = 0; e < 3; e++) {
+                cell[3 * d + e] = hbox.H[d][e] * scale;
+            }
+        }
+        for (int dx = -grid.s[0]; dx <= grid.s[0]; dx++) {
+            for (int dy = -grid.s[1]; dy <= grid.s[1]; dy++) {
+                for (int dz = -grid.s[2]; dz <= grid.s[2]; dz++) {
+                    if (at >= n_dropped) {
+                        return 2;
+                    }
+                    dropped[at++] = vesin_hip::stencil_entry_too_far(g, dx, dy, dz) ? 1 : 0;
+                }
+            }
+        }
+    } catch (const std::exception&) {
+        return 1;
+    }
+    return 0;
+}

@@ -28,7 +28,33 @@ def probe(tmp_path_factory):
     lib.probe_box.argtypes = [ctypes.c_void_p] * 5
     lib.probe_grid.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_double, ctypes.c_size_t, ctypes.c_void_p,
                                ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    lib.probe_pruning.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_double, ctypes.c_size_t, ctypes.c_void_p,
+                                  ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                  ctypes.c_void_p, ctypes.c_size_t]
     return lib
+
+
+def run_pruning(probe, box, periodic, cutoff, n_points, lo=(0, 0, 0), hi=(0, 0, 0), single_cell=False):
+    """Grid, edge vectors of one cell (rows), and which stencil entries are dropped, as a dict keyed by (dx, dy, dz)."""
+    box = np.ascontiguousarray(box, dtype=np.float64)
+    periodic = np.ascontiguousarray(periodic, dtype=np.uint8)
+    lo = np.ascontiguousarray(lo, dtype=np.float64)
+    hi = np.ascontiguousarray(hi, dtype=np.float64)
+    n, s = np.zeros(3, dtype=np.int32), np.zeros(3, dtype=np.int32)
+    cell = np.zeros((3, 3))
+    dropped = np.zeros(1 << 16, dtype=np.uint8)
+    status = probe.probe_pruning(box.ctypes.data, periodic.ctypes.data, cutoff, n_points, lo.ctypes.data, hi.ctypes.data,
+                                 int(single_cell), n.ctypes.data, s.ctypes.data, cell.ctypes.data, dropped.ctypes.data,
+                                 dropped.size)
+    assert status == 0
+    entries = {}
+    at = 0
+    for dx in range(-s[0], s[0] + 1):
+        for dy in range(-s[1], s[1] + 1):
+            for dz in range(-s[2], s[2] + 1):
+                entries[(dx, dy, dz)] = bool(dropped[at])
+                at += 1
+    return n, s, cell, entries
 
 
 def run_box(probe, box, periodic):
@@ -123,3 +149,72 @@ def test_grid_open_directions_and_single_cell(probe):
 def test_too_many_images_is_an_error(probe):
     status, _, _ = run_grid(probe, np.eye(3) * 0.01, [1, 1, 1], 10.0, 10, [0] * 3, [0] * 3)
     assert status == 1
+
+
+def closest_approach(cell, offset):
+    """Smallest distance between a point of the cell at the origin and a point of the cell `offset` cells away: the
+    minimum of |(offset + f) . cell| over f in [-1, 1]^3 (f = difference of the two places inside the cells), a
+    convex problem with bounds."""
+    from scipy.optimize import minimize
+
+    offset = np.asarray(offset, dtype=np.float64)
+    gram = cell @ cell.T
+
+    def squared(f):
+        t = offset + f
+        return t @ gram @ t
+
+    def gradient(f):
+        return 2.0 * gram @ (offset + f)
+
+    best = min(
+        minimize(squared, start, jac=gradient, bounds=[(-1.0, 1.0)] * 3, method="L-BFGS-B", options={"ftol": 1e-15, "gtol": 1e-12}).fun
+        for start in (np.zeros(3), -np.sign(offset) * 1.0, -np.sign(offset) * 0.5)
+    )
+    return np.sqrt(max(best, 0.0))
+
+
+def test_dropped_stencil_entries_of_the_small_cell_case(probe):
+    # 7.134 A cube, cutoff 10 A: one cell, 5^3 images; those with two components of +-2 are at least sqrt(2) * 7.134 A
+    # away and go, the other 81 stay (the distance between two boxes one image apart along a direction is zero)
+    n, s, cell, entries = run_pruning(probe, np.eye(3) * 7.134, [1, 1, 1], 10.0, 64)
+    assert list(n) == [1, 1, 1] and list(s) == [2, 2, 2]
+    kept = [offset for offset, gone in entries.items() if not gone]
+    assert len(entries) == 125 and len(kept) == 81
+    assert all(sum(abs(c) == 2 for c in offset) <= 1 for offset in kept)
+    # radius one: every cell of the stencil touches the centre cell
+    n, s, cell, entries = run_pruning(probe, np.eye(3) * 40.0, [1, 1, 1], 5.0, 1000)
+    assert list(s) == [1, 1, 1] and not any(entries.values())
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_dropped_stencil_entries_cannot_hold_a_neighbour(probe, seed):
+    # For boxes of every shape: an entry is only dropped when no two points of the two cells are within the cutoff
+    # (checked with the true closest approach of the two cells, a bounded convex minimisation), and the bound is
+    # not idle: in narrow boxes of orthogonal vectors every entry beyond the cutoff is dropped.
+    rng = np.random.default_rng(400 + seed)
+    edges = rng.uniform(1.5, 6.0, size=3)
+    box = np.diag(edges)
+    kind = seed % 4
+    if kind == 1:
+        q, _ = np.linalg.qr(rng.normal(size=(3, 3)))
+        box = box @ q
+    elif kind >= 2:
+        box = box + rng.normal(scale=0.35 * edges.min(), size=(3, 3))
+        if abs(np.linalg.det(box)) < 0.3 * np.prod(edges):
+            box = np.diag(edges) + np.triu(box - np.diag(edges)) * 0.3
+    periodic = [1, 1, 1] if kind != 3 else [1, 0, 1]
+    cutoff = float(rng.uniform(5.0, 9.0))
+    n, s, cell, entries = run_pruning(probe, box, periodic, cutoff, 50, lo=(-1.0, -2.0, -3.0), hi=(4.0, 7.5, 2.0))
+    assert max(s) >= 2
+    n_dropped = 0
+    for offset, gone in entries.items():
+        apart = closest_approach(cell, offset)
+        if gone:
+            n_dropped += 1
+            assert apart > cutoff, f"entry {offset} is dropped, its cell comes as close as {apart} (cutoff {cutoff})"
+        elif kind <= 1:
+            # orthogonal vectors: the bound is the closest approach itself, up to the margins
+            assert apart <= cutoff * (1 + 1e-5), f"entry {offset} at {apart} is kept (cutoff {cutoff})"
+    if kind <= 1 and min(s) >= 2:
+        assert n_dropped > 0

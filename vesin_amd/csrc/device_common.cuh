@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "geometry.hpp"
+
 namespace vesin_hip {
 
 constexpr int WAVE = 64;
@@ -42,20 +44,6 @@ struct GridParams {
     double prune_limit;
     int32_t prune;
 };
-
-/// Whether the stencil entry (dx, dy, dz) is too far from the centre cell to hold a neighbour (GridParams::prune_edges).
-__host__ __device__ __forceinline__ bool stencil_entry_too_far(const GridParams& g, int32_t dx, int32_t dy, int32_t dz) {
-    if (g.prune == 0) {
-        return false;
-    }
-    const double fx = static_cast<double>(dx);
-    const double fy = static_cast<double>(dy);
-    const double fz = static_cast<double>(dz);
-    const double ax = fmax(fabs(fx * g.prune_edges[0] + fy * g.prune_edges[1] + fz * g.prune_edges[2]) - g.prune_slack[0], 0.0);
-    const double ay = fmax(fabs(fy * g.prune_edges[3] + fz * g.prune_edges[4]) - g.prune_slack[1], 0.0);
-    const double az = fmax(fabs(fz * g.prune_edges[5]) - g.prune_slack[2], 0.0);
-    return ax * ax + ay * ay + az * az > g.prune_limit;
-}
 
 /// One row of TILE_POINTS i-points (or fewer) that one wave searches for.
 struct Tile {

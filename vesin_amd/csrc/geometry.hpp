@@ -225,6 +225,30 @@ inline HostGrid choose_grid(
     return grid;
 }
 
+// this header is read by the host compiler alone (tests) and by hipcc, where the function below also runs in kernels
+#ifdef __HIPCC__
+#define VESIN_HOST_DEVICE __host__ __device__
+#else
+#define VESIN_HOST_DEVICE
+#endif
+
+/// Whether the stencil entry (dx, dy, dz) is too far from the centre cell to hold a neighbour, from the fields
+/// `choose_pruning` fills (GridParams::prune_edges).
+template <typename Grid>
+VESIN_HOST_DEVICE inline bool stencil_entry_too_far(const Grid& g, int32_t dx, int32_t dy, int32_t dz) {
+    if (g.prune == 0) {
+        return false;
+    }
+    const double fx = static_cast<double>(dx);
+    const double fy = static_cast<double>(dy);
+    const double fz = static_cast<double>(dz);
+    const double ax =
+        ::fmax(::fabs(fx * g.prune_edges[0] + fy * g.prune_edges[1] + fz * g.prune_edges[2]) - g.prune_slack[0], 0.0);
+    const double ay = ::fmax(::fabs(fy * g.prune_edges[3] + fz * g.prune_edges[4]) - g.prune_slack[1], 0.0);
+    const double az = ::fmax(::fabs(fz * g.prune_edges[5]) - g.prune_slack[2], 0.0);
+    return ax * ax + ay * ay + az * az > g.prune_limit;
+}
+
 /// Which stencil entries can be dropped (see GridParams::prune_edges). Only when some direction has a stencil radius
 /// of two or more: with radius one every cell of the stencil touches the centre cell. The slack carries a millionth
 /// of a cell for the rounding of the fractional coordinates that put the points into their cells.
