@@ -159,7 +159,10 @@ def main():
 
     if not args.no_other_configs:
         del outputs, calculator, d_points
-        result["other_configs"] = other_configs(np, torch)
+        try:
+            result["other_configs"] = other_configs(np, torch)
+        except Exception as error:  # the headline line is printed whatever happens to the extra measurements
+            result["other_configs_error"] = f"{type(error).__name__}: {error}"
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(points, box, periodic, options, n_pairs, np)
