@@ -3,6 +3,7 @@
 #include <cstring>
 
 #include "geometry.hpp"
+#include "policy.hpp"
 
 extern "C" int probe_box(const double box[9], const unsigned char periodic[3], double H[9], double Hinv[9], double face[3]) {
     bool flags[3] = {periodic[0] != 0, periodic[1] != 0, periodic[2] != 0};
@@ -80,4 +81,28 @@ extern "C" int probe_pruning(
         return 1;
     }
     return 0;
+}
+
+/// Runs the bookkeeping of the remembered box (vesin_hip::BoxGuess) over a sequence of calls. Call k asks for
+/// `n_points[k]` points with cutoff `cutoff[k]` and finds that the box `changed[k]` (non-zero) since the call before.
+/// `guessed[k]` receives whether the call started from the remembered box. The driver's use of the struct is
+/// reproduced: a wrong guess is followed by a call that reads the box, which is then remembered.
+extern "C" void probe_box_guess(
+    const size_t* n_points, const double* cutoff, const unsigned char* changed, size_t n_calls, unsigned char* guessed
+) {
+    vesin_hip::BoxGuess guess;
+    for (size_t k = 0; k < n_calls; k++) {
+        const vesin_hip::BoxKey key = {n_points[k], cutoff[k], 0, true, false};
+        const bool guessing = guess.begin(key);
+        guessed[k] = guessing ? 1 : 0;
+        if (guessing) {
+            if (changed[k] == 0) {
+                guess.was_right();
+                continue;
+            }
+            guess.was_wrong();
+        }
+        guess.have_box = true; // the call read its box
+        guess.stored(key);
+    }
 }

@@ -52,6 +52,19 @@ def test_replicas_of_the_small_cell_case(full):
         assert_same_list(lists[r], expected, what=f"replica {r}")
 
 
+def test_waves_that_give_up_waiting_fall_back_to_the_two_passes(monkeypatch):
+    # a batch places its rows through the chain of workgroup totals; with VESIN_HIP_CHAIN_SPINS=0 every wait gives up
+    # at once (the kernels still run to their end) and the second call of the list must notice and start over
+    monkeypatch.setenv("VESIN_HIP_CHAIN_SPINS", "0")
+    replicas = [configs.config3(r) for r in range(40, 64)]
+    cutoff = replicas[0][3]["cutoff"]
+    calculator = NeighborList(cutoff=cutoff, full_list=True)
+    lists = run_batch(calculator, [r[0] for r in replicas], [r[1] for r in replicas])
+    for r, (points, box, periodic, _) in enumerate(replicas):
+        expected = oracle.neighbors(points, box, periodic, cutoff, True, False, "ijSdD")
+        assert_same_list(lists[r], expected, what=f"replica {r}")
+
+
 def test_systems_of_different_sizes_and_shapes():
     rng = np.random.default_rng(31)
     all_points, all_boxes = [], []

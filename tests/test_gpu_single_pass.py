@@ -91,6 +91,29 @@ def test_ordered_rows_with_crowded_tiles_and_growth(timings, monkeypatch):
     assert used_single_pass(calculator)
 
 
+def test_waves_that_give_up_waiting_fall_back_to_the_two_passes(timings, capfd, monkeypatch):
+    # the ordered placement waits for the rows of other workgroups, with a bound: VESIN_HIP_CHAIN_SPINS=0 makes every
+    # such wait give up at once (all kernels still run to their end), and the call must notice and start over
+    monkeypatch.setenv("VESIN_HIP_ROWS", "ordered")
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    points, box, periodic, _ = configs.config1(12)
+    expected = oracle.neighbors(points, box, periodic, 5.0, True, False, "ijSdD")
+    calculator = NeighborList(cutoff=5.0, full_list=True)
+    call(calculator, points, box, periodic)
+    assert_same_list(call(calculator, points, box, periodic), expected, what="patient")
+    assert used_single_pass(calculator)
+    capfd.readouterr()
+    monkeypatch.setenv("VESIN_HIP_CHAIN_SPINS", "0")
+    for repeat in range(2):
+        assert_same_list(call(calculator, points, box, periodic), expected, what=f"impatient {repeat}")
+        assert not used_single_pass(calculator)
+    gave_up = [line for line in capfd.readouterr().err.splitlines() if line.startswith("single pass:")]
+    assert gave_up and all(" timeout 0 " not in line for line in gave_up), gave_up
+    monkeypatch.delenv("VESIN_HIP_CHAIN_SPINS")
+    assert_same_list(call(calculator, points, box, periodic), expected, what="patient again")
+    assert used_single_pass(calculator)
+
+
 def test_environment_switch_keeps_the_two_passes(timings):
     points, box, periodic, _ = configs.config1(8)
     calculator = NeighborList(cutoff=5.0, full_list=True)
@@ -234,6 +257,27 @@ def test_a_box_that_changes_between_calls():
     open_box = oracle.neighbors(points, box, [True, False, True], 5.0, True, False, "ijSdD")
     assert_same_list(call(calculator, points, box, [True, False, True]), open_box, what="periodicity changed")
     assert_same_list(call(calculator, points, box, [True, False, True]), open_box, what="periodicity kept")
+
+
+def test_a_box_that_changes_with_every_call():
+    # a trajectory at constant pressure, or structures of a dataset one after the other: every guess is wrong, the list
+    # guesses less and less often, and every call still returns the rows of its own box
+    rng = np.random.default_rng(13)
+    points, box, periodic, _ = configs.config1(4)
+    calculator = NeighborList(cutoff=5.0, full_list=True)
+    for step in range(75):
+        scale = 1.0 + 0.002 * step
+        current = box * scale
+        moved = points * scale
+        result = call(calculator, moved, current, periodic)
+        if step % 8 == 0 or step in (33, 34, 66, 67):
+            expected = oracle.neighbors(moved, current, periodic, 5.0, True, False, "ijSdD")
+            assert_same_list(result, expected, what=f"step {step}")
+    # another system through the same list (other number of points, much larger box): never searched with the small box
+    other = configs.config1(7)
+    expected = oracle.neighbors(*other[:3], 5.0, True, False, "ijSdD")
+    assert_same_list(call(calculator, *other[:3]), expected, what="another system")
+    del rng
 
 
 def test_a_box_that_becomes_singular():

@@ -31,7 +31,57 @@ def probe(tmp_path_factory):
     lib.probe_pruning.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_double, ctypes.c_size_t, ctypes.c_void_p,
                                   ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                   ctypes.c_void_p, ctypes.c_size_t]
+    lib.probe_box_guess.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+    lib.probe_box_guess.restype = None
     return lib
+
+
+def run_box_guess(probe, n_points, cutoff, changed):
+    n_points = np.ascontiguousarray(n_points, dtype=np.uint64)
+    cutoff = np.ascontiguousarray(cutoff, dtype=np.float64)
+    changed = np.ascontiguousarray(changed, dtype=np.uint8)
+    guessed = np.zeros(len(changed), dtype=np.uint8)
+    probe.probe_box_guess(n_points.ctypes.data, cutoff.ctypes.data, changed.ctypes.data, len(changed), guessed.ctypes.data)
+    return guessed.astype(bool)
+
+
+def test_a_constant_box_is_guessed_from_the_second_call_on(probe):
+    guessed = run_box_guess(probe, [1000] * 10, [5.0] * 10, [0] * 10)
+    assert not guessed[0] and guessed[1:].all()
+
+
+def test_no_guess_for_another_question(probe):
+    # other number of points, other cutoff: the remembered box belongs to another system
+    n_points = [1000, 1000, 64, 64, 1000, 1000, 1000, 1000]
+    cutoff = [5.0, 5.0, 5.0, 5.0, 5.0, 5.0, 6.0, 6.0]
+    guessed = run_box_guess(probe, n_points, cutoff, [0] * 8)
+    assert guessed.tolist() == [False, True, False, True, False, True, False, True]
+    # and nothing to guess for no points at all
+    assert not run_box_guess(probe, [0] * 4, [5.0] * 4, [0] * 4).any()
+
+
+def test_wrong_guesses_are_made_less_and_less_often(probe):
+    # the box changes with every call: guesses at calls 1, 34, 99, 228, ... (32, 64, 128, ... calls of rest after each)
+    n = 20000
+    guessed = run_box_guess(probe, [1000] * n, [5.0] * n, [1] * n)
+    at = np.flatnonzero(guessed)
+    assert at[0] == 1
+    rests = np.diff(at) - 1
+    assert rests[:7].tolist() == [32, 64, 128, 256, 512, 1024, 2048]
+    assert (rests[7:] == 4096).all() and len(rests) > 8
+    assert guessed.sum() <= 12
+
+
+def test_a_right_guess_restores_the_short_rest(probe):
+    # three wrong guesses (rests 32, 64, 128), then the box stays: guesses on every call; the next change costs 32 again
+    changed = [1] * 100 + [0] * 140 + [1] + [0] * 40
+    n = len(changed)
+    guessed = run_box_guess(probe, [1000] * n, [5.0] * n, changed)
+    at = np.flatnonzero(guessed)
+    assert at[:4].tolist() == [1, 34, 99, 228]
+    assert guessed[228:241].all()
+    assert changed[240] == 1
+    assert not guessed[241:273].any() and guessed[273]
 
 
 def run_pruning(probe, box, periodic, cutoff, n_points, lo=(0, 0, 0), hi=(0, 0, 0), single_cell=False):

@@ -18,6 +18,7 @@
 #include <exception>
 #include <stdexcept>
 #include <memory>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -28,6 +29,7 @@
 #include "fused.cuh"
 #include "geometry.hpp"
 #include "ordered.cuh"
+#include "policy.hpp"
 #include "scan.cuh"
 #include "search.cuh"
 #include "sort.cuh"
@@ -54,6 +56,22 @@ void enable_timings(bool enabled) {
 static bool ordered_rows() {
     const char* text = std::getenv("VESIN_HIP_ROWS");
     return text != nullptr && std::strcmp(text, "ordered") == 0;
+}
+
+/// VESIN_HIP_CHAIN_SPINS=<n> bounds the polls a wave of the single-pass search makes while it waits for another
+/// workgroup's rows (ordered placement). 0 makes every wait give up at once, which is how the tests reach the
+/// fallback that follows without any kernel having to hang for it.
+static uint32_t chain_spin_limit() {
+    const char* text = std::getenv("VESIN_HIP_CHAIN_SPINS");
+    if (text == nullptr || *text == '\0') {
+        return CHAIN_SPIN_LIMIT;
+    }
+    char* end = nullptr;
+    const unsigned long parsed = std::strtoul(text, &end, 10);
+    if (*end != '\0' || parsed > CHAIN_SPIN_LIMIT) {
+        return CHAIN_SPIN_LIMIT;
+    }
+    return static_cast<uint32_t>(parsed);
 }
 
 /// VESIN_HIP_SEARCH=two-pass keeps every call on the count / scan / write sequence (for comparisons and tests).
@@ -120,6 +138,18 @@ __global__ void publish_ordered_status(
     }
 }
 
+/// Everything the kernels report to the host, in one block. A list's own block is pinned host memory that the
+/// kernels write into directly; the entry point that allocates nothing keeps the block in device memory and copies
+/// it to the host before every wait (see HipExtras::wait).
+struct Mailbox {
+    DeviceStatus status;
+    FusedStatus fused;
+    OrderedHostStatus ordered;
+    unsigned char small[128];            // box (72 bytes) + periodic (3 bytes)
+    BlockBounds bounds[BOUNDING_BLOCKS]; // one slot per workgroup of the bounding pass
+    ShiftRange ranges[SHIFT_RANGE_BLOCKS]; // one slot per workgroup of the sort's range pass
+};
+
 /// Makes `device` current for a scope and gives the caller's device back afterwards.
 struct DeviceGuard {
     int previous = -1;
@@ -150,10 +180,17 @@ struct DeviceBuffer {
     void* ptr = nullptr;
     size_t bytes = 0;
     uint64_t generation = 0; // counts the allocations: what was written into an earlier one is gone
+    bool fixed = false;      // memory that is not this buffer's to free or to grow (the entry point that allocates nothing)
 
     void reserve(size_t wanted) {
         if (wanted <= bytes) {
             return;
+        }
+        if (fixed) {
+            throw std::runtime_error(
+                "this calculation needs " + std::to_string(wanted) + " bytes of work memory, the entry point that "
+                "allocates nothing holds " + std::to_string(bytes) + ": use vesin_neighbors for it"
+            );
         }
         release();
         size_t padded = wanted + wanted / 4;
@@ -163,7 +200,7 @@ struct DeviceBuffer {
     }
 
     void release() {
-        if (ptr != nullptr) {
+        if (ptr != nullptr && !fixed) {
             (void)hipFree(ptr);
             ptr = nullptr;
             bytes = 0;
@@ -201,7 +238,6 @@ constexpr double DIRECT_MEAN_MAX = 24.0;
 constexpr int DIRECT_REST = 1024;
 
 constexpr int SINGLE_PASS_REST = 64;
-constexpr int BOX_REST = 32;
 constexpr size_t BOX_BYTES = 75; // 9 doubles and 3 flags, as fetch_box lays them out
 
 enum Stage { T_START = 0, T_CELLS, T_COUNT, T_SCAN, T_WRITE_BEGIN, T_WRITE, T_SORT, T_STAGES };
@@ -282,16 +318,14 @@ struct HipExtras {
     DeviceBuffer work;
     DeviceBuffer sort_work;
     DeviceStatus* d_status = nullptr;
-    DeviceStatus* h_status = nullptr; // pinned
-    unsigned char* h_small = nullptr; // pinned: box (72 bytes) + periodic (3 bytes)
-    BlockBounds* h_bounds = nullptr;  // pinned: one slot per workgroup of the bounding pass
-    FusedStatus* h_fused = nullptr;   // pinned
-    ShiftRange* h_shift_ranges = nullptr; // pinned: one slot per workgroup of the sort's range pass
-    OrderedHostStatus* h_ordered = nullptr; // pinned
+    Mailbox* mail = nullptr;          // what the host reads after a wait
+    Mailbox* mail_device = nullptr;   // what the kernels write: the same pinned block, or device memory
+    /// The entry point that allocates nothing: work memory, status block and mailbox are pieces of a fixed device
+    /// array, the output arrays are the caller's, and nothing of it is ever freed or grown.
+    bool fixed_memory = false;
     size_t capacity = 0;              // rows every allocated output array can hold
     unsigned char last_box[BOX_BYTES] = {}; // box and periodicity of the last call that read them
-    bool have_last_box = false;
-    int box_rest = 0;                 // calls left before a changing box is assumed constant again
+    BoxGuess guess;                   // when a call starts from that box without reading this call's first
     int single_pass_rest = 0;         // calls left before the single-pass search is tried again after it did not fit
     int direct_rest = 0;              // calls left before the one-pass cell build is tried again after a cell overflowed
     int in_order_rest = 0;            // calls left before the in-order search is tried again on a system it did not cover
@@ -301,30 +335,29 @@ struct HipExtras {
     VesinHipTimings timings = {};
     VerletCache* verlet = nullptr;    // only while the caller asks for a skin
 
+    HipExtras() = default;
+    HipExtras(const HipExtras&) = delete;
+    HipExtras& operator=(const HipExtras&) = delete;
+
+    /// Wait for the stream; afterwards `mail` holds what the kernels queued before this call reported.
+    void wait(hipStream_t stream) {
+        if (mail_device != mail) {
+            HIP_CHECK(hipMemcpyAsync(mail, mail_device, sizeof(Mailbox), hipMemcpyDeviceToHost, stream));
+        }
+        HIP_CHECK(hipStreamSynchronize(stream));
+    }
+
     ~HipExtras() {
         delete verlet;
         work.release();
         sort_work.release();
-        if (d_status != nullptr) {
-            (void)hipFree(d_status);
-        }
-        if (h_status != nullptr) {
-            (void)hipHostFree(h_status);
-        }
-        if (h_small != nullptr) {
-            (void)hipHostFree(h_small);
-        }
-        if (h_bounds != nullptr) {
-            (void)hipHostFree(h_bounds);
-        }
-        if (h_fused != nullptr) {
-            (void)hipHostFree(h_fused);
-        }
-        if (h_shift_ranges != nullptr) {
-            (void)hipHostFree(h_shift_ranges);
-        }
-        if (h_ordered != nullptr) {
-            (void)hipHostFree(h_ordered);
+        if (!fixed_memory) {
+            if (d_status != nullptr) {
+                (void)hipFree(d_status);
+            }
+            if (mail != nullptr) {
+                (void)hipHostFree(mail);
+            }
         }
         if (have_events) {
             for (auto& event : events) {
@@ -336,20 +369,13 @@ struct HipExtras {
 
 HipExtras& extras_of(VesinNeighborList& neighbors) {
     if (neighbors.opaque == nullptr) {
-        auto* extras = new HipExtras();
+        // the list only gets a state whose allocations all succeeded
+        auto extras = std::make_unique<HipExtras>();
         extras->device_id = neighbors.device.device_id;
-        neighbors.opaque = extras;
         HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&extras->d_status), sizeof(DeviceStatus)));
-        HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&extras->h_status), sizeof(DeviceStatus), hipHostMallocDefault));
-        HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&extras->h_small), 128, hipHostMallocDefault));
-        HIP_CHECK(hipHostMalloc(
-            reinterpret_cast<void**>(&extras->h_bounds), BOUNDING_BLOCKS * sizeof(BlockBounds), hipHostMallocDefault
-        ));
-        HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&extras->h_fused), sizeof(FusedStatus), hipHostMallocDefault));
-        HIP_CHECK(hipHostMalloc(
-            reinterpret_cast<void**>(&extras->h_shift_ranges), SHIFT_RANGE_BLOCKS * sizeof(ShiftRange), hipHostMallocDefault
-        ));
-        HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&extras->h_ordered), sizeof(OrderedHostStatus), hipHostMallocDefault));
+        HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&extras->mail), sizeof(Mailbox), hipHostMallocDefault));
+        extras->mail_device = extras->mail;
+        neighbors.opaque = extras.release();
     }
     return *static_cast<HipExtras*>(neighbors.opaque);
 }
@@ -387,9 +413,29 @@ void free_outputs(VesinNeighborList& neighbors) {
     neighbors.vectors = nullptr;
 }
 
+/// The list of the entry point that allocates nothing has more rows than the caller's arrays hold.
+struct RowsDoNotFit: std::runtime_error {
+    size_t rows;
+
+    RowsDoNotFit(size_t needed, size_t capacity):
+        std::runtime_error(
+            "the neighbor list has " + std::to_string(needed) + " pairs, the output arrays of the caller hold " +
+            std::to_string(capacity)
+        ),
+        rows(needed) {}
+};
+
 /// Make every requested output array hold `rows` rows and drop the ones that were not requested (like the CPU
 /// engine of the reference does, vesin/src/cpu_cell_list.cpp:605-627).
 void size_outputs(VesinNeighborList& neighbors, HipExtras& extras, size_t rows, const VesinOptions& options) {
+    if (extras.fixed_memory) {
+        // the arrays are the caller's: they hold the rows or the call fails, and `length` says what it takes
+        if (rows > extras.capacity) {
+            neighbors.length = rows;
+            throw RowsDoNotFit(rows, extras.capacity);
+        }
+        return;
+    }
     if (rows > extras.capacity) {
         free_outputs(neighbors);
         size_t capacity = rows + rows / 8;
@@ -506,35 +552,9 @@ void non_finite_error(const double (*points)[3], unsigned int flat) {
     );
 }
 
-bool compute(
-    const double (*points)[3], size_t n_points, const double box[3][3], const bool periodic[3], VesinOptions options,
-    VesinNeighborList& neighbors, HipExtras& extras, bool speculate, hipStream_t stream
-);
-
-void verlet_neighbors(
-    const double (*points)[3], size_t n_points, const double box[3][3], const bool periodic[3], VesinOptions options,
-    VesinNeighborList& neighbors, HipExtras& extras, hipStream_t stream
-);
-
-void direct_neighbors(
-    const double (*points)[3], size_t n_points, const double box[3][3], const bool periodic[3], VesinOptions options,
-    VesinNeighborList& neighbors, HipExtras& extras, hipStream_t stream
-);
-
-} // namespace
-
-void neighbors(
-    const double (*points)[3],
-    size_t n_points,
-    const double box[3][3],
-    const bool periodic[3],
-    VesinOptions options,
-    VesinNeighborList& neighbors,
-    void* caller_stream
-) {
-    // the null stream when the caller names none, like the reference (vesin/src/vesin_cuda.cpp:798)
-    hipStream_t stream = static_cast<hipStream_t>(caller_stream);
-    const int device_id = neighbors.device.device_id;
+/// The requirements of the reference on the inputs of a GPU call, with its texts
+/// (vesin/src/vesin_cuda.cpp:831-854), and this library's own limit on the number of points.
+void check_inputs(const double (*points)[3], size_t n_points, const double box[3][3], const bool periodic[3], int device_id) {
     int device_count = 0;
     if (hipGetDeviceCount(&device_count) != hipSuccess || device_count == 0) {
         (void)hipGetLastError();
@@ -569,6 +589,38 @@ void neighbors(
     if (n_points >= 0xFFFFFFF0ull) {
         throw std::runtime_error("too many points: the GPU path indexes points with 32 bits");
     }
+}
+
+bool compute(
+    const double (*points)[3], size_t n_points, const double box[3][3], const bool periodic[3], VesinOptions options,
+    VesinNeighborList& neighbors, HipExtras& extras, bool speculate, hipStream_t stream
+);
+
+void verlet_neighbors(
+    const double (*points)[3], size_t n_points, const double box[3][3], const bool periodic[3], VesinOptions options,
+    VesinNeighborList& neighbors, HipExtras& extras, hipStream_t stream
+);
+
+void direct_neighbors(
+    const double (*points)[3], size_t n_points, const double box[3][3], const bool periodic[3], VesinOptions options,
+    VesinNeighborList& neighbors, HipExtras& extras, hipStream_t stream
+);
+
+} // namespace
+
+void neighbors(
+    const double (*points)[3],
+    size_t n_points,
+    const double box[3][3],
+    const bool periodic[3],
+    VesinOptions options,
+    VesinNeighborList& neighbors,
+    void* caller_stream
+) {
+    // the null stream when the caller names none, like the reference (vesin/src/vesin_cuda.cpp:798)
+    hipStream_t stream = static_cast<hipStream_t>(caller_stream);
+    const int device_id = neighbors.device.device_id;
+    check_inputs(points, n_points, box, periodic, device_id);
 
     const DeviceGuard guard(device_id);
     HipExtras& extras = extras_of(neighbors);
@@ -593,13 +645,10 @@ void direct_neighbors(
     const double (*points)[3], size_t n_points, const double box[3][3], const bool periodic[3], VesinOptions options,
     VesinNeighborList& neighbors, HipExtras& extras, hipStream_t stream
 ) {
-    // The grid is picked on the host from the box, which lives on the device: reading it costs a round trip before
-    // anything else can be launched. A box that did not change over the last calls is assumed not to have changed
-    // now either: the call runs with the remembered one and checks the assumption at its last synchronisation.
-    bool speculate = extras.have_last_box && extras.box_rest == 0 && n_points > 0;
-    if (extras.box_rest > 0) {
-        extras.box_rest -= 1;
-    }
+    // A box that did not change over the last calls is assumed not to have changed now either: the call runs with
+    // the remembered one and checks the assumption at its last synchronisation (see BoxGuess).
+    const BoxKey key = {n_points, options.cutoff, static_cast<int>(options.algorithm), options.full, options.sorted};
+    const bool speculate = extras.guess.begin(key);
     if (speculate) {
         bool box_was_right = false;
         bool failed = false;
@@ -614,20 +663,22 @@ void direct_neighbors(
             // the error may be a consequence of the wrong box: fetch the one of this call and find out
             hipLaunchKernelGGL(
                 fetch_box, dim3(1), dim3(64), 0, stream,
-                reinterpret_cast<const double*>(box), periodic, extras.h_small, extras.d_status
+                reinterpret_cast<const double*>(box), periodic, extras.mail_device->small, extras.d_status
             );
-            HIP_CHECK(hipStreamSynchronize(stream));
-            box_was_right = std::memcmp(extras.h_small, extras.last_box, BOX_BYTES) == 0;
+            extras.wait(stream);
+            box_was_right = std::memcmp(extras.mail->small, extras.last_box, BOX_BYTES) == 0;
             if (box_was_right) {
                 std::rethrow_exception(failure);
             }
         }
         if (box_was_right) {
+            extras.guess.was_right();
             return;
         }
-        extras.box_rest = BOX_REST;
+        extras.guess.was_wrong();
     }
     (void)compute(points, n_points, box, periodic, options, neighbors, extras, false, stream);
+    extras.guess.stored(key);
 }
 
 bool compute(
@@ -643,7 +694,7 @@ bool compute(
 ) {
     const size_t pair_limit = pairs_per_point_limit();
 
-    const bool timed = TIMINGS_ENABLED.load();
+    const bool timed = TIMINGS_ENABLED.load() && !extras.fixed_memory; // creating events allocates
     if (timed && !extras.have_events) {
         for (auto& event : extras.events) {
             HIP_CHECK(hipEventCreate(&event));
@@ -661,7 +712,7 @@ bool compute(
     auto launch_fetch = [&]() {
         hipLaunchKernelGGL(
             fetch_box, dim3(1), dim3(64), 0, stream,
-            reinterpret_cast<const double*>(box), periodic, extras.h_small, extras.d_status
+            reinterpret_cast<const double*>(box), periodic, extras.mail_device->small, extras.d_status
         );
     };
     bool fetched = false;
@@ -671,12 +722,12 @@ bool compute(
     } else {
         launch_fetch();
         fetched = true;
-        HIP_CHECK(hipStreamSynchronize(stream));
-        std::memcpy(used_box, extras.h_small, BOX_BYTES);
-        extras.have_last_box = false; // remembered once it proved usable, below
+        extras.wait(stream);
+        std::memcpy(used_box, extras.mail->small, BOX_BYTES);
+        extras.guess.have_box = false; // remembered once it proved usable, below
     }
     // valid after any synchronisation of the stream that follows the launch of fetch_box
-    auto box_was_right = [&]() { return std::memcmp(extras.h_small, used_box, BOX_BYTES) == 0; };
+    auto box_was_right = [&]() { return std::memcmp(extras.mail->small, used_box, BOX_BYTES) == 0; };
 
     double host_box[9];
     bool host_periodic[3];
@@ -687,7 +738,7 @@ bool compute(
     const HostBox hbox = normalise_box(host_box, host_periodic);
     if (!speculate) {
         std::memcpy(extras.last_box, used_box, BOX_BYTES);
-        extras.have_last_box = true;
+        extras.guess.have_box = true;
     }
 
     if (n_points == 0) {
@@ -723,9 +774,9 @@ bool compute(
         const uint32_t blocks = static_cast<uint32_t>(std::min<size_t>(BOUNDING_BLOCKS, (n_points + BLOCK - 1) / BLOCK));
         hipLaunchKernelGGL(
             bounding_kernel, dim3(blocks), dim3(BLOCK), 0, stream,
-            reinterpret_cast<const double*>(points), g.n_points, g, extras.h_bounds
+            reinterpret_cast<const double*>(points), g.n_points, g, extras.mail_device->bounds
         );
-        HIP_CHECK(hipStreamSynchronize(stream));
+        extras.wait(stream);
         if (!box_was_right()) {
             return false;
         }
@@ -735,7 +786,7 @@ bool compute(
             hi[d] = -INFINITY;
         }
         for (uint32_t block = 0; block < blocks; block++) {
-            const BlockBounds& part = extras.h_bounds[block];
+            const BlockBounds& part = extras.mail->bounds[block];
             bad = std::min(bad, part.first_bad_coordinate);
             for (int d = 0; d < 3; d++) {
                 lo[d] = std::fmin(lo[d], part.lo[d]);
@@ -911,7 +962,7 @@ bool compute(
             clear_and_fetch, dim3(fill_blocks), dim3(BLOCK), 0, stream,
             reinterpret_cast<uint4*>(cell_counts), blocks16,
             fetched ? static_cast<const double*>(nullptr) : reinterpret_cast<const double*>(box), periodic,
-            extras.h_small, extras.d_status
+            extras.mail_device->small, extras.d_status
         );
         fetched = true;
     };
@@ -955,7 +1006,7 @@ bool compute(
             build_cells_small, dim3(1), dim3(SMALL_BUILD_THREADS), 0, stream,
             flat_points, g, reinterpret_cast<uint4*>(cell_counts), (to_clear + 15) / 16,
             fetched ? static_cast<const double*>(nullptr) : reinterpret_cast<const double*>(box), periodic,
-            extras.h_small, sorted, tiles, cell_scan, extras.d_status
+            extras.mail_device->small, sorted, tiles, cell_scan, extras.d_status
         );
         fetched = true;
     } else if (single_cell && point_blocks == 1) {
@@ -965,7 +1016,7 @@ bool compute(
         hipLaunchKernelGGL(
             prepare_single_cell, dim3(1), dim3(BLOCK), 0, stream,
             flat_points, g, sorted, tiles, cell_scan, extras.d_status, reinterpret_cast<uint4*>(first), (to_clear + 15) / 16,
-            fetched ? static_cast<const double*>(nullptr) : reinterpret_cast<const double*>(box), periodic, extras.h_small
+            fetched ? static_cast<const double*>(nullptr) : reinterpret_cast<const double*>(box), periodic, extras.mail_device->small
         );
         fetched = true;
     } else if (direct_cells) {
@@ -1023,6 +1074,7 @@ bool compute(
         fargs.chain = chain;
         fargs.first_rows = offsets;
         fargs.status = fused_status;
+        fargs.spin_limit = chain_spin_limit();
         uint32_t blocks = static_cast<uint32_t>(search_workgroups);
         if (direct_cells) {
             fargs.search.direct_capacity = DIRECT_CAPACITY;
@@ -1036,12 +1088,12 @@ bool compute(
                                    : (ordered ? fused_search_kernel<false, true> : fused_search_kernel<false, false>);
         hipLaunchKernelGGL(kernel, dim3(blocks), dim3(SEARCH_BLOCK), 0, stream, fargs, g);
         mark(T_WRITE);
-        hipLaunchKernelGGL(publish_fused_status, dim3(1), dim3(1), 0, stream, extras.d_status, fused_status, extras.h_fused);
-        HIP_CHECK(hipStreamSynchronize(stream));
+        hipLaunchKernelGGL(publish_fused_status, dim3(1), dim3(1), 0, stream, extras.d_status, fused_status, &extras.mail_device->fused);
+        extras.wait(stream);
         if (!box_was_right()) {
             return false;
         }
-        const FusedStatus result = *extras.h_fused;
+        const FusedStatus result = extras.mail->fused;
         if (result.first_bad_coordinate != 0xFFFFFFFFu) {
             non_finite_error(points, result.first_bad_coordinate);
         }
@@ -1065,12 +1117,11 @@ bool compute(
                 stencil_kept, stencil_cells
             );
         }
-        if (result.chain_timeout != 0) {
-            throw std::runtime_error("internal error: the single-pass search gave up waiting for an earlier workgroup");
-        }
         // the one-pass cell build is void when a cell overflowed, and the write pass cannot read its layout
         const bool cells_ok = !direct_cells || (result.crowded_cells == 0 && result.deferred == 0);
-        if (result.general == 0 && result.overflow == 0 && cells_ok) {
+        // a wave that gave up waiting for another workgroup's rows wrote its own at the wrong place: like a system
+        // that kernel does not cover, the call starts over with the two passes
+        if (result.general == 0 && result.overflow == 0 && cells_ok && result.chain_timeout == 0) {
             check_pair_limit(result.total_rows);
             if (result.deferred != 0) {
                 // work items too large for the single pass: their rows are counted and placed, the write pass of
@@ -1166,13 +1217,13 @@ bool compute(
         }
         hipLaunchKernelGGL(
             publish_ordered_status, dim3(1), dim3(1), 0, stream,
-            ordered_status, first_row_of_point + n_points, extras.d_status, extras.h_ordered
+            ordered_status, first_row_of_point + n_points, extras.d_status, &extras.mail_device->ordered
         );
-        HIP_CHECK(hipStreamSynchronize(stream));
+        extras.wait(stream);
         if (!box_was_right()) {
             return false;
         }
-        const OrderedHostStatus found = *extras.h_ordered;
+        const OrderedHostStatus found = extras.mail->ordered;
         if (found.first_bad_coordinate != 0xFFFFFFFFu) {
             non_finite_error(points, found.first_bad_coordinate);
         }
@@ -1233,7 +1284,7 @@ bool compute(
     exclusive_scan<SCAN_U32>(counts, n_slots, offsets, scan_scratch, stream);
     mark(T_SCAN);
 
-    hipLaunchKernelGGL(publish_status, dim3(1), dim3(1), 0, stream, extras.d_status, offsets + n_slots, extras.h_status);
+    hipLaunchKernelGGL(publish_status, dim3(1), dim3(1), 0, stream, extras.d_status, offsets + n_slots, &extras.mail_device->status);
 
     // ---- pass 2: write. Without sorting the rows go straight to the caller's arrays, and the launch does not
     // wait for the host to learn their number: the arrays keep the capacity of earlier calls, and a launch that
@@ -1248,14 +1299,14 @@ bool compute(
         mark(T_WRITE);
     }
 
-    HIP_CHECK(hipStreamSynchronize(stream));
+    extras.wait(stream);
     if (!box_was_right()) {
         return false;
     }
-    if (extras.h_status->first_bad_coordinate != 0xFFFFFFFFu) {
-        non_finite_error(points, extras.h_status->first_bad_coordinate);
+    if (extras.mail->status.first_bad_coordinate != 0xFFFFFFFFu) {
+        non_finite_error(points, extras.mail->status.first_bad_coordinate);
     }
-    const size_t total = extras.h_status->total_pairs;
+    const size_t total = extras.mail->status.total_pairs;
 
     check_pair_limit(total);
 
@@ -1266,7 +1317,8 @@ bool compute(
     const bool sorting = options.sorted && total > 1;
     SearchOutputs unsorted = final_out;
     SortWorkspace sort_space = {};
-    sort_space.host_ranges = extras.h_shift_ranges;
+    sort_space.host_ranges = extras.mail->ranges;
+    sort_space.device_ranges = extras.mail_device->ranges;
     if (sorting) {
         carve_sort_space(extras, total, options, unsorted, sort_space);
     }
@@ -1366,6 +1418,9 @@ void verlet_neighbors(
             verlet_store_reference, dim3(1), dim3(64), 0, stream, reinterpret_cast<const double*>(box), periodic,
             cache.reference
         );
+        // the snapshot is complete before the call returns: the caller may change points and box right after
+        HIP_CHECK(hipGetLastError());
+        HIP_CHECK(hipStreamSynchronize(stream));
         cache.options = options;
         cache.n_ref = n_points;
         cache.valid = true;
@@ -1405,7 +1460,8 @@ void verlet_neighbors(
     }
 
     SortWorkspace sort_space = {};
-    sort_space.host_ranges = extras.h_shift_ranges;
+    sort_space.host_ranges = extras.mail->ranges;
+    sort_space.device_ranges = extras.mail_device->ranges;
     size_t total = 0;
     bool through_scratch = options.sorted;
     for (int attempt = 0;; attempt++) {
@@ -1591,7 +1647,7 @@ void neighbors_batch(
     const DeviceGuard guard(device_id);
     HipExtras& extras = extras_of(neighbors);
     extras.timings_valid = false;
-    extras.have_last_box = false; // the work buffers of the single-system path are about to be reused
+    extras.guess.have_box = false; // the work buffers of the single-system path are about to be reused
     hipStream_t stream = static_cast<hipStream_t>(caller_stream);
     const size_t pair_limit = pairs_per_point_limit();
 
@@ -1845,7 +1901,7 @@ void neighbors_batch(
     const auto* flat_points = reinterpret_cast<const double*>(points);
     hipLaunchKernelGGL(
         fetch_box, dim3(1), dim3(64), 0, stream,
-        reinterpret_cast<const double*>(boxes), reinterpret_cast<const bool*>(periodic), extras.h_small, extras.d_status
+        reinterpret_cast<const double*>(boxes), reinterpret_cast<const bool*>(periodic), extras.mail_device->small, extras.d_status
     );
     {
         const size_t to_clear = reinterpret_cast<char*>(fused_status + 1) - reinterpret_cast<char*>(cell_counts);
@@ -1893,6 +1949,7 @@ void neighbors_batch(
         fargs.chain = chain;
         fargs.first_rows = offsets;
         fargs.status = fused_status;
+        fargs.spin_limit = chain_spin_limit();
         const uint32_t blocks = static_cast<uint32_t>(search_workgroups);
         if (options.full) {
             hipLaunchKernelGGL(
@@ -1903,7 +1960,7 @@ void neighbors_batch(
                 (fused_search_kernel<false, true, true>), dim3(blocks), dim3(SEARCH_BLOCK), 0, stream, fargs, GridParams{}
             );
         }
-        hipLaunchKernelGGL(publish_fused_status, dim3(1), dim3(1), 0, stream, extras.d_status, fused_status, extras.h_fused);
+        hipLaunchKernelGGL(publish_fused_status, dim3(1), dim3(1), 0, stream, extras.d_status, fused_status, &extras.mail_device->fused);
         hipLaunchKernelGGL(
             system_rows_kernel, dim3(system_blocks), dim3(BLOCK), 0, stream,
             cell_scan, d_cell_base, offsets, static_cast<uint32_t>(n_systems), n_slices, static_cast<uint32_t>(n_slots),
@@ -1911,7 +1968,7 @@ void neighbors_batch(
         );
         HIP_CHECK(hipMemcpyAsync(first_pair, d_first_pair, (n_systems + 1) * sizeof(size_t), hipMemcpyDeviceToHost, stream));
         HIP_CHECK(hipStreamSynchronize(stream));
-        const FusedStatus result = *extras.h_fused;
+        const FusedStatus result = extras.mail->fused;
         if (result.first_bad_coordinate != 0xFFFFFFFFu) {
             non_finite_error(points, result.first_bad_coordinate);
         }
@@ -1938,12 +1995,12 @@ void neighbors_batch(
 
     launch_search_batch<false>(options.full, args, stream);
     exclusive_scan<SCAN_U32>(counts, n_slots, offsets, scan_scratch, stream);
-    hipLaunchKernelGGL(publish_status, dim3(1), dim3(1), 0, stream, extras.d_status, offsets + n_slots, extras.h_status);
+    hipLaunchKernelGGL(publish_status, dim3(1), dim3(1), 0, stream, extras.d_status, offsets + n_slots, &extras.mail_device->status);
     HIP_CHECK(hipStreamSynchronize(stream));
-    if (extras.h_status->first_bad_coordinate != 0xFFFFFFFFu) {
-        non_finite_error(points, extras.h_status->first_bad_coordinate);
+    if (extras.mail->status.first_bad_coordinate != 0xFFFFFFFFu) {
+        non_finite_error(points, extras.mail->status.first_bad_coordinate);
     }
-    const size_t total = extras.h_status->total_pairs;
+    const size_t total = extras.mail->status.total_pairs;
     if (pair_limit != 0 && total > n_points * pair_limit) {
         throw std::runtime_error(
             "The number of neighbor pairs exceeds the maximum capacity of " + std::to_string(n_points * pair_limit) +

@@ -12,9 +12,12 @@
 // a ticket (candidate slot, tile point) into the wave's LDS ring; whenever 64 tickets are pending all lanes redeem
 // one each, exactly like the write pass of the two-pass search, and store dense rows.
 //
-// A workgroup waits only for workgroups with a smaller index, which the hardware started earlier, so the chain always
-// advances; the wait is bounded anyway, and a wave that runs out of patience raises a flag for the host instead of
-// spinning for ever.
+// The leader of a group (its last workgroup) waits for workgroups with a smaller index; the other workgroups of a
+// group wait for the word their leader publishes, i.e. for a workgroup with a larger index. The chain therefore
+// advances only as long as the hardware starts workgroups in index order and a group's leader gets a wave slot while
+// its members wait, which a grid of this shape has always done here but which nothing guarantees. Every wait is
+// bounded for that reason: a wave that runs out of patience raises a flag and goes on with whatever it has (its rows
+// land inside the arrays, at wrong places), and the host starts the call over with the two-pass search.
 //
 // A work item with more than FUSED_UNITS x 64 candidates cannot keep its columns: it is swept and counted here, its
 // rows are placed by the chain like all others, and its first row goes to `offsets` with a mark in `counts`; the
@@ -35,7 +38,7 @@ namespace vesin_hip {
 constexpr int FUSED_UNITS = 32;         // 64-candidate units of one work item whose columns stay in registers
 constexpr int FUSED_SLOTS = 2 * WAVE;   // candidate records in LDS: two units, so that tickets survive a unit change
 constexpr int32_t PACKED_SHIFT_LIMIT = 500;
-constexpr uint32_t CHAIN_SPIN_LIMIT = 1u << 18;
+constexpr uint32_t CHAIN_SPIN_LIMIT = 1u << 18; // polls a wave makes before it gives up (FusedArgs::spin_limit)
 constexpr uint32_t CHAIN_GROUP = 32;    // workgroups per group of the chain (at most 64)
 
 constexpr uint64_t CHAIN_FLAG_SHIFT = 62;
@@ -55,6 +58,7 @@ struct FusedArgs {
     uint64_t* first_rows; // [work items]: first output row of the work items left to the write pass
     Chain chain;
     FusedStatus* status; // zero on entry
+    uint32_t spin_limit; // polls of the chain before a wave gives up; 0 makes every wait fail at once (tests)
 };
 
 /// LDS of one wave.
@@ -348,9 +352,9 @@ __device__ __forceinline__ void chain_store(uint64_t* word, uint64_t value) {
 }
 
 /// Bounded wait between two polls of the chain; returns false when patience ran out.
-__device__ __forceinline__ bool chain_wait(uint32_t& spins, int lane, FusedStatus* status) {
+__device__ __forceinline__ bool chain_wait(uint32_t& spins, uint32_t spin_limit, int lane, FusedStatus* status) {
     spins += 1;
-    if (spins > CHAIN_SPIN_LIMIT) {
+    if (spins > spin_limit) {
         if (lane == 0) {
             atomicAdd(&status->chain_timeout, 1u);
         }
@@ -368,7 +372,8 @@ __device__ __forceinline__ bool chain_wait(uint32_t& spins, int lane, FusedStatu
 /// array, and publishes them in `chain.bases`. The other workgroups of the group poll that one word, then add the
 /// rows of the earlier workgroups of their group. Every word carries its own flag, so no fences are needed.
 __device__ __forceinline__ uint64_t chain_position(
-    const Chain& chain, uint32_t block, uint32_t n_blocks, uint64_t own_rows, int lane, FusedStatus* status
+    const Chain& chain, uint32_t block, uint32_t n_blocks, uint64_t own_rows, int lane, FusedStatus* status,
+    uint32_t spin_limit
 ) {
     if (lane == 0) {
         chain_store(&chain.blocks[block], CHAIN_AGGREGATE | own_rows);
@@ -389,7 +394,7 @@ __device__ __forceinline__ uint64_t chain_position(
                 word = chain_load(&chain.blocks[group_first + lane]);
             }
             rows_of_member = word & CHAIN_VALUE;
-            if (__ballot((word >> CHAIN_FLAG_SHIFT) == 0) == 0 || !chain_wait(spins, lane, status)) {
+            if (__ballot((word >> CHAIN_FLAG_SHIFT) == 0) == 0 || !chain_wait(spins, spin_limit, lane, status)) {
                 break;
             }
         }
@@ -428,7 +433,7 @@ __device__ __forceinline__ uint64_t chain_position(
                 nearest -= usable;
                 if (reaches_prefix) {
                     done = true;
-                } else if (usable == 0 && !chain_wait(spins, lane, status)) {
+                } else if (usable == 0 && !chain_wait(spins, spin_limit, lane, status)) {
                     done = true;
                 }
             }
@@ -450,7 +455,7 @@ __device__ __forceinline__ uint64_t chain_position(
             group_before = word & CHAIN_VALUE;
             break;
         }
-        if (!chain_wait(spins, lane, status)) {
+        if (!chain_wait(spins, spin_limit, lane, status)) {
             break;
         }
     }
@@ -676,7 +681,7 @@ __global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fa
         uint64_t before = 0;
         if (ORDERED) {
             // rows in work-item order: the workgroup chains with the earlier workgroups
-            before = chain_position(fargs.chain, blockIdx.x, gridDim.x, block_rows, lane, fargs.status);
+            before = chain_position(fargs.chain, blockIdx.x, gridDim.x, block_rows, lane, fargs.status, fargs.spin_limit);
         } else if (lane == 0 && block_rows != 0) {
             // rows in order of arrival: no workgroup waits for another
             before = atomicAdd(&fargs.status->total_rows, static_cast<unsigned long long>(block_rows));

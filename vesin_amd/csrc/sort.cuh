@@ -250,7 +250,9 @@ struct SortWorkspace {
     uint32_t* table;
     uint64_t* table_scan;
     uint64_t* scan_scratch;
-    ShiftRange* host_ranges; // pinned host memory, SHIFT_RANGE_BLOCKS entries
+    ShiftRange* host_ranges;   // SHIFT_RANGE_BLOCKS entries the host reads
+    ShiftRange* device_ranges; // where the kernel writes them: the same pinned host memory, or device memory that
+                               // is copied to `host_ranges` before the host looks
 };
 
 inline size_t sort_blocks(size_t n) {
@@ -285,7 +287,12 @@ inline void sort_pairs(
     const uint32_t n_key_blocks = static_cast<uint32_t>((n + BLOCK - 1) / BLOCK);
 
     const uint32_t range_blocks = n_key_blocks > SHIFT_RANGE_BLOCKS ? SHIFT_RANGE_BLOCKS : n_key_blocks;
-    hipLaunchKernelGGL(shift_range_kernel, dim3(range_blocks), dim3(BLOCK), 0, stream, from.shifts, n, w.host_ranges);
+    hipLaunchKernelGGL(shift_range_kernel, dim3(range_blocks), dim3(BLOCK), 0, stream, from.shifts, n, w.device_ranges);
+    if (w.device_ranges != w.host_ranges &&
+        hipMemcpyAsync(w.host_ranges, w.device_ranges, range_blocks * sizeof(ShiftRange), hipMemcpyDeviceToHost, stream) !=
+            hipSuccess) {
+        throw std::runtime_error("HIP error while reading the range of the shifts");
+    }
     if (hipStreamSynchronize(stream) != hipSuccess) {
         throw std::runtime_error("HIP error while reading the range of the shifts");
     }
