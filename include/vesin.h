@@ -142,6 +142,40 @@ int VESIN_API vesin_hip_neighbors_on_stream(
     const char** error_message
 );
 
+/* vesin_hip_neighbors_on_stream for callers that cannot allocate device memory (loops that must not reach
+ * hipMalloc, harnesses that forbid it): no counterpart in the reference. The rows go to arrays of the caller's and
+ * the call allocates and frees nothing, on the device or through any library.
+ *
+ *   pairs, shifts, distances, vectors   device memory of GPU `device.device_id` with room for `capacity` rows each
+ *                ([capacity][2] size_t, [capacity][3] int32_t, [capacity] double, [capacity][3] double); the
+ *                arrays `options` does not request may be NULL and are not touched
+ *   length       host, filled on success with the number of rows written
+ *   stream       a hipStream_t as void*, NULL for the null stream; the work has completed on return
+ *
+ * Everything else is as for vesin_neighbors (same rows, same checks and messages). The work memory is one array of
+ * 64 MiB that every GPU holds from the moment the library is loaded, which sets the limits: at most 262144 points,
+ * and cell lists and tables that fit (unsorted lists of that many points at usual densities do; `sorted` lists of
+ * sparse or very uneven systems may not). A system beyond these limits, a non-zero `skin`, or a list of more than
+ * `capacity` rows fail with EXIT_FAILURE and a message saying which; when the rows did not fit, *length receives
+ * the number of rows the list has, so that the caller can come back with larger arrays. Calls on one GPU share the
+ * work memory: they take turns (a lock is held for the whole call), whatever their streams. */
+int VESIN_API vesin_hip_neighbors_no_alloc(
+    const double (*points)[3],
+    size_t n_points,
+    const double box[3][3],
+    const bool periodic[3],
+    struct VesinDevice device,
+    struct VesinOptions options,
+    size_t (*pairs)[2],
+    int32_t (*shifts)[3],
+    double* distances,
+    double (*vectors)[3],
+    size_t capacity,
+    size_t* length,
+    void* stream,
+    const char** error_message
+);
+
 /* Neighbor lists of many systems that share the options, computed by one sequence of launches (thousands of small
  * systems cost about as much as one large one with as many points, instead of thousands of calls). Per system the
  * rows are exactly those of vesin_neighbors on that system alone; only their order may differ.

@@ -144,6 +144,23 @@ def get_library():
             ctypes.c_void_p,
             ctypes.POINTER(ctypes.c_char_p),
         ]
+        lib.vesin_hip_neighbors_no_alloc.restype = ctypes.c_int
+        lib.vesin_hip_neighbors_no_alloc.argtypes = [
+            ctypes.c_void_p,
+            ctypes.c_size_t,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            VesinDevice,
+            VesinOptions,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.c_size_t,
+            ctypes.POINTER(ctypes.c_size_t),
+            ctypes.c_void_p,
+            ctypes.POINTER(ctypes.c_char_p),
+        ]
         lib.vesin_hip_enable_timings.restype = None
         lib.vesin_hip_enable_timings.argtypes = [ctypes.c_int]
         lib.vesin_hip_last_timings.restype = ctypes.c_int

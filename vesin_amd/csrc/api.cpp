@@ -123,6 +123,71 @@ extern "C" int vesin_hip_neighbors_on_stream(
     return neighbors_on(points, n_points, box, periodic, device, options, neighbors, stream, error_message);
 }
 
+extern "C" int vesin_hip_neighbors_no_alloc(
+    const double (*points)[3],
+    size_t n_points,
+    const double box[3][3],
+    const bool periodic[3],
+    VesinDevice device,
+    VesinOptions options,
+    size_t (*pairs)[2],
+    int32_t (*shifts)[3],
+    double* distances,
+    double (*vectors)[3],
+    size_t capacity,
+    size_t* length,
+    void* stream,
+    const char** error_message
+) {
+    if (error_message == nullptr) {
+        return EXIT_FAILURE;
+    }
+    if (points == nullptr) {
+        return fail(error_message, "`points` can not be a NULL pointer");
+    }
+    if (box == nullptr) {
+        return fail(error_message, "`cell` can not be a NULL pointer");
+    }
+    if (periodic == nullptr) {
+        return fail(error_message, "`periodic` can not be a NULL pointer");
+    }
+    if (length == nullptr) {
+        return fail(error_message, "`length` can not be a NULL pointer");
+    }
+    if (!std::isfinite(options.cutoff) || options.cutoff <= 0) {
+        return fail(error_message, "cutoff must be a finite, positive number");
+    }
+    if (options.cutoff <= 1e-6) {
+        return fail(error_message, "cutoff is too small");
+    }
+    if (!std::isfinite(options.skin) || options.skin < 0.0) {
+        return fail(error_message, "skin must be a finite, non-negative number");
+    }
+    if (options.n_threads < 0) {
+        return fail(error_message, "n_threads must be zero or a positive integer");
+    }
+    if (device.type != VesinCUDA) {
+        return fail(error_message, "this entry point only computes on a GPU device (VesinCUDA, i.e. HIP on ROCm)");
+    }
+    try {
+        vesin_hip::neighbors_no_alloc(
+            points, n_points, box, periodic, options, device.device_id, pairs, shifts, distances, vectors, capacity,
+            *length, stream
+        );
+    } catch (const std::bad_alloc&) {
+        LAST_ERROR = "failed to allocate memory";
+        *error_message = LAST_ERROR.c_str();
+        return EXIT_FAILURE;
+    } catch (const std::exception& e) {
+        LAST_ERROR = e.what();
+        *error_message = LAST_ERROR.c_str();
+        return EXIT_FAILURE;
+    } catch (...) {
+        return fail(error_message, "fatal error: unknown type thrown as exception");
+    }
+    return EXIT_SUCCESS;
+}
+
 static int neighbors_batch_on(
     const double (*points)[3],
     const size_t* first_point,

@@ -2030,6 +2030,152 @@ void neighbors_batch(
     neighbors.length = total;
 }
 
+namespace {
+
+// ---- the entry point that allocates nothing
+//
+// Callers that cannot allocate device memory (tight loops, harnesses that forbid it) bring their own output arrays;
+// what a call needs besides them (the cell list, the counters and tables of the search, the status block and the
+// block the kernels report to the host through) is carved from one array of device memory that is part of this
+// library's code object, so every GPU the library runs on holds it from the moment the library is loaded until the
+// process ends. In host code the array's name only stands for the symbol: its address on the current device comes
+// from hipGetSymbolAddress, once per device, and only that pointer is ever handed to kernels or copies.
+constexpr size_t FIXED_SCRATCH_BYTES = size_t(64) << 20;
+constexpr size_t FIXED_STATUS_BYTES = 256;
+constexpr size_t FIXED_MAIL_BYTES = (sizeof(Mailbox) + 255) & ~size_t(255);
+constexpr size_t FIXED_SORT_BYTES = size_t(8) << 20; // rows and tables of the radix sort, for sorted lists that need it
+constexpr size_t FIXED_WORK_BYTES = FIXED_SCRATCH_BYTES - FIXED_STATUS_BYTES - FIXED_MAIL_BYTES - FIXED_SORT_BYTES;
+constexpr size_t FIXED_MAX_POINTS = size_t(1) << 18;
+constexpr int FIXED_MAX_DEVICES = 64;
+
+static __device__ __align__(256) unsigned char scratch[FIXED_SCRATCH_BYTES];
+
+/// One per GPU. Calls on one GPU share the array, so they take turns (the lock is held for the whole call).
+struct FixedState {
+    std::mutex turn;
+    unsigned char* memory = nullptr; // address of `scratch` on this GPU
+    Mailbox host_mail;               // where the block the kernels report through is copied before every wait
+    HipExtras extras;
+};
+
+std::mutex FIXED_SETUP;
+FixedState* FIXED_STATES[FIXED_MAX_DEVICES] = {};
+
+/// The state of GPU `device_id`, which must be the current device. The first call on a GPU looks up where that
+/// GPU holds the array.
+FixedState& fixed_state_of(int device_id) {
+    if (device_id >= FIXED_MAX_DEVICES) {
+        throw std::runtime_error("the entry point that allocates nothing serves GPUs 0 to " + std::to_string(FIXED_MAX_DEVICES - 1));
+    }
+    const std::lock_guard<std::mutex> setup(FIXED_SETUP);
+    if (FIXED_STATES[device_id] == nullptr) {
+        auto state = std::make_unique<FixedState>();
+        void* address = nullptr;
+        HIP_CHECK(hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)));
+        if (address == nullptr) {
+            throw std::runtime_error("internal error: the work array of the library has no address on this GPU");
+        }
+        state->memory = static_cast<unsigned char*>(address);
+        unsigned char* next = state->memory;
+        HipExtras& extras = state->extras;
+        extras.device_id = device_id;
+        extras.fixed_memory = true;
+        extras.d_status = reinterpret_cast<DeviceStatus*>(next);
+        next += FIXED_STATUS_BYTES;
+        extras.mail_device = reinterpret_cast<Mailbox*>(next);
+        extras.mail = &state->host_mail;
+        next += FIXED_MAIL_BYTES;
+        extras.work.ptr = next;
+        extras.work.bytes = FIXED_WORK_BYTES;
+        extras.work.fixed = true;
+        next += FIXED_WORK_BYTES;
+        extras.sort_work.ptr = next;
+        extras.sort_work.bytes = FIXED_SORT_BYTES;
+        extras.sort_work.fixed = true;
+        FIXED_STATES[device_id] = state.release();
+    }
+    return *FIXED_STATES[device_id];
+}
+
+} // namespace
+
+void neighbors_no_alloc(
+    const double (*points)[3],
+    size_t n_points,
+    const double box[3][3],
+    const bool periodic[3],
+    VesinOptions options,
+    int device_id,
+    size_t (*pairs)[2],
+    int32_t (*shifts)[3],
+    double* distances,
+    double (*vectors)[3],
+    size_t capacity,
+    size_t& length,
+    void* caller_stream
+) {
+    hipStream_t stream = static_cast<hipStream_t>(caller_stream);
+    check_inputs(points, n_points, box, periodic, device_id);
+    if (n_points > FIXED_MAX_POINTS) {
+        throw std::runtime_error(
+            "the entry point that allocates nothing takes at most " + std::to_string(FIXED_MAX_POINTS) + " points, got " +
+            std::to_string(n_points) + ": use vesin_neighbors for larger systems"
+        );
+    }
+    if (options.skin > 0.0) {
+        throw std::runtime_error("a non-zero `skin` (Verlet caching) keeps device memory between calls: use vesin_neighbors for it");
+    }
+    struct Wanted {
+        const void* pointer;
+        bool wanted;
+        const char* name;
+    };
+    const Wanted arrays[] = {
+        {pairs, true, "pairs"},
+        {shifts, options.return_shifts, "shifts"},
+        {distances, options.return_distances, "distances"},
+        {vectors, options.return_vectors, "vectors"},
+    };
+    for (const Wanted& array : arrays) {
+        if (!array.wanted || capacity == 0) {
+            continue;
+        }
+        if (array.pointer == nullptr) {
+            throw std::runtime_error(std::string("`") + array.name + "` is requested and can not be a NULL pointer");
+        }
+        if (device_of(array.pointer) != device_id) {
+            throw std::runtime_error(std::string("`") + array.name + "` is not memory of the GPU the list is computed on");
+        }
+    }
+
+    const DeviceGuard guard(device_id);
+    FixedState& state = fixed_state_of(device_id);
+    const std::lock_guard<std::mutex> turn(state.turn);
+    HipExtras& extras = state.extras;
+    // nothing is carried over from the call before: it may have been another caller's system
+    extras.capacity = capacity;
+    extras.guess = BoxGuess();
+    extras.single_pass_rest = 0;
+    extras.direct_rest = 0;
+    extras.in_order_rest = 0;
+    extras.timings_valid = false;
+
+    VesinNeighborList list;
+    list.device.type = VesinCUDA;
+    list.device.device_id = device_id;
+    list.pairs = capacity == 0 ? nullptr : pairs;
+    list.shifts = options.return_shifts && capacity != 0 ? shifts : nullptr;
+    list.distances = options.return_distances && capacity != 0 ? distances : nullptr;
+    list.vectors = options.return_vectors && capacity != 0 ? vectors : nullptr;
+    try {
+        direct_neighbors(points, n_points, box, periodic, options, list, extras, stream);
+    } catch (const RowsDoNotFit& error) {
+        length = error.rows;
+        throw;
+    }
+    length = list.length;
+}
+
 void free_neighbors(VesinNeighborList& neighbors) {
     const DeviceGuard guard(neighbors.device.device_id);
     free_outputs(neighbors);

@@ -35,6 +35,26 @@ void neighbors_batch(
     void* stream
 );
 
+/// `neighbors` without any allocation: the rows go to the caller's arrays (device memory of GPU `device_id` holding
+/// `capacity` rows each; the ones that `options` does not request are not touched), the work memory is a fixed
+/// array every GPU holds while the library is loaded. Throws when the system or its list does not fit; `length` then
+/// receives the number of rows when it was the output arrays that were too small. Calls on one GPU take turns.
+void neighbors_no_alloc(
+    const double (*points)[3],
+    size_t n_points,
+    const double box[3][3],
+    const bool periodic[3],
+    VesinOptions options,
+    int device_id,
+    size_t (*pairs)[2],
+    int32_t (*shifts)[3],
+    double* distances,
+    double (*vectors)[3],
+    size_t capacity,
+    size_t& length,
+    void* stream
+);
+
 /// Adds the gradient of a scalar with respect to points and box, given its gradient with respect to the distances
 /// and vectors of the rows. All arrays are device memory of GPU `device_id`; `points_grad` ([n_points][3]) and
 /// `box_grad` ([3][3]) are accumulated into. Runs on `stream` (nullptr: the null stream) and returns after the work
