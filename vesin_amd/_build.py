@@ -26,8 +26,15 @@ FLAGS = [
     "-target-feature",
     "-Xclang",
     "-packed-fp32-ops",
+    # arrays indexed with wave-uniform values (the hit columns of the single-pass search: 32 registers) stay in
+    # registers whatever occupancy a kernel asks for; by default the compiler moves an array larger than a quarter of
+    # the kernel's register budget to scratch memory
+    "-mllvm",
+    "-amdgpu-promote-alloca-to-vector-vgpr-ratio=1",
+    "-mllvm",
+    "-amdgpu-promote-alloca-to-vector-max-regs=64",
     "-Wno-unused-command-line-argument",
-]
+] + os.environ.get("VESIN_EXTRA_FLAGS", "").split()
 
 
 TORCH_SOURCE = os.path.join(CSRC, "torch", "neighbor_list_class.cpp")

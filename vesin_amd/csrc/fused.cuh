@@ -473,8 +473,13 @@ __device__ __forceinline__ uint64_t chain_position(
 /// BATCH: many systems in one launch (see search_kernel_batch): the grid is the one of the tile's system, tiles are
 /// taken in their order (systems stay together) and every work item reports its first row, from which the host
 /// learns where each system's rows start. Only used with ORDERED.
+///
+/// Five waves per SIMD: the kernel needs 96 vector registers for that (the 32 hit columns among them), one fewer
+/// than the compiler takes when left alone, which would be four waves (measured: the clustered 500,000-atom system
+/// 0.59 -> 0.54 ms, the batch of 4096 small cells 1.78 -> 1.75 ms, the 1,000,000-atom lattice unchanged, being bound
+/// by its row stores; six waves with 8 columns instead of 32 made that one slower).
 template <bool FULL, bool ORDERED, bool BATCH = false>
-__global__ __launch_bounds__(SEARCH_BLOCK) void fused_search_kernel(FusedArgs fargs, GridParams single_grid) {
+__global__ __launch_bounds__(SEARCH_BLOCK) __attribute__((amdgpu_waves_per_eu(5, 5))) void fused_search_kernel(FusedArgs fargs, GridParams single_grid) {
     constexpr int R = 2;
     __shared__ FusedShared shared;
     const SearchArgs& args = fargs.search;
