@@ -38,6 +38,18 @@ def main():
         print(name, entry["n_pairs"], flush=True)
         del result
 
+    if full_size:
+        # the batch of 4096 small cells (every replica one call of the reference)
+        from vesin_amd import configs
+
+        per_system = []
+        for replica in range(4096):
+            points, box, periodic, options = configs.config3(replica)
+            result = oracle.ref_neighbors(points, box, periodic, options["cutoff"], True, False, "ijSd")
+            per_system.append(systems.fingerprints(result))
+        golden["config3-batch4096"] = systems.fingerprints_of_systems(per_system)
+        print("config3-batch4096", golden["config3-batch4096"]["n_pairs"], flush=True)
+
     with open(OUT, "w") as fd:
         json.dump(golden, fd, indent=1, sort_keys=True)
 

@@ -208,3 +208,16 @@ def fingerprints(result):
                 hv = _combine(hv, np.ascontiguousarray(v[:, d]).view(np.uint64))
             out["D"] = (out["D"] + int(hv.sum(dtype=np.uint64))) & 0xFFFFFFFFFFFFFFFF
     return out
+
+
+def fingerprints_of_systems(per_system):
+    """One fingerprint for a batch of systems from the fingerprints of its members: the sum (mod 2^64) of a mix of
+    each member's sums with the member's number, so that rows reported under the wrong system change it.
+    ``per_system`` is a sequence of ``fingerprints()`` results (or of dicts with the same keys)."""
+    out = {"n_systems": len(per_system), "n_pairs": 0, "ijS": 0, "d": 0}
+    for number, prints in enumerate(per_system):
+        out["n_pairs"] += int(prints["n_pairs"])
+        for key in ("ijS", "d"):
+            mixed = _mix(np.array([(int(prints[key]) ^ (number + 1)) & 0xFFFFFFFFFFFFFFFF], dtype=np.uint64))[0]
+            out[key] = (out[key] + int(mixed)) & 0xFFFFFFFFFFFFFFFF
+    return out

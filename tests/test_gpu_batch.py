@@ -281,3 +281,101 @@ def test_outputs_on_request_only():
         expected = oracle.neighbors(points, box, periodic, 10.0, True, False, "ijSd")
         assert len(lists[r]["pairs"]) == len(expected["pairs"])
         assert np.array_equal(np.sort(lists[r]["distances"]), np.sort(expected["distances"]))
+
+
+# ---- the full batch of the small-cell configuration: 4096 replicas in one call
+
+_SIGNED = 1 << 63
+
+
+def _signed(value):
+    """A 64-bit pattern as the int64 that torch keeps it in."""
+    value &= 0xFFFFFFFFFFFFFFFF
+    return value - (1 << 64) if value >= _SIGNED else value
+
+
+def _mix_on_device(x):
+    """systems._mix on int64 tensors (same bits; shifts made logical by masking)."""
+    x = x ^ ((x >> 30) & ((1 << 34) - 1))
+    x = x * _signed(0xBF58476D1CE4E5B9)
+    x = x ^ ((x >> 27) & ((1 << 37) - 1))
+    x = x * _signed(0x94D049BB133111EB)
+    return x ^ ((x >> 31) & ((1 << 33) - 1))
+
+
+def _combine_on_device(h, column):
+    return _mix_on_device(h * _signed(0x9E3779B97F4A7C15) + column + _signed(0x7F4A7C15))
+
+
+def fingerprints_per_system_on_device(pairs, shifts, distances, first_pair):
+    """The sums of ``systems.fingerprints`` (hash of (i, j, S) and of (i, j, S, bits of d), modulo 2^64) for every
+    system of a batch, computed where the rows are: 190 million rows do not have to cross to the host."""
+    import torch
+
+    h = _combine_on_device(torch.zeros(pairs.shape[0], dtype=torch.int64, device=pairs.device), pairs[:, 0].view(torch.int64))
+    h = _combine_on_device(h, pairs[:, 1].view(torch.int64))
+    for d in range(3):
+        h = _combine_on_device(h, shifts[:, d].to(torch.int64))
+    hd = _combine_on_device(h, distances.view(torch.int64))
+    edges = torch.as_tensor(np.asarray(first_pair, dtype=np.int64), device=pairs.device)
+    out = []
+    for hashes in (h, hd):
+        running = torch.cat([torch.zeros(1, dtype=torch.int64, device=pairs.device), torch.cumsum(hashes, 0)])
+        out.append((running[edges[1:]] - running[edges[:-1]]).cpu().numpy().view(np.uint64))
+    return out
+
+
+def test_the_device_side_fingerprints_are_those_of_the_host():
+    import torch
+
+    points, box, periodic, options = configs.config3(7)
+    rows = oracle.neighbors(points, box, periodic, options["cutoff"], True, False, "ijSd")
+    expected = systems.fingerprints(rows)
+    n = len(rows["pairs"])
+    ijS, d = fingerprints_per_system_on_device(
+        torch.as_tensor(rows["pairs"].astype(np.int64), device="cuda:0"), torch.as_tensor(rows["shifts"], device="cuda:0"),
+        torch.as_tensor(rows["distances"], device="cuda:0"), [0, n // 3, n],
+    )
+    with np.errstate(over="ignore"):
+        assert int(ijS.sum(dtype=np.uint64)) == expected["ijS"] and int(d.sum(dtype=np.uint64)) == expected["d"]
+    first = systems.fingerprints({key: value[: n // 3] for key, value in rows.items()})
+    assert int(ijS[0]) == first["ijS"] and int(d[0]) == first["d"]
+
+
+def test_config3_full_batch_of_4096_replicas():
+    """64 atoms, box 7.134 A, cutoff 10 A, 4096 seeded replicas in ONE call: every system's rows against the oracle
+    (fingerprints of (i, j, S) and of the distances' bits), both for the first call of a list (count, scan, write) and
+    for the second (single-pass search); the whole batch against the compiled reference's fingerprint on record."""
+    import json
+    import os
+
+    import torch
+
+    replicas = [configs.config3(r) for r in range(4096)]
+    cutoff = replicas[0][3]["cutoff"]
+    expected = []
+    for points, box, periodic, _ in replicas:
+        expected.append(systems.fingerprints(oracle.neighbors(points, box, periodic, cutoff, True, False, "ijSd")))
+    with open(os.path.join(os.path.dirname(systems.__file__), "reference_checksums.json")) as fd:
+        golden = json.load(fd)["config3-batch4096"]
+    assert systems.fingerprints_of_systems(expected) == golden
+
+    first_point = np.cumsum([0] + [len(r[0]) for r in replicas])
+    points = torch.as_tensor(np.concatenate([r[0] for r in replicas]), device="cuda:0")
+    boxes = torch.as_tensor(np.stack([r[1] for r in replicas]), device="cuda:0")
+    calculator = NeighborList(cutoff=cutoff, full_list=True)
+    for call in ("first call", "second call"):
+        (pairs, shifts, distances), first_pair = calculator.compute_batch(points, first_point, boxes, True, "PSd", copy=False)
+        assert pairs.shape[0] == golden["n_pairs"] == 190477980
+        assert first_pair[0] == 0 and first_pair[-1] == pairs.shape[0]
+        assert int(pairs.view(torch.int64).max()) == 63  # indices count inside each system
+        ijS, d = fingerprints_per_system_on_device(pairs, shifts, distances, first_pair)
+        per_system = []
+        for s, prints in enumerate(expected):
+            rows = int(first_pair[s + 1] - first_pair[s])
+            assert rows == prints["n_pairs"], f"{call}, system {s}: {rows} rows, expected {prints['n_pairs']}"
+            assert int(ijS[s]) == prints["ijS"], f"{call}, system {s}: pairs or shifts differ from the oracle's"
+            assert int(d[s]) == prints["d"], f"{call}, system {s}: distances differ from the oracle's"
+            per_system.append({"n_pairs": rows, "ijS": int(ijS[s]), "d": int(d[s])})
+        assert systems.fingerprints_of_systems(per_system) == golden, call
+        del pairs, shifts, distances, ijS, d
