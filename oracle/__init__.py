@@ -20,11 +20,19 @@ import numpy as np
 HERE = os.path.dirname(os.path.realpath(__file__))
 ORACLE_LIB = os.path.join(HERE, "liboracle.so")
 REF_LIB = os.path.join(HERE, "_ref", "libvesin_ref.so")
+REF_TORCH_LIB = os.path.join(HERE, "_ref", "libvesin_torch_ref.so")
 
 
 def build(reference="/root/reference"):
     """Compile liboracle.so and, when the reference checkout exists, _ref/libvesin_ref.so."""
     subprocess.run(["make", "-C", HERE, "-s", "liboracle.so", "ref", f"REFERENCE={reference}"], check=True)
+
+
+def build_ref_torch(reference="/root/reference"):
+    """Compile the reference's TorchScript class, unmodified, against this repository's header and library
+    (_ref/libvesin_torch_ref.so); needs the reference checkout and a built vesin_amd/lib/libvesin.so."""
+    subprocess.run(["make", "-C", HERE, "-s", "ref_torch", f"REFERENCE={reference}"], check=True)
+    return REF_TORCH_LIB
 
 
 class _Options(ctypes.Structure):
