@@ -178,7 +178,7 @@ int VESIN_API vesin_hip_neighbors_no_alloc(
 
 /* Neighbor lists of many systems that share the options, computed by one sequence of launches (thousands of small
  * systems cost about as much as one large one with as many points, instead of thousands of calls). Per system the
- * rows are exactly those of vesin_neighbors on that system alone; only their order may differ.
+ * rows are exactly those of vesin_neighbors on that system alone; only the order of an unsorted list may differ.
  *
  *   points       device: the points of all systems, one system after the other
  *   first_point  host, n_systems + 1 entries: first_point[s] is the index in `points` of the first point of system
@@ -191,8 +191,9 @@ int VESIN_API vesin_hip_neighbors_no_alloc(
  *   first_pair   host, n_systems + 1 entries, filled on success: rows [first_pair[s], first_pair[s + 1]) belong to
  *                system s
  *
- * options.sorted must be false. Returns EXIT_SUCCESS / EXIT_FAILURE like vesin_neighbors, with the same message
- * ownership. */
+ * With options.sorted every system's rows are ordered as vesin_neighbors orders them for that system alone (by
+ * (i, j, shift)); options.skin must be zero. Returns EXIT_SUCCESS / EXIT_FAILURE like vesin_neighbors, with the same
+ * message ownership. */
 int VESIN_API vesin_hip_neighbors_batch(
     const double (*points)[3],
     const size_t* first_point,

@@ -258,8 +258,6 @@ def test_batch_errors():
     points, box, periodic, _ = configs.config3(0)
     device_points = torch.as_tensor(points, device="cuda:0")
     boxes = torch.as_tensor(box[None], device="cuda:0")
-    with pytest.raises(RuntimeError, match="sorted output is not available for a batch"):
-        NeighborList(cutoff=5.0, full_list=True, sorted=True).compute_batch(device_points, [0, len(points)], boxes)
     with pytest.raises(RuntimeError, match="non-finite coordinate along axis 1"):
         flags = torch.as_tensor([[True, False, True]], device="cuda:0")
         broken = device_points.clone()
@@ -271,6 +269,48 @@ def test_batch_errors():
     singular[0, 2] = singular[0, 1]
     with pytest.raises(RuntimeError, match="the box matrix is not invertible"):
         NeighborList(cutoff=5.0, full_list=True).compute_batch(device_points, [0, len(points)], singular)
+
+
+@pytest.mark.parametrize("full", [True, False], ids=["full", "half"])
+def test_sorted_batch_equals_sorted_single_calls(full):
+    """sorted=True in a batch: every system's rows in the order vesin_neighbors gives for that system alone
+    ((i, j, shift) lexicographic), compared in place with the oracle's rows put in that order and with single calls."""
+    import torch
+
+    rng = np.random.default_rng(57)
+    all_points, all_boxes, all_flags = [], [], []
+    for replica in (0, 1, 2):
+        points, box, _, _ = configs.config3(replica)  # many images of every pair
+        all_points.append(points)
+        all_boxes.append(box)
+        all_flags.append((True, True, True))
+    for n, flags in ((0, (True, True, True)), (1, (True, True, True)), (150, (False, False, False)), (400, (True, False, True)),
+                     (700, (True, True, True))):
+        edge = 7.0 + 3.0 * rng.random()
+        box = np.eye(3) * edge + 0.4 * rng.normal(size=(3, 3))
+        all_points.append(rng.random((n, 3)) @ box + rng.integers(-1, 2, size=(n, 3)) @ box)
+        all_boxes.append(box)
+        all_flags.append(flags)
+    cutoff = 4.2
+    calculator = NeighborList(cutoff=cutoff, full_list=full, sorted=True)
+    complete = None
+    for letters in ("PSdD", "Pd"):
+        lists = run_batch(calculator, all_points, all_boxes, letters=letters, periodic=np.array(all_flags))
+        for s, (points, box, flags) in enumerate(zip(all_points, all_boxes, all_flags)):
+            expected = oracle.canonicalize(oracle.neighbors(points, box, list(flags), cutoff, full, False, "ijSdD"))
+            for key in lists[s]:
+                assert np.array_equal(lists[s][key], expected[key]), f"system {s}, {letters}: {key} differ or are out of order"
+        complete = complete or lists
+    # the same through one call per system
+    single = NeighborList(cutoff=cutoff, full_list=full, sorted=True)
+    for s in (0, 6, 7):
+        pairs, shifts, distances = single.compute(
+            torch.as_tensor(all_points[s], device="cuda:0"), torch.as_tensor(all_boxes[s], device="cuda:0"),
+            list(all_flags[s]), "PSd",
+        )
+        assert np.array_equal(pairs.cpu().numpy(), complete[s]["pairs"])
+        assert np.array_equal(shifts.cpu().numpy(), complete[s]["shifts"])
+        assert np.array_equal(distances.cpu().numpy(), complete[s]["distances"])
 
 
 def test_outputs_on_request_only():

@@ -1631,9 +1631,6 @@ void neighbors_batch(
     if (n_points >= 0xFFFFFFF0ull || n_systems >= 0x7FFFFFF0ull) {
         throw std::runtime_error("too many points or systems: the GPU path indexes them with 32 bits");
     }
-    if (options.sorted) {
-        throw std::runtime_error("sorted output is not available for a batch of systems");
-    }
     if (device_of(points) != device_id && n_points > 0) {
         throw std::runtime_error("`points` pointer is not allocated on the GPU of the neighbor list");
     }
@@ -1937,7 +1934,8 @@ void neighbors_batch(
 
     // ---- a list that has arrays from earlier calls: single-pass search straight into them, rows in work-item order
     // (the rows of a system stay together). Whatever does not fit its shape starts over with the two passes below.
-    if (extras.capacity > 0 && !two_pass_only()) {
+    // (a sorted list is sorted afterwards: its rows go to scratch memory first, through the two passes)
+    if (extras.capacity > 0 && !two_pass_only() && !options.sorted) {
         size_outputs(neighbors, extras, 0, options);
         FusedArgs fargs = {};
         fargs.search = args;
@@ -2011,11 +2009,23 @@ void neighbors_batch(
     }
 
     size_outputs(neighbors, extras, total, options);
-    args.out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
-    args.out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
-    args.out.distances = neighbors.distances;
-    args.out.vectors = reinterpret_cast<double*>(neighbors.vectors);
-    args.capacity = extras.capacity;
+    SearchOutputs final_out;
+    final_out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
+    final_out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
+    final_out.distances = neighbors.distances;
+    final_out.vectors = reinterpret_cast<double*>(neighbors.vectors);
+    // a sorted list: the rows go to scratch rows (shifts always among them, they are part of the order) and the
+    // sort's last step fills the caller's arrays
+    const bool sorting = options.sorted && total > 1;
+    SearchOutputs unsorted = final_out;
+    SortWorkspace sort_space = {};
+    sort_space.host_ranges = extras.mail->ranges;
+    sort_space.device_ranges = extras.mail_device->ranges;
+    if (sorting) {
+        carve_sort_space(extras, total, options, unsorted, sort_space);
+    }
+    args.out = unsorted;
+    args.capacity = sorting ? total : extras.capacity;
     if (total > 0) {
         launch_search_batch<true>(options.full, args, stream);
     }
@@ -2025,6 +2035,15 @@ void neighbors_batch(
         static_cast<const FusedStatus*>(nullptr), d_first_pair
     );
     HIP_CHECK(hipMemcpyAsync(first_pair, d_first_pair, (n_systems + 1) * sizeof(size_t), hipMemcpyDeviceToHost, stream));
+    if (sorting) {
+        // every system's rows stay in their range and come out ordered by (i, j, shift) inside it: the order of
+        // vesin_neighbors on that system alone
+        BatchRows rows_of_systems;
+        rows_of_systems.first_pair = d_first_pair;
+        rows_of_systems.first_point = d_first_point;
+        rows_of_systems.n_systems = static_cast<uint32_t>(n_systems);
+        sort_pairs(unsorted, final_out, total, n_points, sort_space, stream, rows_of_systems);
+    }
     HIP_CHECK(hipStreamSynchronize(stream));
     HIP_CHECK(hipGetLastError());
     neighbors.length = total;

@@ -91,10 +91,19 @@ __global__ __launch_bounds__(BLOCK) void shift_range_kernel(
     }
 }
 
+/// The rows of many systems, system after system, whose indices count inside each system: the first index of a
+/// row is sorted as if it counted over all points of the batch (first point of the row's system + index), which
+/// keeps every system's rows where they are and orders them inside.
+struct BatchRows {
+    const unsigned long long* first_pair; // [n_systems + 1]: first row of every system
+    const uint32_t* first_point;          // [n_systems + 1]: first point of every system
+    uint32_t n_systems;                   // 0: the rows are those of one system
+};
+
 /// keys[k] = packed fields of row perm[k] (or row k when perm is null); rows[k] = that row number.
 __global__ __launch_bounds__(BLOCK) void build_keys_kernel(
     const unsigned long long* __restrict__ pairs, const int32_t* __restrict__ shifts,
-    const uint32_t* __restrict__ perm, size_t n, KeyLayout layout,
+    const uint32_t* __restrict__ perm, size_t n, KeyLayout layout, BatchRows batch,
     uint64_t* __restrict__ keys, uint32_t* __restrict__ rows
 ) {
     size_t k = static_cast<size_t>(blockIdx.x) * BLOCK + threadIdx.x;
@@ -105,6 +114,20 @@ __global__ __launch_bounds__(BLOCK) void build_keys_kernel(
     uint64_t key = 0;
     if (layout.use_i) {
         key = pairs[2 * row];
+        if (batch.n_systems != 0) {
+            // the system whose rows include this one: the last with first_pair <= row
+            uint32_t lo = 0;
+            uint32_t hi = batch.n_systems;
+            while (hi - lo > 1) {
+                const uint32_t mid = (lo + hi) >> 1;
+                if (batch.first_pair[mid] <= row) {
+                    lo = mid;
+                } else {
+                    hi = mid;
+                }
+            }
+            key += batch.first_point[lo];
+        }
     }
     if (layout.use_j_and_shift) {
         key = (key << layout.bits_index) | pairs[2 * row + 1];
@@ -277,9 +300,11 @@ inline int radix_sort(SortWorkspace& w, size_t n, uint32_t bits, hipStream_t str
     return current;
 }
 
-/// Sort `n` unsorted payload rows (`from`, shifts always present) into `to`.
+/// Sort `n` unsorted payload rows (`from`, shifts always present) into `to`. `n_points` bounds both indices of a row
+/// (with `batch`: the points of all systems together).
 inline void sort_pairs(
-    const SearchOutputs& from, const SearchOutputs& to, size_t n, size_t n_points, SortWorkspace& w, hipStream_t stream
+    const SearchOutputs& from, const SearchOutputs& to, size_t n, size_t n_points, SortWorkspace& w, hipStream_t stream,
+    BatchRows batch = BatchRows{nullptr, nullptr, 0}
 ) {
     if (n >= 0xFFFFFFFFull) {
         throw std::runtime_error("too many pairs to sort: the sort indexes rows with 32 bits");
@@ -322,7 +347,7 @@ inline void sort_pairs(
         layout.use_j_and_shift = 1;
         hipLaunchKernelGGL(
             build_keys_kernel, dim3(n_key_blocks), dim3(BLOCK), 0, stream,
-            from.pairs, from.shifts, static_cast<const uint32_t*>(nullptr), n, layout, w.keys[0], w.rows[0]
+            from.pairs, from.shifts, static_cast<const uint32_t*>(nullptr), n, layout, batch, w.keys[0], w.rows[0]
         );
         result = radix_sort(w, n, low_bits + layout.bits_index, stream);
     } else {
@@ -331,7 +356,7 @@ inline void sort_pairs(
         layout.use_j_and_shift = 1;
         hipLaunchKernelGGL(
             build_keys_kernel, dim3(n_key_blocks), dim3(BLOCK), 0, stream,
-            from.pairs, from.shifts, static_cast<const uint32_t*>(nullptr), n, layout, w.keys[0], w.rows[0]
+            from.pairs, from.shifts, static_cast<const uint32_t*>(nullptr), n, layout, batch, w.keys[0], w.rows[0]
         );
         result = radix_sort(w, n, low_bits, stream);
         if (result != 0) {
@@ -343,7 +368,7 @@ inline void sort_pairs(
         // keys are rebuilt from the rows in their current order; rows[1] is free to receive the copy
         hipLaunchKernelGGL(
             build_keys_kernel, dim3(n_key_blocks), dim3(BLOCK), 0, stream,
-            from.pairs, from.shifts, static_cast<const uint32_t*>(w.rows[0]), n, layout, w.keys[1], w.rows[1]
+            from.pairs, from.shifts, static_cast<const uint32_t*>(w.rows[0]), n, layout, batch, w.keys[1], w.rows[1]
         );
         std::swap(w.keys[0], w.keys[1]);
         std::swap(w.rows[0], w.rows[1]);
