@@ -928,9 +928,9 @@ bool compute(
         sorted.y = carver.take<double>(sorted_slots + SORTED_PADDING);
         sorted.z = carver.take<double>(sorted_slots + SORTED_PADDING);
         sorted.index = carver.take<uint32_t>(sorted_slots + SORTED_PADDING);
-        sorted.wx = carver.take<int32_t>(sorted_slots);
-        sorted.wy = carver.take<int32_t>(sorted_slots);
-        sorted.wz = carver.take<int32_t>(sorted_slots);
+        sorted.wx = carver.take<int32_t>(sorted_slots + SORTED_PADDING);
+        sorted.wy = carver.take<int32_t>(sorted_slots + SORTED_PADDING);
+        sorted.wz = carver.take<int32_t>(sorted_slots + SORTED_PADDING);
         counts = carver.take<uint32_t>(std::max(n_slots, direct_slots * n_slices));
         offsets = carver.take<uint64_t>(std::max(n_slots, direct_slots * n_slices) + 1);
         scan_scratch = carver.take<uint64_t>(scratch_elements);
@@ -1857,9 +1857,9 @@ void neighbors_batch(
         sorted.y = carver.take<double>(n_points + SORTED_PADDING);
         sorted.z = carver.take<double>(n_points + SORTED_PADDING);
         sorted.index = carver.take<uint32_t>(n_points + SORTED_PADDING);
-        sorted.wx = carver.take<int32_t>(n_points);
-        sorted.wy = carver.take<int32_t>(n_points);
-        sorted.wz = carver.take<int32_t>(n_points);
+        sorted.wx = carver.take<int32_t>(n_points + SORTED_PADDING);
+        sorted.wy = carver.take<int32_t>(n_points + SORTED_PADDING);
+        sorted.wz = carver.take<int32_t>(n_points + SORTED_PADDING);
         counts = carver.take<uint32_t>(n_slots);
         offsets = carver.take<uint64_t>(n_slots + 1);
         scan_scratch = carver.take<uint64_t>(scratch_elements);

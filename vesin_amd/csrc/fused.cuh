@@ -178,32 +178,42 @@ __device__ __forceinline__ uint32_t sweep_columns_wrapped(
     uint32_t (&column)[R]
 ) {
     uint32_t total = 0;
-    for (uint32_t i = 0; i < n_i; i++) {
-        const uint32_t at = first_i + i;
-        const double xi = sorted.x[at];
-        const double yi = sorted.y[at];
-        const double zi = sorted.z[at];
-        const int32_t wix = static_cast<int32_t>(uniform(static_cast<uint32_t>(sorted.wx[at])));
-        const int32_t wiy = static_cast<int32_t>(uniform(static_cast<uint32_t>(sorted.wy[at])));
-        const int32_t wiz = static_cast<int32_t>(uniform(static_cast<uint32_t>(sorted.wz[at])));
-        const bool moved = (wix | wiy | wiz) != 0;
+    for (uint32_t i0 = 0; i0 < n_i; i0 += POINTS_PER_LOAD) {
+        // coordinates and wraps of four points come in through scalar loads, like in sweep_columns
+        const uint32_t at0 = first_i + i0;
+        const FourPoints p = load_four_points(sorted.x + at0, sorted.y + at0, sorted.z + at0);
+        const FourWraps w = load_four_wraps(sorted.wx + at0, sorted.wy + at0, sorted.wz + at0);
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            double tx = c.tx[r];
-            double ty = c.ty[r];
-            double tz = c.tz[r];
-            if (moved) {
-                int32_t bx, by, bz;
-                unpack_shift(c.shift[r], bx, by, bz);
-                shift_vector(g, bx + wix, by + wiy, bz + wiz, tx, ty, tz);
+        for (int u = 0; u < POINTS_PER_LOAD; u++) {
+            if (u > 0 && i0 + u >= n_i) {
+                break;
             }
-            const double vx = (c.x[r] - xi) + tx;
-            const double vy = (c.y[r] - yi) + ty;
-            const double vz = (c.z[r] - zi) + tz;
-            const double d2 = vx * vx + vy * vy + vz * vz;
-            const uint64_t mask = __ballot(d2 < g.cutoff2) & __ballot(c.position[r] > at);
-            total += __popcll(mask);
-            column[r] = shift_in(column[r], mask);
+            const uint32_t at = at0 + u;
+            const double xi = words_to_double(p.x[2 * u], p.x[2 * u + 1]);
+            const double yi = words_to_double(p.y[2 * u], p.y[2 * u + 1]);
+            const double zi = words_to_double(p.z[2 * u], p.z[2 * u + 1]);
+            const int32_t wix = static_cast<int32_t>(w.x[u]);
+            const int32_t wiy = static_cast<int32_t>(w.y[u]);
+            const int32_t wiz = static_cast<int32_t>(w.z[u]);
+            const bool moved = (wix | wiy | wiz) != 0;
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                double tx = c.tx[r];
+                double ty = c.ty[r];
+                double tz = c.tz[r];
+                if (moved) {
+                    int32_t bx, by, bz;
+                    unpack_shift(c.shift[r], bx, by, bz);
+                    shift_vector(g, bx + wix, by + wiy, bz + wiz, tx, ty, tz);
+                }
+                const double vx = (c.x[r] - xi) + tx;
+                const double vy = (c.y[r] - yi) + ty;
+                const double vz = (c.z[r] - zi) + tz;
+                const double d2 = vx * vx + vy * vy + vz * vz;
+                const uint64_t mask = __ballot(d2 < g.cutoff2) & __ballot(c.position[r] > at);
+                total += __popcll(mask);
+                column[r] = shift_in(column[r], mask);
+            }
         }
     }
     return total;

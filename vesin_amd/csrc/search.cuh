@@ -471,6 +471,27 @@ __device__ __forceinline__ FourPoints load_four_points(const double* x, const do
     return p;
 }
 
+typedef uint32_t ScalarWords4 __attribute__((ext_vector_type(4)));
+
+/// The box vectors four consecutive cell-sorted points were moved by, in scalar registers (wave-uniform address;
+/// the three arrays are padded like the coordinates).
+struct FourWraps {
+    ScalarWords4 x, y, z;
+};
+
+__device__ __forceinline__ FourWraps load_four_wraps(const int32_t* wx, const int32_t* wy, const int32_t* wz) {
+    FourWraps w;
+    asm volatile(
+        "s_load_dwordx4 %0, %3, 0x0\n\t"
+        "s_load_dwordx4 %1, %4, 0x0\n\t"
+        "s_load_dwordx4 %2, %5, 0x0\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&s"(w.x), "=&s"(w.y), "=&s"(w.z)
+        : "s"(wx), "s"(wy), "s"(wz)
+    );
+    return w;
+}
+
 __device__ __forceinline__ double words_to_double(uint32_t lo, uint32_t hi) {
     return __longlong_as_double(static_cast<long long>((static_cast<uint64_t>(hi) << 32) | lo));
 }
