@@ -41,12 +41,12 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes moved by ONE launch of the single-pass search kernel on the 1M-atom workload, from rocprofv3 --pmc
-# FETCH_SIZE and WRITE_SIZE runs scaled by a device copy of known size. The figure belongs to the kernel sources whose
+# FETCH_SIZE and WRITE_SIZE runs scaled by a device copy of known size (191.4 MB fetched + 3237.5 MB written). The figure belongs to the kernel sources whose
 # digest is recorded with it: a run with other sources reports no traffic instead of a stale one.
 SEARCH_KERNEL_TRAFFIC = {
-    "bytes": 3_385_800_000,
+    "bytes": 3_428_900_000,
     "profile": "profiles/fused_search_config1_pmc.txt",
-    "kernel_sources_sha256": "unset",
+    "kernel_sources_sha256": "d949fa53303a3bf5575e41724858d573d26887388639e8a120d1b2b55a22957e",
 }
 KERNEL_SOURCES = ["device_common.cuh", "geometry.hpp", "cells.cuh", "search.cuh", "fused.cuh"]
 
