@@ -118,6 +118,13 @@ static bool radix_sort_only() {
     return text != nullptr && std::strcmp(text, "radix") == 0;
 }
 
+/// VESIN_HIP_STREAMS=one keeps every kernel of a call on the call's stream (for comparisons and tests); otherwise the
+/// in-order search orders the candidates of the tiles on a second stream while it counts the rows.
+static bool ordered_one_stream() {
+    const char* text = std::getenv("VESIN_HIP_STREAMS");
+    return text != nullptr && std::strcmp(text, "one") == 0;
+}
+
 namespace {
 
 /// What the counting pass of the in-order search reports (pinned host memory).
@@ -331,6 +338,11 @@ struct HipExtras {
     int in_order_rest = 0;            // calls left before the in-order search is tried again on a system it did not cover
     hipEvent_t events[T_STAGES] = {};
     bool have_events = false;
+    // a second stream of the list's own, for a kernel that can run beside another of the same call (forked from and
+    // joined back into the call's stream with the two events); made when first needed
+    hipStream_t side_stream = nullptr;
+    hipEvent_t side_fork = nullptr;
+    hipEvent_t side_join = nullptr;
     bool timings_valid = false;
     VesinHipTimings timings = {};
     VerletCache* verlet = nullptr;    // only while the caller asks for a skin
@@ -364,6 +376,29 @@ struct HipExtras {
                 (void)hipEventDestroy(event);
             }
         }
+        if (side_fork != nullptr) {
+            (void)hipEventDestroy(side_fork);
+        }
+        if (side_join != nullptr) {
+            (void)hipEventDestroy(side_join);
+        }
+        if (side_stream != nullptr) {
+            (void)hipStreamDestroy(side_stream);
+        }
+    }
+
+    /// The side stream and its events (default priority, like every stream here); nullptr for the entry point that
+    /// allocates nothing, whose kernels all run on the caller's stream.
+    hipStream_t side() {
+        if (fixed_memory) {
+            return nullptr;
+        }
+        if (side_stream == nullptr) {
+            HIP_CHECK(hipEventCreateWithFlags(&side_fork, hipEventDisableTiming));
+            HIP_CHECK(hipEventCreateWithFlags(&side_join, hipEventDisableTiming));
+            HIP_CHECK(hipStreamCreateWithFlags(&side_stream, hipStreamNonBlocking));
+        }
+        return side_stream;
     }
 };
 
@@ -1177,20 +1212,35 @@ bool compute(
         oargs.status = ordered_status;
         oargs.report_order = std::getenv("VESIN_HIP_DEBUG") != nullptr ? 1u : 0u;
         const uint32_t blocks = ordered_blocks;
+        // The order of every tile's candidates, for the writing pass (wasted when the counting pass finds the
+        // system unsuitable, which the host only knows after both). Small systems do without: one more launch
+        // costs them more than ranking the rows of every point does. It reads the cell list only, like the
+        // counting pass, and neither fills the GPU on systems of a few hundred thousand points (one wave per tile,
+        // two waves per SIMD on 100,000 points): the two run side by side, the ordering on a stream of the list's
+        // own that starts after the cell build and that the call's stream waits for right after the counting pass.
+        const bool presorted = ordered_items_per_tile == 1;
+        hipStream_t side = presorted && !ordered_one_stream() ? extras.side() : nullptr;
+        auto launch_order = [&](hipStream_t where) {
+            hipLaunchKernelGGL(
+                ordered_sort_kernel, dim3(static_cast<uint32_t>((tiles_bound + ORDER_WAVES - 1) / ORDER_WAVES)),
+                dim3(ORDER_BLOCK), 0, where, oargs, g
+            );
+        };
+        if (side != nullptr) {
+            HIP_CHECK(hipEventRecord(extras.side_fork, stream));
+            HIP_CHECK(hipStreamWaitEvent(side, extras.side_fork, 0));
+            launch_order(side);
+            HIP_CHECK(hipEventRecord(extras.side_join, side));
+        }
         if (options.full) {
             hipLaunchKernelGGL((ordered_search_kernel<false, true>), dim3(blocks), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
         } else {
             hipLaunchKernelGGL((ordered_search_kernel<false, false>), dim3(blocks), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
         }
-        // The order of every tile's candidates, for the writing pass (wasted when the counting pass finds the
-        // system unsuitable, which the host only knows after both). Small systems do without: one more launch
-        // costs them more than ranking the rows of every point does.
-        const bool presorted = ordered_items_per_tile == 1;
-        if (presorted) {
-            hipLaunchKernelGGL(
-                ordered_sort_kernel, dim3(static_cast<uint32_t>((tiles_bound + ORDER_WAVES - 1) / ORDER_WAVES)),
-                dim3(ORDER_BLOCK), 0, stream, oargs, g
-            );
+        if (side != nullptr) {
+            HIP_CHECK(hipStreamWaitEvent(stream, extras.side_join, 0));
+        } else if (presorted) {
+            launch_order(stream);
         }
         mark(T_COUNT);
         exclusive_scan<SCAN_U32>(rows_of_point, n_points, first_row_of_point, scan_scratch, stream);
