@@ -307,6 +307,30 @@ def test_stencils_larger_than_the_single_pass_tables(timings):
         assert not used_single_pass(calculator)
 
 
+def test_the_single_pass_is_tried_again_after_its_rest(timings):
+    """A list that met a system the single pass does not cover leaves it alone for 64 calls, whatever comes, and
+    takes it up again afterwards: rows right at every step."""
+    rng = np.random.default_rng(42)
+    small_box = np.array([[3.1, 0.0, 0.0], [0.4, 2.9, 0.0], [-0.3, 0.5, 3.3]])
+    awkward = rng.random((40, 3)) @ small_box  # cutoff 8: 7^3 images, beyond the single pass's tables
+    points, box, periodic, _ = configs.config1(4)
+    expected = oracle.neighbors(points, box, periodic, 8.0, True, False, "ijSdD")
+    calculator = NeighborList(cutoff=8.0, full_list=True)
+    call(calculator, points, box, periodic)
+    call(calculator, points, box, periodic)
+    assert used_single_pass(calculator)
+    for _ in range(2):  # the first of these tries the single pass and finds the stencil too large
+        call(calculator, awkward, small_box, True)
+        assert not used_single_pass(calculator)
+    used = []
+    for step in range(70):
+        result = call(calculator, points, box, periodic)
+        used.append(used_single_pass(calculator))
+        if step in (0, 30, 62, 63, 64, 69):
+            assert_same_list(result, expected, what=f"step {step}")
+    assert not any(used[:63]) and all(used[63:]), used
+
+
 def _single_pass_reports(capfd):
     return [line for line in capfd.readouterr().err.splitlines() if line.startswith("single pass:")]
 
