@@ -1,0 +1,211 @@
+"""Sorted lists of small systems on a reused list: cell list, counting, scan and writing happen in ONE launch whose
+workgroups wait for each other (ordered_small_kernel). Checked in place against the canonicalised oracle: the three
+shapes of the launch, half and full lists, boxes with images, mixed periodicity, the cases the launch leaves to the
+other paths (too many rows per point, too many candidates, wraps beyond the key's range, rows that do not fit,
+workgroups that give up waiting, which the host forces through the spin limit), and VESIN_HIP_LAUNCHES=separate."""
+
+import numpy as np
+import pytest
+
+import oracle
+from vesin_amd import NeighborList, configs
+
+pytestmark = pytest.mark.gpu
+
+NAMES = {"P": "pairs", "S": "shifts", "d": "distances", "D": "vectors"}
+
+
+def _compute(calculator, points, box, periodic, quantities="PSdD"):
+    import torch
+
+    outputs = calculator.compute(
+        torch.tensor(np.ascontiguousarray(points), device="cuda:0"),
+        torch.tensor(np.ascontiguousarray(box), device="cuda:0"),
+        periodic,
+        quantities,
+    )
+    return {NAMES[q]: out.cpu().numpy() for q, out in zip(quantities, outputs)}
+
+
+def _expected(points, box, periodic, cutoff, full):
+    flags = [bool(periodic)] * 3 if isinstance(periodic, (bool, np.bool_)) else [bool(p) for p in periodic]
+    return oracle.canonicalize(oracle.neighbors(points, box, flags, cutoff, full, False, "ijSdD"))
+
+
+def _same(result, expected, what):
+    for key in result:
+        assert result[key].shape == expected[key].shape, (what, key, result[key].shape, expected[key].shape)
+        assert np.array_equal(result[key], expected[key]), (what, key)
+
+
+def _one_launch_lines(err):
+    return [line for line in err.splitlines() if line.startswith("one launch:")]
+
+
+def _liquid(n, density, seed, triclinic=False):
+    rng = np.random.default_rng(seed)
+    edge = (n / density) ** (1.0 / 3.0)
+    box = np.eye(3) * edge
+    if triclinic:
+        box = box + 0.15 * edge * rng.normal(size=(3, 3)) * (np.arange(3)[:, None] > np.arange(3)[None, :])
+    return rng.random((n, 3)) @ box, box
+
+
+@pytest.mark.parametrize("full", [True, False], ids=["full", "half"])
+@pytest.mark.parametrize("n", [1, 3, 64, 216, 960, 961, 1920, 1921, 2048])
+def test_every_shape_of_the_launch(n, full, capfd, monkeypatch):
+    """4, 8 and 16 waves per workgroup, at the sizes where one shape hands over to the next; the second and third call
+    of a list go through the one launch and say so."""
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    points, box = _liquid(n, 0.05, seed=n, triclinic=n % 2 == 1)
+    expected = _expected(points, box, True, 4.0, full)
+    calculator = NeighborList(cutoff=4.0, full_list=full, sorted=True)
+    for call in range(3):
+        capfd.readouterr()
+        result = _compute(calculator, points, box, True)
+        lines = _one_launch_lines(capfd.readouterr().err)
+        _same(result, expected, f"n={n} call {call}")
+        if call == 0:
+            assert not lines  # a list without arrays sizes them with the counting pass first
+        elif n >= 64:  # (the boxes of the smallest ones need more images than the in-order search takes)
+            assert len(lines) == 1 and "gave up 0" in lines[0], lines
+
+
+def test_config0_on_a_reused_list(capfd, monkeypatch):
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    points, box, periodic, options = configs.config0()
+    expected = _expected(points, box, True, options["cutoff"], True)
+    calculator = NeighborList(cutoff=options["cutoff"], full_list=True, sorted=True)
+    for call in range(4):
+        capfd.readouterr()
+        for letters in ("PSdD", "P", "Sd"):
+            result = _compute(calculator, points, box, True, letters)
+            _same(result, {key: expected[key] for key in result}, f"call {call} {letters}")
+    assert _one_launch_lines(capfd.readouterr().err)
+
+
+@pytest.mark.parametrize("full", [True, False], ids=["full", "half"])
+def test_images_of_a_small_box_and_mixed_periodicity(full, capfd, monkeypatch):
+    """One cell whose stencil is the images of the box (every point pairs with its own images), slabs and free
+    clusters, points outside of the box: all on one reused list."""
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    rng = np.random.default_rng(23)
+    calculator = NeighborList(cutoff=3.0, full_list=full, sorted=True)
+    small = np.array([[3.2, 0.0, 0.0], [0.4, 3.1, 0.0], [-0.3, 0.2, 3.3]])
+    wide = np.array([[11.0, 0.0, 0.0], [1.5, 10.0, 0.0], [-2.0, 0.7, 12.0]])
+    used = 0
+    for step in range(12):
+        box = small if step % 3 == 0 else wide
+        n = int(rng.choice([5, 7])) if box is small else int(rng.choice([40, 150, 400]))
+        points = rng.random((n, 3)) @ box
+        if step % 2 == 1:
+            points = points + rng.integers(-2, 3, size=(n, 3)) @ box  # wraps within the key's range
+        periodic = [(True, True, True), (True, True, False), (False, False, False), (True, False, True)][step % 4]
+        if box is small:
+            periodic = (True, True, True)
+        expected = _expected(points, box, periodic, 3.0, full)
+        capfd.readouterr()
+        result = _compute(calculator, points, box, list(periodic))
+        used += len(_one_launch_lines(capfd.readouterr().err))
+        _same(result, expected, f"step {step} n={n} periodic={periodic}")
+    assert used >= 8
+
+
+def test_what_the_launch_leaves_to_the_other_paths(capfd, monkeypatch):
+    """Too many rows per point (more than 256), too many candidates per point (more than 1024), wraps beyond +-255,
+    more rows than the arrays hold: the call's result is the oracle's all the same, and the list then stays away
+    from the one launch for a while."""
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    calculator = NeighborList(cutoff=4.0, full_list=True, sorted=True)
+    ordinary, box = _liquid(300, 0.05, seed=1)
+    _same(_compute(calculator, ordinary, box, True), _expected(ordinary, box, True, 4.0, True), "first call")
+    capfd.readouterr()
+    _same(_compute(calculator, ordinary, box, True), _expected(ordinary, box, True, 4.0, True), "second call")
+    assert _one_launch_lines(capfd.readouterr().err)
+
+    # dense: 1.2 points per cubic A, 320 rows per point
+    dense, dense_box = _liquid(500, 1.2, seed=2)
+    expected = _expected(dense, dense_box, True, 4.0, True)
+    assert len(expected["pairs"]) / 500 > 256
+    capfd.readouterr()
+    _same(_compute(calculator, dense, dense_box, True), expected, "dense")
+    lines = _one_launch_lines(capfd.readouterr().err)
+    assert len(lines) == 1 and "gave up 0" in lines[0]
+    # ... and the next calls do not ask again
+    capfd.readouterr()
+    _same(_compute(calculator, ordinary, box, True), _expected(ordinary, box, True, 4.0, True), "after dense")
+    assert not _one_launch_lines(capfd.readouterr().err)
+
+    # a fresh list for each of the other cases, warmed up with the ordinary system
+    def warmed():
+        fresh = NeighborList(cutoff=4.0, full_list=True, sorted=True)
+        _compute(fresh, ordinary, box, True)
+        return fresh
+
+    # points hundreds of boxes away
+    far = ordinary + np.array([300, -400, 260]) @ box
+    fresh = warmed()
+    capfd.readouterr()
+    _same(_compute(fresh, far, box, True), _expected(far, box, True, 4.0, True), "far away")
+    lines = _one_launch_lines(capfd.readouterr().err)
+    assert len(lines) == 1 and "unsuitable 0" not in lines[0]
+
+    # more rows than the arrays of the list hold: the ordinary system, then one four times as dense
+    denser, denser_box = _liquid(1200, 0.2, seed=3)
+    fresh = warmed()
+    capfd.readouterr()
+    _same(_compute(fresh, denser, denser_box, True), _expected(denser, denser_box, True, 4.0, True), "grown")
+    assert len(_one_launch_lines(capfd.readouterr().err)) == 1
+
+
+def test_a_coordinate_that_is_not_finite(monkeypatch):
+    import torch
+
+    calculator = NeighborList(cutoff=4.0, full_list=True, sorted=True)
+    points, box = _liquid(100, 0.05, seed=4)
+    _compute(calculator, points, box, True)
+    _compute(calculator, points, box, True)
+    broken = points.copy()
+    broken[37, 1] = np.inf
+    with pytest.raises(RuntimeError, match="point 37"):
+        calculator.compute(torch.tensor(broken, device="cuda:0"), torch.tensor(box, device="cuda:0"), True, "P")
+    # the list is as good as before
+    _same(_compute(calculator, points, box, True), _expected(points, box, True, 4.0, True), "after the error")
+
+
+@pytest.mark.parametrize("full", [True, False], ids=["full", "half"])
+def test_workgroups_that_give_up_waiting(full, capfd, monkeypatch):
+    """A spin limit of zero makes every workgroup that is not the last to arrive give up at once: nothing is written
+    by that launch, the host goes on with the separate passes, the rows are the oracle's."""
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    points, box = _liquid(700, 0.05, seed=5, triclinic=True)
+    expected = _expected(points, box, True, 4.0, full)
+    calculator = NeighborList(cutoff=4.0, full_list=full, sorted=True)
+    _same(_compute(calculator, points, box, True), expected, "first call")
+    monkeypatch.setenv("VESIN_HIP_CHAIN_SPINS", "0")
+    capfd.readouterr()
+    _same(_compute(calculator, points, box, True), expected, "gave up")
+    lines = _one_launch_lines(capfd.readouterr().err)
+    assert len(lines) == 1 and "gave up 1" in lines[0], lines
+    monkeypatch.delenv("VESIN_HIP_CHAIN_SPINS")
+    # the list leaves the one launch alone for 64 calls, then comes back to it
+    for call in range(64):
+        capfd.readouterr()
+        result = _compute(calculator, points, box, True, "P")
+        assert not _one_launch_lines(capfd.readouterr().err), call
+    _same(result, {"pairs": expected["pairs"]}, "while resting")
+    capfd.readouterr()
+    _same(_compute(calculator, points, box, True), expected, "back")
+    lines = _one_launch_lines(capfd.readouterr().err)
+    assert len(lines) == 1 and "gave up 0" in lines[0], lines
+
+
+def test_separate_launches_on_request(capfd, monkeypatch):
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    monkeypatch.setenv("VESIN_HIP_LAUNCHES", "separate")
+    points, box, periodic, options = configs.config0()
+    expected = _expected(points, box, True, options["cutoff"], True)
+    calculator = NeighborList(cutoff=options["cutoff"], full_list=True, sorted=True)
+    for call in range(3):
+        _same(_compute(calculator, points, box, True), expected, f"call {call}")
+    assert not _one_launch_lines(capfd.readouterr().err)

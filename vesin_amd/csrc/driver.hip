@@ -120,6 +120,13 @@ static bool radix_sort_only() {
     return text != nullptr && std::strcmp(text, "radix") == 0;
 }
 
+/// VESIN_HIP_LAUNCHES=separate keeps the passes of a small system's search in launches of their own (for comparisons
+/// and tests) instead of one launch whose workgroups wait for each other between the passes.
+static bool separate_launches() {
+    const char* text = std::getenv("VESIN_HIP_LAUNCHES");
+    return text != nullptr && std::strcmp(text, "separate") == 0;
+}
+
 /// VESIN_HIP_STREAMS=one keeps every kernel of a call on the call's stream (for comparisons and tests); otherwise the
 /// in-order search orders the candidates of the tiles on a second stream while it counts the rows.
 static bool ordered_one_stream() {
@@ -128,14 +135,6 @@ static bool ordered_one_stream() {
 }
 
 namespace {
-
-/// What the counting pass of the in-order search reports (pinned host memory).
-struct OrderedHostStatus {
-    OrderedStatus found;
-    unsigned long long total_rows;
-    unsigned int first_bad_coordinate;
-    unsigned int padding;
-};
 
 __global__ void publish_ordered_status(
     const OrderedStatus* found, const uint64_t* total, const DeviceStatus* status, OrderedHostStatus* host
@@ -338,6 +337,10 @@ struct HipExtras {
     int single_pass_rest = 0;         // calls left before the single-pass search is tried again after it did not fit
     int direct_rest = 0;              // calls left before the one-pass cell build is tried again after a cell overflowed
     int in_order_rest = 0;            // calls left before the in-order search is tried again on a system it did not cover
+    int one_launch_rest = 0;          // calls left before a small system is tried in one launch again
+    SmallMeeting* meetings = nullptr; // device, two of them (see SmallMeeting); allocated at the first small system
+    bool own_meetings = false;        // allocated by this state (not part of memory that was handed to it)
+    uint32_t meeting_turn = 0;
     hipEvent_t events[T_STAGES] = {};
     bool have_events = false;
     // a second stream of the list's own, for a kernel that can run beside another of the same call (forked from and
@@ -366,6 +369,9 @@ struct HipExtras {
         work.release();
         sort_work.release();
         if (!fixed_memory) {
+            if (meetings != nullptr && own_meetings) {
+                (void)hipFree(meetings);
+            }
             if (d_status != nullptr) {
                 (void)hipFree(d_status);
             }
@@ -987,6 +993,105 @@ bool compute(
     carve(carver);
     extras.batch.on_device = false; // what a batch left in this buffer is about to be overwritten
 
+    auto check_pair_limit = [&](size_t total) {
+        if (pair_limit != 0 && total > n_points * pair_limit) {
+            throw std::runtime_error(
+                "The number of neighbor pairs exceeds the maximum capacity of " + std::to_string(n_points * pair_limit) +
+                " (max_pairs_per_point=" + std::to_string(pair_limit) + "; n_points=" + std::to_string(n_points) + "). " +
+                "Consider reducing the cutoff distance, or explicitly setting " +
+                "VESIN_CUDA_MAX_PAIRS_PER_POINT as an environment variable."
+            );
+        }
+    };
+
+    // ---- small systems with arrays from earlier calls, sorted lists: cell list, counting, scan, report to the host
+    // and writing in one launch (ordered_small_kernel). Its workgroups wait for each other, which needs all of them
+    // resident at once; when they were not, or the system does not suit the in-order search, or the rows do not
+    // fit, the call goes on as if nothing had happened, and the list leaves that launch alone for a while.
+    bool one_launch = try_in_order && extras.capacity > 0 && n_points <= ORDERED_SMALL_POINTS &&
+                      n_cells <= ORDERED_SMALL_POINTS && !separate_launches() && !ordered_rows() &&
+                      std::getenv("VESIN_HIP_CELLS") == nullptr;
+    if (one_launch && extras.one_launch_rest > 0) {
+        extras.one_launch_rest -= 1;
+        one_launch = false;
+    }
+    if (one_launch && extras.meetings == nullptr) {
+        if (extras.fixed_memory) {
+            one_launch = false; // no allocation there
+        } else {
+            HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&extras.meetings), 2 * sizeof(SmallMeeting)));
+            extras.own_meetings = true;
+            HIP_CHECK(hipMemset(extras.meetings, 0, 2 * sizeof(SmallMeeting)));
+        }
+    }
+    if (one_launch) {
+        size_outputs(neighbors, extras, 0, options);
+        SmallArgs sargs = {};
+        sargs.points = reinterpret_cast<const double*>(points);
+        sargs.box = fetched ? nullptr : reinterpret_cast<const double*>(box);
+        sargs.periodic = periodic;
+        sargs.host_small = extras.mail_device->small;
+        sargs.rows_of_point = rows_of_point;
+        sargs.meeting = extras.meetings + (extras.meeting_turn & 1u);
+        sargs.next_meeting = extras.meetings + ((extras.meeting_turn + 1u) & 1u);
+        extras.meeting_turn += 1;
+        sargs.host = &extras.mail_device->ordered;
+        sargs.spin_limit = std::min(chain_spin_limit(), ORDERED_SMALL_SPINS);
+        sargs.capacity = extras.capacity;
+        sargs.out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
+        sargs.out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
+        sargs.out.distances = neighbors.distances;
+        sargs.out.vectors = reinterpret_cast<double*>(neighbors.vectors);
+        // few waves per workgroup when that still covers the points: the arithmetic spreads over more compute units
+        if (n_points <= SmallShape<4>::MAX_POINTS && n_cells <= SmallShape<4>::CAPACITY) {
+            auto kernel = options.full ? ordered_small_kernel<true, 4> : ordered_small_kernel<false, 4>;
+            hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>((n_points + 3) / 4)), dim3(4 * WAVE), 0, stream, sargs, g);
+        } else if (n_points <= SmallShape<8>::MAX_POINTS) {
+            auto kernel = options.full ? ordered_small_kernel<true, 8> : ordered_small_kernel<false, 8>;
+            hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>((n_points + 7) / 8)), dim3(8 * WAVE), 0, stream, sargs, g);
+        } else {
+            auto kernel = options.full ? ordered_small_kernel<true, 16> : ordered_small_kernel<false, 16>;
+            hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>((n_points + 15) / 16)), dim3(16 * WAVE), 0, stream, sargs, g);
+        }
+        fetched = true;
+        mark(T_CELLS);
+        mark(T_WRITE);
+        extras.wait(stream);
+        if (!box_was_right()) {
+            return false;
+        }
+        const OrderedHostStatus found = extras.mail->ordered;
+        if (found.first_bad_coordinate != 0xFFFFFFFFu) {
+            non_finite_error(points, found.first_bad_coordinate);
+        }
+        const bool suitable = found.found.gave_up == 0 && found.found.max_rows <= ORDERED_MAX_ROWS &&
+                              found.found.max_candidates <= ORDERED_CANDIDATES && found.found.unsuitable == 0;
+        if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
+            std::fprintf(
+                stderr, "one launch: rows %llu, most rows of a point %u, most candidates of a point %u, unsuitable %u, gave up %u\n",
+                found.total_rows, found.found.max_rows, found.found.max_candidates, found.found.unsuitable, found.found.gave_up
+            );
+        }
+        if (suitable && found.total_rows <= extras.capacity) {
+            check_pair_limit(found.total_rows);
+            HIP_CHECK(hipGetLastError());
+            neighbors.length = found.total_rows;
+            if (timed) {
+                float ms = 0.0f;
+                HIP_CHECK(hipEventElapsedTime(&ms, extras.events[T_START], extras.events[T_WRITE]));
+                extras.timings = {};
+                extras.timings.total = ms;
+                extras.timings.write = ms;
+                extras.timings_valid = true;
+            }
+            return true;
+        }
+        if (!suitable) {
+            // (rows that do not fit are no reason: the arrays grow below and the next call finds room)
+            extras.one_launch_rest = SINGLE_PASS_REST;
+        }
+    }
+
     // ---- cell list
     const uint32_t point_blocks = static_cast<uint32_t>((n_points + BLOCK - 1) / BLOCK);
     const auto* flat_points = reinterpret_cast<const double*>(points);
@@ -1084,16 +1189,6 @@ bool compute(
         out.distances = neighbors.distances;
         out.vectors = reinterpret_cast<double*>(neighbors.vectors);
         return out;
-    };
-    auto check_pair_limit = [&](size_t total) {
-        if (pair_limit != 0 && total > n_points * pair_limit) {
-            throw std::runtime_error(
-                "The number of neighbor pairs exceeds the maximum capacity of " + std::to_string(n_points * pair_limit) +
-                " (max_pairs_per_point=" + std::to_string(pair_limit) + "; n_points=" + std::to_string(n_points) + "). " +
-                "Consider reducing the cutoff distance, or explicitly setting " +
-                "VESIN_CUDA_MAX_PAIRS_PER_POINT as an environment variable."
-            );
-        }
     };
     auto elapsed = [&](Stage from, Stage to) {
         float ms = 0.0f;
@@ -1221,32 +1316,12 @@ bool compute(
         // two waves per SIMD on 100,000 points): the two run side by side, the ordering on a stream of the list's
         // own that starts after the cell build and that the call's stream waits for right after the counting pass.
         const bool presorted = ordered_items_per_tile == 1;
-        hipStream_t side = presorted && !ordered_one_stream() ? extras.side() : nullptr;
         auto launch_order = [&](hipStream_t where) {
             hipLaunchKernelGGL(
                 ordered_sort_kernel, dim3(static_cast<uint32_t>((tiles_bound + ORDER_WAVES - 1) / ORDER_WAVES)),
                 dim3(ORDER_BLOCK), 0, where, oargs, g
             );
         };
-        if (side != nullptr) {
-            HIP_CHECK(hipEventRecord(extras.side_fork, stream));
-            HIP_CHECK(hipStreamWaitEvent(side, extras.side_fork, 0));
-            launch_order(side);
-            HIP_CHECK(hipEventRecord(extras.side_join, side));
-        }
-        if (options.full) {
-            hipLaunchKernelGGL((ordered_search_kernel<false, true>), dim3(blocks), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
-        } else {
-            hipLaunchKernelGGL((ordered_search_kernel<false, false>), dim3(blocks), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
-        }
-        if (side != nullptr) {
-            HIP_CHECK(hipStreamWaitEvent(stream, extras.side_join, 0));
-        } else if (presorted) {
-            launch_order(stream);
-        }
-        mark(T_COUNT);
-        exclusive_scan<SCAN_U32>(rows_of_point, n_points, first_row_of_point, scan_scratch, stream);
-        mark(T_SCAN);
         auto launch_write = [&]() {
             auto kernel = presorted ? (options.full ? ordered_search_kernel<true, true, true> : ordered_search_kernel<true, false, true>)
                                     : (options.full ? ordered_search_kernel<true, true, false> : ordered_search_kernel<true, false, false>);
@@ -1263,17 +1338,44 @@ bool compute(
             oargs.out = outputs_of();
             oargs.capacity = early_capacity;
             oargs.guarded = 1;
-            mark(T_WRITE_BEGIN);
-            launch_write();
-            mark(T_WRITE);
         }
-        hipLaunchKernelGGL(
-            publish_ordered_status, dim3(1), dim3(1), 0, stream,
-            ordered_status, first_row_of_point + n_points, extras.d_status, &extras.mail_device->ordered
-        );
-        extras.wait(stream);
-        if (!box_was_right()) {
-            return false;
+        auto launch_count_and_scan = [&]() {
+            hipStream_t side = presorted && !ordered_one_stream() ? extras.side() : nullptr;
+            if (side != nullptr) {
+                HIP_CHECK(hipEventRecord(extras.side_fork, stream));
+                HIP_CHECK(hipStreamWaitEvent(side, extras.side_fork, 0));
+                launch_order(side);
+                HIP_CHECK(hipEventRecord(extras.side_join, side));
+            }
+            if (options.full) {
+                hipLaunchKernelGGL((ordered_search_kernel<false, true>), dim3(blocks), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
+            } else {
+                hipLaunchKernelGGL((ordered_search_kernel<false, false>), dim3(blocks), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
+            }
+            if (side != nullptr) {
+                HIP_CHECK(hipStreamWaitEvent(stream, extras.side_join, 0));
+            } else if (presorted) {
+                launch_order(stream);
+            }
+            mark(T_COUNT);
+            exclusive_scan<SCAN_U32>(rows_of_point, n_points, first_row_of_point, scan_scratch, stream);
+            mark(T_SCAN);
+        };
+        {
+            launch_count_and_scan();
+            if (early_write) {
+                mark(T_WRITE_BEGIN);
+                launch_write();
+                mark(T_WRITE);
+            }
+            hipLaunchKernelGGL(
+                publish_ordered_status, dim3(1), dim3(1), 0, stream,
+                ordered_status, first_row_of_point + n_points, extras.d_status, &extras.mail_device->ordered
+            );
+            extras.wait(stream);
+            if (!box_was_right()) {
+                return false;
+            }
         }
         const OrderedHostStatus found = extras.mail->ordered;
         if (found.first_bad_coordinate != 0xFFFFFFFFu) {
@@ -2229,6 +2331,7 @@ void neighbors_no_alloc(
     extras.single_pass_rest = 0;
     extras.direct_rest = 0;
     extras.in_order_rest = 0;
+    extras.one_launch_rest = 0;
     extras.timings_valid = false;
 
     VesinNeighborList list;

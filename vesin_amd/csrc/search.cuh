@@ -170,10 +170,11 @@ __device__ __forceinline__ void wave_sync() {
 
 /// Stencil entries [first_linear, first_linear + n_batch) around cell (cx, cy, cz) go to the wave's LDS tables:
 /// neighbour cell start, packed cell shift, and the running number of candidates (scanned in place). Linear stencil
-/// offsets run dx major, dz minor.
+/// offsets run dx major, dz minor. `cell_scan`: exclusive scan of the points per cell in the low 32 bits of its words.
+template <typename ScanWord>
 __device__ __forceinline__ void fill_stencil_tables(
     SearchTables& sh, int lane, uint32_t first_linear, uint32_t n_batch, int32_t cx, int32_t cy, int32_t cz,
-    int32_t span_y, int32_t span_z, const GridParams& g, const uint64_t* __restrict__ cell_scan,
+    int32_t span_y, int32_t span_z, const GridParams& g, const ScanWord* __restrict__ cell_scan,
     const uint32_t* __restrict__ direct_counts = nullptr, uint32_t direct_capacity = 0
 ) {
     const uint32_t centre = static_cast<uint32_t>(2 * g.s[0] + 1) * span_y * span_z / 2;
