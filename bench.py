@@ -23,7 +23,7 @@ The line carries, next to the throughput:
   and one thread on a bounded sample of the same workload.
 
 ``--config NAME`` makes another configuration the workload of the line (profiling runs use it):
-config0, config1 (default), config1_shuffled, config2, config3, config4a, config4b.
+config0, config1 (default), config1_shuffled, config2, config3, config3_single, config4a, config4b.
 """
 
 import argparse
@@ -44,13 +44,13 @@ HBM_PEAK_GBS = 8000.0
 # FETCH_SIZE and WRITE_SIZE runs scaled by a device copy of known size (191.4 MB fetched + 3237.5 MB written). The figure belongs to the kernel sources whose
 # digest is recorded with it: a run with other sources reports no traffic instead of a stale one.
 SEARCH_KERNEL_TRAFFIC = {
-    "bytes": 3_428_900_000,
+    "bytes": 3_428_500_000,
     "profile": "profiles/fused_search_config1_pmc.txt",
-    "kernel_sources_sha256": "d949fa53303a3bf5575e41724858d573d26887388639e8a120d1b2b55a22957e",
+    "kernel_sources_sha256": "198320dba42ed6cae640ba23653817a773590997c50ec4219f9527668098dcb3",
 }
 KERNEL_SOURCES = ["device_common.cuh", "geometry.hpp", "cells.cuh", "search.cuh", "fused.cuh"]
 
-CONFIG_NAMES = ["config0", "config1", "config1_shuffled", "config2", "config3", "config4a", "config4b"]
+CONFIG_NAMES = ["config0", "config1", "config1_shuffled", "config2", "config3", "config3_single", "config4a", "config4b"]
 DESCRIPTIONS = {
     "config0": "config0: 216 atoms, cutoff 5 A, full, sorted, i j S d",
     "config1": "config1: jittered diamond {replicas}^3 cells = {n_points} atoms, periodic cube, cutoff 5 A, full list, "
@@ -59,6 +59,7 @@ DESCRIPTIONS = {
     "config1_box_changes": "config1 with a box that differs from the call before on every call",
     "config2": "config2: 100000 atoms, triclinic, cutoff 6 A, half, sorted, i j S d D",
     "config3": "config3: 4096 replicas of 64 atoms, box 7.134 A, cutoff 10 A, full, i j S d, one batched call",
+    "config3_single": "one replica of config3 in a call of its own: 64 atoms, box 7.134 A, cutoff 10 A, full, i j S d",
     "config4a": "config4a: 500000 clustered atoms, no periodic direction, cutoff 4.5 A, full, i j d",
     "config4b": "config4b: the same atoms, periodic (T, T, F)",
 }
@@ -88,6 +89,8 @@ def host_system(name, replicas=50):
         return points[np.random.default_rng(1).permutation(len(points))], box, periodic, options
     if name == "config2":
         return configs.config2()
+    if name == "config3_single":
+        return configs.config3(0)
     if name == "config4a":
         return configs.config4(periodic=(False, False, False))
     if name == "config4b":
@@ -366,7 +369,7 @@ def main():
 def other_configs(args, torch, np):
     """Steady-state figures of the other configurations: 10 timed calls each after the list's first call and 3 more."""
     results = []
-    names = [name for name in ["config0", "config2", "config3", "config4a", "config4b"] if name != args.config]
+    names = [name for name in ["config0", "config2", "config3", "config3_single", "config4a", "config4b"] if name != args.config]
     if args.config == "config1":
         names += ["config1_shuffled", "config1_box_changes"]
     for name in names:

@@ -35,6 +35,13 @@ def call(calculator, points, box, periodic, letters="PSdD"):
     return {NAMES[q]: out.cpu().numpy() for q, out in zip(letters, outputs)}
 
 
+@pytest.fixture(autouse=True)
+def separate_launches(monkeypatch):
+    """Small systems with arrays from earlier calls would go through the one launch of tests/test_gpu_small_*.py
+    instead; here they are what drives the single-pass search through its branches."""
+    monkeypatch.setenv("VESIN_HIP_LAUNCHES", "separate")
+
+
 @pytest.fixture
 def timings():
     enable_timings(True)

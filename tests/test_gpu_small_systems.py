@@ -1,13 +1,15 @@
-"""Sorted lists of small systems on a reused list: cell list, counting, scan and writing happen in ONE launch whose
-workgroups wait for each other (ordered_small_kernel). Checked in place against the canonicalised oracle: the three
-shapes of the launch, half and full lists, boxes with images, mixed periodicity, the cases the launch leaves to the
-other paths (too many rows per point, too many candidates, wraps beyond the key's range, rows that do not fit,
-workgroups that give up waiting, which the host forces through the spin limit), and VESIN_HIP_LAUNCHES=separate."""
+"""Small systems on a reused list: cell list, counting, scan and writing happen in ONE launch whose workgroups wait
+for each other (small_system_kernel). Sorted lists are checked in place against the canonicalised oracle, unsorted
+ones as sets of rows: the shapes of the launch, half and full lists, several work items per point, boxes with images,
+mixed periodicity, the cases the launch leaves to the other paths (too many rows per point, too many candidates,
+wraps beyond the key's range, rows that do not fit, workgroups that give up waiting, which the host forces through
+the spin limit), and VESIN_HIP_LAUNCHES=separate."""
 
 import numpy as np
 import pytest
 
 import oracle
+from _helpers import assert_same_list
 from vesin_amd import NeighborList, configs
 
 pytestmark = pytest.mark.gpu
@@ -209,3 +211,121 @@ def test_separate_launches_on_request(capfd, monkeypatch):
     for call in range(3):
         _same(_compute(calculator, points, box, True), expected, f"call {call}")
     assert not _one_launch_lines(capfd.readouterr().err)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# unsorted lists: one work item per point and slice of its candidates, the upper half of the stencil
+
+
+def _unsorted_expected(points, box, periodic, cutoff, full):
+    flags = [bool(periodic)] * 3 if isinstance(periodic, (bool, np.bool_)) else [bool(p) for p in periodic]
+    return oracle.neighbors(points, box, flags, cutoff, full, False, "ijSdD")
+
+
+def _items_per_point(lines):
+    return [int(line.split(" items per point")[0].split()[-1]) for line in lines]
+
+
+@pytest.mark.parametrize("full", [True, False], ids=["full", "half"])
+@pytest.mark.parametrize("n,density", [(30, 0.05), (64, 0.3), (216, 0.05), (216, 0.4), (300, 0.2), (700, 0.05), (960, 0.05)])
+def test_unsorted_lists_with_one_or_several_items_per_point(n, density, full, capfd, monkeypatch):
+    """From one item per point to as many as the launch takes; with three items per point and four waves per
+    workgroup the slices of most points are counted by different workgroups, whose copies of the points are in
+    different orders inside the cells."""
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    points, box = _liquid(n, density, seed=n + int(100 * density), triclinic=True)
+    points = points + np.random.default_rng(n).integers(-1, 2, size=(n, 3)) @ box
+    expected = _unsorted_expected(points, box, True, 4.0, full)
+    calculator = NeighborList(cutoff=4.0, full_list=full)
+    seen = []
+    for call in range(4):
+        capfd.readouterr()
+        result = _compute(calculator, points, box, True)
+        lines = _one_launch_lines(capfd.readouterr().err)
+        assert_same_list(result, expected, what=f"n={n} density={density} call {call}")
+        if call > 0:
+            assert len(lines) == 1 and "gave up 0" in lines[0], lines
+            seen += _items_per_point(lines)
+    assert len(set(seen)) == 1
+    if density >= 0.2 and n <= 300:
+        assert seen[0] > 1
+
+
+def test_unsorted_single_replica_of_the_small_cell_case(capfd, monkeypatch):
+    """64 atoms in a box of 7.134 A with a cutoff of 10 A: 63 stencil entries of images, 726 rows per point."""
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    for replica in (0, 5):
+        points, box, periodic, options = configs.config3(replica)
+        expected = _unsorted_expected(points, box, True, options["cutoff"], True)
+        calculator = NeighborList(cutoff=options["cutoff"], full_list=True)
+        for call in range(3):
+            capfd.readouterr()
+            result = _compute(calculator, points, box, True)
+            lines = _one_launch_lines(capfd.readouterr().err)
+            assert_same_list(result, expected, what=f"replica {replica} call {call}")
+            assert len(lines) == (0 if call == 0 else 1)
+        assert _items_per_point(lines)[0] > 4
+
+
+@pytest.mark.parametrize("full", [True, False], ids=["full", "half"])
+def test_unsorted_mixed_periodicity_images_and_changing_systems(full, capfd, monkeypatch):
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    rng = np.random.default_rng(31)
+    calculator = NeighborList(cutoff=3.0, full_list=full)
+    small = np.array([[3.2, 0.0, 0.0], [0.4, 3.1, 0.0], [-0.3, 0.2, 3.3]])
+    wide = np.array([[11.0, 0.0, 0.0], [1.5, 10.0, 0.0], [-2.0, 0.7, 12.0]])
+    used = 0
+    for step in range(16):
+        box = small if step % 3 == 0 else wide
+        n = int(rng.choice([5, 7, 12])) if box is small else int(rng.choice([40, 150, 400, 900]))
+        points = rng.random((n, 3)) @ box
+        if step % 2 == 1:
+            points = points + rng.integers(-2, 3, size=(n, 3)) @ box
+        periodic = [(True, True, True), (True, True, False), (False, False, False), (True, False, True)][step % 4]
+        if box is small:
+            periodic = (True, True, True)
+        expected = _unsorted_expected(points, box, periodic, 3.0, full)
+        capfd.readouterr()
+        result = _compute(calculator, points, box, list(periodic))
+        used += len(_one_launch_lines(capfd.readouterr().err))
+        assert_same_list(result, expected, what=f"step {step} n={n} periodic={periodic}")
+    assert used >= 10
+
+
+def test_what_the_unsorted_launch_leaves_to_the_other_paths(capfd, monkeypatch):
+    """More rows than the arrays hold, wraps beyond +-255, workgroups that give up: the rows are the oracle's."""
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    ordinary, box = _liquid(300, 0.05, seed=1)
+
+    def warmed():
+        fresh = NeighborList(cutoff=4.0, full_list=True)
+        _compute(fresh, ordinary, box, True)
+        capfd.readouterr()
+        assert_same_list(_compute(fresh, ordinary, box, True), _unsorted_expected(ordinary, box, True, 4.0, True))
+        assert _one_launch_lines(capfd.readouterr().err)
+        return fresh
+
+    # 260 of the 300 points within 1 A of one place: 67,000 rows where the list's arrays hold 4,000. The launch counts
+    # them, writes nothing, the call goes on with the other passes and grown arrays, and the next call fits
+    clump = ordinary.copy()
+    clump[:260] = clump[0] + np.random.default_rng(2).normal(scale=0.5, size=(260, 3))
+    calculator = warmed()
+    for call in range(2):
+        capfd.readouterr()
+        assert_same_list(_compute(calculator, clump, box, True), _unsorted_expected(clump, box, True, 4.0, True), what="clump")
+        lines = _one_launch_lines(capfd.readouterr().err)
+        assert len(lines) == 1 and "gave up 0" in lines[0] and "unsuitable 0" in lines[0]
+
+    far = ordinary + np.array([300, -400, 260]) @ box
+    calculator = warmed()
+    capfd.readouterr()
+    assert_same_list(_compute(calculator, far, box, True), _unsorted_expected(far, box, True, 4.0, True), what="far away")
+    lines = _one_launch_lines(capfd.readouterr().err)
+    assert len(lines) == 1 and "unsuitable 0" not in lines[0]
+
+    calculator = warmed()
+    monkeypatch.setenv("VESIN_HIP_CHAIN_SPINS", "0")
+    capfd.readouterr()
+    assert_same_list(_compute(calculator, ordinary, box, True), _unsorted_expected(ordinary, box, True, 4.0, True), what="gave up")
+    lines = _one_launch_lines(capfd.readouterr().err)
+    assert len(lines) == 1 and "gave up 1" in lines[0], lines

@@ -29,6 +29,7 @@
 #include "fused.cuh"
 #include "geometry.hpp"
 #include "ordered.cuh"
+#include "small.cuh"
 #include "policy.hpp"
 #include "scan.cuh"
 #include "search.cuh"
@@ -932,6 +933,38 @@ bool compute(
         extras.in_order_rest -= 1;
         try_in_order = false;
     }
+    // Small systems with arrays from earlier calls: everything in one launch (small.cuh), as one work item per point
+    // for a sorted list, as one per point and slice of its candidates otherwise (about four units of 64 candidates
+    // per item, as many items as the smallest shape of that launch takes).
+    const bool small_allowed = extras.capacity > 0 && n_points <= SMALL_POINTS && n_cells <= SMALL_POINTS &&
+                               !separate_launches() && !ordered_rows() && std::getenv("VESIN_HIP_CELLS") == nullptr;
+    bool one_launch = false;
+    uint32_t small_slices = 1;
+    if (small_allowed && options.sorted) {
+        one_launch = try_in_order;
+    } else if (small_allowed && try_single_pass && full_stencil - full_stencil / 2 <= MAX_ENTRIES &&
+               n_points <= SmallShape<4>::MAX_ITEMS && n_cells <= SmallShape<4>::CAPACITY) {
+        const double per_cell = std::max(1.0, static_cast<double>(n_points) / static_cast<double>(n_cells));
+        const double units = std::ceil(upper_stencil_cells(g) * per_cell / WAVE);
+        const double most = std::floor(static_cast<double>(SmallShape<4>::MAX_ITEMS) / static_cast<double>(n_points));
+        small_slices = static_cast<uint32_t>(std::max(1.0, std::min(most, std::ceil(units / 4.0))));
+        one_launch = true;
+    }
+    if (one_launch && extras.one_launch_rest > 0) {
+        extras.one_launch_rest -= 1;
+        one_launch = false;
+    }
+    if (one_launch && extras.meetings == nullptr) {
+        if (extras.fixed_memory) {
+            one_launch = false; // no allocation there
+        } else {
+            HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&extras.meetings), 2 * sizeof(SmallMeeting)));
+            extras.own_meetings = true;
+            HIP_CHECK(hipMemset(extras.meetings, 0, 2 * sizeof(SmallMeeting)));
+        }
+    }
+    const size_t small_items = one_launch ? n_points * small_slices : 0;
+    uint32_t* rows_of_item = nullptr;
     OrderedStatus* ordered_status = nullptr;
     uint32_t* rows_of_point = nullptr;
     uint64_t* first_row_of_point = nullptr;
@@ -977,6 +1010,7 @@ bool compute(
         counts = carver.take<uint32_t>(std::max(n_slots, direct_slots * n_slices));
         offsets = carver.take<uint64_t>(std::max(n_slots, direct_slots * n_slices) + 1);
         scan_scratch = carver.take<uint64_t>(scratch_elements);
+        rows_of_item = carver.take<uint32_t>(small_items);
         if (try_in_order) {
             rows_of_point = carver.take<uint32_t>(n_points);
             first_row_of_point = carver.take<uint64_t>(n_points + 1);
@@ -1004,26 +1038,10 @@ bool compute(
         }
     };
 
-    // ---- small systems with arrays from earlier calls, sorted lists: cell list, counting, scan, report to the host
-    // and writing in one launch (ordered_small_kernel). Its workgroups wait for each other, which needs all of them
-    // resident at once; when they were not, or the system does not suit the in-order search, or the rows do not
-    // fit, the call goes on as if nothing had happened, and the list leaves that launch alone for a while.
-    bool one_launch = try_in_order && extras.capacity > 0 && n_points <= ORDERED_SMALL_POINTS &&
-                      n_cells <= ORDERED_SMALL_POINTS && !separate_launches() && !ordered_rows() &&
-                      std::getenv("VESIN_HIP_CELLS") == nullptr;
-    if (one_launch && extras.one_launch_rest > 0) {
-        extras.one_launch_rest -= 1;
-        one_launch = false;
-    }
-    if (one_launch && extras.meetings == nullptr) {
-        if (extras.fixed_memory) {
-            one_launch = false; // no allocation there
-        } else {
-            HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&extras.meetings), 2 * sizeof(SmallMeeting)));
-            extras.own_meetings = true;
-            HIP_CHECK(hipMemset(extras.meetings, 0, 2 * sizeof(SmallMeeting)));
-        }
-    }
+    // ---- small systems with arrays from earlier calls: cell list, counting, scan, report to the host and writing
+    // in one launch (small_system_kernel). Its workgroups wait for each other, which needs all of them resident at
+    // once; when they were not, or the system does not suit that launch, or the rows do not fit, the call goes on
+    // as if nothing had happened, and (except in the last case) the list leaves that launch alone for a while.
     if (one_launch) {
         size_outputs(neighbors, extras, 0, options);
         SmallArgs sargs = {};
@@ -1031,26 +1049,30 @@ bool compute(
         sargs.box = fetched ? nullptr : reinterpret_cast<const double*>(box);
         sargs.periodic = periodic;
         sargs.host_small = extras.mail_device->small;
-        sargs.rows_of_point = rows_of_point;
+        sargs.rows_of_item = rows_of_item;
+        sargs.n_slices = small_slices;
         sargs.meeting = extras.meetings + (extras.meeting_turn & 1u);
         sargs.next_meeting = extras.meetings + ((extras.meeting_turn + 1u) & 1u);
         extras.meeting_turn += 1;
         sargs.host = &extras.mail_device->ordered;
-        sargs.spin_limit = std::min(chain_spin_limit(), ORDERED_SMALL_SPINS);
+        sargs.spin_limit = std::min(chain_spin_limit(), SMALL_SPINS);
         sargs.capacity = extras.capacity;
         sargs.out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
         sargs.out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
         sargs.out.distances = neighbors.distances;
         sargs.out.vectors = reinterpret_cast<double*>(neighbors.vectors);
-        // few waves per workgroup when that still covers the points: the arithmetic spreads over more compute units
-        if (n_points <= SmallShape<4>::MAX_POINTS && n_cells <= SmallShape<4>::CAPACITY) {
-            auto kernel = options.full ? ordered_small_kernel<true, 4> : ordered_small_kernel<false, 4>;
+        // few waves per workgroup when that still covers the items: the arithmetic spreads over more compute units
+        if (!options.sorted) {
+            auto kernel = options.full ? small_system_kernel<true, 4, false> : small_system_kernel<false, 4, false>;
+            hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>((small_items + 3) / 4)), dim3(4 * WAVE), 0, stream, sargs, g);
+        } else if (n_points <= SmallShape<4>::MAX_ITEMS && n_cells <= SmallShape<4>::CAPACITY) {
+            auto kernel = options.full ? small_system_kernel<true, 4, true> : small_system_kernel<false, 4, true>;
             hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>((n_points + 3) / 4)), dim3(4 * WAVE), 0, stream, sargs, g);
-        } else if (n_points <= SmallShape<8>::MAX_POINTS) {
-            auto kernel = options.full ? ordered_small_kernel<true, 8> : ordered_small_kernel<false, 8>;
+        } else if (n_points <= SmallShape<8>::MAX_ITEMS) {
+            auto kernel = options.full ? small_system_kernel<true, 8, true> : small_system_kernel<false, 8, true>;
             hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>((n_points + 7) / 8)), dim3(8 * WAVE), 0, stream, sargs, g);
         } else {
-            auto kernel = options.full ? ordered_small_kernel<true, 16> : ordered_small_kernel<false, 16>;
+            auto kernel = options.full ? small_system_kernel<true, 16, true> : small_system_kernel<false, 16, true>;
             hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>((n_points + 15) / 16)), dim3(16 * WAVE), 0, stream, sargs, g);
         }
         fetched = true;
@@ -1068,8 +1090,9 @@ bool compute(
                               found.found.max_candidates <= ORDERED_CANDIDATES && found.found.unsuitable == 0;
         if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
             std::fprintf(
-                stderr, "one launch: rows %llu, most rows of a point %u, most candidates of a point %u, unsuitable %u, gave up %u\n",
-                found.total_rows, found.found.max_rows, found.found.max_candidates, found.found.unsuitable, found.found.gave_up
+                stderr, "one launch: rows %llu, %u items per point, most rows of a point %u, most candidates of an item %u, unsuitable %u, gave up %u\n",
+                found.total_rows, small_slices, found.found.max_rows, found.found.max_candidates, found.found.unsuitable,
+                found.found.gave_up
             );
         }
         if (suitable && found.total_rows <= extras.capacity) {

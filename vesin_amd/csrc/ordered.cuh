@@ -26,7 +26,6 @@
 #ifndef VESIN_HIP_ORDERED_CUH
 #define VESIN_HIP_ORDERED_CUH
 
-#include "cells.cuh"
 #include "fused.cuh"
 #include "search.cuh"
 
@@ -60,11 +59,6 @@ struct OrderedHostStatus {
     unsigned int padding;
 };
 
-/// One-launch search of small systems: points (and cells) it takes, polls of a workgroup that waits for the
-/// others, the mark a workgroup that stops waiting leaves in the count of arrivals.
-constexpr uint32_t ORDERED_SMALL_POINTS = 2048;
-constexpr uint32_t ORDERED_SMALL_SPINS = 1u << 14;
-constexpr uint32_t ORDERED_GAVE_UP = 1u << 31;
 
 struct OrderedArgs {
     SortedPoints sorted;
@@ -522,472 +516,6 @@ __global__ __launch_bounds__(ORDERED_BLOCK) void ordered_search_kernel(OrderedAr
             sh.tile_x[p], sh.tile_y[p], sh.tile_z[p], sh.tile_index[p], sh.tile_row[p], lane
         );
     }
-}
-
-// ---------------------------------------------------------------------------------------------------------------
-// Small systems: everything in one launch
-
-/// Shapes of the launch: WAVES waves per workgroup, one point each. Every workgroup holds all points, so one fits
-/// a compute unit and the grid must not have more workgroups than there are compute units; few waves per workgroup
-/// spread the arithmetic over more compute units, many allow more points.
-template <int WAVES>
-struct SmallShape {
-    static constexpr int BLOCK_THREADS = WAVES * WAVE;
-    static constexpr uint32_t PER_THREAD = WAVES == 16 ? 2 : 4;          // points (and cells) a thread places
-    static constexpr uint32_t CAPACITY = PER_THREAD * BLOCK_THREADS;      // points and cells the LDS arrays hold
-    static constexpr uint32_t MAX_POINTS = WAVES == 16 ? CAPACITY : 240u * WAVES; // at most 240 workgroups
-};
-static_assert(SmallShape<16>::CAPACITY == ORDERED_SMALL_POINTS, "the largest shape takes every small system");
-
-/// What the workgroups of one launch of ordered_small_kernel tell each other. A list keeps two of them and
-/// alternates: a launch works on one and leaves the other cleared for the next launch.
-struct SmallMeeting {
-    unsigned int arrived;        // workgroups that are done counting (and ORDERED_GAVE_UP)
-    unsigned int max_rows;       // as in OrderedStatus
-    unsigned int max_candidates;
-    unsigned int unsuitable;
-};
-
-/// What ordered_small_kernel takes besides the grid.
-struct SmallArgs {
-    const double* points;
-    const double* box;           // null when the host has them already
-    const bool* periodic;
-    unsigned char* host_small;   // where the host reads box and periodic (see fetch_box)
-    uint32_t* rows_of_point;     // [n_points] work memory
-    SmallMeeting* meeting;       // zero on entry
-    SmallMeeting* next_meeting;  // cleared here
-    OrderedHostStatus* host;
-    uint32_t spin_limit;
-    uint64_t capacity;
-    SearchOutputs out;
-};
-
-/// LDS of one wave of ordered_small_kernel.
-struct SmallWaveShared: SearchTables {
-    __attribute__((aligned(16))) uint64_t keys[ORDERED_MAX_ROWS + 4];
-    uint32_t key_at[ORDERED_MAX_ROWS];
-};
-
-/// LDS of a workgroup: its own cell-sorted copy of all points, and the waves' tables.
-template <int WAVES>
-struct SmallShared {
-    static constexpr uint32_t CAPACITY = SmallShape<WAVES>::CAPACITY;
-    double x[CAPACITY], y[CAPACITY], z[CAPACITY];
-    uint32_t index[CAPACITY];
-    uint32_t wraps[CAPACITY];          // biased_shift of the wrap, every component clamped to +-511
-    uint32_t cell_start[CAPACITY + 1]; // points per cell, then their exclusive scan
-    uint32_t first_row[CAPACITY + 1];  // after the meeting: exclusive scan of the rows of the points
-    SmallWaveShared wave[WAVES];
-    uint64_t wave_sums[WAVES];
-    // the points of this workgroup's waves, as the thread that placed them saw them
-    double own_x[WAVES], own_y[WAVES], own_z[WAVES];
-    uint32_t own_cell[WAVES];
-    int32_t own_wx[WAVES], own_wy[WAVES], own_wz[WAVES];
-    uint32_t first_bad;
-    uint32_t all_arrived;
-};
-
-__device__ __forceinline__ double uniform(double v) {
-    return __longlong_as_double(static_cast<long long>(uniform(static_cast<uint64_t>(__double_as_longlong(v)))));
-}
-
-/// Exclusive scan of one value per thread over the threads of a workgroup of WAVES waves; `total` for everybody.
-template <int WAVES>
-__device__ __forceinline__ uint64_t small_block_scan(uint64_t value, uint64_t& total, uint64_t* wave_sums) {
-    const int lane = lane_id();
-    const int wave = threadIdx.x / WAVE;
-    const uint64_t inclusive = wave_inclusive_scan(value);
-    if (lane == WAVE - 1) {
-        wave_sums[wave] = inclusive;
-    }
-    __syncthreads();
-    uint64_t before = 0;
-    uint64_t all = 0;
-#pragma unroll
-    for (int w = 0; w < WAVES; w++) {
-        const uint64_t sum = wave_sums[w];
-        before += w < wave ? sum : 0;
-        all += sum;
-    }
-    __syncthreads();
-    total = all;
-    return before + inclusive - value;
-}
-
-/// locate_candidate for four candidates at once: the four searches advance together, one LDS round trip per step
-/// for all of them instead of one per step and candidate.
-__device__ __forceinline__ void locate_four_candidates(
-    const SearchTables& sh, uint32_t n_batch, const uint32_t (&k)[4], uint32_t (&at)[4], int32_t (&packed)[4]
-) {
-    static_assert(MAX_ENTRIES <= 64, "six steps cover the table");
-    uint32_t lo[4] = {0, 0, 0, 0};
-#pragma unroll
-    for (uint32_t step = 32; step > 0; step >>= 1) {
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            // largest e < n_batch with ent_prefix[e] <= k; the table has MAX_ENTRIES + 1 words, what lies beyond
-            // n_batch is read and ignored
-            const uint32_t probe = lo[r] + step;
-            const uint32_t before = sh.ent_prefix[min(probe, static_cast<uint32_t>(MAX_ENTRIES))];
-            const uint32_t take = (probe < n_batch ? 1u : 0u) & (before <= k[r] ? 1u : 0u); // no branch: the read is not skipped
-            lo[r] = take != 0 ? probe : lo[r];
-        }
-    }
-#pragma unroll
-    for (int r = 0; r < 4; r++) {
-        at[r] = sh.ent_start[lo[r]] + (k[r] - sh.ent_prefix[lo[r]]);
-        packed[r] = sh.ent_shift[lo[r]];
-    }
-}
-
-/// Sorted list of a small system (at most SmallShape<WAVES>::MAX_POINTS points, ...::CAPACITY cells) in ONE launch, cell list
-/// included: at this size every pass takes a few microseconds, most of them spent waiting for one memory access
-/// after the other, and the launches of cell build, counting pass, scan, report and writing pass with the gaps
-/// between them take several times what the passes do.
-///
-/// * Every workgroup sorts ALL points into cells for itself, in LDS (same steps as build_cells_small:
-///   histogram with the slot coming back from the atomic, scan, placement; the order inside a cell differs from
-///   workgroup to workgroup, which no result depends on). From then on candidates are read from LDS.
-/// * One wave per point, in original order: the wave takes the candidates of the point's stencil into registers,
-///   four units of 64 at a time, tests them (the decisions of ordered_sweep_pair: arithmetic of the file header; a
-///   point is no neighbour of itself, a half list keeps the smaller index first and a point's own image under the
-///   reference's rule) and keeps per candidate a hit bit, its place in LDS, original index and shift. It stores the
-///   number of rows of its point in `rows_of_point`.
-/// * All workgroups meet: they count themselves in `meeting->arrived` and wait until all have. The grid (at most
-///   240 workgroups, one per compute unit) is resident at once on a GPU that runs nothing else, and the wait is
-///   bounded (`spin_limit` polls) for the case that it is not: the first workgroup that stops waiting marks the
-///   word, then no workgroup writes, workgroup 0 reports `gave_up` and the host goes on with separate launches.
-/// * After the wait every workgroup scans the rows of all points for itself (no second meeting), workgroup 0
-///   reports to the host what publish_ordered_status reports, and if the system suits this search (see the file
-///   header) and the rows fit `capacity`, every wave ranks and writes the rows of its point.
-///
-/// What crosses from one workgroup to another is `rows_of_point` and the maxima of the meeting, all written and
-/// read with device-scope atomics (no cache-wide write-back or invalidation: those cost more than the passes).
-template <bool FULL, int WAVES>
-__global__ __launch_bounds__(WAVES * WAVE) void ordered_small_kernel(SmallArgs args, GridParams g) {
-    constexpr uint32_t SMALL_BLOCK = SmallShape<WAVES>::BLOCK_THREADS;
-    constexpr uint32_t SMALL_PER_THREAD = SmallShape<WAVES>::PER_THREAD;
-    constexpr uint32_t CAPACITY = SmallShape<WAVES>::CAPACITY;
-    constexpr uint32_t SMALL_WAVES = WAVES;
-    __shared__ SmallShared<WAVES> shared;
-    static_assert(sizeof(SmallShared<WAVES>) <= 160 * 1024, "one workgroup per compute unit");
-    static_assert(ORDERED_UNITS % 4 == 0, "units are taken four at a time");
-    const uint32_t t = threadIdx.x;
-    const int lane = lane_id();
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(t / WAVE);
-    SmallWaveShared& sh = shared.wave[wave];
-    const uint32_t n = g.n_points;
-
-    // ---- the cell list, in LDS
-    if (blockIdx.x == 0 && args.box != nullptr) {
-        if (t < 9) {
-            reinterpret_cast<double*>(args.host_small)[t] = args.box[t];
-        } else if (t < 12) {
-            args.host_small[72 + (t - 9)] = args.periodic[t - 9] ? 1 : 0;
-        }
-    }
-    if (t == 0) {
-        shared.first_bad = 0xFFFFFFFFu;
-    }
-#pragma unroll
-    for (uint32_t k = 0; k < SMALL_PER_THREAD; k++) {
-        shared.cell_start[k * SMALL_BLOCK + t] = 0;
-    }
-    __syncthreads();
-    double px[SMALL_PER_THREAD], py[SMALL_PER_THREAD], pz[SMALL_PER_THREAD];
-    uint32_t cell_of[SMALL_PER_THREAD], slot_of[SMALL_PER_THREAD];
-    int32_t pwx[SMALL_PER_THREAD], pwy[SMALL_PER_THREAD], pwz[SMALL_PER_THREAD];
-#pragma unroll
-    for (uint32_t k = 0; k < SMALL_PER_THREAD; k++) {
-        const uint32_t i = k * SMALL_BLOCK + t;
-        cell_of[k] = 0;
-        slot_of[k] = 0;
-        pwx[k] = pwy[k] = pwz[k] = 0;
-        px[k] = py[k] = pz[k] = 0.0;
-        if (i < n) {
-            px[k] = args.points[3 * static_cast<size_t>(i) + 0];
-            py[k] = args.points[3 * static_cast<size_t>(i) + 1];
-            pz[k] = args.points[3 * static_cast<size_t>(i) + 2];
-            int32_t where[3] = {0, 0, 0};
-            int32_t wrap[3] = {0, 0, 0};
-            unsigned int axis;
-            if (all_finite(px[k], py[k], pz[k], axis)) {
-                locate(g, px[k], py[k], pz[k], where, wrap);
-            } else {
-                atomicMin(&shared.first_bad, 3u * i + axis);
-            }
-            cell_of[k] = (static_cast<uint32_t>(where[2]) * g.n[1] + where[1]) * g.n[0] + where[0];
-            pwx[k] = wrap[0];
-            pwy[k] = wrap[1];
-            pwz[k] = wrap[2];
-            slot_of[k] = atomicAdd(&shared.cell_start[cell_of[k]], 1u);
-            if (i / SMALL_WAVES == blockIdx.x) {
-                const uint32_t w = i % SMALL_WAVES;
-                shared.own_x[w] = px[k];
-                shared.own_y[w] = py[k];
-                shared.own_z[w] = pz[k];
-                shared.own_cell[w] = cell_of[k];
-                shared.own_wx[w] = pwx[k];
-                shared.own_wy[w] = pwy[k];
-                shared.own_wz[w] = pwz[k];
-            }
-        }
-    }
-    __syncthreads();
-    {
-        uint32_t counts[SMALL_PER_THREAD];
-        uint64_t own_total = 0;
-#pragma unroll
-        for (uint32_t k = 0; k < SMALL_PER_THREAD; k++) {
-            const uint32_t c = t * SMALL_PER_THREAD + k;
-            counts[k] = c < g.n_cells ? shared.cell_start[c] : 0u;
-            own_total += counts[k];
-        }
-        uint64_t total_points = 0;
-        uint32_t running = static_cast<uint32_t>(small_block_scan<WAVES>(own_total, total_points, shared.wave_sums));
-#pragma unroll
-        for (uint32_t k = 0; k < SMALL_PER_THREAD; k++) {
-            shared.cell_start[t * SMALL_PER_THREAD + k] = running;
-            running += counts[k];
-        }
-        if (t == SMALL_BLOCK - 1) {
-            shared.cell_start[CAPACITY] = running;
-        }
-    }
-    __syncthreads();
-#pragma unroll
-    for (uint32_t k = 0; k < SMALL_PER_THREAD; k++) {
-        const uint32_t i = k * SMALL_BLOCK + t;
-        if (i < n) {
-            const uint32_t to = shared.cell_start[cell_of[k]] + slot_of[k];
-            shared.x[to] = px[k];
-            shared.y[to] = py[k];
-            shared.z[to] = pz[k];
-            shared.index[to] = i;
-            shared.wraps[to] = biased_shift(max(-511, min(511, pwx[k])), max(-511, min(511, pwy[k])), max(-511, min(511, pwz[k])));
-        }
-    }
-    __syncthreads();
-
-    // ---- the candidates of this wave's point, its rows
-    const uint32_t oi = blockIdx.x * SMALL_WAVES + wave;
-    uint32_t columns[ORDERED_UNITS];
-    uint32_t cand_at[ORDERED_UNITS];
-    uint32_t cand_index[ORDERED_UNITS];
-    uint32_t cand_biased[ORDERED_UNITS];
-#pragma unroll
-    for (int u = 0; u < ORDERED_UNITS; u++) {
-        columns[u] = 0;
-        cand_at[u] = 0;
-        cand_index[u] = 0;
-        cand_biased[u] = 0;
-    }
-    uint32_t n_units = 0;
-    uint32_t rows = 0;
-    double xi = 0.0, yi = 0.0, zi = 0.0;
-    int32_t wix = 0, wiy = 0, wiz = 0;
-    const int32_t span_y = 2 * g.s[1] + 1;
-    const int32_t span_z = 2 * g.s[2] + 1;
-    const uint32_t n_stencil = static_cast<uint32_t>(2 * g.s[0] + 1) * span_y * span_z;
-    if (oi < n && n_stencil <= MAX_ENTRIES) {
-        xi = uniform(shared.own_x[wave]);
-        yi = uniform(shared.own_y[wave]);
-        zi = uniform(shared.own_z[wave]);
-        wix = static_cast<int32_t>(uniform(static_cast<uint32_t>(shared.own_wx[wave])));
-        wiy = static_cast<int32_t>(uniform(static_cast<uint32_t>(shared.own_wy[wave])));
-        wiz = static_cast<int32_t>(uniform(static_cast<uint32_t>(shared.own_wz[wave])));
-        const uint32_t cell = uniform(shared.own_cell[wave]);
-        const int32_t cx = cell % g.n[0];
-        const int32_t cy = (cell / g.n[0]) % g.n[1];
-        const int32_t cz = cell / (g.n[0] * g.n[1]);
-        fill_stencil_tables(sh, lane, 0, n_stencil, cx, cy, cz, span_y, span_z, g, shared.cell_start);
-        const uint32_t n_candidates = __builtin_amdgcn_readfirstlane(sh.n_candidates);
-        if (lane == 0 && n_candidates > __hip_atomic_load(&args.meeting->max_candidates, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
-            atomicMax(&args.meeting->max_candidates, n_candidates);
-        }
-        if (n_candidates <= ORDERED_CANDIDATES) {
-            n_units = (n_candidates + WAVE - 1) / WAVE;
-            bool out_of_range = beyond(wix, wiy, wiz, ORDERED_SHIFT_LIMIT);
-#pragma unroll
-            for (int chunk = 0; chunk < ORDERED_UNITS / 4; chunk++) {
-                if (static_cast<uint32_t>(4 * chunk) < n_units) {
-                    uint32_t k[4], at[4];
-                    int32_t packed_q[4];
-                    bool valid[4];
-#pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        k[r] = static_cast<uint32_t>(4 * chunk + r) * WAVE + lane;
-                        valid[r] = k[r] < n_candidates;
-                        k[r] = valid[r] ? k[r] : 0u; // candidate 0 exists: every read below has an address
-                    }
-                    locate_four_candidates(sh, n_stencil, k, at, packed_q);
-                    double xj[4], yj[4], zj[4];
-                    uint32_t oj[4], wj[4];
-#pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        xj[r] = shared.x[at[r]];
-                        yj[r] = shared.y[at[r]];
-                        zj[r] = shared.z[at[r]];
-                        oj[r] = shared.index[at[r]];
-                        wj[r] = shared.wraps[at[r]];
-                    }
-#pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        const int u = 4 * chunk + r;
-                        int32_t qx, qy, qz;
-                        unpack_shift(packed_q[r], qx, qy, qz);
-                        const int32_t bx = qx - (static_cast<int32_t>((wj[r] >> 20) & 0x3ffu) - 512);
-                        const int32_t by = qy - (static_cast<int32_t>((wj[r] >> 10) & 0x3ffu) - 512);
-                        const int32_t bz = qz - (static_cast<int32_t>(wj[r] & 0x3ffu) - 512);
-                        out_of_range = out_of_range || (valid[r] && beyond(bx, by, bz, ORDERED_SHIFT_LIMIT));
-                        const int32_t sx = bx + wix;
-                        const int32_t sy = by + wiy;
-                        const int32_t sz = bz + wiz;
-                        double tx, ty, tz;
-                        shift_vector(g, sx, sy, sz, tx, ty, tz);
-                        const double vx = (xj[r] - xi) + tx;
-                        const double vy = (yj[r] - yi) + ty;
-                        const double vz = (zj[r] - zi) + tz;
-                        const double d2 = vx * vx + vy * vy + vz * vz;
-                        const bool shifted = (sx | sy | sz) != 0;
-                        bool keep;
-                        if (oj[r] == oi) {
-                            // the point and one of its own images
-                            keep = shifted && (FULL || half_keeps_self_image(sx, sy, sz));
-                        } else {
-                            keep = FULL || oi < oj[r];
-                        }
-                        const bool hit = valid[r] && keep && d2 < g.cutoff2;
-                        rows += __popcll(__ballot(hit));
-                        columns[u] = hit ? 1u : 0u;
-                        cand_at[u] = at[r];
-                        cand_index[u] = oj[r];
-                        // a clamped wrap gives a wrong shift here: such a system is reported unsuitable
-                        cand_biased[u] = biased_shift(max(-511, min(511, bx)), max(-511, min(511, by)), max(-511, min(511, bz)));
-                    }
-                }
-            }
-            if (lane == 0 && rows > __hip_atomic_load(&args.meeting->max_rows, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
-                atomicMax(&args.meeting->max_rows, rows);
-            }
-            if (__ballot(out_of_range) != 0 && lane == 0) {
-                atomicAdd(&args.meeting->unsuitable, 1u);
-            }
-        }
-    }
-    if (oi < n && lane == 0) {
-        // read by other workgroups of this launch: straight to where the whole device sees it
-        __hip_atomic_store(&args.rows_of_point[oi], rows, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-
-    // ---- all workgroups meet. Once a wave's device-scope stores have completed they are what any device-scope
-    // load returns, so the workgroup's arrival only has to come after.
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (t == 0) {
-        // One word decides for everybody: the count of the workgroups that are done, and a mark that the first
-        // workgroup to lose patience sets with a compare-and-swap on a count that is not yet complete. A workgroup
-        // goes on iff it reads the complete count without the mark, which cannot be set any more after that.
-        if (args.spin_limit == 0) {
-            // no patience at all (how the tests reach the host's way back): marked before anybody can be the last
-            __hip_atomic_fetch_or(&args.meeting->arrived, ORDERED_GAVE_UP, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        __hip_atomic_fetch_add(&args.meeting->arrived, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        uint32_t spins = 0;
-        bool all = false;
-        while (true) {
-            uint32_t seen = __hip_atomic_load(&args.meeting->arrived, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if ((seen & ORDERED_GAVE_UP) != 0) {
-                break;
-            }
-            if (seen == gridDim.x) {
-                all = true;
-                break;
-            }
-            spins += 1;
-            if (spins > args.spin_limit) {
-                if (__hip_atomic_compare_exchange_strong(
-                        &args.meeting->arrived, &seen, seen | ORDERED_GAVE_UP, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
-                        __HIP_MEMORY_SCOPE_AGENT
-                    )) {
-                    break;
-                }
-                continue; // somebody arrived or gave up in between: look again
-            }
-            __builtin_amdgcn_s_sleep(4);
-        }
-        shared.all_arrived = all ? 1u : 0u;
-        if (blockIdx.x == 0) {
-            // nobody looks at the other meeting during this launch: the next launch finds it cleared
-            __hip_atomic_store(&args.next_meeting->arrived, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(&args.next_meeting->max_rows, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(&args.next_meeting->max_candidates, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(&args.next_meeting->unsuitable, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-    }
-    __syncthreads();
-    if (shared.all_arrived == 0) {
-        if (blockIdx.x == 0 && t == 0) {
-            args.host->found.gave_up = 1;
-            args.host->first_bad_coordinate = shared.first_bad;
-        }
-        return;
-    }
-
-    // ---- the first row of every point: every workgroup scans the rows of all points
-    {
-        uint32_t items[SMALL_PER_THREAD];
-        uint64_t local = 0;
-#pragma unroll
-        for (uint32_t k = 0; k < SMALL_PER_THREAD; k++) {
-            const uint32_t i = t * SMALL_PER_THREAD + k;
-            items[k] = i < n ? __hip_atomic_load(&args.rows_of_point[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
-            local += items[k];
-        }
-        uint64_t total = 0;
-        uint32_t running = static_cast<uint32_t>(small_block_scan<WAVES>(local, total, shared.wave_sums));
-#pragma unroll
-        for (uint32_t k = 0; k < SMALL_PER_THREAD; k++) {
-            shared.first_row[t * SMALL_PER_THREAD + k] = running;
-            running += items[k];
-        }
-        if (t == SMALL_BLOCK - 1) {
-            shared.first_row[CAPACITY] = running;
-        }
-    }
-    __syncthreads();
-    const uint64_t total = shared.first_row[CAPACITY];
-    OrderedStatus found;
-    found.max_rows = __hip_atomic_load(&args.meeting->max_rows, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    found.max_candidates = __hip_atomic_load(&args.meeting->max_candidates, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    found.unsuitable = __hip_atomic_load(&args.meeting->unsuitable, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    found.windowed = 0;
-    found.bucketed = 0;
-    found.arrived = gridDim.x;
-    found.gave_up = 0;
-    found.padding = 0;
-    const bool suitable = found.max_rows <= ORDERED_MAX_ROWS && found.max_candidates <= ORDERED_CANDIDATES &&
-                          found.unsuitable == 0 && shared.first_bad == 0xFFFFFFFFu;
-    if (blockIdx.x == 0 && t == 0) {
-        args.host->found = found;
-        args.host->total_rows = total;
-        args.host->first_bad_coordinate = shared.first_bad;
-    }
-    if (!suitable || total > args.capacity || rows == 0) {
-        return;
-    }
-
-    // ---- the rows of the point
-    SortedPoints in_lds = {};
-    in_lds.x = shared.x;
-    in_lds.y = shared.y;
-    in_lds.z = shared.z;
-    const uint32_t wrap_i = (static_cast<uint32_t>(wix) << 20) + (static_cast<uint32_t>(wiy) << 10) + static_cast<uint32_t>(wiz);
-    write_rows_of_point<false>(
-        sh, in_lds, g, args.out, columns, cand_at, cand_index, cand_biased, n_units, 0u, wrap_i, xi, yi, zi, oi,
-        static_cast<uint64_t>(shared.first_row[oi]), lane
-    );
 }
 
 // ---------------------------------------------------------------------------------------------------------------
