@@ -181,7 +181,8 @@ class NeighborList:
             periodic = [bool(periodic)] * 3
 
         if is_torch:
-            box = torch.as_tensor(box)
+            if not isinstance(box, torch.Tensor):
+                box = torch.as_tensor(box)
             initial_dtype = points.dtype
             if box.dtype != initial_dtype:
                 raise RuntimeError(
@@ -218,35 +219,47 @@ class NeighborList:
         if isinstance(periodic, torch.Tensor):
             periodic = periodic.to(dtype=torch.bool, device=device).contiguous()
         else:
-            # the three flags rarely change between calls: keep their device copy
-            flags = np.asarray(periodic).astype(np.bool_)
-            key = (flags.tobytes(), flags.shape, str(device))
+            # the three flags rarely change between calls: keep their device copy (a list or tuple of three plain
+            # booleans, the usual argument, is recognised without going through numpy)
+            plain = type(periodic) in (list, tuple) and len(periodic) == 3 and all(type(f) is bool for f in periodic)
+            key = (tuple(periodic), device) if plain else None
             cached = getattr(self, "_periodic_on_device", None)
-            if cached is None or cached[0] != key:
-                cached = (key, torch.as_tensor(flags).to(device=device))
-                self._periodic_on_device = cached
+            if key is None or cached is None or cached[0] != key:
+                flags = np.asarray(periodic).astype(np.bool_)
+                key = (tuple(bool(f) for f in flags), device) if flags.shape == (3,) else (flags.tobytes(), flags.shape, device)
+                if cached is None or cached[0] != key:
+                    cached = (key, torch.as_tensor(flags).to(device=device))
+                    self._periodic_on_device = cached
             periodic = cached[1]
         if tuple(periodic.shape) != (3,):
             raise ValueError(
                 f"`periodic` must be a single boolean or a sequence of three booleans, got {periodic}"
             )
 
-        points = points.to(device=device, dtype=torch.float64).contiguous()
-        box = box.to(device=device, dtype=torch.float64).contiguous()
-
-        options = VesinOptions()
-        options.cutoff = self.cutoff
-        options.full = self.full_list
-        options.sorted = self.sorted
-        options.algorithm = self._c_algorithm
-        options.n_threads = self.n_threads
-        options.return_shifts = "S" in quantities
-        options.return_distances = "d" in quantities
-        options.return_vectors = "D" in quantities
-        options.skin = self.skin
+        if points.dtype != torch.float64 or points.device != device or not points.is_contiguous():
+            points = points.to(device=device, dtype=torch.float64).contiguous()
+        if box.dtype != torch.float64 or box.device != device or not box.is_contiguous():
+            box = box.to(device=device, dtype=torch.float64).contiguous()
 
         index = device.index if device.index is not None else torch.cuda.current_device()
-        c_device = VesinDevice(VesinCUDA, index)
+
+        # options and device of the call: the same objects while nothing they are made of changes
+        settings = (self.cutoff, self.full_list, self.sorted, self._c_algorithm, self.n_threads, self.skin, quantities, index)
+        kept = self.__dict__.get("_call_settings")
+        if kept is None or kept[0] != settings:
+            options = VesinOptions()
+            options.cutoff = self.cutoff
+            options.full = self.full_list
+            options.sorted = self.sorted
+            options.algorithm = self._c_algorithm
+            options.n_threads = self.n_threads
+            options.return_shifts = "S" in quantities
+            options.return_distances = "d" in quantities
+            options.return_vectors = "D" in quantities
+            options.skin = self.skin
+            kept = (settings, options, VesinDevice(VesinCUDA, index))
+            self._call_settings = kept
+        options, c_device = kept[1], kept[2]
 
         if self._neighbors.device.type != VesinUnknownDevice and (
             self._neighbors.device.type != c_device.type or self._neighbors.device.device_id != c_device.device_id
@@ -255,8 +268,11 @@ class NeighborList:
             self._lib.vesin_free(ctypes.byref(self._neighbors))
             ctypes.memset(ctypes.byref(self._neighbors), 0, ctypes.sizeof(self._neighbors))
 
-        # inputs may still be in flight on torch's current stream
-        torch.cuda.current_stream(device).synchronize()
+        # inputs may still be in flight on torch's current stream. The library works on the null stream, which waits
+        # for everything earlier on torch's default stream by itself; only a stream of the caller's own does not
+        stream = torch.cuda.current_stream(device)
+        if stream.cuda_stream != 0:
+            stream.synchronize()
 
         # an empty tensor has no storage; the ABI still wants a device pointer
         points_ptr = points.data_ptr() if points.shape[0] > 0 else box.data_ptr()
@@ -276,6 +292,17 @@ class NeighborList:
             raise RuntimeError(error_message.value.decode("utf8"))
 
         n_pairs = self._neighbors.length
+        if not copy:
+            # views of arrays that did not move, asked for in the same way: the tuple of the call before
+            result_key = (
+                quantities, n_pairs, self._neighbors.pairs, self._neighbors.shifts, self._neighbors.distances,
+                self._neighbors.vectors, float_dtype, index,
+                # (distances and vectors in another precision are converted copies, made again on every call)
+                namespace is None and is_torch and float_dtype == torch.float64,
+            )
+            last = self.__dict__.get("_last_views")
+            if last is not None and last[0] == result_key and result_key[-1]:
+                return last[1]
         device_str = f"cuda:{index}"
 
         views = self.__dict__.setdefault("_views", {})
@@ -318,7 +345,10 @@ class NeighborList:
                 data.append(to_result(distances))
             elif quantity == "D":
                 data.append(to_result(vectors))
-        return tuple(data)
+        data = tuple(data)
+        if not copy and n_pairs != 0:
+            self._last_views = (result_key, data)
+        return data
 
     def compute_batch(self, points, first_point, boxes, periodic=True, quantities: str = "ij", copy: bool = True):
         """Neighbor lists of many systems in one go (``vesin_hip_neighbors_batch``).
