@@ -329,3 +329,40 @@ def test_what_the_unsorted_launch_leaves_to_the_other_paths(capfd, monkeypatch):
     assert_same_list(_compute(calculator, ordinary, box, True), _unsorted_expected(ordinary, box, True, 4.0, True), what="gave up")
     lines = _one_launch_lines(capfd.readouterr().err)
     assert len(lines) == 1 and "gave up 1" in lines[0], lines
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# directions that are not periodic: the extent of the points is remembered from call to call
+
+
+@pytest.mark.parametrize("is_sorted", [True, False], ids=["sorted", "unsorted"])
+@pytest.mark.parametrize("periodic", [(False, False, False), (True, False, True)], ids=["free", "slab"])
+def test_a_cluster_that_moves_grows_and_jumps(periodic, is_sorted, capfd, monkeypatch):
+    """The same number of points on every call, so that every call after the second starts from the box and the
+    extent the call before left: points that drift, a cluster that doubles its size, one that is suddenly somewhere
+    else entirely (every point outside of the remembered extent), one that collapses. The rows are the oracle's
+    every time."""
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    rng = np.random.default_rng(41)
+    box = np.array([[14.0, 0.0, 0.0], [2.0, 13.0, 0.0], [0.0, -1.0, 15.0]])
+    points = rng.random((180, 3)) * 12.0
+    calculator = NeighborList(cutoff=3.5, full_list=True, sorted=is_sorted)
+    used = 0
+    for step in range(24):
+        if step in (6, 7):
+            points = points * 1.4  # grows
+        elif step == 12:
+            points = points + np.array([500.0, -300.0, 120.0])  # jumps
+        elif step == 16:
+            points = (points - points.mean(axis=0)) * 0.3 + points.mean(axis=0)  # collapses
+        else:
+            points = points + rng.normal(scale=0.15, size=points.shape)
+        expected = oracle.neighbors(points, box, list(periodic), 3.5, True, False, "ijSdD")
+        capfd.readouterr()
+        result = _compute(calculator, points, box, list(periodic))
+        used += len(_one_launch_lines(capfd.readouterr().err))
+        if is_sorted:
+            _same(result, oracle.canonicalize(expected), f"step {step}")
+        else:
+            assert_same_list(result, expected, what=f"step {step}")
+    assert used >= 18

@@ -339,6 +339,15 @@ struct HipExtras {
     int direct_rest = 0;              // calls left before the one-pass cell build is tried again after a cell overflowed
     int in_order_rest = 0;            // calls left before the in-order search is tried again on a system it did not cover
     int one_launch_rest = 0;          // calls left before a small system is tried in one launch again
+    /// Extent of the points along the directions that are not periodic, as the last call found it: a small system
+    /// that went through the one launch reports it on the way, and the next call of the same kind (see BoxGuess) on
+    /// the same box picks its grid from it without a pass over the points and a round trip to the host first. A
+    /// point outside of the remembered extent ends up in the outermost cell of its direction, which is as wide as
+    /// the cutoff at least and has no neighbours beyond: the rows are the same, a stale extent only costs time
+    /// (crowded cells), and with at most 2048 points never much.
+    bool extent_valid = false;
+    double extent_lo[3] = {0, 0, 0};
+    double extent_hi[3] = {0, 0, 0};
     SmallMeeting* meetings = nullptr; // device, two of them (see SmallMeeting); allocated at the first small system
     bool own_meetings = false;        // allocated by this state (not part of memory that was handed to it)
     uint32_t meeting_turn = 0;
@@ -810,7 +819,17 @@ bool compute(
     const bool any_open = !(hbox.periodic[0] && hbox.periodic[1] && hbox.periodic[2]);
     double lo[3] = {0, 0, 0};
     double hi[3] = {0, 0, 0};
-    if (any_open) {
+    // (valid for one call: whatever happens below, only a call that reports a fresh extent makes it valid again)
+    const bool remembered_extent = any_open && speculate && extras.extent_valid && n_points <= SMALL_POINTS &&
+                                   extras.one_launch_rest == 0;
+    extras.extent_valid = false;
+    if (remembered_extent) {
+        for (int d = 0; d < 3; d++) {
+            lo[d] = extras.extent_lo[d];
+            hi[d] = extras.extent_hi[d];
+        }
+    }
+    if (any_open && !remembered_extent) {
         if (!fetched) {
             launch_fetch(); // the synchronisation below is where a remembered box is checked first
             fetched = true;
@@ -1042,6 +1061,10 @@ bool compute(
     // in one launch (small_system_kernel). Its workgroups wait for each other, which needs all of them resident at
     // once; when they were not, or the system does not suit that launch, or the rows do not fit, the call goes on
     // as if nothing had happened, and (except in the last case) the list leaves that launch alone for a while.
+    if (remembered_extent && !one_launch) {
+        // the grid came from an extent that only the one launch refreshes: start over with a pass over the points
+        return false;
+    }
     if (one_launch) {
         size_outputs(neighbors, extras, 0, options);
         SmallArgs sargs = {};
@@ -1055,6 +1078,7 @@ bool compute(
         sargs.next_meeting = extras.meetings + ((extras.meeting_turn + 1u) & 1u);
         extras.meeting_turn += 1;
         sargs.host = &extras.mail_device->ordered;
+        sargs.host_bounds = any_open ? extras.mail_device->bounds : nullptr;
         sargs.spin_limit = std::min(chain_spin_limit(), SMALL_SPINS);
         sargs.capacity = extras.capacity;
         sargs.out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
@@ -1099,6 +1123,14 @@ bool compute(
             check_pair_limit(found.total_rows);
             HIP_CHECK(hipGetLastError());
             neighbors.length = found.total_rows;
+            if (any_open) {
+                const BlockBounds& fresh = extras.mail->bounds[0];
+                for (int d = 0; d < 3; d++) {
+                    extras.extent_lo[d] = fresh.lo[d];
+                    extras.extent_hi[d] = fresh.hi[d];
+                }
+                extras.extent_valid = true;
+            }
             if (timed) {
                 float ms = 0.0f;
                 HIP_CHECK(hipEventElapsedTime(&ms, extras.events[T_START], extras.events[T_WRITE]));

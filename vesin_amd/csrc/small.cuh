@@ -77,6 +77,7 @@ struct SmallArgs {
     SmallMeeting* meeting;       // zero on entry
     SmallMeeting* next_meeting;  // cleared here
     OrderedHostStatus* host;
+    BlockBounds* host_bounds;    // not null: workgroup 0 reports the extent of the points there (see bounding_kernel)
     uint32_t spin_limit;         // 0: no workgroup waits at all (tests)
     uint64_t capacity;
     SearchOutputs out;
@@ -105,6 +106,7 @@ struct SmallShared {
     int32_t own_wx[WAVES], own_wy[WAVES], own_wz[WAVES];
     uint32_t first_bad;
     uint32_t all_arrived;
+    BlockBounds extent[WAVES];   // workgroup 0: the waves' shares of the extent of the points
 };
 
 __device__ __forceinline__ double uniform(double v) {
@@ -274,6 +276,9 @@ __global__ __launch_bounds__(WAVES * WAVE) void small_system_kernel(SmallArgs ar
     double px[PER_THREAD], py[PER_THREAD], pz[PER_THREAD];
     uint32_t cell_of[PER_THREAD], slot_of[PER_THREAD];
     int32_t pwx[PER_THREAD], pwy[PER_THREAD], pwz[PER_THREAD];
+    const bool report_extent = args.host_bounds != nullptr && blockIdx.x == 0;
+    double extent_lo[3] = {INFINITY, INFINITY, INFINITY};
+    double extent_hi[3] = {-INFINITY, -INFINITY, -INFINITY};
 #pragma unroll
     for (uint32_t k = 0; k < PER_THREAD; k++) {
         const uint32_t i = k * BLOCK_THREADS + t;
@@ -290,6 +295,15 @@ __global__ __launch_bounds__(WAVES * WAVE) void small_system_kernel(SmallArgs ar
             unsigned int axis;
             if (all_finite(px[k], py[k], pz[k], axis)) {
                 locate(g, px[k], py[k], pz[k], where, wrap);
+                if (report_extent) {
+                    double f[3];
+                    fractional(g, px[k], py[k], pz[k], f);
+#pragma unroll
+                    for (int d = 0; d < 3; d++) {
+                        extent_lo[d] = fmin(extent_lo[d], f[d]);
+                        extent_hi[d] = fmax(extent_hi[d], f[d]);
+                    }
+                }
             } else {
                 atomicMin(&shared.first_bad, 3u * i + axis);
             }
@@ -313,7 +327,38 @@ __global__ __launch_bounds__(WAVES * WAVE) void small_system_kernel(SmallArgs ar
             }
         }
     }
+    if (report_extent) {
+        // the extent of the points, for the grid of the next call on this list (a list remembers it like its box)
+#pragma unroll
+        for (int offset = WAVE / 2; offset > 0; offset >>= 1) {
+#pragma unroll
+            for (int d = 0; d < 3; d++) {
+                extent_lo[d] = fmin(extent_lo[d], __shfl_xor(extent_lo[d], offset));
+                extent_hi[d] = fmax(extent_hi[d], __shfl_xor(extent_hi[d], offset));
+            }
+        }
+        if (lane == 0) {
+#pragma unroll
+            for (int d = 0; d < 3; d++) {
+                shared.extent[wave].lo[d] = extent_lo[d];
+                shared.extent[wave].hi[d] = extent_hi[d];
+            }
+        }
+    }
     __syncthreads();
+    if (report_extent && t == 0) {
+        BlockBounds all = shared.extent[0];
+        for (int w = 1; w < WAVES; w++) {
+#pragma unroll
+            for (int d = 0; d < 3; d++) {
+                all.lo[d] = fmin(all.lo[d], shared.extent[w].lo[d]);
+                all.hi[d] = fmax(all.hi[d], shared.extent[w].hi[d]);
+            }
+        }
+        all.first_bad_coordinate = 0xFFFFFFFFu; // reported with the rest, below
+        all.padding = 0;
+        args.host_bounds[0] = all;
+    }
     {
         uint32_t counts[PER_THREAD];
         uint64_t own_total = 0;
