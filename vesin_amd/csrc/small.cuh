@@ -40,7 +40,7 @@
 namespace vesin_hip {
 
 constexpr uint32_t SMALL_POINTS = 2048;        // points (and cells, and work items) the largest shape takes
-constexpr uint32_t SMALL_SPINS = 1u << 14;     // polls of a workgroup that waits for the others
+constexpr uint32_t SMALL_SPINS = 1u << 12;     // polls of a workgroup that waits for the others (a few milliseconds)
 constexpr uint32_t SMALL_GAVE_UP = 1u << 31;   // in SmallMeeting::arrived: a workgroup stopped waiting
 constexpr uint32_t SMALL_WORKGROUPS = 240;     // of a launch: fewer than there are compute units
 
