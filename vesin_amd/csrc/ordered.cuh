@@ -118,27 +118,36 @@ __device__ __forceinline__ uint4 load_four_indices(const uint32_t* index) {
 ///     neighbour of itself, and a half list keeps a point with its own image under the rule of the reference only;
 ///   - a half list keeps the orientation whose first index is the smaller one (!FULL);
 ///   - lane p of `rows` adds up the hits of the item's point p (a scalar population count per test).
-template <int R, bool SHIFTED, bool FULL>
+template <int R, bool SHIFTED, bool FULL, typename Shared>
 __device__ __forceinline__ void sweep_and_count(
-    const SortedPoints& sorted, uint32_t first, uint32_t count, const SweepCandidates<R>& c, double cutoff2,
+    const Shared& sh, uint32_t first, uint32_t count, const SweepCandidates<R>& c, double cutoff2,
     const uint32_t (&original)[R], int lane, uint32_t (&column)[R], uint32_t& rows
 ) {
+    // The item's points come from the wave's LDS (every lane reads the same words: broadcasts), four at a time:
+    // the compiler keeps the reads of the next points in flight while the tests of these run, which the scalar
+    // loads of the other sweeps, each waited for where it is issued, do not allow.
     for (uint32_t i0 = 0; i0 < count; i0 += POINTS_PER_LOAD) {
-        const uint32_t at = first + i0;
-        const FourPoints p = load_four_points(sorted.x + at, sorted.y + at, sorted.z + at);
-        uint4 indices = uint4{0u, 0u, 0u, 0u};
-        if (!FULL) {
-            indices = load_four_indices(sorted.index + at);
+        double px[POINTS_PER_LOAD], py[POINTS_PER_LOAD], pz[POINTS_PER_LOAD];
+        uint32_t pi[POINTS_PER_LOAD];
+#pragma unroll
+        for (int u = 0; u < POINTS_PER_LOAD; u++) {
+            // (the arrays hold TILE_POINTS entries; what lies beyond `count` is read and not used)
+            const uint32_t p = min(i0 + u, static_cast<uint32_t>(TILE_POINTS - 1));
+            px[u] = sh.tile_x[p];
+            py[u] = sh.tile_y[p];
+            pz[u] = sh.tile_z[p];
+            pi[u] = FULL ? 0u : sh.tile_index[p];
         }
 #pragma unroll
         for (int u = 0; u < POINTS_PER_LOAD; u++) {
             if (u > 0 && i0 + u >= count) {
                 break;
             }
-            const double xi = words_to_double(p.x[2 * u], p.x[2 * u + 1]);
-            const double yi = words_to_double(p.y[2 * u], p.y[2 * u + 1]);
-            const double zi = words_to_double(p.z[2 * u], p.z[2 * u + 1]);
-            const uint32_t index_i = u == 0 ? indices.x : u == 1 ? indices.y : u == 2 ? indices.z : indices.w;
+            const double xi = px[u];
+            const double yi = py[u];
+            const double zi = pz[u];
+            const uint32_t index_i = pi[u];
+            const uint32_t at = first + i0 + u;
             uint32_t found = 0;
 #pragma unroll
             for (int r = 0; r < R; r++) {
@@ -151,7 +160,7 @@ __device__ __forceinline__ void sweep_and_count(
                     vz += c.tz[r];
                 }
                 const double d2 = vx * vx + vy * vy + vz * vz;
-                uint64_t mask = __ballot(d2 < cutoff2) & __ballot(c.position[r] != at + u);
+                uint64_t mask = __ballot(d2 < cutoff2) & __ballot(c.position[r] != at);
                 if (!FULL) {
                     mask &= __ballot(index_i <= original[r]);
                 }
@@ -222,9 +231,9 @@ __device__ __forceinline__ void ordered_sweep_pair(
 
     if (!WRAPPED) {
         if (any_shift) {
-            sweep_and_count<R, true, FULL>(sorted, first_i, n_i, c, g.cutoff2, original, lane, column, rows);
+            sweep_and_count<R, true, FULL>(sh, first_i, n_i, c, g.cutoff2, original, lane, column, rows);
         } else {
-            sweep_and_count<R, false, FULL>(sorted, first_i, n_i, c, g.cutoff2, original, lane, column, rows);
+            sweep_and_count<R, false, FULL>(sh, first_i, n_i, c, g.cutoff2, original, lane, column, rows);
         }
         return;
     }
@@ -405,10 +414,10 @@ __global__ __launch_bounds__(ORDERED_BLOCK) void ordered_search_kernel(OrderedAr
         const int32_t wy = sorted.wy[at];
         const int32_t wz = sorted.wz[at];
         out_of_range = beyond(wx, wy, wz, ORDERED_SHIFT_LIMIT);
+        sh.tile_x[lane] = sorted.x[at];
+        sh.tile_y[lane] = sorted.y[at];
+        sh.tile_z[lane] = sorted.z[at];
         if (WRITE) {
-            sh.tile_x[lane] = sorted.x[at];
-            sh.tile_y[lane] = sorted.y[at];
-            sh.tile_z[lane] = sorted.z[at];
             sh.tile_wx[lane] = wx;
             sh.tile_wy[lane] = wy;
             sh.tile_wz[lane] = wz;

@@ -269,16 +269,17 @@ __device__ __forceinline__ void fill_stencil_tables(
 __device__ __forceinline__ void locate_candidate(
     const SearchTables& sh, uint32_t n_batch, uint32_t k, uint32_t& at, int32_t& packed
 ) {
-    // largest e with ent_prefix[e] <= k
+    // largest e < n_batch with ent_prefix[e] <= k: six steps without a branch, so that lookups that do not depend
+    // on each other (the units a wave takes together) advance side by side instead of one loop after the other.
+    // The table has MAX_ENTRIES + 1 words; what lies beyond n_batch is read and ignored.
+    static_assert(MAX_ENTRIES <= 64, "six steps cover the table");
     uint32_t lo = 0;
-    uint32_t hi = n_batch;
-    while (hi - lo > 1) {
-        uint32_t mid = (lo + hi) >> 1;
-        if (sh.ent_prefix[mid] <= k) {
-            lo = mid;
-        } else {
-            hi = mid;
-        }
+#pragma unroll
+    for (uint32_t step = 32; step > 0; step >>= 1) {
+        const uint32_t probe = lo + step;
+        const uint32_t before = sh.ent_prefix[min(probe, static_cast<uint32_t>(MAX_ENTRIES))];
+        const uint32_t take = (probe < n_batch ? 1u : 0u) & (before <= k ? 1u : 0u);
+        lo = take != 0 ? probe : lo;
     }
     at = sh.ent_start[lo] + (k - sh.ent_prefix[lo]);
     packed = sh.ent_shift[lo];
