@@ -175,6 +175,35 @@ def test_unrequested_arrays_are_left_alone_and_shapes_vary():
         assert int(arrays.shifts[0, 0]) == 77 and float(arrays.vectors[0, 0]) == -1.0
 
 
+@pytest.mark.parametrize("sorted", [False, True], ids=["unsorted", "sorted"])
+def test_small_systems_take_one_launch_here_too(sorted, capfd, monkeypatch):
+    """Systems of at most 2048 points go through the one launch that builds the cells, searches and writes (its two
+    meeting words live in the library's work array); several in a row through the same array, each against the
+    allocating entry point and the oracle."""
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    lib = get_library()
+    arrays = CallerArrays(400_000)
+    rng = np.random.default_rng(19)
+    systems = [configs.diamond(3, seed=1), configs.diamond(4, seed=2), configs.diamond(3, seed=3)]
+    systems.append((rng.uniform(0.0, 9.0, (150, 3)), np.zeros((3, 3)), (False, False, False)))
+    used = 0
+    for points, box, periodic in systems:
+        periodic = [bool(p) for p in np.broadcast_to(np.asarray(periodic), (3,))]
+        options = _options(4.5, True, sorted)
+        d_points, d_box, d_periodic = _device(points, box, periodic)
+        expected = _allocating(lib, d_points, d_box, d_periodic, options)
+        arrays.reset()
+        capfd.readouterr()
+        n = _no_alloc(lib, d_points, d_box, d_periodic, options, arrays)
+        used += sum(line.startswith("one launch:") and "gave up 0" in line for line in capfd.readouterr().err.splitlines())
+        assert n == len(expected["pairs"])
+        _same_rows(arrays.rows(n, options), expected, in_place=sorted)
+        reference = oracle.neighbors(points, box, periodic, 4.5, True, False, "ijSdD")
+        _same_rows(arrays.rows(n, options), oracle.canonicalize(reference) if sorted else reference, in_place=sorted)
+        assert int(arrays.pairs[n, 0]) == -1
+    assert used == len(systems)
+
+
 def test_on_a_stream_of_the_caller():
     import torch
 

@@ -351,6 +351,7 @@ struct HipExtras {
     SmallMeeting* meetings = nullptr; // device, two of them (see SmallMeeting); allocated at the first small system
     bool own_meetings = false;        // allocated by this state (not part of memory that was handed to it)
     uint32_t meeting_turn = 0;
+    int compute_units = 0;            // of the device (asked once)
     hipEvent_t events[T_STAGES] = {};
     bool have_events = false;
     // a second stream of the list's own, for a kernel that can run beside another of the same call (forked from and
@@ -972,6 +973,23 @@ bool compute(
     if (one_launch && extras.one_launch_rest > 0) {
         extras.one_launch_rest -= 1;
         one_launch = false;
+    }
+    if (one_launch) {
+        // every workgroup of that launch must be resident at once: never more workgroups than the device has
+        // compute units (a workgroup of the largest shape fills the LDS of one)
+        if (extras.compute_units == 0) {
+            int units = 0;
+            HIP_CHECK(hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, extras.device_id));
+            extras.compute_units = units;
+        }
+        const size_t items = n_points * small_slices;
+        const size_t waves = !options.sorted                                                        ? 4
+                             : n_points <= SmallShape<4>::MAX_ITEMS && n_cells <= SmallShape<4>::CAPACITY ? 4
+                             : n_points <= SmallShape<8>::MAX_ITEMS                                       ? 8
+                                                                                                          : 16;
+        if ((items + waves - 1) / waves > static_cast<size_t>(extras.compute_units)) {
+            one_launch = false;
+        }
     }
     if (one_launch && extras.meetings == nullptr) {
         if (extras.fixed_memory) {
@@ -2309,6 +2327,11 @@ FixedState& fixed_state_of(int device_id) {
         extras.device_id = device_id;
         extras.fixed_memory = true;
         extras.d_status = reinterpret_cast<DeviceStatus*>(next);
+        // the two meetings of the one launch of small systems: zero like the whole array when the library is loaded,
+        // and left zero for the next launch by every launch that uses them
+        static_assert(sizeof(DeviceStatus) <= 128 && 128 + 2 * sizeof(SmallMeeting) <= FIXED_STATUS_BYTES, "status block");
+        extras.meetings = reinterpret_cast<SmallMeeting*>(next + 128);
+        extras.own_meetings = false;
         next += FIXED_STATUS_BYTES;
         extras.mail_device = reinterpret_cast<Mailbox*>(next);
         extras.mail = &state->host_mail;
@@ -2387,6 +2410,7 @@ void neighbors_no_alloc(
     extras.direct_rest = 0;
     extras.in_order_rest = 0;
     extras.one_launch_rest = 0;
+    extras.extent_valid = false;
     extras.timings_valid = false;
 
     VesinNeighborList list;
