@@ -219,6 +219,15 @@ __device__ __forceinline__ void locate(
     }
 }
 
+/// Points per tile of a cell of `count` points: the cell is cut into ceil(count / TILE_POINTS) tiles of equal size
+/// (the last one short by less than the number of tiles) instead of full tiles and a rest: a cell of 40 points is
+/// two tiles of 20, not 32 + 8, whose waves would sit at the same workgroup barriers with four times the work of
+/// one another.
+__device__ __forceinline__ uint32_t tile_size_of(uint32_t count) {
+    const uint32_t n_tiles = (count + TILE_POINTS - 1) >> TILE_SHIFT;
+    return n_tiles <= 1 ? static_cast<uint32_t>(TILE_POINTS) : (count + n_tiles - 1) / n_tiles;
+}
+
 /// One thread per point: cell id, wrap shift, and the histogram of points per cell. The value returned by the
 /// histogram atomic is kept as the point's provisional slot inside its cell. Lanes of a wave that fall in the same
 /// cell (the usual case for spatially coherent input) are grouped first, for up to ASSIGN_ROUNDS distinct cells
@@ -425,14 +434,15 @@ __global__ __launch_bounds__(BLOCK) void place_points(
     sorted.wx[to] = wx;
     sorted.wy[to] = wy;
     sorted.wz[to] = wz;
+    const uint32_t tile_size = tile_size_of(count);
     if ((wx | wy | wz) != 0) {
-        atomicOr(&tiles[first_tile + k / TILE_POINTS].wrapped, 1u);
+        atomicOr(&tiles[first_tile + k / tile_size].wrapped, 1u);
     }
-    if (k % TILE_POINTS == 0) {
-        Tile* tile = &tiles[first_tile + k / TILE_POINTS];
+    if (k % tile_size == 0) {
+        Tile* tile = &tiles[first_tile + k / tile_size];
         tile->cell = cell;
         tile->first = to;
-        tile->count = min(TILE_POINTS, count - k);
+        tile->count = min(tile_size, count - k);
         if (system != 0) {
             atomicOr(&tile->wrapped, system << 1);
         }
@@ -616,15 +626,16 @@ __global__ __launch_bounds__(BLOCK) void gather_points(
     sorted.wz[to] = wz;
     if ((wx | wy | wz) != 0) {
         // tiles holding a wrapped point take the search kernel's general path
-        atomicOr(&tiles[first_tile + rank / TILE_POINTS].wrapped, 1u);
+        atomicOr(&tiles[first_tile + rank / tile_size_of(count)].wrapped, 1u);
     }
 
     const uint32_t k = p - start;
-    if (k % TILE_POINTS == 0) {
-        Tile* tile = &tiles[first_tile + k / TILE_POINTS];
+    const uint32_t tile_size = tile_size_of(count);
+    if (k % tile_size == 0) {
+        Tile* tile = &tiles[first_tile + k / tile_size];
         tile->cell = cell;
         tile->first = start + k;
-        tile->count = min(TILE_POINTS, count - k);
+        tile->count = min(tile_size, count - k);
     }
 }
 
@@ -752,14 +763,15 @@ __global__ __launch_bounds__(SMALL_BUILD_THREADS) void build_cells_small(
             sorted.wx[to] = wx[k];
             sorted.wy[to] = wy[k];
             sorted.wz[to] = wz[k];
-            Tile* tile = &tiles[first_tile + slot_of[k] / TILE_POINTS];
+            const uint32_t tile_size = tile_size_of(count);
+            Tile* tile = &tiles[first_tile + slot_of[k] / tile_size];
             if ((wx[k] | wy[k] | wz[k]) != 0) {
                 atomicOr(&tile->wrapped, 1u);
             }
-            if (slot_of[k] % TILE_POINTS == 0) {
+            if (slot_of[k] % tile_size == 0) {
                 tile->cell = cell_of[k];
                 tile->first = to;
-                tile->count = min(TILE_POINTS, count - slot_of[k]);
+                tile->count = min(tile_size, count - slot_of[k]);
             }
         }
     }
