@@ -161,7 +161,7 @@ def _modes(err):
     return int(found[-1][0]), int(found[-1][1])
 
 
-def _check_order_once(points, box, periodic, cutoff, full, capfd, monkeypatch):
+def _check_order_once(points, box, periodic, cutoff, full, capfd, monkeypatch, report=_modes):
     expected = oracle.canonicalize(oracle.neighbors(points, box, periodic, cutoff, full, False, "ijSdD"))
     monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
     capfd.readouterr()
@@ -171,7 +171,7 @@ def _check_order_once(points, box, periodic, cutoff, full, capfd, monkeypatch):
     assert result["pairs"].shape == expected["pairs"].shape
     for key in result:
         assert np.array_equal(result[key], expected[key]), key
-    return _modes(err)
+    return report(err)
 
 
 @pytest.mark.parametrize("full", [True, False])
@@ -229,3 +229,55 @@ def test_slab_with_free_directions(capfd, monkeypatch):
     points, box = _lattice(40, 40, 6, seed=8)
     windowed, bucketed = _check_order_once(points, box, [True, True, False], 5.0, False, capfd, monkeypatch)
     assert windowed + bucketed > 2048
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# The points of a tile dealt to several waves of the writing pass
+
+
+def _waves_per_tile(err):
+    import re
+
+    found = re.findall(r"(\d+) tiles written by (\d+) waves each", err)
+    assert found, err
+    return int(found[-1][0]), int(found[-1][1])
+
+
+@pytest.mark.parametrize("waves", [2, 3, 4])
+@pytest.mark.parametrize("full", [True, False])
+def test_any_number_of_waves_per_tile_writes_the_same_rows(waves, full, capfd, monkeypatch):
+    monkeypatch.setenv("VESIN_HIP_WRITE_SPLIT", str(waves))
+    # candidates in the order found once per tile (more than 2048 tiles) ...
+    points, box = _lattice(20, 20, 20, seed=11)
+    tiles, each = _check_order_once(points, box, [True] * 3, 5.0, full, capfd, monkeypatch, report=_waves_per_tile)
+    assert tiles > 2048 and each == waves
+    # ... ranked per point (few tiles), with tiles of fewer points than waves, outside points and a free direction
+    rng = np.random.default_rng(waves)
+    box = np.diag([11.0, 12.0, 13.0])
+    points = rng.uniform(-6.0, 18.0, size=(900, 3))
+    _check(points, box, (True, False, True), 3.0, full, capfd, monkeypatch, "used")
+
+
+def test_well_filled_tiles_that_barely_exceed_the_resident_waves_get_four_waves_each(capfd, monkeypatch):
+    """110,592 atoms in 4,913 cells: the list's first call learns the number of tiles, the calls after it deal
+    every tile's points to four waves; both give the oracle's list."""
+    import torch
+
+    points, box = _lattice(24, 24, 24, seed=12)
+    expected = oracle.canonicalize(oracle.neighbors(points, box, [True] * 3, 5.0, False, False, "ijSdD"))
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    calculator = NeighborList(cutoff=5.0, full_list=False, sorted=True)
+    device_points = torch.tensor(points, device="cuda:0")
+    device_box = torch.tensor(box, device="cuda:0")
+    waves = []
+    for _ in range(3):
+        capfd.readouterr()
+        P, S, d, D = calculator.compute(device_points, device_box, True, "PSdD")
+        tiles, each = _waves_per_tile(capfd.readouterr().err)
+        assert 4096 < tiles < 6144
+        waves.append(each)
+        assert np.array_equal(P.cpu().numpy(), expected["pairs"])
+        assert np.array_equal(S.cpu().numpy(), expected["shifts"])
+        assert np.array_equal(d.cpu().numpy(), expected["distances"])
+        assert np.array_equal(D.cpu().numpy(), expected["vectors"])
+    assert waves == [1, 4, 4]

@@ -138,12 +138,14 @@ static bool ordered_one_stream() {
 namespace {
 
 __global__ void publish_ordered_status(
-    const OrderedStatus* found, const uint64_t* total, const DeviceStatus* status, OrderedHostStatus* host
+    const OrderedStatus* found, const uint64_t* total, const DeviceStatus* status, const uint64_t* cell_scan_end,
+    OrderedHostStatus* host
 ) {
     if (threadIdx.x == 0 && blockIdx.x == 0) {
         host->found = *found;
         host->total_rows = *total;
         host->first_bad_coordinate = status->first_bad_coordinate;
+        host->n_tiles = static_cast<unsigned int>(*cell_scan_end >> 32);
     }
 }
 
@@ -339,6 +341,8 @@ struct HipExtras {
     int direct_rest = 0;              // calls left before the one-pass cell build is tried again after a cell overflowed
     int in_order_rest = 0;            // calls left before the in-order search is tried again on a system it did not cover
     int one_launch_rest = 0;          // calls left before a small system is tried in one launch again
+    uint32_t ordered_tiles = 0;       // tiles of the last call through the in-order search, and its number of points:
+    size_t ordered_tiles_points = 0;  // how the next one deals its writing pass to the waves (see write_split)
     /// Extent of the points along the directions that are not periodic, as the last call found it: a small system
     /// that went through the one launch reports it on the way, and the next call of the same kind (see BoxGuess) on
     /// the same box picks its grid from it without a pass over the points and a round trip to the host first. A
@@ -1005,7 +1009,7 @@ bool compute(
     OrderedStatus* ordered_status = nullptr;
     uint32_t* rows_of_point = nullptr;
     uint64_t* first_row_of_point = nullptr;
-    uint32_t* hit_columns = nullptr;
+    CandidateRecord* candidate_records = nullptr;
     uint16_t* candidate_order = nullptr;
     // small systems: the points of a tile are dealt to several waves, about 2048 in all
     uint32_t ordered_points_per_item = TILE_POINTS;
@@ -1051,7 +1055,7 @@ bool compute(
         if (try_in_order) {
             rows_of_point = carver.take<uint32_t>(n_points);
             first_row_of_point = carver.take<uint64_t>(n_points + 1);
-            hit_columns = carver.take<uint32_t>(static_cast<size_t>(ordered_blocks) * ORDERED_WAVES * ORDERED_UNITS * WAVE);
+            candidate_records = carver.take<CandidateRecord>(static_cast<size_t>(ordered_blocks) * ORDERED_WAVES * ORDERED_UNITS * WAVE);
             if (ordered_items_per_tile == 1) {
                 candidate_order = carver.take<uint16_t>(tiles_bound * ORDERED_CANDIDATES);
             }
@@ -1376,7 +1380,31 @@ bool compute(
         oargs.points_per_item = ordered_points_per_item;
         oargs.items_per_tile = ordered_items_per_tile;
         oargs.rows_of_point = rows_of_point;
-        oargs.columns = hit_columns;
+        oargs.records = candidate_records;
+        // The writing pass runs four waves per SIMD: 4096 at a time on this GPU. A system of a few more tiles than that
+        // leaves the stragglers running alone for as long as everything before them took (the 100,000-atom
+        // benchmark: 4,260 tiles, 188 us where a wave lives 110 us). The points of every tile can be dealt to two or
+        // four waves instead, which brings the work in shorter pieces; the waves of a tile read the same records
+        // and tables, a fixed cost worth about eight points' rows per wave, so it only pays for well-filled tiles
+        // and up to about three times as many tiles as the GPU holds waves (measured on half lists at 24 points
+        // per tile: 4,500 tiles 357 -> 316 us per call with four waves per tile, 9,000 tiles 567 -> 541 us with
+        // two, 19,000 tiles 911 -> 924 us). Decided from the number of tiles the call before had on the same number
+        // of points; a list's first call on a system keeps one wave per tile.
+        oargs.write_split = 1;
+        if (ordered_items_per_tile == 1 && extras.ordered_tiles_points == n_points && extras.ordered_tiles > 0) {
+            const double slots = 4096.0;
+            const double tiles = static_cast<double>(extras.ordered_tiles);
+            const double per_tile = static_cast<double>(n_points) / tiles;
+            if (per_tile >= 16.0 && tiles > 0.85 * slots && tiles <= 1.5 * slots) {
+                oargs.write_split = 4;
+            } else if (per_tile >= 16.0 && tiles > 1.5 * slots && tiles <= 3.0 * slots) {
+                oargs.write_split = 2;
+            }
+        }
+        if (const char* text = std::getenv("VESIN_HIP_WRITE_SPLIT")) {
+            oargs.write_split = static_cast<uint32_t>(std::max(1, std::min(4, std::atoi(text))));
+        }
+        oargs.points = reinterpret_cast<const double*>(points);
         oargs.order = candidate_order;
         oargs.first_row = first_row_of_point;
         oargs.status = ordered_status;
@@ -1398,7 +1426,7 @@ bool compute(
         auto launch_write = [&]() {
             auto kernel = presorted ? (options.full ? ordered_search_kernel<true, true, true> : ordered_search_kernel<true, false, true>)
                                     : (options.full ? ordered_search_kernel<true, true, false> : ordered_search_kernel<true, false, false>);
-            hipLaunchKernelGGL(kernel, dim3(blocks), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
+            hipLaunchKernelGGL(kernel, dim3(blocks * oargs.write_split), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
         };
         // A list that has arrays from earlier calls writes into them without waiting for the host to learn what the
         // counting pass found: the launch checks on the device that the system suits this search and that the rows
@@ -1443,7 +1471,8 @@ bool compute(
             }
             hipLaunchKernelGGL(
                 publish_ordered_status, dim3(1), dim3(1), 0, stream,
-                ordered_status, first_row_of_point + n_points, extras.d_status, &extras.mail_device->ordered
+                ordered_status, first_row_of_point + n_points, extras.d_status, cell_scan + n_cells,
+                &extras.mail_device->ordered
             );
             extras.wait(stream);
             if (!box_was_right()) {
@@ -1454,15 +1483,18 @@ bool compute(
         if (found.first_bad_coordinate != 0xFFFFFFFFu) {
             non_finite_error(points, found.first_bad_coordinate);
         }
+        extras.ordered_tiles = found.n_tiles;
+        extras.ordered_tiles_points = n_points;
         const bool suitable = found.found.max_rows <= ORDERED_MAX_ROWS &&
                               found.found.max_candidates <= ORDERED_CANDIDATES && found.found.unsuitable == 0;
         if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
             std::fprintf(
                 stderr,
                 "in-order search: rows %llu, most rows of a point %u, most candidates of a tile %u, unsuitable %u, "
-                "candidates of %u tiles ordered by window and of %u by buckets: %s\n",
+                "candidates of %u tiles ordered by window and of %u by buckets, %u tiles written by %u waves each: %s\n",
                 found.total_rows, found.found.max_rows, found.found.max_candidates, found.found.unsuitable,
-                found.found.windowed, found.found.bucketed, suitable ? "used" : "left to the radix sort"
+                found.found.windowed, found.found.bucketed, found.n_tiles, oargs.write_split,
+                suitable ? "used" : "left to the radix sort"
             );
         }
         if (suitable) {

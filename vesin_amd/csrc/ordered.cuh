@@ -39,6 +39,14 @@ constexpr uint32_t ORDERED_CANDIDATES = ORDERED_UNITS * WAVE;
 constexpr uint32_t ORDERED_MAX_ROWS = 256;              // rows of one point that are ranked in one go
 constexpr int32_t ORDERED_SHIFT_LIMIT = 255;            // per operand: sums stay inside the key's 10-bit fields
 
+/// What the counting pass leaves to the writing pass per candidate of a work item: hit column against the item's
+/// points, original index, biased shift less the wrap of the first point.
+struct CandidateRecord {
+    uint32_t column;
+    uint32_t index;
+    uint32_t biased;
+};
+
 /// What the counting pass found, for the host to decide between this path and the radix sort.
 struct OrderedStatus {
     unsigned int max_rows;       // largest number of rows of one point
@@ -56,7 +64,7 @@ struct OrderedHostStatus {
     OrderedStatus found;
     unsigned long long total_rows;
     unsigned int first_bad_coordinate;
-    unsigned int padding;
+    unsigned int n_tiles; // of the cell list the passes worked on
 };
 
 
@@ -67,10 +75,13 @@ struct OrderedArgs {
     uint32_t points_per_item;   // a tile's points are dealt to ceil(TILE_POINTS / points_per_item) waves
     uint32_t items_per_tile;
     uint32_t* rows_of_point;    // COUNT: [n_points], by original index
-    uint32_t* columns;          // COUNT -> WRITE: hit columns, [work item][ORDERED_UNITS][64], candidates in table order
+    CandidateRecord* records;   // COUNT -> WRITE: [work item][ORDERED_UNITS][64], candidates in table order: hit column,
+                                // original index, biased shift (see CandidateRecord)
+    const double* points;       // WRITE: the caller's points, by original index
     uint16_t* order;            // SORT -> WRITE: [tile][ORDERED_CANDIDATES], candidate number at each place of the order
     const uint64_t* first_row;  // WRITE: [n_points + 1], exclusive scan of rows_of_point
     OrderedStatus* status;
+    uint32_t write_split;       // WRITE: waves that share the points of one work item of the counting pass (at least 1)
     uint32_t report_order;      // SORT: count the tiles ordered either way (an atomic per tile on one word: for tests)
     uint32_t guarded;           // WRITE launched before the host has seen what COUNT found: write nothing unless the
                                 // system suits this search and the rows fit the `capacity` of the arrays
@@ -180,12 +191,11 @@ template <bool FULL, bool WRAPPED>
 __device__ __forceinline__ void ordered_sweep_pair(
     const OrderedWaveShared& sh, const SortedPoints& sorted, const GridParams& g, uint32_t unit0, uint32_t n_stencil,
     uint32_t n_candidates, uint32_t first_i, uint32_t n_i, int lane, uint32_t (&column)[ORDERED_R], uint32_t& rows,
-    bool& out_of_range
+    bool& out_of_range, uint32_t (&at)[ORDERED_R], uint32_t (&original)[ORDERED_R], uint32_t (&biased)[ORDERED_R]
 ) {
     constexpr int R = ORDERED_R;
     SweepCandidates<R> c;
     int32_t packed_q[R];
-    uint32_t at[R], original[R];
     bool any_shift = false;
 #pragma unroll
     for (int r = 0; r < R; r++) {
@@ -199,6 +209,7 @@ __device__ __forceinline__ void ordered_sweep_pair(
         column[r] = 0;
         at[r] = 0xFFFFFFFFu;
         original[r] = 0;
+        biased[r] = 0;
         packed_q[r] = 0;
         int32_t bx = 0, by = 0, bz = 0;
         if (k < n_candidates) {
@@ -213,6 +224,9 @@ __device__ __forceinline__ void ordered_sweep_pair(
             by = qy - sorted.wy[at[r]];
             bz = qz - sorted.wz[at[r]];
             c.shift[r] = pack_shift(bx, by, bz);
+            // what the writing pass keeps of the candidate (a shift outside of the fields makes the system unsuitable:
+            // nothing is written then)
+            biased[r] = biased_shift(bx, by, bz);
             out_of_range = out_of_range || beyond(bx, by, bz, ORDERED_SHIFT_LIMIT);
             if (!WRAPPED) {
                 // a point is no neighbour of itself (of its images it is: the unshifted entry of the tile's own
@@ -277,14 +291,38 @@ __device__ __forceinline__ void ordered_sweep_pair(
     }
 }
 
+/// Where write_rows_of_point reads the coordinates of a second point: the caller's array of points by original
+/// index (x, y, z next to each other: one or two cache lines per point where the cell-sorted arrays take three), or
+/// three arrays by a position of the caller's choice.
+struct PointsByIndex {
+    const double* points;
+    __device__ __forceinline__ void load(uint32_t where, double& x, double& y, double& z) const {
+        x = points[3 * static_cast<size_t>(where) + 0];
+        y = points[3 * static_cast<size_t>(where) + 1];
+        z = points[3 * static_cast<size_t>(where) + 2];
+    }
+};
+
+struct PointsByPlace {
+    const double* x;
+    const double* y;
+    const double* z;
+    __device__ __forceinline__ void load(uint32_t where, double& px, double& py, double& pz) const {
+        px = x[where];
+        py = y[where];
+        pz = z[where];
+    }
+};
+
 /// The rows of one first point, from what the lanes hold per place of the order of the candidates (registers,
-/// indexed by unit): hit columns (the point's bit is `bit`), positions, original indices and biased shifts without
+/// indexed by unit): hit columns (the point's bit is `bit`), where `coordinates` finds the candidate (`cand_where`;
+/// the same array as `cand_index` when that is by original index), original indices and biased shifts without
 /// the wrap of the first point (`wrap_i`: the three wraps in the fields of the key, added in one integer addition).
 /// The hits are collected in lane order into `sh.keys` / `sh.key_at`, ranked where that is not their final order
 /// (!PRESORTED), and stored from row `first_row` on.
-template <bool PRESORTED, typename Shared>
+template <bool PRESORTED, typename Shared, typename Coordinates>
 __device__ __forceinline__ void write_rows_of_point(
-    Shared& sh, const SortedPoints& sorted, const GridParams& g, const SearchOutputs& out,
+    Shared& sh, const Coordinates& coordinates, const GridParams& g, const SearchOutputs& out,
     const uint32_t (&columns)[ORDERED_UNITS], const uint32_t (&cand_at)[ORDERED_UNITS],
     const uint32_t (&cand_index)[ORDERED_UNITS], const uint32_t (&cand_biased)[ORDERED_UNITS], uint32_t n_units,
     uint32_t bit, uint32_t wrap_i, double xi, double yi, double zi, uint32_t oi, uint64_t first_row, int lane
@@ -317,9 +355,8 @@ __device__ __forceinline__ void write_rows_of_point(
         const uint64_t key = active ? sh.keys[e] : ~0ull;
         // the position in the cell-sorted arrays is known before the rank is: the loads overlap the ranking
         const uint32_t at = active ? sh.key_at[e] : 0;
-        const double xj = sorted.x[at];
-        const double yj = sorted.y[at];
-        const double zj = sorted.z[at];
+        double xj, yj, zj;
+        coordinates.load(at, xj, yj, zj);
         uint32_t rank = e;
         if (!PRESORTED) {
             rank = 0;
@@ -364,7 +401,7 @@ __device__ __forceinline__ void write_rows_of_point(
 /// of a point in lane order are its rows in final order. Otherwise (small systems, where one more launch costs more
 /// than it saves) candidates come in table order and the rows of every point are ranked by comparing all its keys.
 template <bool WRITE, bool FULL, bool PRESORTED = false>
-__global__ __launch_bounds__(ORDERED_BLOCK) void ordered_search_kernel(OrderedArgs args, GridParams g) {
+__global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void ordered_search_kernel(OrderedArgs args, GridParams g) {
     constexpr int R = ORDERED_R;
     __shared__ OrderedShared shared;
     const int lane = lane_id();
@@ -379,7 +416,11 @@ __global__ __launch_bounds__(ORDERED_BLOCK) void ordered_search_kernel(OrderedAr
         }
     }
     const uint32_t n_tiles = static_cast<uint32_t>(args.cell_scan[g.n_cells] >> 32);
-    const uint32_t work = blockIdx.x * ORDERED_WAVES + wave;
+    // WRITE may deal the points of a work item of the counting pass to several waves (`write_split`): they read the
+    // same records and each writes the rows of its share of the points
+    const uint32_t split = WRITE ? args.write_split : 1u;
+    const uint32_t part = (blockIdx.x * ORDERED_WAVES + wave) % split;
+    const uint32_t work = (blockIdx.x * ORDERED_WAVES + wave) / split;
     const uint32_t slot = work / args.items_per_tile;
     const uint32_t item = work % args.items_per_tile;
     // workgroups are dealt to the 8 XCDs round-robin: each XCD walks one contiguous range of tiles, so that its L2
@@ -446,26 +487,31 @@ __global__ __launch_bounds__(ORDERED_BLOCK) void ordered_search_kernel(OrderedAr
         return; // the host does not use this path for such a tile: nothing to count, nothing may be written
     }
 
-    uint32_t* item_columns = args.columns + static_cast<size_t>(work) * (ORDERED_UNITS * WAVE);
+    CandidateRecord* item_records = args.records + static_cast<size_t>(work) * (ORDERED_UNITS * WAVE);
     if constexpr (!WRITE) {
         // ---- COUNT: the number of rows of every point (lane p adds up the hits of point p) and, for the writing
         // pass, the hit column of every candidate: a plain loop over the pairs of units, small code
         uint32_t own_rows = 0;
         for (uint32_t unit0 = 0; unit0 < n_units; unit0 += R) {
-            uint32_t column[R];
+            uint32_t column[R], at[R], original[R], biased[R];
             if (tile_wrapped) {
                 ordered_sweep_pair<FULL, true>(
-                    sh, sorted, g, unit0, n_stencil, n_candidates, first_i, n_i, lane, column, own_rows, out_of_range
+                    sh, sorted, g, unit0, n_stencil, n_candidates, first_i, n_i, lane, column, own_rows, out_of_range,
+                    at, original, biased
                 );
             } else {
                 ordered_sweep_pair<FULL, false>(
-                    sh, sorted, g, unit0, n_stencil, n_candidates, first_i, n_i, lane, column, own_rows, out_of_range
+                    sh, sorted, g, unit0, n_stencil, n_candidates, first_i, n_i, lane, column, own_rows, out_of_range,
+                    at, original, biased
                 );
             }
+            // everything the writing pass needs of a candidate in one 12-byte record, so that it takes one load per
+            // place of the tile's order instead of a table lookup and five scattered ones
 #pragma unroll
             for (int r = 0; r < R; r++) {
                 if (unit0 + r < n_units) {
-                    __builtin_nontemporal_store(column[r], &item_columns[(unit0 + r) * WAVE + lane]);
+                    // (plain stores: the writing pass reads them soon, out of the caches where they still are)
+                    item_records[(unit0 + r) * WAVE + lane] = CandidateRecord{column[r], original[r], biased[r]};
                 }
             }
         }
@@ -491,37 +537,38 @@ __global__ __launch_bounds__(ORDERED_BLOCK) void ordered_search_kernel(OrderedAr
     // without the wrap of the first point: that one is added per point, field by field in one integer addition)
     const uint16_t* tile_order = args.order + static_cast<size_t>(tile_id) * ORDERED_CANDIDATES;
     uint32_t columns[ORDERED_UNITS];
-    uint32_t cand_at[ORDERED_UNITS];
     uint32_t cand_index[ORDERED_UNITS];
     uint32_t cand_biased[ORDERED_UNITS];
 #pragma unroll
     for (int u = 0; u < ORDERED_UNITS; u++) {
         columns[u] = 0;
-        cand_at[u] = 0;
         cand_index[u] = 0;
         cand_biased[u] = 0;
         const uint32_t place = u * WAVE + lane;
         if (static_cast<uint32_t>(u) < n_units && place < n_candidates) {
             const uint32_t k = PRESORTED ? min(static_cast<uint32_t>(tile_order[place]), n_candidates - 1) : place;
-            columns[u] = __builtin_nontemporal_load(&item_columns[k]);
-            int32_t packed_q;
-            locate_candidate(sh, n_stencil, k, cand_at[u], packed_q);
-            int32_t qx, qy, qz;
-            unpack_shift(packed_q, qx, qy, qz);
-            cand_index[u] = sorted.index[cand_at[u]];
-            cand_biased[u] = biased_shift(qx - sorted.wx[cand_at[u]], qy - sorted.wy[cand_at[u]], qz - sorted.wz[cand_at[u]]);
+            const CandidateRecord record = item_records[k]; // one 12-byte load
+            columns[u] = record.column;
+            cand_index[u] = record.index;
+            cand_biased[u] = record.biased;
+        }
+        if (u % 4 == 3) {
+            // four units' loads in flight at a time: with all sixteen, their addresses alone take 32 registers
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 
     // ---- WRITE: point by point, collect the hits in lane order, rank them where that is not their final order,
     // store the rows
     wave_sync();
-    for (uint32_t p = 0; p < n_i; p++) {
+    const uint32_t per_part = (n_i + split - 1) / split;
+    for (uint32_t p = part * per_part; p < min(n_i, (part + 1) * per_part); p++) {
         // every field of the sum stays inside its ten bits (operands within +-255), so the fields add independently
         const uint32_t wrap_i = (static_cast<uint32_t>(sh.tile_wx[p]) << 20) + (static_cast<uint32_t>(sh.tile_wy[p]) << 10) +
                                 static_cast<uint32_t>(sh.tile_wz[p]);
+        // (the second points are looked up by their original index: no position to keep per candidate)
         write_rows_of_point<PRESORTED>(
-            sh, sorted, g, args.out, columns, cand_at, cand_index, cand_biased, n_units, n_i - 1 - p, wrap_i,
+            sh, PointsByIndex{args.points}, g, args.out, columns, cand_index, cand_index, cand_biased, n_units, n_i - 1 - p, wrap_i,
             sh.tile_x[p], sh.tile_y[p], sh.tile_z[p], sh.tile_index[p], sh.tile_row[p], lane
         );
     }

@@ -634,12 +634,8 @@ __global__ __launch_bounds__(WAVES * WAVE) void small_system_kernel(SmallArgs ar
     // ---- the rows of the item
     const uint32_t wrap_i = (static_cast<uint32_t>(wix) << 20) + (static_cast<uint32_t>(wiy) << 10) + static_cast<uint32_t>(wiz);
     if (SORTED) {
-        SortedPoints in_lds = {};
-        in_lds.x = shared.x;
-        in_lds.y = shared.y;
-        in_lds.z = shared.z;
         write_rows_of_point<false>(
-            sh, in_lds, g, args.out, columns, cand_at, cand_index, cand_biased, n_units, 0u, wrap_i, xi, yi, zi, oi,
+            sh, PointsByPlace{shared.x, shared.y, shared.z}, g, args.out, columns, cand_at, cand_index, cand_biased, n_units, 0u, wrap_i, xi, yi, zi, oi,
             static_cast<uint64_t>(shared.first_row[item]), lane
         );
     } else {
