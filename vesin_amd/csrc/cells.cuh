@@ -22,6 +22,8 @@ struct FusedStatus {
     unsigned int chain_timeout;    // waves that gave up waiting for an earlier workgroup
     unsigned int first_bad_coordinate;
     unsigned int crowded_cells;    // fixed-capacity layout: points that found their cell full (the result is void)
+    unsigned int far_outside;      // points more than a cell outside the extent the grid was chosen for (same)
+    unsigned int padding;
 };
 
 /// Cell-sorted copy of the points, one array per component: 64 consecutive candidates load coalesced, and four
@@ -53,17 +55,18 @@ __global__ void fetch_box(
         status->total_pairs = 0;
         status->first_bad_coordinate = 0xFFFFFFFFu;
         status->crowded_cells = 0;
+        status->far_outside = 0;
     }
 }
 
 /// Clears `n_blocks16` 16-byte blocks from `begin` (the histogram, the tiles' flags and the state of the single-pass
 /// search live next to each other), and does the work of fetch_box on the way when `box` is not null: one launch
 /// at the start of a call instead of a fetch and two fills.
-__global__ __launch_bounds__(BLOCK) void clear_and_fetch(
-    uint4* __restrict__ begin, size_t n_blocks16, const double* __restrict__ box, const bool* __restrict__ periodic,
-    unsigned char* host_small, DeviceStatus* status
+__device__ __forceinline__ void clear_and_fetch_as(
+    uint32_t block, uint32_t n_blocks, uint4* __restrict__ begin, size_t n_blocks16, const double* __restrict__ box,
+    const bool* __restrict__ periodic, unsigned char* host_small, DeviceStatus* status
 ) {
-    if (box != nullptr && blockIdx.x == 0) {
+    if (box != nullptr && block == 0) {
         const int t = threadIdx.x;
         if (t < 9) {
             reinterpret_cast<double*>(host_small)[t] = box[t];
@@ -73,13 +76,21 @@ __global__ __launch_bounds__(BLOCK) void clear_and_fetch(
             status->total_pairs = 0;
             status->first_bad_coordinate = 0xFFFFFFFFu;
             status->crowded_cells = 0;
+            status->far_outside = 0;
         }
     }
     const uint4 zero = {0u, 0u, 0u, 0u};
-    for (size_t k = static_cast<size_t>(blockIdx.x) * BLOCK + threadIdx.x; k < n_blocks16;
-         k += static_cast<size_t>(gridDim.x) * BLOCK) {
+    for (size_t k = static_cast<size_t>(block) * BLOCK + threadIdx.x; k < n_blocks16;
+         k += static_cast<size_t>(n_blocks) * BLOCK) {
         begin[k] = zero;
     }
+}
+
+__global__ __launch_bounds__(BLOCK) void clear_and_fetch(
+    uint4* __restrict__ begin, size_t n_blocks16, const double* __restrict__ box, const bool* __restrict__ periodic,
+    unsigned char* host_small, DeviceStatus* status
+) {
+    clear_and_fetch_as(blockIdx.x, gridDim.x, begin, n_blocks16, box, periodic, host_small, status);
 }
 
 /// After the counting pass: what the host needs to know goes to pinned host memory, read after the next
@@ -97,6 +108,8 @@ __global__ void publish_fused_status(const DeviceStatus* status, const FusedStat
         FusedStatus copy = *fused;
         copy.first_bad_coordinate = status->first_bad_coordinate;
         copy.crowded_cells = status->crowded_cells;
+        copy.far_outside = status->far_outside;
+        copy.padding = 0;
         *host_fused = copy;
     }
 }
@@ -127,15 +140,16 @@ __device__ __forceinline__ bool all_finite(double x, double y, double z, unsigne
 /// Smallest and largest fractional coordinate over all points (needed for non-periodic directions), plus the
 /// check for non-finite input. Grid-stride loop, wave then workgroup reduction; every workgroup reports to its own
 /// slot of `host_bounds` (pinned host memory), so no atomics are involved.
-__global__ __launch_bounds__(BLOCK) void bounding_kernel(
-    const double* __restrict__ points, uint32_t n_points, GridParams g, BlockBounds* host_bounds
+__device__ __forceinline__ void bounding_as(
+    uint32_t block, uint32_t n_blocks, const double* __restrict__ points, uint32_t n_points, const GridParams& g,
+    BlockBounds* host_bounds
 ) {
     __shared__ BlockBounds partial[WAVES_PER_BLOCK];
     double lo[3] = {INFINITY, INFINITY, INFINITY};
     double hi[3] = {-INFINITY, -INFINITY, -INFINITY};
     unsigned int bad = 0xFFFFFFFFu;
 
-    for (uint32_t i = blockIdx.x * BLOCK + threadIdx.x; i < n_points; i += gridDim.x * BLOCK) {
+    for (uint32_t i = block * BLOCK + threadIdx.x; i < n_points; i += n_blocks * BLOCK) {
         double x = points[3 * static_cast<size_t>(i) + 0];
         double y = points[3 * static_cast<size_t>(i) + 1];
         double z = points[3 * static_cast<size_t>(i) + 2];
@@ -184,14 +198,35 @@ __global__ __launch_bounds__(BLOCK) void bounding_kernel(
             all.first_bad_coordinate = min(all.first_bad_coordinate, partial[w].first_bad_coordinate);
         }
         all.padding = 0;
-        host_bounds[blockIdx.x] = all;
+        host_bounds[block] = all;
+    }
+}
+
+__global__ __launch_bounds__(BLOCK) void bounding_kernel(
+    const double* __restrict__ points, uint32_t n_points, GridParams g, BlockBounds* host_bounds
+) {
+    bounding_as(blockIdx.x, gridDim.x, points, n_points, g, host_bounds);
+}
+
+/// Both of the above in one launch, for a call whose grid follows the extent the call before found: the first
+/// `clear_blocks` workgroups clear and fetch the box, the others find the extent of this call's points, which the
+/// host reads at the end of the call (for the call after this one).
+__global__ __launch_bounds__(BLOCK) void clear_fetch_and_bound(
+    uint32_t clear_blocks, uint4* __restrict__ begin, size_t n_blocks16, const double* __restrict__ box,
+    const bool* __restrict__ periodic, unsigned char* host_small, DeviceStatus* status,
+    const double* __restrict__ points, uint32_t n_points, GridParams g, BlockBounds* host_bounds
+) {
+    if (blockIdx.x < clear_blocks) {
+        clear_and_fetch_as(blockIdx.x, clear_blocks, begin, n_blocks16, box, periodic, host_small, status);
+    } else {
+        bounding_as(blockIdx.x - clear_blocks, gridDim.x - clear_blocks, points, n_points, g, host_bounds);
     }
 }
 
 /// Cell coordinates and wrap shift of one point. Periodic directions: cell = floor(frac * n) brought back into
 /// [0, n) with the quotient kept as the wrap shift. Non-periodic directions: clamped, never wrapped.
 __device__ __forceinline__ void locate(
-    const GridParams& g, double x, double y, double z, int32_t cell[3], int32_t wrap[3]
+    const GridParams& g, double x, double y, double z, int32_t cell[3], int32_t wrap[3], bool* far_outside = nullptr
 ) {
     double f[3];
     fractional(g, x, y, z, f);
@@ -212,6 +247,12 @@ __device__ __forceinline__ void locate(
             wrap[d] = q;
         } else {
             double scaled = floor((f[d] - g.np_min[d]) * g.np_scale[d] * static_cast<double>(n));
+            if (far_outside != nullptr && (scaled < -1.0 || scaled > static_cast<double>(n))) {
+                // (a grid chosen for the points of this call holds them all; one chosen for those of the call
+                // before still gives the right list while points land in the outermost cells instead, but not
+                // in a sensible time once the points are somewhere else altogether)
+                *far_outside = true;
+            }
             scaled = fmin(fmax(scaled, 0.0), static_cast<double>(n - 1));
             cell[d] = static_cast<int32_t>(scaled);
             wrap[d] = 0;
@@ -240,7 +281,7 @@ __global__ __launch_bounds__(BLOCK) void assign_cells(
     uint32_t* __restrict__ cell_counts, DeviceStatus* status
 ) {
     const uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
-    const bool active = i < g.n_points;
+    bool active = i < g.n_points;
     const int lane = lane_id();
 
     int32_t cell[3] = {0, 0, 0};
@@ -251,7 +292,13 @@ __global__ __launch_bounds__(BLOCK) void assign_cells(
         double z = points[3 * static_cast<size_t>(i) + 2];
         unsigned int axis;
         if (all_finite(x, y, z, axis)) {
-            locate(g, x, y, z, cell, wrap);
+            bool far_outside = false;
+            locate(g, x, y, z, cell, wrap, &far_outside);
+            if (far_outside) {
+                // left out of the cell list (place_points does the same): the result is void, the search short
+                atomicAdd(&status->far_outside, 1u);
+                active = false;
+            }
         } else {
             atomicMin(&status->first_bad_coordinate, 3u * i + axis);
         }
@@ -304,7 +351,7 @@ __global__ __launch_bounds__(BLOCK) void place_direct(
     uint32_t* __restrict__ wrapped, SortedPoints sorted, DeviceStatus* status
 ) {
     const uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
-    const bool active = i < g.n_points;
+    bool active = i < g.n_points;
     const int lane = lane_id();
 
     int32_t cell[3] = {0, 0, 0};
@@ -316,7 +363,12 @@ __global__ __launch_bounds__(BLOCK) void place_direct(
         z = points[3 * static_cast<size_t>(i) + 2];
         unsigned int axis;
         if (all_finite(x, y, z, axis)) {
-            locate(g, x, y, z, cell, wrap);
+            bool far_outside = false;
+            locate(g, x, y, z, cell, wrap, &far_outside);
+            if (far_outside) {
+                atomicAdd(&status->far_outside, 1u); // dropped, like a point that finds its cell full
+                active = false;
+            }
         } else {
             atomicMin(&status->first_bad_coordinate, 3u * i + axis);
         }
@@ -383,7 +435,8 @@ __global__ __launch_bounds__(BLOCK) void scatter_points(
 /// the points inside a cell to be the same on every run: the slot handed out by the histogram atomic is final.
 /// Also appends the cell's tiles. `tiles[].wrapped` must be zero on entry. Cell and wrap shift of the point come
 /// from `cell_of` / `wrap_of` when given (a batch of systems), else the point is located again with `g`: cheaper
-/// than carrying 16 bytes per point from assign_cells through memory.
+/// than carrying 16 bytes per point from assign_cells through memory; in that case `sorted.wx / wy / wz` must be
+/// zero on entry, only the shifts of moved points are stored.
 __global__ __launch_bounds__(BLOCK) void place_points(
     const double* __restrict__ points, GridParams g, const int32_t* __restrict__ wrap_of,
     const uint32_t* __restrict__ cell_of, const uint32_t* __restrict__ slot_of,
@@ -410,7 +463,11 @@ __global__ __launch_bounds__(BLOCK) void place_points(
         int32_t wrap[3] = {0, 0, 0};
         unsigned int axis;
         if (all_finite(x, y, z, axis)) {
-            locate(g, x, y, z, where, wrap);
+            bool far_outside = false;
+            locate(g, x, y, z, where, wrap, &far_outside);
+            if (far_outside) {
+                return; // assign_cells did not count it
+            }
         }
         cell = (static_cast<uint32_t>(where[2]) * g.n[1] + where[1]) * g.n[0] + where[0];
         wx = wrap[0];
@@ -431,10 +488,14 @@ __global__ __launch_bounds__(BLOCK) void place_points(
     sorted.x[to] = x;
     sorted.y[to] = y;
     sorted.z[to] = z;
-    sorted.wx[to] = wx;
-    sorted.wy[to] = wy;
-    sorted.wz[to] = wz;
     const uint32_t tile_size = tile_size_of(count);
+    // A single system's caller hands the wrap arrays over cleared: points in arbitrary order scatter their stores, a
+    // 32-byte sector of memory traffic for each, and most points were not moved by any box vector.
+    if (cell_of != nullptr || (wx | wy | wz) != 0) {
+        sorted.wx[to] = wx;
+        sorted.wy[to] = wy;
+        sorted.wz[to] = wz;
+    }
     if ((wx | wy | wz) != 0) {
         atomicOr(&tiles[first_tile + k / tile_size].wrapped, 1u);
     }
@@ -670,6 +731,7 @@ __global__ __launch_bounds__(SMALL_BUILD_THREADS) void build_cells_small(
             status->total_pairs = 0;
             status->first_bad_coordinate = 0xFFFFFFFFu;
             status->crowded_cells = 0;
+            status->far_outside = 0;
         }
     }
     const uint4 zero = {0u, 0u, 0u, 0u};
@@ -799,6 +861,7 @@ __global__ __launch_bounds__(BLOCK) void prepare_single_cell(
                 status->total_pairs = 0;
                 status->first_bad_coordinate = 0xFFFFFFFFu;
                 status->crowded_cells = 0;
+                status->far_outside = 0;
             }
         }
         const uint4 zero = {0u, 0u, 0u, 0u};

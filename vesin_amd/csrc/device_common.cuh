@@ -58,6 +58,8 @@ struct DeviceStatus {
     unsigned long long total_pairs;
     unsigned int first_bad_coordinate; // 3 * point + axis of the first non-finite coordinate, or 0xFFFFFFFF
     unsigned int crowded_cells;        // fixed-capacity layout: points that found their cell full
+    unsigned int far_outside;          // points more than a cell outside the extent the grid was chosen for
+    unsigned int padding;
 };
 
 /// What one workgroup of the bounding pass reports (to pinned host memory; the host folds the workgroups).

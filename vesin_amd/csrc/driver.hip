@@ -128,6 +128,13 @@ static bool separate_launches() {
     return text != nullptr && std::strcmp(text, "separate") == 0;
 }
 
+/// VESIN_HIP_EXTENT=fresh makes every call on a larger system with a non-periodic direction find the extent of its
+/// points before it picks the grid (for comparisons and tests), instead of starting from the extent of the call before.
+static bool fresh_extent_only() {
+    const char* text = std::getenv("VESIN_HIP_EXTENT");
+    return text != nullptr && std::strcmp(text, "fresh") == 0;
+}
+
 /// VESIN_HIP_STREAMS=one keeps every kernel of a call on the call's stream (for comparisons and tests); otherwise the
 /// in-order search orders the candidates of the tiles on a second stream while it counts the rows.
 static bool ordered_one_stream() {
@@ -238,6 +245,10 @@ struct Carver {
 /// half the memory bandwidth, and a filter has to read every candidate on top of writing the same rows. Measured
 /// on jittered diamond (cutoff 5, skin 0.5): the filter takes 0.038 ms against 0.077 ms at 0.2 M candidates,
 /// breaks even near 1.6 M and takes twice the direct search's time at 15 M.
+/// Calls that find the extent of their points first after one that started from the extent of the call before and
+/// found its points somewhere else.
+constexpr int EXTENT_REST = 8;
+
 constexpr size_t VERLET_MAX_CANDIDATES = size_t(1) << 20;
 
 /// One-pass cell build: slots per cell (one tile: with two the search has as many empty tiles as full ones and
@@ -350,6 +361,8 @@ struct HipExtras {
     /// the cutoff at least and has no neighbours beyond: the rows are the same, a stale extent only costs time
     /// (crowded cells), and with at most 2048 points never much.
     bool extent_valid = false;
+    bool extent_missed = false;       // the call started from that extent and found its points far outside of it
+    int extent_rest = 0;              // calls that find the extent first after such a call
     double extent_lo[3] = {0, 0, 0};
     double extent_hi[3] = {0, 0, 0};
     SmallMeeting* meetings = nullptr; // device, two of them (see SmallMeeting); allocated at the first small system
@@ -733,7 +746,11 @@ void direct_neighbors(
             extras.guess.was_right();
             return;
         }
-        extras.guess.was_wrong();
+        if (extras.extent_missed) {
+            extras.extent_missed = false; // nothing wrong with the box
+        } else {
+            extras.guess.was_wrong();
+        }
     }
     (void)compute(points, n_points, box, periodic, options, neighbors, extras, false, stream);
     extras.guess.stored(key);
@@ -825,8 +842,18 @@ bool compute(
     double lo[3] = {0, 0, 0};
     double hi[3] = {0, 0, 0};
     // (valid for one call: whatever happens below, only a call that reports a fresh extent makes it valid again)
-    const bool remembered_extent = any_open && speculate && extras.extent_valid && n_points <= SMALL_POINTS &&
-                                   extras.one_launch_rest == 0;
+    // Small systems: for the one launch that does everything. Larger ones: for the single-pass search, which then
+    // needs no pass over the points and no answer from the device before its kernels are launched. Either way the
+    // call finds the extent of its own points on the way and leaves it for the call after it. A grid that fits
+    // the points of the call before still gives the right list: points beyond it land in the outermost cells.
+    const bool small_guess = n_points <= SMALL_POINTS && extras.one_launch_rest == 0;
+    const bool large_guess = n_points > SMALL_POINTS && !options.sorted && extras.capacity > 0 && !two_pass_only() &&
+                             extras.single_pass_rest == 0 && !ordered_rows() && options.algorithm != VesinBruteForce &&
+                             extras.extent_rest == 0 && !fresh_extent_only();
+    if (any_open && extras.extent_rest > 0) {
+        extras.extent_rest -= 1;
+    }
+    const bool remembered_extent = any_open && speculate && extras.extent_valid && (small_guess || large_guess);
     extras.extent_valid = false;
     if (remembered_extent) {
         for (int d = 0; d < 3; d++) {
@@ -863,6 +890,13 @@ bool compute(
         }
         if (bad != 0xFFFFFFFFu) {
             non_finite_error(points, bad);
+        }
+        if (n_points > SMALL_POINTS) {
+            for (int d = 0; d < 3; d++) {
+                extras.extent_lo[d] = lo[d];
+                extras.extent_hi[d] = hi[d];
+            }
+            extras.extent_valid = true;
         }
     }
 
@@ -1011,6 +1045,7 @@ bool compute(
     uint64_t* first_row_of_point = nullptr;
     CandidateRecord* candidate_records = nullptr;
     uint16_t* candidate_order = nullptr;
+    char* wraps_end = nullptr;
     // small systems: the points of a tile are dealt to several waves, about 2048 in all
     uint32_t ordered_points_per_item = TILE_POINTS;
     while (ordered_points_per_item > 1 && tiles_bound * (TILE_POINTS / ordered_points_per_item) < 2048) {
@@ -1034,6 +1069,11 @@ bool compute(
         direct_wrapped = carver.take<uint32_t>(direct_slots);
         fused_status = carver.take<FusedStatus>(1);
         ordered_status = carver.take<OrderedStatus>(1);
+        // (behind the state that every call clears: place_points wants them cleared too)
+        sorted.wx = carver.take<int32_t>(sorted_slots + SORTED_PADDING);
+        sorted.wy = carver.take<int32_t>(sorted_slots + SORTED_PADDING);
+        sorted.wz = carver.take<int32_t>(sorted_slots + SORTED_PADDING);
+        wraps_end = reinterpret_cast<char*>(carver.take<uint32_t>(0));
         cell_scan = carver.take<uint64_t>(n_cells + 1);
         if (!single_cell) {
             cell_of = carver.take<uint32_t>(n_points);
@@ -1045,9 +1085,6 @@ bool compute(
         sorted.y = carver.take<double>(sorted_slots + SORTED_PADDING);
         sorted.z = carver.take<double>(sorted_slots + SORTED_PADDING);
         sorted.index = carver.take<uint32_t>(sorted_slots + SORTED_PADDING);
-        sorted.wx = carver.take<int32_t>(sorted_slots + SORTED_PADDING);
-        sorted.wy = carver.take<int32_t>(sorted_slots + SORTED_PADDING);
-        sorted.wz = carver.take<int32_t>(sorted_slots + SORTED_PADDING);
         counts = carver.take<uint32_t>(std::max(n_slots, direct_slots * n_slices));
         offsets = carver.take<uint64_t>(std::max(n_slots, direct_slots * n_slices) + 1);
         scan_scratch = carver.take<uint64_t>(scratch_elements);
@@ -1083,8 +1120,9 @@ bool compute(
     // in one launch (small_system_kernel). Its workgroups wait for each other, which needs all of them resident at
     // once; when they were not, or the system does not suit that launch, or the rows do not fit, the call goes on
     // as if nothing had happened, and (except in the last case) the list leaves that launch alone for a while.
-    if (remembered_extent && !one_launch) {
-        // the grid came from an extent that only the one launch refreshes: start over with a pass over the points
+    const bool guessed_grid = remembered_extent && !one_launch && try_single_pass && !single_cell && !small_build;
+    if (remembered_extent && !one_launch && !guessed_grid) {
+        // the grid came from an extent that only these two ways refresh: start over with a pass over the points
         return false;
     }
     if (one_launch) {
@@ -1171,12 +1209,25 @@ bool compute(
 
     // ---- cell list
     const uint32_t point_blocks = static_cast<uint32_t>((n_points + BLOCK - 1) / BLOCK);
+    const uint32_t bounding_blocks = std::min<uint32_t>(BOUNDING_BLOCKS, point_blocks);
     const auto* flat_points = reinterpret_cast<const double*>(points);
-    auto clear_work_state = [&]() {
+    auto clear_work_state = [&](bool wraps_too) {
         // every piece of the work buffer is padded to 256 bytes: clearing whole 16-byte blocks stays inside
-        const size_t to_clear = reinterpret_cast<char*>(ordered_status + 1) - reinterpret_cast<char*>(cell_counts);
+        const char* end = wraps_too ? wraps_end : reinterpret_cast<char*>(ordered_status + 1);
+        const size_t to_clear = end - reinterpret_cast<char*>(cell_counts);
         const size_t blocks16 = (to_clear + 15) / 16;
         const uint32_t fill_blocks = static_cast<uint32_t>(std::min<size_t>(1024, (blocks16 + BLOCK - 1) / BLOCK));
+        if (guessed_grid) {
+            // ... and the extent of this call's points, for the call after it
+            hipLaunchKernelGGL(
+                clear_fetch_and_bound, dim3(fill_blocks + bounding_blocks), dim3(BLOCK), 0, stream,
+                fill_blocks, reinterpret_cast<uint4*>(cell_counts), blocks16,
+                fetched ? static_cast<const double*>(nullptr) : reinterpret_cast<const double*>(box), periodic,
+                extras.mail_device->small, extras.d_status, flat_points, g.n_points, g, extras.mail_device->bounds
+            );
+            fetched = true;
+            return;
+        }
         hipLaunchKernelGGL(
             clear_and_fetch, dim3(fill_blocks), dim3(BLOCK), 0, stream,
             reinterpret_cast<uint4*>(cell_counts), blocks16,
@@ -1239,13 +1290,13 @@ bool compute(
         );
         fetched = true;
     } else if (direct_cells) {
-        clear_work_state();
+        clear_work_state(false);
         hipLaunchKernelGGL(
             place_direct, dim3(point_blocks), dim3(BLOCK), 0, stream,
             flat_points, g, DIRECT_CAPACITY, cell_counts, direct_wrapped, sorted, extras.d_status
         );
     } else {
-        clear_work_state();
+        clear_work_state(!single_cell);
         build_packed_cells();
     }
     mark(T_CELLS);
@@ -1305,6 +1356,30 @@ bool compute(
         const FusedStatus result = extras.mail->fused;
         if (result.first_bad_coordinate != 0xFFFFFFFFu) {
             non_finite_error(points, result.first_bad_coordinate);
+        }
+        if (guessed_grid) {
+            if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
+                std::fprintf(stderr, "grid from the extent of the call before: %u points far outside\n", result.far_outside);
+            }
+            if (result.far_outside != 0) {
+                // the points are somewhere else altogether: those were left out, the call starts over with the
+                // same box, and the list finds the extent first for a while
+                extras.extent_rest = EXTENT_REST;
+                extras.extent_missed = true;
+                return false;
+            }
+            for (int d = 0; d < 3; d++) {
+                extras.extent_lo[d] = INFINITY;
+                extras.extent_hi[d] = -INFINITY;
+            }
+            for (uint32_t block = 0; block < bounding_blocks; block++) {
+                const BlockBounds& part = extras.mail->bounds[block];
+                for (int d = 0; d < 3; d++) {
+                    extras.extent_lo[d] = std::fmin(extras.extent_lo[d], part.lo[d]);
+                    extras.extent_hi[d] = std::fmax(extras.extent_hi[d], part.hi[d]);
+                }
+            }
+            extras.extent_valid = true;
         }
         if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
             uint32_t stencil_cells = 0;
@@ -1366,7 +1441,7 @@ bool compute(
             if (!cells_ok) {
                 extras.direct_rest = DIRECT_REST;
             }
-            clear_work_state();
+            clear_work_state(!single_cell);
             build_packed_cells();
         }
     }
@@ -2154,6 +2229,7 @@ void neighbors_batch(
 
     // ---- cell lists of all systems, in one sequence of launches
     const uint32_t point_blocks = static_cast<uint32_t>((n_points + BLOCK - 1) / BLOCK);
+    const uint32_t bounding_blocks = std::min<uint32_t>(BOUNDING_BLOCKS, point_blocks);
     const auto* flat_points = reinterpret_cast<const double*>(points);
     hipLaunchKernelGGL(
         fetch_box, dim3(1), dim3(64), 0, stream,
