@@ -281,3 +281,27 @@ def test_well_filled_tiles_that_barely_exceed_the_resident_waves_get_four_waves_
         assert np.array_equal(d.cpu().numpy(), expected["distances"])
         assert np.array_equal(D.cpu().numpy(), expected["vectors"])
     assert waves == [1, 4, 4]
+
+
+@pytest.mark.parametrize("waves", [2, 3, 4])
+@pytest.mark.parametrize("full", [True, False])
+def test_any_number_of_waves_per_tile_counts_the_same_rows(waves, full, capfd, monkeypatch):
+    """The candidates of a tile dealt to several waves of the counting pass, which add up their rows per point."""
+    monkeypatch.setenv("VESIN_HIP_COUNT_SPLIT", str(waves))
+    points, box = _lattice(20, 20, 20, seed=13)
+    _check_order_once(points, box, [True] * 3, 5.0, full, capfd, monkeypatch)
+    # a tile with fewer pairs of units than waves, points outside of the box, a free direction
+    rng = np.random.default_rng(waves)
+    box = np.diag([31.0, 32.0, 33.0])
+    points = rng.uniform(-6.0, 38.0, size=(9000, 3))
+    _check(points, box, (True, False, True), 3.0, full, capfd, monkeypatch, "used")
+
+
+def test_rows_of_one_point_beyond_the_ranking_counted_by_several_waves(capfd, monkeypatch):
+    """The most rows of a point are known to the wave of the tile that adds its share last."""
+    monkeypatch.setenv("VESIN_HIP_COUNT_SPLIT", "2")
+    rng = np.random.default_rng(29)
+    directions = rng.normal(size=(400, 3))
+    ball = 1.2 * directions / np.linalg.norm(directions, axis=1)[:, None] * rng.random((400, 1)) ** (1 / 3) + 10.0
+    points = np.concatenate([ball, rng.random((5000, 3)) * 40.0])
+    _check(points, np.diag([40.0, 40.0, 40.0]), True, 3.0, True, capfd, monkeypatch, "left to the radix sort")

@@ -410,10 +410,11 @@ __global__ __launch_bounds__(BLOCK) void place_direct(
     sorted.x[to] = x;
     sorted.y[to] = y;
     sorted.z[to] = z;
-    sorted.wx[to] = wrap[0];
-    sorted.wy[to] = wrap[1];
-    sorted.wz[to] = wrap[2];
     if ((wrap[0] | wrap[1] | wrap[2]) != 0) {
+        // (the caller hands the wrap arrays over cleared, as for place_points)
+        sorted.wx[to] = wrap[0];
+        sorted.wy[to] = wrap[1];
+        sorted.wz[to] = wrap[2];
         atomicOr(&wrapped[(linear * capacity + k) / TILE_POINTS], 1u);
     }
 }

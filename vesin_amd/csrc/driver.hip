@@ -1073,6 +1073,9 @@ bool compute(
         sorted.wx = carver.take<int32_t>(sorted_slots + SORTED_PADDING);
         sorted.wy = carver.take<int32_t>(sorted_slots + SORTED_PADDING);
         sorted.wz = carver.take<int32_t>(sorted_slots + SORTED_PADDING);
+        if (try_in_order) {
+            rows_of_point = carver.take<uint32_t>(n_points); // (cleared as well: its counting pass may add to it)
+        }
         wraps_end = reinterpret_cast<char*>(carver.take<uint32_t>(0));
         cell_scan = carver.take<uint64_t>(n_cells + 1);
         if (!single_cell) {
@@ -1090,7 +1093,6 @@ bool compute(
         scan_scratch = carver.take<uint64_t>(scratch_elements);
         rows_of_item = carver.take<uint32_t>(small_items);
         if (try_in_order) {
-            rows_of_point = carver.take<uint32_t>(n_points);
             first_row_of_point = carver.take<uint64_t>(n_points + 1);
             candidate_records = carver.take<CandidateRecord>(static_cast<size_t>(ordered_blocks) * ORDERED_WAVES * ORDERED_UNITS * WAVE);
             if (ordered_items_per_tile == 1) {
@@ -1290,7 +1292,7 @@ bool compute(
         );
         fetched = true;
     } else if (direct_cells) {
-        clear_work_state(false);
+        clear_work_state(true);
         hipLaunchKernelGGL(
             place_direct, dim3(point_blocks), dim3(BLOCK), 0, stream,
             flat_points, g, DIRECT_CAPACITY, cell_counts, direct_wrapped, sorted, extras.d_status
@@ -1479,6 +1481,23 @@ bool compute(
         if (const char* text = std::getenv("VESIN_HIP_WRITE_SPLIT")) {
             oargs.write_split = static_cast<uint32_t>(std::max(1, std::min(4, std::atoi(text))));
         }
+        // The counting pass runs seven waves per SIMD (7168 at a time) and lasts as long as its slowest wave, the
+        // one of the tile with the most points and candidates. While the tiles of a system do not fill those
+        // slots much more than once, the candidates of every well-filled tile are dealt to two waves (pairs of
+        // units of 64 in turn) that add up their rows per point, in memory that the cell build cleared. Measured
+        // per call on half lists, cutoff 6: 24 points per tile, 25,000 / 50,000 / 100,000 / 200,000 atoms 168 -> 155,
+        // 217 -> 201, 312 -> 304, 529 -> 519 us (four waves: 166, 205, 297, 537), 400,000 atoms (17,576 tiles)
+        // 833 -> 841; 12 points per tile, 30,000 / 100,000 atoms 137 -> 143, 275 -> 282 us.
+        oargs.count_split = 1;
+        const bool rows_cleared = !single_cell && !small_build;
+        if (ordered_items_per_tile == 1 && rows_cleared && extras.ordered_tiles_points == n_points &&
+            extras.ordered_tiles > 0 && extras.ordered_tiles <= 9216 &&
+            static_cast<double>(n_points) >= 16.0 * static_cast<double>(extras.ordered_tiles)) {
+            oargs.count_split = 2;
+        }
+        if (const char* text = std::getenv("VESIN_HIP_COUNT_SPLIT")) {
+            oargs.count_split = rows_cleared ? static_cast<uint32_t>(std::max(1, std::min(4, std::atoi(text)))) : 1u;
+        }
         oargs.points = reinterpret_cast<const double*>(points);
         oargs.order = candidate_order;
         oargs.first_row = first_row_of_point;
@@ -1524,9 +1543,9 @@ bool compute(
                 HIP_CHECK(hipEventRecord(extras.side_join, side));
             }
             if (options.full) {
-                hipLaunchKernelGGL((ordered_search_kernel<false, true>), dim3(blocks), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
+                hipLaunchKernelGGL((ordered_search_kernel<false, true>), dim3(blocks * oargs.count_split), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
             } else {
-                hipLaunchKernelGGL((ordered_search_kernel<false, false>), dim3(blocks), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
+                hipLaunchKernelGGL((ordered_search_kernel<false, false>), dim3(blocks * oargs.count_split), dim3(ORDERED_BLOCK), 0, stream, oargs, g);
             }
             if (side != nullptr) {
                 HIP_CHECK(hipStreamWaitEvent(stream, extras.side_join, 0));
@@ -1566,9 +1585,9 @@ bool compute(
             std::fprintf(
                 stderr,
                 "in-order search: rows %llu, most rows of a point %u, most candidates of a tile %u, unsuitable %u, "
-                "candidates of %u tiles ordered by window and of %u by buckets, %u tiles written by %u waves each: %s\n",
+                "candidates of %u tiles ordered by window and of %u by buckets, %u tiles written by %u waves each and counted by %u: %s\n",
                 found.total_rows, found.found.max_rows, found.found.max_candidates, found.found.unsuitable,
-                found.found.windowed, found.found.bucketed, found.n_tiles, oargs.write_split,
+                found.found.windowed, found.found.bucketed, found.n_tiles, oargs.write_split, oargs.count_split,
                 suitable ? "used" : "left to the radix sort"
             );
         }

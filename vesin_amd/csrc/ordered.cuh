@@ -82,6 +82,8 @@ struct OrderedArgs {
     const uint64_t* first_row;  // WRITE: [n_points + 1], exclusive scan of rows_of_point
     OrderedStatus* status;
     uint32_t write_split;       // WRITE: waves that share the points of one work item of the counting pass (at least 1)
+    uint32_t count_split;       // COUNT: waves that share the candidates of one work item (at least 1; more than 1:
+                                // `rows_of_point` is zero on entry and the waves add to it)
     uint32_t report_order;      // SORT: count the tiles ordered either way (an atomic per tile on one word: for tests)
     uint32_t guarded;           // WRITE launched before the host has seen what COUNT found: write nothing unless the
                                 // system suits this search and the rows fit the `capacity` of the arrays
@@ -418,7 +420,8 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
     const uint32_t n_tiles = static_cast<uint32_t>(args.cell_scan[g.n_cells] >> 32);
     // WRITE may deal the points of a work item of the counting pass to several waves (`write_split`): they read the
     // same records and each writes the rows of its share of the points
-    const uint32_t split = WRITE ? args.write_split : 1u;
+    // COUNT may deal the candidates of a work item to several waves (`count_split`), by pairs of units in turn
+    const uint32_t split = WRITE ? args.write_split : args.count_split;
     const uint32_t part = (blockIdx.x * ORDERED_WAVES + wave) % split;
     const uint32_t work = (blockIdx.x * ORDERED_WAVES + wave) / split;
     const uint32_t slot = work / args.items_per_tile;
@@ -479,7 +482,8 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
 
     if (!WRITE) {
         // thousands of waves report to the same words: an atomic only where it would change something
-        if (lane == 0 && item == 0 && n_candidates > __atomic_load_n(&args.status->max_candidates, __ATOMIC_RELAXED)) {
+        if (lane == 0 && item == 0 && part == 0 &&
+            n_candidates > __atomic_load_n(&args.status->max_candidates, __ATOMIC_RELAXED)) {
             atomicMax(&args.status->max_candidates, n_candidates);
         }
     }
@@ -492,7 +496,7 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
         // ---- COUNT: the number of rows of every point (lane p adds up the hits of point p) and, for the writing
         // pass, the hit column of every candidate: a plain loop over the pairs of units, small code
         uint32_t own_rows = 0;
-        for (uint32_t unit0 = 0; unit0 < n_units; unit0 += R) {
+        for (uint32_t unit0 = part * R; unit0 < n_units; unit0 += split * R) {
             uint32_t column[R], at[R], original[R], biased[R];
             if (tile_wrapped) {
                 ordered_sweep_pair<FULL, true>(
@@ -516,7 +520,13 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
             }
         }
         if (static_cast<uint32_t>(lane) < n_i) {
-            args.rows_of_point[sh.tile_index[lane]] = own_rows;
+            if (split == 1) {
+                args.rows_of_point[sh.tile_index[lane]] = own_rows;
+            } else {
+                // whichever wave of the item comes last sees the sum of the others: the largest number any of
+                // them sees for a point is the point's number of rows
+                own_rows += atomicAdd(&args.rows_of_point[sh.tile_index[lane]], own_rows);
+            }
         }
         uint32_t most = own_rows;
 #pragma unroll
