@@ -1048,8 +1048,30 @@ bool compute(
     char* wraps_end = nullptr;
     // small systems: the points of a tile are dealt to several waves, about 2048 in all
     uint32_t ordered_points_per_item = TILE_POINTS;
+    const double filled_cells = static_cast<double>(std::max<size_t>(1, std::min(n_cells, n_points)));
+    const double mean_per_cell = std::min<double>(TILE_POINTS, static_cast<double>(n_points) / filled_cells);
+    if (!extras.fixed_memory && (filled_cells < 2048.0 || (filled_cells < 3072.0 && mean_per_cell <= 12.0))) {
+        // Too few tiles for one wave each to fill the GPU, and too few points for the order of a tile's candidates
+        // to be worth a launch of its own: what counts is how long the slowest wave of either pass lives, and that
+        // grows with the points it has to write the rows of. Shares of 8 points, of 4 where that leaves fewer than
+        // about 1300 waves with any points at all (measured per call, cutoff 5, full lists, shares of 32 / 16 / 8 / 4
+        // / 2 points: 10,000 atoms at 0.05 per cubic A 116 / 100 / 93 / 100 / 127 us, at 0.1 137 / 125 / 101 / 108 /
+        // 115 us; 4,000 atoms 101 / 85 / 76 / 74 / 86 and 125 / 122 / 94 / 82 / 81 us). Shares that most tiles have
+        // no points for cost next to nothing in time, their waves leave at once, but each has room for its
+        // candidates' records: the entry point that allocates nothing keeps the coarser shares below.
+        ordered_points_per_item = filled_cells * std::ceil(mean_per_cell / 8.0) < 1300.0 ? 4 : 8;
+    }
+    // the smallest systems: as many waves as the GPU runs at once, down to one point each
     while (ordered_points_per_item > 1 && tiles_bound * (TILE_POINTS / ordered_points_per_item) < 2048) {
         ordered_points_per_item /= 2;
+    }
+    if (const char* text = std::getenv("VESIN_HIP_ORDERED_SHARE")) {
+        // (for measurements and tests: a power of two)
+        uint32_t wanted = static_cast<uint32_t>(std::max(1, std::min<int>(TILE_POINTS, std::atoi(text))));
+        while ((wanted & (wanted - 1)) != 0) {
+            wanted &= wanted - 1;
+        }
+        ordered_points_per_item = wanted;
     }
     const uint32_t ordered_items_per_tile = TILE_POINTS / ordered_points_per_item;
     const uint32_t ordered_blocks =
