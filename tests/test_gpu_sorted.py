@@ -305,3 +305,13 @@ def test_rows_of_one_point_beyond_the_ranking_counted_by_several_waves(capfd, mo
     ball = 1.2 * directions / np.linalg.norm(directions, axis=1)[:, None] * rng.random((400, 1)) ** (1 / 3) + 10.0
     points = np.concatenate([ball, rng.random((5000, 3)) * 40.0])
     _check(points, np.diag([40.0, 40.0, 40.0]), True, 3.0, True, capfd, monkeypatch, "left to the radix sort")
+
+
+@pytest.mark.parametrize("share", [1, 2, 4, 8, 16, 32])
+def test_any_share_of_a_tile_per_wave_gives_the_same_list(share, capfd, monkeypatch):
+    """The points of a tile that one wave takes: chosen by the size of the system, forced here."""
+    monkeypatch.setenv("VESIN_HIP_ORDERED_SHARE", str(share))
+    rng = np.random.default_rng(share)
+    box = np.array([[44.0, 0.0, 0.0], [5.0, 41.0, 0.0], [-3.0, 2.0, 46.0]])
+    points = rng.uniform(-0.2, 1.2, size=(7000, 3)) @ box
+    _check(points, box, (True, True, False), 4.0, share % 3 != 0, capfd, monkeypatch, "used")
