@@ -106,3 +106,16 @@ extern "C" void probe_box_guess(
         guess.stored(key);
     }
 }
+
+/// The cut of the in-order search's work into waves (policy.hpp), as the driver asks for it.
+extern "C" unsigned int probe_ordered_share(size_t n_points, size_t n_cells, size_t tile_slots, int coarse) {
+    return vesin_hip::ordered_share(n_points, n_cells, tile_slots, coarse != 0);
+}
+
+extern "C" unsigned int probe_ordered_write_split(size_t n_points, size_t tiles_before) {
+    return vesin_hip::ordered_write_split(n_points, tiles_before);
+}
+
+extern "C" unsigned int probe_ordered_count_split(size_t n_points, size_t tiles_before) {
+    return vesin_hip::ordered_count_split(n_points, tiles_before);
+}

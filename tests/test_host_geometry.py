@@ -33,6 +33,11 @@ def probe(tmp_path_factory):
                                   ctypes.c_void_p, ctypes.c_size_t]
     lib.probe_box_guess.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
     lib.probe_box_guess.restype = None
+    lib.probe_ordered_share.argtypes = [ctypes.c_size_t, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_int]
+    lib.probe_ordered_share.restype = ctypes.c_uint
+    for name in ("probe_ordered_write_split", "probe_ordered_count_split"):
+        getattr(lib, name).argtypes = [ctypes.c_size_t, ctypes.c_size_t]
+        getattr(lib, name).restype = ctypes.c_uint
     return lib
 
 
@@ -268,3 +273,71 @@ def test_dropped_stencil_entries_cannot_hold_a_neighbour(probe, seed):
             assert apart <= cutoff * (1 + 1e-5), f"entry {offset} at {apart} is kept (cutoff {cutoff})"
     if kind <= 1 and min(s) >= 2:
         assert n_dropped > 0
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# How the search that writes a sorted list in order cuts its work into waves (policy.hpp)
+
+
+def _tile_slots(n_points, n_cells):
+    """What the driver holds tiles for: a tile per occupied cell and one more per 32 points, in multiples of 32."""
+    slots = min(n_cells, n_points) + n_points // 32 + 1
+    return (slots + 31) // 32 * 32
+
+
+def test_share_of_a_tile_per_wave(probe):
+    def share(n_points, n_cells, coarse=False):
+        return probe.probe_ordered_share(n_points, n_cells, _tile_slots(n_points, n_cells), int(coarse))
+
+    # large systems: a wave per tile
+    assert share(100_000, 4096) == 32
+    assert share(1_000_000, 42_875) == 32
+    assert share(30_000, 3375) == 32  # 8.9 points per cell, but enough tiles
+    # mid-size systems: 8 points, or 4 where shares of 8 would be too few
+    assert share(10_000, 1331) == 8
+    assert share(10_000, 729) == 8   # 13.7 points per cell: two shares of 8 per tile, 1458 in all
+    assert share(6_000, 343) == 4    # 17.5 points per cell: three shares of 8 per tile are only 1029
+    assert share(4_000, 512) == 4
+    assert share(15_000, 2197) == 8  # more than 2048 cells, few points in each
+    assert share(50_000, 2197) == 32  # the same cells well filled: the tiles are worth a wave each
+    # the smallest systems: down to a point per wave
+    assert share(216, 27) == 1
+    assert share(2_000, 343) == 4
+    assert share(1, 1) == 1
+    # fixed work memory: the coarser rule, which only counts the slots
+    assert share(10_000, 1331, coarse=True) == 16
+    assert share(6_000, 343, coarse=True) == 8
+    assert share(100_000, 4096, coarse=True) == 32
+    # always a power of two between 1 and 32
+    rng = np.random.default_rng(5)
+    for _ in range(2000):
+        n_points = int(rng.integers(1, 400_000))
+        n_cells = int(rng.integers(1, 2 * n_points + 2))
+        for coarse in (False, True):
+            found = share(n_points, n_cells, coarse)
+            assert found in (1, 2, 4, 8, 16, 32)
+            if not coarse:
+                assert found <= share(n_points, n_cells, True) or found in (4, 8)
+
+
+def test_waves_per_tile_of_the_two_passes(probe):
+    write = probe.probe_ordered_write_split
+    count = probe.probe_ordered_count_split
+    # nothing known about the system yet
+    assert write(100_000, 0) == 1 and count(100_000, 0) == 1
+    # the 100,000-atom benchmark: 4,260 tiles of 23.5 points
+    assert write(100_000, 4260) == 4 and count(100_000, 4260) == 2
+    # twice and four times the size at the same filling
+    assert write(200_000, 9000) == 2 and count(200_000, 9000) == 2
+    assert write(400_000, 19_000) == 1 and count(400_000, 19_000) == 1
+    # few tiles: the writing pass has room for all of them at once
+    assert write(50_000, 2300) == 1 and count(50_000, 2300) == 2
+    # 12 points per tile: one wave each, whatever the number of tiles
+    assert write(100_000, 8100) == 1 and count(100_000, 8100) == 1
+    assert write(50_000, 4200) == 1 and count(50_000, 4200) == 1
+    for tiles in range(1, 40_000, 97):
+        for per_tile in (3, 15, 16, 31):
+            assert write(tiles * per_tile, tiles) in (1, 2, 4)
+            assert count(tiles * per_tile, tiles) in (1, 2)
+            if per_tile < 16:
+                assert write(tiles * per_tile, tiles) == 1 and count(tiles * per_tile, tiles) == 1

@@ -1047,24 +1047,8 @@ bool compute(
     uint16_t* candidate_order = nullptr;
     char* wraps_end = nullptr;
     // small systems: the points of a tile are dealt to several waves, about 2048 in all
-    uint32_t ordered_points_per_item = TILE_POINTS;
-    const double filled_cells = static_cast<double>(std::max<size_t>(1, std::min(n_cells, n_points)));
-    const double mean_per_cell = std::min<double>(TILE_POINTS, static_cast<double>(n_points) / filled_cells);
-    if (!extras.fixed_memory && (filled_cells < 2048.0 || (filled_cells < 3072.0 && mean_per_cell <= 12.0))) {
-        // Too few tiles for one wave each to fill the GPU, and too few points for the order of a tile's candidates
-        // to be worth a launch of its own: what counts is how long the slowest wave of either pass lives, and that
-        // grows with the points it has to write the rows of. Shares of 8 points, of 4 where that leaves fewer than
-        // about 1300 waves with any points at all (measured per call, cutoff 5, full lists, shares of 32 / 16 / 8 / 4
-        // / 2 points: 10,000 atoms at 0.05 per cubic A 116 / 100 / 93 / 100 / 127 us, at 0.1 137 / 125 / 101 / 108 /
-        // 115 us; 4,000 atoms 101 / 85 / 76 / 74 / 86 and 125 / 122 / 94 / 82 / 81 us). Shares that most tiles have
-        // no points for cost next to nothing in time, their waves leave at once, but each has room for its
-        // candidates' records: the entry point that allocates nothing keeps the coarser shares below.
-        ordered_points_per_item = filled_cells * std::ceil(mean_per_cell / 8.0) < 1300.0 ? 4 : 8;
-    }
-    // the smallest systems: as many waves as the GPU runs at once, down to one point each
-    while (ordered_points_per_item > 1 && tiles_bound * (TILE_POINTS / ordered_points_per_item) < 2048) {
-        ordered_points_per_item /= 2;
-    }
+    static_assert(ORDERED_TILE_POINTS == TILE_POINTS, "policy.hpp and the kernels agree on the size of a tile");
+    uint32_t ordered_points_per_item = ordered_share(n_points, n_cells, tiles_bound, extras.fixed_memory);
     if (const char* text = std::getenv("VESIN_HIP_ORDERED_SHARE")) {
         // (for measurements and tests: a power of two)
         uint32_t wanted = static_cast<uint32_t>(std::max(1, std::min<int>(TILE_POINTS, std::atoi(text))));
@@ -1480,43 +1464,16 @@ bool compute(
         oargs.items_per_tile = ordered_items_per_tile;
         oargs.rows_of_point = rows_of_point;
         oargs.records = candidate_records;
-        // The writing pass runs four waves per SIMD: 4096 at a time on this GPU. A system of a few more tiles than that
-        // leaves the stragglers running alone for as long as everything before them took (the 100,000-atom
-        // benchmark: 4,260 tiles, 188 us where a wave lives 110 us). The points of every tile can be dealt to two or
-        // four waves instead, which brings the work in shorter pieces; the waves of a tile read the same records
-        // and tables, a fixed cost worth about eight points' rows per wave, so it only pays for well-filled tiles
-        // and up to about three times as many tiles as the GPU holds waves (measured on half lists at 24 points
-        // per tile: 4,500 tiles 357 -> 316 us per call with four waves per tile, 9,000 tiles 567 -> 541 us with
-        // two, 19,000 tiles 911 -> 924 us). Decided from the number of tiles the call before had on the same number
-        // of points; a list's first call on a system keeps one wave per tile.
-        oargs.write_split = 1;
-        if (ordered_items_per_tile == 1 && extras.ordered_tiles_points == n_points && extras.ordered_tiles > 0) {
-            const double slots = 4096.0;
-            const double tiles = static_cast<double>(extras.ordered_tiles);
-            const double per_tile = static_cast<double>(n_points) / tiles;
-            if (per_tile >= 16.0 && tiles > 0.85 * slots && tiles <= 1.5 * slots) {
-                oargs.write_split = 4;
-            } else if (per_tile >= 16.0 && tiles > 1.5 * slots && tiles <= 3.0 * slots) {
-                oargs.write_split = 2;
-            }
-        }
+        // How many waves share a tile in either pass follows the number of tiles the call before had on the same
+        // number of points (policy.hpp); a list's first call on a system keeps one wave per tile.
+        const size_t tiles_before = ordered_items_per_tile == 1 && extras.ordered_tiles_points == n_points ? extras.ordered_tiles : 0;
+        oargs.write_split = ordered_write_split(n_points, tiles_before);
         if (const char* text = std::getenv("VESIN_HIP_WRITE_SPLIT")) {
             oargs.write_split = static_cast<uint32_t>(std::max(1, std::min(4, std::atoi(text))));
         }
-        // The counting pass runs seven waves per SIMD (7168 at a time) and lasts as long as its slowest wave, the
-        // one of the tile with the most points and candidates. While the tiles of a system do not fill those
-        // slots much more than once, the candidates of every well-filled tile are dealt to two waves (pairs of
-        // units of 64 in turn) that add up their rows per point, in memory that the cell build cleared. Measured
-        // per call on half lists, cutoff 6: 24 points per tile, 25,000 / 50,000 / 100,000 / 200,000 atoms 168 -> 155,
-        // 217 -> 201, 312 -> 304, 529 -> 519 us (four waves: 166, 205, 297, 537), 400,000 atoms (17,576 tiles)
-        // 833 -> 841; 12 points per tile, 30,000 / 100,000 atoms 137 -> 143, 275 -> 282 us.
-        oargs.count_split = 1;
+        // (the waves of a tile add their rows in memory that the cell build cleared)
         const bool rows_cleared = !single_cell && !small_build;
-        if (ordered_items_per_tile == 1 && rows_cleared && extras.ordered_tiles_points == n_points &&
-            extras.ordered_tiles > 0 && extras.ordered_tiles <= 9216 &&
-            static_cast<double>(n_points) >= 16.0 * static_cast<double>(extras.ordered_tiles)) {
-            oargs.count_split = 2;
-        }
+        oargs.count_split = rows_cleared ? ordered_count_split(n_points, tiles_before) : 1;
         if (const char* text = std::getenv("VESIN_HIP_COUNT_SPLIT")) {
             oargs.count_split = rows_cleared ? static_cast<uint32_t>(std::max(1, std::min(4, std::atoi(text)))) : 1u;
         }

@@ -63,6 +63,84 @@ struct BoxGuess {
     }
 };
 
+// ---------------------------------------------------------------------------------------------------------------
+// The search that writes a sorted list in order (ordered.cuh): how its work is cut into waves. Every choice gives
+// the same list; the figures are what the passes were measured at on one MI355X (256 compute units, 1024 SIMDs).
+
+constexpr unsigned int ORDERED_TILE_POINTS = 32; // the points a tile holds at most (TILE_POINTS of the kernels)
+
+/// Points of a tile that one wave of the counting and the writing pass takes (a power of two, at most 32).
+///
+/// Large systems: a whole tile, and the candidates of every tile are put in order once by a launch of its own.
+/// Systems of fewer than 2048 occupied cells (up to 3072 at 12 points per cell or fewer) are latency, not throughput:
+/// either pass lasts as long as its slowest wave, which grows with the points the wave writes the rows of. Shares of
+/// 8 points, of 4 where 8 would leave fewer than about 1300 waves with any points at all (per call, cutoff 5, full
+/// lists, shares of 32 / 16 / 8 / 4 / 2 points: 10,000 atoms at 0.05 per cubic A 116 / 100 / 93 / 100 / 127 us, at
+/// 0.1 137 / 125 / 101 / 108 / 115 us; 4,000 atoms 101 / 85 / 76 / 74 / 86 and 125 / 122 / 94 / 82 / 81 us). Shares
+/// that most tiles have no points for cost next to nothing in time, their waves leave at once, but each has room for
+/// its candidates' records: a caller with a fixed amount of work memory (`coarse`) keeps the rule for the smallest
+/// systems only, which halves the share until every possible share of every tile slot makes 2048 waves.
+inline unsigned int ordered_share(size_t n_points, size_t n_cells, size_t tile_slots, bool coarse) {
+    unsigned int share = ORDERED_TILE_POINTS;
+    const size_t occupied = n_cells < n_points ? n_cells : n_points;
+    const double filled = occupied < 1 ? 1.0 : static_cast<double>(occupied);
+    double mean = static_cast<double>(n_points) / filled;
+    if (mean > ORDERED_TILE_POINTS) {
+        mean = ORDERED_TILE_POINTS;
+    }
+    if (!coarse && (filled < 2048.0 || (filled < 3072.0 && mean <= 12.0))) {
+        const double shares_of_eight = mean <= 8.0 ? 1.0 : (mean <= 16.0 ? 2.0 : (mean <= 24.0 ? 3.0 : 4.0));
+        share = filled * shares_of_eight < 1300.0 ? 4 : 8;
+    }
+    while (share > 1 && tile_slots * (ORDERED_TILE_POINTS / share) < 2048) {
+        share /= 2;
+    }
+    return share;
+}
+
+/// Waves that share the points of a tile in the writing pass (1, 2 or 4), from the number of tiles the call before
+/// had on the same points (0: not known, one wave).
+///
+/// The pass keeps four waves per SIMD resident, 4096 on this GPU. A system of a few more tiles than that leaves the
+/// stragglers running alone for as long as everything before them took (100,000 atoms, 4,260 tiles: 172 us where a
+/// wave lives 110 us; two waves per tile 142 us, four 133 us). The waves of a tile read the same records, a fixed
+/// cost worth about eight points' rows each, so it only pays for well-filled tiles and up to about three times as
+/// many tiles as resident waves (half lists at 24 points per tile, per call: 4,500 tiles 357 -> 316 us with four
+/// waves, 9,000 tiles 567 -> 541 us with two, 19,000 tiles 911 -> 924 us; 12 points per tile, 8,000 tiles: 281 ->
+/// 302 us).
+inline unsigned int ordered_write_split(size_t n_points, size_t tiles_before) {
+    if (tiles_before == 0) {
+        return 1;
+    }
+    const double resident = 4096.0;
+    const double tiles = static_cast<double>(tiles_before);
+    if (static_cast<double>(n_points) < 16.0 * tiles) {
+        return 1;
+    }
+    if (tiles > 0.85 * resident && tiles <= 1.5 * resident) {
+        return 4;
+    }
+    if (tiles > 1.5 * resident && tiles <= 3.0 * resident) {
+        return 2;
+    }
+    return 1;
+}
+
+/// Waves that share the candidates of a tile in the counting pass (1 or 2), decided like the other.
+///
+/// That pass runs seven waves per SIMD (7168 at a time) and lasts as long as its slowest wave, the one of the tile
+/// with the most points and candidates. While the tiles of a system do not fill those slots much more than once, the
+/// candidates of every well-filled tile are dealt to two waves, pairs of units of 64 in turn, that add up their rows
+/// per point (half lists, cutoff 6, per call: 24 points per tile, 25,000 / 50,000 / 100,000 / 200,000 atoms 168 ->
+/// 155, 217 -> 201, 312 -> 304, 529 -> 519 us; 400,000 atoms, 17,576 tiles: 833 -> 841 us; 12 points per tile,
+/// 30,000 / 100,000 atoms: 137 -> 143, 275 -> 282 us).
+inline unsigned int ordered_count_split(size_t n_points, size_t tiles_before) {
+    if (tiles_before == 0 || tiles_before > 9216) {
+        return 1;
+    }
+    return static_cast<double>(n_points) >= 16.0 * static_cast<double>(tiles_before) ? 2 : 1;
+}
+
 } // namespace vesin_hip
 
 #endif
