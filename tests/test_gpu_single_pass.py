@@ -164,11 +164,17 @@ def test_crowded_tiles_are_left_to_the_write_pass(timings, capfd, monkeypatch):
     first = call(calculator, points, box, True)
     monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
     capfd.readouterr()
+    # (the list's first call with arrays tries the cell build with 32 slots per cell, which the blob overflows: the
+    # call starts over with the packed build and the two passes, and the list stays away from that build)
+    learning = call(calculator, points, box, True)
+    report = [line for line in capfd.readouterr().err.splitlines() if line.startswith("single pass:")]
+    assert report and "one-pass cell build, crowded" in report[-1] and "crowded 0," not in report[-1], report
     second = call(calculator, points, box, True)
     report = [line for line in capfd.readouterr().err.splitlines() if line.startswith("single pass:")]
-    assert report and " deferred 0 " not in report[-1], report
+    assert report and " deferred 0 " not in report[-1] and "packed cells" in report[-1], report
     assert used_single_pass(calculator)
     assert_same_list(first, expected, what="two-pass")
+    assert_same_list(learning, expected, what="after an overflowing cell")
     assert_same_list(second, expected, what="single pass with deferred tiles")
 
 

@@ -241,21 +241,33 @@ struct Carver {
     }
 };
 
-/// Candidates beyond which a cached list is not worth filtering: the direct search writes its rows at more than
-/// half the memory bandwidth, and a filter has to read every candidate on top of writing the same rows. Measured
-/// on jittered diamond (cutoff 5, skin 0.5): the filter takes 0.038 ms against 0.077 ms at 0.2 M candidates,
-/// breaks even near 1.6 M and takes twice the direct search's time at 15 M.
 /// Calls that find the extent of their points first after one that started from the extent of the call before and
 /// found its points somewhere else.
 constexpr int EXTENT_REST = 8;
 
+/// Candidates beyond which a cached list is not worth filtering: the direct search writes its rows at more than
+/// half the memory bandwidth, and a filter has to read every candidate on top of writing the same rows. Measured
+/// on jittered diamond (cutoff 5, skin 0.5): the filter takes 0.038 ms against 0.077 ms at 0.2 M candidates,
+/// breaks even near 1.6 M and takes twice the direct search's time at 15 M.
 constexpr size_t VERLET_MAX_CANDIDATES = size_t(1) << 20;
 
 /// One-pass cell build: slots per cell (one tile: with two the search has as many empty tiles as full ones and
 /// loses more than the build gains) and the mean occupations between which it is tried. A cell that overflows voids
 /// the call's result (the packed build and the two passes start over) and the list stays away from it for long.
+/// The build saves two launches and a pass over the points; what it costs grows with the number of cells, whose 32
+/// slots each are cleared (wrap shifts) and visited by a wave of the search whether filled or not. Per call, cutoff
+/// 5, full lists, packed build -> one-pass build: 3.8 points per cell, 10,000 / 100,000 / 300,000 / 1,000,000 atoms
+/// 55 -> 47, 131 -> 126, 319 -> 318, 937 -> 938 us; 6.3 points per cell, 10,000 / 30,000 / 100,000 / 1,000,000
+/// atoms 58 -> 52, 69 -> 60, 115 -> 109, 641 -> 613 us; 2.5 points per cell, 3,000 / 10,000 / 30,000 / 100,000 atoms
+/// 44 -> 39, 56 -> 49, 80 -> 78, 166 -> 172 us. The entry point that allocates nothing keeps the higher minimum: the
+/// layout takes 32 slots of memory per cell.
 constexpr uint32_t DIRECT_CAPACITY = TILE_POINTS;
-constexpr double DIRECT_MEAN_MIN = 10.0;
+constexpr double DIRECT_MEAN_MIN = 5.0;              // any number of cells
+constexpr double DIRECT_MEAN_MIN_SOME_CELLS = 3.0;   // at most DIRECT_SOME_CELLS cells
+constexpr size_t DIRECT_SOME_CELLS = 65536;
+constexpr double DIRECT_MEAN_MIN_FEW_CELLS = 2.0;    // at most DIRECT_FEW_CELLS cells
+constexpr size_t DIRECT_FEW_CELLS = 16384;
+constexpr double DIRECT_MEAN_MIN_FIXED_MEMORY = 10.0;
 constexpr double DIRECT_MEAN_MAX = 24.0;
 constexpr int DIRECT_REST = 1024;
 
@@ -964,9 +976,13 @@ bool compute(
     }
     // Cells of ordinary occupation: the cells are built in one pass over the points, every cell owning
     // DIRECT_CAPACITY slots (place_direct); only the single-pass search reads that layout.
+    const double direct_mean_min = extras.fixed_memory             ? DIRECT_MEAN_MIN_FIXED_MEMORY
+                                   : n_cells <= DIRECT_FEW_CELLS  ? DIRECT_MEAN_MIN_FEW_CELLS
+                                   : n_cells <= DIRECT_SOME_CELLS ? DIRECT_MEAN_MIN_SOME_CELLS
+                                                                  : DIRECT_MEAN_MIN;
     bool direct_cells = try_single_pass && !single_cell && !ordered_rows() && !packed_cells_only() &&
                         static_cast<double>(n_points) <= DIRECT_MEAN_MAX * static_cast<double>(n_cells) &&
-                        static_cast<double>(n_points) >= DIRECT_MEAN_MIN * static_cast<double>(n_cells) &&
+                        static_cast<double>(n_points) >= direct_mean_min * static_cast<double>(n_cells) &&
                         n_cells * DIRECT_CAPACITY < 0xFFFFFF00ull;
     if (direct_cells && extras.direct_rest > 0) {
         extras.direct_rest -= 1;
