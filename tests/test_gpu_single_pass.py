@@ -407,3 +407,32 @@ def test_cell_build_of_small_systems(n_points, periodic, monkeypatch):
         calculator = NeighborList(cutoff=3.0, full_list=True)
         for repeat in range(3):
             assert_same_list(call(calculator, points, box, list(periodic)), expected, what=f"{mode} call {repeat}")
+
+
+def test_the_one_pass_cell_build_is_tried_again_after_its_rest(capfd, monkeypatch):
+    """A list that met a cell of more than 32 points stays with the packed cell build for 1024 calls that would have
+    taken the one-pass build, and takes that up again afterwards: rows right at every step looked at."""
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    rng = np.random.default_rng(43)
+    box = np.eye(3) * 40.0
+    gas = rng.random((3000, 3)) * 40.0
+    with_blob = gas.copy()
+    with_blob[:300] = rng.random((300, 3)) * 2.0 + 11.0  # 300 points in one or two cells
+    expected = oracle.neighbors(gas, box, True, 4.0, True, False, "ijSdD")
+    expected_blob = oracle.neighbors(with_blob, box, True, 4.0, True, False, "ijSdD")
+    calculator = NeighborList(cutoff=4.0, full_list=True)
+
+    def build_of(result_expected=None, points=gas):
+        capfd.readouterr()
+        result = call(calculator, points, box, True)
+        lines = _single_pass_reports(capfd)
+        if result_expected is not None:
+            assert_same_list(result, result_expected)
+        assert len(lines) == 1, lines
+        return "one-pass" if "one-pass cell build" in lines[0] else "packed"
+
+    call(calculator, gas, box, True)  # sizes the arrays
+    assert build_of(expected) == "one-pass"
+    assert build_of(expected_blob, with_blob) == "one-pass"  # tried, a cell overflowed, the call started over
+    builds = [build_of(expected if step in (0, 1, 500, 1023, 1024, 1029) else None) for step in range(1030)]
+    assert builds[:1024] == ["packed"] * 1024 and builds[1024:] == ["one-pass"] * 6, (builds[:3], builds[1020:])
