@@ -1554,15 +1554,20 @@ bool compute(
         {
             launch_count_and_scan();
             if (early_write) {
+                // (the launch's first wave tells the host what the counting pass found)
+                oargs.publish_to = &extras.mail_device->ordered;
+                oargs.build_status = extras.d_status;
                 mark(T_WRITE_BEGIN);
                 launch_write();
                 mark(T_WRITE);
+                oargs.publish_to = nullptr;
+            } else {
+                hipLaunchKernelGGL(
+                    publish_ordered_status, dim3(1), dim3(1), 0, stream,
+                    ordered_status, first_row_of_point + n_points, extras.d_status, cell_scan + n_cells,
+                    &extras.mail_device->ordered
+                );
             }
-            hipLaunchKernelGGL(
-                publish_ordered_status, dim3(1), dim3(1), 0, stream,
-                ordered_status, first_row_of_point + n_points, extras.d_status, cell_scan + n_cells,
-                &extras.mail_device->ordered
-            );
             extras.wait(stream);
             if (!box_was_right()) {
                 return false;

@@ -89,6 +89,10 @@ struct OrderedArgs {
                                 // system suits this search and the rows fit the `capacity` of the arrays
     uint64_t capacity;
     SearchOutputs out;
+    // WRITE launched before the host has seen what COUNT found: its first wave hands that to the host on the way
+    // (everything is known when WRITE starts), which saves the launch that would do it afterwards.
+    OrderedHostStatus* publish_to;
+    const DeviceStatus* build_status;
 };
 
 /// LDS of one wave. What is known per candidate (hit column, position, original index, shift) stays in the
@@ -409,6 +413,14 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
     const int lane = lane_id();
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     OrderedWaveShared& sh = shared.wave[wave];
+    if (WRITE && args.publish_to != nullptr && blockIdx.x == 0 && threadIdx.x == 0) {
+        OrderedHostStatus report;
+        report.found = *args.status;
+        report.total_rows = args.first_row[g.n_points];
+        report.first_bad_coordinate = args.build_status->first_bad_coordinate;
+        report.n_tiles = static_cast<unsigned int>(args.cell_scan[g.n_cells] >> 32);
+        *args.publish_to = report;
+    }
     if (WRITE && args.guarded != 0) {
         const OrderedStatus found = *args.status;
         const bool suitable = found.max_rows <= ORDERED_MAX_ROWS && found.max_candidates <= ORDERED_CANDIDATES &&
