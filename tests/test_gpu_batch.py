@@ -419,3 +419,54 @@ def test_config3_full_batch_of_4096_replicas():
             per_system.append({"n_pairs": rows, "ijS": int(ijS[s]), "d": int(d[s])})
         assert systems.fingerprints_of_systems(per_system) == golden, call
         del pairs, shifts, distances, ijS, d
+
+
+def test_boxes_are_compared_on_the_device_and_a_change_is_never_missed(capfd, monkeypatch):
+    """A batch whose other inputs are those of the call before starts from the grids it has while a kernel compares
+    the boxes; a box that changed by one bit makes the call start over, and the list then reads the boxes first for
+    32 calls. The rows are the oracle's every time."""
+    import torch
+
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    rng = np.random.default_rng(92)
+    sizes = [40, 25, 60, 33, 48, 52]
+    boxes = [np.diag(6.0 + rng.random(3)) + 0.3 * np.triu(rng.normal(size=(3, 3)), 1).T for _ in sizes]
+    points = [rng.random((n, 3)) @ box for n, box in zip(sizes, boxes)]
+    first_point = np.cumsum([0] + sizes)
+    calculator = NeighborList(cutoff=4.0, full_list=True)
+    started_over = []
+
+    def run(boxes, check=True):
+        capfd.readouterr()
+        outputs, first_pair = calculator.compute_batch(
+            torch.as_tensor(np.concatenate(points), device="cuda:0"), first_point,
+            torch.as_tensor(np.stack(boxes), device="cuda:0"), True, "PSdD",
+        )
+        err = capfd.readouterr().err.splitlines()
+        lines = [line for line in err if line.startswith("single pass (batch):")]
+        started_over.append(any(line.startswith("batch: the boxes are not those of the call before") for line in err))
+        if check:
+            whole = {NAMES[q]: out.cpu().numpy() for q, out in zip("PSdD", outputs)}
+            for s, (p, box) in enumerate(zip(points, boxes)):
+                rows = slice(int(first_pair[s]), int(first_pair[s + 1]))
+                expected = oracle.neighbors(p, box, True, 4.0, True, False, "ijSdD")
+                assert_same_list({k: v[rows] for k, v in whole.items()}, expected, what=f"system {s}")
+        return [("grids of the call before" in line) for line in lines]
+
+    assert run(boxes) == []            # sizes the arrays with the two passes
+    assert run(boxes) == [True]
+    assert run(boxes) == [True]
+    nudged = [box.copy() for box in boxes]
+    nudged[4][1, 1] = np.nextafter(nudged[4][1, 1], 10.0)  # one bit of one box
+    # started from the old grids, found the box changed, started over with the boxes on the host
+    assert run(nudged) == [False] and started_over == [False, False, False, True]
+    guessed = [run(nudged, check=step in (0, 31, 32)) for step in range(34)]
+    assert guessed[:31] == [[False]] * 31 and guessed[32:] == [[True]] * 2, guessed
+    assert not any(started_over[4:])
+    # a box that keeps changing: every wrong guess doubles the time until the next one
+    del started_over[:]
+    for step in range(70):
+        other = [box.copy() for box in nudged]
+        other[0][0, 0] += 1e-3 * (step + 1)
+        assert run(other, check=step % 23 == 0) == [False]
+    assert started_over[0] and sum(started_over) <= 2, started_over

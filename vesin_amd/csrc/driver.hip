@@ -156,6 +156,26 @@ __global__ void publish_ordered_status(
     }
 }
 
+/// Whether the boxes and flags of a batch are, bit for bit, the ones its grids were picked from (kept on the device):
+/// a workgroup that finds a difference says so in the word the host reads (which the host cleared before the launch).
+__global__ __launch_bounds__(BLOCK) void compare_boxes_kernel(
+    const unsigned long long* __restrict__ boxes, const unsigned char* __restrict__ periodic,
+    const unsigned long long* __restrict__ kept_boxes, const unsigned char* __restrict__ kept_periodic,
+    size_t n_systems, unsigned int* changed
+) {
+    bool differs = false;
+    const size_t stride = static_cast<size_t>(gridDim.x) * BLOCK;
+    for (size_t k = static_cast<size_t>(blockIdx.x) * BLOCK + threadIdx.x; k < 9 * n_systems; k += stride) {
+        differs = differs || boxes[k] != kept_boxes[k];
+    }
+    for (size_t k = static_cast<size_t>(blockIdx.x) * BLOCK + threadIdx.x; k < 3 * n_systems; k += stride) {
+        differs = differs || (periodic[k] != 0) != (kept_periodic[k] != 0);
+    }
+    if (differs) {
+        *changed = 1u;
+    }
+}
+
 /// Everything the kernels report to the host, in one block. A list's own block is pinned host memory that the
 /// kernels write into directly; the entry point that allocates nothing keeps the block in device memory and copies
 /// it to the host before every wait (see HipExtras::wait).
@@ -166,6 +186,8 @@ struct Mailbox {
     unsigned char small[128];            // box (72 bytes) + periodic (3 bytes)
     BlockBounds bounds[BOUNDING_BLOCKS]; // one slot per workgroup of the bounding pass
     ShiftRange ranges[SHIFT_RANGE_BLOCKS]; // one slot per workgroup of the sort's range pass
+    unsigned int batch_changed;          // a batch that started from the boxes of the call before: they are others now
+    unsigned int padding;
 };
 
 /// Makes `device` current for a scope and gives the caller's device back afterwards.
@@ -344,6 +366,15 @@ struct BatchSetup {
     const void* d_first_point = nullptr;
     const void* d_cell_base = nullptr;
     uint64_t work_generation = 0;
+    // The boxes and flags the grids were picked from, on the device (9 doubles per system, then 3 bytes per system):
+    // a call may start from the grids it has and let a kernel compare this call's boxes with them, instead of
+    // bringing 75 bytes per system to the host and waiting for them before anything can be launched.
+    DeviceBuffer kept_boxes;
+    bool kept_on_device = false;
+    BoxGuess guess;
+    // where the first rows of the systems land before they are copied into the caller's array (pinned)
+    size_t* first_pair_landing = nullptr;
+    size_t first_pair_capacity = 0;
 };
 
 struct HipExtras {
@@ -408,6 +439,10 @@ struct HipExtras {
         delete verlet;
         work.release();
         sort_work.release();
+        batch.kept_boxes.release();
+        if (batch.first_pair_landing != nullptr) {
+            (void)hipHostFree(batch.first_pair_landing);
+        }
         if (!fixed_memory) {
             if (meetings != nullptr && own_meetings) {
                 (void)hipFree(meetings);
@@ -1947,6 +1982,12 @@ void launch_search_batch(bool full, const SearchArgs& args, hipStream_t stream) 
     }
 }
 
+bool batch_attempt(
+    const double (*points)[3], const size_t* first_point, size_t n_systems, const double (*boxes)[3][3],
+    const bool (*periodic)[3], VesinOptions options, VesinNeighborList& neighbors, size_t* first_pair,
+    HipExtras& extras, bool speculate, hipStream_t stream
+);
+
 } // namespace
 
 void neighbors_batch(
@@ -1999,30 +2040,95 @@ void neighbors_batch(
     extras.timings_valid = false;
     extras.guess.have_box = false; // the work buffers of the single-system path are about to be reused
     hipStream_t stream = static_cast<hipStream_t>(caller_stream);
-    const size_t pair_limit = pairs_per_point_limit();
-
-    // ---- every system's box comes to the host: the grids are picked there
-    BatchSetup& setup = extras.batch;
-    setup.incoming_boxes.resize(9 * n_systems);
-    setup.incoming_periodic.resize(3 * n_systems);
-    HIP_CHECK(hipMemcpyAsync(
-        setup.incoming_boxes.data(), boxes, setup.incoming_boxes.size() * sizeof(double), hipMemcpyDeviceToHost, stream
-    ));
-    HIP_CHECK(hipMemcpyAsync(
-        setup.incoming_periodic.data(), periodic, setup.incoming_periodic.size(), hipMemcpyDeviceToHost, stream
-    ));
-    HIP_CHECK(hipStreamSynchronize(stream));
 
     // The grids follow from the boxes, the flags, the division into systems, the cutoff and the algorithm alone,
     // unless some direction is open: then they also follow the points. Same inputs as the call before: same grids.
-    const bool same_setup =
-        setup.valid && !setup.any_open_direction && setup.cutoff == options.cutoff &&
+    // Whether the boxes and flags are the same is for the device to say, where they live: a call whose other inputs
+    // are those of the call before starts from the grids it has, a kernel compares the boxes on the way, and the
+    // host looks at its answer at the call's last synchronisation (the bookkeeping of the single-system path:
+    // BoxGuess). Otherwise, and after a wrong guess, the boxes come to the host first.
+    BatchSetup& setup = extras.batch;
+    const BoxKey key = {n_points, options.cutoff, static_cast<int>(options.algorithm), options.full, options.sorted};
+    const bool may_guess = setup.guess.begin(key);
+    const bool rest_is_the_same =
+        setup.valid && setup.kept_on_device && !setup.any_open_direction && setup.cutoff == options.cutoff &&
         setup.algorithm == static_cast<int>(options.algorithm) && setup.full_stencil == full_stencil_only() &&
         setup.first_point.size() == n_systems + 1 &&
         std::memcmp(setup.first_point.data(), first_point, (n_systems + 1) * sizeof(size_t)) == 0 &&
-        setup.boxes.size() == setup.incoming_boxes.size() &&
-        std::memcmp(setup.boxes.data(), setup.incoming_boxes.data(), setup.boxes.size() * sizeof(double)) == 0 &&
-        std::memcmp(setup.periodic.data(), setup.incoming_periodic.data(), setup.periodic.size()) == 0;
+        setup.boxes.size() == 9 * n_systems && extras.mail == extras.mail_device;
+    if (may_guess && rest_is_the_same) {
+        bool right = false;
+        std::exception_ptr failure;
+        try {
+            right = batch_attempt(points, first_point, n_systems, boxes, periodic, options, neighbors, first_pair, extras, true, stream);
+        } catch (...) {
+            // the error may be a consequence of boxes that changed
+            failure = std::current_exception();
+            HIP_CHECK(hipStreamSynchronize(stream));
+            right = extras.mail->batch_changed == 0;
+            if (right) {
+                std::rethrow_exception(failure);
+            }
+        }
+        if (right) {
+            setup.guess.was_right();
+            return;
+        }
+        setup.guess.was_wrong();
+        if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
+            std::fprintf(stderr, "batch: the boxes are not those of the call before, the call starts over\n");
+        }
+    }
+    (void)batch_attempt(points, first_point, n_systems, boxes, periodic, options, neighbors, first_pair, extras, false, stream);
+    setup.guess.have_box = setup.kept_on_device;
+    setup.guess.stored(key);
+}
+
+namespace {
+
+/// The batch itself. `speculate`: from the grids of the call before, with the boxes compared on the device; false is
+/// returned when they turned out to be others (nothing of the result is to be used then).
+bool batch_attempt(
+    const double (*points)[3], const size_t* first_point, size_t n_systems, const double (*boxes)[3][3],
+    const bool (*periodic)[3], VesinOptions options, VesinNeighborList& neighbors, size_t* first_pair,
+    HipExtras& extras, bool speculate, hipStream_t stream
+) {
+    const size_t n_points = first_point[n_systems];
+    const size_t pair_limit = pairs_per_point_limit();
+    BatchSetup& setup = extras.batch;
+
+    bool same_setup = false;
+    if (speculate) {
+        const auto* kept = static_cast<const unsigned char*>(setup.kept_boxes.ptr);
+        extras.mail->batch_changed = 0; // (pinned memory, written before the launch is queued)
+        const uint32_t compare_blocks = static_cast<uint32_t>(std::min<size_t>(256, (9 * n_systems + BLOCK - 1) / BLOCK));
+        hipLaunchKernelGGL(
+            compare_boxes_kernel, dim3(compare_blocks), dim3(BLOCK), 0, stream,
+            reinterpret_cast<const unsigned long long*>(boxes), reinterpret_cast<const unsigned char*>(periodic),
+            reinterpret_cast<const unsigned long long*>(kept), kept + 72 * n_systems, n_systems,
+            &extras.mail_device->batch_changed
+        );
+        same_setup = true;
+    } else {
+        // ---- every system's box comes to the host: the grids are picked there
+        setup.incoming_boxes.resize(9 * n_systems);
+        setup.incoming_periodic.resize(3 * n_systems);
+        HIP_CHECK(hipMemcpyAsync(
+            setup.incoming_boxes.data(), boxes, setup.incoming_boxes.size() * sizeof(double), hipMemcpyDeviceToHost, stream
+        ));
+        HIP_CHECK(hipMemcpyAsync(
+            setup.incoming_periodic.data(), periodic, setup.incoming_periodic.size(), hipMemcpyDeviceToHost, stream
+        ));
+        HIP_CHECK(hipStreamSynchronize(stream));
+        same_setup =
+            setup.valid && !setup.any_open_direction && setup.cutoff == options.cutoff &&
+            setup.algorithm == static_cast<int>(options.algorithm) && setup.full_stencil == full_stencil_only() &&
+            setup.first_point.size() == n_systems + 1 &&
+            std::memcmp(setup.first_point.data(), first_point, (n_systems + 1) * sizeof(size_t)) == 0 &&
+            setup.boxes.size() == setup.incoming_boxes.size() &&
+            std::memcmp(setup.boxes.data(), setup.incoming_boxes.data(), setup.boxes.size() * sizeof(double)) == 0 &&
+            std::memcmp(setup.periodic.data(), setup.incoming_periodic.data(), setup.periodic.size()) == 0;
+    }
 
     std::vector<GridParams>& grids = setup.grids;
     std::vector<uint32_t>& cell_base_host = setup.cell_base;
@@ -2030,6 +2136,7 @@ void neighbors_batch(
     if (!same_setup) {
         setup.valid = false;
         setup.on_device = false;
+        setup.kept_on_device = false;
         setup.boxes.swap(setup.incoming_boxes);
         setup.periodic.swap(setup.incoming_periodic);
         setup.first_point.assign(first_point, first_point + n_systems + 1);
@@ -2144,6 +2251,14 @@ void neighbors_batch(
         setup.most_units = most_units;
         setup.valid = true;
     }
+    if (!setup.kept_on_device) {
+        // what the next call's boxes are compared with
+        setup.kept_boxes.reserve(75 * n_systems);
+        auto* kept = static_cast<unsigned char*>(setup.kept_boxes.ptr);
+        HIP_CHECK(hipMemcpyAsync(kept, setup.boxes.data(), 72 * n_systems, hipMemcpyHostToDevice, stream));
+        HIP_CHECK(hipMemcpyAsync(kept + 72 * n_systems, setup.periodic.data(), 3 * n_systems, hipMemcpyHostToDevice, stream));
+        setup.kept_on_device = true;
+    }
     const uint64_t total_cells = setup.total_cells;
 
     if (n_points == 0) {
@@ -2152,7 +2267,18 @@ void neighbors_batch(
         for (size_t s = 0; s <= n_systems; s++) {
             first_pair[s] = 0;
         }
-        return;
+        return true;
+    }
+    // the first rows of the systems come to pinned memory and go on to the caller's array from there
+    if (setup.first_pair_capacity < n_systems + 1) {
+        if (setup.first_pair_landing != nullptr) {
+            (void)hipHostFree(setup.first_pair_landing);
+            setup.first_pair_landing = nullptr;
+            setup.first_pair_capacity = 0;
+        }
+        const size_t wanted = (n_systems + 1) + (n_systems + 1) / 4;
+        HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&setup.first_pair_landing), wanted * sizeof(size_t), hipHostMallocDefault));
+        setup.first_pair_capacity = wanted;
     }
 
     // ---- work buffers
@@ -2192,6 +2318,7 @@ void neighbors_batch(
     uint32_t* d_first_point = nullptr;
     uint32_t* d_cell_base = nullptr;
     unsigned long long* d_first_pair = nullptr;
+    char* clear_end = nullptr;
     const size_t scratch_elements = std::max(scan_scratch_elements(total_cells), scan_scratch_elements(n_slots));
     auto carve = [&](Carver& carver) {
         // adjacent, so that one fill clears the histogram, the tiles' flags and the state of the single-pass search
@@ -2201,6 +2328,8 @@ void neighbors_batch(
         chain.groups = carver.take<uint64_t>(chain_groups);
         chain.bases = carver.take<uint64_t>(chain_groups);
         fused_status = carver.take<FusedStatus>(1);
+        counts = carver.take<uint32_t>(n_slots);
+        clear_end = reinterpret_cast<char*>(carver.take<uint32_t>(0));
         cell_scan = carver.take<uint64_t>(total_cells + 1);
         cell_of = carver.take<uint32_t>(n_points);
         slot_of = carver.take<uint32_t>(n_points);
@@ -2213,7 +2342,6 @@ void neighbors_batch(
         sorted.wx = carver.take<int32_t>(n_points + SORTED_PADDING);
         sorted.wy = carver.take<int32_t>(n_points + SORTED_PADDING);
         sorted.wz = carver.take<int32_t>(n_points + SORTED_PADDING);
-        counts = carver.take<uint32_t>(n_slots);
         offsets = carver.take<uint64_t>(n_slots + 1);
         scan_scratch = carver.take<uint64_t>(scratch_elements);
         d_grids = carver.take<GridParams>(n_systems);
@@ -2250,14 +2378,16 @@ void neighbors_batch(
     const uint32_t point_blocks = static_cast<uint32_t>((n_points + BLOCK - 1) / BLOCK);
     const uint32_t bounding_blocks = std::min<uint32_t>(BOUNDING_BLOCKS, point_blocks);
     const auto* flat_points = reinterpret_cast<const double*>(points);
-    hipLaunchKernelGGL(
-        fetch_box, dim3(1), dim3(64), 0, stream,
-        reinterpret_cast<const double*>(boxes), reinterpret_cast<const bool*>(periodic), extras.mail_device->small, extras.d_status
-    );
     {
-        const size_t to_clear = reinterpret_cast<char*>(fused_status + 1) - reinterpret_cast<char*>(cell_counts);
-        HIP_CHECK(hipMemsetAsync(cell_counts, 0, to_clear, stream));
-        HIP_CHECK(hipMemsetAsync(counts, 0, n_slots * sizeof(uint32_t), stream));
+        // one launch clears the histogram, the tiles' flags, the state of the single-pass search and the counts, and
+        // resets the status block (every piece of the work buffer is padded to 256 bytes: whole 16-byte blocks)
+        const size_t blocks16 = (clear_end - reinterpret_cast<char*>(cell_counts) + 15) / 16;
+        const uint32_t fill_blocks = static_cast<uint32_t>(std::min<size_t>(1024, (blocks16 + BLOCK - 1) / BLOCK));
+        hipLaunchKernelGGL(
+            clear_and_fetch, dim3(fill_blocks), dim3(BLOCK), 0, stream,
+            reinterpret_cast<uint4*>(cell_counts), blocks16, reinterpret_cast<const double*>(boxes),
+            reinterpret_cast<const bool*>(periodic), extras.mail_device->small, extras.d_status
+        );
     }
     hipLaunchKernelGGL(
         assign_cells_batch, dim3(point_blocks), dim3(BLOCK), 0, stream,
@@ -2318,16 +2448,22 @@ void neighbors_batch(
             cell_scan, d_cell_base, offsets, static_cast<uint32_t>(n_systems), n_slices, static_cast<uint32_t>(n_slots),
             fused_status, d_first_pair
         );
-        HIP_CHECK(hipMemcpyAsync(first_pair, d_first_pair, (n_systems + 1) * sizeof(size_t), hipMemcpyDeviceToHost, stream));
+        HIP_CHECK(hipMemcpyAsync(
+            setup.first_pair_landing, d_first_pair, (n_systems + 1) * sizeof(size_t), hipMemcpyDeviceToHost, stream
+        ));
         HIP_CHECK(hipStreamSynchronize(stream));
+        if (speculate && extras.mail->batch_changed != 0) {
+            return false;
+        }
         const FusedStatus result = extras.mail->fused;
         if (result.first_bad_coordinate != 0xFFFFFFFFu) {
             non_finite_error(points, result.first_bad_coordinate);
         }
         if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
             std::fprintf(
-                stderr, "single pass (batch): rows %llu general %u deferred %u overflow %u timeout %u (slices %u)\n",
-                result.total_rows, result.general, result.deferred, result.overflow, result.chain_timeout, n_slices
+                stderr, "single pass (batch): rows %llu general %u deferred %u overflow %u timeout %u (slices %u%s)\n",
+                result.total_rows, result.general, result.deferred, result.overflow, result.chain_timeout, n_slices,
+                speculate ? ", grids of the call before" : ""
             );
         }
         if (result.general == 0 && result.deferred == 0 && result.overflow == 0 && result.chain_timeout == 0) {
@@ -2340,8 +2476,9 @@ void neighbors_batch(
                 );
             }
             HIP_CHECK(hipGetLastError());
+            std::memcpy(first_pair, setup.first_pair_landing, (n_systems + 1) * sizeof(size_t));
             neighbors.length = result.total_rows;
-            return;
+            return true;
         }
     }
 
@@ -2349,6 +2486,9 @@ void neighbors_batch(
     exclusive_scan<SCAN_U32>(counts, n_slots, offsets, scan_scratch, stream);
     hipLaunchKernelGGL(publish_status, dim3(1), dim3(1), 0, stream, extras.d_status, offsets + n_slots, &extras.mail_device->status);
     HIP_CHECK(hipStreamSynchronize(stream));
+    if (speculate && extras.mail->batch_changed != 0) {
+        return false;
+    }
     if (extras.mail->status.first_bad_coordinate != 0xFFFFFFFFu) {
         non_finite_error(points, extras.mail->status.first_bad_coordinate);
     }
@@ -2388,7 +2528,9 @@ void neighbors_batch(
         cell_scan, d_cell_base, offsets, static_cast<uint32_t>(n_systems), n_slices, static_cast<uint32_t>(n_slots),
         static_cast<const FusedStatus*>(nullptr), d_first_pair
     );
-    HIP_CHECK(hipMemcpyAsync(first_pair, d_first_pair, (n_systems + 1) * sizeof(size_t), hipMemcpyDeviceToHost, stream));
+    HIP_CHECK(hipMemcpyAsync(
+        setup.first_pair_landing, d_first_pair, (n_systems + 1) * sizeof(size_t), hipMemcpyDeviceToHost, stream
+    ));
     if (sorting) {
         // every system's rows stay in their range and come out ordered by (i, j, shift) inside it: the order of
         // vesin_neighbors on that system alone
@@ -2400,10 +2542,10 @@ void neighbors_batch(
     }
     HIP_CHECK(hipStreamSynchronize(stream));
     HIP_CHECK(hipGetLastError());
+    std::memcpy(first_pair, setup.first_pair_landing, (n_systems + 1) * sizeof(size_t));
     neighbors.length = total;
+    return true;
 }
-
-namespace {
 
 // ---- the entry point that allocates nothing
 //
