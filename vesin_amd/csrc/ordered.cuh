@@ -108,8 +108,17 @@ struct OrderedWaveShared: SearchTables {
     uint32_t key_at[ORDERED_MAX_ROWS];
 };
 
+/// LDS of one wave of the counting pass: the tables and the item's points. (A third of what the writing pass takes:
+/// the ordering of the candidates runs beside the counting pass and needs 13 KB per wave itself; with the larger
+/// struct the two kept each other's workgroups waiting for room.)
+struct OrderedCountWaveShared: SearchTables {
+    uint32_t tile_index[TILE_POINTS];
+    double tile_x[TILE_POINTS], tile_y[TILE_POINTS], tile_z[TILE_POINTS];
+};
+
+template <bool WRITE>
 struct OrderedShared {
-    OrderedWaveShared wave[ORDERED_WAVES];
+    std::conditional_t<WRITE, OrderedWaveShared, OrderedCountWaveShared> wave[ORDERED_WAVES];
 };
 
 __device__ __forceinline__ uint32_t biased_shift(int32_t sx, int32_t sy, int32_t sz) {
@@ -193,9 +202,9 @@ __device__ __forceinline__ void sweep_and_count(
 
 /// Two units of candidates (numbers unit0 * 64 ... + 127 of the tables) against the item's points: hit columns
 /// (the item's first point in the highest bit used); lane p of `rows` adds up the hits of the item's point p.
-template <bool FULL, bool WRAPPED>
+template <bool FULL, bool WRAPPED, typename Shared>
 __device__ __forceinline__ void ordered_sweep_pair(
-    const OrderedWaveShared& sh, const SortedPoints& sorted, const GridParams& g, uint32_t unit0, uint32_t n_stencil,
+    const Shared& sh, const SortedPoints& sorted, const GridParams& g, uint32_t unit0, uint32_t n_stencil,
     uint32_t n_candidates, uint32_t first_i, uint32_t n_i, int lane, uint32_t (&column)[ORDERED_R], uint32_t& rows,
     bool& out_of_range, uint32_t (&at)[ORDERED_R], uint32_t (&original)[ORDERED_R], uint32_t (&biased)[ORDERED_R]
 ) {
@@ -409,10 +418,10 @@ __device__ __forceinline__ void write_rows_of_point(
 template <bool WRITE, bool FULL, bool PRESORTED = false>
 __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void ordered_search_kernel(OrderedArgs args, GridParams g) {
     constexpr int R = ORDERED_R;
-    __shared__ OrderedShared shared;
+    __shared__ OrderedShared<WRITE> shared;
     const int lane = lane_id();
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
-    OrderedWaveShared& sh = shared.wave[wave];
+    auto& sh = shared.wave[wave];
     if (WRITE && args.publish_to != nullptr && blockIdx.x == 0 && threadIdx.x == 0) {
         OrderedHostStatus report;
         report.found = *args.status;
@@ -473,7 +482,7 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
         sh.tile_x[lane] = sorted.x[at];
         sh.tile_y[lane] = sorted.y[at];
         sh.tile_z[lane] = sorted.z[at];
-        if (WRITE) {
+        if constexpr (WRITE) {
             sh.tile_wx[lane] = wx;
             sh.tile_wy[lane] = wy;
             sh.tile_wz[lane] = wz;
@@ -554,45 +563,49 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
         return;
     }
 
-    // ---- per place of the tile's order (registers of its lane, indexed by unit): the candidate there, the hit
-    // column the counting pass found for it against this item's points, its original index and its shift (biased,
-    // without the wrap of the first point: that one is added per point, field by field in one integer addition)
-    const uint16_t* tile_order = args.order + static_cast<size_t>(tile_id) * ORDERED_CANDIDATES;
-    uint32_t columns[ORDERED_UNITS];
-    uint32_t cand_index[ORDERED_UNITS];
-    uint32_t cand_biased[ORDERED_UNITS];
+    if constexpr (WRITE) {
+        // ---- per place of the tile's order (registers of its lane, indexed by unit): the candidate there, the hit
+        // column the counting pass found for it against this item's points, its original index and its shift
+        // (biased, without the wrap of the first point: that one is added per point, field by field in one integer
+        // addition)
+        const uint16_t* tile_order = args.order + static_cast<size_t>(tile_id) * ORDERED_CANDIDATES;
+        uint32_t columns[ORDERED_UNITS];
+        uint32_t cand_index[ORDERED_UNITS];
+        uint32_t cand_biased[ORDERED_UNITS];
 #pragma unroll
-    for (int u = 0; u < ORDERED_UNITS; u++) {
-        columns[u] = 0;
-        cand_index[u] = 0;
-        cand_biased[u] = 0;
-        const uint32_t place = u * WAVE + lane;
-        if (static_cast<uint32_t>(u) < n_units && place < n_candidates) {
-            const uint32_t k = PRESORTED ? min(static_cast<uint32_t>(tile_order[place]), n_candidates - 1) : place;
-            const CandidateRecord record = item_records[k]; // one 12-byte load
-            columns[u] = record.column;
-            cand_index[u] = record.index;
-            cand_biased[u] = record.biased;
+        for (int u = 0; u < ORDERED_UNITS; u++) {
+            columns[u] = 0;
+            cand_index[u] = 0;
+            cand_biased[u] = 0;
+            const uint32_t place = u * WAVE + lane;
+            if (static_cast<uint32_t>(u) < n_units && place < n_candidates) {
+                const uint32_t k = PRESORTED ? min(static_cast<uint32_t>(tile_order[place]), n_candidates - 1) : place;
+                const CandidateRecord record = item_records[k]; // one 12-byte load
+                columns[u] = record.column;
+                cand_index[u] = record.index;
+                cand_biased[u] = record.biased;
+            }
+            if (u % 4 == 3) {
+                // four units' loads in flight at a time: with all sixteen, their addresses alone take 32 registers
+                // (reading the places of all units first and then the records, eight at a time, took as long)
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
-        if (u % 4 == 3) {
-            // four units' loads in flight at a time: with all sixteen, their addresses alone take 32 registers
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    }
 
-    // ---- WRITE: point by point, collect the hits in lane order, rank them where that is not their final order,
-    // store the rows
-    wave_sync();
-    const uint32_t per_part = (n_i + split - 1) / split;
-    for (uint32_t p = part * per_part; p < min(n_i, (part + 1) * per_part); p++) {
-        // every field of the sum stays inside its ten bits (operands within +-255), so the fields add independently
-        const uint32_t wrap_i = (static_cast<uint32_t>(sh.tile_wx[p]) << 20) + (static_cast<uint32_t>(sh.tile_wy[p]) << 10) +
-                                static_cast<uint32_t>(sh.tile_wz[p]);
-        // (the second points are looked up by their original index: no position to keep per candidate)
-        write_rows_of_point<PRESORTED>(
-            sh, PointsByIndex{args.points}, g, args.out, columns, cand_index, cand_index, cand_biased, n_units, n_i - 1 - p, wrap_i,
-            sh.tile_x[p], sh.tile_y[p], sh.tile_z[p], sh.tile_index[p], sh.tile_row[p], lane
-        );
+        // ---- WRITE: point by point, collect the hits in lane order, rank them where that is not their final order,
+        // store the rows
+        wave_sync();
+        const uint32_t per_part = (n_i + split - 1) / split;
+        for (uint32_t p = part * per_part; p < min(n_i, (part + 1) * per_part); p++) {
+            // every field of the sum stays inside its ten bits (operands within +-255), so the fields add independently
+            const uint32_t wrap_i = (static_cast<uint32_t>(sh.tile_wx[p]) << 20) + (static_cast<uint32_t>(sh.tile_wy[p]) << 10) +
+                                    static_cast<uint32_t>(sh.tile_wz[p]);
+            // (the second points are looked up by their original index: no position to keep per candidate)
+            write_rows_of_point<PRESORTED>(
+                sh, PointsByIndex{args.points}, g, args.out, columns, cand_index, cand_index, cand_biased, n_units, n_i - 1 - p, wrap_i,
+                sh.tile_x[p], sh.tile_y[p], sh.tile_z[p], sh.tile_index[p], sh.tile_row[p], lane
+            );
+        }
     }
 }
 
