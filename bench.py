@@ -41,12 +41,12 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes moved by ONE launch of the single-pass search kernel on the 1M-atom workload, from rocprofv3 --pmc
-# FETCH_SIZE and WRITE_SIZE runs scaled by a device copy of known size (193.4 MB fetched + 3238.1 MB written). The figure belongs to the kernel sources whose
+# FETCH_SIZE and WRITE_SIZE runs scaled by a device copy of known size (167.3 MB fetched + 3238.2 MB written). The figure belongs to the kernel sources whose
 # digest is recorded with it: a run with other sources reports no traffic instead of a stale one.
 SEARCH_KERNEL_TRAFFIC = {
-    "bytes": 3_431_500_000,
+    "bytes": 3_405_400_000,
     "profile": "profiles/fused_search_config1_pmc.txt",
-    "kernel_sources_sha256": "d1fea6f3c34d952ed862143057755cd007ef227cdec64a0cc57f5c2bc442e9be",
+    "kernel_sources_sha256": "049da47c9ab97cf4962a926de641178ab5c88e297b2c67aafb3fd89dd029fd42",
 }
 KERNEL_SOURCES = ["device_common.cuh", "geometry.hpp", "cells.cuh", "search.cuh", "fused.cuh"]
 

@@ -1,6 +1,7 @@
 // Cell-list construction on the GPU: projected bounding box, cell assignment in fractional coordinates,
 // counting sort of the points by cell (histogram -> device-wide scan -> scatter), and the per-cell pass that
-// puts every cell in a canonical order and lays the points out as structure-of-arrays for the search kernel.
+// puts every cell in a canonical order and lays the points out as 32-byte records, cell by cell, for the search
+// kernel.
 //
 // Reference roles replaced: compute_bounding_box (vesin/src/cuda/cell_list.cu:69-133), assign_cell_indices
 // (:279-333), count_particles_per_cell (:335-345), prefix_sum_cells (:347-390), scatter_particles (:392-421);
@@ -26,15 +27,21 @@ struct FusedStatus {
     unsigned int padding;
 };
 
-/// Cell-sorted copy of the points, one array per component: 64 consecutive candidates load coalesced, and four
-/// consecutive points of a tile arrive with one scalar load per component. x, y, z and index are allocated with
-/// SORTED_PADDING extra elements so that those scalar loads may run past the last point.
+/// One cell-sorted point: coordinates and original index in 32 bytes, aligned. A point in arbitrary input order is
+/// stored wherever its cell lies: one 32-byte sector of memory traffic then, where a store per component (and one
+/// for the index) cost four; 64 consecutive candidates still load coalesced (2 KB in a row), and a point of a tile
+/// arrives with one scalar load.
+struct alignas(32) SortedPoint {
+    double x, y, z;
+    uint32_t index; // original point index
+    uint32_t spare;
+};
+
+/// Cell-sorted copy of the points. `p` is allocated with SORTED_PADDING extra elements so that the scalar loads of
+/// four consecutive points may run past the last point; the shifts (rarely non-zero, rarely read) keep an array each.
 struct SortedPoints {
-    double* x;
-    double* y;
-    double* z;
-    uint32_t* index; // original point index
-    int32_t* wx;     // number of box vectors the point was moved by to land inside the box
+    SortedPoint* p;
+    int32_t* wx; // number of box vectors the point was moved by to land inside the box
     int32_t* wy;
     int32_t* wz;
 };
@@ -406,10 +413,7 @@ __global__ __launch_bounds__(BLOCK) void place_direct(
         return;
     }
     const size_t to = static_cast<size_t>(linear) * capacity + k;
-    sorted.index[to] = i;
-    sorted.x[to] = x;
-    sorted.y[to] = y;
-    sorted.z[to] = z;
+    sorted.p[to] = SortedPoint{x, y, z, i, 0u};
     if ((wrap[0] | wrap[1] | wrap[2]) != 0) {
         // (the caller hands the wrap arrays over cleared, as for place_points)
         sorted.wx[to] = wrap[0];
@@ -432,7 +436,7 @@ __global__ __launch_bounds__(BLOCK) void scatter_points(
     provisional[start + slot_of[i]] = i;
 }
 
-/// Counting-sort scatter straight into the structure-of-arrays layout, for callers that do not need the order of
+/// Counting-sort scatter straight into the cell-sorted records, for callers that do not need the order of
 /// the points inside a cell to be the same on every run: the slot handed out by the histogram atomic is final.
 /// Also appends the cell's tiles. `tiles[].wrapped` must be zero on entry. Cell and wrap shift of the point come
 /// from `cell_of` / `wrap_of` when given (a batch of systems), else the point is located again with `g`: cheaper
@@ -485,10 +489,7 @@ __global__ __launch_bounds__(BLOCK) void place_points(
     // in a batch (system_of not null) the index counts from the first point of the point's system, and the tile
     // carries the system above its flag bit
     const uint32_t system = system_of != nullptr ? system_of[i] : 0;
-    sorted.index[to] = system_of != nullptr ? i - first_point[system] : i;
-    sorted.x[to] = x;
-    sorted.y[to] = y;
-    sorted.z[to] = z;
+    sorted.p[to] = SortedPoint{x, y, z, system_of != nullptr ? i - first_point[system] : i, 0u};
     const uint32_t tile_size = tile_size_of(count);
     // A single system's caller hands the wrap arrays over cleared: points in arbitrary order scatter their stores, a
     // 32-byte sector of memory traffic for each, and most points were not moved by any box vector.
@@ -647,7 +648,7 @@ constexpr uint32_t CANONICAL_LIMIT = 4096;
 
 /// One thread per slot of the counting sort. The atomics of assign_cells leave the points of a cell in arbitrary
 /// order; here every point is ranked by original index among the points of its cell (so the whole pipeline is
-/// deterministic), gathered into the structure-of-arrays layout, and the first point of every run of 32 appends
+/// deterministic), gathered into the cell-sorted records, and the first point of every run of 32 appends
 /// the tile to the tile list. Work is proportional to the number of points, whatever the number of empty cells.
 /// `tiles[].wrapped` must be zero on entry: points moved by a box vector set it with an atomic.
 __global__ __launch_bounds__(BLOCK) void gather_points(
@@ -679,10 +680,10 @@ __global__ __launch_bounds__(BLOCK) void gather_points(
     const int32_t wx = wrap_of[3 * static_cast<size_t>(mine) + 0];
     const int32_t wy = wrap_of[3 * static_cast<size_t>(mine) + 1];
     const int32_t wz = wrap_of[3 * static_cast<size_t>(mine) + 2];
-    sorted.index[to] = mine;
-    sorted.x[to] = points[3 * static_cast<size_t>(mine) + 0];
-    sorted.y[to] = points[3 * static_cast<size_t>(mine) + 1];
-    sorted.z[to] = points[3 * static_cast<size_t>(mine) + 2];
+    sorted.p[to] = SortedPoint{
+        points[3 * static_cast<size_t>(mine) + 0], points[3 * static_cast<size_t>(mine) + 1],
+        points[3 * static_cast<size_t>(mine) + 2], mine, 0u
+    };
     sorted.wx[to] = wx;
     sorted.wy[to] = wy;
     sorted.wz[to] = wz;
@@ -819,10 +820,7 @@ __global__ __launch_bounds__(SMALL_BUILD_THREADS) void build_cells_small(
             const uint32_t first_tile = static_cast<uint32_t>(here >> 32);
             const uint32_t count = cell_count[cell_of[k]];
             const uint32_t to = start + slot_of[k];
-            sorted.index[to] = i;
-            sorted.x[to] = x[k];
-            sorted.y[to] = y[k];
-            sorted.z[to] = z[k];
+            sorted.p[to] = SortedPoint{x[k], y[k], z[k], i, 0u};
             sorted.wx[to] = wx[k];
             sorted.wy[to] = wy[k];
             sorted.wz[to] = wz[k];
@@ -893,10 +891,7 @@ __global__ __launch_bounds__(BLOCK) void prepare_single_cell(
             atomicMin(&status->first_bad_coordinate, 3u * i + axis);
         }
         wrapped = (wrap[0] | wrap[1] | wrap[2]) != 0;
-        sorted.index[i] = i;
-        sorted.x[i] = x;
-        sorted.y[i] = y;
-        sorted.z[i] = z;
+        sorted.p[i] = SortedPoint{x, y, z, i, 0u};
         sorted.wx[i] = wrap[0];
         sorted.wy[i] = wrap[1];
         sorted.wz[i] = wrap[2];

@@ -1141,10 +1141,7 @@ bool compute(
             wrap_of = carver.take<int32_t>(3 * n_points);
             provisional = carver.take<uint32_t>(n_points);
         }
-        sorted.x = carver.take<double>(sorted_slots + SORTED_PADDING);
-        sorted.y = carver.take<double>(sorted_slots + SORTED_PADDING);
-        sorted.z = carver.take<double>(sorted_slots + SORTED_PADDING);
-        sorted.index = carver.take<uint32_t>(sorted_slots + SORTED_PADDING);
+        sorted.p = carver.take<SortedPoint>(sorted_slots + SORTED_PADDING);
         counts = carver.take<uint32_t>(std::max(n_slots, direct_slots * n_slices));
         offsets = carver.take<uint64_t>(std::max(n_slots, direct_slots * n_slices) + 1);
         scan_scratch = carver.take<uint64_t>(scratch_elements);
@@ -2335,10 +2332,7 @@ bool batch_attempt(
         slot_of = carver.take<uint32_t>(n_points);
         system_of = carver.take<uint32_t>(n_points);
         wrap_of = carver.take<int32_t>(3 * n_points);
-        sorted.x = carver.take<double>(n_points + SORTED_PADDING);
-        sorted.y = carver.take<double>(n_points + SORTED_PADDING);
-        sorted.z = carver.take<double>(n_points + SORTED_PADDING);
-        sorted.index = carver.take<uint32_t>(n_points + SORTED_PADDING);
+        sorted.p = carver.take<SortedPoint>(n_points + SORTED_PADDING);
         sorted.wx = carver.take<int32_t>(n_points + SORTED_PADDING);
         sorted.wy = carver.take<int32_t>(n_points + SORTED_PADDING);
         sorted.wz = carver.take<int32_t>(n_points + SORTED_PADDING);

@@ -137,15 +137,15 @@ __device__ __forceinline__ uint32_t sweep_columns(
     uint32_t total = 0;
     for (uint32_t i0 = 0; i0 < count; i0 += POINTS_PER_LOAD) {
         const uint32_t at = first + i0;
-        const FourPoints p = load_four_points(sorted.x + at, sorted.y + at, sorted.z + at);
+        const FourPoints p = load_four_points(sorted.p + at);
 #pragma unroll
         for (int u = 0; u < POINTS_PER_LOAD; u++) {
             if (u > 0 && i0 + u >= count) {
                 break;
             }
-            const double xi = words_to_double(p.x[2 * u], p.x[2 * u + 1]);
-            const double yi = words_to_double(p.y[2 * u], p.y[2 * u + 1]);
-            const double zi = words_to_double(p.z[2 * u], p.z[2 * u + 1]);
+            const double xi = words_to_double(p.q[u][0], p.q[u][1]);
+            const double yi = words_to_double(p.q[u][2], p.q[u][3]);
+            const double zi = words_to_double(p.q[u][4], p.q[u][5]);
 #pragma unroll
             for (int r = 0; r < R; r++) {
                 double vx = c.x[r] - xi;
@@ -181,7 +181,7 @@ __device__ __forceinline__ uint32_t sweep_columns_wrapped(
     for (uint32_t i0 = 0; i0 < n_i; i0 += POINTS_PER_LOAD) {
         // coordinates and wraps of four points come in through scalar loads, like in sweep_columns
         const uint32_t at0 = first_i + i0;
-        const FourPoints p = load_four_points(sorted.x + at0, sorted.y + at0, sorted.z + at0);
+        const FourPoints p = load_four_points(sorted.p + at0);
         const FourWraps w = load_four_wraps(sorted.wx + at0, sorted.wy + at0, sorted.wz + at0);
 #pragma unroll
         for (int u = 0; u < POINTS_PER_LOAD; u++) {
@@ -189,9 +189,9 @@ __device__ __forceinline__ uint32_t sweep_columns_wrapped(
                 break;
             }
             const uint32_t at = at0 + u;
-            const double xi = words_to_double(p.x[2 * u], p.x[2 * u + 1]);
-            const double yi = words_to_double(p.y[2 * u], p.y[2 * u + 1]);
-            const double zi = words_to_double(p.z[2 * u], p.z[2 * u + 1]);
+            const double xi = words_to_double(p.q[u][0], p.q[u][1]);
+            const double yi = words_to_double(p.q[u][2], p.q[u][3]);
+            const double zi = words_to_double(p.q[u][4], p.q[u][5]);
             const int32_t wix = static_cast<int32_t>(w.x[u]);
             const int32_t wiy = static_cast<int32_t>(w.y[u]);
             const int32_t wiz = static_cast<int32_t>(w.z[u]);
@@ -578,10 +578,10 @@ __global__ __launch_bounds__(SEARCH_BLOCK) __attribute__((amdgpu_waves_per_eu(5,
             } else {
                 if (static_cast<uint32_t>(lane) < item.n_i) {
                     const uint32_t at = item.first_i + lane;
-                    sh.tile_x[lane] = sorted.x[at];
-                    sh.tile_y[lane] = sorted.y[at];
-                    sh.tile_z[lane] = sorted.z[at];
-                    sh.tile_index[lane] = sorted.index[at];
+                    sh.tile_x[lane] = sorted.p[at].x;
+                    sh.tile_y[lane] = sorted.p[at].y;
+                    sh.tile_z[lane] = sorted.p[at].z;
+                    sh.tile_index[lane] = sorted.p[at].index;
                     sh.tile_wx[lane] = sorted.wx[at];
                     sh.tile_wy[lane] = sorted.wy[at];
                     sh.tile_wz[lane] = sorted.wz[at];
@@ -616,9 +616,9 @@ __global__ __launch_bounds__(SEARCH_BLOCK) __attribute__((amdgpu_waves_per_eu(5,
                         c.tx[r] = c.ty[r] = c.tz[r] = 0.0;
                         c.position[r] = 0xFFFFFFFFu;
                         if (u.valid) {
-                            c.x[r] = sorted.x[u.at];
-                            c.y[r] = sorted.y[u.at];
-                            c.z[r] = sorted.z[u.at];
+                            c.x[r] = sorted.p[u.at].x;
+                            c.y[r] = sorted.p[u.at].y;
+                            c.z[r] = sorted.p[u.at].z;
                             if (u.same_cell) {
                                 c.position[r] = u.at;
                             }
@@ -761,10 +761,10 @@ __global__ __launch_bounds__(SEARCH_BLOCK) __attribute__((amdgpu_waves_per_eu(5,
         const UnitCandidates u = locate_unit(sh, item.n_batch, item.n_candidates, k, sorted);
         if (u.valid) {
             const int record = half * WAVE + lane;
-            sh.cand_x[record] = sorted.x[u.at];
-            sh.cand_y[record] = sorted.y[u.at];
-            sh.cand_z[record] = sorted.z[u.at];
-            sh.cand_index[record] = sorted.index[u.at];
+            sh.cand_x[record] = sorted.p[u.at].x;
+            sh.cand_y[record] = sorted.p[u.at].y;
+            sh.cand_z[record] = sorted.p[u.at].z;
+            sh.cand_index[record] = sorted.p[u.at].index;
             sh.cand_shift[record] = pack_shift(u.bx, u.by, u.bz);
         }
         wave_sync();

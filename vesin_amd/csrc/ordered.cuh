@@ -130,14 +130,6 @@ __device__ __forceinline__ bool beyond(int32_t a, int32_t b, int32_t c, int32_t 
     return a > limit || a < -limit || b > limit || b < -limit || c > limit || c < -limit;
 }
 
-/// Original indices of four consecutive cell-sorted points in scalar registers (wave-uniform address; reading
-/// past the end of a tile is harmless: the arrays are padded).
-__device__ __forceinline__ uint4 load_four_indices(const uint32_t* index) {
-    uint4 four;
-    asm volatile("s_load_dwordx4 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=&s"(four) : "s"(index));
-    return four;
-}
-
 /// sweep_columns for the counting pass of the in-order search, for a tile without wrapped points: what the
 /// distance test does not decide is decided per test as well, and the rows of every point are counted on the way.
 ///   - candidate lanes whose `c.position` is the position of the point under test sit out: a point is no
@@ -231,10 +223,10 @@ __device__ __forceinline__ void ordered_sweep_pair(
             locate_candidate(sh, n_stencil, k, at[r], packed_q[r]);
             int32_t qx, qy, qz;
             unpack_shift(packed_q[r], qx, qy, qz);
-            c.x[r] = sorted.x[at[r]];
-            c.y[r] = sorted.y[at[r]];
-            c.z[r] = sorted.z[at[r]];
-            original[r] = sorted.index[at[r]];
+            c.x[r] = sorted.p[at[r]].x;
+            c.y[r] = sorted.p[at[r]].y;
+            c.z[r] = sorted.p[at[r]].z;
+            original[r] = sorted.p[at[r]].index;
             bx = qx - sorted.wx[at[r]];
             by = qy - sorted.wy[at[r]];
             bz = qz - sorted.wz[at[r]];
@@ -473,15 +465,15 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
     bool out_of_range = false;
     if (static_cast<uint32_t>(lane) < n_i) {
         const uint32_t at = first_i + lane;
-        const uint32_t original = sorted.index[at];
+        const uint32_t original = sorted.p[at].index;
         sh.tile_index[lane] = original;
         const int32_t wx = sorted.wx[at];
         const int32_t wy = sorted.wy[at];
         const int32_t wz = sorted.wz[at];
         out_of_range = beyond(wx, wy, wz, ORDERED_SHIFT_LIMIT);
-        sh.tile_x[lane] = sorted.x[at];
-        sh.tile_y[lane] = sorted.y[at];
-        sh.tile_z[lane] = sorted.z[at];
+        sh.tile_x[lane] = sorted.p[at].x;
+        sh.tile_y[lane] = sorted.p[at].y;
+        sh.tile_z[lane] = sorted.p[at].z;
         if constexpr (WRITE) {
             sh.tile_wx[lane] = wx;
             sh.tile_wy[lane] = wy;
@@ -694,7 +686,7 @@ __global__ __launch_bounds__(ORDER_BLOCK) void ordered_sort_kernel(OrderedArgs a
         uint32_t at;
         int32_t packed_q;
         locate_candidate(sh, n_stencil, k, at, packed_q);
-        const uint32_t index = sorted.index[at];
+        const uint32_t index = sorted.p[at].index;
         lowest = min(lowest, index);
         highest = max(highest, index);
         if (index >= half) {
@@ -741,7 +733,7 @@ __global__ __launch_bounds__(ORDER_BLOCK) void ordered_sort_kernel(OrderedArgs a
             uint32_t at;
             int32_t packed_q;
             locate_candidate(sh, n_stencil, k, at, packed_q);
-            const uint32_t index = sorted.index[at];
+            const uint32_t index = sorted.p[at].index;
             const uint32_t offset = index >= origin ? index - origin : (g.n_points - origin) + index;
             wrapped_around += index < origin ? 1u : 0u;
             bits.offset[k] = static_cast<uint16_t>(offset % ORDER_BITS);
@@ -833,7 +825,7 @@ __global__ __launch_bounds__(ORDER_BLOCK) void ordered_sort_kernel(OrderedArgs a
         uint32_t at;
         int32_t packed_q;
         locate_candidate(sh, n_stencil, k, at, packed_q);
-        const uint32_t index = sorted.index[at];
+        const uint32_t index = sorted.p[at].index;
         buckets.index_of[k] = index;
         atomicAdd(&buckets.bucket_end[bucket_of(index)], 1u);
     }

@@ -9,7 +9,7 @@
 // a tiled brute force, the candidates of a tile being sliced over several waves.
 //
 // Mapping: lanes hold candidates. A wave loads R groups of 64 consecutive candidates into registers (coalesced
-// reads from the cell-sorted structure-of-arrays), then loops over the tile's points, whose coordinates come in
+// reads of the cell-sorted 32-byte records), then loops over the tile's points, whose coordinates come in
 // through scalar loads (four points per round trip) and are used as scalar operands. One (i, group) test is 9 fp64
 // VALU operations (12 when a shift vector has to be added) and yields a 64-bit hit mask in scalar registers. The
 // loop is compiled in four variants (candidates shifted or not, tile's own cell among them or not), picked per
@@ -452,23 +452,25 @@ typedef uint32_t ScalarWords8 __attribute__((ext_vector_type(8)));
 
 constexpr int POINTS_PER_LOAD = 4;
 
-/// Coordinates of four consecutive cell-sorted points, in scalar registers.
+/// Four consecutive cell-sorted points, in scalar registers: words 0-1 x, 2-3 y, 4-5 z, 6 index of each.
 struct FourPoints {
-    ScalarWords8 x, y, z;
+    ScalarWords8 q[POINTS_PER_LOAD];
 };
 
-/// Three scalar loads (s_load_dwordx8) issued back to back and waited for inside one asm statement, so the
-/// compiler never sees the registers before the data arrived. The addresses are wave-uniform. Reading up to three
-/// points past the end of a tile is harmless: the arrays are padded.
-__device__ __forceinline__ FourPoints load_four_points(const double* x, const double* y, const double* z) {
+/// Four scalar loads (s_load_dwordx8, a point each) issued back to back and waited for inside one asm statement, so
+/// the compiler never sees the registers before the data arrived. The address is wave-uniform. Reading up to three
+/// points past the end of a tile is harmless: the array is padded.
+__device__ __forceinline__ FourPoints load_four_points(const SortedPoint* first) {
+    static_assert(sizeof(SortedPoint) == 32, "one s_load_dwordx8 per point");
     FourPoints p;
     asm volatile(
-        "s_load_dwordx8 %0, %3, 0x0\n\t"
-        "s_load_dwordx8 %1, %4, 0x0\n\t"
-        "s_load_dwordx8 %2, %5, 0x0\n\t"
+        "s_load_dwordx8 %0, %4, 0x0\n\t"
+        "s_load_dwordx8 %1, %4, 0x20\n\t"
+        "s_load_dwordx8 %2, %4, 0x40\n\t"
+        "s_load_dwordx8 %3, %4, 0x60\n\t"
         "s_waitcnt lgkmcnt(0)"
-        : "=&s"(p.x), "=&s"(p.y), "=&s"(p.z)
-        : "s"(x), "s"(y), "s"(z)
+        : "=&s"(p.q[0]), "=&s"(p.q[1]), "=&s"(p.q[2]), "=&s"(p.q[3])
+        : "s"(first)
     );
     return p;
 }
@@ -508,16 +510,16 @@ __device__ __forceinline__ void sweep_unwrapped(
 ) {
     for (uint32_t i0 = 0; i0 < n_i; i0 += POINTS_PER_LOAD) {
         const uint32_t at = first_i + i0;
-        const FourPoints p = load_four_points(sorted.x + at, sorted.y + at, sorted.z + at);
+        const FourPoints p = load_four_points(sorted.p + at);
 #pragma unroll
         for (int u = 0; u < POINTS_PER_LOAD; u++) {
             if (u > 0 && i0 + u >= n_i) {
                 break;
             }
             const uint32_t i = i0 + u;
-            const double xi = words_to_double(p.x[2 * u], p.x[2 * u + 1]);
-            const double yi = words_to_double(p.y[2 * u], p.y[2 * u + 1]);
-            const double zi = words_to_double(p.z[2 * u], p.z[2 * u + 1]);
+            const double xi = words_to_double(p.q[u][0], p.q[u][1]);
+            const double yi = words_to_double(p.q[u][2], p.q[u][3]);
+            const double zi = words_to_double(p.q[u][4], p.q[u][5]);
 #pragma unroll
             for (int r = 0; r < R; r++) {
                 double vx = c.x[r] - xi;
@@ -551,9 +553,9 @@ __device__ __forceinline__ void sweep_wrapped(
 ) {
     for (uint32_t i = 0; i < n_i; i++) {
         const uint32_t at = first_i + i;
-        const double xi = sorted.x[at];
-        const double yi = sorted.y[at];
-        const double zi = sorted.z[at];
+        const double xi = sorted.p[at].x;
+        const double yi = sorted.p[at].y;
+        const double zi = sorted.p[at].z;
         const int32_t wix = static_cast<int32_t>(uniform(static_cast<uint32_t>(sorted.wx[at])));
         const int32_t wiy = static_cast<int32_t>(uniform(static_cast<uint32_t>(sorted.wy[at])));
         const int32_t wiz = static_cast<int32_t>(uniform(static_cast<uint32_t>(sorted.wz[at])));
@@ -620,10 +622,7 @@ __device__ __forceinline__ void search_work_item(
     const int32_t cy = (local_cell / g.n[0]) % g.n[1];
     const int32_t cz = local_cell / (g.n[0] * g.n[1]);
 
-    const double* __restrict__ px = args.sorted.x;
-    const double* __restrict__ py = args.sorted.y;
-    const double* __restrict__ pz = args.sorted.z;
-    const uint32_t* __restrict__ pindex = args.sorted.index;
+    const SortedPoint* __restrict__ pp = args.sorted.p;
     const int32_t* __restrict__ pwx = args.sorted.wx;
     const int32_t* __restrict__ pwy = args.sorted.wy;
     const int32_t* __restrict__ pwz = args.sorted.wz;
@@ -631,10 +630,10 @@ __device__ __forceinline__ void search_work_item(
     if constexpr (WRITE) {
         if (static_cast<uint32_t>(lane) < n_i) {
             const uint32_t at = first_i + lane;
-            sh.tile_x[lane] = px[at];
-            sh.tile_y[lane] = py[at];
-            sh.tile_z[lane] = pz[at];
-            sh.tile_index[lane] = pindex[at];
+            sh.tile_x[lane] = pp[at].x;
+            sh.tile_y[lane] = pp[at].y;
+            sh.tile_z[lane] = pp[at].z;
+            sh.tile_index[lane] = pp[at].index;
             sh.tile_wx[lane] = pwx[at];
             sh.tile_wy[lane] = pwy[at];
             sh.tile_wz[lane] = pwz[at];
@@ -694,9 +693,9 @@ __device__ __forceinline__ void search_work_item(
                     int32_t qx, qy, qz;
                     unpack_shift(packed, qx, qy, qz);
                     same_cell = (packed >> 30) & 1;
-                    c.x[r] = px[at];
-                    c.y[r] = py[at];
-                    c.z[r] = pz[at];
+                    c.x[r] = pp[at].x;
+                    c.y[r] = pp[at].y;
+                    c.z[r] = pp[at].z;
                     c.bx[r] = qx - pwx[at];
                     c.by[r] = qy - pwy[at];
                     c.bz[r] = qz - pwz[at];
@@ -708,7 +707,7 @@ __device__ __forceinline__ void search_work_item(
                         sh.cand_x[slot] = c.x[r];
                         sh.cand_y[slot] = c.y[r];
                         sh.cand_z[slot] = c.z[r];
-                        sh.cand_index[slot] = pindex[at];
+                        sh.cand_index[slot] = pp[at].index;
                         sh.cand_bx[slot] = c.bx[r];
                         sh.cand_by[slot] = c.by[r];
                         sh.cand_bz[slot] = c.bz[r];
