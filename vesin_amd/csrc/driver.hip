@@ -342,21 +342,55 @@ struct VerletCache {
 /// What the host derives from the boxes of a batch of systems, kept between calls: a batch whose boxes, flags and
 /// division into systems are those of the call before (a trajectory at constant volume, the same set of structures
 /// evaluated again) starts its kernels without the host going over the systems one by one again.
+/// Host memory the GPU copies from and to directly (hipHostMalloc): a copy between device memory and an ordinary
+/// std::vector goes through a staging buffer of the runtime's and waits for it, several times per batch.
+template <typename T>
+struct PinnedAllocator {
+    using value_type = T;
+    PinnedAllocator() = default;
+    template <typename U>
+    PinnedAllocator(const PinnedAllocator<U>&) {}
+    T* allocate(size_t n) {
+        void* ptr = nullptr;
+        if (hipHostMalloc(&ptr, n * sizeof(T), hipHostMallocDefault) != hipSuccess) {
+            (void)hipGetLastError();
+            throw std::bad_alloc();
+        }
+        return static_cast<T*>(ptr);
+    }
+    void deallocate(T* ptr, size_t) {
+        (void)hipHostFree(ptr);
+    }
+    template <typename U>
+    bool operator==(const PinnedAllocator<U>&) const {
+        return true;
+    }
+    template <typename U>
+    bool operator!=(const PinnedAllocator<U>&) const {
+        return false;
+    }
+};
+
+template <typename T>
+using PinnedVector = std::vector<T, PinnedAllocator<T>>;
+
 struct BatchSetup {
     bool valid = false;
     bool any_open_direction = false;
     double cutoff = 0.0;
     int algorithm = 0;
     bool full_stencil = false;              // VESIN_HIP_STENCIL=full was set
-    std::vector<double> boxes;              // 9 per system, as the caller gave them
-    std::vector<unsigned char> periodic;    // 3 per system
-    std::vector<double> incoming_boxes;     // where a call's boxes land before they are compared
-    std::vector<unsigned char> incoming_periodic;
+    // (what is copied from or to the device lives in pinned memory)
+    PinnedVector<double> boxes;              // 9 per system, as the caller gave them
+    PinnedVector<unsigned char> periodic;    // 3 per system
+    PinnedVector<double> incoming_boxes;     // where a call's boxes land before they are compared
+    PinnedVector<unsigned char> incoming_periodic;
     std::vector<size_t> first_point;
     std::vector<HostBox> host_boxes;        // normalised
-    std::vector<GridParams> grids;
-    std::vector<uint32_t> cell_base;
-    std::vector<uint32_t> first_point32;
+    PinnedVector<GridParams> grids;
+    PinnedVector<uint32_t> cell_base;
+    PinnedVector<uint32_t> first_point32;
+    PinnedVector<BlockBounds> bounds;        // extent of every system's points (systems with an open direction)
     uint64_t total_cells = 0;
     double most_units = 1.0;
     // where the last batch left grids, first points and first cells in the work buffer; a call on a single system
@@ -2127,9 +2161,9 @@ bool batch_attempt(
             std::memcmp(setup.periodic.data(), setup.incoming_periodic.data(), setup.periodic.size()) == 0;
     }
 
-    std::vector<GridParams>& grids = setup.grids;
-    std::vector<uint32_t>& cell_base_host = setup.cell_base;
-    std::vector<uint32_t>& first_point_host = setup.first_point32;
+    PinnedVector<GridParams>& grids = setup.grids;
+    PinnedVector<uint32_t>& cell_base_host = setup.cell_base;
+    PinnedVector<uint32_t>& first_point_host = setup.first_point32;
     if (!same_setup) {
         setup.valid = false;
         setup.on_device = false;
@@ -2140,8 +2174,8 @@ bool batch_attempt(
         setup.cutoff = options.cutoff;
         setup.algorithm = static_cast<int>(options.algorithm);
         setup.full_stencil = full_stencil_only();
-        const std::vector<double>& host_boxes = setup.boxes;
-        const std::vector<unsigned char>& host_periodic = setup.periodic;
+        const PinnedVector<double>& host_boxes = setup.boxes;
+        const PinnedVector<unsigned char>& host_periodic = setup.periodic;
 
         grids.resize(n_systems);
         std::vector<HostBox>& host_grids_box = setup.host_boxes;
@@ -2173,7 +2207,8 @@ bool batch_attempt(
 
         // ---- systems with a non-periodic direction need the extent of their points along it (reference:
         // BoundingBox::make_bounding_for, vesin/src/types.hpp:159-200): one wave per system finds it
-        std::vector<BlockBounds> bounds;
+        PinnedVector<BlockBounds>& bounds = setup.bounds;
+        bounds.clear();
         if (any_open_direction && n_points > 0) {
             const size_t grids_bytes = (n_systems * sizeof(GridParams) + 255) & ~size_t(255);
             const size_t firsts_bytes = ((n_systems + 1) * sizeof(uint32_t) + 255) & ~size_t(255);
@@ -2248,8 +2283,8 @@ bool batch_attempt(
         setup.most_units = most_units;
         setup.valid = true;
     }
-    if (!setup.kept_on_device) {
-        // what the next call's boxes are compared with
+    if (!setup.kept_on_device && !setup.any_open_direction) {
+        // what the next call's boxes are compared with (never with an open direction: the grids follow the points)
         setup.kept_boxes.reserve(75 * n_systems);
         auto* kept = static_cast<unsigned char*>(setup.kept_boxes.ptr);
         HIP_CHECK(hipMemcpyAsync(kept, setup.boxes.data(), 72 * n_systems, hipMemcpyHostToDevice, stream));
