@@ -141,6 +141,65 @@ __global__ __launch_bounds__(BLOCK) void scan_tile_write_few(
     }
 }
 
+/// The whole scan of a short input in one workgroup of 1024 threads, SCAN_ONE_CHUNK elements at a time: one launch
+/// where the tiles of the general scheme take two (a launch and the gap before it cost about as much as the
+/// workgroup needs for all of it).
+constexpr int SCAN_ONE_THREADS = 1024;
+constexpr size_t SCAN_ONE_CHUNK = static_cast<size_t>(SCAN_ONE_THREADS) * SCAN_ITEMS;
+constexpr size_t SCAN_ONE_MAX = 2 * SCAN_ONE_CHUNK;
+
+template <int INPUT>
+__global__ __launch_bounds__(SCAN_ONE_THREADS) void scan_one_workgroup(
+    const void* __restrict__ in, size_t n, uint64_t* __restrict__ out
+) {
+    constexpr int WAVES = SCAN_ONE_THREADS / WAVE;
+    __shared__ uint64_t wave_sums[WAVES];
+    const int lane = lane_id();
+    const int wave = threadIdx.x / WAVE;
+    uint64_t carried = 0;
+    for (size_t chunk = 0; chunk < n; chunk += SCAN_ONE_CHUNK) {
+        const size_t base = chunk + static_cast<size_t>(threadIdx.x) * SCAN_ITEMS;
+        uint64_t items[SCAN_ITEMS];
+        uint64_t local = 0;
+#pragma unroll
+        for (int k = 0; k < SCAN_ITEMS; k++) {
+            const size_t i = base + k;
+            items[k] = i < n ? scan_load<INPUT>(in, i) : 0;
+            local += items[k];
+        }
+        const uint64_t inclusive = wave_inclusive_scan(local);
+        if (lane == WAVE - 1) {
+            wave_sums[wave] = inclusive;
+        }
+        __syncthreads();
+        uint64_t before = 0;
+        uint64_t all = 0;
+#pragma unroll
+        for (int w = 0; w < WAVES; w++) {
+            const uint64_t sum = wave_sums[w];
+            before += w < wave ? sum : 0;
+            all += sum;
+        }
+        __syncthreads();
+        uint64_t running = carried + before + inclusive - local;
+#pragma unroll
+        for (int k = 0; k < SCAN_ITEMS; k++) {
+            const size_t i = base + k;
+            if (i < n) {
+                out[i] = running;
+            }
+            running += items[k];
+            if (i + 1 == n) {
+                out[n] = running;
+            }
+        }
+        carried += all;
+    }
+    if (n == 0 && threadIdx.x == 0) {
+        out[0] = 0;
+    }
+}
+
 inline size_t scan_tiles(size_t n) {
     return n == 0 ? 1 : (n + SCAN_TILE - 1) / SCAN_TILE;
 }
@@ -162,6 +221,10 @@ inline void exclusive_scan(const void* in, size_t n, uint64_t* out, uint64_t* sc
     size_t tiles = scan_tiles(n);
     if (tiles == 1) {
         hipLaunchKernelGGL(scan_tile_write<INPUT>, dim3(1), dim3(BLOCK), 0, stream, in, n, nullptr, out);
+        return;
+    }
+    if (n <= SCAN_ONE_MAX) {
+        hipLaunchKernelGGL(scan_one_workgroup<INPUT>, dim3(1), dim3(SCAN_ONE_THREADS), 0, stream, in, n, out);
         return;
     }
     uint64_t* sums = scratch;
