@@ -470,3 +470,64 @@ def test_boxes_are_compared_on_the_device_and_a_change_is_never_missed(capfd, mo
         other[0][0, 0] += 1e-3 * (step + 1)
         assert run(other, check=step % 23 == 0) == [False]
     assert started_over[0] and sum(started_over) <= 2, started_over
+
+
+@pytest.mark.parametrize("algorithm", ["auto", "cell_list", "brute_force"])
+def test_free_molecules_get_their_grids_on_the_device(algorithm, capfd, monkeypatch):
+    """A batch of systems without any periodic direction: from the second call with arrays on, the grids are picked
+    on the device from the extent of this call's points. Molecules that drift, stretch and collapse, from one atom
+    to a few hundred; the rows are the oracle's every time, and a flag that changes is noticed."""
+    import torch
+
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    rng = np.random.default_rng(93)
+    sizes = [1, 2, 5, 17, 40, 64, 90, 300, 33, 3, 31, 32, 700]
+    molecules = [rng.normal(scale=1.0 + 0.1 * n ** (1 / 3), size=(n, 3)) + rng.uniform(-40, 40, size=3) for n in sizes]
+    first_point = np.cumsum([0] + sizes)
+    boxes = np.zeros((len(sizes), 3, 3))
+    calculator = NeighborList(cutoff=3.2, full_list=True, algorithm=algorithm)
+
+    def run(molecules, flags, check=True):
+        capfd.readouterr()
+        outputs, first_pair = calculator.compute_batch(
+            torch.as_tensor(np.concatenate(molecules), device="cuda:0"), first_point,
+            torch.as_tensor(boxes, device="cuda:0"), flags, "PSdD",
+        )
+        err = capfd.readouterr().err.splitlines()
+        if check:
+            whole = {NAMES[q]: out.cpu().numpy() for q, out in zip("PSdD", outputs)}
+            per_system = np.broadcast_to(np.asarray(flags, dtype=bool), (len(sizes), 3))
+            for s, points in enumerate(molecules):
+                rows = slice(int(first_pair[s]), int(first_pair[s + 1]))
+                box = np.eye(3) * 500.0 if per_system[s].any() else boxes[s]
+                expected = oracle.neighbors(points, box, [bool(f) for f in per_system[s]], 3.2, True, False, "ijSdD")
+                assert_same_list({k: v[rows] for k, v in whole.items()}, expected, what=f"system {s}")
+        return sum("grids picked on the device" in line for line in err)
+
+    assert run(molecules, False) == 0  # sizes the arrays
+    assert run(molecules, False) == 1
+    for step in range(6):
+        if step == 2:
+            molecules = [(m - m.mean(axis=0)) * 2.5 + m.mean(axis=0) for m in molecules]  # stretch
+        elif step == 4:
+            molecules = [(m - m.mean(axis=0)) * 0.2 + m.mean(axis=0) + 300.0 for m in molecules]  # collapse, far away
+        else:
+            molecules = [m + rng.normal(scale=0.2, size=m.shape) for m in molecules]
+        assert run(molecules, False) == 1, step
+    # one system becomes periodic along z: the flags are others, the call starts over with the boxes on the host
+    flags = np.zeros((len(sizes), 3), dtype=bool)
+    flags[4, 2] = True
+    boxes[4] = np.eye(3) * 500.0
+    assert run(molecules, flags) == 0
+    assert run(molecules, flags) == 0
+    # a coordinate that is not finite is reported by the kernels that pick the grids as by any other
+    calculator2 = NeighborList(cutoff=3.2, full_list=True, algorithm=algorithm)
+    calculator, kept = calculator2, calculator
+    boxes[4] = 0.0
+    assert run(molecules, False) == 0
+    assert run(molecules, False) == 1
+    broken = [m.copy() for m in molecules]
+    broken[7][5, 1] = np.nan
+    with pytest.raises(RuntimeError, match="point"):
+        run(broken, False, check=False)
+    assert run(molecules, False) in (0, 1)

@@ -567,6 +567,151 @@ __global__ __launch_bounds__(BLOCK) void bounding_batch_kernel(
     }
 }
 
+/// Grids of a batch whose systems have no periodic direction at all (free molecules), picked where the points are:
+/// one wave per system finds the extent of its points and its first lane picks the grid, as `choose_grid`
+/// (geometry.hpp) does on the host for such a system: the box counts for nothing (the three directions are unit
+/// vectors), cells at least as wide as the cutoff over the extent of the points with a margin of 1 %, never more
+/// cells than twice the points (or 64), nothing beyond the last cell. `single_cell`: 1 always (brute force), 0 for
+/// systems that fill more than a cell and have 32 points or more (automatic choice), -1 never (cell list).
+__global__ __launch_bounds__(BLOCK) void open_grids_kernel(
+    const double* __restrict__ points, const uint32_t* __restrict__ first_point, uint32_t n_systems, double cutoff,
+    int single_cell, GridParams* __restrict__ grids, uint32_t* __restrict__ cells_of_system, unsigned int* first_bad
+) {
+    const uint32_t system = blockIdx.x * WAVES_PER_BLOCK + threadIdx.x / WAVE;
+    if (system >= n_systems) {
+        return;
+    }
+    double lo[3] = {INFINITY, INFINITY, INFINITY};
+    double hi[3] = {-INFINITY, -INFINITY, -INFINITY};
+    unsigned int bad = 0xFFFFFFFFu;
+    const uint32_t begin = first_point[system];
+    const uint32_t end = first_point[system + 1];
+    for (uint32_t i = begin + lane_id(); i < end; i += WAVE) {
+        const double r[3] = {
+            points[3 * static_cast<size_t>(i) + 0], points[3 * static_cast<size_t>(i) + 1],
+            points[3 * static_cast<size_t>(i) + 2]
+        };
+        unsigned int axis;
+        if (!all_finite(r[0], r[1], r[2], axis)) {
+            bad = min(bad, 3u * i + axis);
+            continue;
+        }
+#pragma unroll
+        for (int d = 0; d < 3; d++) {
+            lo[d] = fmin(lo[d], r[d]);
+            hi[d] = fmax(hi[d], r[d]);
+        }
+    }
+#pragma unroll
+    for (int offset = WAVE / 2; offset > 0; offset >>= 1) {
+#pragma unroll
+        for (int d = 0; d < 3; d++) {
+            lo[d] = fmin(lo[d], __shfl_xor(lo[d], offset));
+            hi[d] = fmax(hi[d], __shfl_xor(hi[d], offset));
+        }
+        bad = min(bad, static_cast<unsigned int>(__shfl_xor(static_cast<int>(bad), offset)));
+    }
+    if (lane_id() != 0) {
+        return;
+    }
+    if (bad != 0xFFFFFFFFu) {
+        atomicMin(first_bad, bad);
+    }
+    const uint32_t n_here = end - begin;
+    const double padded = cutoff * (1.0 + 1e-9);
+    GridParams g;
+    for (int k = 0; k < 9; k++) {
+        g.H[k] = (k % 4 == 0) ? 1.0 : 0.0;
+        g.Hinv[k] = (k % 4 == 0) ? 1.0 : 0.0;
+    }
+    double extent[3];
+    for (int d = 0; d < 3; d++) {
+        double width = (n_here > 0 && hi[d] >= lo[d]) ? hi[d] - lo[d] : 0.0;
+        if (!(width >= 1e-6)) {
+            width = 1.0;
+        }
+        extent[d] = fmax(width * 1.01, 1.0);
+        g.np_min[d] = (n_here > 0 && hi[d] >= lo[d]) ? lo[d] : 0.0;
+        g.np_scale[d] = 1.0 / extent[d];
+        g.periodic[d] = 0;
+        g.prune_slack[d] = 0.0;
+    }
+    for (int k = 0; k < 6; k++) {
+        g.prune_edges[k] = 0.0;
+    }
+    g.prune = 0;
+    g.prune_limit = padded * padded;
+    g.cutoff2 = cutoff * cutoff;
+    g.n_points = n_here;
+    bool one_cell = single_cell > 0;
+    for (int attempt = 0; attempt < 2; attempt++) {
+        double cells[3];
+        for (int d = 0; d < 3; d++) {
+            cells[d] = one_cell ? 1.0 : fmin(fmax(floor(extent[d] / padded), 1.0), 1048576.0);
+        }
+        const double most = fmin(fmax(2.0 * static_cast<double>(n_here), 64.0), 16777216.0);
+        const double total = cells[0] * cells[1] * cells[2];
+        if (total > most) {
+            const double shrink = cbrt(most / total);
+            for (int d = 0; d < 3; d++) {
+                cells[d] = fmax(floor(cells[d] * shrink), 1.0);
+            }
+        }
+        uint32_t n_cells = 1;
+        for (int d = 0; d < 3; d++) {
+            g.n[d] = static_cast<int32_t>(cells[d]);
+            n_cells *= static_cast<uint32_t>(g.n[d]);
+            // nothing exists beyond the last cell of a direction that is not periodic
+            const double radius = fmin(fmax(ceil(padded * cells[d] / extent[d]), 1.0), cells[d] - 1.0);
+            g.s[d] = static_cast<int32_t>(radius);
+        }
+        g.n_cells = n_cells;
+        if (single_cell == 0 && !one_cell && (n_cells == 1 || n_here < 32)) {
+            one_cell = true; // too little for a cell list: one cell, every point against every other
+            continue;
+        }
+        break;
+    }
+    grids[system] = g;
+    cells_of_system[system] = g.n_cells;
+}
+
+/// First cell of every system of a batch (exclusive scan of the cells per system, one workgroup), and what the
+/// host wants to know at the end of the call: all cells and the most cells of one system.
+__global__ __launch_bounds__(1024) void open_bases_kernel(
+    const uint32_t* __restrict__ cells_of_system, uint32_t n_systems, uint32_t* __restrict__ cell_base,
+    unsigned long long* __restrict__ total_cells
+) {
+    __shared__ uint64_t wave_sums[16];
+    const int lane = lane_id();
+    const int wave = threadIdx.x / WAVE;
+    uint64_t carried = 0;
+    for (uint32_t chunk = 0; chunk < n_systems; chunk += 1024) {
+        const uint32_t system = chunk + threadIdx.x;
+        const uint64_t own = system < n_systems ? cells_of_system[system] : 0;
+        const uint64_t inclusive = wave_inclusive_scan(own);
+        if (lane == WAVE - 1) {
+            wave_sums[wave] = inclusive;
+        }
+        __syncthreads();
+        uint64_t before = 0;
+        uint64_t all = 0;
+        for (int w = 0; w < 16; w++) {
+            before += w < wave ? wave_sums[w] : 0;
+            all += wave_sums[w];
+        }
+        __syncthreads();
+        if (system < n_systems) {
+            cell_base[system] = static_cast<uint32_t>(carried + before + inclusive - own);
+        }
+        carried += all;
+    }
+    if (threadIdx.x == 0) {
+        cell_base[n_systems] = static_cast<uint32_t>(carried);
+        *total_cells = carried;
+    }
+}
+
 /// assign_cells for many systems at once: every point looks up its system (binary search in `first_point`), uses
 /// that system's grid, and counts itself in the system's range of cells. Lanes of a wave in the same cell share one
 /// atomic, like in assign_cells: small systems put a whole wave into one cell.

@@ -161,14 +161,14 @@ __global__ void publish_ordered_status(
 __global__ __launch_bounds__(BLOCK) void compare_boxes_kernel(
     const unsigned long long* __restrict__ boxes, const unsigned char* __restrict__ periodic,
     const unsigned long long* __restrict__ kept_boxes, const unsigned char* __restrict__ kept_periodic,
-    size_t n_systems, unsigned int* changed
+    size_t n_box_words, size_t n_flags, unsigned int* changed
 ) {
     bool differs = false;
     const size_t stride = static_cast<size_t>(gridDim.x) * BLOCK;
-    for (size_t k = static_cast<size_t>(blockIdx.x) * BLOCK + threadIdx.x; k < 9 * n_systems; k += stride) {
+    for (size_t k = static_cast<size_t>(blockIdx.x) * BLOCK + threadIdx.x; k < n_box_words; k += stride) {
         differs = differs || boxes[k] != kept_boxes[k];
     }
-    for (size_t k = static_cast<size_t>(blockIdx.x) * BLOCK + threadIdx.x; k < 3 * n_systems; k += stride) {
+    for (size_t k = static_cast<size_t>(blockIdx.x) * BLOCK + threadIdx.x; k < n_flags; k += stride) {
         differs = differs || (periodic[k] != 0) != (kept_periodic[k] != 0);
     }
     if (differs) {
@@ -188,6 +188,7 @@ struct Mailbox {
     ShiftRange ranges[SHIFT_RANGE_BLOCKS]; // one slot per workgroup of the sort's range pass
     unsigned int batch_changed;          // a batch that started from the boxes of the call before: they are others now
     unsigned int padding;
+    unsigned long long batch_total_cells; // a batch whose grids were picked on the device: all its cells
 };
 
 /// Makes `device` current for a scope and gives the caller's device back afterwards.
@@ -377,6 +378,8 @@ using PinnedVector = std::vector<T, PinnedAllocator<T>>;
 struct BatchSetup {
     bool valid = false;
     bool any_open_direction = false;
+    bool all_open = false;                  // no system has a periodic direction: the boxes count for nothing
+    uint64_t cells_bound = 0;               // most cells the grids of these systems can have, whatever their points
     double cutoff = 0.0;
     int algorithm = 0;
     bool full_stencil = false;              // VESIN_HIP_STENCIL=full was set
@@ -2081,10 +2084,12 @@ void neighbors_batch(
     BatchSetup& setup = extras.batch;
     const BoxKey key = {n_points, options.cutoff, static_cast<int>(options.algorithm), options.full, options.sorted};
     const bool may_guess = setup.guess.begin(key);
+    // (systems without any periodic direction: the grids follow the points and are picked on the device, see
+    // batch_attempt; only the flags have to be the same)
     const bool rest_is_the_same =
-        setup.valid && setup.kept_on_device && !setup.any_open_direction && setup.cutoff == options.cutoff &&
-        setup.algorithm == static_cast<int>(options.algorithm) && setup.full_stencil == full_stencil_only() &&
-        setup.first_point.size() == n_systems + 1 &&
+        setup.valid && setup.kept_on_device && (!setup.any_open_direction || setup.all_open) &&
+        setup.cutoff == options.cutoff && setup.algorithm == static_cast<int>(options.algorithm) &&
+        setup.full_stencil == full_stencil_only() && setup.first_point.size() == n_systems + 1 &&
         std::memcmp(setup.first_point.data(), first_point, (n_systems + 1) * sizeof(size_t)) == 0 &&
         setup.boxes.size() == 9 * n_systems && extras.mail == extras.mail_device;
     if (may_guess && rest_is_the_same) {
@@ -2136,8 +2141,8 @@ bool batch_attempt(
         hipLaunchKernelGGL(
             compare_boxes_kernel, dim3(compare_blocks), dim3(BLOCK), 0, stream,
             reinterpret_cast<const unsigned long long*>(boxes), reinterpret_cast<const unsigned char*>(periodic),
-            reinterpret_cast<const unsigned long long*>(kept), kept + 72 * n_systems, n_systems,
-            &extras.mail_device->batch_changed
+            reinterpret_cast<const unsigned long long*>(kept), kept + 72 * n_systems,
+            setup.all_open ? size_t(0) : 9 * n_systems, 3 * n_systems, &extras.mail_device->batch_changed
         );
         same_setup = true;
     } else {
@@ -2183,12 +2188,17 @@ bool batch_attempt(
         cell_base_host.resize(n_systems + 1);
         first_point_host.resize(n_systems + 1);
         bool any_open_direction = false;
+        bool any_periodic_direction = false;
+        uint64_t cells_bound = 0;
         for (size_t s = 0; s < n_systems; s++) {
             bool flags[3];
             for (int d = 0; d < 3; d++) {
                 flags[d] = host_periodic[3 * s + d] != 0;
                 any_open_direction = any_open_direction || !flags[d];
+                any_periodic_direction = any_periodic_direction || flags[d];
             }
+            // (choose_grid never makes more cells than twice the points, or 64)
+            cells_bound += std::min<uint64_t>(16777216, std::max<uint64_t>(64, 2 * (first_point[s + 1] - first_point[s])));
             const HostBox hbox = normalise_box(&host_boxes[9 * s], flags);
             host_grids_box[s] = hbox;
             GridParams& g = grids[s];
@@ -2204,6 +2214,8 @@ bool batch_attempt(
         }
         first_point_host[n_systems] = static_cast<uint32_t>(n_points);
         setup.any_open_direction = any_open_direction;
+        setup.all_open = !any_periodic_direction;
+        setup.cells_bound = cells_bound;
 
         // ---- systems with a non-periodic direction need the extent of their points along it (reference:
         // BoundingBox::make_bounding_for, vesin/src/types.hpp:159-200): one wave per system finds it
@@ -2283,15 +2295,24 @@ bool batch_attempt(
         setup.most_units = most_units;
         setup.valid = true;
     }
-    if (!setup.kept_on_device && !setup.any_open_direction) {
-        // what the next call's boxes are compared with (never with an open direction: the grids follow the points)
+    if (!setup.kept_on_device && (!setup.any_open_direction || setup.all_open)) {
+        // what the next call's boxes are compared with (never with some directions open and others not: the grids
+        // follow the points and the boxes)
         setup.kept_boxes.reserve(75 * n_systems);
         auto* kept = static_cast<unsigned char*>(setup.kept_boxes.ptr);
         HIP_CHECK(hipMemcpyAsync(kept, setup.boxes.data(), 72 * n_systems, hipMemcpyHostToDevice, stream));
         HIP_CHECK(hipMemcpyAsync(kept + 72 * n_systems, setup.periodic.data(), 3 * n_systems, hipMemcpyHostToDevice, stream));
         setup.kept_on_device = true;
     }
-    const uint64_t total_cells = setup.total_cells;
+    // Systems without any periodic direction, on a call that starts from the set-up of the call before: their grids
+    // follow this call's points and are picked on the device, right before the cell lists are built (the host would
+    // have to wait for the extents, pick the grids and send them back). The work buffers are sized for the most
+    // cells such grids can have.
+    const bool device_grids = speculate && setup.all_open;
+    const uint64_t total_cells = device_grids ? setup.cells_bound : setup.total_cells;
+    if (total_cells >= 0xFFFFFFF0ull) {
+        throw std::runtime_error("too many cells in this batch");
+    }
 
     if (n_points == 0) {
         size_outputs(neighbors, extras, 0, options);
@@ -2350,6 +2371,7 @@ bool batch_attempt(
     uint32_t* d_first_point = nullptr;
     uint32_t* d_cell_base = nullptr;
     unsigned long long* d_first_pair = nullptr;
+    uint32_t* d_cells_of_system = nullptr;
     char* clear_end = nullptr;
     const size_t scratch_elements = std::max(scan_scratch_elements(total_cells), scan_scratch_elements(n_slots));
     auto carve = [&](Carver& carver) {
@@ -2377,6 +2399,7 @@ bool batch_attempt(
         d_first_point = carver.take<uint32_t>(n_systems + 1);
         d_cell_base = carver.take<uint32_t>(n_systems + 1);
         d_first_pair = carver.take<unsigned long long>(n_systems + 1);
+        d_cells_of_system = carver.take<uint32_t>(n_systems);
     };
     Carver measure(nullptr);
     carve(measure);
@@ -2387,7 +2410,12 @@ bool batch_attempt(
     const bool already_there = same_setup && setup.on_device && setup.work_generation == extras.work.generation &&
                                setup.d_grids == d_grids &&
                                setup.d_first_point == d_first_point && setup.d_cell_base == d_cell_base;
-    if (!already_there) {
+    if (device_grids) {
+        setup.on_device = false; // (grids and first cells of this call are the device's own)
+        HIP_CHECK(hipMemcpyAsync(
+            d_first_point, first_point_host.data(), (n_systems + 1) * sizeof(uint32_t), hipMemcpyHostToDevice, stream
+        ));
+    } else if (!already_there) {
         setup.on_device = false;
         HIP_CHECK(hipMemcpyAsync(d_grids, grids.data(), n_systems * sizeof(GridParams), hipMemcpyHostToDevice, stream));
         HIP_CHECK(hipMemcpyAsync(
@@ -2416,6 +2444,20 @@ bool batch_attempt(
             clear_and_fetch, dim3(fill_blocks), dim3(BLOCK), 0, stream,
             reinterpret_cast<uint4*>(cell_counts), blocks16, reinterpret_cast<const double*>(boxes),
             reinterpret_cast<const bool*>(periodic), extras.mail_device->small, extras.d_status
+        );
+    }
+    if (device_grids) {
+        // (behind the launch that resets the status block: a coordinate that is not finite is reported there)
+        extras.mail->batch_total_cells = 0;
+        const int single_cell = options.algorithm == VesinBruteForce ? 1 : options.algorithm == VesinAutoAlgorithm ? 0 : -1;
+        hipLaunchKernelGGL(
+            open_grids_kernel, dim3(static_cast<uint32_t>((n_systems + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK)), dim3(BLOCK),
+            0, stream, flat_points, d_first_point, static_cast<uint32_t>(n_systems), options.cutoff, single_cell, d_grids,
+            d_cells_of_system, &extras.d_status->first_bad_coordinate
+        );
+        hipLaunchKernelGGL(
+            open_bases_kernel, dim3(1), dim3(1024), 0, stream,
+            d_cells_of_system, static_cast<uint32_t>(n_systems), d_cell_base, &extras.mail_device->batch_total_cells
         );
     }
     hipLaunchKernelGGL(
@@ -2492,7 +2534,7 @@ bool batch_attempt(
             std::fprintf(
                 stderr, "single pass (batch): rows %llu general %u deferred %u overflow %u timeout %u (slices %u%s)\n",
                 result.total_rows, result.general, result.deferred, result.overflow, result.chain_timeout, n_slices,
-                speculate ? ", grids of the call before" : ""
+                device_grids ? ", grids picked on the device" : speculate ? ", grids of the call before" : ""
             );
         }
         if (result.general == 0 && result.deferred == 0 && result.overflow == 0 && result.chain_timeout == 0) {
