@@ -1132,6 +1132,7 @@ bool compute(
     uint32_t* rows_of_point = nullptr;
     uint64_t* first_row_of_point = nullptr;
     CandidateRecord* candidate_records = nullptr;
+    uint32_t* candidates_of_item = nullptr;
     uint16_t* candidate_order = nullptr;
     char* wraps_end = nullptr;
     // small systems: the points of a tile are dealt to several waves, about 2048 in all
@@ -1186,6 +1187,7 @@ bool compute(
         if (try_in_order) {
             first_row_of_point = carver.take<uint64_t>(n_points + 1);
             candidate_records = carver.take<CandidateRecord>(static_cast<size_t>(ordered_blocks) * ORDERED_WAVES * ORDERED_UNITS * WAVE);
+            candidates_of_item = carver.take<uint32_t>(static_cast<size_t>(ordered_blocks) * ORDERED_WAVES);
             if (ordered_items_per_tile == 1) {
                 candidate_order = carver.take<uint16_t>(tiles_bound * ORDERED_CANDIDATES);
             }
@@ -1549,6 +1551,7 @@ bool compute(
         oargs.items_per_tile = ordered_items_per_tile;
         oargs.rows_of_point = rows_of_point;
         oargs.records = candidate_records;
+        oargs.candidates_of_item = candidates_of_item;
         // How many waves share a tile in either pass follows the number of tiles the call before had on the same
         // number of points (policy.hpp); a list's first call on a system keeps one wave per tile.
         const size_t tiles_before = ordered_items_per_tile == 1 && extras.ordered_tiles_points == n_points ? extras.ordered_tiles : 0;

@@ -77,6 +77,7 @@ struct OrderedArgs {
     uint32_t* rows_of_point;    // COUNT: [n_points], by original index
     CandidateRecord* records;   // COUNT -> WRITE: [work item][ORDERED_UNITS][64], candidates in table order: hit column,
                                 // original index, biased shift (see CandidateRecord)
+    uint32_t* candidates_of_item; // COUNT -> WRITE: [work item], how many of them there are
     const double* points;       // WRITE: the caller's points, by original index
     uint16_t* order;            // SORT -> WRITE: [tile][ORDERED_CANDIDATES], candidate number at each place of the order
     const uint64_t* first_row;  // WRITE: [n_points + 1], exclusive scan of rows_of_point
@@ -97,7 +98,7 @@ struct OrderedArgs {
 
 /// LDS of one wave. What is known per candidate (hit column, position, original index, shift) stays in the
 /// registers of the lane that loaded it: a lane only ever needs its own candidates until it hands a hit over as a key.
-struct OrderedWaveShared: SearchTables {
+struct OrderedWaveShared {
     uint32_t tile_index[TILE_POINTS];
     double tile_x[TILE_POINTS], tile_y[TILE_POINTS], tile_z[TILE_POINTS];
     int32_t tile_wx[TILE_POINTS], tile_wy[TILE_POINTS], tile_wz[TILE_POINTS];
@@ -119,6 +120,14 @@ struct OrderedCountWaveShared: SearchTables {
 template <bool WRITE>
 struct OrderedShared {
     std::conditional_t<WRITE, OrderedWaveShared, OrderedCountWaveShared> wave[ORDERED_WAVES];
+};
+
+/// The writing pass also keeps the records of one work item, for the launches in which the four waves of a workgroup
+/// share a work item: they fetch the records together, once, instead of each for itself.
+template <>
+struct OrderedShared<true> {
+    OrderedWaveShared wave[ORDERED_WAVES];
+    CandidateRecord records[ORDERED_CANDIDATES];
 };
 
 __device__ __forceinline__ uint32_t biased_shift(int32_t sx, int32_t sy, int32_t sz) {
@@ -489,8 +498,17 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
     if (n_stencil > MAX_ENTRIES) {
         return; // the host does not launch this kernel for such a stencil
     }
-    fill_stencil_tables(sh, lane, 0, n_stencil, cx, cy, cz, span_y, span_z, g, args.cell_scan);
-    const uint32_t n_candidates = __builtin_amdgcn_readfirstlane(sh.n_candidates);
+    uint32_t n_candidates;
+    if constexpr (WRITE) {
+        // (the counting pass left the number: no tables here, everything about a candidate is in its record)
+        n_candidates = uniform(args.candidates_of_item[work]);
+    } else {
+        fill_stencil_tables(sh, lane, 0, n_stencil, cx, cy, cz, span_y, span_z, g, args.cell_scan);
+        n_candidates = __builtin_amdgcn_readfirstlane(sh.n_candidates);
+        if (lane == 0 && part == 0) {
+            args.candidates_of_item[work] = n_candidates;
+        }
+    }
     const uint32_t n_units = (n_candidates + WAVE - 1) / WAVE;
 
     if (!WRITE) {
@@ -564,6 +582,18 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
         uint32_t columns[ORDERED_UNITS];
         uint32_t cand_index[ORDERED_UNITS];
         uint32_t cand_biased[ORDERED_UNITS];
+        // The four waves of a workgroup that share a work item (every wave of the workgroup got this far then, or
+        // none) bring its records to LDS together, already in the order of the tile: a place each per step, its
+        // candidate number and then the record from memory, two round trips for the workgroup where every wave
+        // made two per group of four units.
+        const bool together = split == ORDERED_WAVES;
+        if (together) {
+            for (uint32_t place = threadIdx.x; place < n_candidates; place += ORDERED_BLOCK) {
+                const uint32_t k = PRESORTED ? min(static_cast<uint32_t>(tile_order[place]), n_candidates - 1) : place;
+                shared.records[place] = item_records[k];
+            }
+            __syncthreads();
+        }
 #pragma unroll
         for (int u = 0; u < ORDERED_UNITS; u++) {
             columns[u] = 0;
@@ -571,8 +601,13 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
             cand_biased[u] = 0;
             const uint32_t place = u * WAVE + lane;
             if (static_cast<uint32_t>(u) < n_units && place < n_candidates) {
-                const uint32_t k = PRESORTED ? min(static_cast<uint32_t>(tile_order[place]), n_candidates - 1) : place;
-                const CandidateRecord record = item_records[k]; // one 12-byte load
+                CandidateRecord record; // 12 bytes
+                if (together) {
+                    record = shared.records[place];
+                } else {
+                    const uint32_t k = PRESORTED ? min(static_cast<uint32_t>(tile_order[place]), n_candidates - 1) : place;
+                    record = item_records[k];
+                }
                 columns[u] = record.column;
                 cand_index[u] = record.index;
                 cand_biased[u] = record.biased;
