@@ -98,16 +98,18 @@ inline unsigned int ordered_share(size_t n_points, size_t n_cells, size_t tile_s
     return share;
 }
 
-/// Waves that share the points of a tile in the writing pass (1, 2 or 4), from the number of tiles the call before
-/// had on the same points (0: not known, one wave).
+/// Waves that share the points of a tile in the writing pass (1 or 4), from the number of tiles the call before had
+/// on the same points (0: not known, one wave).
 ///
 /// The pass keeps four waves per SIMD resident, 4096 on this GPU. A system of a few more tiles than that leaves the
 /// stragglers running alone for as long as everything before them took (100,000 atoms, 4,260 tiles: 172 us where a
-/// wave lives 110 us; two waves per tile 142 us, four 133 us). The waves of a tile read the same records, a fixed
-/// cost worth about eight points' rows each, so it only pays for well-filled tiles and up to about three times as
-/// many tiles as resident waves (half lists at 24 points per tile, per call: 4,500 tiles 357 -> 316 us with four
-/// waves, 9,000 tiles 567 -> 541 us with two, 19,000 tiles 911 -> 924 us; 12 points per tile, 8,000 tiles: 281 ->
-/// 302 us).
+/// wave lives 110 us; four waves per tile 121 us). With four waves per tile a workgroup is a tile: its waves fetch
+/// the tile's records together and each writes the rows of a quarter of the points, so the work comes in shorter
+/// pieces at little extra cost. It pays for well-filled tiles up to about five times as many tiles as resident
+/// waves (half lists at 24 points per tile, cutoff 6, per call with one wave -> four: 4,500 tiles 318 -> 283 us,
+/// 9,000 tiles 551 -> 515 us, 19,000 tiles 833 -> 794 us, 39,000 tiles 1613 -> 1613 us; full lists at 23 points per
+/// tile, 52,000 tiles: 2.04 -> 2.07 ms) and not for tiles of few points (12 per tile, full lists: 8,000 tiles 276 ->
+/// 311 us, 27,000 tiles 483 -> 606 us).
 inline unsigned int ordered_write_split(size_t n_points, size_t tiles_before) {
     if (tiles_before == 0) {
         return 1;
@@ -117,13 +119,7 @@ inline unsigned int ordered_write_split(size_t n_points, size_t tiles_before) {
     if (static_cast<double>(n_points) < 16.0 * tiles) {
         return 1;
     }
-    if (tiles > 0.85 * resident && tiles <= 1.5 * resident) {
-        return 4;
-    }
-    if (tiles > 1.5 * resident && tiles <= 3.0 * resident) {
-        return 2;
-    }
-    return 1;
+    return tiles > 0.85 * resident && tiles <= 5.0 * resident ? 4 : 1;
 }
 
 /// Waves that share the candidates of a tile in the counting pass (1 or 2), decided like the other.
