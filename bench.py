@@ -41,12 +41,12 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes moved by ONE launch of the single-pass search kernel on the 1M-atom workload, from rocprofv3 --pmc
-# FETCH_SIZE and WRITE_SIZE runs scaled by a device copy of known size (167.3 MB fetched + 3238.2 MB written). The figure belongs to the kernel sources whose
+# FETCH_SIZE and WRITE_SIZE runs scaled by a device copy of known size (167.2 MB fetched + 3238.4 MB written). The figure belongs to the kernel sources whose
 # digest is recorded with it: a run with other sources reports no traffic instead of a stale one.
 SEARCH_KERNEL_TRAFFIC = {
-    "bytes": 3_405_400_000,
+    "bytes": 3_405_600_000,
     "profile": "profiles/fused_search_config1_pmc.txt",
-    "kernel_sources_sha256": "049da47c9ab97cf4962a926de641178ab5c88e297b2c67aafb3fd89dd029fd42",
+    "kernel_sources_sha256": "5a91f5894ff6ee4aa542af534d2da79f4257238e2c10cd1c2fb4a8d7fa1b0e64",
 }
 KERNEL_SOURCES = ["device_common.cuh", "geometry.hpp", "cells.cuh", "search.cuh", "fused.cuh"]
 
