@@ -129,3 +129,30 @@ def test_a_coordinate_that_is_not_finite_is_still_reported(monkeypatch):
     points[1234, 1] = 3.0
     expected = oracle.neighbors(points, box, [False] * 3, 3.0, True, False, "ijSdD")
     assert_same_list(_compute(calculator, points, box, [False] * 3), expected, what="after the error")
+
+
+def test_a_dense_cluster_on_the_one_pass_cell_build_jumps(capfd, monkeypatch):
+    """Cells of ordinary occupation: the one-pass cell build leaves out the points it finds far outside of the
+    remembered extent, as the packed build does; the call starts over and the rows are the oracle's."""
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    rng = np.random.default_rng(55)
+    points = rng.random((9000, 3)) * np.array([50.0, 40.0, 30.0])
+    box = np.zeros((3, 3))
+    calculator = NeighborList(cutoff=3.0, full_list=False, sorted=False)
+    far = []
+    builds = []
+    for step in range(9):
+        if step == 5:
+            points = points + np.array([-400.0, 250.0, 90.0])
+        else:
+            points = points + rng.normal(scale=0.05, size=points.shape)
+        expected = oracle.neighbors(points, box, [False] * 3, 3.0, False, False, "ijSdD")
+        capfd.readouterr()
+        result = _compute(calculator, points, box, [False] * 3)
+        err = capfd.readouterr().err
+        far.append(_far_outside(err))
+        builds += [line for line in err.splitlines() if line.startswith("single pass:") and "one-pass cell build" in line]
+        assert_same_list(result, expected, what=f"step {step}")
+    assert builds, "these cells are what the one-pass build takes"
+    assert all(f == [0] for f in far[3:5]), far
+    assert len(far[5]) == 1 and far[5][0] > 0, far
