@@ -639,7 +639,8 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
 // ---------------------------------------------------------------------------------------------------------------
 // SORT: the order of a tile's candidates
 
-// one wave per workgroup: a wave's scratch takes 22 KB of LDS, and a workgroup of four left room for one per CU
+// one wave per workgroup: a wave's 13 KB of LDS are free again as soon as its tile is done (four waves held 52 KB
+// until the slowest was, beside the counting pass's workgroups: measured a fifth slower)
 constexpr int ORDER_WAVES = 1;
 constexpr int ORDER_BLOCK = ORDER_WAVES * WAVE;
 constexpr uint32_t ORDER_BUCKETS = 4 * WAVE;
