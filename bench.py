@@ -23,7 +23,7 @@ The line carries, next to the throughput:
   and one thread on a bounded sample of the same workload.
 
 ``--config NAME`` makes another configuration the workload of the line (profiling runs use it):
-config0, config1 (default), config1_shuffled, config2, config3, config3_single, config4a, config4b.
+config0, config1 (default), config1_shuffled, config1_sorted, config2, config3, config3_single, config4a, config4b.
 """
 
 import argparse
@@ -50,13 +50,14 @@ SEARCH_KERNEL_TRAFFIC = {
 }
 KERNEL_SOURCES = ["device_common.cuh", "geometry.hpp", "cells.cuh", "search.cuh", "fused.cuh"]
 
-CONFIG_NAMES = ["config0", "config1", "config1_shuffled", "config2", "config3", "config3_single", "config4a", "config4b"]
+CONFIG_NAMES = ["config0", "config1", "config1_shuffled", "config1_sorted", "config2", "config3", "config3_single", "config4a", "config4b"]
 DESCRIPTIONS = {
     "config0": "config0: 216 atoms, cutoff 5 A, full, sorted, i j S d",
     "config1": "config1: jittered diamond {replicas}^3 cells = {n_points} atoms, periodic cube, cutoff 5 A, full list, "
                "unsorted, returns i j S d",
     "config1_shuffled": "config1 with its atoms in random order",
     "config1_box_changes": "config1 with a box that differs from the call before on every call",
+    "config1_sorted": "config1 with sorted=true (rows in the order of i, j, S)",
     "config2": "config2: 100000 atoms, triclinic, cutoff 6 A, half, sorted, i j S d D",
     "config3": "config3: 4096 replicas of 64 atoms, box 7.134 A, cutoff 10 A, full, i j S d, one batched call",
     "config3_single": "one replica of config3 in a call of its own: 64 atoms, box 7.134 A, cutoff 10 A, full, i j S d",
@@ -87,6 +88,9 @@ def host_system(name, replicas=50):
     if name == "config1_shuffled":
         points, box, periodic, options = configs.config1(replicas)
         return points[np.random.default_rng(1).permutation(len(points))], box, periodic, options
+    if name == "config1_sorted":
+        points, box, periodic, options = configs.config1(replicas)
+        return points, box, periodic, dict(options, sorted=True)
     if name == "config2":
         return configs.config2()
     if name == "config3_single":
@@ -371,7 +375,7 @@ def other_configs(args, torch, np):
     results = []
     names = [name for name in ["config0", "config2", "config3", "config3_single", "config4a", "config4b"] if name != args.config]
     if args.config == "config1":
-        names += ["config1_shuffled", "config1_box_changes"]
+        names += ["config1_shuffled", "config1_box_changes", "config1_sorted"]
     for name in names:
         workload = Workload(name, args.replicas)
         measured = measure(workload, 10, 3, torch, np)
