@@ -119,3 +119,22 @@ extern "C" unsigned int probe_ordered_write_split(size_t n_points, size_t tiles_
 extern "C" unsigned int probe_ordered_count_split(size_t n_points, size_t tiles_before) {
     return vesin_hip::ordered_count_split(n_points, tiles_before);
 }
+
+/// Runs the bookkeeping of a launch with waiting workgroups (vesin_hip::WaitRest) over a sequence of calls:
+/// `gives_up[k]` says whether the launch would give up in call k if it were used; `used[k]` receives whether call k
+/// used it.
+extern "C" void probe_wait_rest(const unsigned char* gives_up, size_t n_calls, unsigned char* used) {
+    vesin_hip::WaitRest rest;
+    for (size_t k = 0; k < n_calls; k++) {
+        if (rest.resting()) {
+            used[k] = 0;
+            continue;
+        }
+        used[k] = 1;
+        if (gives_up[k] != 0) {
+            rest.gave_up();
+        } else {
+            rest.went_through();
+        }
+    }
+}

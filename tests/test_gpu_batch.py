@@ -52,17 +52,40 @@ def test_replicas_of_the_small_cell_case(full):
         assert_same_list(lists[r], expected, what=f"replica {r}")
 
 
-def test_waves_that_give_up_waiting_fall_back_to_the_two_passes(monkeypatch):
+def test_waves_that_give_up_waiting_fall_back_to_the_two_passes(capfd, monkeypatch):
     # a batch places its rows through the chain of workgroup totals; with VESIN_HIP_CHAIN_SPINS=0 every wait gives up
     # at once (the kernels still run to their end) and the second call of the list must notice and start over
+    import torch
+
     monkeypatch.setenv("VESIN_HIP_CHAIN_SPINS", "0")
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
     replicas = [configs.config3(r) for r in range(40, 64)]
     cutoff = replicas[0][3]["cutoff"]
     calculator = NeighborList(cutoff=cutoff, full_list=True)
+    capfd.readouterr()
     lists = run_batch(calculator, [r[0] for r in replicas], [r[1] for r in replicas])
+    launched = [line for line in capfd.readouterr().err.splitlines() if line.startswith("single pass (batch)")]
+    assert len(launched) == 1 and " timeout 0 " not in launched[0], launched
     for r, (points, box, periodic, _) in enumerate(replicas):
         expected = oracle.neighbors(points, box, periodic, cutoff, True, False, "ijSdD")
         assert_same_list(lists[r], expected, what=f"replica {r}")
+    # The list stays away from the launch that gave up: the next 64 calls go to the two passes directly (they do not
+    # pay for the wait again), whatever the patience of the waves by then; the call after them is back on it.
+    monkeypatch.delenv("VESIN_HIP_CHAIN_SPINS")
+    first_point = np.cumsum([0] + [len(r[0]) for r in replicas])
+    points = torch.as_tensor(np.concatenate([r[0] for r in replicas]), device="cuda:0")
+    boxes = torch.as_tensor(np.stack([r[1] for r in replicas]), device="cuda:0")
+    for rest in range(64):
+        outputs, first_pair = calculator.compute_batch(points, first_point, boxes, True, "P")
+        assert not [line for line in capfd.readouterr().err.splitlines() if line.startswith("single pass (batch)")], rest
+    assert int(first_pair[-1]) == sum(len(rows["pairs"]) for rows in lists)
+    outputs, first_pair = calculator.compute_batch(points, first_point, boxes, True, "PSdD")
+    launched = [line for line in capfd.readouterr().err.splitlines() if line.startswith("single pass (batch)")]
+    assert len(launched) == 1 and " timeout 0 " in launched[0], launched
+    whole = {NAMES[q]: out.cpu().numpy() for q, out in zip("PSdD", outputs)}
+    for r in range(len(replicas)):
+        rows = slice(int(first_pair[r]), int(first_pair[r + 1]))
+        assert_same_list({key: value[rows] for key, value in whole.items()}, lists[r], what=f"replica {r}, back on the chain")
 
 
 def test_systems_of_different_sizes_and_shapes():
@@ -531,3 +554,47 @@ def test_free_molecules_get_their_grids_on_the_device(algorithm, capfd, monkeypa
     with pytest.raises(RuntimeError, match="point"):
         run(broken, False, check=False)
     assert run(molecules, False) in (0, 1)
+
+
+@pytest.mark.parametrize("algorithm", ["auto", "cell_list"])
+def test_stretched_open_systems_keep_to_the_room_for_their_cells(algorithm, capfd, monkeypatch):
+    """Systems that are long in one direction and thin in the others (stretched chains, a pair of atoms moving apart)
+    must not get more cells than the batch's buffers were sized for (64, or twice the points, per system), also when
+    the grids are picked on the device: a chain that keeps getting longer from call to call, checked against the
+    oracle on every call."""
+    import torch
+
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    rng = np.random.default_rng(11)
+    sizes = [40, 2, 1000, 33, 64, 7]
+    first_point = np.cumsum([0] + sizes)
+    boxes = np.zeros((len(sizes), 3, 3))
+    cutoff = 5.0
+    calculator = NeighborList(cutoff=cutoff, full_list=True, algorithm=algorithm)
+
+    def systems(stretch):
+        out = []
+        for k, n in enumerate(sizes):
+            axis = k % 3
+            points = rng.uniform(0.0, 3.0, size=(n, 3))
+            # 1.5 points per cutoff along the chain at stretch 1: neighbours stay, cells multiply
+            points[:, axis] = np.sort(rng.uniform(0.0, n * cutoff / 1.5 * stretch, size=n))
+            out.append(points + rng.uniform(-50, 50, size=3))
+        return out
+
+    # (the longest chain stays below 100,000 cutoffs: beyond that many cells the reference's own grid, which the
+    # oracle restates, has no cells left in the thin directions, vesin/src/cpu_cell_list.cpp:294-304)
+    for call, stretch in enumerate([1.0, 1.0, 4.0, 25.0, 0.1, 100.0]):
+        molecules = systems(stretch)
+        capfd.readouterr()
+        outputs, first_pair = calculator.compute_batch(
+            torch.as_tensor(np.concatenate(molecules), device="cuda:0"), first_point,
+            torch.as_tensor(boxes, device="cuda:0"), False, "PSdD",
+        )
+        err = capfd.readouterr().err
+        assert ("grids picked on the device" in err) == (call >= 1), (call, err)
+        whole = {NAMES[q]: out.cpu().numpy() for q, out in zip("PSdD", outputs)}
+        for s, points in enumerate(molecules):
+            rows = slice(int(first_pair[s]), int(first_pair[s + 1]))
+            expected = oracle.neighbors(points, np.eye(3) * 500.0, [False] * 3, cutoff, True, False, "ijSdD")
+            assert_same_list({k: v[rows] for k, v in whole.items()}, expected, what=f"call {call}, system {s}")

@@ -33,6 +33,8 @@ def probe(tmp_path_factory):
                                   ctypes.c_void_p, ctypes.c_size_t]
     lib.probe_box_guess.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
     lib.probe_box_guess.restype = None
+    lib.probe_wait_rest.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+    lib.probe_wait_rest.restype = None
     lib.probe_ordered_share.argtypes = [ctypes.c_size_t, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_int]
     lib.probe_ordered_share.restype = ctypes.c_uint
     for name in ("probe_ordered_write_split", "probe_ordered_count_split"):
@@ -201,6 +203,41 @@ def test_grid_open_directions_and_single_cell(probe):
     assert n.tolist() == [1, 1, 1] and s.tolist() == [0, 0, 0]
 
 
+def test_never_more_cells_than_twice_the_points(probe):
+    """The work buffers of a batch are sized for max(64, 2 n) cells per system whatever its points do: a system that
+    is long in one direction and thin in the others (a stretched chain, a dissociating pair) must not keep more
+    cells along its length than that because the thin directions cannot go below one cell."""
+    open_box = np.eye(3)
+    cases = [
+        (40, 5.0, [1000.0, 3.0, 3.0]),      # 199 cells along x before the limit, 80 allowed
+        (1000, 5.0, [20000.0, 0.0, 0.0]),   # a line of points
+        (2, 1.0, [1.0e6, 0.5, 0.5]),        # two atoms far apart
+        (500, 2.0, [3000.0, 3000.0, 1.0]),  # a sheet
+        (33, 0.5, [700.0, 650.0, 600.0]),
+        (100000, 3.0, [1.0e5, 1.0e5, 2.0]),
+    ]
+    for n_points, cutoff, width in cases:
+        for order in ([0, 1, 2], [1, 2, 0], [2, 0, 1]):
+            hi = [width[k] for k in order]
+            status, n, s = run_grid(probe, open_box, [0, 0, 0], cutoff, n_points, [0.0] * 3, hi)
+            assert status == 0
+            cells = int(np.prod(n.astype(np.int64)))
+            assert cells <= max(64, 2 * n_points), (n_points, cutoff, hi, n.tolist())
+            # and still cells: the limit does not collapse a long system into a handful of cells
+            assert cells >= min(0.4 * max(64, 2 * n_points), np.prod(np.maximum(np.floor(np.array(hi) * 1.01 / cutoff), 1)) * 0.4)
+            # cells at least as wide as the cutoff, stencil reaching beyond it or to the last cell
+            extent = np.maximum(np.where(np.array(hi) >= 1e-6, np.array(hi), 1.0) * 1.01, 1.0)
+            assert np.all((extent / n > cutoff) | (n == 1))
+            assert np.all((s * extent / n > cutoff) | (s == n - 1))
+    rng = np.random.default_rng(5)
+    for _ in range(500):
+        n_points = int(rng.integers(1, 5000))
+        cutoff = rng.uniform(0.5, 8.0)
+        hi = (10.0 ** rng.uniform(-2, 5, size=3)).tolist()
+        status, n, s = run_grid(probe, open_box, [0, 0, 0], cutoff, n_points, [0.0] * 3, hi)
+        assert status == 0 and int(np.prod(n.astype(np.int64))) <= max(64, 2 * n_points)
+
+
 def test_too_many_images_is_an_error(probe):
     status, _, _ = run_grid(probe, np.eye(3) * 0.01, [1, 1, 1], 10.0, 10, [0] * 3, [0] * 3)
     assert status == 1
@@ -342,3 +379,29 @@ def test_waves_per_tile_of_the_two_passes(probe):
             assert count(tiles * per_tile, tiles) in (1, 2)
             if per_tile < 16:
                 assert write(tiles * per_tile, tiles) == 1 and count(tiles * per_tile, tiles) == 1
+
+
+def run_wait_rest(probe, gives_up):
+    gives_up = np.ascontiguousarray(gives_up, dtype=np.uint8)
+    used = np.zeros(len(gives_up), dtype=np.uint8)
+    probe.probe_wait_rest(gives_up.ctypes.data, len(gives_up), used.ctypes.data)
+    return used.astype(bool)
+
+
+def test_a_launch_whose_waves_gave_up_is_left_alone_for_longer_and_longer(probe):
+    # never a give-up: used by every call
+    assert run_wait_rest(probe, [0] * 50).all()
+    # a GPU on which the launch gives up whenever it is tried: tried at calls 0, 65, 194, 451, ... (64, 128, 256 ...
+    # calls of rest in between, 4096 at most)
+    used = run_wait_rest(probe, [1] * 20000)
+    tried = np.flatnonzero(used)
+    assert tried[:5].tolist() == [0, 65, 194, 451, 964]
+    assert np.diff(tried).max() == 4097 and np.diff(tried)[-1] == 4097
+    # one give-up, then fine again: 64 calls of rest once, and the next give-up starts from 64 again
+    gives_up = np.zeros(400, dtype=np.uint8)
+    gives_up[10] = 1
+    gives_up[200] = 1
+    used = run_wait_rest(probe, gives_up)
+    assert used[:11].all() and not used[11:75].any() and used[75:201].all() and not used[201:265].any() and used[265:].all()
+
+

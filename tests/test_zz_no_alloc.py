@@ -204,6 +204,42 @@ def test_small_systems_take_one_launch_here_too(sorted, capfd, monkeypatch):
     assert used == len(systems)
 
 
+def test_device_memory_in_use_does_not_change():
+    """The contract is that nothing is allocated or freed: the free memory of the device (hipMemGetInfo) is, byte for
+    byte, what it was, after calls of every kind through the same work array: a large system unsorted and sorted, small
+    ones through the one launch, a system without periodic directions, and a sorted list that needs the radix sort (a
+    cell of many images). One call of each kind comes first: the runtime itself sets up what it needs for a kernel or
+    a copy (code objects, staging) the first time that one is used."""
+    import torch
+
+    lib = get_library()
+    arrays = CallerArrays(1_400_000)
+    rng = np.random.default_rng(23)
+    cases = []
+    for points, box, periodic, cutoff in (
+        (*configs.diamond(12, seed=5), 5.0),
+        (*configs.diamond(3, seed=1), 5.0),
+        (rng.normal(0.0, 6.0, (4000, 3)), np.zeros((3, 3)), (False, False, False), 3.0),
+        (rng.uniform(0.0, 9.0, (150, 3)), np.zeros((3, 3)), (False, False, False), 4.5),
+        (rng.uniform(0.0, 4.0, (40, 3)), np.array([[4.0, 0.0, 0.0], [1.0, 4.0, 0.0], [0.5, 0.7, 4.0]]), (True, True, True), 7.5),
+    ):
+        periodic = [bool(p) for p in np.broadcast_to(np.asarray(periodic), (3,))]
+        for sorted in (False, True):
+            cases.append((_device(points, box, periodic), _options(cutoff, True, sorted)))
+    counts = []
+    for (d_points, d_box, d_periodic), options in cases:  # warm-up
+        counts.append(_no_alloc(lib, d_points, d_box, d_periodic, options, arrays))
+    torch.cuda.synchronize()
+    free_before, total = torch.cuda.mem_get_info()
+    for repeat in range(3):
+        for k, ((d_points, d_box, d_periodic), options) in enumerate(cases):
+            assert _no_alloc(lib, d_points, d_box, d_periodic, options, arrays) == counts[k]
+            free_now, _ = torch.cuda.mem_get_info()
+            assert free_now == free_before, (repeat, k, free_before - free_now)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info() == (free_before, total)
+
+
 def test_on_a_stream_of_the_caller():
     import torch
 

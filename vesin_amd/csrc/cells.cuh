@@ -649,13 +649,11 @@ __global__ __launch_bounds__(BLOCK) void open_grids_kernel(
         for (int d = 0; d < 3; d++) {
             cells[d] = one_cell ? 1.0 : fmin(fmax(floor(extent[d] / padded), 1.0), 1048576.0);
         }
+        // (the host sized the buffers of the batch for `most` cells per system)
         const double most = fmin(fmax(2.0 * static_cast<double>(n_here), 64.0), 16777216.0);
-        const double total = cells[0] * cells[1] * cells[2];
-        if (total > most) {
-            const double shrink = cbrt(most / total);
-            for (int d = 0; d < 3; d++) {
-                cells[d] = fmax(floor(cells[d] * shrink), 1.0);
-            }
+        limit_cells(cells, most);
+        if (!(cells[0] * cells[1] * cells[2] <= most)) {
+            cells[0] = cells[1] = cells[2] = 1.0; // never more cells than there is room for
         }
         uint32_t n_cells = 1;
         for (int d = 0; d < 3; d++) {

@@ -9,6 +9,7 @@
 
 #include <cerrno>
 #include <cmath>
+#include <cstddef>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -75,6 +76,21 @@ static uint32_t chain_spin_limit() {
         return CHAIN_SPIN_LIMIT;
     }
     return static_cast<uint32_t>(parsed);
+}
+
+/// VESIN_HIP_CHAIN_WAIT_US=<n> is the time such a wave waits at most, in microseconds (2000 unless set; for
+/// measurements).
+static uint32_t chain_wait_ticks() {
+    const char* text = std::getenv("VESIN_HIP_CHAIN_WAIT_US");
+    if (text == nullptr || *text == '\0') {
+        return CHAIN_WAIT_TICKS;
+    }
+    char* end = nullptr;
+    const unsigned long parsed = std::strtoul(text, &end, 10);
+    if (*end != '\0' || parsed > 1000000ul) {
+        return CHAIN_WAIT_TICKS;
+    }
+    return static_cast<uint32_t>(parsed * 100ul); // the clock runs at 100 MHz
 }
 
 /// VESIN_HIP_SEARCH=two-pass keeps every call on the count / scan / write sequence (for comparisons and tests).
@@ -180,15 +196,17 @@ __global__ __launch_bounds__(BLOCK) void compare_boxes_kernel(
 /// kernels write into directly; the entry point that allocates nothing keeps the block in device memory and copies
 /// it to the host before every wait (see HipExtras::wait).
 struct Mailbox {
+    // what every wait reads
     DeviceStatus status;
     FusedStatus fused;
     OrderedHostStatus ordered;
     unsigned char small[128];            // box (72 bytes) + periodic (3 bytes)
-    BlockBounds bounds[BOUNDING_BLOCKS]; // one slot per workgroup of the bounding pass
-    ShiftRange ranges[SHIFT_RANGE_BLOCKS]; // one slot per workgroup of the sort's range pass
     unsigned int batch_changed;          // a batch that started from the boxes of the call before: they are others now
     unsigned int padding;
     unsigned long long batch_total_cells; // a batch whose grids were picked on the device: all its cells
+    // what only some do
+    BlockBounds bounds[BOUNDING_BLOCKS]; // one slot per workgroup of the bounding pass
+    ShiftRange ranges[SHIFT_RANGE_BLOCKS]; // one slot per workgroup of the sort's range pass
 };
 
 /// Makes `device` current for a scope and gives the caller's device back afterwards.
@@ -409,6 +427,9 @@ struct BatchSetup {
     DeviceBuffer kept_boxes;
     bool kept_on_device = false;
     BoxGuess guess;
+    // The single-pass search of a batch places its rows through the chain of workgroups: after a launch whose waves
+    // gave up waiting, reused lists go straight to the two passes for a while.
+    WaitRest chain_rest;
     // where the first rows of the systems land before they are copied into the caller's array (pinned)
     size_t* first_pair_landing = nullptr;
     size_t first_pair_capacity = 0;
@@ -432,6 +453,8 @@ struct HipExtras {
     int direct_rest = 0;              // calls left before the one-pass cell build is tried again after a cell overflowed
     int in_order_rest = 0;            // calls left before the in-order search is tried again on a system it did not cover
     int one_launch_rest = 0;          // calls left before a small system is tried in one launch again
+    WaitRest meeting_rest;            // ... after workgroups of that launch gave up waiting for the others
+    WaitRest chain_rest;              // the same for the chain of the single-pass search (rows in work-item order)
     uint32_t ordered_tiles = 0;       // tiles of the last call through the in-order search, and its number of points:
     size_t ordered_tiles_points = 0;  // how the next one deals its writing pass to the waves (see write_split)
     /// Extent of the points along the directions that are not periodic, as the last call found it: a small system
@@ -464,10 +487,17 @@ struct HipExtras {
     HipExtras(const HipExtras&) = delete;
     HipExtras& operator=(const HipExtras&) = delete;
 
-    /// Wait for the stream; afterwards `mail` holds what the kernels queued before this call reported.
-    void wait(hipStream_t stream) {
+    /// Wait for the stream; afterwards `mail` holds what the kernels queued before this call reported, and the first
+    /// `n_bounds` slots of the bounding pass. (A block in device memory is copied piece by piece: a few hundred bytes
+    /// for most waits, where the whole block is 20 KB that the runtime would stage on every wait.)
+    void wait(hipStream_t stream, size_t n_bounds = 0) {
         if (mail_device != mail) {
-            HIP_CHECK(hipMemcpyAsync(mail, mail_device, sizeof(Mailbox), hipMemcpyDeviceToHost, stream));
+            HIP_CHECK(hipMemcpyAsync(mail, mail_device, offsetof(Mailbox, bounds), hipMemcpyDeviceToHost, stream));
+            if (n_bounds > 0) {
+                HIP_CHECK(hipMemcpyAsync(
+                    mail->bounds, mail_device->bounds, n_bounds * sizeof(BlockBounds), hipMemcpyDeviceToHost, stream
+                ));
+            }
         }
         HIP_CHECK(hipStreamSynchronize(stream));
     }
@@ -930,7 +960,7 @@ bool compute(
     // needs no pass over the points and no answer from the device before its kernels are launched. Either way the
     // call finds the extent of its own points on the way and leaves it for the call after it. A grid that fits
     // the points of the call before still gives the right list: points beyond it land in the outermost cells.
-    const bool small_guess = n_points <= SMALL_POINTS && extras.one_launch_rest == 0;
+    const bool small_guess = n_points <= SMALL_POINTS && extras.one_launch_rest == 0 && extras.meeting_rest.rest == 0;
     const bool large_guess = n_points > SMALL_POINTS && !options.sorted && extras.capacity > 0 && !two_pass_only() &&
                              extras.single_pass_rest == 0 && !ordered_rows() && options.algorithm != VesinBruteForce &&
                              extras.extent_rest == 0 && !fresh_extent_only();
@@ -955,7 +985,7 @@ bool compute(
             bounding_kernel, dim3(blocks), dim3(BLOCK), 0, stream,
             reinterpret_cast<const double*>(points), g.n_points, g, extras.mail_device->bounds
         );
-        extras.wait(stream);
+        extras.wait(stream, blocks);
         if (!box_was_right()) {
             return false;
         }
@@ -1046,6 +1076,9 @@ bool compute(
         extras.single_pass_rest -= 1;
         try_single_pass = false;
     }
+    if (try_single_pass && ordered_rows() && extras.chain_rest.resting()) {
+        try_single_pass = false; // (the two passes give the rows in the same order on every run as well)
+    }
     // Cells of ordinary occupation: the cells are built in one pass over the points, every cell owning
     // DIRECT_CAPACITY slots (place_direct); only the single-pass search reads that layout.
     const double direct_mean_min = extras.fixed_memory             ? DIRECT_MEAN_MIN_FIXED_MEMORY
@@ -1125,6 +1158,9 @@ bool compute(
             extras.own_meetings = true;
             HIP_CHECK(hipMemset(extras.meetings, 0, 2 * sizeof(SmallMeeting)));
         }
+    }
+    if (one_launch && extras.meeting_rest.resting()) {
+        one_launch = false; // its workgroups gave up waiting for each other not long ago
     }
     const size_t small_items = one_launch ? n_points * small_slices : 0;
     uint32_t* rows_of_item = nullptr;
@@ -1218,6 +1254,8 @@ bool compute(
     const bool guessed_grid = remembered_extent && !one_launch && try_single_pass && !single_cell && !small_build;
     if (remembered_extent && !one_launch && !guessed_grid) {
         // the grid came from an extent that only these two ways refresh: start over with a pass over the points
+        // (nothing is known against the box: its guess is not to be blamed)
+        extras.extent_missed = true;
         return false;
     }
     if (one_launch) {
@@ -1257,7 +1295,7 @@ bool compute(
         fetched = true;
         mark(T_CELLS);
         mark(T_WRITE);
-        extras.wait(stream);
+        extras.wait(stream, any_open ? 1 : 0);
         if (!box_was_right()) {
             return false;
         }
@@ -1275,6 +1313,7 @@ bool compute(
             );
         }
         if (suitable && found.total_rows <= extras.capacity) {
+            extras.meeting_rest.went_through();
             check_pair_limit(found.total_rows);
             HIP_CHECK(hipGetLastError());
             neighbors.length = found.total_rows;
@@ -1296,9 +1335,16 @@ bool compute(
             }
             return true;
         }
-        if (!suitable) {
-            // (rows that do not fit are no reason: the arrays grow below and the next call finds room)
-            extras.one_launch_rest = SINGLE_PASS_REST;
+        if (found.found.gave_up != 0) {
+            // the workgroups were not all running at once (a GPU shared with other work): the separate launches take
+            // over, for longer and longer while that keeps happening
+            extras.meeting_rest.gave_up();
+        } else {
+            extras.meeting_rest.went_through();
+            if (!suitable) {
+                // (rows that do not fit are no reason: the arrays grow below and the next call finds room)
+                extras.one_launch_rest = SINGLE_PASS_REST;
+            }
         }
     }
 
@@ -1430,6 +1476,7 @@ bool compute(
         fargs.first_rows = offsets;
         fargs.status = fused_status;
         fargs.spin_limit = chain_spin_limit();
+        fargs.wait_ticks = chain_wait_ticks();
         uint32_t blocks = static_cast<uint32_t>(search_workgroups);
         if (direct_cells) {
             fargs.search.direct_capacity = DIRECT_CAPACITY;
@@ -1444,7 +1491,7 @@ bool compute(
         hipLaunchKernelGGL(kernel, dim3(blocks), dim3(SEARCH_BLOCK), 0, stream, fargs, g);
         mark(T_WRITE);
         hipLaunchKernelGGL(publish_fused_status, dim3(1), dim3(1), 0, stream, extras.d_status, fused_status, &extras.mail_device->fused);
-        extras.wait(stream);
+        extras.wait(stream, guessed_grid ? bounding_blocks : 0);
         if (!box_was_right()) {
             return false;
         }
@@ -1518,6 +1565,9 @@ bool compute(
             }
             HIP_CHECK(hipGetLastError());
             neighbors.length = result.total_rows;
+            if (ordered) {
+                extras.chain_rest.went_through();
+            }
             if (timed) {
                 extras.timings = {};
                 extras.timings.total = elapsed(T_START, T_WRITE);
@@ -1530,6 +1580,9 @@ bool compute(
         if (result.general != 0) {
             // the shape of this system is not the single-pass kernel's: leave it alone for a while
             extras.single_pass_rest = SINGLE_PASS_REST;
+        }
+        if (result.chain_timeout != 0) {
+            extras.chain_rest.gave_up();
         }
         if (direct_cells) {
             // everything below reads the packed layout: build it now
@@ -2200,7 +2253,7 @@ bool batch_attempt(
                 any_open_direction = any_open_direction || !flags[d];
                 any_periodic_direction = any_periodic_direction || flags[d];
             }
-            // (choose_grid never makes more cells than twice the points, or 64)
+            // (choose_grid and open_grids_kernel never make more cells than twice the points, or 64: limit_cells)
             cells_bound += std::min<uint64_t>(16777216, std::max<uint64_t>(64, 2 * (first_point[s + 1] - first_point[s])));
             const HostBox hbox = normalise_box(&host_boxes[9 * s], flags);
             host_grids_box[s] = hbox;
@@ -2493,7 +2546,7 @@ bool batch_attempt(
     // ---- a list that has arrays from earlier calls: single-pass search straight into them, rows in work-item order
     // (the rows of a system stay together). Whatever does not fit its shape starts over with the two passes below.
     // (a sorted list is sorted afterwards: its rows go to scratch memory first, through the two passes)
-    if (extras.capacity > 0 && !two_pass_only() && !options.sorted) {
+    if (extras.capacity > 0 && !two_pass_only() && !options.sorted && !setup.chain_rest.resting()) {
         size_outputs(neighbors, extras, 0, options);
         FusedArgs fargs = {};
         fargs.search = args;
@@ -2506,6 +2559,7 @@ bool batch_attempt(
         fargs.first_rows = offsets;
         fargs.status = fused_status;
         fargs.spin_limit = chain_spin_limit();
+        fargs.wait_ticks = chain_wait_ticks();
         const uint32_t blocks = static_cast<uint32_t>(search_workgroups);
         if (options.full) {
             hipLaunchKernelGGL(
@@ -2526,7 +2580,9 @@ bool batch_attempt(
             setup.first_pair_landing, d_first_pair, (n_systems + 1) * sizeof(size_t), hipMemcpyDeviceToHost, stream
         ));
         HIP_CHECK(hipStreamSynchronize(stream));
-        if (speculate && extras.mail->batch_changed != 0) {
+        if (speculate && (extras.mail->batch_changed != 0 || (device_grids && extras.mail->batch_total_cells > total_cells))) {
+            // other boxes than the grids were picked from, or (which open_grids_kernel rules out) more cells than
+            // the buffers were sized for: nothing of this attempt is used, the host picks the grids
             return false;
         }
         const FusedStatus result = extras.mail->fused;
@@ -2552,7 +2608,13 @@ bool batch_attempt(
             HIP_CHECK(hipGetLastError());
             std::memcpy(first_pair, setup.first_pair_landing, (n_systems + 1) * sizeof(size_t));
             neighbors.length = result.total_rows;
+            setup.chain_rest.went_through();
             return true;
+        }
+        if (result.chain_timeout != 0) {
+            // waves gave up waiting for the rows of earlier workgroups (a GPU shared with other work): the two passes
+            // below give this call's rows, and the next calls go there directly
+            setup.chain_rest.gave_up();
         }
     }
 
@@ -2560,7 +2622,7 @@ bool batch_attempt(
     exclusive_scan<SCAN_U32>(counts, n_slots, offsets, scan_scratch, stream);
     hipLaunchKernelGGL(publish_status, dim3(1), dim3(1), 0, stream, extras.d_status, offsets + n_slots, &extras.mail_device->status);
     HIP_CHECK(hipStreamSynchronize(stream));
-    if (speculate && extras.mail->batch_changed != 0) {
+    if (speculate && (extras.mail->batch_changed != 0 || (device_grids && extras.mail->batch_total_cells > total_cells))) {
         return false;
     }
     if (extras.mail->status.first_bad_coordinate != 0xFFFFFFFFu) {
@@ -2639,16 +2701,18 @@ constexpr int FIXED_MAX_DEVICES = 64;
 
 static __device__ __align__(256) unsigned char scratch[FIXED_SCRATCH_BYTES];
 
-/// One per GPU. Calls on one GPU share the array, so they take turns (the lock is held for the whole call).
+/// One per GPU, part of the library's own data: nothing is allocated for it, not on the host either. Calls on one
+/// GPU share the array, so they take turns (the lock is held for the whole call).
 struct FixedState {
     std::mutex turn;
+    bool ready = false;
     unsigned char* memory = nullptr; // address of `scratch` on this GPU
     Mailbox host_mail;               // where the block the kernels report through is copied before every wait
     HipExtras extras;
 };
 
 std::mutex FIXED_SETUP;
-FixedState* FIXED_STATES[FIXED_MAX_DEVICES] = {};
+FixedState FIXED_STATES[FIXED_MAX_DEVICES];
 
 /// The state of GPU `device_id`, which must be the current device. The first call on a GPU looks up where that
 /// GPU holds the array.
@@ -2657,16 +2721,16 @@ FixedState& fixed_state_of(int device_id) {
         throw std::runtime_error("the entry point that allocates nothing serves GPUs 0 to " + std::to_string(FIXED_MAX_DEVICES - 1));
     }
     const std::lock_guard<std::mutex> setup(FIXED_SETUP);
-    if (FIXED_STATES[device_id] == nullptr) {
-        auto state = std::make_unique<FixedState>();
+    FixedState& state = FIXED_STATES[device_id];
+    if (!state.ready) {
         void* address = nullptr;
         HIP_CHECK(hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)));
         if (address == nullptr) {
             throw std::runtime_error("internal error: the work array of the library has no address on this GPU");
         }
-        state->memory = static_cast<unsigned char*>(address);
-        unsigned char* next = state->memory;
-        HipExtras& extras = state->extras;
+        state.memory = static_cast<unsigned char*>(address);
+        unsigned char* next = state.memory;
+        HipExtras& extras = state.extras;
         extras.device_id = device_id;
         extras.fixed_memory = true;
         extras.d_status = reinterpret_cast<DeviceStatus*>(next);
@@ -2677,7 +2741,7 @@ FixedState& fixed_state_of(int device_id) {
         extras.own_meetings = false;
         next += FIXED_STATUS_BYTES;
         extras.mail_device = reinterpret_cast<Mailbox*>(next);
-        extras.mail = &state->host_mail;
+        extras.mail = &state.host_mail;
         next += FIXED_MAIL_BYTES;
         extras.work.ptr = next;
         extras.work.bytes = FIXED_WORK_BYTES;
@@ -2686,9 +2750,9 @@ FixedState& fixed_state_of(int device_id) {
         extras.sort_work.ptr = next;
         extras.sort_work.bytes = FIXED_SORT_BYTES;
         extras.sort_work.fixed = true;
-        FIXED_STATES[device_id] = state.release();
+        state.ready = true;
     }
-    return *FIXED_STATES[device_id];
+    return state;
 }
 
 } // namespace
@@ -2755,6 +2819,8 @@ void neighbors_no_alloc(
     extras.one_launch_rest = 0;
     extras.extent_valid = false;
     extras.timings_valid = false;
+    // (`meeting_rest` stays: workgroups that gave up waiting for each other say something about this GPU, not about
+    // the system of the call before)
 
     VesinNeighborList list;
     list.device.type = VesinCUDA;

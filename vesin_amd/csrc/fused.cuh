@@ -16,8 +16,11 @@
 // group wait for the word their leader publishes, i.e. for a workgroup with a larger index. The chain therefore
 // advances only as long as the hardware starts workgroups in index order and a group's leader gets a wave slot while
 // its members wait, which a grid of this shape has always done here but which nothing guarantees. Every wait is
-// bounded for that reason: a wave that runs out of patience raises a flag and goes on with whatever it has (its rows
-// land inside the arrays, at wrong places), and the host starts the call over with the two-pass search.
+// bounded for that reason, in time (CHAIN_WAIT_TICKS of the 100 MHz clock, 2 ms) and not in polls, whose duration
+// depends on what else the GPU is doing: a wave that runs out of patience raises a flag and goes on with whatever it
+// has (it writes nothing), every wave that polls afterwards sees the flag and gives up at once, so a launch whose
+// chain is stuck ends a few milliseconds after the first wave lost patience, and the host starts the call over with
+// the two-pass search and leaves the chain alone for a while (see Rest, policy.hpp).
 //
 // A work item with more than FUSED_UNITS x 64 candidates cannot keep its columns: it is swept and counted here, its
 // rows are placed by the chain like all others, and its first row goes to `offsets` with a mark in `counts`; the
@@ -38,13 +41,15 @@ namespace vesin_hip {
 constexpr int FUSED_UNITS = 32;         // 64-candidate units of one work item whose columns stay in registers
 constexpr int FUSED_SLOTS = 2 * WAVE;   // candidate records in LDS: two units, so that tickets survive a unit change
 constexpr int32_t PACKED_SHIFT_LIMIT = 500;
-constexpr uint32_t CHAIN_SPIN_LIMIT = 1u << 18; // polls a wave makes before it gives up (FusedArgs::spin_limit)
+constexpr uint32_t CHAIN_SPIN_LIMIT = 1u << 18; // polls a wave makes at most before it gives up (FusedArgs::spin_limit)
+constexpr uint32_t CHAIN_WAIT_TICKS = 200000;   // and how long it waits at most: 2 ms of the 100 MHz clock
 constexpr uint32_t CHAIN_GROUP = 32;    // workgroups per group of the chain (at most 64)
 
 constexpr uint64_t CHAIN_FLAG_SHIFT = 62;
 constexpr uint64_t CHAIN_AGGREGATE = 1ull << CHAIN_FLAG_SHIFT; // value = rows of this workgroup
 constexpr uint64_t CHAIN_PREFIX = 2ull << CHAIN_FLAG_SHIFT;    // value = rows of this and all earlier workgroups
 constexpr uint64_t CHAIN_VALUE = (1ull << CHAIN_FLAG_SHIFT) - 1;
+constexpr uint64_t CHAIN_GAVE_UP = ~0ull; // chain_position: the wave ran out of patience, its place is not known
 
 /// The words through which the workgroups learn where their rows start; all zero on entry.
 struct Chain {
@@ -59,6 +64,7 @@ struct FusedArgs {
     Chain chain;
     FusedStatus* status; // zero on entry
     uint32_t spin_limit; // polls of the chain before a wave gives up; 0 makes every wait fail at once (tests)
+    uint32_t wait_ticks; // and the time it waits at most, in ticks of the 100 MHz clock
 };
 
 /// LDS of one wave.
@@ -361,10 +367,33 @@ __device__ __forceinline__ void chain_store(uint64_t* word, uint64_t value) {
     __hip_atomic_store(word, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-/// Bounded wait between two polls of the chain; returns false when patience ran out.
-__device__ __forceinline__ bool chain_wait(uint32_t& spins, uint32_t spin_limit, int lane, FusedStatus* status) {
-    spins += 1;
-    if (spins > spin_limit) {
+/// What a wave of the chain waits with: when it started waiting, how often it has polled.
+struct ChainPatience {
+    uint64_t since;
+    uint32_t spins;
+    uint32_t spin_limit;
+    uint32_t wait_ticks;
+};
+
+__device__ __forceinline__ ChainPatience chain_patience(uint32_t spin_limit, uint32_t wait_ticks) {
+    ChainPatience patience;
+    patience.since = wall_clock64();
+    patience.spins = 0;
+    patience.spin_limit = spin_limit;
+    patience.wait_ticks = wait_ticks;
+    return patience;
+}
+
+/// Bounded wait between two polls of the chain; returns false when patience ran out: after `wait_ticks` of waiting
+/// (the 100 MHz clock, the same on every compute unit whatever its own clock does), after `spin_limit` polls, or as
+/// soon as another wave of the launch has given up (the rows of the launch are void then, there is nothing to wait for).
+__device__ __forceinline__ bool chain_wait(ChainPatience& patience, int lane, FusedStatus* status) {
+    patience.spins += 1;
+    const bool someone_gave_up =
+        (patience.spins & 7u) == 0 && __hip_atomic_load(&status->chain_timeout, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
+    const bool out_of_patience =
+        patience.spins > patience.spin_limit || someone_gave_up || wall_clock64() - patience.since > patience.wait_ticks;
+    if (__ballot(out_of_patience) != 0) { // (the same answer for every lane of the wave)
         if (lane == 0) {
             atomicAdd(&status->chain_timeout, 1u);
         }
@@ -383,7 +412,7 @@ __device__ __forceinline__ bool chain_wait(uint32_t& spins, uint32_t spin_limit,
 /// rows of the earlier workgroups of their group. Every word carries its own flag, so no fences are needed.
 __device__ __forceinline__ uint64_t chain_position(
     const Chain& chain, uint32_t block, uint32_t n_blocks, uint64_t own_rows, int lane, FusedStatus* status,
-    uint32_t spin_limit
+    uint32_t spin_limit, uint32_t wait_ticks
 ) {
     if (lane == 0) {
         chain_store(&chain.blocks[block], CHAIN_AGGREGATE | own_rows);
@@ -392,7 +421,8 @@ __device__ __forceinline__ uint64_t chain_position(
     const uint32_t group_first = group * CHAIN_GROUP;
     const uint32_t member = block - group_first;
     const bool leader = member == CHAIN_GROUP - 1 || block == n_blocks - 1;
-    uint32_t spins = 0;
+    ChainPatience patience = chain_patience(spin_limit, wait_ticks);
+    bool gave_up = false;
 
     uint64_t group_before = 0;
     if (leader) {
@@ -404,7 +434,11 @@ __device__ __forceinline__ uint64_t chain_position(
                 word = chain_load(&chain.blocks[group_first + lane]);
             }
             rows_of_member = word & CHAIN_VALUE;
-            if (__ballot((word >> CHAIN_FLAG_SHIFT) == 0) == 0 || !chain_wait(spins, spin_limit, lane, status)) {
+            if (__ballot((word >> CHAIN_FLAG_SHIFT) == 0) == 0) {
+                break;
+            }
+            if (!chain_wait(patience, lane, status)) {
+                gave_up = true;
                 break;
             }
         }
@@ -443,7 +477,8 @@ __device__ __forceinline__ uint64_t chain_position(
                 nearest -= usable;
                 if (reaches_prefix) {
                     done = true;
-                } else if (usable == 0 && !chain_wait(spins, spin_limit, lane, status)) {
+                } else if (usable == 0 && !chain_wait(patience, lane, status)) {
+                    gave_up = true;
                     done = true;
                 }
             }
@@ -454,8 +489,9 @@ __device__ __forceinline__ uint64_t chain_position(
         if (lane == 0) {
             chain_store(&chain.bases[group], CHAIN_PREFIX | (group_before & CHAIN_VALUE));
         }
+        // (the words are published also by a leader that gave up: nobody should wait for them any longer)
         // rows of the earlier workgroups of this group: everything but the own rows
-        return group_before + (group_rows - own_rows);
+        return gave_up ? CHAIN_GAVE_UP : group_before + (group_rows - own_rows);
     }
 
     // ---- not the leader: wait for the group's base, then add the earlier members (all published by then)
@@ -465,8 +501,8 @@ __device__ __forceinline__ uint64_t chain_position(
             group_before = word & CHAIN_VALUE;
             break;
         }
-        if (!chain_wait(spins, spin_limit, lane, status)) {
-            break;
+        if (!chain_wait(patience, lane, status)) {
+            return CHAIN_GAVE_UP;
         }
     }
     uint64_t rows_of_member = 0;
@@ -696,16 +732,20 @@ __global__ __launch_bounds__(SEARCH_BLOCK) __attribute__((amdgpu_waves_per_eu(5,
         uint64_t before = 0;
         if (ORDERED) {
             // rows in work-item order: the workgroup chains with the earlier workgroups
-            before = chain_position(fargs.chain, blockIdx.x, gridDim.x, block_rows, lane, fargs.status, fargs.spin_limit);
+            before = chain_position(
+                fargs.chain, blockIdx.x, gridDim.x, block_rows, lane, fargs.status, fargs.spin_limit, fargs.wait_ticks
+            );
         } else if (lane == 0 && block_rows != 0) {
             // rows in order of arrival: no workgroup waits for another
             before = atomicAdd(&fargs.status->total_rows, static_cast<unsigned long long>(block_rows));
         }
-        const bool fits = before + block_rows <= args.capacity;
+        // (a workgroup that does not know its place writes nothing; the host reads `chain_timeout`)
+        const bool placed = !ORDERED || before != CHAIN_GAVE_UP;
+        const bool fits = placed && before + block_rows <= args.capacity;
         if (lane == 0) {
             shared.base = before;
             shared.writable = fits ? 1u : 0u;
-            if (!fits) {
+            if (placed && !fits) {
                 atomicAdd(&fargs.status->overflow, 1u);
             }
             if (ORDERED && blockIdx.x == gridDim.x - 1) {

@@ -138,6 +138,46 @@ struct HostGrid {
 constexpr double CELL_MARGIN = 1.0 + 1e-9;
 constexpr int32_t MAX_STENCIL_RADIUS = 500;
 
+// this header is read by the host compiler alone (tests) and by hipcc, where some of its functions also run in kernels
+#ifdef __HIPCC__
+#define VESIN_HOST_DEVICE __host__ __device__
+#else
+#define VESIN_HOST_DEVICE
+#endif
+
+/// Shrinks a grid of cells[0] x cells[1] x cells[2] cells (whole numbers, 1 at least) until it holds at most `most`
+/// cells (1 at least), all directions that have more than one cell by the same factor. A direction that the factor
+/// takes below one cell keeps one, and the others then shrink again: a long thin system (a stretched chain, a
+/// dissociating pair) ends up with cells along its length only. The buffers of the callers are sized by `most`, so
+/// the bound holds whatever the rounding of the roots does: the last loop takes single layers off the direction with
+/// the most cells.
+VESIN_HOST_DEVICE inline void limit_cells(double cells[3], double most) {
+    for (int round = 0; round < 3; round++) {
+        const double total = cells[0] * cells[1] * cells[2];
+        if (total <= most) {
+            return;
+        }
+        int wide = 0;
+        for (int d = 0; d < 3; d++) {
+            wide += cells[d] > 1.0 ? 1 : 0;
+        }
+        const double ratio = most / total;
+        const double shrink = wide == 3 ? ::cbrt(ratio) : wide == 2 ? ::sqrt(ratio) : ratio;
+        for (int d = 0; d < 3; d++) {
+            if (cells[d] > 1.0) {
+                cells[d] = ::fmax(::floor(cells[d] * shrink), 1.0);
+            }
+        }
+    }
+    while (cells[0] * cells[1] * cells[2] > most) {
+        const int widest = cells[0] >= cells[1] ? (cells[0] >= cells[2] ? 0 : 2) : (cells[1] >= cells[2] ? 1 : 2);
+        if (!(cells[widest] > 1.0)) {
+            return;
+        }
+        cells[widest] -= 1.0;
+    }
+}
+
 /// Choose the cell grid. `lo`/`hi` are the extrema of the fractional (projected) coordinates; they are only read
 /// for non-periodic directions. With `single_cell` every point goes to one cell and the stencil enumerates the
 /// periodic images directly (the brute-force and multi-image path).
@@ -189,16 +229,7 @@ inline HostGrid choose_grid(
     if (max_cells > 16777216.0) {
         max_cells = 16777216.0;
     }
-    double total = cells[0] * cells[1] * cells[2];
-    if (total > max_cells) {
-        double shrink = std::cbrt(max_cells / total);
-        for (int d = 0; d < 3; d++) {
-            cells[d] = std::floor(cells[d] * shrink);
-            if (cells[d] < 1.0) {
-                cells[d] = 1.0;
-            }
-        }
-    }
+    limit_cells(cells, max_cells);
 
     grid.n_cells = 1;
     for (int d = 0; d < 3; d++) {
@@ -224,13 +255,6 @@ inline HostGrid choose_grid(
     }
     return grid;
 }
-
-// this header is read by the host compiler alone (tests) and by hipcc, where the function below also runs in kernels
-#ifdef __HIPCC__
-#define VESIN_HOST_DEVICE __host__ __device__
-#else
-#define VESIN_HOST_DEVICE
-#endif
 
 /// Whether the stencil entry (dx, dy, dz) is too far from the centre cell to hold a neighbour, from the fields
 /// `choose_pruning` fills (GridParams::prune_edges).

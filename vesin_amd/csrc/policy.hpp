@@ -63,6 +63,39 @@ struct BoxGuess {
     }
 };
 
+constexpr int WAIT_REST = 64;        // calls that leave a launch with waiting workgroups alone after it gave up
+constexpr int WAIT_REST_MAX = 4096;  // and after it gave up many times in a row
+
+/// Some launches make workgroups wait for each other (the chain that places the rows of the single-pass search in
+/// work-item order, the meeting of a small system's one launch). That only advances while the workgroups that are
+/// waited for get to run, which holds on a GPU the launch has to itself and may not on one it shares with other
+/// streams or processes. Every such wait is bounded, and a launch whose waves gave up is followed by the passes that
+/// need no waiting; this is the bookkeeping that keeps a list from paying for the give-up on every call: after one,
+/// the list leaves that launch alone for WAIT_REST calls, and every further give-up in a row doubles that, up to
+/// WAIT_REST_MAX; a launch that went through brings the time back to WAIT_REST.
+struct WaitRest {
+    int rest = 0;
+    int next_rest = WAIT_REST;
+
+    /// Once per call that could use the launch: true while the list stays away from it.
+    bool resting() {
+        if (rest > 0) {
+            rest -= 1;
+            return true;
+        }
+        return false;
+    }
+
+    void gave_up() {
+        rest = next_rest;
+        next_rest = next_rest >= WAIT_REST_MAX / 2 ? WAIT_REST_MAX : 2 * next_rest;
+    }
+
+    void went_through() {
+        next_rest = WAIT_REST;
+    }
+};
+
 // ---------------------------------------------------------------------------------------------------------------
 // The search that writes a sorted list in order (ordered.cuh): how its work is cut into waves. Every choice gives
 // the same list; the figures are what the passes were measured at on one MI355X (256 compute units, 1024 SIMDs).

@@ -40,7 +40,9 @@
 namespace vesin_hip {
 
 constexpr uint32_t SMALL_POINTS = 2048;        // points (and cells, and work items) the largest shape takes
-constexpr uint32_t SMALL_SPINS = 1u << 12;     // polls of a workgroup that waits for the others (a few milliseconds)
+constexpr uint32_t SMALL_SPINS = 1u << 12;     // polls of a workgroup that waits for the others, at most
+constexpr uint32_t SMALL_WAIT_TICKS = 50000;   // and the time it waits at most: 500 us of the 100 MHz clock, 25 times
+                                               // what the whole launch takes when its workgroups run side by side
 constexpr uint32_t SMALL_GAVE_UP = 1u << 31;   // in SmallMeeting::arrived: a workgroup stopped waiting
 constexpr uint32_t SMALL_WORKGROUPS = 240;     // of a launch: fewer than there are compute units
 
@@ -538,7 +540,11 @@ __global__ __launch_bounds__(WAVES * WAVE) void small_system_kernel(SmallArgs ar
     }
 
     // ---- all workgroups meet. Once a wave's device-scope stores have completed they are what any device-scope
-    // load returns, so the workgroup's arrival only has to come after.
+    // load returns, so the workgroup's arrival only has to come after. This leans on two properties of this
+    // architecture (gfx9 family, gfx950 included) instead of release / acquire orderings, whose cache-wide write-back
+    // and invalidation doubled the launch's time when tried: vmcnt counts stores as well as loads, so vmcnt(0) means
+    // that every store this wave issued has been acknowledged by the L2 cache, and device-scope atomic stores and loads
+    // go to that cache, which all compute units of the device share.
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (t == 0) {
@@ -549,6 +555,7 @@ __global__ __launch_bounds__(WAVES * WAVE) void small_system_kernel(SmallArgs ar
         __hip_atomic_fetch_add(&args.meeting->arrived, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         uint32_t spins = 0;
         bool all = false;
+        const uint64_t since = wall_clock64();
         while (true) {
             uint32_t seen = __hip_atomic_load(&args.meeting->arrived, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if ((seen & SMALL_GAVE_UP) != 0) {
@@ -559,7 +566,7 @@ __global__ __launch_bounds__(WAVES * WAVE) void small_system_kernel(SmallArgs ar
                 break;
             }
             spins += 1;
-            if (spins > args.spin_limit) {
+            if (spins > args.spin_limit || wall_clock64() - since > SMALL_WAIT_TICKS) {
                 if (__hip_atomic_compare_exchange_strong(
                         &args.meeting->arrived, &seen, seen | SMALL_GAVE_UP, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
                         __HIP_MEMORY_SCOPE_AGENT
