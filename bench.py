@@ -371,14 +371,15 @@ def main():
 
 
 def other_configs(args, torch, np):
-    """Steady-state figures of the other configurations: 10 timed calls each after the list's first call and 3 more."""
+    """Steady-state figures of the other configurations: after the list's first call and 5 more, a timed region of 20
+    calls, then 20 calls timed one by one (the median of those is `ms_per_call`) and 20 between HIP events."""
     results = []
     names = [name for name in ["config0", "config2", "config3", "config3_single", "config4a", "config4b"] if name != args.config]
     if args.config == "config1":
         names += ["config1_shuffled", "config1_box_changes", "config1_sorted"]
     for name in names:
         workload = Workload(name, args.replicas)
-        measured = measure(workload, 10, 3, torch, np)
+        measured = measure(workload, 20, 5, torch, np)
         ms = measured["ms_median"]
         entry = {
             "name": name,

@@ -142,6 +142,50 @@ int VESIN_API vesin_hip_neighbors_on_stream(
     const char** error_message
 );
 
+/* vesin_hip_neighbors_on_stream in two halves, for callers that want to queue more work behind the list without
+ * the host waiting in between (a molecular dynamics step that evaluates forces from the list on the same stream).
+ * The syncs this takes out of the caller's way are the reference's own (vesin/src/vesin_cuda.cpp:793-803, :899: every
+ * call there ends with a device synchronisation); there is no counterpart of the two entry points in the reference.
+ *
+ * vesin_hip_neighbors_enqueue does everything a call can do before it needs an answer from the GPU, and returns.
+ * For a list in its steady state (same number of points, cutoff and options as the call before, a box that did not
+ * change, arrays that hold the rows) that is the whole calculation: cell list, search and rows are queued on
+ * `stream`, into the arrays `neighbors` already has, whose addresses do not change before vesin_hip_neighbors_collect.
+ * Otherwise (first call of a list, another box, another system) only the first kernels are queued and the rest is
+ * done by vesin_hip_neighbors_collect; the call may then also block, as every call that has to allocate does.
+ *
+ *   device_length   receives the address of a 64-bit word in the memory of the GPU (the same for every call on this
+ *                   list): work queued on `stream` after this call finds there the number of rows when the queued
+ *                   kernels left the complete list in the arrays, and VESIN_HIP_ROWS_PENDING when they did not
+ *                   (then nothing may be read from the arrays before vesin_hip_neighbors_collect has returned)
+ *
+ * vesin_hip_neighbors_collect waits for the kernels of the queued call (not for what was queued behind them),
+ * looks at what they found and, if the list is not complete yet, completes it as vesin_hip_neighbors_on_stream
+ * would have (growing the arrays, the general search), on the stream of the queued call. On return `length` and
+ * the arrays are final, the device word holds `length`, and errors of the calculation are reported here, with the
+ * usual message ownership. Any host thread may call it.
+ *
+ * Between the two calls the inputs (`points`, `box`, `periodic`) must stay as they are, `neighbors` must not be
+ * passed to any other entry point (they refuse it; vesin_free completes the queued call first), and the values in
+ * the struct are those of the call before. With options.skin > 0 the call is queued as far as the cache's own
+ * bookkeeping allows, which is usually not at all. */
+#define VESIN_HIP_ROWS_PENDING (~0ull)
+
+int VESIN_API vesin_hip_neighbors_enqueue(
+    const double (*points)[3],
+    size_t n_points,
+    const double box[3][3],
+    const bool periodic[3],
+    struct VesinDevice device,
+    struct VesinOptions options,
+    struct VesinNeighborList* neighbors,
+    void* stream,
+    const unsigned long long** device_length,
+    const char** error_message
+);
+
+int VESIN_API vesin_hip_neighbors_collect(struct VesinNeighborList* neighbors, const char** error_message);
+
 /* vesin_hip_neighbors_on_stream for callers that cannot allocate device memory (loops that must not reach
  * hipMalloc, harnesses that forbid it): no counterpart in the reference. The rows go to arrays of the caller's and
  * the call allocates and frees nothing, on the device or through any library.

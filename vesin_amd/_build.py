@@ -26,15 +26,42 @@ FLAGS = [
     "-target-feature",
     "-Xclang",
     "-packed-fp32-ops",
-    # arrays indexed with wave-uniform values (the hit columns of the single-pass search: 32 registers) stay in
-    # registers whatever occupancy a kernel asks for; by default the compiler moves an array larger than a quarter of
-    # the kernel's register budget to scratch memory
-    "-mllvm",
-    "-amdgpu-promote-alloca-to-vector-vgpr-ratio=1",
-    "-mllvm",
-    "-amdgpu-promote-alloca-to-vector-max-regs=64",
     "-Wno-unused-command-line-argument",
-] + os.environ.get("VESIN_EXTRA_FLAGS", "").split()
+]
+
+# Arrays indexed with wave-uniform values (the hit columns of the single-pass search: 32 registers) stay in registers
+# whatever occupancy a kernel asks for; by default the compiler moves an array larger than a quarter of the kernel's
+# register budget to scratch memory. These are options of the compiler's back end, not of its command line: another
+# release may not know them, and an unknown one is an error. They are tried on an empty kernel first and left out when
+# the compiler refuses them (the kernels are as correct without them, only slower).
+TUNING_FLAGS = [
+    ["-mllvm", "-amdgpu-promote-alloca-to-vector-vgpr-ratio=1"],
+    ["-mllvm", "-amdgpu-promote-alloca-to-vector-max-regs=64"],
+]
+
+
+def _accepted(hipcc, flags):
+    import tempfile
+
+    with tempfile.TemporaryDirectory() as scratch:
+        source = os.path.join(scratch, "probe.hip")
+        with open(source, "w") as out:
+            out.write("#include <hip/hip_runtime.h>\n__global__ void probe() {}\n")
+        command = [hipcc, "--offload-arch=gfx950", "-c", *flags, source, "-o", os.path.join(scratch, "probe.o")]
+        return subprocess.run(command, capture_output=True, text=True).returncode == 0
+
+
+def extra_flags():
+    """What the environment adds to the command line, for developers only: VESIN_EXTRA_FLAGS (measurements with other
+    code generation) is read when VESIN_BUILD_DEBUG=1 says that this is meant, so that a variable left over in a
+    user's environment does not change the code of a library whose results are compared bit for bit;
+    VESIN_HIP_ROCTX=1 compiles the named ranges for profilers in (see TraceRange in driver.hip)."""
+    flags = []
+    if os.environ.get("VESIN_BUILD_DEBUG") == "1":
+        flags += os.environ.get("VESIN_EXTRA_FLAGS", "").split()
+    if os.environ.get("VESIN_HIP_ROCTX") == "1":
+        flags += ["-DVESIN_HIP_ROCTX", "-L/opt/rocm/lib", "-lrocprofiler-sdk-roctx", "-Wl,-rpath,/opt/rocm/lib"]
+    return flags
 
 
 TORCH_SOURCE = os.path.join(CSRC, "torch", "neighbor_list_class.cpp")
@@ -82,12 +109,22 @@ def build(verbose=False):
     if not os.path.exists(hipcc):
         hipcc = "hipcc"
     os.makedirs(LIB_DIR, exist_ok=True)
-    command = [hipcc, *FLAGS, "-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
+    flags = list(FLAGS)
+    for tuning in TUNING_FLAGS:
+        if _accepted(hipcc, tuning):
+            flags += tuning
+        elif verbose:
+            print("left out (the compiler does not know it): " + " ".join(tuning))
+    flags += extra_flags()
+    command = [hipcc, *flags, "-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
     command += [os.path.join(CSRC, source) for source in SOURCES]
     command += ["-o", LIB_PATH]
     result = subprocess.run(command, capture_output=True, text=True)
     if result.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + result.stdout + result.stderr)
+    # what the library was built with, next to it
+    with open(LIB_PATH + ".flags", "w") as record:
+        record.write(" ".join(flags) + "\n")
     if verbose:
         print(result.stderr)
     return LIB_PATH

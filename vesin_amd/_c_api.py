@@ -144,6 +144,21 @@ def get_library():
             ctypes.c_void_p,
             ctypes.POINTER(ctypes.c_char_p),
         ]
+        lib.vesin_hip_neighbors_enqueue.restype = ctypes.c_int
+        lib.vesin_hip_neighbors_enqueue.argtypes = [
+            ctypes.c_void_p,
+            ctypes.c_size_t,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            VesinDevice,
+            VesinOptions,
+            ctypes.POINTER(VesinNeighborList),
+            ctypes.c_void_p,
+            ctypes.POINTER(ctypes.c_void_p),
+            ctypes.POINTER(ctypes.c_char_p),
+        ]
+        lib.vesin_hip_neighbors_collect.restype = ctypes.c_int
+        lib.vesin_hip_neighbors_collect.argtypes = [ctypes.POINTER(VesinNeighborList), ctypes.POINTER(ctypes.c_char_p)]
         lib.vesin_hip_neighbors_no_alloc.restype = ctypes.c_int
         lib.vesin_hip_neighbors_no_alloc.argtypes = [
             ctypes.c_void_p,

@@ -22,6 +22,8 @@ static int fail(const char** error_message, const char* text) {
     return EXIT_FAILURE;
 }
 
+/// vesin_neighbors and its variants on a stream. `device_length` not null: the call is queued only (see
+/// vesin_hip_neighbors_enqueue) and the address of its device word goes there.
 static int neighbors_on(
     const double (*points)[3],
     size_t n_points,
@@ -31,7 +33,8 @@ static int neighbors_on(
     VesinOptions options,
     VesinNeighborList* neighbors,
     void* stream,
-    const char** error_message
+    const char** error_message,
+    const unsigned long long** device_length = nullptr
 ) {
     if (error_message == nullptr) {
         return EXIT_FAILURE;
@@ -74,7 +77,11 @@ static int neighbors_on(
             if (neighbors->device.type == VesinUnknownDevice) {
                 neighbors->device = device;
             }
-            vesin_hip::neighbors(points, n_points, box, periodic, options, *neighbors, stream);
+            if (device_length != nullptr) {
+                *device_length = vesin_hip::neighbors_enqueue(points, n_points, box, periodic, options, *neighbors, stream);
+            } else {
+                vesin_hip::neighbors(points, n_points, box, periodic, options, *neighbors, stream);
+            }
         } else if (device.type == VesinCPU) {
             throw std::runtime_error(
                 "this library only implements GPU devices (VesinCUDA, i.e. HIP on ROCm); there is no CPU engine in it"
@@ -121,6 +128,56 @@ extern "C" int vesin_hip_neighbors_on_stream(
     const char** error_message
 ) {
     return neighbors_on(points, n_points, box, periodic, device, options, neighbors, stream, error_message);
+}
+
+extern "C" int vesin_hip_neighbors_enqueue(
+    const double (*points)[3],
+    size_t n_points,
+    const double box[3][3],
+    const bool periodic[3],
+    VesinDevice device,
+    VesinOptions options,
+    VesinNeighborList* neighbors,
+    void* stream,
+    const unsigned long long** device_length,
+    const char** error_message
+) {
+    if (error_message == nullptr) {
+        return EXIT_FAILURE;
+    }
+    if (device_length == nullptr) {
+        return fail(error_message, "`device_length` can not be a NULL pointer");
+    }
+    if (device.type != VesinCUDA) {
+        return fail(error_message, "a calculation is only queued on a GPU device (VesinCUDA, i.e. HIP on ROCm)");
+    }
+    return neighbors_on(points, n_points, box, periodic, device, options, neighbors, stream, error_message, device_length);
+}
+
+extern "C" int vesin_hip_neighbors_collect(VesinNeighborList* neighbors, const char** error_message) {
+    if (error_message == nullptr) {
+        return EXIT_FAILURE;
+    }
+    if (neighbors == nullptr) {
+        return fail(error_message, "`neighbors` can not be a NULL pointer");
+    }
+    if (neighbors->device.type != VesinCUDA) {
+        return fail(error_message, "no calculation was queued on this list");
+    }
+    try {
+        vesin_hip::neighbors_collect(*neighbors);
+    } catch (const std::bad_alloc&) {
+        LAST_ERROR = "failed to allocate memory";
+        *error_message = LAST_ERROR.c_str();
+        return EXIT_FAILURE;
+    } catch (const std::exception& e) {
+        LAST_ERROR = e.what();
+        *error_message = LAST_ERROR.c_str();
+        return EXIT_FAILURE;
+    } catch (...) {
+        return fail(error_message, "fatal error: unknown type thrown as exception");
+    }
+    return EXIT_SUCCESS;
 }
 
 extern "C" int vesin_hip_neighbors_no_alloc(

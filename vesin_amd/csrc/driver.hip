@@ -7,6 +7,8 @@
 // vesin/src/cuda_buffers.cpp.
 #include <hip/hip_runtime.h>
 
+#include <ucontext.h>
+
 #include <cerrno>
 #include <cmath>
 #include <cstddef>
@@ -17,6 +19,7 @@
 #include <algorithm>
 #include <atomic>
 #include <exception>
+#include <functional>
 #include <stdexcept>
 #include <memory>
 #include <mutex>
@@ -46,6 +49,30 @@ namespace vesin_hip {
             throw std::runtime_error(std::string("HIP error in ") + #expr + ": " + hipGetErrorString(status_));      \
         }                                                                                                            \
     } while (false)
+
+// Named ranges on a profiler's timeline (rocprofv3 --marker-trace), around the stages that VesinHipTimings names.
+// Compiled in with -DVESIN_HIP_ROCTX (python -m vesin_amd._build with VESIN_HIP_ROCTX=1) and absent otherwise: the
+// counterpart of the reference's optional NVTX ranges (vesin/src/vesin_cuda.cpp:16-28). A range covers the host
+// side of a stage, i.e. the launches; the kernels it launched follow on the stream's own line of the timeline.
+#ifdef VESIN_HIP_ROCTX
+#include <rocprofiler-sdk-roctx/roctx.h>
+struct TraceRange {
+    explicit TraceRange(const char* name) { roctxRangePush(name); }
+    ~TraceRange() { roctxRangePop(); }
+    /// Ends the stage that is open and starts the next one.
+    void next(const char* name) {
+        roctxRangePop();
+        roctxRangePush(name);
+    }
+    TraceRange(const TraceRange&) = delete;
+    TraceRange& operator=(const TraceRange&) = delete;
+};
+#else
+struct TraceRange {
+    explicit TraceRange(const char*) {}
+    void next(const char*) {}
+};
+#endif
 
 static std::atomic<bool> TIMINGS_ENABLED{false};
 
@@ -314,6 +341,7 @@ constexpr int DIRECT_REST = 1024;
 
 constexpr int SINGLE_PASS_REST = 64;
 constexpr size_t BOX_BYTES = 75; // 9 doubles and 3 flags, as fetch_box lays them out
+constexpr size_t BOX_BYTES_PADDED = 80;
 
 enum Stage { T_START = 0, T_CELLS, T_COUNT, T_SCAN, T_WRITE_BEGIN, T_WRITE, T_SORT, T_STAGES };
 
@@ -435,6 +463,160 @@ struct BatchSetup {
     size_t first_pair_capacity = 0;
 };
 
+/// A call that stops where the host would wait for the GPU and goes on later (vesin_hip_neighbors_enqueue /
+/// vesin_hip_neighbors_collect). The call runs on a stack of its own: where it first has to wait for the stream
+/// (HipExtras::wait), control goes back to whoever started it, with everything up to there queued; resumed, it waits
+/// and carries on as the blocking call would have, every decision and every way back included. Nothing that is
+/// bound to a host thread is held across the stop (no lock, no exception in flight), so the call may be resumed by
+/// another thread.
+struct SuspendedCall {
+    static constexpr size_t STACK_BYTES = size_t(1) << 20;
+
+    ucontext_t starter = {};
+    ucontext_t call = {};
+    std::unique_ptr<unsigned char[]> stack;
+    std::function<void()> body;
+    std::exception_ptr error;
+    bool stop_at_next_wait = false;
+    bool finished = true;
+    hipEvent_t reached = nullptr; // recorded where the call stopped: resuming waits for that, not for what the caller
+                                  // queued behind it
+
+    SuspendedCall() = default;
+    SuspendedCall(const SuspendedCall&) = delete;
+    SuspendedCall& operator=(const SuspendedCall&) = delete;
+
+    ~SuspendedCall() {
+        if (reached != nullptr) {
+            (void)hipEventDestroy(reached);
+        }
+    }
+
+    static void entry(unsigned int low, unsigned int high) {
+        auto* self = reinterpret_cast<SuspendedCall*>((static_cast<uintptr_t>(high) << 32) | static_cast<uintptr_t>(low));
+        try {
+            self->body();
+        } catch (...) {
+            self->error = std::current_exception();
+        }
+        self->finished = true;
+        // (back to the starter through uc_link)
+    }
+
+    /// Runs `work` until it stops at its first wait or ends.
+    void start(std::function<void()> work) {
+        if (stack == nullptr) {
+            stack.reset(new unsigned char[STACK_BYTES]);
+        }
+        if (reached == nullptr) {
+            HIP_CHECK(hipEventCreateWithFlags(&reached, hipEventDisableTiming));
+        }
+        body = std::move(work);
+        error = nullptr;
+        finished = false;
+        stop_at_next_wait = true;
+        if (getcontext(&call) != 0) {
+            throw std::runtime_error("getcontext failed");
+        }
+        call.uc_stack.ss_sp = stack.get();
+        call.uc_stack.ss_size = STACK_BYTES;
+        call.uc_link = &starter;
+        const uintptr_t self = reinterpret_cast<uintptr_t>(this);
+        makecontext(
+            &call, reinterpret_cast<void (*)()>(&SuspendedCall::entry), 2, static_cast<unsigned int>(self & 0xFFFFFFFFu),
+            static_cast<unsigned int>(self >> 32)
+        );
+        resume();
+    }
+
+    /// Carries on until the call stops again or ends.
+    void resume() {
+        if (swapcontext(&starter, &call) != 0) {
+            throw std::runtime_error("swapcontext failed");
+        }
+    }
+
+    /// From inside the call: back to whoever started or resumed it.
+    void stop() {
+        if (swapcontext(&call, &starter) != 0) {
+            throw std::runtime_error("swapcontext failed");
+        }
+    }
+};
+
+/// The value of the device word of a queued call (see vesin_hip_neighbors_enqueue) while the rows are not known to
+/// be complete.
+constexpr unsigned long long ROWS_PENDING = ~0ull;
+
+/// What tells, on the device, whether the kernels queued by a call left the complete list in the arrays.
+struct QueuedOutcome {
+    int kind;                          // 0: single-pass search, 1: small system in one launch, 2: in-order search
+    const FusedStatus* fused;          // (0)
+    const DeviceStatus* build;         // (0, 2)
+    const OrderedHostStatus* small;    // (1) what workgroup 0 of the launch reported
+    const OrderedStatus* ordered;      // (2)
+    const uint64_t* ordered_total;     // (2)
+    unsigned long long capacity;       // rows the arrays hold
+    unsigned long long row_limit;      // more rows than this are an error of the caller's making (0: no limit)
+    int one_pass_cells;                // (0) the cells were built with a fixed number of slots each
+    int guessed_extent;                // (0) the grid came from the extent of the call before
+    unsigned char used_box[BOX_BYTES_PADDED]; // the box and flags the host picked the grid from
+};
+
+/// Last kernel of the queued part of a call: the device word gets the number of rows if the list is complete in the
+/// arrays, which is the case when the kernels before found what the host is going to check once it looks (the same
+/// conditions, in the same words), and stays ROWS_PENDING otherwise.
+__global__ void publish_queued_length(
+    QueuedOutcome outcome, const double* __restrict__ box, const bool* __restrict__ periodic, unsigned long long* word
+) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) {
+        return;
+    }
+    bool complete = true;
+    for (int k = 0; k < 9; k++) {
+        double used;
+        memcpy(&used, outcome.used_box + 8 * k, 8);
+        unsigned long long a, b;
+        memcpy(&a, &used, 8);
+        const double now = box[k];
+        memcpy(&b, &now, 8);
+        complete = complete && a == b;
+    }
+    for (int d = 0; d < 3; d++) {
+        complete = complete && (outcome.used_box[72 + d] != 0) == periodic[d];
+    }
+    unsigned long long rows = 0;
+    if (outcome.kind == 0) {
+        const FusedStatus found = *outcome.fused;
+        rows = found.total_rows;
+        complete = complete && found.general == 0 && found.overflow == 0 && found.chain_timeout == 0 && found.deferred == 0 &&
+                   outcome.build->first_bad_coordinate == 0xFFFFFFFFu &&
+                   (outcome.one_pass_cells == 0 || outcome.build->crowded_cells == 0) &&
+                   (outcome.guessed_extent == 0 || outcome.build->far_outside == 0);
+    } else if (outcome.kind == 1) {
+        const OrderedHostStatus report = *outcome.small;
+        rows = report.total_rows;
+        complete = complete && report.found.gave_up == 0 && report.found.max_rows <= ORDERED_MAX_ROWS &&
+                   report.found.max_candidates <= ORDERED_CANDIDATES && report.found.unsuitable == 0 &&
+                   report.first_bad_coordinate == 0xFFFFFFFFu && rows <= outcome.capacity;
+    } else {
+        const OrderedStatus found = *outcome.ordered;
+        rows = *outcome.ordered_total;
+        complete = complete && found.max_rows <= ORDERED_MAX_ROWS && found.max_candidates <= ORDERED_CANDIDATES &&
+                   found.unsuitable == 0 && outcome.build->first_bad_coordinate == 0xFFFFFFFFu && rows <= outcome.capacity;
+    }
+    if (outcome.row_limit != 0 && rows > outcome.row_limit) {
+        complete = false;
+    }
+    *word = complete ? rows : ROWS_PENDING;
+}
+
+__global__ void set_queued_length(unsigned long long* word, unsigned long long value) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        *word = value;
+    }
+}
+
 struct HipExtras {
     int device_id = 0;
     BatchSetup batch;
@@ -482,6 +664,14 @@ struct HipExtras {
     bool timings_valid = false;
     VesinHipTimings timings = {};
     VerletCache* verlet = nullptr;    // only while the caller asks for a skin
+    // vesin_hip_neighbors_enqueue / _collect: the call that stopped at its first wait, and the device word that tells
+    // kernels queued behind it whether the rows are complete (made when first needed)
+    SuspendedCall* queued = nullptr;
+    bool enqueued = false;            // a call was queued and not collected yet
+    hipStream_t queued_stream = nullptr;
+    unsigned long long* d_queued_length = nullptr;
+    bool length_published = false;    // the kernels of the queued part were followed by the one that fills that word
+    bool queued_part_sufficed = false; // ... and the host found, like that kernel, that they left the complete list
 
     HipExtras() = default;
     HipExtras(const HipExtras&) = delete;
@@ -490,6 +680,8 @@ struct HipExtras {
     /// Wait for the stream; afterwards `mail` holds what the kernels queued before this call reported, and the first
     /// `n_bounds` slots of the bounding pass. (A block in device memory is copied piece by piece: a few hundred bytes
     /// for most waits, where the whole block is 20 KB that the runtime would stage on every wait.)
+    /// A queued call (see SuspendedCall) stops at its first wait and, once resumed, waits for what it had queued up
+    /// to here only.
     void wait(hipStream_t stream, size_t n_bounds = 0) {
         if (mail_device != mail) {
             HIP_CHECK(hipMemcpyAsync(mail, mail_device, offsetof(Mailbox, bounds), hipMemcpyDeviceToHost, stream));
@@ -499,11 +691,35 @@ struct HipExtras {
                 ));
             }
         }
+        if (queued != nullptr && queued->stop_at_next_wait) {
+            queued->stop_at_next_wait = false;
+            HIP_CHECK(hipEventRecord(queued->reached, stream));
+            queued->stop();
+            HIP_CHECK(hipEventSynchronize(queued->reached));
+            return;
+        }
         HIP_CHECK(hipStreamSynchronize(stream));
+    }
+
+    /// The kernels queued so far leave the complete list in the arrays if `outcome` says so: the device word of a
+    /// queued call is told, if this is the part of the call that is queued (only such calls pay for the launch).
+    /// Returns whether it did: the caller then says, once it has looked, whether the host came to the same conclusion
+    /// (`queued_part_sufficed`).
+    bool publish_length(const QueuedOutcome& outcome, const double* box, const bool* periodic, hipStream_t stream) {
+        if (queued != nullptr && queued->stop_at_next_wait) {
+            hipLaunchKernelGGL(publish_queued_length, dim3(1), dim3(1), 0, stream, outcome, box, periodic, d_queued_length);
+            length_published = true;
+            return true;
+        }
+        return false;
     }
 
     ~HipExtras() {
         delete verlet;
+        delete queued;
+        if (d_queued_length != nullptr) {
+            (void)hipFree(d_queued_length);
+        }
         work.release();
         sort_work.release();
         batch.kept_boxes.release();
@@ -793,6 +1009,60 @@ void direct_neighbors(
 
 } // namespace
 
+namespace {
+
+/// The call itself, on a list that has its state and whose inputs were checked, with the list's device current.
+void run_call(
+    const double (*points)[3], size_t n_points, const double box[3][3], const bool periodic[3], VesinOptions options,
+    VesinNeighborList& neighbors, HipExtras& extras, hipStream_t stream
+) {
+    const TraceRange whole_call(options.skin > 0.0 ? "vesin_neighbors (skin)" : "vesin_neighbors");
+    extras.timings_valid = false;
+    if (options.skin > 0.0) {
+        verlet_neighbors(points, n_points, box, periodic, options, neighbors, extras, stream);
+        return;
+    }
+    if (extras.verlet != nullptr) {
+        // no skin any more: the cache goes, like in the reference (vesin/src/cpu_cell_list.cpp:235-238)
+        delete extras.verlet;
+        extras.verlet = nullptr;
+    }
+    direct_neighbors(points, n_points, box, periodic, options, neighbors, extras, stream);
+}
+
+void refuse_while_queued(const HipExtras& extras) {
+    if (extras.enqueued) {
+        throw std::runtime_error(
+            "a calculation queued with vesin_hip_neighbors_enqueue is pending on this list: call "
+            "vesin_hip_neighbors_collect first"
+        );
+    }
+}
+
+/// After the queued call ran to its end: hand on its error, and make the device word say what `length` says unless
+/// the queued kernels did that themselves.
+void finish_queued(VesinNeighborList& neighbors, HipExtras& extras, hipStream_t stream) {
+    SuspendedCall& call = *extras.queued;
+    extras.enqueued = false;
+    call.stop_at_next_wait = false;
+    call.body = nullptr;
+    if (call.error != nullptr) {
+        std::exception_ptr error = call.error;
+        call.error = nullptr;
+        std::rethrow_exception(error);
+    }
+    if (!(extras.length_published && extras.queued_part_sufficed)) {
+        hipLaunchKernelGGL(
+            set_queued_length, dim3(1), dim3(1), 0, stream, extras.d_queued_length,
+            static_cast<unsigned long long>(neighbors.length)
+        );
+        HIP_CHECK(hipGetLastError());
+        HIP_CHECK(hipStreamSynchronize(stream));
+    }
+}
+
+} // namespace
+
 void neighbors(
     const double (*points)[3],
     size_t n_points,
@@ -809,18 +1079,63 @@ void neighbors(
 
     const DeviceGuard guard(device_id);
     HipExtras& extras = extras_of(neighbors);
-    extras.timings_valid = false;
+    refuse_while_queued(extras);
+    run_call(points, n_points, box, periodic, options, neighbors, extras, stream);
+}
 
-    if (options.skin > 0.0) {
-        verlet_neighbors(points, n_points, box, periodic, options, neighbors, extras, stream);
-        return;
+const unsigned long long* neighbors_enqueue(
+    const double (*points)[3],
+    size_t n_points,
+    const double box[3][3],
+    const bool periodic[3],
+    VesinOptions options,
+    VesinNeighborList& neighbors,
+    void* caller_stream
+) {
+    hipStream_t stream = static_cast<hipStream_t>(caller_stream);
+    const int device_id = neighbors.device.device_id;
+    check_inputs(points, n_points, box, periodic, device_id);
+
+    const DeviceGuard guard(device_id);
+    HipExtras& extras = extras_of(neighbors);
+    refuse_while_queued(extras);
+    if (extras.d_queued_length == nullptr) {
+        HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&extras.d_queued_length), 256));
     }
-    if (extras.verlet != nullptr) {
-        // no skin any more: the cache goes, like in the reference (vesin/src/cpu_cell_list.cpp:235-238)
-        delete extras.verlet;
-        extras.verlet = nullptr;
+    if (extras.queued == nullptr) {
+        extras.queued = new SuspendedCall();
     }
-    direct_neighbors(points, n_points, box, periodic, options, neighbors, extras, stream);
+    // whatever was queued behind an earlier call has read its word by the time this one is overwritten: same stream,
+    // or the caller's own ordering between streams
+    hipLaunchKernelGGL(set_queued_length, dim3(1), dim3(1), 0, stream, extras.d_queued_length, ROWS_PENDING);
+    HIP_CHECK(hipGetLastError());
+    extras.length_published = false;
+    extras.queued_part_sufficed = false;
+    extras.enqueued = true;
+    extras.queued_stream = stream;
+    VesinNeighborList* list = &neighbors;
+    HipExtras* state = &extras;
+    extras.queued->start([=]() { run_call(points, n_points, box, periodic, options, *list, *state, stream); });
+    if (extras.queued->finished) {
+        // nothing to wait for (no points), or an error before the first wait
+        finish_queued(neighbors, extras, stream);
+    }
+    return extras.d_queued_length;
+}
+
+void neighbors_collect(VesinNeighborList& neighbors) {
+    auto* extras = static_cast<HipExtras*>(neighbors.opaque);
+    if (extras == nullptr || extras->queued == nullptr) {
+        throw std::runtime_error("no calculation was queued on this list");
+    }
+    if (!extras->enqueued) {
+        return; // the queued call ended inside vesin_hip_neighbors_enqueue already, or was collected
+    }
+    const DeviceGuard guard(neighbors.device.device_id);
+    if (!extras->queued->finished) {
+        extras->queued->resume();
+    }
+    finish_queued(neighbors, *extras, extras->queued_stream);
 }
 
 namespace {
@@ -890,7 +1205,12 @@ bool compute(
         }
         extras.have_events = true;
     }
+    // (the stages of VesinHipTimings, by the stage that each mark ends)
+    static const char* const STAGE_AFTER[T_STAGES] = {"cell build", "search", "scan", "after the scan",
+                                                       "write", "sort", "end of call"};
+    TraceRange stage_range(speculate ? "set-up (box of the call before)" : "set-up (box read from the device)");
     auto mark = [&](Stage stage) {
+        stage_range.next(STAGE_AFTER[stage]);
         if (timed) {
             HIP_CHECK(hipEventRecord(extras.events[stage], stream));
         }
@@ -1247,6 +1567,17 @@ bool compute(
         }
     };
 
+    // (for a queued call: see HipExtras::publish_length)
+    auto queued_outcome = [&](int kind) {
+        QueuedOutcome outcome = {};
+        outcome.kind = kind;
+        outcome.build = extras.d_status;
+        outcome.capacity = extras.capacity;
+        outcome.row_limit = pair_limit != 0 ? n_points * pair_limit : 0;
+        std::memcpy(outcome.used_box, used_box, BOX_BYTES);
+        return outcome;
+    };
+
     // ---- small systems with arrays from earlier calls: cell list, counting, scan, report to the host and writing
     // in one launch (small_system_kernel). Its workgroups wait for each other, which needs all of them resident at
     // once; when they were not, or the system does not suit that launch, or the rows do not fit, the call goes on
@@ -1295,6 +1626,12 @@ bool compute(
         fetched = true;
         mark(T_CELLS);
         mark(T_WRITE);
+        bool published_here = false;
+        {
+            QueuedOutcome outcome = queued_outcome(1);
+            outcome.small = &extras.mail_device->ordered;
+            published_here = extras.publish_length(outcome, reinterpret_cast<const double*>(box), periodic, stream);
+        }
         extras.wait(stream, any_open ? 1 : 0);
         if (!box_was_right()) {
             return false;
@@ -1315,6 +1652,7 @@ bool compute(
         if (suitable && found.total_rows <= extras.capacity) {
             extras.meeting_rest.went_through();
             check_pair_limit(found.total_rows);
+            extras.queued_part_sufficed = published_here;
             HIP_CHECK(hipGetLastError());
             neighbors.length = found.total_rows;
             if (any_open) {
@@ -1491,6 +1829,14 @@ bool compute(
         hipLaunchKernelGGL(kernel, dim3(blocks), dim3(SEARCH_BLOCK), 0, stream, fargs, g);
         mark(T_WRITE);
         hipLaunchKernelGGL(publish_fused_status, dim3(1), dim3(1), 0, stream, extras.d_status, fused_status, &extras.mail_device->fused);
+        bool published_here = false;
+        {
+            QueuedOutcome outcome = queued_outcome(0);
+            outcome.fused = fused_status;
+            outcome.one_pass_cells = direct_cells ? 1 : 0;
+            outcome.guessed_extent = guessed_grid ? 1 : 0;
+            published_here = extras.publish_length(outcome, reinterpret_cast<const double*>(box), periodic, stream);
+        }
         extras.wait(stream, guessed_grid ? bounding_blocks : 0);
         if (!box_was_right()) {
             return false;
@@ -1565,6 +1911,7 @@ bool compute(
             }
             HIP_CHECK(hipGetLastError());
             neighbors.length = result.total_rows;
+            extras.queued_part_sufficed = published_here && result.deferred == 0;
             if (ordered) {
                 extras.chain_rest.went_through();
             }
@@ -1647,6 +1994,7 @@ bool compute(
         // fit, and writes nothing otherwise. One round trip to the host instead of two.
         const bool early_write = extras.capacity > 0;
         size_t early_capacity = 0;
+        bool published_here = false;
         if (early_write) {
             size_outputs(neighbors, extras, 0, options);
             early_capacity = extras.capacity;
@@ -1686,6 +2034,11 @@ bool compute(
                 launch_write();
                 mark(T_WRITE);
                 oargs.publish_to = nullptr;
+                QueuedOutcome outcome = queued_outcome(2);
+                outcome.ordered = ordered_status;
+                outcome.ordered_total = first_row_of_point + n_points;
+                outcome.capacity = early_capacity;
+                published_here = extras.publish_length(outcome, reinterpret_cast<const double*>(box), periodic, stream);
             } else {
                 hipLaunchKernelGGL(
                     publish_ordered_status, dim3(1), dim3(1), 0, stream,
@@ -1732,6 +2085,7 @@ bool compute(
                 mark(T_SORT);
                 HIP_CHECK(hipStreamSynchronize(stream));
             } else {
+                extras.queued_part_sufficed = published_here;
                 mark(T_SORT);
                 if (timed) {
                     HIP_CHECK(hipStreamSynchronize(stream));
@@ -2127,6 +2481,7 @@ void neighbors_batch(
 
     const DeviceGuard guard(device_id);
     HipExtras& extras = extras_of(neighbors);
+    refuse_while_queued(extras);
     extras.timings_valid = false;
     extras.guess.have_box = false; // the work buffers of the single-system path are about to be reused
     hipStream_t stream = static_cast<hipStream_t>(caller_stream);
@@ -2185,6 +2540,7 @@ bool batch_attempt(
     const bool (*periodic)[3], VesinOptions options, VesinNeighborList& neighbors, size_t* first_pair,
     HipExtras& extras, bool speculate, hipStream_t stream
 ) {
+    const TraceRange whole_call(speculate ? "vesin_hip_neighbors_batch (grids of the call before)" : "vesin_hip_neighbors_batch");
     const size_t n_points = first_point[n_systems];
     const size_t pair_limit = pairs_per_point_limit();
     BatchSetup& setup = extras.batch;
@@ -2840,6 +3196,18 @@ void neighbors_no_alloc(
 
 void free_neighbors(VesinNeighborList& neighbors) {
     const DeviceGuard guard(neighbors.device.device_id);
+    if (auto* extras = static_cast<HipExtras*>(neighbors.opaque)) {
+        if (extras->enqueued) {
+            // a queued call that nobody collected: it runs to its end first (its kernels write into these arrays)
+            try {
+                if (!extras->queued->finished) {
+                    extras->queued->resume();
+                }
+                finish_queued(neighbors, *extras, extras->queued_stream);
+            } catch (...) {
+            }
+        }
+    }
     free_outputs(neighbors);
     delete static_cast<HipExtras*>(neighbors.opaque);
     neighbors.opaque = nullptr;

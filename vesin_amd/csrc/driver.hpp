@@ -19,6 +19,23 @@ void neighbors(
     void* stream
 );
 
+/// `neighbors` that comes back as soon as the host would have to wait for the GPU: what the call can decide without
+/// an answer from the device is queued on `stream` by then, the rest happens in `neighbors_collect` (which any host
+/// thread may call; the inputs must stay as they are until then). Returns the device word that receives the number
+/// of rows once the queued kernels have run, or ~0 when they did not leave the complete list.
+const unsigned long long* neighbors_enqueue(
+    const double (*points)[3],
+    size_t n_points,
+    const double box[3][3],
+    const bool periodic[3],
+    VesinOptions options,
+    VesinNeighborList& neighbors,
+    void* stream
+);
+
+/// Ends the call that `neighbors_enqueue` started on this list: waits for its kernels, and does whatever is left.
+void neighbors_collect(VesinNeighborList& neighbors);
+
 /// The lists of many systems in one sequence of launches. `points`, `boxes`, `periodic` are device
 /// memory holding the systems one after the other; `first_point` (host, n_systems + 1 entries) says where each
 /// system starts. Rows come out system after system with indices counted inside each system; `first_pair` (host,
