@@ -3,10 +3,11 @@ oracle/Makefile from the reference's own sources) on every golden case and store
 
 Needs the reference checkout (for the build); run from the repository root:
 
-    python -m tests.golden.make_golden [--full-size]
+    python -m tests.golden.make_golden [--full-size | --large]
 
 Small cases are always regenerated; full-size benchmark configurations are kept from the existing file unless
---full-size is given (they take minutes and several GB of host memory).
+--full-size is given (they take minutes and several GB of host memory). --large regenerates nothing but the system
+of 17,000,000 points (minutes as well: the reference's grid holds at most 100,000 cells).
 """
 
 import json
@@ -21,6 +22,7 @@ OUT = os.path.join(os.path.dirname(os.path.realpath(__file__)), "reference_check
 
 def main():
     full_size = "--full-size" in sys.argv
+    large = "--large" in sys.argv
     oracle.build()
     if not oracle.have_ref():
         raise SystemExit("oracle/_ref/libvesin_ref.so is missing: the reference checkout is needed to build it")
@@ -30,8 +32,8 @@ def main():
         with open(OUT) as fd:
             golden = json.load(fd)
 
-    for name, points, box, periodic, cutoff, full in systems.golden_cases(full_size=full_size):
-        result = oracle.ref_neighbors(points, box, periodic, cutoff, full, False, "ijSdD")
+    for name, points, box, periodic, cutoff, full in systems.golden_cases(full_size=full_size, large=large):
+        result = oracle.ref_neighbors(points, box, periodic, cutoff, full, False, "ijSd" if large else "ijSdD")
         entry = systems.fingerprints(result)
         entry.update(cutoff=cutoff, full=full, n_points=int(len(points)))
         golden[name] = entry

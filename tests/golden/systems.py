@@ -116,10 +116,28 @@ def small_systems():
     return systems
 
 
-def golden_cases(full_size=False):
+LARGE_POINTS = 17_000_000  # more than 2^24
+
+
+def uniform_large(n_points=LARGE_POINTS, pairs_per_point=4.0, cutoff=1.0, seed=77):
+    """Uniformly random points in a periodic cube, at the density that gives every point `pairs_per_point` neighbours
+    within `cutoff` on average: a system whose point indices, cells and rows go beyond 2^24 while its list stays
+    small enough to check (the reference's own guard for large values: python/vesin/tests/test_cupy.py:339-350)."""
+    density = pairs_per_point / (4.0 / 3.0 * np.pi * cutoff**3)
+    length = (n_points / density) ** (1.0 / 3.0)
+    rng = np.random.default_rng(seed)
+    points = rng.random((n_points, 3)) * length
+    return points, np.eye(3) * length, np.array([True, True, True])
+
+
+def golden_cases(full_size=False, large=False):
     """Yield (name, points, box, periodic, cutoff, full_list). Small cases always; with ``full_size`` also the
-    benchmark configurations at their real sizes."""
+    benchmark configurations at their real sizes; with ``large`` only the system of more than 2^24 points."""
     from vesin_amd import configs
+
+    if large:
+        yield "uniform-17m", *uniform_large(), 1.0, True
+        return
 
     for name, system in small_systems().items():
         for cutoff in (3.0, 5.0, 7.0, 10.0):

@@ -138,3 +138,7 @@ extern "C" void probe_wait_rest(const unsigned char* gives_up, size_t n_calls, u
         }
     }
 }
+
+extern "C" int probe_ordered_records_fit(size_t n_points, size_t record_bytes) {
+    return vesin_hip::ordered_records_fit(n_points, record_bytes) ? 1 : 0;
+}

@@ -33,6 +33,8 @@ def probe(tmp_path_factory):
                                   ctypes.c_void_p, ctypes.c_size_t]
     lib.probe_box_guess.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
     lib.probe_box_guess.restype = None
+    lib.probe_ordered_records_fit.argtypes = [ctypes.c_size_t, ctypes.c_size_t]
+    lib.probe_ordered_records_fit.restype = ctypes.c_int
     lib.probe_wait_rest.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
     lib.probe_wait_rest.restype = None
     lib.probe_ordered_share.argtypes = [ctypes.c_size_t, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_int]
@@ -405,3 +407,14 @@ def test_a_launch_whose_waves_gave_up_is_left_alone_for_longer_and_longer(probe)
     assert used[:11].all() and not used[11:75].any() and used[75:201].all() and not used[201:265].any() and used[265:].all()
 
 
+
+
+def test_work_memory_of_the_in_order_search_is_bounded(probe):
+    # 12 KB per tile slot. Diamond at cutoff 5: 1,000,000 atoms have about 74,000 slots, 8,000,000 about 600,000
+    assert probe.probe_ordered_records_fit(1_000_000, 74_000 * 12288)
+    assert probe.probe_ordered_records_fit(8_000_000, 600_000 * 12288)
+    # a cell per point: 17,000,000 points would take 212 GB
+    assert not probe.probe_ordered_records_fit(17_000_000, 17_300_000 * 12288)
+    # small systems always fit
+    assert probe.probe_ordered_records_fit(216, 2048 * 12288)
+    assert probe.probe_ordered_records_fit(1, 64 * 12288)

@@ -74,6 +74,31 @@ struct TraceRange {
 };
 #endif
 
+#ifdef VESIN_HIP_HOST_PROFILE
+// developer's instrumentation: where the host's time of a call goes (printed every 1000 calls)
+#include <time.h>
+struct HostProfile {
+    double sums[8] = {};
+    long calls = 0;
+    double last = 0;
+    static double now() { timespec t; clock_gettime(CLOCK_MONOTONIC, &t); return t.tv_sec * 1e6 + t.tv_nsec * 1e-3; }
+    void begin() { last = now(); }
+    void lap(int k) { const double t = now(); sums[k] += t - last; last = t; }
+    void end() {
+        calls += 1;
+        if (calls % 1000 == 0) {
+            std::fprintf(stderr, "host profile (us per call): checks %.2f state %.2f setup %.2f launch %.2f wait %.2f after %.2f\n",
+                         sums[0] / 1000, sums[1] / 1000, sums[2] / 1000, sums[3] / 1000, sums[4] / 1000, sums[5] / 1000);
+            for (double& s : sums) s = 0;
+        }
+    }
+};
+static thread_local HostProfile HOST_PROFILE;
+#define HOST_LAP(k) HOST_PROFILE.lap(k)
+#else
+#define HOST_LAP(k) do {} while (false)
+#endif
+
 static std::atomic<bool> TIMINGS_ENABLED{false};
 
 void enable_timings(bool enabled) {
@@ -1075,12 +1100,21 @@ void neighbors(
     // the null stream when the caller names none, like the reference (vesin/src/vesin_cuda.cpp:798)
     hipStream_t stream = static_cast<hipStream_t>(caller_stream);
     const int device_id = neighbors.device.device_id;
+#ifdef VESIN_HIP_HOST_PROFILE
+    HOST_PROFILE.begin();
+#endif
     check_inputs(points, n_points, box, periodic, device_id);
+    HOST_LAP(0);
 
     const DeviceGuard guard(device_id);
     HipExtras& extras = extras_of(neighbors);
     refuse_while_queued(extras);
+    HOST_LAP(1);
     run_call(points, n_points, box, periodic, options, neighbors, extras, stream);
+    HOST_LAP(5);
+#ifdef VESIN_HIP_HOST_PROFILE
+    HOST_PROFILE.end();
+#endif
 }
 
 const unsigned long long* neighbors_enqueue(
@@ -1505,6 +1539,11 @@ bool compute(
     const uint32_t ordered_items_per_tile = TILE_POINTS / ordered_points_per_item;
     const uint32_t ordered_blocks =
         static_cast<uint32_t>((tiles_bound * ordered_items_per_tile + ORDERED_WAVES - 1) / ORDERED_WAVES);
+    const size_t ordered_record_bytes =
+        static_cast<size_t>(ordered_blocks) * ORDERED_WAVES * ORDERED_UNITS * WAVE * sizeof(CandidateRecord);
+    if (try_in_order && !extras.fixed_memory && !ordered_records_fit(n_points, ordered_record_bytes)) {
+        try_in_order = false; // a sparse system of many cells: see ordered_records_fit
+    }
     const size_t scratch_elements = std::max(
         std::max(scan_scratch_elements(n_cells), scan_scratch_elements(n_slots)),
         try_in_order ? scan_scratch_elements(n_points) : 0
@@ -1590,6 +1629,7 @@ bool compute(
         return false;
     }
     if (one_launch) {
+        HOST_LAP(2);
         size_outputs(neighbors, extras, 0, options);
         SmallArgs sargs = {};
         sargs.points = reinterpret_cast<const double*>(points);
@@ -1624,6 +1664,7 @@ bool compute(
             hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>((n_points + 15) / 16)), dim3(16 * WAVE), 0, stream, sargs, g);
         }
         fetched = true;
+        HOST_LAP(3);
         mark(T_CELLS);
         mark(T_WRITE);
         bool published_here = false;
@@ -1633,6 +1674,7 @@ bool compute(
             published_here = extras.publish_length(outcome, reinterpret_cast<const double*>(box), periodic, stream);
         }
         extras.wait(stream, any_open ? 1 : 0);
+        HOST_LAP(4);
         if (!box_was_right()) {
             return false;
         }

@@ -131,6 +131,17 @@ inline unsigned int ordered_share(size_t n_points, size_t n_cells, size_t tile_s
     return share;
 }
 
+/// Whether the in-order search may take the work memory it asks for. Its counting pass leaves a record per
+/// candidate for the writing pass, in a block of fixed size per tile *slot* (12 KB, room for 1024 candidates), and the
+/// number of slots follows the cells as well as the points: a dense system takes about 1 KB per point (1,000,000
+/// atoms of diamond: 0.9 GB), a sparse one with a cell per point would take 12 KB per point (17,000,000 points: 212
+/// GB). Beyond 2 GiB + 1.5 KB per point the sorted list is made by the search that needs no such records, followed
+/// by the radix sort.
+inline bool ordered_records_fit(size_t n_points, size_t record_bytes) {
+    const double allowed = 2147483648.0 + 1536.0 * static_cast<double>(n_points);
+    return static_cast<double>(record_bytes) <= allowed;
+}
+
 /// Waves that share the points of a tile in the writing pass (1 or 4), from the number of tiles the call before had
 /// on the same points (0: not known, one wave).
 ///
