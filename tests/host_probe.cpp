@@ -142,3 +142,50 @@ extern "C" void probe_wait_rest(const unsigned char* gives_up, size_t n_calls, u
 extern "C" int probe_ordered_records_fit(size_t n_points, size_t record_bytes) {
     return vesin_hip::ordered_records_fit(n_points, record_bytes) ? 1 : 0;
 }
+
+// The fields choose_prefilter reads of a grid.
+struct ProbeGridForPrefilter {
+    double H[9];
+    double Hinv[9];
+    double np_min[3];
+    double np_scale[3];
+    int n[3];
+    int s[3];
+    int periodic[3];
+};
+
+/// Grid of a system and the single-precision pre-test chosen for it: `out` receives use32, lo32, hi32 (as doubles)
+/// and the nine components of the cell edges; `n` and `s` the grid.
+extern "C" int probe_prefilter(
+    const double box[9], const unsigned char periodic[3], double cutoff, size_t n_points,
+    const double lo[3], const double hi[3], int single_cell, int n[3], int s[3], double out[12]
+) {
+    bool flags[3] = {periodic[0] != 0, periodic[1] != 0, periodic[2] != 0};
+    try {
+        auto hbox = vesin_hip::normalise_box(box, flags);
+        auto grid = vesin_hip::choose_grid(hbox, cutoff, n_points, lo, hi, single_cell != 0);
+        ProbeGridForPrefilter g;
+        for (int d = 0; d < 3; d++) {
+            for (int e = 0; e < 3; e++) {
+                g.H[3 * d + e] = hbox.H[d][e];
+                g.Hinv[3 * d + e] = hbox.Hinv[d][e];
+            }
+            g.np_min[d] = grid.np_min[d];
+            g.np_scale[d] = grid.np_scale[d];
+            g.n[d] = n[d] = grid.n[d];
+            g.s[d] = s[d] = grid.s[d];
+            g.periodic[d] = flags[d] ? 1 : 0;
+        }
+        vesin_hip::Prefilter pre;
+        vesin_hip::choose_prefilter(g, cutoff, pre);
+        out[0] = pre.use32;
+        out[1] = pre.lo32;
+        out[2] = pre.hi32;
+        for (int k = 0; k < 9; k++) {
+            out[3 + k] = pre.cell_edges[k];
+        }
+    } catch (const std::exception&) {
+        return 1;
+    }
+    return 0;
+}

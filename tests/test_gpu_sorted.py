@@ -315,3 +315,47 @@ def test_any_share_of_a_tile_per_wave_gives_the_same_list(share, capfd, monkeypa
     box = np.array([[44.0, 0.0, 0.0], [5.0, 41.0, 0.0], [-3.0, 2.0, 46.0]])
     points = rng.uniform(-0.2, 1.2, size=(7000, 3)) @ box
     _check(points, box, (True, True, False), 4.0, share % 3 != 0, capfd, monkeypatch, "used")
+
+
+def _pairs_at_the_cutoff(n_pairs, cutoff, box, seed):
+    """Points in pairs whose distance is the cutoff to within a few units in the last place, some below, some at,
+    some above: `n_pairs` pairs spread over the box, far enough from each other to stay pairs."""
+    rng = np.random.default_rng(seed)
+    per_edge = int(np.ceil(n_pairs ** (1.0 / 3.0)))
+    grid = np.stack(np.meshgrid(*[np.arange(per_edge)] * 3, indexing="ij"), axis=-1).reshape(-1, 3)[:n_pairs]
+    first = (grid + 0.5 + rng.uniform(-0.05, 0.05, size=grid.shape)) / per_edge @ box
+    direction = rng.normal(size=first.shape)
+    direction /= np.linalg.norm(direction, axis=1)[:, None]
+    # distances cutoff * (1 + m 2^-52), m from -6 to 6: squared distances a few units in the last place around cutoff^2
+    steps = rng.integers(-6, 7, size=len(first)).astype(np.float64)
+    second = first + direction * (cutoff * (1.0 + steps * 2.0**-52))[:, None]
+    return np.concatenate([first, second])
+
+
+@pytest.mark.parametrize("full", [True, False])
+@pytest.mark.parametrize(
+    "name",
+    ["cube", "triclinic", "points moved by box vectors", "slab"],
+)
+def test_pairs_next_to_the_cutoff(name, full, capfd, monkeypatch):
+    """The counting pass decides most pairs in single precision; what that cannot decide, pairs within rounding of the
+    cutoff above all, must come out as the reference's own arithmetic has it: thousands of pairs whose squared
+    distance is within a few units in the last place of the squared cutoff, on either side."""
+    cutoff = 3.0
+    periodic = True
+    if name == "triclinic":
+        box = np.array([[64.0, 0.0, 0.0], [11.0, 61.0, 0.0], [-9.0, 13.0, 66.0]])
+    else:
+        box = np.eye(3) * 64.0
+    points = _pairs_at_the_cutoff(4096, cutoff, box, seed=len(name))
+    if name == "points moved by box vectors":
+        moves = np.random.default_rng(3).integers(-3, 4, size=points.shape)
+        points = points + moves @ box
+    if name == "slab":
+        periodic = (True, True, False)
+    flags = [bool(periodic)] * 3 if isinstance(periodic, bool) else list(periodic)
+    expected = oracle.neighbors(points, box, flags, cutoff, True, False, "ijd")
+    # the system is what it is meant to be: about half of the pairs are in, and their distances crowd the cutoff
+    near = np.abs(expected["distances"] - cutoff) < 1e-12
+    assert 1000 < near.sum() // 2 < 3500
+    _check(points, box, periodic, cutoff, full, capfd, monkeypatch, "used")

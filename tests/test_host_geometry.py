@@ -35,6 +35,8 @@ def probe(tmp_path_factory):
     lib.probe_box_guess.restype = None
     lib.probe_ordered_records_fit.argtypes = [ctypes.c_size_t, ctypes.c_size_t]
     lib.probe_ordered_records_fit.restype = ctypes.c_int
+    lib.probe_prefilter.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_double, ctypes.c_size_t, ctypes.c_void_p,
+                                    ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
     lib.probe_wait_rest.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
     lib.probe_wait_rest.restype = None
     lib.probe_ordered_share.argtypes = [ctypes.c_size_t, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_int]
@@ -418,3 +420,89 @@ def test_work_memory_of_the_in_order_search_is_bounded(probe):
     # small systems always fit
     assert probe.probe_ordered_records_fit(216, 2048 * 12288)
     assert probe.probe_ordered_records_fit(1, 64 * 12288)
+
+
+def run_prefilter(probe, box, periodic, cutoff, n_points, lo, hi, single_cell=False):
+    box = np.ascontiguousarray(box, dtype=np.float64)
+    flags = np.ascontiguousarray(periodic, dtype=np.uint8)
+    lo = np.ascontiguousarray(lo, dtype=np.float64)
+    hi = np.ascontiguousarray(hi, dtype=np.float64)
+    n = np.zeros(3, dtype=np.int32)
+    s = np.zeros(3, dtype=np.int32)
+    out = np.zeros(12)
+    status = probe.probe_prefilter(box.ctypes.data, flags.ctypes.data, cutoff, n_points, lo.ctypes.data, hi.ctypes.data,
+                                   int(single_cell), n.ctypes.data, s.ctypes.data, out.ctypes.data)
+    assert status == 0
+    return bool(out[0]), np.float32(out[1]), np.float32(out[2]), out[3:].reshape(3, 3), n, s
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_single_precision_pre_test_never_decides_a_pair_it_should_not(probe, seed):
+    """The counting pass of the in-order search decides a pair in single precision when its squared distance, worked
+    out from the places of the two points inside their cells and the offset between the cells, lies below `lo32` or
+    above `hi32`. Here that arithmetic is repeated in numpy's float32 for pairs at the cutoff to within a part in a
+    million, in boxes of every shape, against the squared distance in double precision (extended precision where
+    numpy has it): no pair may be decided the wrong way, and the error stays within half of what the thresholds
+    allow (the bound in geometry.hpp is doubled)."""
+    rng = np.random.default_rng(100 + seed)
+    worst = 0.0
+    for case in range(40):
+        cutoff = float(rng.uniform(1.0, 9.0))
+        kind = case % 4
+        if kind == 0:
+            box = np.diag(rng.uniform(2.5, 40.0, size=3) * cutoff / 3.0)
+        else:
+            box = rng.normal(size=(3, 3)) * rng.uniform(3.0, 30.0)
+            if abs(np.linalg.det(box)) < 0.2 * np.prod(np.linalg.norm(box, axis=1)):
+                continue
+        periodic = [1, 1, 1] if kind < 3 else [1, 0, 1]
+        use32, lo32, hi32, edges, n, s = run_prefilter(probe, box, periodic, cutoff, 50000, [0, -20.0, 0], [0, 35.0, 0],
+                                                      single_cell=(kind == 2))
+        if np.prod(2 * s + 1) > 64:
+            continue  # (the search with the pre-test is not used for such a stencil)
+        assert use32, (box, cutoff)
+        assert float(lo32) < cutoff * cutoff < float(hi32)
+        allowed = (float(hi32) - float(lo32)) / 2.0
+        m = 20000
+        # place of the first point in its cell, direction and length of the pair: the second point's cell follows
+        inside_i = rng.random((m, 3))
+        length = cutoff * (1.0 + rng.uniform(-1e-6, 1e-6, size=m))
+        direction = rng.normal(size=(m, 3))
+        direction /= np.linalg.norm(direction, axis=1)[:, None]
+        in_cells_j = inside_i + (direction * length[:, None]) @ np.linalg.inv(edges)
+        offset = np.floor(in_cells_j)
+        inside_j = in_cells_j - offset
+        reachable = np.all(np.abs(offset) <= s, axis=1)
+        inside_i, inside_j, offset = inside_i[reachable], inside_j[reachable], offset[reachable]
+        # double (or extended) precision: the vector the reference tests
+        wide = np.longdouble
+        exact = (inside_j.astype(wide) + offset.astype(wide) - inside_i.astype(wide)) @ edges.astype(wide)
+        d2 = np.sum(exact * exact, axis=1).astype(np.float64)
+        # single precision, as the kernel does it
+        place_i = (inside_i @ edges).astype(np.float32)
+        place_j = (inside_j @ edges).astype(np.float32)
+        between = (offset @ edges).astype(np.float32)
+        seen = (place_j + between).astype(np.float32)
+        v = (seen - place_i).astype(np.float32)
+        d2_32 = ((v[:, 0] * v[:, 0] + v[:, 1] * v[:, 1]).astype(np.float32) + v[:, 2] * v[:, 2]).astype(np.float32)
+        inside_cutoff = d2 < cutoff * cutoff
+        assert not np.any(inside_cutoff & (d2_32 > hi32)), (box, cutoff)
+        assert not np.any(~inside_cutoff & (d2_32 < lo32)), (box, cutoff)
+        worst = max(worst, float(np.max(np.abs(d2_32.astype(np.float64) - d2)) / allowed))
+    assert 0.0 < worst <= 0.5, worst
+
+
+def test_pre_test_is_switched_off_where_its_bound_is_no_use(probe):
+    # one cell much wider than the cutoff: the margin would be a sizeable part of the squared cutoff
+    use32, *_ = run_prefilter(probe, np.eye(3), [0, 0, 0], 1e-3, 100, [0] * 3, [5000.0] * 3, single_cell=True)
+    assert not use32
+    # an open system very far from the origin: its coordinates have too few digits left for the places
+    use32, *_ = run_prefilter(probe, np.eye(3), [0, 0, 0], 3.0, 100000, [1e12] * 3, [1e12 + 100.0] * 3)
+    assert not use32
+    # a box squeezed almost flat
+    flat = np.array([[1.0e4, 0.0, 0.0], [0.0, 1.0e4, 0.0], [1.0e4, 1.0e4, 10.0]])
+    use32, *_ = run_prefilter(probe, flat, [1, 1, 1], 3.0, 100000000, [0] * 3, [0] * 3)
+    assert not use32
+    # ordinary systems have it
+    use32, *_ = run_prefilter(probe, np.eye(3) * 178.35, [1, 1, 1], 5.0, 1000000, [0] * 3, [0] * 3)
+    assert use32

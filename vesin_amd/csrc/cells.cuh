@@ -44,7 +44,15 @@ struct SortedPoints {
     int32_t* wx; // number of box vectors the point was moved by to land inside the box
     int32_t* wy;
     int32_t* wz;
+    float4* l;   // the place of the point inside its cell, in single precision (choose_prefilter, geometry.hpp); same
+                 // padding as `p`
 };
+
+__device__ __forceinline__ float4 local_record(const Prefilter& g, const double inside[3], const int32_t wrap[3]) {
+    float place[3];
+    local_place(g, inside, wrap, place);
+    return float4{place[0], place[1], place[2], 0.0f};
+}
 
 constexpr uint32_t SORTED_PADDING = 8;
 
@@ -232,8 +240,11 @@ __global__ __launch_bounds__(BLOCK) void clear_fetch_and_bound(
 
 /// Cell coordinates and wrap shift of one point. Periodic directions: cell = floor(frac * n) brought back into
 /// [0, n) with the quotient kept as the wrap shift. Non-periodic directions: clamped, never wrapped.
+/// `inside` (when asked for): where the point lies in its cell along every direction, in units of the cell, 0 to 1
+/// for a point the cell holds (a point of an open direction that was put into the outermost cell may lie beyond).
 __device__ __forceinline__ void locate(
-    const GridParams& g, double x, double y, double z, int32_t cell[3], int32_t wrap[3], bool* far_outside = nullptr
+    const GridParams& g, double x, double y, double z, int32_t cell[3], int32_t wrap[3], bool* far_outside = nullptr,
+    double* inside = nullptr
 ) {
     double f[3];
     fractional(g, x, y, z, f);
@@ -241,7 +252,11 @@ __device__ __forceinline__ void locate(
     for (int d = 0; d < 3; d++) {
         const int32_t n = g.n[d];
         if (g.periodic[d]) {
-            double scaled = floor(f[d] * static_cast<double>(n));
+            const double in_cells = f[d] * static_cast<double>(n);
+            double scaled = floor(in_cells);
+            if (inside != nullptr) {
+                inside[d] = in_cells - scaled;
+            }
             scaled = fmin(fmax(scaled, -2.0e9), 2.0e9);
             int32_t c = static_cast<int32_t>(scaled);
             int32_t q = c / n;
@@ -253,7 +268,11 @@ __device__ __forceinline__ void locate(
             cell[d] = r;
             wrap[d] = q;
         } else {
-            double scaled = floor((f[d] - g.np_min[d]) * g.np_scale[d] * static_cast<double>(n));
+            const double in_cells = (f[d] - g.np_min[d]) * g.np_scale[d] * static_cast<double>(n);
+            double scaled = floor(in_cells);
+            if (inside != nullptr) {
+                inside[d] = in_cells - fmin(fmax(scaled, 0.0), static_cast<double>(n - 1));
+            }
             if (far_outside != nullptr && (scaled < -1.0 || scaled > static_cast<double>(n))) {
                 // (a grid chosen for the points of this call holds them all; one chosen for those of the call
                 // before still gives the right list while points land in the outermost cells instead, but not
@@ -446,7 +465,7 @@ __global__ __launch_bounds__(BLOCK) void place_points(
     const double* __restrict__ points, GridParams g, const int32_t* __restrict__ wrap_of,
     const uint32_t* __restrict__ cell_of, const uint32_t* __restrict__ slot_of,
     const uint64_t* __restrict__ cell_scan, uint32_t n_points, SortedPoints sorted, Tile* __restrict__ tiles,
-    const uint32_t* __restrict__ system_of, const uint32_t* __restrict__ first_point
+    const uint32_t* __restrict__ system_of, const uint32_t* __restrict__ first_point, Prefilter pre = Prefilter()
 ) {
     const uint32_t i = blockIdx.x * BLOCK + threadIdx.x;
     if (i >= n_points) {
@@ -457,6 +476,7 @@ __global__ __launch_bounds__(BLOCK) void place_points(
     const double z = points[3 * static_cast<size_t>(i) + 2];
     uint32_t cell;
     int32_t wx, wy, wz;
+    float4 place = {0.0f, 0.0f, 0.0f, 0.0f};
     if (cell_of != nullptr) {
         cell = cell_of[i];
         wx = wrap_of[3 * static_cast<size_t>(i) + 0];
@@ -466,10 +486,11 @@ __global__ __launch_bounds__(BLOCK) void place_points(
         // same inputs and code as in assign_cells: the same cell
         int32_t where[3] = {0, 0, 0};
         int32_t wrap[3] = {0, 0, 0};
+        double inside[3] = {0.0, 0.0, 0.0};
         unsigned int axis;
         if (all_finite(x, y, z, axis)) {
             bool far_outside = false;
-            locate(g, x, y, z, where, wrap, &far_outside);
+            locate(g, x, y, z, where, wrap, &far_outside, inside);
             if (far_outside) {
                 return; // assign_cells did not count it
             }
@@ -478,6 +499,9 @@ __global__ __launch_bounds__(BLOCK) void place_points(
         wx = wrap[0];
         wy = wrap[1];
         wz = wrap[2];
+        if (sorted.l != nullptr) {
+            place = local_record(pre, inside, wrap);
+        }
     }
     const uint64_t here = cell_scan[cell];
     const uint32_t start = static_cast<uint32_t>(here);
@@ -490,6 +514,9 @@ __global__ __launch_bounds__(BLOCK) void place_points(
     // carries the system above its flag bit
     const uint32_t system = system_of != nullptr ? system_of[i] : 0;
     sorted.p[to] = SortedPoint{x, y, z, system_of != nullptr ? i - first_point[system] : i, 0u};
+    if (sorted.l != nullptr) {
+        sorted.l[to] = place;
+    }
     const uint32_t tile_size = tile_size_of(count);
     // A single system's caller hands the wrap arrays over cleared: points in arbitrary order scatter their stores, a
     // 32-byte sector of memory traffic for each, and most points were not moved by any box vector.
@@ -990,7 +1017,7 @@ __global__ __launch_bounds__(BLOCK) void prepare_single_cell(
     const double* __restrict__ points, GridParams g, SortedPoints sorted, Tile* __restrict__ tiles,
     uint64_t* __restrict__ cell_scan, DeviceStatus* status, uint4* __restrict__ clear = nullptr,
     size_t clear_blocks16 = 0, const double* __restrict__ box = nullptr, const bool* __restrict__ periodic = nullptr,
-    unsigned char* host_small = nullptr
+    unsigned char* host_small = nullptr, Prefilter pre = Prefilter()
 ) {
     if (blockIdx.x == 0) {
         const int t = threadIdx.x;
@@ -1027,14 +1054,18 @@ __global__ __launch_bounds__(BLOCK) void prepare_single_cell(
         const double z = points[3 * static_cast<size_t>(i) + 2];
         int32_t cell[3] = {0, 0, 0};
         int32_t wrap[3] = {0, 0, 0};
+        double inside[3] = {0.0, 0.0, 0.0};
         unsigned int axis;
         if (all_finite(x, y, z, axis)) {
-            locate(g, x, y, z, cell, wrap);
+            locate(g, x, y, z, cell, wrap, nullptr, inside);
         } else {
             atomicMin(&status->first_bad_coordinate, 3u * i + axis);
         }
         wrapped = (wrap[0] | wrap[1] | wrap[2]) != 0;
         sorted.p[i] = SortedPoint{x, y, z, i, 0u};
+        if (sorted.l != nullptr) {
+            sorted.l[i] = local_record(pre, inside, wrap);
+        }
         sorted.wx[i] = wrap[0];
         sorted.wy[i] = wrap[1];
         sorted.wz[i] = wrap[2];

@@ -175,6 +175,13 @@ static bool full_stencil_only() {
     return text != nullptr && std::strcmp(text, "full") == 0;
 }
 
+/// VESIN_HIP_TESTS=double keeps the distance tests of the searches in double precision throughout (for comparisons
+/// and tests), instead of deciding all pairs but those next to the cutoff in single precision first.
+static bool double_precision_only() {
+    const char* text = std::getenv("VESIN_HIP_TESTS");
+    return text != nullptr && std::strcmp(text, "double") == 0;
+}
+
 /// VESIN_HIP_CELLS=packed keeps every call on the counting-sort cell build (for comparisons and tests) instead of
 /// the one-pass build with a fixed number of slots per cell that the single-pass search can read.
 static bool packed_cells_only() {
@@ -1386,6 +1393,11 @@ bool compute(
     if (full_stencil_only()) {
         g.prune = 0;
     }
+    Prefilter pre;
+    choose_prefilter(g, options.cutoff, pre);
+    if (double_precision_only()) {
+        pre.use32 = 0;
+    }
 
     // ---- carve the work buffers
     const size_t n_cells = grid.n_cells;
@@ -1566,6 +1578,7 @@ bool compute(
         if (try_in_order) {
             rows_of_point = carver.take<uint32_t>(n_points); // (cleared as well: its counting pass may add to it)
         }
+
         wraps_end = reinterpret_cast<char*>(carver.take<uint32_t>(0));
         cell_scan = carver.take<uint64_t>(n_cells + 1);
         if (!single_cell) {
@@ -1575,6 +1588,11 @@ bool compute(
             provisional = carver.take<uint32_t>(n_points);
         }
         sorted.p = carver.take<SortedPoint>(sorted_slots + SORTED_PADDING);
+        // (the places of the points inside their cells, for the single-precision pre-test of the in-order search's
+        // counting pass; the cell builds of small systems and of the reproducible order do not fill them in)
+        sorted.l = try_in_order && pre.use32 != 0 && !small_build && !ordered_rows()
+                       ? carver.take<float4>(sorted_slots + SORTED_PADDING)
+                       : nullptr;
         counts = carver.take<uint32_t>(std::max(n_slots, direct_slots * n_slices));
         offsets = carver.take<uint64_t>(std::max(n_slots, direct_slots * n_slices) + 1);
         scan_scratch = carver.take<uint64_t>(scratch_elements);
@@ -1586,6 +1604,7 @@ bool compute(
             if (ordered_items_per_tile == 1) {
                 candidate_order = carver.take<uint16_t>(tiles_bound * ORDERED_CANDIDATES);
             }
+
         }
     };
     Carver measure(nullptr);
@@ -1761,7 +1780,8 @@ bool compute(
         if (single_cell) {
             hipLaunchKernelGGL(
                 prepare_single_cell, dim3(point_blocks), dim3(BLOCK), 0, stream,
-                flat_points, g, sorted, tiles, cell_scan, extras.d_status
+                flat_points, g, sorted, tiles, cell_scan, extras.d_status, static_cast<uint4*>(nullptr), size_t(0),
+                static_cast<const double*>(nullptr), static_cast<const bool*>(nullptr), static_cast<unsigned char*>(nullptr), pre
             );
             return;
         }
@@ -1787,7 +1807,7 @@ bool compute(
                 place_points, dim3(point_blocks), dim3(BLOCK), 0, stream,
                 flat_points, g, static_cast<const int32_t*>(nullptr), static_cast<const uint32_t*>(nullptr), slot_of,
                 cell_scan, g.n_points, sorted, tiles,
-                static_cast<const uint32_t*>(nullptr), static_cast<const uint32_t*>(nullptr)
+                static_cast<const uint32_t*>(nullptr), static_cast<const uint32_t*>(nullptr), pre
             );
         }
     };
@@ -1807,7 +1827,8 @@ bool compute(
         hipLaunchKernelGGL(
             prepare_single_cell, dim3(1), dim3(BLOCK), 0, stream,
             flat_points, g, sorted, tiles, cell_scan, extras.d_status, reinterpret_cast<uint4*>(first), (to_clear + 15) / 16,
-            fetched ? static_cast<const double*>(nullptr) : reinterpret_cast<const double*>(box), periodic, extras.mail_device->small
+            fetched ? static_cast<const double*>(nullptr) : reinterpret_cast<const double*>(box), periodic, extras.mail_device->small,
+            pre
         );
         fetched = true;
     } else if (direct_cells) {
@@ -2008,6 +2029,7 @@ bool compute(
             oargs.count_split = rows_cleared ? static_cast<uint32_t>(std::max(1, std::min(4, std::atoi(text)))) : 1u;
         }
         oargs.points = reinterpret_cast<const double*>(points);
+        oargs.pre = pre;
         oargs.order = candidate_order;
         oargs.first_row = first_row_of_point;
         oargs.status = ordered_status;
@@ -2844,6 +2866,7 @@ bool batch_attempt(
         system_of = carver.take<uint32_t>(n_points);
         wrap_of = carver.take<int32_t>(3 * n_points);
         sorted.p = carver.take<SortedPoint>(n_points + SORTED_PADDING);
+        sorted.l = nullptr; // (no search of a batch uses the places inside the cells)
         sorted.wx = carver.take<int32_t>(n_points + SORTED_PADDING);
         sorted.wy = carver.take<int32_t>(n_points + SORTED_PADDING);
         sorted.wz = carver.take<int32_t>(n_points + SORTED_PADDING);

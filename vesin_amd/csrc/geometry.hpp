@@ -331,6 +331,105 @@ inline void choose_pruning(const HostBox& box, const HostGrid& grid, double cuto
     g.prune = 1;
 }
 
+/// Largest number of box vectors a point may have been moved by (per direction) for its place inside its cell to be
+/// kept in single precision (see choose_prefilter); points further out are tested in double precision only.
+constexpr int32_t LOCAL_WRAP_LIMIT = 400;
+
+/// The single-precision pre-test of the searches. Every cell-sorted point also carries its place inside its cell
+/// as three floats: x_local = (x - w . H) - origin of the cell (w: the box vectors the point was moved by), computed
+/// in double precision and rounded once. For a tile point i, a candidate j and the stencil offset (dx, dy, dz)
+/// between their cells, the vector the reference tests, v = (r_j - r_i) + S . H, is
+///     v = x_local_j + (dx E_0 + dy E_1 + dz E_2) - x_local_i          (E_d: the edge vectors of one cell)
+/// whatever the wraps of the two points and the box shift of the entry are (they are what makes the cells
+/// neighbours). The searches evaluate that in single precision, |v|^2 = d2_32, and decide
+///     d2_32 < lo32: the pair is within the cutoff;   d2_32 > hi32: it is not;
+///     otherwise (or when a place is not a number): the reference's own arithmetic in double precision decides,
+/// so the result is the reference's bit for bit as long as |d2_32 - fl64(d2)| <= eps for every pair whose true
+/// squared distance is at or near the cutoff, with lo32 = cutoff^2 - eps and hi32 = cutoff^2 + eps. The bound:
+/// every place satisfies |x_local_k| <= R (R = twice the extent of a cell along the axis, twice because points of an
+/// open direction may sit up to one cell outside theirs; places beyond that are stored as NaN), offsets satisfy
+/// |offset_k| <= D (the stencil radius times the extent of a cell), each is rounded once (u = 2^-24 relative), the
+/// sum x_local_j + offset is rounded, the difference is rounded: every component of v carries at most
+/// A = u (3 R + 2 D) + u |v_k| of error, and the three squares and two sums add 3 u |v|^2. With |v| at the cutoff rc
+/// that is |d2_32 - d2| <= 2 sqrt(3) rc A + 3 A^2 + 5 u rc^2 (first order in u), which the formula below doubles.
+/// The double-precision quantities behind the places (fractional coordinates, cell origins) carry errors of the
+/// order of 1e-16 x (box length) x (condition of the box) x (number of boxes the point was moved by): the pre-test is
+/// switched off (use32 = 0) for boxes so skewed, or open systems so far from the origin, that this could come near
+/// a thousandth of eps, and when eps is no longer small against the cutoff (cells much larger than the cutoff).
+struct Prefilter {
+    int32_t use32;        // the pre-test is used at all
+    float lo32, hi32;     // squared distances below / above which a pair is certainly within / beyond the cutoff
+    double cell_edges[9]; // row d: the Cartesian vector of one cell along direction d
+};
+
+template <typename Grid>
+VESIN_HOST_DEVICE inline void choose_prefilter(const Grid& grid, double cutoff, Prefilter& g) {
+    g.use32 = 0;
+    g.lo32 = 0.0f;
+    g.hi32 = 0.0f;
+    double extent_of_cell[3] = {0.0, 0.0, 0.0}; // per Cartesian axis: sum over the directions of |E_dk|
+    double reach[3] = {0.0, 0.0, 0.0};          // the same with every direction taken s_d times
+    double box_size = 0.0;
+    double inverse_size = 0.0;
+    double far_from_origin = 0.0;
+    for (int d = 0; d < 3; d++) {
+        const double scale = (grid.periodic[d] ? 1.0 : 1.0 / grid.np_scale[d]) / static_cast<double>(grid.n[d]);
+        double row = 0.0;
+        double inverse_row = 0.0;
+        for (int k = 0; k < 3; k++) {
+            g.cell_edges[3 * d + k] = grid.H[3 * d + k] * scale;
+            extent_of_cell[k] += ::fabs(g.cell_edges[3 * d + k]);
+            reach[k] += static_cast<double>(grid.s[d]) * ::fabs(g.cell_edges[3 * d + k]);
+            row += ::fabs(grid.H[3 * d + k]) * (grid.periodic[d] ? 1.0 : 1.0 / grid.np_scale[d]);
+            inverse_row += ::fabs(grid.Hinv[3 * k + d]);
+        }
+        box_size = ::fmax(box_size, row);
+        inverse_size = ::fmax(inverse_size, inverse_row * (grid.periodic[d] ? 1.0 : grid.np_scale[d]));
+        if (!grid.periodic[d]) {
+            far_from_origin = ::fmax(far_from_origin, ::fabs(grid.np_min[d]) + 1.0 / grid.np_scale[d]);
+        }
+    }
+    const double R = 2.0 * ::fmax(extent_of_cell[0], ::fmax(extent_of_cell[1], extent_of_cell[2]));
+    const double D = ::fmax(reach[0], ::fmax(reach[1], reach[2]));
+    const double u = 5.9604644775390625e-08; // 2^-24
+    const double A = u * (3.0 * R + 2.0 * D + cutoff);
+    const double eps = 2.0 * (3.4641016151377544 * cutoff * A + 3.0 * A * A + 5.0 * u * cutoff * cutoff);
+    // what double precision leaves in a place: fractional coordinates of a point up to LOCAL_WRAP_LIMIT boxes away,
+    // turned back into a length; along open directions the projected coordinate of a point far from the origin
+    const double u64 = 1.1102230246251565e-16;
+    const double behind = 16.0 * u64 * ((LOCAL_WRAP_LIMIT + 2.0) * box_size * inverse_size * box_size + far_from_origin);
+    const double cutoff2 = cutoff * cutoff;
+    if (!(eps <= 0.01 * cutoff2) || !(4.0 * cutoff * behind <= 1e-3 * eps) || !(eps > 0.0)) {
+        return;
+    }
+    // thresholds rounded away from the cutoff
+    float lo = static_cast<float>(cutoff2 - eps);
+    float hi = static_cast<float>(cutoff2 + eps);
+    if (static_cast<double>(lo) > cutoff2 - eps) {
+        lo = ::nextafterf(lo, 0.0f);
+    }
+    if (static_cast<double>(hi) < cutoff2 + eps) {
+        hi = ::nextafterf(hi, 3.0e38f);
+    }
+    g.lo32 = lo;
+    g.hi32 = hi;
+    g.use32 = 1;
+}
+
+/// The place of a point inside its cell (see choose_prefilter), from the position of the point in units of cells
+/// along every direction, counted from the origin of its cell (`inside[d]`: 0 to 1 for a point the cell holds).
+/// Not a number when the point lies too far outside of its cell or was moved by too many box vectors.
+VESIN_HOST_DEVICE inline void local_place(const Prefilter& g, const double inside[3], const int32_t wrap[3], float place[3]) {
+    bool usable = true;
+    for (int d = 0; d < 3; d++) {
+        usable = usable && inside[d] >= -1.0 && inside[d] <= 2.0 && wrap[d] <= LOCAL_WRAP_LIMIT && wrap[d] >= -LOCAL_WRAP_LIMIT;
+    }
+    for (int k = 0; k < 3; k++) {
+        const double value = inside[0] * g.cell_edges[k] + inside[1] * g.cell_edges[3 + k] + inside[2] * g.cell_edges[6 + k];
+        place[k] = usable ? static_cast<float>(value) : __builtin_nanf("");
+    }
+}
+
 } // namespace vesin_hip
 
 #endif

@@ -94,6 +94,8 @@ struct OrderedArgs {
     // (everything is known when WRITE starts), which saves the launch that would do it afterwards.
     OrderedHostStatus* publish_to;
     const DeviceStatus* build_status;
+    // COUNT: the single-precision pre-test (choose_prefilter, geometry.hpp); used when `sorted.l` is there
+    Prefilter pre;
 };
 
 /// LDS of one wave. What is known per candidate (hit column, position, original index, shift) stays in the
@@ -115,6 +117,10 @@ struct OrderedWaveShared {
 struct OrderedCountWaveShared: SearchTables {
     uint32_t tile_index[TILE_POINTS];
     double tile_x[TILE_POINTS], tile_y[TILE_POINTS], tile_z[TILE_POINTS];
+    // for the single-precision pre-test (choose_prefilter, geometry.hpp): the places of the item's points inside
+    // their cell, and the offsets of the stencil entries
+    float tile_lx[TILE_POINTS], tile_ly[TILE_POINTS], tile_lz[TILE_POINTS];
+    SearchOffsets offsets;
 };
 
 template <bool WRITE>
@@ -201,8 +207,127 @@ __device__ __forceinline__ void sweep_and_count(
     }
 }
 
+/// What a lane holds of a candidate for the single-precision pre-test (choose_prefilter, geometry.hpp): its place
+/// as seen from the origin of the tile's cell. Lanes past the last candidate hold a place far away.
+template <int R>
+struct SweepPlaces {
+    float x[R], y[R], z[R];
+    uint32_t position[R]; // the candidate's position in the cell-sorted arrays when it must not pair with itself
+};
+
+constexpr float NOWHERE = 1.0e30f;
+
+/// sweep_and_count in single precision: a pair whose squared distance falls below `lo32` is within the cutoff, one
+/// above `hi32` is not, any pair in between sets its lane in `uncertain` and the caller repeats the candidates in
+/// double precision. For any tile: the places account for points that were moved into the box.
+template <int R, bool FULL, typename Shared>
+__device__ __forceinline__ void sweep_and_count32(
+    const Shared& sh, uint32_t first, uint32_t count, const SweepPlaces<R>& c, float lo32, float hi32,
+    const uint32_t (&original)[R], int lane, uint32_t (&column)[R], uint32_t& rows, uint64_t& uncertain
+) {
+    for (uint32_t i0 = 0; i0 < count; i0 += POINTS_PER_LOAD) {
+        float px[POINTS_PER_LOAD], py[POINTS_PER_LOAD], pz[POINTS_PER_LOAD];
+        uint32_t pi[POINTS_PER_LOAD];
+#pragma unroll
+        for (int u = 0; u < POINTS_PER_LOAD; u++) {
+            const uint32_t p = min(i0 + u, static_cast<uint32_t>(TILE_POINTS - 1));
+            px[u] = sh.tile_lx[p];
+            py[u] = sh.tile_ly[p];
+            pz[u] = sh.tile_lz[p];
+            pi[u] = FULL ? 0u : sh.tile_index[p];
+        }
+#pragma unroll
+        for (int u = 0; u < POINTS_PER_LOAD; u++) {
+            if (u > 0 && i0 + u >= count) {
+                break;
+            }
+            const uint32_t at = first + i0 + u;
+            uint32_t found = 0;
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const float vx = c.x[r] - px[u];
+                const float vy = c.y[r] - py[u];
+                const float vz = c.z[r] - pz[u];
+                const float d2 = __builtin_fmaf(vz, vz, __builtin_fmaf(vy, vy, vx * vx));
+                const uint64_t within = __ballot(d2 < lo32);
+                uncertain |= __ballot(d2 < hi32) & ~within;
+                uint64_t mask = within & __ballot(c.position[r] != at);
+                if (!FULL) {
+                    mask &= __ballot(pi[u] <= original[r]);
+                }
+                found += __popcll(mask);
+                column[r] = shift_in(column[r], mask);
+            }
+            if (static_cast<uint32_t>(lane) == i0 + u) {
+                rows += found;
+            }
+        }
+    }
+}
+
 /// Two units of candidates (numbers unit0 * 64 ... + 127 of the tables) against the item's points: hit columns
 /// (the item's first point in the highest bit used); lane p of `rows` adds up the hits of the item's point p.
+/// The same in single precision, for the counting pass of a work item whose points all have a place on record.
+/// Returns false when some pair is too close to the cutoff to call, or some candidate has no place: nothing was
+/// counted then, and the caller goes through ordered_sweep_pair.
+template <bool FULL, typename Shared>
+__device__ __forceinline__ bool ordered_sweep_pair32(
+    const Shared& sh, const SortedPoints& sorted, float lo32, float hi32, uint32_t unit0, uint32_t n_stencil,
+    uint32_t n_candidates, uint32_t first_i, uint32_t n_i, int lane, uint32_t (&column)[ORDERED_R], uint32_t& rows,
+    bool& out_of_range, uint32_t (&at)[ORDERED_R], uint32_t (&original)[ORDERED_R], uint32_t (&biased)[ORDERED_R]
+) {
+    constexpr int R = ORDERED_R;
+    SweepPlaces<R> c;
+    uint64_t uncertain = 0;
+    bool beyond_fields = false;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const uint32_t k = (unit0 + r) * WAVE + lane;
+        c.x[r] = c.y[r] = c.z[r] = NOWHERE;
+        c.position[r] = 0xFFFFFFFFu;
+        column[r] = 0;
+        at[r] = 0xFFFFFFFFu;
+        original[r] = 0;
+        biased[r] = 0;
+        bool unknown = false;
+        if (k < n_candidates) {
+            int32_t packed_q;
+            uint32_t entry;
+            locate_candidate(sh, n_stencil, k, at[r], packed_q, entry);
+            int32_t qx, qy, qz;
+            unpack_shift(packed_q, qx, qy, qz);
+            const float4 place = sorted.l[at[r]];
+            c.x[r] = place.x + sh.offsets.ent_dx[entry];
+            c.y[r] = place.y + sh.offsets.ent_dy[entry];
+            c.z[r] = place.z + sh.offsets.ent_dz[entry];
+            unknown = !(place.x == place.x);
+            original[r] = sorted.p[at[r]].index;
+            const int32_t bx = qx - sorted.wx[at[r]];
+            const int32_t by = qy - sorted.wy[at[r]];
+            const int32_t bz = qz - sorted.wz[at[r]];
+            biased[r] = biased_shift(bx, by, bz);
+            beyond_fields = beyond_fields || beyond(bx, by, bz, ORDERED_SHIFT_LIMIT);
+            // a point is no neighbour of itself (of its images it is: the unshifted entry of the tile's own cell is
+            // meant); a half list keeps a point with its own image under the rule of the reference (the total
+            // shift of such a pair is the cell shift, whatever box vectors the point itself was moved by)
+            const bool never_with_itself = (qx | qy | qz) == 0 || (!FULL && !half_keeps_self_image(qx, qy, qz));
+            c.position[r] = never_with_itself ? at[r] : 0xFFFFFFFFu;
+        }
+        uncertain |= __ballot(unknown);
+    }
+    if (uncertain != 0) {
+        return false;
+    }
+    uint32_t counted = 0;
+    sweep_and_count32<R, FULL>(sh, first_i, n_i, c, lo32, hi32, original, lane, column, counted, uncertain);
+    if (uncertain != 0) {
+        return false;
+    }
+    rows += counted;
+    out_of_range = out_of_range || beyond_fields;
+    return true;
+}
+
 template <bool FULL, bool WRAPPED, typename Shared>
 __device__ __forceinline__ void ordered_sweep_pair(
     const Shared& sh, const SortedPoints& sorted, const GridParams& g, uint32_t unit0, uint32_t n_stencil,
@@ -472,6 +597,9 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
     const int32_t cz = tile.cell / (g.n[0] * g.n[1]);
 
     bool out_of_range = false;
+    // COUNT: the single-precision pre-test, when the grid allows it and every point of the item has a place on record
+    bool pretest = !WRITE && args.pre.use32 != 0 && sorted.l != nullptr;
+    bool place_unknown = false;
     if (static_cast<uint32_t>(lane) < n_i) {
         const uint32_t at = first_i + lane;
         const uint32_t original = sorted.p[at].index;
@@ -483,6 +611,15 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
         sh.tile_x[lane] = sorted.p[at].x;
         sh.tile_y[lane] = sorted.p[at].y;
         sh.tile_z[lane] = sorted.p[at].z;
+        if constexpr (!WRITE) {
+            if (pretest) {
+                const float4 place = sorted.l[at];
+                sh.tile_lx[lane] = place.x;
+                sh.tile_ly[lane] = place.y;
+                sh.tile_lz[lane] = place.z;
+                place_unknown = !(place.x == place.x);
+            }
+        }
         if constexpr (WRITE) {
             sh.tile_wx[lane] = wx;
             sh.tile_wy[lane] = wy;
@@ -503,7 +640,11 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
         // (the counting pass left the number: no tables here, everything about a candidate is in its record)
         n_candidates = uniform(args.candidates_of_item[work]);
     } else {
-        fill_stencil_tables(sh, lane, 0, n_stencil, cx, cy, cz, span_y, span_z, g, args.cell_scan);
+        pretest = pretest && __ballot(place_unknown) == 0;
+        fill_stencil_tables(
+            sh, lane, 0, n_stencil, cx, cy, cz, span_y, span_z, g, args.cell_scan, static_cast<const uint32_t*>(nullptr), 0u,
+            pretest ? &sh.offsets : nullptr, &args.pre
+        );
         n_candidates = __builtin_amdgcn_readfirstlane(sh.n_candidates);
         if (lane == 0 && part == 0) {
             args.candidates_of_item[work] = n_candidates;
@@ -529,7 +670,12 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
         uint32_t own_rows = 0;
         for (uint32_t unit0 = part * R; unit0 < n_units; unit0 += split * R) {
             uint32_t column[R], at[R], original[R], biased[R];
-            if (tile_wrapped) {
+            if (pretest && ordered_sweep_pair32<FULL>(
+                               sh, sorted, args.pre.lo32, args.pre.hi32, unit0, n_stencil, n_candidates, first_i, n_i, lane, column, own_rows,
+                               out_of_range, at, original, biased
+                           )) {
+                // decided in single precision
+            } else if (tile_wrapped) {
                 ordered_sweep_pair<FULL, true>(
                     sh, sorted, g, unit0, n_stencil, n_candidates, first_i, n_i, lane, column, own_rows, out_of_range,
                     at, original, biased

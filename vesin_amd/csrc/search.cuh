@@ -143,6 +143,12 @@ struct SearchTables {
     uint32_t n_candidates;
 };
 
+/// For the kernels with the single-precision pre-test (choose_prefilter in geometry.hpp): from the origin of the
+/// tile's cell to the origin of each entry's cell, box shift included, in single precision.
+struct SearchOffsets {
+    float ent_dx[MAX_ENTRIES], ent_dy[MAX_ENTRIES], ent_dz[MAX_ENTRIES];
+};
+
 struct SearchSharedCount: SearchTables {
     uint16_t ring[1];
 };
@@ -175,7 +181,8 @@ template <typename ScanWord>
 __device__ __forceinline__ void fill_stencil_tables(
     SearchTables& sh, int lane, uint32_t first_linear, uint32_t n_batch, int32_t cx, int32_t cy, int32_t cz,
     int32_t span_y, int32_t span_z, const GridParams& g, const ScanWord* __restrict__ cell_scan,
-    const uint32_t* __restrict__ direct_counts = nullptr, uint32_t direct_capacity = 0
+    const uint32_t* __restrict__ direct_counts = nullptr, uint32_t direct_capacity = 0, SearchOffsets* offsets = nullptr,
+    const Prefilter* pre = nullptr
 ) {
     const uint32_t centre = static_cast<uint32_t>(2 * g.s[0] + 1) * span_y * span_z / 2;
     for (uint32_t e = lane; e < n_batch; e += WAVE) {
@@ -245,6 +252,12 @@ __device__ __forceinline__ void fill_stencil_tables(
         sh.ent_start[e] = start;
         sh.ent_shift[e] = packed;
         sh.ent_prefix[e + 1] = count; // scanned in place below
+        if (offsets != nullptr) {
+            const double ox = static_cast<double>(dx), oy = static_cast<double>(dy), oz = static_cast<double>(dz);
+            offsets->ent_dx[e] = static_cast<float>(ox * pre->cell_edges[0] + oy * pre->cell_edges[3] + oz * pre->cell_edges[6]);
+            offsets->ent_dy[e] = static_cast<float>(ox * pre->cell_edges[1] + oy * pre->cell_edges[4] + oz * pre->cell_edges[7]);
+            offsets->ent_dz[e] = static_cast<float>(ox * pre->cell_edges[2] + oy * pre->cell_edges[5] + oz * pre->cell_edges[8]);
+        }
     }
     wave_sync();
 
@@ -283,6 +296,23 @@ __device__ __forceinline__ void locate_candidate(
     }
     at = sh.ent_start[lo] + (k - sh.ent_prefix[lo]);
     packed = sh.ent_shift[lo];
+}
+
+/// The same, also telling the entry the candidate belongs to.
+__device__ __forceinline__ void locate_candidate(
+    const SearchTables& sh, uint32_t n_batch, uint32_t k, uint32_t& at, int32_t& packed, uint32_t& entry
+) {
+    uint32_t lo = 0;
+#pragma unroll
+    for (uint32_t step = 32; step > 0; step >>= 1) {
+        const uint32_t probe = lo + step;
+        const uint32_t before = sh.ent_prefix[min(probe, static_cast<uint32_t>(MAX_ENTRIES))];
+        const uint32_t take = (probe < n_batch ? 1u : 0u) & (before <= k ? 1u : 0u);
+        lo = take != 0 ? probe : lo;
+    }
+    at = sh.ent_start[lo] + (k - sh.ent_prefix[lo]);
+    packed = sh.ent_shift[lo];
+    entry = lo;
 }
 
 /// Stores of 64 consecutive rows are fastest when they start on whole cache lines in all three arrays (16, 12 and
