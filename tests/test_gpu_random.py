@@ -15,10 +15,14 @@ pytestmark = pytest.mark.gpu
 NAMES = {"P": "pairs", "S": "shifts", "d": "distances", "D": "vectors"}
 
 
-def random_system(rng):
+def random_system(rng, larger=False):
     kind = rng.integers(0, 6)
     n = int(rng.choice([1, 2, 3, 17, 64, 65, 200, 700, 1500]))
     edge = float(rng.uniform(3.0, 14.0))
+    if larger:
+        # beyond the 2048 points that one launch takes: the searches of the large systems, at a liquid's density
+        n = int(rng.choice([2100, 3000, 5000, 9000]))
+        edge = float((n / rng.uniform(0.03, 0.12)) ** (1.0 / 3.0))
     if kind == 0:  # cubic
         box = np.eye(3) * edge
     elif kind == 1:  # orthorhombic, one short axis (several images along it)
@@ -38,7 +42,7 @@ def random_system(rng):
 
 
 @pytest.mark.parametrize("full", [True, False], ids=["full", "half"])
-@pytest.mark.parametrize("seed", [0, 1, 2])
+@pytest.mark.parametrize("seed", range(8))
 def test_random_systems_on_one_reused_list(seed, full):
     import torch
 
@@ -56,7 +60,7 @@ def test_random_systems_on_one_reused_list(seed, full):
             assert_same_list(actual, expected, what=f"seed {seed} step {step} repeat {repeat} n={len(points)} periodic={periodic}")
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(60))
 def test_random_options_and_moves_on_one_reused_list(seed):
     """Sorted or not, half or full, with or without a skin; a system is followed for a few small moves (which the
     Verlet filter and the remembered box meet) before the next one replaces it."""
@@ -71,7 +75,8 @@ def test_random_options_and_moves_on_one_reused_list(seed):
     points = None
     for step in range(8):
         if points is None or rng.random() < 0.5:
-            points, box, periodic = random_system(rng)
+            # (every third sequence mixes in systems of a few thousand points)
+            points, box, periodic = random_system(rng, larger=seed % 3 == 2 and rng.random() < 0.5)
         else:
             points = points + rng.normal(scale=rng.choice([0.01, 0.1, 0.6]), size=points.shape)
             if rng.random() < 0.3:
