@@ -23,7 +23,8 @@ The line carries, next to the throughput:
   and one thread on a bounded sample of the same workload.
 
 ``--config NAME`` makes another configuration the workload of the line (profiling runs use it):
-config0, config1 (default), config1_shuffled, config1_sorted, config2, config3, config3_single, config4a, config4b.
+config0, config1 (default), config1_shuffled, config1_sorted, config2, config3, config3_sorted, config3_single, config4a,
+config4b.
 """
 
 import argparse
@@ -50,7 +51,8 @@ SEARCH_KERNEL_TRAFFIC = {
 }
 KERNEL_SOURCES = ["device_common.cuh", "geometry.hpp", "cells.cuh", "search.cuh", "fused.cuh"]
 
-CONFIG_NAMES = ["config0", "config1", "config1_shuffled", "config1_sorted", "config2", "config3", "config3_single", "config4a", "config4b"]
+CONFIG_NAMES = ["config0", "config1", "config1_shuffled", "config1_sorted", "config2", "config3", "config3_sorted", "config3_single", "config4a",
+                "config4b"]
 DESCRIPTIONS = {
     "config0": "config0: 216 atoms, cutoff 5 A, full, sorted, i j S d",
     "config1": "config1: jittered diamond {replicas}^3 cells = {n_points} atoms, periodic cube, cutoff 5 A, full list, "
@@ -60,6 +62,7 @@ DESCRIPTIONS = {
     "config1_sorted": "config1 with sorted=true (rows in the order of i, j, S)",
     "config2": "config2: 100000 atoms, triclinic, cutoff 6 A, half, sorted, i j S d D",
     "config3": "config3: 4096 replicas of 64 atoms, box 7.134 A, cutoff 10 A, full, i j S d, one batched call",
+    "config3_sorted": "config3 with sorted=true (every replica's rows in the order of i, j, S)",
     "config3_single": "one replica of config3 in a call of its own: 64 atoms, box 7.134 A, cutoff 10 A, full, i j S d",
     "config4a": "config4a: 500000 clustered atoms, no periodic direction, cutoff 4.5 A, full, i j d",
     "config4b": "config4b: the same atoms, periodic (T, T, F)",
@@ -112,10 +115,10 @@ class Workload:
         from vesin_amd import NeighborList, configs
 
         self.name = name
-        self.batch = name == "config3"
+        self.batch = name in ("config3", "config3_sorted")
         if self.batch:
             systems = [configs.config3(r) for r in range(BATCH_REPLICAS)]
-            self.options = systems[0][3]
+            self.options = dict(systems[0][3], sorted=name == "config3_sorted")
             self.first_point = np.cumsum([0] + [len(s[0]) for s in systems])
             self.n_points = int(self.first_point[-1])
             self.points = torch.as_tensor(np.concatenate([s[0] for s in systems]), device="cuda:0")
@@ -351,7 +354,7 @@ def main():
     if not args.no_cpu_baseline:
         # after the GPU work, so that the host threads of the timed calls never compete with it for cores
         wanted = [args.config] + [entry["name"] for entry in result.get("other_configs", []) if entry["name"] in DESCRIPTIONS
-                                  and not entry["name"].startswith("config1_")]
+                                  and not entry["name"].startswith("config1_") and entry["name"] != "config3_sorted"]
         collected = CpuBaselines(wanted, args.replicas).collect()
         own = collected.get(args.config)
         if own is not None:
@@ -374,7 +377,8 @@ def other_configs(args, torch, np):
     """Steady-state figures of the other configurations: after the list's first call and 5 more, a timed region of 20
     calls, then 20 calls timed one by one (the median of those is `ms_per_call`) and 20 between HIP events."""
     results = []
-    names = [name for name in ["config0", "config2", "config3", "config3_single", "config4a", "config4b"] if name != args.config]
+    names = [name for name in ["config0", "config2", "config3", "config3_sorted", "config3_single", "config4a", "config4b"]
+             if name != args.config]
     if args.config == "config1":
         names += ["config1_shuffled", "config1_box_changes", "config1_sorted"]
     for name in names:

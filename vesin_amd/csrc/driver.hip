@@ -32,6 +32,7 @@
 #include "driver.hpp"
 #include "fused.cuh"
 #include "geometry.hpp"
+#include "images.cuh"
 #include "ordered.cuh"
 #include "small.cuh"
 #include "policy.hpp"
@@ -490,6 +491,14 @@ struct BatchSetup {
     // The single-pass search of a batch places its rows through the chain of workgroups: after a launch whose waves
     // gave up waiting, reused lists go straight to the two passes for a while.
     WaitRest chain_rest;
+    // Sorted lists come straight from a search that writes the rows in order where the systems have the shape for
+    // it; after a batch that did not, the next calls go to the two passes and the sort without asking again.
+    int in_order_rest = 0;
+    size_t systems_for_images = 0;          // systems the search over images covers (grids picked on the host)
+    size_t systems_with_points = 0;
+    PinnedVector<uint64_t> pair_base;       // pairs of points (n^2 per system of few points) before every system
+    uint32_t image_words = 1;               // words of 64 images per pair of points, the most any system needs
+    const void* d_pair_base = nullptr;
     // where the first rows of the systems land before they are copied into the caller's array (pinned)
     size_t* first_pair_landing = nullptr;
     size_t first_pair_capacity = 0;
@@ -2732,6 +2741,11 @@ bool batch_attempt(
         }
 
         uint64_t cells_so_far = 0;
+        setup.systems_for_images = 0;
+        setup.systems_with_points = 0;
+        setup.image_words = 1;
+        setup.pair_base.resize(n_systems + 1);
+        uint64_t pairs_so_far = 0;
         double most_units = 1.0; // candidates per tile, in units of 64, of the system with the most (estimate)
         const double zeros[3] = {0.0, 0.0, 0.0};
         for (size_t s = 0; s < n_systems; s++) {
@@ -2760,6 +2774,13 @@ bool batch_attempt(
             }
             const double per_cell = std::max(1.0, static_cast<double>(g.n_points) / std::max(1u, g.n_cells));
             most_units = std::max(most_units, std::ceil(upper_stencil_cells(g) * per_cell / WAVE));
+            setup.systems_with_points += n_here > 0 ? 1 : 0;
+            if (n_here > 0 && images_cover(g)) {
+                setup.systems_for_images += 1;
+                setup.image_words = std::max(setup.image_words, image_words(g));
+            }
+            setup.pair_base[s] = pairs_so_far;
+            pairs_so_far += n_here <= IMAGE_MAX_POINTS ? n_here * n_here : 0;
             cell_base_host[s] = static_cast<uint32_t>(cells_so_far);
             cells_so_far += grid.n_cells;
             if (cells_so_far >= 0xFFFFFFF0ull) {
@@ -2767,6 +2788,7 @@ bool batch_attempt(
             }
         }
         cell_base_host[n_systems] = static_cast<uint32_t>(cells_so_far);
+        setup.pair_base[n_systems] = pairs_so_far;
         setup.total_cells = cells_so_far;
         setup.most_units = most_units;
         setup.valid = true;
@@ -2849,7 +2871,33 @@ bool batch_attempt(
     unsigned long long* d_first_pair = nullptr;
     uint32_t* d_cells_of_system = nullptr;
     char* clear_end = nullptr;
-    const size_t scratch_elements = std::max(scan_scratch_elements(total_cells), scan_scratch_elements(n_slots));
+    // A sorted list straight from the search (images.cuh), when every system has the shape for it. With grids picked
+    // on the device the host does not know: the kernels say.
+    bool try_in_order = options.sorted && !radix_sort_only() &&
+                        (device_grids || setup.systems_for_images == setup.systems_with_points);
+    // (what the counting pass leaves for the writing pass: a bit per pair of points and image)
+    const size_t hit_words = static_cast<size_t>(setup.pair_base[n_systems]) * setup.image_words;
+    try_in_order = try_in_order && ordered_records_fit(n_points, hit_words * sizeof(uint64_t));
+    if (try_in_order && setup.in_order_rest > 0) {
+        setup.in_order_rest -= 1;
+        try_in_order = false;
+    }
+    if (options.sorted && !device_grids && setup.systems_for_images != setup.systems_with_points &&
+        std::getenv("VESIN_HIP_DEBUG") != nullptr) {
+        std::fprintf(
+            stderr, "sorted batch: %zu of %zu systems are of one cell, the rows are sorted after the search\n",
+            setup.systems_for_images, setup.systems_with_points
+        );
+    }
+    OrderedStatus* ordered_status = nullptr;
+    uint32_t* rows_of_point = nullptr;
+    uint64_t* first_row_of_point = nullptr;
+    uint64_t* image_hits = nullptr;
+    uint64_t* d_pair_base = nullptr;
+    const size_t scratch_elements = std::max(
+        std::max(scan_scratch_elements(total_cells), scan_scratch_elements(n_slots)),
+        try_in_order ? scan_scratch_elements(n_points) : size_t(0)
+    );
     auto carve = [&](Carver& carver) {
         // adjacent, so that one fill clears the histogram, the tiles' flags and the state of the single-pass search
         cell_counts = carver.take<uint32_t>(total_cells);
@@ -2859,7 +2907,10 @@ bool batch_attempt(
         chain.bases = carver.take<uint64_t>(chain_groups);
         fused_status = carver.take<FusedStatus>(1);
         counts = carver.take<uint32_t>(n_slots);
+        ordered_status = carver.take<OrderedStatus>(try_in_order ? 1 : 0);
+        rows_of_point = carver.take<uint32_t>(try_in_order ? n_points : 0);
         clear_end = reinterpret_cast<char*>(carver.take<uint32_t>(0));
+        first_row_of_point = carver.take<uint64_t>(try_in_order ? n_points + 1 : 0);
         cell_scan = carver.take<uint64_t>(total_cells + 1);
         cell_of = carver.take<uint32_t>(n_points);
         slot_of = carver.take<uint32_t>(n_points);
@@ -2877,6 +2928,8 @@ bool batch_attempt(
         d_cell_base = carver.take<uint32_t>(n_systems + 1);
         d_first_pair = carver.take<unsigned long long>(n_systems + 1);
         d_cells_of_system = carver.take<uint32_t>(n_systems);
+        d_pair_base = carver.take<uint64_t>(try_in_order ? n_systems + 1 : 0);
+        image_hits = carver.take<uint64_t>(try_in_order ? hit_words : 0);
     };
     Carver measure(nullptr);
     carve(measure);
@@ -2884,6 +2937,13 @@ bool batch_attempt(
     Carver carver(extras.work.ptr);
     carve(carver);
 
+    if (try_in_order && !(same_setup && setup.on_device && setup.work_generation == extras.work.generation &&
+                          setup.d_pair_base == d_pair_base)) {
+        HIP_CHECK(hipMemcpyAsync(
+            d_pair_base, setup.pair_base.data(), (n_systems + 1) * sizeof(uint64_t), hipMemcpyHostToDevice, stream
+        ));
+        setup.d_pair_base = d_pair_base;
+    }
     const bool already_there = same_setup && setup.on_device && setup.work_generation == extras.work.generation &&
                                setup.d_grids == d_grids &&
                                setup.d_first_point == d_first_point && setup.d_cell_base == d_cell_base;
@@ -2963,6 +3023,125 @@ bool batch_attempt(
     args.total_cells = static_cast<uint32_t>(total_cells);
     const uint32_t system_blocks = static_cast<uint32_t>((n_systems + 1 + BLOCK - 1) / BLOCK);
     static_assert(sizeof(size_t) == sizeof(unsigned long long), "size_t is 64 bits wide here");
+
+    auto setup_changed = [&]() {
+        // other boxes than the grids were picked from, or (which open_grids_kernel rules out) more cells than the
+        // buffers were sized for: nothing of this attempt is used, the host picks the grids
+        return speculate && (extras.mail->batch_changed != 0 || (device_grids && extras.mail->batch_total_cells > total_cells));
+    };
+    auto check_pair_limit = [&](size_t total) {
+        if (pair_limit != 0 && total > n_points * pair_limit) {
+            throw std::runtime_error(
+                "The number of neighbor pairs exceeds the maximum capacity of " + std::to_string(n_points * pair_limit) +
+                " (max_pairs_per_point=" + std::to_string(pair_limit) + "; n_points=" + std::to_string(n_points) + "). " +
+                "Consider reducing the cutoff distance, or explicitly setting " +
+                "VESIN_CUDA_MAX_PAIRS_PER_POINT as an environment variable."
+            );
+        }
+    };
+
+    // ---- a sorted list straight from the search: systems of one cell, by brute force over their images in the
+    // order of the list (images.cuh)
+    if (try_in_order) {
+        ImageArgs iargs = {};
+        iargs.sorted = sorted;
+        iargs.cell_scan = cell_scan;
+        iargs.grids = d_grids;
+        iargs.cell_base = d_cell_base;
+        iargs.first_point = d_first_point;
+        iargs.pair_base = d_pair_base;
+        iargs.hits = image_hits;
+        iargs.words = setup.image_words;
+        iargs.n_systems = static_cast<uint32_t>(n_systems);
+        iargs.total_points = static_cast<uint32_t>(n_points);
+        iargs.rows_of_point = rows_of_point;
+        iargs.first_row = first_row_of_point;
+        iargs.status = ordered_status;
+        const dim3 image_grid(static_cast<uint32_t>(n_systems));
+        auto launch_write = [&]() {
+            if (options.full) {
+                hipLaunchKernelGGL(image_write_kernel<true>, image_grid, dim3(IMAGE_BLOCK), 0, stream, iargs);
+            } else {
+                hipLaunchKernelGGL(image_write_kernel<false>, image_grid, dim3(IMAGE_BLOCK), 0, stream, iargs);
+            }
+        };
+        if (options.full) {
+            hipLaunchKernelGGL(image_count_kernel<true>, image_grid, dim3(IMAGE_BLOCK), 0, stream, iargs);
+        } else {
+            hipLaunchKernelGGL(image_count_kernel<false>, image_grid, dim3(IMAGE_BLOCK), 0, stream, iargs);
+        }
+        exclusive_scan<SCAN_U32>(rows_of_point, n_points, first_row_of_point, scan_scratch, stream);
+        // A list that has arrays from earlier calls writes into them without waiting for the host to learn what the
+        // counting pass found: the launch checks on the device that every system was covered and that the rows fit
+        const bool early_write = extras.capacity > 0;
+        size_t early_capacity = 0;
+        if (early_write) {
+            size_outputs(neighbors, extras, 0, options);
+            early_capacity = extras.capacity;
+            iargs.out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
+            iargs.out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
+            iargs.out.distances = neighbors.distances;
+            iargs.out.vectors = reinterpret_cast<double*>(neighbors.vectors);
+            iargs.capacity = early_capacity;
+            iargs.guarded = 1;
+            iargs.publish_to = &extras.mail_device->ordered;
+            iargs.build_status = extras.d_status;
+            launch_write();
+            iargs.publish_to = nullptr;
+        } else {
+            hipLaunchKernelGGL(
+                publish_ordered_status, dim3(1), dim3(1), 0, stream,
+                ordered_status, first_row_of_point + n_points, extras.d_status, cell_scan + total_cells,
+                &extras.mail_device->ordered
+            );
+        }
+        hipLaunchKernelGGL(
+            first_rows_of_systems_kernel, dim3(system_blocks), dim3(BLOCK), 0, stream,
+            first_row_of_point, d_first_point, static_cast<uint32_t>(n_systems), d_first_pair
+        );
+        HIP_CHECK(hipMemcpyAsync(
+            setup.first_pair_landing, d_first_pair, (n_systems + 1) * sizeof(size_t), hipMemcpyDeviceToHost, stream
+        ));
+        HIP_CHECK(hipStreamSynchronize(stream));
+        if (setup_changed()) {
+            return false;
+        }
+        const OrderedHostStatus found = extras.mail->ordered;
+        if (found.first_bad_coordinate != 0xFFFFFFFFu) {
+            non_finite_error(points, found.first_bad_coordinate);
+        }
+        if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
+            std::fprintf(
+                stderr, "in-order search (batch): rows %llu, systems left uncovered %u%s: %s\n", found.total_rows,
+                found.found.unsuitable, device_grids ? ", grids picked on the device" : "",
+                found.found.unsuitable == 0 ? "used" : "left to the radix sort"
+            );
+        }
+        if (found.found.unsuitable == 0) {
+            const size_t total = found.total_rows;
+            check_pair_limit(total);
+            if (!(early_write && total <= early_capacity)) {
+                // first call of the list, or more rows than its arrays hold
+                size_outputs(neighbors, extras, total, options);
+                iargs.out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
+                iargs.out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
+                iargs.out.distances = neighbors.distances;
+                iargs.out.vectors = reinterpret_cast<double*>(neighbors.vectors);
+                iargs.guarded = 0;
+                if (total > 0) {
+                    launch_write();
+                }
+                HIP_CHECK(hipStreamSynchronize(stream));
+            }
+            HIP_CHECK(hipGetLastError());
+            std::memcpy(first_pair, setup.first_pair_landing, (n_systems + 1) * sizeof(size_t));
+            neighbors.length = total;
+            return true;
+        }
+        // a system of several cells, of many points or of very many images: the two passes and the sort below, and
+        // for a while without asking again
+        setup.in_order_rest = SINGLE_PASS_REST;
+    }
 
     // ---- a list that has arrays from earlier calls: single-pass search straight into them, rows in work-item order
     // (the rows of a system stay together). Whatever does not fit its shape starts over with the two passes below.
