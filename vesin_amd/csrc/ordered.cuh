@@ -38,6 +38,8 @@ constexpr int ORDERED_UNITS = 16;                       // units of 64 candidate
 constexpr uint32_t ORDERED_CANDIDATES = ORDERED_UNITS * WAVE;
 constexpr uint32_t ORDERED_MAX_ROWS = 256;              // rows of one point that are ranked in one go
 constexpr int32_t ORDERED_SHIFT_LIMIT = 255;            // per operand: sums stay inside the key's 10-bit fields
+constexpr uint32_t ORDERED_STAGED = ORDERED_MAX_ROWS + WAVE; // rows lined up before they are stored: what a run of
+                                                             // consecutive rows left short of 64, and one point's
 
 /// What the counting pass leaves to the writing pass per candidate of a work item: hit column against the item's
 /// points, original index, biased shift less the wrap of the first point.
@@ -105,10 +107,13 @@ struct OrderedWaveShared {
     double tile_x[TILE_POINTS], tile_y[TILE_POINTS], tile_z[TILE_POINTS];
     int32_t tile_wx[TILE_POINTS], tile_wy[TILE_POINTS], tile_wz[TILE_POINTS];
     uint64_t tile_row[TILE_POINTS];   // WRITE: first output row of each point
+    uint32_t by_index[TILE_POINTS];   // WRITE: the tile's points in the order of their original indices
     // WRITE: the rows of one point: (second point << 32) | biased shift, and the position of the second point in
-    // the cell-sorted arrays; read four at a time when they are ranked, hence the padding
-    __attribute__((aligned(16))) uint64_t keys[ORDERED_MAX_ROWS + 4];
-    uint32_t key_at[ORDERED_MAX_ROWS];
+    // the cell-sorted arrays; read four at a time when they are ranked, hence the padding. With the candidates in
+    // order: rows of points of consecutive original indices, which are consecutive rows of the list, and for each the
+    // number of its first point in the tile
+    __attribute__((aligned(16))) uint64_t keys[ORDERED_STAGED + 4];
+    uint32_t key_at[ORDERED_STAGED];
 };
 
 /// LDS of one wave of the counting pass: the tables and the item's points. (A third of what the writing pass takes:
@@ -538,6 +543,74 @@ __device__ __forceinline__ void write_rows_of_point(
     wave_sync(); // the keys are about to be overwritten by the next point's
 }
 
+/// The hits of one first point (number `point` of the tile), in lane order, behind the `staged` keys that wait in
+/// `sh.keys`: returns how many there were. (Candidates in their final order: the hits are the point's rows in order.)
+template <typename Shared>
+__device__ __forceinline__ uint32_t stage_rows_of_point(
+    Shared& sh, const uint32_t (&columns)[ORDERED_UNITS], const uint32_t (&cand_index)[ORDERED_UNITS],
+    const uint32_t (&cand_biased)[ORDERED_UNITS], uint32_t n_units, uint32_t bit, uint32_t wrap_i, uint32_t point,
+    uint32_t staged
+) {
+    uint32_t n_rows = 0;
+#pragma unroll
+    for (int u = 0; u < ORDERED_UNITS; u++) {
+        if (static_cast<uint32_t>(u) < n_units) {
+            const bool hit = ((columns[u] >> bit) & 1u) != 0;
+            const uint64_t mask = __ballot(hit);
+            if (hit) {
+                const uint32_t slot = min(staged + n_rows + rank_in_mask(mask), ORDERED_STAGED - 1);
+                sh.keys[slot] = (static_cast<uint64_t>(cand_index[u]) << 32) | (cand_biased[u] + wrap_i);
+                sh.key_at[slot] = point;
+            }
+            n_rows += __popcll(mask);
+        }
+    }
+    return n_rows;
+}
+
+/// Stores the first `count` staged keys as the rows `first_row` ... of the list: 64 consecutive rows per step, each
+/// step ending on a multiple of 64 rows (whole cache lines in every output array; the first step stores fewer).
+template <typename Shared>
+__device__ __forceinline__ void store_staged_rows(
+    const Shared& sh, const double* __restrict__ points, const GridParams& g, const SearchOutputs& out, uint32_t count,
+    uint64_t first_row, int lane
+) {
+    const uint32_t skew = static_cast<uint32_t>(first_row % WAVE);
+    for (uint32_t e0 = 0; e0 < count + skew; e0 += WAVE) {
+        const uint32_t e = e0 + lane - skew;
+        if (e >= count) {
+            continue; // (before the first row as well: unsigned)
+        }
+        const uint64_t key = sh.keys[e];
+        const uint32_t point = sh.key_at[e];
+        const uint32_t oj = static_cast<uint32_t>(key >> 32);
+        const double xj = points[3 * static_cast<size_t>(oj) + 0];
+        const double yj = points[3 * static_cast<size_t>(oj) + 1];
+        const double zj = points[3 * static_cast<size_t>(oj) + 2];
+        const uint32_t biased = static_cast<uint32_t>(key);
+        const int32_t sx = static_cast<int32_t>((biased >> 20) & 0x3ffu) - 512;
+        const int32_t sy = static_cast<int32_t>((biased >> 10) & 0x3ffu) - 512;
+        const int32_t sz = static_cast<int32_t>(biased & 0x3ffu) - 512;
+        double tx, ty, tz;
+        shift_vector(g, sx, sy, sz, tx, ty, tz);
+        const double vx = (xj - sh.tile_x[point]) + tx;
+        const double vy = (yj - sh.tile_y[point]) + ty;
+        const double vz = (zj - sh.tile_z[point]) + tz;
+        const uint64_t row = first_row + e;
+        stream_store(out.pairs + 2 * row, PairRow{sh.tile_index[point], oj});
+        if (out.shifts != nullptr) {
+            stream_store(out.shifts + 3 * row, ShiftRow{sx, sy, sz});
+        }
+        if (out.distances != nullptr) {
+            stream_store(out.distances + row, sqrt(vx * vx + vy * vy + vz * vz));
+        }
+        if (out.vectors != nullptr) {
+            stream_store(out.vectors + 3 * row, VectorHead{vx, vy});
+            stream_store(out.vectors + 3 * row + 2, vz);
+        }
+    }
+}
+
 /// PRESORTED (WRITE only): the candidates are taken in the order ordered_sort_kernel left for the tile, and the hits
 /// of a point in lane order are its rows in final order. Otherwise (small systems, where one more launch costs more
 /// than it saves) candidates come in table order and the rows of every point are ranked by comparing all its keys.
@@ -769,6 +842,60 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
         // store the rows
         wave_sync();
         const uint32_t per_part = (n_i + split - 1) / split;
+        if constexpr (PRESORTED) {
+            // The points in the order of their original indices: the rows of points with consecutive indices are
+            // consecutive rows of the list (inputs in the order of a lattice have runs of them in every cell). Their
+            // rows are lined up in LDS one point after the other and stored 64 at a time, from multiples of 64 rows.
+            if (static_cast<uint32_t>(lane) < n_i) {
+                const uint32_t own = sh.tile_index[lane];
+                uint32_t smaller = 0;
+                for (uint32_t other = 0; other < n_i; other++) {
+                    smaller += sh.tile_index[other] < own ? 1u : 0u;
+                }
+                sh.by_index[smaller] = lane;
+            }
+            wave_sync();
+            uint32_t staged = 0;
+            uint64_t staged_row = 0; // row of the first staged key
+            for (uint32_t turn = part * per_part; turn < min(n_i, (part + 1) * per_part); turn++) {
+                const uint32_t p = uniform(sh.by_index[turn]);
+                const uint64_t row_p = uniform(sh.tile_row[p]);
+                if (staged != 0 && row_p != staged_row + staged) {
+                    store_staged_rows(sh, args.points, g, args.out, staged, staged_row, lane);
+                    staged = 0;
+                    wave_sync();
+                }
+                if (staged == 0) {
+                    staged_row = row_p;
+                }
+                const uint32_t wrap_i = (static_cast<uint32_t>(sh.tile_wx[p]) << 20) + (static_cast<uint32_t>(sh.tile_wy[p]) << 10) +
+                                        static_cast<uint32_t>(sh.tile_wz[p]);
+                staged += stage_rows_of_point(sh, columns, cand_index, cand_biased, n_units, n_i - 1 - p, wrap_i, p, staged);
+                staged = min(staged, ORDERED_STAGED); // (a point has at most ORDERED_MAX_ROWS rows here)
+                wave_sync();
+                const uint64_t whole = ((staged_row + staged) & ~static_cast<uint64_t>(WAVE - 1));
+                if (whole > staged_row) {
+                    // everything up to the last multiple of 64 rows; what is left moves to the front
+                    const uint32_t count = static_cast<uint32_t>(whole - staged_row);
+                    store_staged_rows(sh, args.points, g, args.out, count, staged_row, lane);
+                    const uint32_t left = staged - count; // < 64
+                    const uint64_t key = sh.keys[min(count + lane, ORDERED_STAGED - 1)];
+                    const uint32_t point = sh.key_at[min(count + lane, ORDERED_STAGED - 1)];
+                    wave_sync();
+                    if (static_cast<uint32_t>(lane) < left) {
+                        sh.keys[lane] = key;
+                        sh.key_at[lane] = point;
+                    }
+                    staged_row = whole;
+                    staged = left;
+                    wave_sync();
+                }
+            }
+            if (staged != 0) {
+                store_staged_rows(sh, args.points, g, args.out, staged, staged_row, lane);
+            }
+            return;
+        }
         for (uint32_t p = part * per_part; p < min(n_i, (part + 1) * per_part); p++) {
             // every field of the sum stays inside its ten bits (operands within +-255), so the fields add independently
             const uint32_t wrap_i = (static_cast<uint32_t>(sh.tile_wx[p]) << 20) + (static_cast<uint32_t>(sh.tile_wy[p]) << 10) +
