@@ -295,10 +295,14 @@ def test_batch_errors():
 
 
 @pytest.mark.parametrize("full", [True, False], ids=["full", "half"])
-def test_sorted_batch_equals_sorted_single_calls(full):
+def test_sorted_batch_equals_sorted_single_calls(full, capfd, monkeypatch):
     """sorted=True in a batch: every system's rows in the order vesin_neighbors gives for that system alone
-    ((i, j, shift) lexicographic), compared in place with the oracle's rows put in that order and with single calls."""
+    ((i, j, shift) lexicographic), compared in place with the oracle's rows put in that order and with single calls.
+    Systems of one cell and of several: the rows come out of the two searches that write them in order, and
+    through the two passes and the radix sort when VESIN_HIP_SORT=radix asks for that."""
     import torch
+
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
 
     rng = np.random.default_rng(57)
     all_points, all_boxes, all_flags = [], [], []
@@ -309,21 +313,32 @@ def test_sorted_batch_equals_sorted_single_calls(full):
         all_flags.append((True, True, True))
     for n, flags in ((0, (True, True, True)), (1, (True, True, True)), (150, (False, False, False)), (400, (True, False, True)),
                      (700, (True, True, True))):
-        edge = 7.0 + 3.0 * rng.random()
+        # (at most 0.08 points per cubic A: the search that writes rows in order holds 1024 candidates around a tile)
+        edge = max(7.0 + 3.0 * rng.random(), (n / 0.08) ** (1.0 / 3.0))
         box = np.eye(3) * edge + 0.4 * rng.normal(size=(3, 3))
         all_points.append(rng.random((n, 3)) @ box + rng.integers(-1, 2, size=(n, 3)) @ box)
         all_boxes.append(box)
         all_flags.append(flags)
     cutoff = 4.2
-    calculator = NeighborList(cutoff=cutoff, full_list=full, sorted=True)
     complete = None
-    for letters in ("PSdD", "Pd"):
-        lists = run_batch(calculator, all_points, all_boxes, letters=letters, periodic=np.array(all_flags))
-        for s, (points, box, flags) in enumerate(zip(all_points, all_boxes, all_flags)):
-            expected = oracle.canonicalize(oracle.neighbors(points, box, list(flags), cutoff, full, False, "ijSdD"))
-            for key in lists[s]:
-                assert np.array_equal(lists[s][key], expected[key]), f"system {s}, {letters}: {key} differ or are out of order"
-        complete = complete or lists
+    for way in ("in order", "radix"):
+        if way == "radix":
+            monkeypatch.setenv("VESIN_HIP_SORT", "radix")
+        calculator = NeighborList(cutoff=cutoff, full_list=full, sorted=True)
+        for letters in ("PSdD", "Pd"):
+            capfd.readouterr()
+            lists = run_batch(calculator, all_points, all_boxes, letters=letters, periodic=np.array(all_flags))
+            taken = [line for line in capfd.readouterr().err.splitlines() if line.startswith("in-order search (batch)")]
+            if way == "radix":
+                assert not taken
+            else:
+                assert len(taken) == 2 and all(line.endswith(": used") for line in taken), taken
+            for s, (points, box, flags) in enumerate(zip(all_points, all_boxes, all_flags)):
+                expected = oracle.canonicalize(oracle.neighbors(points, box, list(flags), cutoff, full, False, "ijSdD"))
+                for key in lists[s]:
+                    assert np.array_equal(lists[s][key], expected[key]), f"system {s}, {letters}, {way}: {key} differ or are out of order"
+            complete = complete or lists
+    monkeypatch.delenv("VESIN_HIP_SORT")
     # the same through one call per system
     single = NeighborList(cutoff=cutoff, full_list=full, sorted=True)
     for s in (0, 6, 7):

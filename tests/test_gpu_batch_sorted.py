@@ -1,5 +1,6 @@
-"""``sorted=True`` on ``vesin_hip_neighbors_batch`` for systems of a single cell (``-m gpu``): the rows come out of the
-search in (i, j, shift) order, system after system, with nothing sorted afterwards. Every call is compared row by row,
+"""``sorted=True`` on ``vesin_hip_neighbors_batch`` (``-m gpu``): the rows come out of the search in (i, j, shift)
+order, system after system, with nothing sorted afterwards: systems of a single cell through the search over their
+images, the others through the search over the tiles of their whole stencil. Every call is compared row by row,
 in place, with the oracle's rows put in that order (vesin/include/vesin.h:55-57, vesin/src/cpu_cell_list.cpp:634-730),
 and what the library says about the way it took (VESIN_HIP_DEBUG) is checked too."""
 
@@ -135,10 +136,15 @@ def test_a_list_that_grows_and_brute_force(capfd, monkeypatch):
     _call_and_check(calculator, systems_of([250, 256, 200, 3], 9.0), cutoff, True, "PSdD", "dense")
     lines = _in_order_lines(capfd)
     assert len(lines) == 3 and all(line.endswith(": used") for line in lines), lines
-    # a system of 300 points in one cell is not this search's: the host knows, and does not ask the device
+    # a system of 300 points in one cell is left to the search over tiles, whose counting pass finds more candidates
+    # around a tile than it holds: the rows come from the two passes and the sort, and the next call does not ask again
     _call_and_check(calculator, systems_of([300, 20], 9.0), cutoff, True, "PSdD", "too many points in one cell")
-    assert not _in_order_lines(capfd)
+    lines = _in_order_lines(capfd)
+    assert len(lines) == 1 and lines[0].endswith(": left to the radix sort"), lines
     _call_and_check(calculator, systems_of([30, 20], 9.0), cutoff, True, "PSdD", "small again")
+    assert not _in_order_lines(capfd)
+    another = NeighborList(cutoff=cutoff, full_list=True, sorted=True, algorithm="brute_force")
+    _call_and_check(another, systems_of([30, 20], 9.0), cutoff, True, "PSdD", "small, another list")
     assert _in_order_lines(capfd)[-1].endswith(": used")
 
 
@@ -171,4 +177,63 @@ def test_molecules_whose_grids_are_picked_on_the_device(capfd, monkeypatch):
     lines = _in_order_lines(capfd)
     assert len(lines) == 1 and lines[0].endswith(": left to the radix sort"), lines
     _call_and_check(calculator, systems(), cutoff, True, "PSdD", "the call after")
+    assert not _in_order_lines(capfd)
+
+
+def _systems_of_several_cells(rng, sizes_and_flags):
+    systems = []
+    for n, flags in sizes_and_flags:
+        edge = (n / 0.06) ** (1.0 / 3.0)
+        box = np.eye(3) * edge + 0.05 * edge * rng.normal(size=(3, 3))
+        moved = (rng.integers(-1, 2, size=(n, 3)) * np.array(flags)) @ box
+        systems.append((rng.random((n, 3)) @ box + moved, box, flags))
+    return systems
+
+
+@pytest.mark.parametrize("full", [True, False], ids=["full", "half"])
+def test_systems_of_several_cells_come_out_in_order(full, capfd, monkeypatch):
+    """Systems of a few hundred to a few thousand points with several cells each (periodic, slabs, wires, clusters;
+    points up to a box vector outside of the box), and the same together with systems of one cell: both searches in
+    one call, one scan over the points of all systems."""
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    rng = np.random.default_rng(575)
+    cutoff = 4.0
+    several = _systems_of_several_cells(rng, [
+        (700, (True, True, True)), (300, (True, True, False)), (1500, (True, False, False)), (450, (False, False, False)),
+        (3000, (True, True, True)), (33, (True, True, True)),
+    ])
+    calculator = NeighborList(cutoff=cutoff, full_list=full, sorted=True)
+    capfd.readouterr()
+    for call, letters in (("first call", "PSdD"), ("second call", "PSdD"), ("third call", "Pd")):
+        _call_and_check(calculator, several, cutoff, full, letters, call)
+        lines = _in_order_lines(capfd)
+        assert len(lines) == 1 and lines[0].endswith(": used") and " 0 systems by images" in lines[0], (call, lines)
+    mixed = several[:3] + _small_cell_systems(rng) + several[3:]
+    for call in ("mixed, first call", "mixed, second call"):
+        _call_and_check(calculator, mixed, cutoff, full, "PSdD", call)
+        lines = _in_order_lines(capfd)
+        assert len(lines) == 1 and lines[0].endswith(": used") and " 0 systems by" not in lines[0], (call, lines)
+
+
+def test_a_dense_system_among_the_others(capfd, monkeypatch):
+    """One system with more candidates around a tile than the search over tiles holds (1024): its counting pass says
+    so, nothing is written in order, and the rows of the whole batch come from the two passes and the sort."""
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    rng = np.random.default_rng(576)
+    cutoff = 4.0
+    systems = _systems_of_several_cells(rng, [(600, (True, True, True)), (900, (True, True, True))])
+    edge = 20.3
+    systems.append((rng.random((2500, 3)) * edge, np.eye(3) * edge, (True, True, True)))  # 0.3 per cubic A: 80 rows per point
+    edge = 12.0
+    systems.append((rng.random((2500, 3)) * edge, np.eye(3) * edge, (True, True, True)))  # 1.45 per cubic A: every point a candidate
+    calculator = NeighborList(cutoff=cutoff, full_list=True, sorted=True)
+    capfd.readouterr()
+    _call_and_check(calculator, systems[:3], cutoff, True, "PSd", "up to 1024 candidates per tile")
+    _call_and_check(calculator, systems[:3], cutoff, True, "PSd", "again")
+    lines = _in_order_lines(capfd)
+    assert len(lines) == 2 and all(line.endswith(": used") for line in lines), lines
+    _call_and_check(calculator, systems, cutoff, True, "PSd", "more than 1024 candidates around a tile")
+    lines = _in_order_lines(capfd)
+    assert len(lines) == 1 and lines[0].endswith(": left to the radix sort"), lines
+    _call_and_check(calculator, systems, cutoff, True, "PSd", "the call after")
     assert not _in_order_lines(capfd)

@@ -495,6 +495,7 @@ struct BatchSetup {
     // it; after a batch that did not, the next calls go to the two passes and the sort without asking again.
     int in_order_rest = 0;
     size_t systems_for_images = 0;          // systems the search over images covers (grids picked on the host)
+    size_t systems_for_tiles = 0;           // other systems whose stencil fits the in-order search over tiles
     size_t systems_with_points = 0;
     PinnedVector<uint64_t> pair_base;       // pairs of points (n^2 per system of few points) before every system
     uint32_t image_words = 1;               // words of 64 images per pair of points, the most any system needs
@@ -2053,7 +2054,7 @@ bool compute(
         const bool presorted = ordered_items_per_tile == 1;
         auto launch_order = [&](hipStream_t where) {
             hipLaunchKernelGGL(
-                ordered_sort_kernel, dim3(static_cast<uint32_t>((tiles_bound + ORDER_WAVES - 1) / ORDER_WAVES)),
+                ordered_sort_kernel<false>, dim3(static_cast<uint32_t>((tiles_bound + ORDER_WAVES - 1) / ORDER_WAVES)),
                 dim3(ORDER_BLOCK), 0, where, oargs, g
             );
         };
@@ -2742,6 +2743,7 @@ bool batch_attempt(
 
         uint64_t cells_so_far = 0;
         setup.systems_for_images = 0;
+        setup.systems_for_tiles = 0;
         setup.systems_with_points = 0;
         setup.image_words = 1;
         setup.pair_base.resize(n_systems + 1);
@@ -2778,6 +2780,8 @@ bool batch_attempt(
             if (n_here > 0 && images_cover(g)) {
                 setup.systems_for_images += 1;
                 setup.image_words = std::max(setup.image_words, image_words(g));
+            } else if (n_here > 0 && static_cast<uint64_t>(2 * g.s[0] + 1) * (2 * g.s[1] + 1) * (2 * g.s[2] + 1) <= MAX_ENTRIES) {
+                setup.systems_for_tiles += 1;
             }
             setup.pair_base[s] = pairs_so_far;
             pairs_so_far += n_here <= IMAGE_MAX_POINTS ? n_here * n_here : 0;
@@ -2871,22 +2875,31 @@ bool batch_attempt(
     unsigned long long* d_first_pair = nullptr;
     uint32_t* d_cells_of_system = nullptr;
     char* clear_end = nullptr;
-    // A sorted list straight from the search (images.cuh), when every system has the shape for it. With grids picked
-    // on the device the host does not know: the kernels say.
+    // A sorted list straight from the search, when every system has the shape for one of the two that write their rows
+    // in order: systems of one cell over their images (images.cuh), the others over the tiles of their whole stencil
+    // (ordered.cuh). With grids picked on the device the host does not know the shapes: only the search over images is
+    // tried then (such systems have no periodic direction and are mostly small), and its kernels say what they met.
     bool try_in_order = options.sorted && !radix_sort_only() &&
-                        (device_grids || setup.systems_for_images == setup.systems_with_points);
-    // (what the counting pass leaves for the writing pass: a bit per pair of points and image)
-    const size_t hit_words = static_cast<size_t>(setup.pair_base[n_systems]) * setup.image_words;
-    try_in_order = try_in_order && ordered_records_fit(n_points, hit_words * sizeof(uint64_t));
+                        (device_grids || setup.systems_for_images + setup.systems_for_tiles == setup.systems_with_points);
+    const bool in_order_images = device_grids || setup.systems_for_images > 0;
+    const bool in_order_tiles = !device_grids && setup.systems_for_tiles > 0;
+    // (what the counting passes leave for the writing passes: a bit per pair of points and image; a record per
+    // candidate of every tile)
+    const size_t hit_words = in_order_images ? static_cast<size_t>(setup.pair_base[n_systems]) * setup.image_words : 0;
+    const size_t record_slots = in_order_tiles ? tiles_bound : 0;
+    try_in_order = try_in_order &&
+                   ordered_records_fit(
+                       n_points, hit_words * sizeof(uint64_t) + record_slots * ORDERED_CANDIDATES * sizeof(CandidateRecord)
+                   );
     if (try_in_order && setup.in_order_rest > 0) {
         setup.in_order_rest -= 1;
         try_in_order = false;
     }
-    if (options.sorted && !device_grids && setup.systems_for_images != setup.systems_with_points &&
-        std::getenv("VESIN_HIP_DEBUG") != nullptr) {
+    if (options.sorted && !device_grids && std::getenv("VESIN_HIP_DEBUG") != nullptr &&
+        setup.systems_for_images + setup.systems_for_tiles != setup.systems_with_points) {
         std::fprintf(
-            stderr, "sorted batch: %zu of %zu systems are of one cell, the rows are sorted after the search\n",
-            setup.systems_for_images, setup.systems_with_points
+            stderr, "sorted batch: %zu of %zu systems have a stencil of more than %d cells, the rows are sorted after the search\n",
+            setup.systems_with_points - setup.systems_for_images - setup.systems_for_tiles, setup.systems_with_points, MAX_ENTRIES
         );
     }
     OrderedStatus* ordered_status = nullptr;
@@ -2894,6 +2907,9 @@ bool batch_attempt(
     uint64_t* first_row_of_point = nullptr;
     uint64_t* image_hits = nullptr;
     uint64_t* d_pair_base = nullptr;
+    CandidateRecord* candidate_records = nullptr;
+    uint32_t* candidates_of_item = nullptr;
+    uint16_t* candidate_order = nullptr;
     const size_t scratch_elements = std::max(
         std::max(scan_scratch_elements(total_cells), scan_scratch_elements(n_slots)),
         try_in_order ? scan_scratch_elements(n_points) : size_t(0)
@@ -2930,6 +2946,9 @@ bool batch_attempt(
         d_cells_of_system = carver.take<uint32_t>(n_systems);
         d_pair_base = carver.take<uint64_t>(try_in_order ? n_systems + 1 : 0);
         image_hits = carver.take<uint64_t>(try_in_order ? hit_words : 0);
+        candidate_records = carver.take<CandidateRecord>(try_in_order ? record_slots * ORDERED_CANDIDATES : 0);
+        candidates_of_item = carver.take<uint32_t>(try_in_order ? record_slots : 0);
+        candidate_order = carver.take<uint16_t>(try_in_order ? record_slots * ORDERED_CANDIDATES : 0);
     };
     Carver measure(nullptr);
     carve(measure);
@@ -3040,8 +3059,9 @@ bool batch_attempt(
         }
     };
 
-    // ---- a sorted list straight from the search: systems of one cell, by brute force over their images in the
-    // order of the list (images.cuh)
+    // ---- a sorted list straight from the search: systems of one cell by brute force over their images in the order
+    // of the list (images.cuh), the others by the tiles of their whole stencil (ordered.cuh); one scan over the points
+    // of all systems gives every point its first row
     if (try_in_order) {
         ImageArgs iargs = {};
         iargs.sorted = sorted;
@@ -3054,21 +3074,76 @@ bool batch_attempt(
         iargs.words = setup.image_words;
         iargs.n_systems = static_cast<uint32_t>(n_systems);
         iargs.total_points = static_cast<uint32_t>(n_points);
+        iargs.others_covered = in_order_tiles ? 1u : 0u;
         iargs.rows_of_point = rows_of_point;
         iargs.first_row = first_row_of_point;
         iargs.status = ordered_status;
+        OrderedArgs oargs = {};
+        oargs.sorted = sorted;
+        oargs.cell_scan = cell_scan;
+        oargs.tiles = tiles;
+        oargs.points_per_item = TILE_POINTS;
+        oargs.items_per_tile = 1;
+        oargs.rows_of_point = rows_of_point;
+        oargs.records = candidate_records;
+        oargs.candidates_of_item = candidates_of_item;
+        oargs.write_split = 1;
+        oargs.count_split = 1;
+        oargs.points = flat_points;
+        oargs.order = candidate_order;
+        oargs.first_row = first_row_of_point;
+        oargs.status = ordered_status;
+        oargs.grids = d_grids;
+        oargs.cell_base = d_cell_base;
+        oargs.first_point = d_first_point;
+        oargs.total_cells = static_cast<uint32_t>(total_cells);
+        oargs.total_points = static_cast<uint32_t>(n_points);
         const dim3 image_grid(static_cast<uint32_t>(n_systems));
-        auto launch_write = [&]() {
-            if (options.full) {
-                hipLaunchKernelGGL(image_write_kernel<true>, image_grid, dim3(IMAGE_BLOCK), 0, stream, iargs);
-            } else {
-                hipLaunchKernelGGL(image_write_kernel<false>, image_grid, dim3(IMAGE_BLOCK), 0, stream, iargs);
+        const dim3 tile_grid(static_cast<uint32_t>((tiles_bound + ORDERED_WAVES - 1) / ORDERED_WAVES));
+        // (whichever writing pass is launched last hands the host what the counting passes found)
+        auto launch_write = [&](OrderedHostStatus* publish_to) {
+            if (in_order_images) {
+                iargs.publish_to = in_order_tiles ? nullptr : publish_to;
+                iargs.build_status = extras.d_status;
+                if (options.full) {
+                    hipLaunchKernelGGL(image_write_kernel<true>, image_grid, dim3(IMAGE_BLOCK), 0, stream, iargs);
+                } else {
+                    hipLaunchKernelGGL(image_write_kernel<false>, image_grid, dim3(IMAGE_BLOCK), 0, stream, iargs);
+                }
+            }
+            if (in_order_tiles) {
+                oargs.publish_to = publish_to;
+                oargs.build_status = extras.d_status;
+                if (options.full) {
+                    hipLaunchKernelGGL((ordered_search_kernel<true, true, true, true>), tile_grid, dim3(ORDERED_BLOCK), 0, stream, oargs, GridParams{});
+                } else {
+                    hipLaunchKernelGGL((ordered_search_kernel<true, false, true, true>), tile_grid, dim3(ORDERED_BLOCK), 0, stream, oargs, GridParams{});
+                }
             }
         };
-        if (options.full) {
-            hipLaunchKernelGGL(image_count_kernel<true>, image_grid, dim3(IMAGE_BLOCK), 0, stream, iargs);
-        } else {
-            hipLaunchKernelGGL(image_count_kernel<false>, image_grid, dim3(IMAGE_BLOCK), 0, stream, iargs);
+        auto outputs_into = [&](SearchOutputs& out) {
+            out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
+            out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
+            out.distances = neighbors.distances;
+            out.vectors = reinterpret_cast<double*>(neighbors.vectors);
+        };
+        if (in_order_images) {
+            if (options.full) {
+                hipLaunchKernelGGL(image_count_kernel<true>, image_grid, dim3(IMAGE_BLOCK), 0, stream, iargs);
+            } else {
+                hipLaunchKernelGGL(image_count_kernel<false>, image_grid, dim3(IMAGE_BLOCK), 0, stream, iargs);
+            }
+        }
+        if (in_order_tiles) {
+            if (options.full) {
+                hipLaunchKernelGGL((ordered_search_kernel<false, true, false, true>), tile_grid, dim3(ORDERED_BLOCK), 0, stream, oargs, GridParams{});
+            } else {
+                hipLaunchKernelGGL((ordered_search_kernel<false, false, false, true>), tile_grid, dim3(ORDERED_BLOCK), 0, stream, oargs, GridParams{});
+            }
+            hipLaunchKernelGGL(
+                ordered_sort_kernel<true>, dim3(static_cast<uint32_t>((tiles_bound + ORDER_WAVES - 1) / ORDER_WAVES)),
+                dim3(ORDER_BLOCK), 0, stream, oargs, GridParams{}
+            );
         }
         exclusive_scan<SCAN_U32>(rows_of_point, n_points, first_row_of_point, scan_scratch, stream);
         // A list that has arrays from earlier calls writes into them without waiting for the host to learn what the
@@ -3078,16 +3153,11 @@ bool batch_attempt(
         if (early_write) {
             size_outputs(neighbors, extras, 0, options);
             early_capacity = extras.capacity;
-            iargs.out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
-            iargs.out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
-            iargs.out.distances = neighbors.distances;
-            iargs.out.vectors = reinterpret_cast<double*>(neighbors.vectors);
-            iargs.capacity = early_capacity;
-            iargs.guarded = 1;
-            iargs.publish_to = &extras.mail_device->ordered;
-            iargs.build_status = extras.d_status;
-            launch_write();
-            iargs.publish_to = nullptr;
+            outputs_into(iargs.out);
+            outputs_into(oargs.out);
+            iargs.capacity = oargs.capacity = early_capacity;
+            iargs.guarded = oargs.guarded = 1;
+            launch_write(&extras.mail_device->ordered);
         } else {
             hipLaunchKernelGGL(
                 publish_ordered_status, dim3(1), dim3(1), 0, stream,
@@ -3110,26 +3180,29 @@ bool batch_attempt(
         if (found.first_bad_coordinate != 0xFFFFFFFFu) {
             non_finite_error(points, found.first_bad_coordinate);
         }
+        const bool suitable = found.found.unsuitable == 0 && found.found.max_rows <= ORDERED_MAX_ROWS &&
+                              found.found.max_candidates <= ORDERED_CANDIDATES;
         if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
             std::fprintf(
-                stderr, "in-order search (batch): rows %llu, systems left uncovered %u%s: %s\n", found.total_rows,
-                found.found.unsuitable, device_grids ? ", grids picked on the device" : "",
-                found.found.unsuitable == 0 ? "used" : "left to the radix sort"
+                stderr,
+                "in-order search (batch): rows %llu, %zu systems by images, %zu by tiles (most rows of a point %u, most "
+                "candidates of a tile %u), unsuitable %u%s: %s\n",
+                found.total_rows, setup.systems_for_images, in_order_tiles ? setup.systems_for_tiles : size_t(0),
+                found.found.max_rows, found.found.max_candidates, found.found.unsuitable,
+                device_grids ? ", grids picked on the device" : "", suitable ? "used" : "left to the radix sort"
             );
         }
-        if (found.found.unsuitable == 0) {
+        if (suitable) {
             const size_t total = found.total_rows;
             check_pair_limit(total);
             if (!(early_write && total <= early_capacity)) {
                 // first call of the list, or more rows than its arrays hold
                 size_outputs(neighbors, extras, total, options);
-                iargs.out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
-                iargs.out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
-                iargs.out.distances = neighbors.distances;
-                iargs.out.vectors = reinterpret_cast<double*>(neighbors.vectors);
-                iargs.guarded = 0;
+                outputs_into(iargs.out);
+                outputs_into(oargs.out);
+                iargs.guarded = oargs.guarded = 0;
                 if (total > 0) {
-                    launch_write();
+                    launch_write(nullptr);
                 }
                 HIP_CHECK(hipStreamSynchronize(stream));
             }
@@ -3138,8 +3211,9 @@ bool batch_attempt(
             neighbors.length = total;
             return true;
         }
-        // a system of several cells, of many points or of very many images: the two passes and the sort below, and
-        // for a while without asking again
+        // a system beyond what either search covers (grids picked on the device: of several cells, of many points; more
+        // than 256 rows for a point or 1024 candidates around a tile; wraps beyond +-255): the two passes and the sort
+        // below, and for a while without asking again
         setup.in_order_rest = SINGLE_PASS_REST;
     }
 

@@ -35,21 +35,13 @@
 
 namespace vesin_hip {
 
-constexpr uint32_t IMAGE_MAX_POINTS = 256;
-constexpr uint32_t IMAGE_MAX_ENTRIES = 128; // a pair of points keeps a bit per image in two words
+// (IMAGE_MAX_POINTS, IMAGE_MAX_ENTRIES and images_cover, which say what systems this search covers: ordered.cuh)
 constexpr uint32_t IMAGE_MAX_WORDS = IMAGE_MAX_ENTRIES / 64;
 constexpr int IMAGE_WAVES = 4;
 constexpr int IMAGE_BLOCK = IMAGE_WAVES * WAVE;
 constexpr int IMAGE_GROUP = 2;             // units of 64 pairs of points a wave tests together
 constexpr uint32_t IMAGE_ROWS = 16 * WAVE; // rows of a first point that a wave lines up in LDS at a time
 static_assert(IMAGE_MAX_POINTS <= 256 && IMAGE_MAX_ENTRIES <= 256, "a row is lined up as (second point << 8) | image in 16 bits");
-
-/// Whether this search covers the system of grid `g`.
-__host__ __device__ inline bool images_cover(const GridParams& g) {
-    const uint64_t n_stencil = static_cast<uint64_t>(2 * g.s[0] + 1) * static_cast<uint64_t>(2 * g.s[1] + 1) *
-                               static_cast<uint64_t>(2 * g.s[2] + 1);
-    return g.n_cells == 1 && g.n_points <= IMAGE_MAX_POINTS && n_stencil <= IMAGE_MAX_ENTRIES;
-}
 
 /// Words of 64 images that a pair of points of this system keeps (an upper bound: before the stencil is pruned).
 __host__ __device__ inline uint32_t image_words(const GridParams& g) {
@@ -71,9 +63,10 @@ struct ImageArgs {
     uint32_t total_points;
     uint32_t* rows_of_point;    // COUNT: [total_points], by first point of the system + index
     const uint64_t* first_row;  // WRITE: [total_points + 1], exclusive scan of rows_of_point
+    uint32_t others_covered;    // systems this search does not cover are another kernel's: they are not reported
     OrderedStatus* status;      // `unsuitable` counts the systems this search does not cover
     uint32_t guarded;           // WRITE launched before the host has seen what COUNT found: write nothing unless every
-                                // system was covered and the rows fit the `capacity` of the arrays
+                                // system suited its search and the rows fit the `capacity` of the arrays
     uint64_t capacity;
     SearchOutputs out;
     OrderedHostStatus* publish_to; // WRITE: when not null, the first workgroup hands the host what COUNT found
@@ -213,7 +206,7 @@ __global__ __launch_bounds__(IMAGE_BLOCK) void image_count_kernel(ImageArgs args
         return;
     }
     if (!images_cover(g) || image_words(g) > args.words) {
-        if (threadIdx.x == 0) {
+        if (threadIdx.x == 0 && args.others_covered == 0) {
             atomicAdd(&args.status->unsuitable, 1u);
         }
         return;
@@ -354,7 +347,10 @@ __global__ __launch_bounds__(IMAGE_BLOCK) void image_write_kernel(ImageArgs args
         *args.publish_to = report;
     }
     if (args.guarded != 0) {
-        const bool usable = args.status->unsuitable == 0 && args.first_row[args.total_points] <= args.capacity;
+        // (the same decision as the writing pass over tiles, which may serve other systems of the batch)
+        const OrderedStatus found = *args.status;
+        const bool usable = found.unsuitable == 0 && found.max_rows <= ORDERED_MAX_ROWS &&
+                            found.max_candidates <= ORDERED_CANDIDATES && args.first_row[args.total_points] <= args.capacity;
         if (!usable) {
             return;
         }

@@ -98,7 +98,26 @@ struct OrderedArgs {
     const DeviceStatus* build_status;
     // COUNT: the single-precision pre-test (choose_prefilter, geometry.hpp); used when `sorted.l` is there
     Prefilter pre;
+    // many systems in one launch (batched entry point; the kernels' BATCH variants): the grid of every system, its
+    // first cell in the concatenated grids and its first point; rows_of_point and first_row go by first point of the
+    // system + index in the system
+    const GridParams* grids;
+    const uint32_t* cell_base;
+    const uint32_t* first_point;
+    uint32_t total_cells;
+    uint32_t total_points;
 };
+
+/// Systems of one cell and few points in a batch are searched over their images instead (images.cuh): the kernels
+/// here leave their tiles alone.
+constexpr uint32_t IMAGE_MAX_POINTS = 256;
+constexpr uint32_t IMAGE_MAX_ENTRIES = 128; // a pair of points keeps a bit per image in two words
+
+__host__ __device__ inline bool images_cover(const GridParams& g) {
+    const uint64_t n_stencil = static_cast<uint64_t>(2 * g.s[0] + 1) * static_cast<uint64_t>(2 * g.s[1] + 1) *
+                               static_cast<uint64_t>(2 * g.s[2] + 1);
+    return g.n_cells == 1 && g.n_points <= IMAGE_MAX_POINTS && n_stencil <= IMAGE_MAX_ENTRIES;
+}
 
 /// LDS of one wave. What is known per candidate (hit column, position, original index, shift) stays in the
 /// registers of the lane that loaded it: a lane only ever needs its own candidates until it hands a hit over as a key.
@@ -614,30 +633,34 @@ __device__ __forceinline__ void store_staged_rows(
 /// PRESORTED (WRITE only): the candidates are taken in the order ordered_sort_kernel left for the tile, and the hits
 /// of a point in lane order are its rows in final order. Otherwise (small systems, where one more launch costs more
 /// than it saves) candidates come in table order and the rows of every point are ranked by comparing all its keys.
-template <bool WRITE, bool FULL, bool PRESORTED = false>
-__global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void ordered_search_kernel(OrderedArgs args, GridParams g) {
+/// BATCH: the tiles of many systems (every tile knows its system, whose grid it takes); systems that the search over
+/// images covers are skipped.
+template <bool WRITE, bool FULL, bool PRESORTED = false, bool BATCH = false>
+__global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4))) void ordered_search_kernel(OrderedArgs args, GridParams single_grid) {
     constexpr int R = ORDERED_R;
     __shared__ OrderedShared<WRITE> shared;
     const int lane = lane_id();
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     auto& sh = shared.wave[wave];
+    const uint32_t all_points = BATCH ? args.total_points : single_grid.n_points;
+    const uint32_t all_cells = BATCH ? args.total_cells : single_grid.n_cells;
     if (WRITE && args.publish_to != nullptr && blockIdx.x == 0 && threadIdx.x == 0) {
         OrderedHostStatus report;
         report.found = *args.status;
-        report.total_rows = args.first_row[g.n_points];
+        report.total_rows = args.first_row[all_points];
         report.first_bad_coordinate = args.build_status->first_bad_coordinate;
-        report.n_tiles = static_cast<unsigned int>(args.cell_scan[g.n_cells] >> 32);
+        report.n_tiles = static_cast<unsigned int>(args.cell_scan[all_cells] >> 32);
         *args.publish_to = report;
     }
     if (WRITE && args.guarded != 0) {
         const OrderedStatus found = *args.status;
         const bool suitable = found.max_rows <= ORDERED_MAX_ROWS && found.max_candidates <= ORDERED_CANDIDATES &&
-                              found.unsuitable == 0 && args.first_row[g.n_points] <= args.capacity;
+                              found.unsuitable == 0 && args.first_row[all_points] <= args.capacity;
         if (!suitable) {
             return;
         }
     }
-    const uint32_t n_tiles = static_cast<uint32_t>(args.cell_scan[g.n_cells] >> 32);
+    const uint32_t n_tiles = static_cast<uint32_t>(args.cell_scan[all_cells] >> 32);
     // WRITE may deal the points of a work item of the counting pass to several waves (`write_split`): they read the
     // same records and each writes the rows of its share of the points
     // COUNT may deal the candidates of a work item to several waves (`count_split`), by pairs of units in turn
@@ -665,9 +688,25 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
     const uint32_t n_i = min(tile.count - p_begin, args.points_per_item);
     const uint32_t first_i = tile.first + p_begin;
     const bool tile_wrapped = (tile.wrapped & 1u) != 0;
-    const int32_t cx = tile.cell % g.n[0];
-    const int32_t cy = (tile.cell / g.n[0]) % g.n[1];
-    const int32_t cz = tile.cell / (g.n[0] * g.n[1]);
+    // the grid: the kernel's argument, or this tile's system's
+    GridParams batch_grid;
+    uint32_t first_cell = 0;
+    uint32_t first_point = 0;
+    if (BATCH) {
+        const uint32_t system = tile_system(tile);
+        batch_grid = args.grids[system];
+        first_cell = args.cell_base[system];
+        first_point = args.first_point[system];
+        if (images_cover(batch_grid)) {
+            return;
+        }
+    }
+    const GridParams& g = BATCH ? batch_grid : single_grid;
+    const uint64_t* __restrict__ cell_scan = args.cell_scan + first_cell;
+    const uint32_t local_cell = tile.cell - first_cell;
+    const int32_t cx = local_cell % g.n[0];
+    const int32_t cy = (local_cell / g.n[0]) % g.n[1];
+    const int32_t cz = local_cell / (g.n[0] * g.n[1]);
 
     bool out_of_range = false;
     // COUNT: the single-precision pre-test, when the grid allows it and every point of the item has a place on record
@@ -697,7 +736,7 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
             sh.tile_wx[lane] = wx;
             sh.tile_wy[lane] = wy;
             sh.tile_wz[lane] = wz;
-            sh.tile_row[lane] = args.first_row[original];
+            sh.tile_row[lane] = args.first_row[first_point + original];
         }
     }
 
@@ -706,7 +745,11 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
     const int32_t span_z = 2 * g.s[2] + 1;
     const uint32_t n_stencil = static_cast<uint32_t>(2 * g.s[0] + 1) * span_y * span_z;
     if (n_stencil > MAX_ENTRIES) {
-        return; // the host does not launch this kernel for such a stencil
+        // the host does not launch this kernel for such a stencil; in a batch some system may have one
+        if (BATCH && !WRITE && lane == 0 && item == 0 && part == 0) {
+            atomicAdd(&args.status->unsuitable, 1u);
+        }
+        return;
     }
     uint32_t n_candidates;
     if constexpr (WRITE) {
@@ -715,7 +758,7 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
     } else {
         pretest = pretest && __ballot(place_unknown) == 0;
         fill_stencil_tables(
-            sh, lane, 0, n_stencil, cx, cy, cz, span_y, span_z, g, args.cell_scan, static_cast<const uint32_t*>(nullptr), 0u,
+            sh, lane, 0, n_stencil, cx, cy, cz, span_y, span_z, g, cell_scan, static_cast<const uint32_t*>(nullptr), 0u,
             pretest ? &sh.offsets : nullptr, &args.pre
         );
         n_candidates = __builtin_amdgcn_readfirstlane(sh.n_candidates);
@@ -771,11 +814,11 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
         }
         if (static_cast<uint32_t>(lane) < n_i) {
             if (split == 1) {
-                args.rows_of_point[sh.tile_index[lane]] = own_rows;
+                args.rows_of_point[first_point + sh.tile_index[lane]] = own_rows;
             } else {
                 // whichever wave of the item comes last sees the sum of the others: the largest number any of
                 // them sees for a point is the point's number of rows
-                own_rows += atomicAdd(&args.rows_of_point[sh.tile_index[lane]], own_rows);
+                own_rows += atomicAdd(&args.rows_of_point[first_point + sh.tile_index[lane]], own_rows);
             }
         }
         uint32_t most = own_rows;
@@ -842,6 +885,7 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
         // store the rows
         wave_sync();
         const uint32_t per_part = (n_i + split - 1) / split;
+        const double* system_points = args.points + 3 * static_cast<size_t>(first_point);
         if constexpr (PRESORTED) {
             // The points in the order of their original indices: the rows of points with consecutive indices are
             // consecutive rows of the list (inputs in the order of a lattice have runs of them in every cell). Their
@@ -861,7 +905,7 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
                 const uint32_t p = uniform(sh.by_index[turn]);
                 const uint64_t row_p = uniform(sh.tile_row[p]);
                 if (staged != 0 && row_p != staged_row + staged) {
-                    store_staged_rows(sh, args.points, g, args.out, staged, staged_row, lane);
+                    store_staged_rows(sh, system_points, g, args.out, staged, staged_row, lane);
                     staged = 0;
                     wave_sync();
                 }
@@ -877,7 +921,7 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
                 if (whole > staged_row) {
                     // everything up to the last multiple of 64 rows; what is left moves to the front
                     const uint32_t count = static_cast<uint32_t>(whole - staged_row);
-                    store_staged_rows(sh, args.points, g, args.out, count, staged_row, lane);
+                    store_staged_rows(sh, system_points, g, args.out, count, staged_row, lane);
                     const uint32_t left = staged - count; // < 64
                     const uint64_t key = sh.keys[min(count + lane, ORDERED_STAGED - 1)];
                     const uint32_t point = sh.key_at[min(count + lane, ORDERED_STAGED - 1)];
@@ -892,7 +936,7 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
                 }
             }
             if (staged != 0) {
-                store_staged_rows(sh, args.points, g, args.out, staged, staged_row, lane);
+                store_staged_rows(sh, system_points, g, args.out, staged, staged_row, lane);
             }
             return;
         }
@@ -902,7 +946,7 @@ __global__ __launch_bounds__(ORDERED_BLOCK) __attribute__((amdgpu_waves_per_eu(4
                                     static_cast<uint32_t>(sh.tile_wz[p]);
             // (the second points are looked up by their original index: no position to keep per candidate)
             write_rows_of_point<PRESORTED>(
-                sh, PointsByIndex{args.points}, g, args.out, columns, cand_index, cand_index, cand_biased, n_units, n_i - 1 - p, wrap_i,
+                sh, PointsByIndex{system_points}, g, args.out, columns, cand_index, cand_index, cand_biased, n_units, n_i - 1 - p, wrap_i,
                 sh.tile_x[p], sh.tile_y[p], sh.tile_z[p], sh.tile_index[p], sh.tile_row[p], lane
             );
         }
@@ -957,28 +1001,44 @@ struct OrderShared {
 /// key is only compared with the keys of its own bucket: few when the indices are spread evenly, as they are in
 /// inputs without any order. Loops over the units are kept rolled: this kernel is small work, it should be small
 /// code.
-__global__ __launch_bounds__(ORDER_BLOCK) void ordered_sort_kernel(OrderedArgs args, GridParams g) {
+template <bool BATCH = false>
+__global__ __launch_bounds__(ORDER_BLOCK) void ordered_sort_kernel(OrderedArgs args, GridParams single_grid) {
     __shared__ OrderShared shared;
     const int lane = lane_id();
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     OrderWaveShared& sh = shared.wave[wave];
-    const uint32_t n_tiles = static_cast<uint32_t>(args.cell_scan[g.n_cells] >> 32);
+    const uint32_t all_cells = BATCH ? args.total_cells : single_grid.n_cells;
+    const uint32_t n_tiles = static_cast<uint32_t>(args.cell_scan[all_cells] >> 32);
     const uint32_t tile_id = blockIdx.x * ORDER_WAVES + wave;
     if (tile_id >= n_tiles) {
         return;
     }
     const SortedPoints& sorted = args.sorted;
     const Tile tile = args.tiles[tile_id];
-    const int32_t cx = tile.cell % g.n[0];
-    const int32_t cy = (tile.cell / g.n[0]) % g.n[1];
-    const int32_t cz = tile.cell / (g.n[0] * g.n[1]);
+    // the grid: the kernel's argument, or this tile's system's (indices count from the first point of the system)
+    GridParams batch_grid;
+    uint32_t first_cell = 0;
+    if (BATCH) {
+        const uint32_t system = tile_system(tile);
+        batch_grid = args.grids[system];
+        first_cell = args.cell_base[system];
+        if (images_cover(batch_grid)) {
+            return;
+        }
+    }
+    const GridParams& g = BATCH ? batch_grid : single_grid;
+    const uint64_t* __restrict__ cell_scan = args.cell_scan + first_cell;
+    const uint32_t local_cell = tile.cell - first_cell;
+    const int32_t cx = local_cell % g.n[0];
+    const int32_t cy = (local_cell / g.n[0]) % g.n[1];
+    const int32_t cz = local_cell / (g.n[0] * g.n[1]);
     const int32_t span_y = 2 * g.s[1] + 1;
     const int32_t span_z = 2 * g.s[2] + 1;
     const uint32_t n_stencil = static_cast<uint32_t>(2 * g.s[0] + 1) * span_y * span_z;
     if (n_stencil > MAX_ENTRIES) {
         return;
     }
-    fill_stencil_tables(sh, lane, 0, n_stencil, cx, cy, cz, span_y, span_z, g, args.cell_scan);
+    fill_stencil_tables(sh, lane, 0, n_stencil, cx, cy, cz, span_y, span_z, g, cell_scan);
     const uint32_t n_candidates = __builtin_amdgcn_readfirstlane(sh.n_candidates);
     if (n_candidates > ORDERED_CANDIDATES || n_candidates == 0) {
         return; // the writing pass is not launched when a tile has too many
