@@ -42,12 +42,12 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes moved by ONE launch of the single-pass search kernel on the 1M-atom workload, from rocprofv3 --pmc
-# FETCH_SIZE and WRITE_SIZE runs scaled by a device copy of known size (167.2 MB fetched + 3238.4 MB written). The figure belongs to the kernel sources whose
+# FETCH_SIZE and WRITE_SIZE runs scaled by a device copy of known size (167.0 MB fetched + 3237.9 MB written). The figure belongs to the kernel sources whose
 # digest is recorded with it: a run with other sources reports no traffic instead of a stale one.
 SEARCH_KERNEL_TRAFFIC = {
-    "bytes": 3_405_600_000,
+    "bytes": 3_404_900_000,
     "profile": "profiles/fused_search_config1_pmc.txt",
-    "kernel_sources_sha256": "5a91f5894ff6ee4aa542af534d2da79f4257238e2c10cd1c2fb4a8d7fa1b0e64",
+    "kernel_sources_sha256": "0da55921174e4e78358fe4991ea0180628294e20c7e33acf6337242888cd6b6d",
 }
 KERNEL_SOURCES = ["device_common.cuh", "geometry.hpp", "cells.cuh", "search.cuh", "fused.cuh"]
 

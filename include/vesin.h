@@ -202,7 +202,14 @@ int VESIN_API vesin_hip_neighbors_collect(struct VesinNeighborList* neighbors, c
  * sparse or very uneven systems may not). A system beyond these limits, a non-zero `skin`, or a list of more than
  * `capacity` rows fail with EXIT_FAILURE and a message saying which; when the rows did not fit, *length receives
  * the number of rows the list has, so that the caller can come back with larger arrays. Calls on one GPU share the
- * work memory: they take turns (a lock is held for the whole call), whatever their streams. */
+ * work memory: they take turns (a lock is held for the whole call), whatever their streams.
+ *
+ * The first call on a GPU is set-up: it asks the HIP runtime for the address of the work array on that GPU
+ * (hipGetSymbolAddress) and launches every kernel for the first time, and the runtime loads the library's code on
+ * that GPU then, which it may allocate memory for. Make one call per GPU where allocating is still allowed (outside
+ * of a graph capture, before the loop starts); from the second call on nothing is allocated or freed: the library's
+ * own state per GPU is static data, what the kernels report comes to the host in copies of a few hundred bytes, and
+ * the device memory in use before and after a series of calls is the same (tests/test_zz_no_alloc.py). */
 int VESIN_API vesin_hip_neighbors_no_alloc(
     const double (*points)[3],
     size_t n_points,

@@ -3,6 +3,8 @@
 * ``tests/abi_caller.c`` includes ``vesin.h`` and links ``-lvesin`` like any C user of vesin. It is compiled and
   linked on every machine (CPU test) and run on the GPU (``-m gpu``): the cases of the reference's GPU test program
   (vesin/tests/cuda.cpp:22-226), with exact ``==`` on distances and vectors and ten host threads at once.
+* ``tests/call_loop.c`` calls ``vesin_neighbors`` a few thousand times on one small system, like a simulation code
+  without any wrapper, and prints the time per call; the test checks the number of rows against the oracle.
 * The reference's ``vesin-torch/src/vesin_torch.cpp`` is compiled UNMODIFIED against this repository's header and
   linked to this repository's library (``oracle/Makefile``, target ``ref_torch``; output in ``oracle/_ref/``, which
   is not part of the repository's history). The CPU test does that where the reference checkout exists; the GPU test
@@ -25,11 +27,11 @@ LIB_DIR = os.path.join(ROOT, "vesin_amd", "lib")
 REFERENCE = "/root/reference"
 
 
-def build_c_caller(directory):
-    out = os.path.join(str(directory), "abi_caller")
+def build_c_caller(directory, name="abi_caller"):
+    out = os.path.join(str(directory), name)
     command = [
         "gcc", "-std=c11", "-Wall", "-Wextra", "-Werror", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include",
-        "-I" + os.path.join(ROOT, "include"), os.path.join(HERE, "abi_caller.c"), "-o", out,
+        "-I" + os.path.join(ROOT, "include"), os.path.join(HERE, name + ".c"), "-o", out,
         "-L" + LIB_DIR, "-lvesin", "-L/opt/rocm/lib", "-lamdhip64", "-lpthread", "-lm",
         "-Wl,-rpath," + LIB_DIR, "-Wl,-rpath,/opt/rocm/lib",
     ]
@@ -50,6 +52,42 @@ def test_c_caller_runs(tmp_path):
     result = subprocess.run([program], capture_output=True, text=True, timeout=100)
     assert result.returncode == 0, result.stdout + result.stderr
     assert result.stdout.strip() == "ok"
+
+
+def test_call_loop_compiles_and_links(tmp_path):
+    build_c_caller(tmp_path, "call_loop")
+
+
+def _call_loop_system(cells):
+    """The atoms tests/call_loop.c makes: diamond with the jitter of its linear congruential generator."""
+    import numpy as np
+
+    a = 3.567
+    basis = np.array([[0, 0, 0], [0, .5, .5], [.5, 0, .5], [.5, .5, 0], [.25, .25, .25], [.25, .75, .75], [.75, .25, .75],
+                      [.75, .75, .25]])
+    points = []
+    state = 12345
+    for x in range(cells):
+        for y in range(cells):
+            for z in range(cells):
+                for b in range(8):
+                    point = []
+                    for d, corner in enumerate((x, y, z)):
+                        state = (state * 1664525 + 1013904223) % 2**32
+                        point.append((corner + basis[b][d]) * a + 0.05 * ((state >> 8) / 16777216.0 - 0.5))
+                    points.append(point)
+    return np.array(points), np.eye(3) * cells * a
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("cells, sorted_rows", [(3, 1), (3, 0), (2, 0), (5, 1)])
+def test_call_loop_runs(tmp_path, cells, sorted_rows):
+    program = build_c_caller(tmp_path, "call_loop")
+    result = subprocess.run([program, str(cells), str(sorted_rows), "300"], capture_output=True, text=True, timeout=100)
+    assert result.returncode == 0, result.stdout + result.stderr
+    points, box = _call_loop_system(cells)
+    expected = oracle.neighbors(points, box, [True, True, True], 5.0, True, False, "ij")
+    assert f"{len(points)} atoms, sorted {sorted_rows}: {len(expected['pairs'])} rows, " in result.stdout, result.stdout
 
 
 @pytest.mark.skipif(not os.path.isdir(os.path.join(REFERENCE, "vesin-torch", "src")), reason="needs the reference checkout")
