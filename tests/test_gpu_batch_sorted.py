@@ -237,3 +237,40 @@ def test_a_dense_system_among_the_others(capfd, monkeypatch):
     assert len(lines) == 1 and lines[0].endswith(": left to the radix sort"), lines
     _call_and_check(calculator, systems, cutoff, True, "PSd", "the call after")
     assert not _in_order_lines(capfd)
+
+
+@pytest.mark.parametrize("full", [True, False], ids=["full", "half"])
+def test_pairs_next_to_the_cutoff_in_systems_of_one_cell(full, capfd, monkeypatch):
+    """The counting pass over images decides most pairs in single precision, from where the points are once they are
+    moved into the box; pairs within rounding of the cutoff must come out as the reference's own arithmetic has them.
+    Every system holds 60 pairs whose distance is the cutoff to within a few units in the last place, across the box's
+    faces and with points up to three boxes outside; the same with every pair tested in double precision."""
+    rng = np.random.default_rng(577)
+    cutoff = 4.0
+    systems = []
+    n_close = 0
+    for s in range(24):
+        edge = rng.uniform(4.4, 7.5)
+        box = np.eye(3) * edge + (0.3 * rng.normal(size=(3, 3)) if s % 2 else 0.0)
+        first = rng.random((60, 3)) @ box
+        direction = rng.normal(size=first.shape)
+        direction /= np.linalg.norm(direction, axis=1)[:, None]
+        steps = rng.integers(-6, 7, size=len(first)).astype(np.float64)
+        second = first + direction * (cutoff * (1.0 + steps * 2.0**-52))[:, None]
+        points = np.concatenate([first, second])
+        if s % 3 == 0:
+            points = points + rng.integers(-3, 4, size=points.shape) @ box
+        systems.append((points, box, (True, True, True)))
+        expected = oracle.neighbors(points, box, [True] * 3, cutoff, True, False, "ijd")
+        n_close += int((np.abs(expected["distances"] - cutoff) < 1e-12).sum()) // 2
+    assert 300 < n_close < 24 * 60  # about half of the pairs made for it are in, and crowd the cutoff
+    for tests in ("single precision first", "double"):
+        if tests == "double":
+            monkeypatch.setenv("VESIN_HIP_TESTS", "double")
+        monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+        calculator = NeighborList(cutoff=cutoff, full_list=full, sorted=True)
+        capfd.readouterr()
+        for call in ("first call", "second call"):
+            _call_and_check(calculator, systems, cutoff, full, "PSdD", f"{tests}, {call}")
+            lines = _in_order_lines(capfd)
+            assert len(lines) == 1 and lines[0].endswith(": used"), (tests, call, lines)

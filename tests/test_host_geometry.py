@@ -492,6 +492,58 @@ def test_single_precision_pre_test_never_decides_a_pair_it_should_not(probe, see
     assert 0.0 < worst <= 0.5, worst
 
 
+@pytest.mark.parametrize("seed", range(4))
+def test_pre_test_of_systems_of_one_cell_stays_within_its_bound(probe, seed):
+    """Sorted batches search systems of one cell over their images, and decide a pair in single precision from where
+    the two points are after they were moved into the box, seen from a point inside the box (each rounded once), and
+    the shift of the image (rounded once): d2_32 = |(u_j - u_i) + q . H|^2 with the squares added by fused
+    multiply-adds. The same in numpy's float32 for pairs at the cutoff to within a part in a million, across up to two
+    boxes, against double (extended) precision: no pair is decided the wrong way and the error stays within half of
+    what the thresholds allow."""
+    rng = np.random.default_rng(200 + seed)
+    worst = 0.0
+    cases = 0
+    for case in range(60):
+        cutoff = float(rng.uniform(1.0, 9.0))
+        if case % 2 == 0:
+            box = np.diag(rng.uniform(0.52, 2.5, size=3) * cutoff)
+        else:
+            box = np.eye(3) * rng.uniform(0.6, 2.0) * cutoff + 0.15 * cutoff * rng.normal(size=(3, 3))
+        use32, lo32, hi32, edges, n, s = run_prefilter(probe, box, [1, 1, 1], cutoff, 64, [0] * 3, [0] * 3, single_cell=True)
+        if np.prod(2 * s + 1) > 128:
+            continue  # (more images than that search keeps)
+        assert use32 and np.all(n == 1), (box, cutoff)
+        cases += 1
+        allowed = (float(hi32) - float(lo32)) / 2.0
+        m = 20000
+        wide = np.longdouble
+        seen_from = rng.random(3) @ box
+        inside_i = rng.random((m, 3)) @ box
+        length = cutoff * (1.0 + rng.uniform(-1e-6, 1e-6, size=m))
+        direction = rng.normal(size=(m, 3))
+        direction /= np.linalg.norm(direction, axis=1)[:, None]
+        target = inside_i + direction * length[:, None]
+        q = np.floor(target @ np.linalg.inv(box))          # the image of j that is meant
+        inside_j = target - q @ box
+        reachable = np.all(np.abs(q) <= s, axis=1)
+        inside_i, inside_j, q = inside_i[reachable], inside_j[reachable], q[reachable]
+        exact = (inside_j.astype(wide) - inside_i.astype(wide)) + q.astype(wide) @ box.astype(wide)
+        d2 = np.sum(exact * exact, axis=1).astype(np.float64)
+        u_i = (inside_i - seen_from).astype(np.float32)
+        u_j = (inside_j - seen_from).astype(np.float32)
+        shift = (q @ box).astype(np.float32)
+        v = ((u_j - u_i).astype(np.float32) + shift).astype(np.float32)
+        v64 = v.astype(np.float64)
+        xx = (v64[:, 0] * v64[:, 0]).astype(np.float32)                                   # vx * vx
+        xy = (v64[:, 1] * v64[:, 1] + xx.astype(np.float64)).astype(np.float32)           # fma(vy, vy, .)
+        d2_32 = (v64[:, 2] * v64[:, 2] + xy.astype(np.float64)).astype(np.float32)        # fma(vz, vz, .)
+        inside_cutoff = d2 < cutoff * cutoff
+        assert not np.any(inside_cutoff & (d2_32 > hi32)), (box, cutoff)
+        assert not np.any(~inside_cutoff & (d2_32 < lo32)), (box, cutoff)
+        worst = max(worst, float(np.max(np.abs(d2_32.astype(np.float64) - d2)) / allowed))
+    assert cases >= 20 and 0.0 < worst <= 0.5, (cases, worst)
+
+
 def test_pre_test_is_switched_off_where_its_bound_is_no_use(probe):
     # one cell much wider than the cutoff: the margin would be a sizeable part of the squared cutoff
     use32, *_ = run_prefilter(probe, np.eye(3), [0, 0, 0], 1e-3, 100, [0] * 3, [5000.0] * 3, single_cell=True)

@@ -3072,6 +3072,8 @@ bool batch_attempt(
         iargs.pair_base = d_pair_base;
         iargs.hits = image_hits;
         iargs.words = setup.image_words;
+        iargs.cutoff = options.cutoff;
+        iargs.double_only = double_precision_only() ? 1u : 0u;
         iargs.n_systems = static_cast<uint32_t>(n_systems);
         iargs.total_points = static_cast<uint32_t>(n_points);
         iargs.others_covered = in_order_tiles ? 1u : 0u;

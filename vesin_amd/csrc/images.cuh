@@ -59,6 +59,8 @@ struct ImageArgs {
     const uint64_t* pair_base;  // pairs of points (n^2 per system of at most IMAGE_MAX_POINTS points) before every system
     uint64_t* hits;             // COUNT -> WRITE: [pair_base + i * n + j][words]: the images of j that are neighbours of i
     uint32_t words;             // words of 64 images per pair (1 or 2), the same for every system of the batch
+    double cutoff;              // COUNT: for the thresholds of the single-precision pre-test (choose_prefilter)
+    uint32_t double_only;       // COUNT: not zero: every pair is tested in double precision (for tests)
     uint32_t n_systems;
     uint32_t total_points;
     uint32_t* rows_of_point;    // COUNT: [total_points], by first point of the system + index
@@ -85,6 +87,14 @@ struct ImageShared {
 struct ImageCountShared: ImageShared {
     uint64_t with_itself[IMAGE_MAX_WORDS]; // the images of a point that may be its own neighbours
     uint32_t rows[IMAGE_MAX_POINTS];       // rows of every point
+    // The single-precision pre-test (choose_prefilter, geometry.hpp), in the form it takes for one cell: where the
+    // points are after they were moved into the box, seen from one of them (r - w . H - the same of the first point:
+    // within the extent of the box along every axis, or not a number), and the shifts of the images, rounded once.
+    // v = (r_j - r_i) + (q - w_j + w_i) . H = (u_j - u_i) + q . H whatever the wraps are.
+    float ux[IMAGE_MAX_POINTS], uy[IMAGE_MAX_POINTS], uz[IMAGE_MAX_POINTS];
+    float sx[IMAGE_MAX_ENTRIES], sy[IMAGE_MAX_ENTRIES], sz[IMAGE_MAX_ENTRIES];
+    uint32_t use32;
+    float lo32, hi32;
 };
 
 struct ImageWriteShared: ImageShared {
@@ -105,6 +115,31 @@ __device__ __forceinline__ void stage_system(
     const int32_t wx0 = args.sorted.wx[at0];
     const int32_t wy0 = args.sorted.wy[at0];
     const int32_t wz0 = args.sorted.wz[at0];
+    // COUNT: the first point after it was moved into the box, which the others are seen from, and how far from it a
+    // point inside the box can be along every axis (twice that is the bound the thresholds were derived for)
+    double seen_from[3] = {0.0, 0.0, 0.0};
+    double reach[3] = {0.0, 0.0, 0.0};
+    if constexpr (COUNT) {
+        if (threadIdx.x == 0) {
+            Prefilter pre;
+            choose_prefilter(g, args.cutoff, pre);
+            sh.use32 = static_cast<uint32_t>(pre.use32);
+            sh.lo32 = pre.lo32;
+            sh.hi32 = pre.hi32;
+        }
+        const SortedPoint first_point = args.sorted.p[at0];
+        double mx, my, mz;
+        shift_vector(g, wx0, wy0, wz0, mx, my, mz);
+        seen_from[0] = first_point.x - mx;
+        seen_from[1] = first_point.y - my;
+        seen_from[2] = first_point.z - mz;
+        for (int d = 0; d < 3; d++) {
+            const double scale = g.periodic[d] != 0 ? 1.0 : 1.0 / g.np_scale[d];
+            for (int k = 0; k < 3; k++) {
+                reach[k] += 2.0 * fabs(g.H[3 * d + k]) * scale;
+            }
+        }
+    }
     for (uint32_t p = threadIdx.x; p < n; p += IMAGE_BLOCK) {
         const SortedPoint point = args.sorted.p[at0 + p];
         const uint32_t index = min(point.index, IMAGE_MAX_POINTS - 1);
@@ -122,6 +157,16 @@ __device__ __forceinline__ void stage_system(
         }
         if constexpr (COUNT) {
             sh.rows[index] = 0;
+            double mx, my, mz;
+            shift_vector(g, wx, wy, wz, mx, my, mz);
+            const double rx = (point.x - mx) - seen_from[0];
+            const double ry = (point.y - my) - seen_from[1];
+            const double rz = (point.z - mz) - seen_from[2];
+            const bool usable = !beyond(wx, wy, wz, LOCAL_WRAP_LIMIT) && fabs(rx) <= reach[0] && fabs(ry) <= reach[1] &&
+                                fabs(rz) <= reach[2];
+            sh.ux[index] = usable ? static_cast<float>(rx) : __builtin_nanf("");
+            sh.uy[index] = usable ? static_cast<float>(ry) : __builtin_nanf("");
+            sh.uz[index] = usable ? static_cast<float>(rz) : __builtin_nanf("");
         }
     }
     if (wave == 0) {
@@ -147,6 +192,11 @@ __device__ __forceinline__ void stage_system(
                 sh.tx[slot] = tx;
                 sh.ty[slot] = ty;
                 sh.tz[slot] = tz;
+                if constexpr (COUNT) {
+                    sh.sx[slot] = static_cast<float>(tx);
+                    sh.sy[slot] = static_cast<float>(ty);
+                    sh.sz[slot] = static_cast<float>(tz);
+                }
             }
             kept += __popcll(mask);
         }
@@ -213,6 +263,9 @@ __global__ __launch_bounds__(IMAGE_BLOCK) void image_count_kernel(ImageArgs args
     }
     stage_system<true, FULL>(sh, args, g, system, wave, lane);
     const uint32_t n_entries = uniform(sh.n_entries);
+    const bool use32 = uniform(sh.use32) != 0 && args.double_only == 0;
+    const float lo32 = sh.lo32;
+    const float hi32 = sh.hi32;
     const uint32_t first = args.first_point[system];
     const uint32_t words = args.words;
     uint64_t* system_hits = args.hits + args.pair_base[system] * words;
@@ -249,44 +302,109 @@ __global__ __launch_bounds__(IMAGE_BLOCK) void image_count_kernel(ImageArgs args
         }
         // (a word of 64 images in two halves: the bits of a half are gathered in one register)
         uint32_t found[2 * IMAGE_MAX_WORDS][IMAGE_GROUP];
-#pragma unroll
-        for (int h = 0; h < 2 * static_cast<int>(IMAGE_MAX_WORDS); h++) {
+        if (use32) {
+            // ---- single precision first: a squared distance below lo32 is within the cutoff, one above hi32 is not
+            // (choose_prefilter); what lies in between, and every image of a pair with a point that has no place, is
+            // decided below by the reference's own arithmetic
+            float fx[IMAGE_GROUP], fy[IMAGE_GROUP], fz[IMAGE_GROUP];
+            uint32_t maybe[2 * IMAGE_MAX_WORDS][IMAGE_GROUP];
 #pragma unroll
             for (int u = 0; u < IMAGE_GROUP; u++) {
-                found[h][u] = 0;
+                fx[u] = sh.ux[pj[u]] - sh.ux[pi[u]];
+                fy[u] = sh.uy[pj[u]] - sh.uy[pi[u]];
+                fz[u] = sh.uz[pj[u]] - sh.uz[pi[u]];
             }
-            const uint32_t e_begin = h * 32;
-            const uint32_t e_end = min(n_entries, e_begin + 32);
-            if (moved_alike) {
-                // the shift of the row is the cell shift of the image: the same vector for every lane
+#pragma unroll
+            for (int h = 0; h < 2 * static_cast<int>(IMAGE_MAX_WORDS); h++) {
+#pragma unroll
+                for (int u = 0; u < IMAGE_GROUP; u++) {
+                    found[h][u] = 0;
+                    maybe[h][u] = 0;
+                }
+                const uint32_t e_begin = h * 32;
+                const uint32_t e_end = min(n_entries, e_begin + 32);
                 for (uint32_t e = e_begin; e < e_end; e++) {
-                    const double tx = sh.tx[e];
-                    const double ty = sh.ty[e];
-                    const double tz = sh.tz[e];
+                    const float tx = sh.sx[e];
+                    const float ty = sh.sy[e];
+                    const float tz = sh.sz[e];
                     const uint32_t bit = 1u << (e % 32);
 #pragma unroll
                     for (int u = 0; u < IMAGE_GROUP; u++) {
-                        const double vx = ax[u] + tx;
-                        const double vy = ay[u] + ty;
-                        const double vz = az[u] + tz;
-                        const double d2 = vx * vx + vy * vy + vz * vz;
-                        found[h][u] |= d2 < g.cutoff2 ? bit : 0u;
+                        const float vx = fx[u] + tx;
+                        const float vy = fy[u] + ty;
+                        const float vz = fz[u] + tz;
+                        const float d2 = __builtin_fmaf(vz, vz, __builtin_fmaf(vy, vy, vx * vx));
+                        found[h][u] |= d2 < lo32 ? bit : 0u;
+                        maybe[h][u] |= d2 < hi32 ? bit : 0u;
                     }
                 }
-            } else {
-                for (uint32_t e = e_begin; e < e_end; e++) {
-                    int32_t qx, qy, qz;
-                    unpack_shift(sh.q[e], qx, qy, qz);
-                    const uint32_t bit = 1u << (e % 32);
+            }
 #pragma unroll
-                    for (int u = 0; u < IMAGE_GROUP; u++) {
-                        double tx, ty, tz;
-                        shift_vector(g, qx + bx[u], qy + by[u], qz + bz[u], tx, ty, tz);
-                        const double vx = ax[u] + tx;
-                        const double vy = ay[u] + ty;
-                        const double vz = az[u] + tz;
-                        const double d2 = vx * vx + vy * vy + vz * vz;
-                        found[h][u] |= d2 < g.cutoff2 ? bit : 0u;
+            for (int u = 0; u < IMAGE_GROUP; u++) {
+                const bool unknown = !(fx[u] == fx[u]) || !(fy[u] == fy[u]) || !(fz[u] == fz[u]);
+#pragma unroll
+                for (int h = 0; h < 2 * static_cast<int>(IMAGE_MAX_WORDS); h++) {
+                    const uint32_t in_table = n_entries >= (h + 1) * 32u ? ~0u : n_entries > h * 32u ? (1u << (n_entries - h * 32u)) - 1u : 0u;
+                    uint32_t open = unknown ? in_table : (maybe[h][u] & ~found[h][u]);
+                    uint32_t decided = unknown ? 0u : found[h][u];
+                    while (__ballot(open != 0) != 0) {
+                        if (open != 0) {
+                            const uint32_t at_bit = static_cast<uint32_t>(__builtin_ctz(open));
+                            open &= open - 1;
+                            int32_t qx, qy, qz;
+                            unpack_shift(sh.q[h * 32 + at_bit], qx, qy, qz);
+                            double tx, ty, tz;
+                            shift_vector(g, qx + bx[u], qy + by[u], qz + bz[u], tx, ty, tz);
+                            const double vx = ax[u] + tx;
+                            const double vy = ay[u] + ty;
+                            const double vz = az[u] + tz;
+                            const double d2 = vx * vx + vy * vy + vz * vz;
+                            decided = d2 < g.cutoff2 ? decided | (1u << at_bit) : decided & ~(1u << at_bit);
+                        }
+                    }
+                    found[h][u] = decided;
+                }
+            }
+        } else {
+        #pragma unroll
+            for (int h = 0; h < 2 * static_cast<int>(IMAGE_MAX_WORDS); h++) {
+    #pragma unroll
+                for (int u = 0; u < IMAGE_GROUP; u++) {
+                    found[h][u] = 0;
+                }
+                const uint32_t e_begin = h * 32;
+                const uint32_t e_end = min(n_entries, e_begin + 32);
+                if (moved_alike) {
+                    // the shift of the row is the cell shift of the image: the same vector for every lane
+                    for (uint32_t e = e_begin; e < e_end; e++) {
+                        const double tx = sh.tx[e];
+                        const double ty = sh.ty[e];
+                        const double tz = sh.tz[e];
+                        const uint32_t bit = 1u << (e % 32);
+    #pragma unroll
+                        for (int u = 0; u < IMAGE_GROUP; u++) {
+                            const double vx = ax[u] + tx;
+                            const double vy = ay[u] + ty;
+                            const double vz = az[u] + tz;
+                            const double d2 = vx * vx + vy * vy + vz * vz;
+                            found[h][u] |= d2 < g.cutoff2 ? bit : 0u;
+                        }
+                    }
+                } else {
+                    for (uint32_t e = e_begin; e < e_end; e++) {
+                        int32_t qx, qy, qz;
+                        unpack_shift(sh.q[e], qx, qy, qz);
+                        const uint32_t bit = 1u << (e % 32);
+    #pragma unroll
+                        for (int u = 0; u < IMAGE_GROUP; u++) {
+                            double tx, ty, tz;
+                            shift_vector(g, qx + bx[u], qy + by[u], qz + bz[u], tx, ty, tz);
+                            const double vx = ax[u] + tx;
+                            const double vy = ay[u] + ty;
+                            const double vz = az[u] + tz;
+                            const double d2 = vx * vx + vy * vy + vz * vz;
+                            found[h][u] |= d2 < g.cutoff2 ? bit : 0u;
+                        }
                     }
                 }
             }
