@@ -123,3 +123,53 @@ def test_random_batches():
             rows = slice(int(first_pair[s]), int(first_pair[s + 1]))
             expected = oracle.neighbors(all_points[s], all_boxes[s], True, cutoff, full, False, "ijSdD")
             assert_same_list({k: v[rows] for k, v in whole.items()}, expected, what=f"trial {trial} system {s}")
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_random_batches_on_one_reused_list(seed):
+    """Batches of random systems, each with its own periodicity, sorted or not, on one reused list: a batch is
+    followed for a few small moves (the set-up kept from the call before, boxes compared on the device, grids of open
+    systems picked on the device, the searches that write sorted rows in order and their fallbacks) before another
+    replaces it. Sorted rows are compared in place with the oracle's rows in (i, j, shift) order."""
+    import torch
+
+    rng = np.random.default_rng(90_000 + seed)
+    cutoff = float(rng.choice([1.5, 2.5, 3.7]))
+    full = bool(rng.integers(0, 2))
+    is_sorted = bool(rng.integers(0, 4) > 0)
+    all_open = seed % 4 == 3
+    calculator = NeighborList(cutoff=cutoff, full_list=full, sorted=is_sorted)
+    systems = None
+    for step in range(7):
+        if systems is None or rng.random() < 0.35:
+            systems = []
+            for _ in range(int(rng.integers(1, 10))):
+                points, box, periodic = random_system(rng, larger=seed % 8 == 5 and rng.random() < 0.2)
+                if all_open:
+                    periodic = [False, False, False]
+                systems.append([points, box, periodic])
+        else:
+            for system in systems:
+                system[0] = system[0] + rng.normal(scale=rng.choice([0.01, 0.1, 0.5]), size=system[0].shape)
+        first_point = np.cumsum([0] + [len(s[0]) for s in systems])
+        outputs, first_pair = calculator.compute_batch(
+            torch.as_tensor(np.concatenate([s[0] for s in systems]).reshape(-1, 3), device="cuda:0"),
+            first_point,
+            torch.as_tensor(np.stack([s[1] for s in systems]), device="cuda:0"),
+            np.array([s[2] for s in systems], dtype=bool),
+            "PSdD",
+        )
+        whole = {NAMES[q]: t.cpu().numpy() for q, t in zip("PSdD", outputs)}
+        assert first_pair[0] == 0 and first_pair[-1] == len(whole["pairs"])
+        for k, (points, box, periodic) in enumerate(systems):
+            rows = slice(int(first_pair[k]), int(first_pair[k + 1]))
+            expected = oracle.neighbors(points, box, periodic, cutoff, full, False, "ijSdD")
+            actual = {key: value[rows] for key, value in whole.items()}
+            what = f"seed {seed} step {step} system {k} n={len(points)} sorted={is_sorted} periodic={periodic}"
+            if is_sorted:
+                in_order = oracle.canonicalize(expected)
+                assert actual["pairs"].shape == in_order["pairs"].shape, what
+                for key in actual:
+                    assert np.array_equal(actual[key], in_order[key]), (what, key)
+            else:
+                assert_same_list(actual, expected, what=what)

@@ -40,8 +40,8 @@ constexpr uint32_t IMAGE_MAX_WORDS = IMAGE_MAX_ENTRIES / 64;
 constexpr int IMAGE_WAVES = 4;
 constexpr int IMAGE_BLOCK = IMAGE_WAVES * WAVE;
 constexpr int IMAGE_GROUP = 2;             // units of 64 pairs of points a wave tests together
-constexpr uint32_t IMAGE_ROWS = 16 * WAVE; // rows of a first point that a wave lines up in LDS at a time
-static_assert(IMAGE_MAX_POINTS <= 256 && IMAGE_MAX_ENTRIES <= 256, "a row is lined up as (second point << 8) | image in 16 bits");
+constexpr uint32_t IMAGE_ROWS = 8 * WAVE;  // rows that a wave lines up in LDS at a time (and up to 63 left over)
+static_assert(IMAGE_MAX_POINTS <= 256 && IMAGE_MAX_ENTRIES <= 256, "a row is lined up as (first point << 16) | (second point << 8) | image");
 
 /// Words of 64 images that a pair of points of this system keeps (an upper bound: before the stencil is pruned).
 __host__ __device__ inline uint32_t image_words(const GridParams& g) {
@@ -98,7 +98,9 @@ struct ImageCountShared: ImageShared {
 };
 
 struct ImageWriteShared: ImageShared {
-    uint16_t rows[IMAGE_WAVES][IMAGE_ROWS]; // (second point << 8) | image, at the place of the row
+    // (first point << 16) | (second point << 8) | image, at the place of the row: what a run of consecutive rows left
+    // short of a multiple of 64, and the rows of the points behind it
+    uint32_t rows[IMAGE_WAVES][IMAGE_ROWS + WAVE];
 };
 
 /// The system's points by index, and the images that can hold a neighbour in the order of their cell shift.
@@ -450,7 +452,54 @@ __global__ __launch_bounds__(IMAGE_BLOCK) void image_count_kernel(ImageArgs args
     }
 }
 
-/// WRITE: one workgroup per system, a first point per wave at a time.
+/// Stores the first `count` rows lined up in `rows` as the rows `first_row` ... of the list: 64 consecutive rows per
+/// step, each step ending on a multiple of 64 rows (whole cache lines in every output array; the first step stores
+/// fewer).
+__device__ __forceinline__ void store_image_rows(
+    const ImageWriteShared& sh, const uint32_t* rows, const GridParams& g, const SearchOutputs& out, bool moved_apart,
+    uint32_t count, uint64_t first_row, int lane
+) {
+    const uint32_t skew = static_cast<uint32_t>(first_row % WAVE);
+    for (uint32_t r0 = 0; r0 < count + skew; r0 += WAVE) {
+        const uint32_t r = r0 + lane - skew;
+        if (r >= count) {
+            continue; // (before the first row as well: unsigned)
+        }
+        const uint32_t ticket = rows[r];
+        const uint32_t i = ticket >> 16;
+        const uint32_t j = (ticket >> 8) & 0xffu;
+        const uint32_t e = ticket & 0xffu;
+        int32_t sx, sy, sz;
+        unpack_shift(sh.q[e], sx, sy, sz);
+        double tx = sh.tx[e];
+        double ty = sh.ty[e];
+        double tz = sh.tz[e];
+        if (moved_apart) {
+            sx += sh.wx[i] - sh.wx[j];
+            sy += sh.wy[i] - sh.wy[j];
+            sz += sh.wz[i] - sh.wz[j];
+            shift_vector(g, sx, sy, sz, tx, ty, tz);
+        }
+        const double vx = (sh.x[j] - sh.x[i]) + tx;
+        const double vy = (sh.y[j] - sh.y[i]) + ty;
+        const double vz = (sh.z[j] - sh.z[i]) + tz;
+        const uint64_t row = first_row + r;
+        stream_store(out.pairs + 2 * row, PairRow{i, j});
+        if (out.shifts != nullptr) {
+            stream_store(out.shifts + 3 * row, ShiftRow{sx, sy, sz});
+        }
+        if (out.distances != nullptr) {
+            stream_store(out.distances + row, sqrt(vx * vx + vy * vy + vz * vz));
+        }
+        if (out.vectors != nullptr) {
+            stream_store(out.vectors + 3 * row, VectorHead{vx, vy});
+            stream_store(out.vectors + 3 * row + 2, vz);
+        }
+    }
+}
+
+/// WRITE: one workgroup per system, every wave a run of consecutive first points: their rows are consecutive rows of
+/// the list, lined up in LDS one point after the other and stored whenever they reach a multiple of 64 rows.
 template <bool FULL>
 __global__ __launch_bounds__(IMAGE_BLOCK) void image_write_kernel(ImageArgs args) {
     __shared__ ImageWriteShared sh;
@@ -487,23 +536,30 @@ __global__ __launch_bounds__(IMAGE_BLOCK) void image_write_kernel(ImageArgs args
     const uint32_t first = args.first_point[system];
     const uint32_t words = args.words;
     const uint64_t* system_hits = args.hits + args.pair_base[system] * words;
-    uint16_t* rows = sh.rows[wave];
+    uint32_t* rows = sh.rows[wave];
     const SearchOutputs& out = args.out;
 
-    for (uint32_t i = wave; i < n; i += IMAGE_WAVES) {
-        const double xi = sh.x[i];
-        const double yi = sh.y[i];
-        const double zi = sh.z[i];
-        const int32_t wix = sh.wx[i];
-        const int32_t wiy = sh.wy[i];
-        const int32_t wiz = sh.wz[i];
-        const uint64_t first_row = args.first_row[first + i];
-        const uint32_t n_rows = static_cast<uint32_t>(args.first_row[first + i + 1] - first_row);
+    const uint32_t per_wave = (n + IMAGE_WAVES - 1) / IMAGE_WAVES;
+    const uint32_t i_begin = wave * per_wave;
+    const uint32_t i_end = min(n, i_begin + per_wave);
+    if (i_begin >= i_end) {
+        return;
+    }
+    uint64_t staged_row = uniform(args.first_row[first + i_begin]); // row of the list of the first row lined up
+    uint32_t staged = 0;                                            // rows lined up
+    uint64_t next_first = staged_row;
+    for (uint32_t i = i_begin; i < i_end; i++) {
+        const uint64_t first_row = next_first;
+        next_first = uniform(args.first_row[first + i + 1]);
+        const uint32_t n_rows = static_cast<uint32_t>(next_first - first_row);
         const uint64_t* hits_of_i = system_hits + static_cast<size_t>(i) * n * words;
-        // IMAGE_ROWS rows at a time (all of them at once, for all but the largest numbers of neighbours)
-        for (uint32_t window = 0; window < n_rows; window += IMAGE_ROWS) {
+        uint32_t done = 0; // rows of this point that are lined up or stored
+        while (done < n_rows) {
+            // as many rows of the point as there is room for (all of them, for all but the largest numbers of
+            // neighbours): the rows [done, done + take) go behind the rows that wait
+            const uint32_t take = min(IMAGE_ROWS + WAVE - staged, n_rows - done);
             uint32_t before = 0; // rows of the second points of earlier lanes
-            for (uint32_t j0 = 0; j0 < n && before < window + IMAGE_ROWS; j0 += WAVE) {
+            for (uint32_t j0 = 0; j0 < n && before < done + take; j0 += WAVE) {
                 const uint32_t j = j0 + lane;
                 // (a half list: the second points before i have no rows, and the counting pass left no words for them)
                 const bool there = j < n && (FULL || j >= i);
@@ -516,17 +572,18 @@ __global__ __launch_bounds__(IMAGE_BLOCK) void image_write_kernel(ImageArgs args
                 }
                 const uint32_t own = __popcll(lo) + __popcll(hi);
                 const uint32_t through = wave_inclusive_scan(own);
-                uint32_t place = before + through - own - window; // (places before the window: far beyond it, unsigned)
+                uint32_t place = before + through - own - done; // (rows before `done`: far beyond `take`, unsigned)
                 before += read_lane(through, WAVE - 1);
-                if (before <= window) {
-                    continue; // the rows of these second points were stored with an earlier window
+                if (before <= done) {
+                    continue; // the rows of these second points went out earlier
                 }
+                const uint32_t ticket = (i << 16) | (j << 8);
                 while (__ballot(lo != 0) != 0) {
                     if (lo != 0) {
                         const uint32_t e = static_cast<uint32_t>(__builtin_ctzll(lo));
                         lo &= lo - 1;
-                        if (place < IMAGE_ROWS) {
-                            rows[place] = static_cast<uint16_t>((j << 8) | e);
+                        if (place < take) {
+                            rows[staged + place] = ticket | e;
                         }
                         place += 1;
                     }
@@ -535,55 +592,35 @@ __global__ __launch_bounds__(IMAGE_BLOCK) void image_write_kernel(ImageArgs args
                     if (hi != 0) {
                         const uint32_t e = 64 + static_cast<uint32_t>(__builtin_ctzll(hi));
                         hi &= hi - 1;
-                        if (place < IMAGE_ROWS) {
-                            rows[place] = static_cast<uint16_t>((j << 8) | e);
+                        if (place < take) {
+                            rows[staged + place] = ticket | e;
                         }
                         place += 1;
                     }
                 }
             }
+            staged += take;
+            done += take;
             wave_sync();
-            const uint32_t n_here = min(IMAGE_ROWS, n_rows - window);
-            // 64 consecutive rows per step, from a multiple of 64 rows on (whole cache lines in every output array;
-            // the first step of a point stores fewer)
-            const uint32_t skew = static_cast<uint32_t>(first_row % WAVE);
-            for (uint32_t r0 = 0; r0 < n_here + skew; r0 += WAVE) {
-                const uint32_t r = r0 + lane - skew;
-                if (r >= n_here) {
-                    continue; // (before the point's first row as well: unsigned)
+            const uint64_t whole = (staged_row + staged) & ~static_cast<uint64_t>(WAVE - 1);
+            if (whole > staged_row) {
+                // everything up to the last multiple of 64 rows; what is left moves to the front
+                const uint32_t count = static_cast<uint32_t>(whole - staged_row);
+                store_image_rows(sh, rows, g, out, moved_apart, count, staged_row, lane);
+                const uint32_t left = staged - count; // < 64
+                const uint32_t ticket = rows[min(count + lane, IMAGE_ROWS + WAVE - 1)];
+                wave_sync();
+                if (static_cast<uint32_t>(lane) < left) {
+                    rows[lane] = ticket;
                 }
-                const uint32_t ticket = rows[r];
-                const uint32_t j = ticket >> 8;
-                const uint32_t e = ticket & 0xffu;
-                int32_t sx, sy, sz;
-                unpack_shift(sh.q[e], sx, sy, sz);
-                double tx = sh.tx[e];
-                double ty = sh.ty[e];
-                double tz = sh.tz[e];
-                if (moved_apart) {
-                    sx += wix - sh.wx[j];
-                    sy += wiy - sh.wy[j];
-                    sz += wiz - sh.wz[j];
-                    shift_vector(g, sx, sy, sz, tx, ty, tz);
-                }
-                const double vx = (sh.x[j] - xi) + tx;
-                const double vy = (sh.y[j] - yi) + ty;
-                const double vz = (sh.z[j] - zi) + tz;
-                const uint64_t row = first_row + window + r;
-                stream_store(out.pairs + 2 * row, PairRow{i, j});
-                if (out.shifts != nullptr) {
-                    stream_store(out.shifts + 3 * row, ShiftRow{sx, sy, sz});
-                }
-                if (out.distances != nullptr) {
-                    stream_store(out.distances + row, sqrt(vx * vx + vy * vy + vz * vz));
-                }
-                if (out.vectors != nullptr) {
-                    stream_store(out.vectors + 3 * row, VectorHead{vx, vy});
-                    stream_store(out.vectors + 3 * row + 2, vz);
-                }
+                staged_row = whole;
+                staged = left;
+                wave_sync();
             }
-            wave_sync();
         }
+    }
+    if (staged != 0) {
+        store_image_rows(sh, rows, g, out, moved_apart, staged, staged_row, lane);
     }
 }
 
