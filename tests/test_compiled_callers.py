@@ -88,6 +88,10 @@ def test_call_loop_runs(tmp_path, cells, sorted_rows):
     points, box = _call_loop_system(cells)
     expected = oracle.neighbors(points, box, [True, True, True], 5.0, True, False, "ij")
     assert f"{len(points)} atoms, sorted {sorted_rows}: {len(expected['pairs'])} rows, " in result.stdout, result.stdout
+    # the same as a queued call and its completion, the word on the device checked after every call
+    result = subprocess.run([program, str(cells), str(sorted_rows), "300", "queued"], capture_output=True, text=True, timeout=100)
+    assert result.returncode == 0, result.stdout + result.stderr
+    assert f"{len(expected['pairs'])} rows, queued: " in result.stdout, result.stdout
 
 
 @pytest.mark.skipif(not os.path.isdir(os.path.join(REFERENCE, "vesin-torch", "src")), reason="needs the reference checkout")
