@@ -339,3 +339,40 @@ def test_collect_on_another_host_thread_free_with_a_call_pending_and_no_points()
     lib.vesin_free(ctypes.byref(neighbors))
     assert neighbors.pairs is None and neighbors.opaque is None
     torch.cuda.synchronize()
+
+
+def test_the_python_caller_in_two_halves():
+    """NeighborList.enqueue / collect: the word on the device as a tensor that work on torch's current stream reads,
+    the rows of compute, a pending call refused, an error raised by collect."""
+    import torch
+
+    from vesin_amd import NeighborList
+
+    points, box, periodic, options = configs.config0()
+    inputs = _device(points, box, [bool(p) for p in np.broadcast_to(periodic, 3)])
+    expected = oracle.canonicalize(oracle.neighbors(points, box, periodic, options["cutoff"], True, False, "ijSd"))
+    calculator = NeighborList(cutoff=options["cutoff"], full_list=True, sorted=True)
+    counts = []
+    for call in range(3):
+        word = calculator.enqueue(*inputs, quantities="PSd")
+        seen = word.clone()  # queued on the same stream, no host synchronisation in between
+        with pytest.raises(RuntimeError, match="pending"):
+            calculator.enqueue(*inputs, quantities="PSd")
+        pairs, shifts, distances = calculator.collect()
+        counts.append(int(seen.item()))
+        assert np.array_equal(pairs.cpu().numpy(), expected["pairs"]), call
+        assert np.array_equal(shifts.cpu().numpy(), expected["shifts"]), call
+        assert np.array_equal(distances.cpu().numpy(), expected["distances"]), call
+        assert int(word.item()) == len(expected["pairs"])
+    # the list's first call cannot be queued whole, its later calls are
+    assert counts == [-1, len(expected["pairs"]), len(expected["pairs"])]
+    with pytest.raises(RuntimeError, match="no call pending"):
+        calculator.collect()
+    bad = inputs[0].clone()
+    bad[7, 1] = float("nan")
+    calculator.enqueue(bad, inputs[1], inputs[2], quantities="P")
+    with pytest.raises(RuntimeError, match="finite|NaN|nan"):
+        calculator.collect()
+    # and the calculator is as usable as before
+    (pairs,) = calculator.compute(inputs[0], inputs[1], periodic, "P")
+    assert np.array_equal(pairs.cpu().numpy(), expected["pairs"])

@@ -440,6 +440,93 @@ class NeighborList:
                 data.append(wrap(self._neighbors.vectors, (n_pairs, 3), "<f8", torch.float64))
         return tuple(data), first_pair
 
+    def enqueue(self, points, box, periodic, quantities: str = "ij"):
+        """``compute`` in two halves (``vesin_hip_neighbors_enqueue``): queues the calculation on torch's current
+        stream and returns without waiting for it, so that the caller can queue whatever consumes the list right
+        behind. Takes contiguous float64 torch tensors on the GPU (``points`` (N, 3), ``box`` (3, 3)) and a boolean
+        tensor of three flags on the GPU for ``periodic``; they must stay as they are until ``collect``.
+
+        Returns a one-element int64 tensor that views the word in GPU memory where work queued on the same stream
+        finds the number of rows, or -1 when the queued kernels did not leave the complete list (a list's first call,
+        another box, rows that outgrew the arrays): then nothing may be read before ``collect`` has returned.
+        """
+        import torch
+
+        for name, tensor in (("points", points), ("box", box), ("periodic", periodic)):
+            if not isinstance(tensor, torch.Tensor) or tensor.device.type != "cuda" or not tensor.is_contiguous():
+                raise RuntimeError(f"enqueue takes contiguous torch tensors on a cuda (HIP) device, `{name}` is not one")
+        if points.dtype != torch.float64 or box.dtype != torch.float64 or periodic.dtype != torch.bool:
+            raise RuntimeError("enqueue takes float64 `points` and `box` and boolean `periodic`")
+        if points.dim() != 2 or points.shape[1] != 3 or tuple(box.shape) != (3, 3) or tuple(periodic.shape) != (3,):
+            raise ValueError("`points` must be a nx3 array, `box` a 3x3 matrix, `periodic` three flags")
+        if self.__dict__.get("_queued") is not None:
+            raise RuntimeError("this calculator has a call pending: collect() it first")
+        device = points.device
+        index = device.index if device.index is not None else torch.cuda.current_device()
+        options = VesinOptions()
+        options.cutoff = self.cutoff
+        options.full = self.full_list
+        options.sorted = self.sorted
+        options.algorithm = self._c_algorithm
+        options.n_threads = self.n_threads
+        options.return_shifts = "S" in quantities
+        options.return_distances = "d" in quantities
+        options.return_vectors = "D" in quantities
+        options.skin = self.skin
+        word = ctypes.c_void_p()
+        error_message = ctypes.c_char_p()
+        status = self._lib.vesin_hip_neighbors_enqueue(
+            points.data_ptr() if points.shape[0] > 0 else box.data_ptr(), points.shape[0], box.data_ptr(),
+            periodic.data_ptr(), VesinDevice(VesinCUDA, index), options, ctypes.byref(self._neighbors),
+            torch.cuda.current_stream(device).cuda_stream, ctypes.byref(word), ctypes.byref(error_message),
+        )
+        if status != 0:
+            raise RuntimeError(error_message.value.decode("utf8"))
+        # (the inputs are referred to until the call is collected)
+        self._queued = (quantities, index, points, box, periodic)
+        return torch.as_tensor(_DeviceView(word.value, (1,), "<i8", self), device=f"cuda:{index}")
+
+    def collect(self, copy: bool = True):
+        """Completes the call that ``enqueue`` started (``vesin_hip_neighbors_collect``) and returns the quantities
+        it asked for, as ``compute`` would have. Errors of the calculation are raised here."""
+        import torch
+
+        queued = self.__dict__.get("_queued")
+        if queued is None:
+            raise RuntimeError("this calculator has no call pending")
+        self._queued = None
+        quantities, index = queued[0], queued[1]
+        error_message = ctypes.c_char_p()
+        if self._lib.vesin_hip_neighbors_collect(ctypes.byref(self._neighbors), ctypes.byref(error_message)) != 0:
+            raise RuntimeError(error_message.value.decode("utf8"))
+        n_pairs = self._neighbors.length
+        device_str = f"cuda:{index}"
+
+        def wrap(pointer, shape, typestr, dtype):
+            if n_pairs == 0:
+                return torch.empty(shape, dtype=dtype, device=device_str)
+            view = torch.as_tensor(_DeviceView(pointer, shape, typestr, self), device=device_str)
+            return view.clone() if copy else view
+
+        data = []
+        pairs = None
+        for quantity in quantities:
+            if quantity in "ijP" and pairs is None:
+                pairs = wrap(self._neighbors.pairs, (n_pairs, 2), "<u8", torch.uint64)
+            if quantity == "P":
+                data.append(pairs)
+            elif quantity == "i":
+                data.append(pairs[:, 0])
+            elif quantity == "j":
+                data.append(pairs[:, 1])
+            elif quantity == "S":
+                data.append(wrap(self._neighbors.shifts, (n_pairs, 3), "<i4", torch.int32))
+            elif quantity == "d":
+                data.append(wrap(self._neighbors.distances, (n_pairs,), "<f8", torch.float64))
+            elif quantity == "D":
+                data.append(wrap(self._neighbors.vectors, (n_pairs, 3), "<f8", torch.float64))
+        return tuple(data)
+
     def timings(self):
         """Per-stage GPU times (ms) of the last ``compute``; needs ``enable_timings(True)`` beforehand."""
         timings = VesinHipTimings()
