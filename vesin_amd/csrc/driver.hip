@@ -2683,8 +2683,11 @@ bool batch_attempt(
                 any_open_direction = any_open_direction || !flags[d];
                 any_periodic_direction = any_periodic_direction || flags[d];
             }
-            // (choose_grid and open_grids_kernel never make more cells than twice the points, or 64: limit_cells)
-            cells_bound += std::min<uint64_t>(16777216, std::max<uint64_t>(64, 2 * (first_point[s + 1] - first_point[s])));
+            // (choose_grid and open_grids_kernel never make more cells than twice the points, or 64: limit_cells; one
+            // cell under brute force, and for fewer than 32 points under the automatic choice)
+            const uint64_t points_here = first_point[s + 1] - first_point[s];
+            const bool one_cell = options.algorithm == VesinBruteForce || (options.algorithm == VesinAutoAlgorithm && points_here < 32);
+            cells_bound += one_cell ? 1 : std::min<uint64_t>(16777216, std::max<uint64_t>(64, 2 * points_here));
             const HostBox hbox = normalise_box(&host_boxes[9 * s], flags);
             host_grids_box[s] = hbox;
             GridParams& g = grids[s];
