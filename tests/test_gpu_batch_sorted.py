@@ -274,3 +274,35 @@ def test_pairs_next_to_the_cutoff_in_systems_of_one_cell(full, capfd, monkeypatc
             _call_and_check(calculator, systems, cutoff, full, "PSdD", f"{tests}, {call}")
             lines = _in_order_lines(capfd)
             assert len(lines) == 1 and lines[0].endswith(": used"), (tests, call, lines)
+
+
+@pytest.mark.parametrize("full", [True, False], ids=["full", "half"])
+def test_batches_whose_systems_all_have_few_points(full, capfd, monkeypatch):
+    """No system with more than 32 points: every system is searched by one wave instead of one workgroup. Crystals of
+    1 to 32 atoms in boxes of every shape (up to 125 images, wraps), slabs, and free molecules, whose grids are picked
+    on the device from the second call on; several hundred systems, so that workgroups hold four of them, some none."""
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    rng = np.random.default_rng(578)
+    cutoff = 4.2
+    crystals = []
+    for k in range(301):
+        n = int(rng.integers(0, 33))
+        edge = rng.uniform(2.2, 7.5) if k % 3 else rng.uniform(4.5, 7.5)
+        box = np.eye(3) * edge + 0.2 * rng.normal(size=(3, 3))
+        flags = (True, True, True) if k % 5 else (True, False, True)
+        moved = (rng.integers(-2, 3, size=(n, 3)) * np.array(flags)) @ box
+        crystals.append((rng.random((n, 3)) @ box + moved, box, flags))
+    calculator = NeighborList(cutoff=cutoff, full_list=full, sorted=True)
+    capfd.readouterr()
+    for call in ("first call", "second call"):
+        _call_and_check(calculator, crystals, cutoff, full, "PSdD", f"crystals, {call}")
+        lines = _in_order_lines(capfd)
+        assert len(lines) == 1 and lines[0].endswith(": used"), (call, lines)
+    molecules = [(rng.normal(scale=1.5, size=(int(rng.integers(1, 33)), 3)) + rng.uniform(-40, 40, size=3), np.zeros((3, 3)),
+                  (False, False, False)) for _ in range(203)]
+    for call in range(3):
+        _call_and_check(calculator, molecules, cutoff, full, "PSd", f"molecules, call {call}")
+        lines = _in_order_lines(capfd)
+        assert len(lines) == 1 and lines[0].endswith(": used"), (call, lines)
+        assert ("grids picked on the device" in lines[0]) == (call >= 1), (call, lines)
+        molecules = [(m[0] + rng.normal(scale=0.03, size=m[0].shape), m[1], m[2]) for m in molecules]

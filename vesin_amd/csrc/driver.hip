@@ -497,6 +497,7 @@ struct BatchSetup {
     size_t systems_for_images = 0;          // systems the search over images covers (grids picked on the host)
     size_t systems_for_tiles = 0;           // other systems whose stencil fits the in-order search over tiles
     size_t systems_with_points = 0;
+    size_t most_points = 0;                 // of one system
     PinnedVector<uint64_t> pair_base;       // pairs of points (n^2 per system of few points) before every system
     uint32_t image_words = 1;               // words of 64 images per pair of points, the most any system needs
     const void* d_pair_base = nullptr;
@@ -2748,6 +2749,7 @@ bool batch_attempt(
         setup.systems_for_images = 0;
         setup.systems_for_tiles = 0;
         setup.systems_with_points = 0;
+        setup.most_points = 0;
         setup.image_words = 1;
         setup.pair_base.resize(n_systems + 1);
         uint64_t pairs_so_far = 0;
@@ -2780,6 +2782,7 @@ bool batch_attempt(
             const double per_cell = std::max(1.0, static_cast<double>(g.n_points) / std::max(1u, g.n_cells));
             most_units = std::max(most_units, std::ceil(upper_stencil_cells(g) * per_cell / WAVE));
             setup.systems_with_points += n_here > 0 ? 1 : 0;
+            setup.most_points = std::max(setup.most_points, n_here);
             if (n_here > 0 && images_cover(g)) {
                 setup.systems_for_images += 1;
                 setup.image_words = std::max(setup.image_words, image_words(g));
@@ -3103,18 +3106,18 @@ bool batch_attempt(
         oargs.first_point = d_first_point;
         oargs.total_cells = static_cast<uint32_t>(total_cells);
         oargs.total_points = static_cast<uint32_t>(n_points);
-        const dim3 image_grid(static_cast<uint32_t>(n_systems));
+        // (a wave per system instead of a workgroup when no system has more than a few points)
+        const bool few_points = setup.most_points <= IMAGE_FEW_POINTS;
+        const dim3 image_grid(static_cast<uint32_t>(few_points ? (n_systems + IMAGE_WAVES - 1) / IMAGE_WAVES : n_systems));
         const dim3 tile_grid(static_cast<uint32_t>((tiles_bound + ORDERED_WAVES - 1) / ORDERED_WAVES));
         // (whichever writing pass is launched last hands the host what the counting passes found)
         auto launch_write = [&](OrderedHostStatus* publish_to) {
             if (in_order_images) {
                 iargs.publish_to = in_order_tiles ? nullptr : publish_to;
                 iargs.build_status = extras.d_status;
-                if (options.full) {
-                    hipLaunchKernelGGL(image_write_kernel<true>, image_grid, dim3(IMAGE_BLOCK), 0, stream, iargs);
-                } else {
-                    hipLaunchKernelGGL(image_write_kernel<false>, image_grid, dim3(IMAGE_BLOCK), 0, stream, iargs);
-                }
+                auto kernel = few_points ? (options.full ? image_write_kernel<true, true> : image_write_kernel<false, true>)
+                                         : (options.full ? image_write_kernel<true, false> : image_write_kernel<false, false>);
+                hipLaunchKernelGGL(kernel, image_grid, dim3(IMAGE_BLOCK), 0, stream, iargs);
             }
             if (in_order_tiles) {
                 oargs.publish_to = publish_to;
@@ -3133,11 +3136,9 @@ bool batch_attempt(
             out.vectors = reinterpret_cast<double*>(neighbors.vectors);
         };
         if (in_order_images) {
-            if (options.full) {
-                hipLaunchKernelGGL(image_count_kernel<true>, image_grid, dim3(IMAGE_BLOCK), 0, stream, iargs);
-            } else {
-                hipLaunchKernelGGL(image_count_kernel<false>, image_grid, dim3(IMAGE_BLOCK), 0, stream, iargs);
-            }
+            auto kernel = few_points ? (options.full ? image_count_kernel<true, true> : image_count_kernel<false, true>)
+                                     : (options.full ? image_count_kernel<true, false> : image_count_kernel<false, false>);
+            hipLaunchKernelGGL(kernel, image_grid, dim3(IMAGE_BLOCK), 0, stream, iargs);
         }
         if (in_order_tiles) {
             if (options.full) {

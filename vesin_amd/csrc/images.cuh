@@ -39,6 +39,10 @@ namespace vesin_hip {
 constexpr uint32_t IMAGE_MAX_WORDS = IMAGE_MAX_ENTRIES / 64;
 constexpr int IMAGE_WAVES = 4;
 constexpr int IMAGE_BLOCK = IMAGE_WAVES * WAVE;
+// Batches whose systems all have at most IMAGE_FEW_POINTS points give every system one wave instead of one workgroup
+// (four systems per workgroup, each with its own part of the LDS; the kernels' FEW variants): three of the four waves
+// of a workgroup would have nothing to do, and tens of thousands of small molecules are a common batch.
+constexpr uint32_t IMAGE_FEW_POINTS = 32;
 constexpr int IMAGE_GROUP = 2;             // units of 64 pairs of points a wave tests together
 constexpr uint32_t IMAGE_ROWS = 8 * WAVE;  // rows that a wave lines up in LDS at a time (and up to 63 left over)
 static_assert(IMAGE_MAX_POINTS <= 256 && IMAGE_MAX_ENTRIES <= 256, "a row is lined up as (first point << 16) | (second point << 8) | image");
@@ -75,45 +79,58 @@ struct ImageArgs {
     const DeviceStatus* build_status;
 };
 
+template <uint32_t POINTS>
 struct ImageShared {
-    double x[IMAGE_MAX_POINTS], y[IMAGE_MAX_POINTS], z[IMAGE_MAX_POINTS]; // by index in the system
-    int32_t wx[IMAGE_MAX_POINTS], wy[IMAGE_MAX_POINTS], wz[IMAGE_MAX_POINTS];
+    double x[POINTS], y[POINTS], z[POINTS]; // by index in the system
+    int32_t wx[POINTS], wy[POINTS], wz[POINTS];
     double tx[IMAGE_MAX_ENTRIES], ty[IMAGE_MAX_ENTRIES], tz[IMAGE_MAX_ENTRIES]; // q . H of every image kept
     int32_t q[IMAGE_MAX_ENTRIES]; // packed cell shift of every image kept
     uint32_t n_entries;
     uint32_t moved_apart; // not zero: some points were moved into the box by other box vectors than the first one
 };
 
-struct ImageCountShared: ImageShared {
+template <uint32_t POINTS>
+struct ImageCountShared: ImageShared<POINTS> {
     uint64_t with_itself[IMAGE_MAX_WORDS]; // the images of a point that may be its own neighbours
-    uint32_t rows[IMAGE_MAX_POINTS];       // rows of every point
+    uint32_t rows[POINTS];                 // rows of every point
     // The single-precision pre-test (choose_prefilter, geometry.hpp), in the form it takes for one cell: where the
     // points are after they were moved into the box, seen from one of them (r - w . H - the same of the first point:
     // within the extent of the box along every axis, or not a number), and the shifts of the images, rounded once.
     // v = (r_j - r_i) + (q - w_j + w_i) . H = (u_j - u_i) + q . H whatever the wraps are.
-    float ux[IMAGE_MAX_POINTS], uy[IMAGE_MAX_POINTS], uz[IMAGE_MAX_POINTS];
+    float ux[POINTS], uy[POINTS], uz[POINTS];
     float sx[IMAGE_MAX_ENTRIES], sy[IMAGE_MAX_ENTRIES], sz[IMAGE_MAX_ENTRIES];
     uint32_t use32;
     float lo32, hi32;
 };
 
-struct ImageWriteShared: ImageShared {
+template <uint32_t POINTS, int WAVES>
+struct ImageWriteShared: ImageShared<POINTS> {
     // (first point << 16) | (second point << 8) | image, at the place of the row: what a run of consecutive rows left
     // short of a multiple of 64, and the rows of the points behind it
-    uint32_t rows[IMAGE_WAVES][IMAGE_ROWS + WAVE];
+    uint32_t rows[WAVES][IMAGE_ROWS + WAVE];
 };
 
 /// The system's points by index, and the images that can hold a neighbour in the order of their cell shift.
-template <bool COUNT, bool FULL, typename Shared>
+/// FEW: the system is one wave's (`wave` is 0 then), not a workgroup's.
+template <bool COUNT, bool FULL, bool FEW, uint32_t POINTS, typename Shared>
 __device__ __forceinline__ void stage_system(
     Shared& sh, const ImageArgs& args, const GridParams& g, uint32_t system, uint32_t wave, int lane
 ) {
     const uint32_t n = g.n_points;
     const uint32_t at0 = static_cast<uint32_t>(args.cell_scan[args.cell_base[system]]);
-    if (threadIdx.x == 0) {
+    const uint32_t thread = FEW ? static_cast<uint32_t>(lane) : threadIdx.x;
+    constexpr uint32_t THREADS = FEW ? WAVE : IMAGE_BLOCK;
+    auto meet = [&]() {
+        if constexpr (FEW) {
+            wave_sync();
+        } else {
+            __syncthreads();
+        }
+    };
+    if (thread == 0) {
         sh.moved_apart = 0;
     }
-    __syncthreads();
+    meet();
     const int32_t wx0 = args.sorted.wx[at0];
     const int32_t wy0 = args.sorted.wy[at0];
     const int32_t wz0 = args.sorted.wz[at0];
@@ -122,7 +139,7 @@ __device__ __forceinline__ void stage_system(
     double seen_from[3] = {0.0, 0.0, 0.0};
     double reach[3] = {0.0, 0.0, 0.0};
     if constexpr (COUNT) {
-        if (threadIdx.x == 0) {
+        if (thread == 0) {
             Prefilter pre;
             choose_prefilter(g, args.cutoff, pre);
             sh.use32 = static_cast<uint32_t>(pre.use32);
@@ -142,9 +159,9 @@ __device__ __forceinline__ void stage_system(
             }
         }
     }
-    for (uint32_t p = threadIdx.x; p < n; p += IMAGE_BLOCK) {
+    for (uint32_t p = thread; p < n; p += THREADS) {
         const SortedPoint point = args.sorted.p[at0 + p];
-        const uint32_t index = min(point.index, IMAGE_MAX_POINTS - 1);
+        const uint32_t index = min(point.index, POINTS - 1);
         const int32_t wx = args.sorted.wx[at0 + p];
         const int32_t wy = args.sorted.wy[at0 + p];
         const int32_t wz = args.sorted.wz[at0 + p];
@@ -221,7 +238,7 @@ __device__ __forceinline__ void stage_system(
             }
         }
     }
-    __syncthreads();
+    meet();
 }
 
 /// The images of i seen from j, from the images of j seen from i: image e of the `n_entries` becomes image
@@ -243,12 +260,18 @@ __device__ __forceinline__ void opposite_images(uint64_t lo, uint64_t hi, uint32
 /// COUNT: one workgroup per system. A test decides two rows at once: image q of j is a neighbour of i exactly when
 /// image -q of i is a neighbour of j (the same numbers with the opposite sign all the way, the same squared norm),
 /// so only the pairs of points with i <= j are tested, 64 pairs to a wave's lanes.
-template <bool FULL>
+template <bool FULL, bool FEW>
 __global__ __launch_bounds__(IMAGE_BLOCK) void image_count_kernel(ImageArgs args) {
-    __shared__ ImageCountShared sh;
+    constexpr uint32_t POINTS = FEW ? IMAGE_FEW_POINTS : IMAGE_MAX_POINTS;
+    constexpr uint32_t WAVES = FEW ? 1 : IMAGE_WAVES;          // of a system
+    constexpr uint32_t THREADS = FEW ? WAVE : IMAGE_BLOCK;
+    __shared__ ImageCountShared<POINTS> shared[FEW ? IMAGE_WAVES : 1];
     const int lane = lane_id();
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
-    const uint32_t system = blockIdx.x;
+    const uint32_t wave_of_block = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    const uint32_t wave = FEW ? 0 : wave_of_block;              // within its system
+    const uint32_t thread = FEW ? static_cast<uint32_t>(lane) : threadIdx.x;
+    ImageCountShared<POINTS>& sh = shared[FEW ? wave_of_block : 0];
+    const uint32_t system = FEW ? blockIdx.x * IMAGE_WAVES + wave_of_block : blockIdx.x;
     if (system >= args.n_systems) {
         return;
     }
@@ -257,13 +280,13 @@ __global__ __launch_bounds__(IMAGE_BLOCK) void image_count_kernel(ImageArgs args
     if (n == 0) {
         return;
     }
-    if (!images_cover(g) || image_words(g) > args.words) {
-        if (threadIdx.x == 0 && args.others_covered == 0) {
+    if (!images_cover(g) || image_words(g) > args.words || n > POINTS) {
+        if (thread == 0 && args.others_covered == 0) {
             atomicAdd(&args.status->unsuitable, 1u);
         }
         return;
     }
-    stage_system<true, FULL>(sh, args, g, system, wave, lane);
+    stage_system<true, FULL, FEW, POINTS>(sh, args, g, system, wave, lane);
     const uint32_t n_entries = uniform(sh.n_entries);
     const bool use32 = uniform(sh.use32) != 0 && args.double_only == 0;
     const float lo32 = sh.lo32;
@@ -277,7 +300,7 @@ __global__ __launch_bounds__(IMAGE_BLOCK) void image_count_kernel(ImageArgs args
     const uint32_t width = n + 1;
     const uint32_t n_lines = (n + 1) / 2;
     const uint32_t n_lanes = n_lines * width;
-    for (uint32_t unit0 = wave * IMAGE_GROUP; unit0 * WAVE < n_lanes; unit0 += IMAGE_WAVES * IMAGE_GROUP) {
+    for (uint32_t unit0 = wave * IMAGE_GROUP; unit0 * WAVE < n_lanes; unit0 += WAVES * IMAGE_GROUP) {
         uint32_t pi[IMAGE_GROUP], pj[IMAGE_GROUP];
         bool there[IMAGE_GROUP];
         double ax[IMAGE_GROUP], ay[IMAGE_GROUP], az[IMAGE_GROUP];
@@ -446,8 +469,12 @@ __global__ __launch_bounds__(IMAGE_BLOCK) void image_count_kernel(ImageArgs args
             }
         }
     }
-    __syncthreads();
-    for (uint32_t p = threadIdx.x; p < n; p += IMAGE_BLOCK) {
+    if constexpr (FEW) {
+        wave_sync();
+    } else {
+        __syncthreads();
+    }
+    for (uint32_t p = thread; p < n; p += THREADS) {
         args.rows_of_point[first + p] = sh.rows[p];
     }
 }
@@ -455,8 +482,9 @@ __global__ __launch_bounds__(IMAGE_BLOCK) void image_count_kernel(ImageArgs args
 /// Stores the first `count` rows lined up in `rows` as the rows `first_row` ... of the list: 64 consecutive rows per
 /// step, each step ending on a multiple of 64 rows (whole cache lines in every output array; the first step stores
 /// fewer).
+template <typename Shared>
 __device__ __forceinline__ void store_image_rows(
-    const ImageWriteShared& sh, const uint32_t* rows, const GridParams& g, const SearchOutputs& out, bool moved_apart,
+    const Shared& sh, const uint32_t* rows, const GridParams& g, const SearchOutputs& out, bool moved_apart,
     uint32_t count, uint64_t first_row, int lane
 ) {
     const uint32_t skew = static_cast<uint32_t>(first_row % WAVE);
@@ -500,11 +528,15 @@ __device__ __forceinline__ void store_image_rows(
 
 /// WRITE: one workgroup per system, every wave a run of consecutive first points: their rows are consecutive rows of
 /// the list, lined up in LDS one point after the other and stored whenever they reach a multiple of 64 rows.
-template <bool FULL>
+template <bool FULL, bool FEW>
 __global__ __launch_bounds__(IMAGE_BLOCK) void image_write_kernel(ImageArgs args) {
-    __shared__ ImageWriteShared sh;
+    constexpr uint32_t POINTS = FEW ? IMAGE_FEW_POINTS : IMAGE_MAX_POINTS;
+    constexpr uint32_t WAVES = FEW ? 1 : IMAGE_WAVES; // of a system
+    __shared__ ImageWriteShared<POINTS, WAVES> shared[FEW ? IMAGE_WAVES : 1];
     const int lane = lane_id();
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    const uint32_t wave_of_block = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    const uint32_t wave = FEW ? 0 : wave_of_block;    // within its system
+    ImageWriteShared<POINTS, WAVES>& sh = shared[FEW ? wave_of_block : 0];
     if (args.publish_to != nullptr && blockIdx.x == 0 && threadIdx.x == 0) {
         OrderedHostStatus report;
         report.found = *args.status;
@@ -522,16 +554,16 @@ __global__ __launch_bounds__(IMAGE_BLOCK) void image_write_kernel(ImageArgs args
             return;
         }
     }
-    const uint32_t system = blockIdx.x;
+    const uint32_t system = FEW ? blockIdx.x * IMAGE_WAVES + wave_of_block : blockIdx.x;
     if (system >= args.n_systems) {
         return;
     }
     const GridParams g = args.grids[system];
     const uint32_t n = g.n_points;
-    if (n == 0 || !images_cover(g) || image_words(g) > args.words) {
+    if (n == 0 || !images_cover(g) || image_words(g) > args.words || n > POINTS) {
         return;
     }
-    stage_system<false, FULL>(sh, args, g, system, wave, lane);
+    stage_system<false, FULL, FEW, POINTS>(sh, args, g, system, wave, lane);
     const bool moved_apart = uniform(sh.moved_apart) != 0;
     const uint32_t first = args.first_point[system];
     const uint32_t words = args.words;
@@ -539,7 +571,7 @@ __global__ __launch_bounds__(IMAGE_BLOCK) void image_write_kernel(ImageArgs args
     uint32_t* rows = sh.rows[wave];
     const SearchOutputs& out = args.out;
 
-    const uint32_t per_wave = (n + IMAGE_WAVES - 1) / IMAGE_WAVES;
+    const uint32_t per_wave = (n + WAVES - 1) / WAVES;
     const uint32_t i_begin = wave * per_wave;
     const uint32_t i_end = min(n, i_begin + per_wave);
     if (i_begin >= i_end) {
