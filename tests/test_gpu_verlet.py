@@ -255,3 +255,26 @@ def test_verlet_no_points_and_no_pairs():
     assert result["pairs"].shape == (0, 2)
     result = _compute(calculator, np.array([[0.0, 0.0, 0.0], [0.5, 0.0, 0.0]]), box, True)
     assert sorted(result["pairs"].tolist()) == [[0, 1], [1, 0]]
+
+
+@pytest.mark.parametrize("full_list", [True, False])
+def test_verlet_points_given_several_boxes_outside_of_a_box_that_changes(full_list):
+    """Points given up to three boxes outside of the box make pairs with shifts of up to seven boxes, and the image
+    of such a pair moves seven times as far as a corner of the box when the box changes: the reference's bound on the
+    change of the box (vesin/src/verlet.cpp:10-34, :80-84) covers the images one box away. The rows must be those of
+    a direct calculation all the same: the cache knows the largest shift among its candidates and rebuilds earlier."""
+    rng = np.random.default_rng(2158)
+    cutoff, skin = 1.1, 0.3
+    box = np.array([[3.735, 0.0, 0.0], [-0.261, 3.735, 0.0], [-0.43, 0.357, 3.735]])
+    points = rng.random((600, 3)) @ box + rng.integers(-3, 4, size=(600, 3)) @ box
+    calculator = NeighborList(cutoff=cutoff, full_list=full_list, skin=skin)
+    checked = 0
+    for step in range(12):
+        result = _compute(calculator, points, box, True)
+        _assert_direct(result, points, box, True, cutoff, full_list)
+        checked += len(result["pairs"])
+        # small moves, which alone would let the cache live on, and a box that changes by up to 0.03 per element
+        points = points + rng.normal(scale=0.01, size=points.shape)
+        if step % 2 == 0:
+            box = box + rng.normal(scale=0.015, size=(3, 3)) * (np.abs(box) > 0)
+    assert checked > 100000 and np.abs(result["shifts"]).max() >= 5

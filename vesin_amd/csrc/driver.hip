@@ -2325,6 +2325,15 @@ void verlet_neighbors(
             verlet_store_reference, dim3(1), dim3(64), 0, stream, reinterpret_cast<const double*>(box), periodic,
             cache.reference
         );
+        if (cache.candidates.length > 0) {
+            // (how far the shifts of the candidates reach: what the box may change by before they are computed again
+            // depends on it, see verlet_check_kernel)
+            const uint32_t blocks = static_cast<uint32_t>(std::min<size_t>(1024, (cache.candidates.length + VERLET_BLOCK - 1) / VERLET_BLOCK));
+            hipLaunchKernelGGL(
+                verlet_shift_reach_kernel, dim3(blocks), dim3(VERLET_BLOCK), 0, stream,
+                reinterpret_cast<const int32_t*>(cache.candidates.shifts), cache.candidates.length, cache.reference
+            );
+        }
         // the snapshot is complete before the call returns: the caller may change points and box right after
         HIP_CHECK(hipGetLastError());
         HIP_CHECK(hipStreamSynchronize(stream));

@@ -26,6 +26,8 @@ constexpr int VERLET_WAVES = VERLET_BLOCK / WAVE;
 struct VerletReference {
     double box[9];
     unsigned char periodic[3];
+    // the largest shift of a candidate along every direction, as an absolute value (verlet_shift_reach_kernel)
+    unsigned int largest_shift[3];
 };
 
 /// Written by the kernels into pinned host memory, read by the host after the call's synchronisation.
@@ -51,6 +53,34 @@ __global__ void verlet_store_reference(
     }
     if (t < 3) {
         reference->periodic[t] = periodic[t] ? 1 : 0;
+        reference->largest_shift[t] = 0;
+    }
+}
+
+/// The largest |S_d| among the candidates, per direction (launched behind verlet_store_reference). Points given far
+/// outside of the box make pairs with shifts of several boxes, and how far the image of such a pair moves when the
+/// box changes grows with the shift: see verlet_check_kernel.
+__global__ __launch_bounds__(VERLET_BLOCK) void verlet_shift_reach_kernel(
+    const int32_t* __restrict__ candidate_shifts, size_t n_candidates, VerletReference* __restrict__ reference
+) {
+    unsigned int reach[3] = {0, 0, 0};
+    const size_t stride = static_cast<size_t>(gridDim.x) * VERLET_BLOCK;
+    for (size_t row = static_cast<size_t>(blockIdx.x) * VERLET_BLOCK + threadIdx.x; row < n_candidates; row += stride) {
+#pragma unroll
+        for (int d = 0; d < 3; d++) {
+            const int32_t shift = candidate_shifts[3 * row + d];
+            reach[d] = max(reach[d], static_cast<unsigned int>(shift < 0 ? -shift : shift));
+        }
+    }
+#pragma unroll
+    for (int d = 0; d < 3; d++) {
+#pragma unroll
+        for (int offset = WAVE / 2; offset > 0; offset >>= 1) {
+            reach[d] = max(reach[d], static_cast<unsigned int>(__shfl_xor(static_cast<int>(reach[d]), offset, WAVE)));
+        }
+        if (lane_id() == 0 && reach[d] > 1) {
+            atomicMax(&reference->largest_shift[d], reach[d]);
+        }
     }
 }
 
@@ -95,7 +125,24 @@ __global__ __launch_bounds__(VERLET_BLOCK) void verlet_check_kernel(
         }
         const double half_skin = skin / 2.0;
         const double half_skin_sq = half_skin * half_skin;
-        const double half_displacement = corner_displacements(box, reference->box) / 2.0;
+        double half_displacement = corner_displacements(box, reference->box) / 2.0;
+        // The reference's bound covers the images one box away: the image of a pair with shift S moves by S . (H -
+        // H_ref) when the box changes, and for |S_d| <= 1 that is at most the two largest corner displacements. Points
+        // given several boxes outside of the box make pairs with larger shifts, whose images move further: for them
+        // the bound is sum_d max|S_d| x |H_d - H_ref_d| (never smaller than needed: more rebuilds, never a missed
+        // pair). Nothing changes while the box stays as it is, or while no candidate has such a shift.
+        if (reference->largest_shift[0] > 1 || reference->largest_shift[1] > 1 || reference->largest_shift[2] > 1) {
+            double reach = 0.0;
+            for (int d = 0; d < 3; d++) {
+                double moved_sq = 0.0;
+                for (int k = 0; k < 3; k++) {
+                    const double moved = box[3 * d + k] - reference->box[3 * d + k];
+                    moved_sq += moved * moved;
+                }
+                reach += static_cast<double>(max(reference->largest_shift[d], 1u)) * sqrt(moved_sq);
+            }
+            half_displacement = fmax(half_displacement, reach / 2.0);
+        }
         // also true when the box holds a NaN
         too_far = too_far || !(half_displacement * half_displacement <= half_skin_sq);
         threshold_sq = (sqrt(half_skin_sq) - half_displacement) * (sqrt(half_skin_sq) - half_displacement);
