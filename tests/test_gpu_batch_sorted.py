@@ -150,14 +150,16 @@ def test_a_list_that_grows_and_brute_force(capfd, monkeypatch):
 
 def test_molecules_whose_grids_are_picked_on_the_device(capfd, monkeypatch):
     """Systems without periodic directions get their grids on the device from the second call on: the host does not
-    know then whether they are of one cell. Small molecules are; when one of them has grown into several cells, the
-    kernels say so, the rows come from the two passes and the sort, and the next calls do not ask again for a while."""
+    know their shapes then. In a sorted batch a molecule of up to 256 atoms is one cell however far it spreads (the
+    search over images is at its best there), so such batches stay with that search; a larger molecule is not its
+    to search: the kernels say so, the rows come from the two passes and the sort, and the next calls do not ask
+    again for a while."""
     monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
     rng = np.random.default_rng(573)
     cutoff = 2.5
-    sizes = [1, 2, 5, 17, 40, 31, 12, 3]
-    # (fewer than 32 points are one cell whatever their extent; the molecule of 40 is, as long as it is compact)
-    molecules = [rng.normal(scale=0.3 if n == 40 else 1.2, size=(n, 3)) + rng.uniform(-30, 30, size=3) for n in sizes]
+    sizes = [1, 2, 5, 17, 40, 31, 12, 3, 200]
+    # (the molecules of 40 and of 200 atoms spread over several cutoffs: a cell list would give them many cells)
+    molecules = [rng.normal(scale=3.0 if n >= 40 else 1.2, size=(n, 3)) + rng.uniform(-30, 30, size=3) for n in sizes]
     zero = np.zeros((3, 3))
 
     def systems():
@@ -168,14 +170,19 @@ def test_molecules_whose_grids_are_picked_on_the_device(capfd, monkeypatch):
     for call in range(4):
         _call_and_check(calculator, systems(), cutoff, True, "PSdD", f"call {call}")
         lines = _in_order_lines(capfd)
-        assert len(lines) == 1 and lines[0].endswith(": used"), (call, lines)
+        assert len(lines) == 1 and lines[0].endswith(": used") and " 0 by tiles" in lines[0], (call, lines)
         assert ("grids picked on the device" in lines[0]) == (call >= 1), (call, lines)
         molecules = [m + rng.normal(scale=0.02, size=m.shape) for m in molecules]
-    # one molecule spreads out over several cells (same number of points: the grids are still the device's)
-    molecules[4] = (molecules[4] - molecules[4].mean(axis=0)) * 8.0
-    _call_and_check(calculator, systems(), cutoff, True, "PSdD", "after spreading out")
+    # with a molecule of 300 atoms: the host gives it to the search over tiles; the device's grids are only for the
+    # search over images
+    molecules.append(rng.normal(scale=3.0, size=(300, 3)))
+    calculator = NeighborList(cutoff=cutoff, full_list=True, sorted=True)
+    _call_and_check(calculator, systems(), cutoff, True, "PSdD", "with a large molecule, first call")
     lines = _in_order_lines(capfd)
-    assert len(lines) == 1 and lines[0].endswith(": left to the radix sort"), lines
+    assert len(lines) == 1 and lines[0].endswith(": used") and " 1 by tiles" in lines[0], lines
+    _call_and_check(calculator, systems(), cutoff, True, "PSdD", "second call")
+    lines = _in_order_lines(capfd)
+    assert len(lines) == 1 and lines[0].endswith(": left to the radix sort") and "grids picked on the device" in lines[0], lines
     _call_and_check(calculator, systems(), cutoff, True, "PSdD", "the call after")
     assert not _in_order_lines(capfd)
 
@@ -200,7 +207,7 @@ def test_systems_of_several_cells_come_out_in_order(full, capfd, monkeypatch):
     cutoff = 4.0
     several = _systems_of_several_cells(rng, [
         (700, (True, True, True)), (300, (True, True, False)), (1500, (True, False, False)), (450, (False, False, False)),
-        (3000, (True, True, True)), (33, (True, True, True)),
+        (3000, (True, True, True)), (100, (True, True, True)),
     ])
     calculator = NeighborList(cutoff=cutoff, full_list=full, sorted=True)
     capfd.readouterr()

@@ -599,10 +599,12 @@ __global__ __launch_bounds__(BLOCK) void bounding_batch_kernel(
 /// (geometry.hpp) does on the host for such a system: the box counts for nothing (the three directions are unit
 /// vectors), cells at least as wide as the cutoff over the extent of the points with a margin of 1 %, never more
 /// cells than twice the points (or 64), nothing beyond the last cell. `single_cell`: 1 always (brute force), 0 for
-/// systems that fill more than a cell and have 32 points or more (automatic choice), -1 never (cell list).
+/// systems that fill more than a cell and have `few_points` points or more (automatic choice: 32, or more where the
+/// search that follows is at its best on systems of one cell), -1 never (cell list).
 __global__ __launch_bounds__(BLOCK) void open_grids_kernel(
     const double* __restrict__ points, const uint32_t* __restrict__ first_point, uint32_t n_systems, double cutoff,
-    int single_cell, GridParams* __restrict__ grids, uint32_t* __restrict__ cells_of_system, unsigned int* first_bad
+    int single_cell, uint32_t few_points, GridParams* __restrict__ grids, uint32_t* __restrict__ cells_of_system,
+    unsigned int* first_bad
 ) {
     const uint32_t system = blockIdx.x * WAVES_PER_BLOCK + threadIdx.x / WAVE;
     if (system >= n_systems) {
@@ -691,7 +693,7 @@ __global__ __launch_bounds__(BLOCK) void open_grids_kernel(
             g.s[d] = static_cast<int32_t>(radius);
         }
         g.n_cells = n_cells;
-        if (single_cell == 0 && !one_cell && (n_cells == 1 || n_here < 32)) {
+        if (single_cell == 0 && !one_cell && (n_cells == 1 || n_here < few_points)) {
             one_cell = true; // too little for a cell list: one cell, every point against every other
             continue;
         }

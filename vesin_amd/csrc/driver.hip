@@ -454,6 +454,18 @@ struct PinnedAllocator {
 template <typename T>
 using PinnedVector = std::vector<T, PinnedAllocator<T>>;
 
+/// The systems of a batch are small, and a small system of several cells is many tiles of a few points each: every
+/// tile costs a wave its fixed work (tables, staging), and the sorted search over tiles needs a record block per
+/// tile. One cell means brute force over points x points x images pairs, which is cheap while that product is small,
+/// and the search over images (images.cuh) writes sorted rows of such systems in order. Under the automatic choice
+/// of the algorithm a system of a batch is therefore given one cell not only below 32 points but whenever the tests
+/// stay few: up to 256 points without images (free molecules: 20,000 molecules of 3 to 40 atoms 0.75 -> 0.29 ms per
+/// unsorted batch, 1.16 -> 0.46 ms sorted), up to 69 points with the 27 images of a box wider than the cutoff.
+constexpr uint64_t ONE_CELL_TESTS = 131072; // points x points x images
+inline bool one_cell_in_a_batch(uint64_t n_points, uint64_t n_images) {
+    return n_points <= IMAGE_MAX_POINTS && n_images <= IMAGE_MAX_ENTRIES && n_points * n_points * n_images <= ONE_CELL_TESTS;
+}
+
 struct BatchSetup {
     bool valid = false;
     bool any_open_direction = false;
@@ -2696,7 +2708,11 @@ bool batch_attempt(
             // (choose_grid and open_grids_kernel never make more cells than twice the points, or 64: limit_cells; one
             // cell under brute force, and for fewer than 32 points under the automatic choice)
             const uint64_t points_here = first_point[s + 1] - first_point[s];
-            const bool one_cell = options.algorithm == VesinBruteForce || (options.algorithm == VesinAutoAlgorithm && points_here < 32);
+            const bool any_periodic_here = flags[0] || flags[1] || flags[2];
+            // (a system without periodic directions has no images: what open_grids_kernel is told below)
+            const bool one_cell = options.algorithm == VesinBruteForce ||
+                                  (options.algorithm == VesinAutoAlgorithm &&
+                                   (points_here < 32 || (!any_periodic_here && one_cell_in_a_batch(points_here, 1))));
             cells_bound += one_cell ? 1 : std::min<uint64_t>(16777216, std::max<uint64_t>(64, 2 * points_here));
             const HostBox hbox = normalise_box(&host_boxes[9 * s], flags);
             host_grids_box[s] = hbox;
@@ -2773,6 +2789,17 @@ bool batch_attempt(
             HostGrid grid = choose_grid(hbox, options.cutoff, n_here, lo, hi, single_cell);
             if (options.algorithm == VesinAutoAlgorithm && !single_cell && (grid.n_cells == 1 || n_here < 32)) {
                 grid = choose_grid(hbox, options.cutoff, n_here, lo, hi, true);
+            } else if (options.algorithm == VesinAutoAlgorithm && !single_cell && n_here <= IMAGE_MAX_POINTS) {
+                // (a radius beyond what a stencil may have is an error of choose_grid: not for a choice that is only
+                // tried)
+                try {
+                    const HostGrid one_cell = choose_grid(hbox, options.cutoff, n_here, lo, hi, true);
+                    const uint64_t images = static_cast<uint64_t>(2 * one_cell.s[0] + 1) * (2 * one_cell.s[1] + 1) * (2 * one_cell.s[2] + 1);
+                    if (one_cell_in_a_batch(n_here, images)) {
+                        grid = one_cell;
+                    }
+                } catch (const std::runtime_error&) {
+                }
             }
             GridParams& g = grids[s];
             for (int d = 0; d < 3; d++) {
@@ -3023,8 +3050,8 @@ bool batch_attempt(
         const int single_cell = options.algorithm == VesinBruteForce ? 1 : options.algorithm == VesinAutoAlgorithm ? 0 : -1;
         hipLaunchKernelGGL(
             open_grids_kernel, dim3(static_cast<uint32_t>((n_systems + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK)), dim3(BLOCK),
-            0, stream, flat_points, d_first_point, static_cast<uint32_t>(n_systems), options.cutoff, single_cell, d_grids,
-            d_cells_of_system, &extras.d_status->first_bad_coordinate
+            0, stream, flat_points, d_first_point, static_cast<uint32_t>(n_systems), options.cutoff, single_cell,
+            IMAGE_MAX_POINTS + 1, d_grids, d_cells_of_system, &extras.d_status->first_bad_coordinate
         );
         hipLaunchKernelGGL(
             open_bases_kernel, dim3(1), dim3(1024), 0, stream,
