@@ -243,7 +243,9 @@ int VESIN_API vesin_hip_neighbors_no_alloc(
  *                system s
  *
  * With options.sorted every system's rows are ordered as vesin_neighbors orders them for that system alone (by
- * (i, j, shift)); options.skin must be zero. Returns EXIT_SUCCESS / EXIT_FAILURE like vesin_neighbors, with the same
+ * (i, j, shift)). With options.skin > 0 the list keeps candidates at cutoff + skin for the whole batch and later
+ * calls with the same division into systems filter them while no point of any system has moved further than the
+ * skin allows (per system, as vesin_neighbors decides it); the rows are always those of skin = 0. Returns EXIT_SUCCESS / EXIT_FAILURE like vesin_neighbors, with the same
  * message ownership. */
 int VESIN_API vesin_hip_neighbors_batch(
     const double (*points)[3],

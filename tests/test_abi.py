@@ -186,10 +186,10 @@ def test_validation_of_the_additions():
     assert (status, text(message)) == (1, "`first_pair` can not be a NULL pointer")
     with_skin = _c_api.VesinOptions()
     with_skin.cutoff = 1.0
-    with_skin.skin = 0.2
+    with_skin.skin = -0.2
     message = ctypes.c_char_p()
     status = lib.vesin_hip_neighbors_batch(
         address, first_point, 1, address, address, gpu, with_skin, ctypes.byref(neighbors), first_pair, ctypes.byref(message)
     )
-    assert status == 1 and "not available for a batch" in text(message)
+    assert (status, text(message)) == (1, "skin must be a finite, non-negative number")
     lib.vesin_free(ctypes.byref(neighbors))

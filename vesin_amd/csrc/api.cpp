@@ -299,9 +299,6 @@ static int neighbors_batch_on(
     }
 
     try {
-        if (options.skin > 0.0) {
-            throw std::runtime_error("a non-zero `skin` (Verlet caching) is not available for a batch of systems");
-        }
         if (neighbors->device.type == VesinUnknownDevice) {
             neighbors->device = device;
         }

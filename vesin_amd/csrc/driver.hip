@@ -454,6 +454,48 @@ struct PinnedAllocator {
 template <typename T>
 using PinnedVector = std::vector<T, PinnedAllocator<T>>;
 
+/// VerletCache for a batch of systems (vesin_hip_neighbors_batch with options.skin > 0): the candidates are the rows
+/// of a batch call at cutoff + skin, kept with the division into systems and the points and boxes they came from.
+struct BatchVerletCache {
+    VesinNeighborList candidates = VesinNeighborList();
+    std::vector<size_t> first_point;          // the division into systems the candidates were built for
+    std::vector<size_t> candidate_first_pair; // where every system's candidates begin
+    DeviceBuffer kept;                        // what lives as long as the candidates (see rebuild)
+    DeviceBuffer scratch;                     // what a filtering call needs
+    double* ref_points = nullptr;
+    BatchVerletReference* reference = nullptr;
+    uint32_t* system_of_point = nullptr;
+    uint32_t* system_of_row = nullptr;
+    unsigned long long* d_first_point = nullptr;
+    VerletStatus* status = nullptr;           // pinned
+    PinnedVector<unsigned long long> first_pair_landing;
+    VesinOptions options = {};
+    bool valid = false;
+    bool direct = false;                      // as in VerletCache
+    size_t direct_n_points = 0;
+
+    BatchVerletCache() = default;
+    BatchVerletCache(const BatchVerletCache&) = delete;
+    BatchVerletCache& operator=(const BatchVerletCache&) = delete;
+
+    void drop_candidates() {
+        if (candidates.device.type == VesinCUDA) {
+            free_neighbors(candidates);
+        }
+        candidates = VesinNeighborList();
+        valid = false;
+    }
+
+    ~BatchVerletCache() {
+        drop_candidates();
+        kept.release();
+        scratch.release();
+        if (status != nullptr) {
+            (void)hipHostFree(status);
+        }
+    }
+};
+
 /// The systems of a batch are small, and a small system of several cells is many tiles of a few points each: every
 /// tile costs a wave its fixed work (tables, staging), and the sorted search over tiles needs a record block per
 /// tile. One cell means brute force over points x points x images pairs, which is cheap while that product is small,
@@ -719,6 +761,7 @@ struct HipExtras {
     bool timings_valid = false;
     VesinHipTimings timings = {};
     VerletCache* verlet = nullptr;    // only while the caller asks for a skin
+    BatchVerletCache* verlet_batch = nullptr; // the same for batches
     // vesin_hip_neighbors_enqueue / _collect: the call that stopped at its first wait, and the device word that tells
     // kernels queued behind it whether the rows are complete (made when first needed)
     SuspendedCall* queued = nullptr;
@@ -771,6 +814,7 @@ struct HipExtras {
 
     ~HipExtras() {
         delete verlet;
+        delete verlet_batch;
         delete queued;
         if (d_queued_length != nullptr) {
             (void)hipFree(d_queued_length);
@@ -2528,6 +2572,18 @@ bool batch_attempt(
     HipExtras& extras, bool speculate, hipStream_t stream
 );
 
+void direct_batch(
+    const double (*points)[3], const size_t* first_point, size_t n_systems, const double (*boxes)[3][3],
+    const bool (*periodic)[3], VesinOptions options, VesinNeighborList& neighbors, size_t* first_pair,
+    HipExtras& extras, hipStream_t stream
+);
+
+void verlet_batch(
+    const double (*points)[3], const size_t* first_point, size_t n_systems, const double (*boxes)[3][3],
+    const bool (*periodic)[3], VesinOptions options, VesinNeighborList& neighbors, size_t* first_pair,
+    HipExtras& extras, hipStream_t stream
+);
+
 } // namespace
 
 void neighbors_batch(
@@ -2579,8 +2635,29 @@ void neighbors_batch(
     HipExtras& extras = extras_of(neighbors);
     refuse_while_queued(extras);
     extras.timings_valid = false;
-    extras.guess.have_box = false; // the work buffers of the single-system path are about to be reused
     hipStream_t stream = static_cast<hipStream_t>(caller_stream);
+    if (options.skin > 0.0) {
+        verlet_batch(points, first_point, n_systems, boxes, periodic, options, neighbors, first_pair, extras, stream);
+        return;
+    }
+    if (extras.verlet_batch != nullptr) {
+        // no skin any more: the cache goes, as for single systems
+        delete extras.verlet_batch;
+        extras.verlet_batch = nullptr;
+    }
+    direct_batch(points, first_point, n_systems, boxes, periodic, options, neighbors, first_pair, extras, stream);
+}
+
+namespace {
+
+/// A batch without a skin, on a list that has its state and whose inputs were checked, with the list's device current.
+void direct_batch(
+    const double (*points)[3], const size_t* first_point, size_t n_systems, const double (*boxes)[3][3],
+    const bool (*periodic)[3], VesinOptions options, VesinNeighborList& neighbors, size_t* first_pair,
+    HipExtras& extras, hipStream_t stream
+) {
+    const size_t n_points = first_point[n_systems];
+    extras.guess.have_box = false; // the work buffers of the single-system path are about to be reused
 
     // The grids follow from the boxes, the flags, the division into systems, the cutoff and the algorithm alone,
     // unless some direction is open: then they also follow the points. Same inputs as the call before: same grids.
@@ -2626,6 +2703,269 @@ void neighbors_batch(
     setup.guess.have_box = setup.kept_on_device;
     setup.guess.stored(key);
 }
+
+/// Candidates beyond which a batch is searched directly on every call (see VERLET_MAX_CANDIDATES): the filter of a
+/// batch reads 36 bytes per candidate and two points on top of writing the rows, in two passes, and takes 0.05 ms
+/// and 36 ns per thousand candidates (i j S d asked for, a fourth of the candidates beyond the cutoff). The direct
+/// search costs more per call and less per row. Measured, direct against filter, full lists with skin 0.5:
+/// 2,000 free molecules of 3 to 40 atoms (1.0 M rows) 0.162 / 0.095 ms; 100,000 of 3 to 8 atoms (2.8 M rows) 0.750 /
+/// 0.248 ms; 512 periodic cells of 64 atoms (3.6 M rows) 0.208 / 0.226 ms; 20,000 molecules of 3 to 40 atoms (10.2 M
+/// rows) 0.456 / 0.493 ms; 4,096 cells of 64 atoms (29 M rows) 0.818 / 1.337 ms. Sorted lists of systems of several
+/// cells are the exception: the search that writes them in order takes 0.809 ms for 1,000 cells of 200 atoms (9.5 M
+/// rows) and 2.71 ms for 4,000 of them, the filter of sorted candidates 0.503 and 1.83 ms.
+constexpr size_t BATCH_VERLET_MAX_CANDIDATES = size_t(1) << 22;
+constexpr size_t BATCH_VERLET_MAX_CANDIDATES_SORTED_CELLS = size_t(1) << 26;
+
+/// options.skin > 0 for a batch: verlet_neighbors with one candidate list for all systems. The candidates are
+/// computed again as a whole when any system's points or box moved too far, when the division into systems or the
+/// options changed; otherwise a call is the two box and point checks, the two passes of the filter with a scan
+/// between them, and one synchronisation.
+void verlet_batch(
+    const double (*points)[3], const size_t* first_point, size_t n_systems, const double (*boxes)[3][3],
+    const bool (*periodic)[3], VesinOptions options, VesinNeighborList& neighbors, size_t* first_pair,
+    HipExtras& extras, hipStream_t stream
+) {
+    const TraceRange whole_call("vesin_hip_neighbors_batch (skin)");
+    if (extras.verlet_batch == nullptr) {
+        auto cache = std::make_unique<BatchVerletCache>();
+        HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&cache->status), sizeof(VerletStatus), hipHostMallocDefault));
+        extras.verlet_batch = cache.release();
+    }
+    BatchVerletCache& cache = *extras.verlet_batch;
+    const size_t n_points = first_point[n_systems];
+    const size_t pair_limit = pairs_per_point_limit();
+
+    const bool options_changed = cache.options.cutoff != options.cutoff || cache.options.skin != options.skin ||
+                                 cache.options.full != options.full || cache.options.sorted != options.sorted;
+    const bool same_division = cache.first_point.size() == n_systems + 1 &&
+                               std::memcmp(cache.first_point.data(), first_point, (n_systems + 1) * sizeof(size_t)) == 0;
+    bool fresh = false;
+    auto rebuild = [&]() {
+        cache.valid = false;
+        VesinOptions build = {};
+        build.cutoff = options.cutoff + options.skin;
+        build.full = options.full;
+        build.sorted = options.sorted; // the filter keeps the order of the candidates
+        build.algorithm = VesinAutoAlgorithm;
+        build.n_threads = options.n_threads;
+        build.return_shifts = true;
+        build.return_distances = false;
+        build.return_vectors = false;
+        build.skin = 0.0;
+        cache.candidates.device = neighbors.device;
+        cache.candidate_first_pair.resize(n_systems + 1);
+        vesin_hip::neighbors_batch(
+            points, first_point, n_systems, boxes, periodic, build, cache.candidates, cache.candidate_first_pair.data(), stream
+        );
+        cache.first_point.assign(first_point, first_point + n_systems + 1);
+        const size_t n_candidates = cache.candidates.length;
+
+        unsigned long long* d_candidate_first = nullptr;
+        auto carve = [&](Carver& c) {
+            cache.ref_points = c.take<double>(3 * n_points);
+            cache.reference = c.take<BatchVerletReference>(n_systems);
+            cache.system_of_point = c.take<uint32_t>(n_points);
+            cache.system_of_row = c.take<uint32_t>(n_candidates);
+            cache.d_first_point = c.take<unsigned long long>(n_systems + 1);
+            d_candidate_first = c.take<unsigned long long>(n_systems + 1);
+        };
+        Carver measure(nullptr);
+        carve(measure);
+        cache.kept.reserve(measure.used);
+        Carver carver(cache.kept.ptr);
+        carve(carver);
+
+        static_assert(sizeof(size_t) == sizeof(unsigned long long), "size_t is 64 bits wide here");
+        if (n_points > 0) {
+            HIP_CHECK(hipMemcpyAsync(cache.ref_points, points, n_points * 3 * sizeof(double), hipMemcpyDeviceToDevice, stream));
+        }
+        HIP_CHECK(hipMemcpyAsync(
+            cache.d_first_point, cache.first_point.data(), (n_systems + 1) * sizeof(size_t), hipMemcpyHostToDevice, stream
+        ));
+        HIP_CHECK(hipMemcpyAsync(
+            d_candidate_first, cache.candidate_first_pair.data(), (n_systems + 1) * sizeof(size_t), hipMemcpyHostToDevice, stream
+        ));
+        const uint32_t system_blocks = static_cast<uint32_t>((n_systems + VERLET_BLOCK - 1) / VERLET_BLOCK);
+        hipLaunchKernelGGL(
+            verlet_batch_store_reference, dim3(system_blocks), dim3(VERLET_BLOCK), 0, stream,
+            reinterpret_cast<const double*>(boxes), reinterpret_cast<const bool*>(periodic), static_cast<uint32_t>(n_systems),
+            cache.reference
+        );
+        if (n_points > 0) {
+            const uint32_t blocks = static_cast<uint32_t>(std::min<size_t>(4096, (n_points + VERLET_BLOCK - 1) / VERLET_BLOCK));
+            hipLaunchKernelGGL(
+                verlet_batch_owner_kernel, dim3(blocks), dim3(VERLET_BLOCK), 0, stream, cache.d_first_point,
+                static_cast<uint32_t>(n_systems), n_points, cache.system_of_point, static_cast<const int32_t*>(nullptr),
+                cache.reference
+            );
+        }
+        if (n_candidates > 0) {
+            const uint32_t blocks = static_cast<uint32_t>(std::min<size_t>(4096, (n_candidates + VERLET_BLOCK - 1) / VERLET_BLOCK));
+            hipLaunchKernelGGL(
+                verlet_batch_owner_kernel, dim3(blocks), dim3(VERLET_BLOCK), 0, stream, d_candidate_first,
+                static_cast<uint32_t>(n_systems), n_candidates, cache.system_of_row,
+                reinterpret_cast<const int32_t*>(cache.candidates.shifts), cache.reference
+            );
+        }
+        // the snapshot is complete before the call returns: the caller may change points and boxes right after
+        HIP_CHECK(hipGetLastError());
+        HIP_CHECK(hipStreamSynchronize(stream));
+        cache.options = options;
+        cache.valid = true;
+        fresh = true;
+    };
+    const char* forced = std::getenv("VESIN_HIP_VERLET");
+    const bool force_cache = forced != nullptr && std::strcmp(forced, "cache") == 0;
+    const bool force_direct = forced != nullptr && std::strcmp(forced, "direct") == 0;
+    auto too_long_for_a_filter = [&](size_t rows) {
+        const double ratio = (options.cutoff + options.skin) / options.cutoff;
+        const double candidates = static_cast<double>(rows) * ratio * ratio * ratio;
+        // (what the last direct search of this list found out about its systems: sorted, and some of them have
+        // several cells)
+        const BatchSetup& setup = extras.batch;
+        const bool sorted_cells = options.sorted && setup.valid && !setup.all_open &&
+                                  setup.systems_for_images < setup.systems_with_points;
+        const size_t limit = sorted_cells ? BATCH_VERLET_MAX_CANDIDATES_SORTED_CELLS : BATCH_VERLET_MAX_CANDIDATES;
+        return force_direct || (!force_cache && candidates > static_cast<double>(limit));
+    };
+    if (options_changed || cache.direct_n_points != n_points) {
+        cache.direct = false;
+    }
+    if (!cache.valid || options_changed || !same_division || cache.direct) {
+        // (as in verlet_neighbors: this call is a direct search, and its row count says whether candidates pay)
+        VesinOptions plain = options;
+        plain.skin = 0.0;
+        direct_batch(points, first_point, n_systems, boxes, periodic, plain, neighbors, first_pair, extras, stream);
+        cache.direct = too_long_for_a_filter(neighbors.length);
+        cache.direct_n_points = n_points;
+        if (cache.direct) {
+            cache.drop_candidates();
+            cache.first_point.clear();
+        } else {
+            rebuild();
+        }
+        return;
+    }
+
+    cache.first_pair_landing.resize(n_systems + 1);
+    size_t total = 0;
+    size_t n_candidates = 0;
+    for (int attempt = 0;; attempt++) {
+        if (attempt > 4) {
+            throw std::runtime_error("internal error: the Verlet filter of a batch did not settle");
+        }
+        n_candidates = cache.candidates.length;
+        const size_t n_chunks = (n_candidates + VERLET_CHUNK - 1) / VERLET_CHUNK;
+        size_outputs(neighbors, extras, 0, options);
+
+        BatchVerletLimits* limits = nullptr;
+        uint32_t* chunk_rows = nullptr;
+        uint64_t* chunk_base = nullptr;
+        uint64_t* scan_scratch = nullptr;
+        unsigned long long* d_first_pair = nullptr;
+        auto carve = [&](Carver& c) {
+            limits = c.take<BatchVerletLimits>(n_systems);
+            chunk_rows = c.take<uint32_t>(n_chunks);
+            chunk_base = c.take<uint64_t>(n_chunks + 1);
+            scan_scratch = c.take<uint64_t>(scan_scratch_elements(n_chunks));
+            d_first_pair = c.take<unsigned long long>(n_systems + 1);
+        };
+        Carver measure(nullptr);
+        carve(measure);
+        cache.scratch.reserve(measure.used);
+        Carver carver(cache.scratch.ptr);
+        carve(carver);
+
+        cache.status->rebuild = 0;
+        cache.status->total_rows = 0;
+        const uint32_t system_blocks = static_cast<uint32_t>((n_systems + VERLET_BLOCK - 1) / VERLET_BLOCK);
+        hipLaunchKernelGGL(
+            verlet_batch_limits_kernel, dim3(system_blocks), dim3(VERLET_BLOCK), 0, stream,
+            reinterpret_cast<const double*>(boxes), reinterpret_cast<const bool*>(periodic), cache.reference,
+            static_cast<uint32_t>(n_systems), options.skin, limits, cache.status
+        );
+        if (n_points > 0) {
+            const uint32_t blocks = static_cast<uint32_t>((n_points + VERLET_BLOCK - 1) / VERLET_BLOCK);
+            hipLaunchKernelGGL(
+                verlet_batch_moved_kernel, dim3(blocks), dim3(VERLET_BLOCK), 0, stream,
+                reinterpret_cast<const double*>(points), cache.ref_points, n_points, cache.system_of_point, limits,
+                cache.status
+            );
+        }
+        if (n_candidates > 0) {
+            BatchVerletFilterArgs fargs;
+            fargs.candidate_pairs = reinterpret_cast<const unsigned long long*>(cache.candidates.pairs);
+            fargs.candidate_shifts = reinterpret_cast<const int32_t*>(cache.candidates.shifts);
+            fargs.system_of_row = cache.system_of_row;
+            fargs.n_candidates = n_candidates;
+            fargs.n_chunks = n_chunks;
+            fargs.points = reinterpret_cast<const double*>(points);
+            fargs.first_point = cache.d_first_point;
+            fargs.limits = limits;
+            fargs.cutoff_sq = options.cutoff * options.cutoff;
+            fargs.chunk_rows = chunk_rows;
+            fargs.chunk_base = chunk_base;
+            fargs.out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
+            fargs.out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
+            fargs.out.distances = neighbors.distances;
+            fargs.out.vectors = reinterpret_cast<double*>(neighbors.vectors);
+            fargs.capacity = extras.capacity;
+            fargs.first_pair = d_first_pair;
+            fargs.n_systems = static_cast<uint32_t>(n_systems);
+            fargs.status = cache.status;
+            const size_t wanted = (n_chunks + VERLET_WAVES - 1) / VERLET_WAVES;
+            const unsigned blocks = static_cast<unsigned>(std::min<size_t>(wanted, 256 * 64));
+            hipLaunchKernelGGL(verlet_batch_filter_kernel<false>, dim3(blocks), dim3(VERLET_BLOCK), 0, stream, fargs);
+            exclusive_scan<SCAN_U32>(chunk_rows, n_chunks, chunk_base, scan_scratch, stream);
+            hipLaunchKernelGGL(verlet_batch_filter_kernel<true>, dim3(blocks), dim3(VERLET_BLOCK), 0, stream, fargs);
+            HIP_CHECK(hipMemcpyAsync(
+                cache.first_pair_landing.data(), d_first_pair, (n_systems + 1) * sizeof(size_t), hipMemcpyDeviceToHost, stream
+            ));
+        }
+        HIP_CHECK(hipStreamSynchronize(stream));
+        HIP_CHECK(hipGetLastError());
+
+        if (cache.status->rebuild != 0) {
+            if (fresh) {
+                throw std::runtime_error("internal error: fresh Verlet candidates of a batch do not cover their own points");
+            }
+            if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
+                std::fprintf(stderr, "batch with a skin: some system moved too far, the candidates are computed again\n");
+            }
+            rebuild();
+            continue;
+        }
+        total = n_candidates > 0 ? cache.status->total_rows : 0;
+        if (pair_limit != 0 && total > n_points * pair_limit) {
+            throw std::runtime_error(
+                "The number of neighbor pairs exceeds the maximum capacity of " + std::to_string(n_points * pair_limit) +
+                " (max_pairs_per_point=" + std::to_string(pair_limit) + "; n_points=" + std::to_string(n_points) + "). " +
+                "Consider reducing the cutoff distance, or explicitly setting " +
+                "VESIN_CUDA_MAX_PAIRS_PER_POINT as an environment variable."
+            );
+        }
+        if (total > extras.capacity) {
+            size_outputs(neighbors, extras, total, options);
+            continue;
+        }
+        break;
+    }
+    neighbors.length = total;
+    if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
+        std::fprintf(stderr, "batch with a skin: %zu rows filtered from %zu candidates\n", total, n_candidates);
+    }
+    if (n_candidates > 0) {
+        std::memcpy(first_pair, cache.first_pair_landing.data(), (n_systems + 1) * sizeof(size_t));
+    } else {
+        std::fill(first_pair, first_pair + n_systems + 1, size_t(0));
+    }
+    if (too_long_for_a_filter(total)) {
+        cache.direct = true;
+        cache.direct_n_points = n_points;
+    }
+}
+
+} // namespace
 
 namespace {
 

@@ -275,6 +275,266 @@ __global__ __launch_bounds__(VERLET_BLOCK) void verlet_filter_kernel(VerletFilte
     }
 }
 
+// ---- batches of systems: one candidate list for the whole batch (the rows of a batch call at cutoff + skin, system
+// after system), filtered in two passes that keep the order of the candidates, so that the rows of a system stay
+// together (and sorted, when the candidates were). Every system has its own box, so every system has its own
+// limit on how far its points may have moved; one system past its limit and all candidates are computed again.
+
+/// What the candidates of one system were built from. The rows of directions that are not periodic are zero: no
+/// shift runs along them, and a system without any periodic direction has a box that is never read.
+struct BatchVerletReference {
+    double box[9];
+    unsigned char periodic[3];
+    unsigned char padding;
+    unsigned int largest_shift[3];
+};
+
+/// Per system and call: the box the filter uses (zero rows for directions that are not periodic) and how far a
+/// point may have moved, squared.
+struct BatchVerletLimits {
+    double H[9];
+    double threshold_sq;
+};
+
+__device__ __forceinline__ void masked_box(
+    const double* __restrict__ box, const bool* __restrict__ periodic, double* out, unsigned char* flags
+) {
+#pragma unroll
+    for (int d = 0; d < 3; d++) {
+        const bool p = periodic[d];
+        flags[d] = p ? 1 : 0;
+#pragma unroll
+        for (int k = 0; k < 3; k++) {
+            out[3 * d + k] = p ? box[3 * d + k] : 0.0;
+        }
+    }
+}
+
+__global__ __launch_bounds__(VERLET_BLOCK) void verlet_batch_store_reference(
+    const double* __restrict__ boxes, const bool* __restrict__ periodic, uint32_t n_systems,
+    BatchVerletReference* __restrict__ reference
+) {
+    const uint32_t s = blockIdx.x * VERLET_BLOCK + threadIdx.x;
+    if (s >= n_systems) {
+        return;
+    }
+    BatchVerletReference mine;
+    masked_box(boxes + 9 * static_cast<size_t>(s), periodic + 3 * static_cast<size_t>(s), mine.box, mine.periodic);
+    mine.padding = 0;
+    mine.largest_shift[0] = mine.largest_shift[1] = mine.largest_shift[2] = 0;
+    reference[s] = mine;
+}
+
+/// owner[item] = the system s with firsts[s] <= item < firsts[s + 1] (`firsts` has n_systems + 1 entries, starts at
+/// 0 and never decreases), for the points and for the candidate rows of a batch. With `shifts`, the items are the
+/// candidates, and the largest |S_d| of every system's candidates is noted as verlet_shift_reach_kernel does.
+__global__ __launch_bounds__(VERLET_BLOCK) void verlet_batch_owner_kernel(
+    const unsigned long long* __restrict__ firsts, uint32_t n_systems, size_t n_items, uint32_t* __restrict__ owner,
+    const int32_t* __restrict__ shifts, BatchVerletReference* __restrict__ reference
+) {
+    const size_t stride = static_cast<size_t>(gridDim.x) * VERLET_BLOCK;
+    for (size_t item = static_cast<size_t>(blockIdx.x) * VERLET_BLOCK + threadIdx.x; item < n_items; item += stride) {
+        uint32_t lo = 0;
+        uint32_t hi = n_systems;
+        while (hi - lo > 1) {
+            const uint32_t middle = lo + (hi - lo) / 2;
+            if (firsts[middle] <= item) {
+                lo = middle;
+            } else {
+                hi = middle;
+            }
+        }
+        owner[item] = lo;
+        if (shifts != nullptr) {
+#pragma unroll
+            for (int d = 0; d < 3; d++) {
+                const int32_t shift = shifts[3 * item + d];
+                const unsigned int reach = static_cast<unsigned int>(shift < 0 ? -shift : shift);
+                if (reach > 1) {
+                    atomicMax(&reference[lo].largest_shift[d], reach);
+                }
+            }
+        }
+    }
+}
+
+/// verlet_check_kernel's decision about the box, for every system of a batch. `status->rebuild` must be 0 at launch.
+__global__ __launch_bounds__(VERLET_BLOCK) void verlet_batch_limits_kernel(
+    const double* __restrict__ boxes, const bool* __restrict__ periodic, const BatchVerletReference* __restrict__ reference,
+    uint32_t n_systems, double skin, BatchVerletLimits* __restrict__ limits, VerletStatus* __restrict__ status
+) {
+    const uint32_t s = blockIdx.x * VERLET_BLOCK + threadIdx.x;
+    if (s >= n_systems) {
+        return;
+    }
+    BatchVerletLimits mine;
+    unsigned char flags[3];
+    masked_box(boxes + 9 * static_cast<size_t>(s), periodic + 3 * static_cast<size_t>(s), mine.H, flags);
+    const BatchVerletReference then = reference[s];
+    bool too_far = false;
+    for (int d = 0; d < 3; d++) {
+        too_far = too_far || flags[d] != then.periodic[d];
+    }
+    const double half_skin = skin / 2.0;
+    const double half_skin_sq = half_skin * half_skin;
+    double half_displacement = corner_displacements(mine.H, then.box) / 2.0;
+    if (then.largest_shift[0] > 1 || then.largest_shift[1] > 1 || then.largest_shift[2] > 1) {
+        // candidates whose shifts reach further than one box: see verlet_check_kernel
+        double reach = 0.0;
+        for (int d = 0; d < 3; d++) {
+            double moved_sq = 0.0;
+            for (int k = 0; k < 3; k++) {
+                const double moved = mine.H[3 * d + k] - then.box[3 * d + k];
+                moved_sq += moved * moved;
+            }
+            reach += static_cast<double>(max(then.largest_shift[d], 1u)) * sqrt(moved_sq);
+        }
+        half_displacement = fmax(half_displacement, reach / 2.0);
+    }
+    // also true when a box row that is read holds a NaN
+    too_far = too_far || !(half_displacement * half_displacement <= half_skin_sq);
+    mine.threshold_sq = (sqrt(half_skin_sq) - half_displacement) * (sqrt(half_skin_sq) - half_displacement);
+    if (too_far) {
+        mine.threshold_sq = -1.0;
+        status->rebuild = 1;
+    }
+    limits[s] = mine;
+}
+
+__global__ __launch_bounds__(VERLET_BLOCK) void verlet_batch_moved_kernel(
+    const double* __restrict__ points, const double* __restrict__ ref_points, size_t n_points,
+    const uint32_t* __restrict__ system_of_point, const BatchVerletLimits* __restrict__ limits,
+    VerletStatus* __restrict__ status
+) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * VERLET_BLOCK + threadIdx.x;
+    if (i >= n_points) {
+        return;
+    }
+    const double dx = points[3 * i + 0] - ref_points[3 * i + 0];
+    const double dy = points[3 * i + 1] - ref_points[3 * i + 1];
+    const double dz = points[3 * i + 2] - ref_points[3 * i + 2];
+    const double moved_sq = dx * dx + dy * dy + dz * dz;
+    // (a NaN coordinate computes the candidates again too: the search then reports it the way it always does)
+    if (!(moved_sq <= limits[system_of_point[i]].threshold_sq)) {
+        status->rebuild = 1;
+    }
+}
+
+struct BatchVerletFilterArgs {
+    const unsigned long long* candidate_pairs; // [n_candidates][2], indices inside the row's system
+    const int32_t* candidate_shifts;           // [n_candidates][3]
+    const uint32_t* system_of_row;             // [n_candidates]
+    size_t n_candidates;
+    size_t n_chunks;                           // of VERLET_CHUNK candidates
+    const double* points;
+    const unsigned long long* first_point;     // [n_systems + 1]
+    const BatchVerletLimits* limits;
+    double cutoff_sq;
+    uint32_t* chunk_rows;                      // [n_chunks]: written by the counting pass
+    const uint64_t* chunk_base;                // [n_chunks + 1]: their exclusive scan, read by the writing pass
+    SearchOutputs out;
+    size_t capacity;                           // rows the output arrays hold: a longer list is not written at all
+    unsigned long long* first_pair;            // [n_systems + 1], filled by the writing pass
+    uint32_t n_systems;
+    VerletStatus* status;
+};
+
+/// One wave takes chunks of 512 candidates. Counting pass: the rows every chunk keeps. Writing pass (behind the scan
+/// of these counts): the same tests again, and every kept row goes where the kept rows before it end, so the rows
+/// keep the order of the candidates; the lane that holds the first candidate of a system also says where that
+/// system's rows begin.
+template <bool WRITE>
+__global__ __launch_bounds__(VERLET_BLOCK) void verlet_batch_filter_kernel(BatchVerletFilterArgs a) {
+    const uint32_t lane = static_cast<uint32_t>(lane_id());
+    const size_t wave = static_cast<size_t>(blockIdx.x) * VERLET_WAVES + threadIdx.x / WAVE;
+    const size_t n_waves = static_cast<size_t>(gridDim.x) * VERLET_WAVES;
+    unsigned long long total = 0;
+    if (WRITE) {
+        total = a.chunk_base[a.n_chunks];
+        if (blockIdx.x == 0 && threadIdx.x == 0) {
+            a.status->total_rows = total;
+        }
+    }
+    const bool fits = total <= a.capacity;
+
+    for (size_t chunk = wave; chunk < a.n_chunks; chunk += n_waves) {
+        const size_t first = chunk * VERLET_CHUNK;
+        uint64_t row = WRITE ? a.chunk_base[chunk] : 0;
+        uint32_t chunk_rows = 0;
+#pragma unroll
+        for (int k = 0; k < VERLET_DEPTH; k++) {
+            const size_t c = first + static_cast<size_t>(k) * WAVE + lane;
+            bool keep = false;
+            unsigned long long pi = 0, pj = 0;
+            int32_t sx = 0, sy = 0, sz = 0;
+            double vx = 0.0, vy = 0.0, vz = 0.0, dd = 0.0;
+            uint32_t system = 0;
+            if (c < a.n_candidates) {
+                system = a.system_of_row[c];
+                pi = a.candidate_pairs[2 * c + 0];
+                pj = a.candidate_pairs[2 * c + 1];
+                sx = a.candidate_shifts[3 * c + 0];
+                sy = a.candidate_shifts[3 * c + 1];
+                sz = a.candidate_shifts[3 * c + 2];
+                const double* H = a.limits[system].H;
+                const double tx = static_cast<double>(sx) * H[0] + static_cast<double>(sy) * H[3] + static_cast<double>(sz) * H[6];
+                const double ty = static_cast<double>(sx) * H[1] + static_cast<double>(sy) * H[4] + static_cast<double>(sz) * H[7];
+                const double tz = static_cast<double>(sx) * H[2] + static_cast<double>(sy) * H[5] + static_cast<double>(sz) * H[8];
+                const double* ri = a.points + 3 * (a.first_point[system] + pi);
+                const double* rj = a.points + 3 * (a.first_point[system] + pj);
+                vx = (rj[0] - ri[0]) + tx;
+                vy = (rj[1] - ri[1]) + ty;
+                vz = (rj[2] - ri[2]) + tz;
+                dd = vx * vx + vy * vy + vz * vz;
+                keep = dd < a.cutoff_sq;
+            }
+            const uint64_t mask = __ballot(keep);
+            if (WRITE) {
+                const uint64_t mine = row + __builtin_amdgcn_mbcnt_hi(
+                    static_cast<uint32_t>(mask >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0u)
+                );
+                if (c < a.n_candidates) {
+                    const uint32_t before = c == 0 ? 0xFFFFFFFFu : a.system_of_row[c - 1];
+                    if (before != system) {
+                        // (systems without candidates in between begin, and end, here as well)
+                        for (uint32_t s = before + 1; s != system + 1; s++) {
+                            a.first_pair[s] = mine;
+                        }
+                    }
+                    if (c == a.n_candidates - 1) {
+                        for (uint32_t s = system + 1; s <= a.n_systems; s++) {
+                            a.first_pair[s] = total;
+                        }
+                    }
+                }
+                if (keep && fits) {
+                    a.out.pairs[2 * mine + 0] = pi;
+                    a.out.pairs[2 * mine + 1] = pj;
+                    if (a.out.shifts != nullptr) {
+                        a.out.shifts[3 * mine + 0] = sx;
+                        a.out.shifts[3 * mine + 1] = sy;
+                        a.out.shifts[3 * mine + 2] = sz;
+                    }
+                    if (a.out.distances != nullptr) {
+                        a.out.distances[mine] = sqrt(dd);
+                    }
+                    if (a.out.vectors != nullptr) {
+                        a.out.vectors[3 * mine + 0] = vx;
+                        a.out.vectors[3 * mine + 1] = vy;
+                        a.out.vectors[3 * mine + 2] = vz;
+                    }
+                }
+                row += static_cast<uint64_t>(__popcll(mask));
+            } else {
+                chunk_rows += static_cast<uint32_t>(__popcll(mask));
+            }
+        }
+        if (!WRITE && lane == 0) {
+            a.chunk_rows[chunk] = chunk_rows;
+        }
+    }
+}
+
 __global__ void verlet_publish(const VerletWork* __restrict__ work, VerletStatus* __restrict__ status) {
     status->total_rows = work->total_rows;
 }
