@@ -228,3 +228,34 @@ def test_a_single_call_between_batches_with_a_skin():
         assert_same_list(got, oracle.neighbors(points, box, True, 2.5, True, False, "ijSdD"), what="single call")
     for _ in range(2):
         check(batch(calculator, all_points, all_boxes, flags), all_points, all_boxes, flags, 2.5, True, False, "batch again")
+
+
+def test_shifts_beyond_what_the_kept_candidates_can_hold(capfd, monkeypatch):
+    """The filter keeps a shift in 21 bits per direction. A point given more than a million boxes away from its
+    neighbours has larger ones: such a batch is searched directly on every call, with the same rows."""
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    rng = np.random.default_rng(31)
+    edge = 4.0
+    all_boxes = [edge * np.eye(3), edge * np.eye(3)]
+    flags = [(True,) * 3] * 2
+    base = [rng.random((20, 3)) * edge, rng.random((30, 3)) * edge]
+    reach = [np.zeros((20, 3)), np.zeros((30, 3))]
+    reach[1][7, 0] = float(2**20 + 5)
+    reach[1][9, 1] = -float(2**20 - 1)  # this one still fits
+    calculator = NeighborList(cutoff=2.0, full_list=True, skin=0.4)
+    for step in range(4):
+        all_points = [p + 0.01 * step + r * edge for p, r in zip(base, reach)]
+        capfd.readouterr()
+        lists = batch(calculator, all_points, all_boxes, flags)
+        assert "rows filtered from" not in capfd.readouterr().err
+        check(lists, all_points, all_boxes, flags, 2.0, True, False, f"step {step}")
+        assert np.abs(lists[1]["shifts"]).max() >= 2**20 + 4
+    # without that point the candidates are kept again, after a while
+    reach[1][7, 0] = 3.0
+    for step in range(24):
+        all_points = [p + 0.01 * step + r * edge for p, r in zip(base, reach)]
+        capfd.readouterr()
+        lists = batch(calculator, all_points, all_boxes, flags)
+        report = capfd.readouterr().err
+        check(lists, all_points, all_boxes, flags, 2.0, True, False, f"step {step} with all shifts in range")
+    assert "rows filtered from" in report

@@ -465,7 +465,7 @@ struct BatchVerletCache {
     double* ref_points = nullptr;
     BatchVerletReference* reference = nullptr;
     uint32_t* system_of_point = nullptr;
-    uint32_t* system_of_row = nullptr;
+    BatchVerletCandidate* packed = nullptr;   // the candidates as the filter reads them
     unsigned long long* d_first_point = nullptr;
     VerletStatus* status = nullptr;           // pinned
     PinnedVector<unsigned long long> first_pair_landing;
@@ -473,6 +473,7 @@ struct BatchVerletCache {
     bool valid = false;
     bool direct = false;                      // as in VerletCache
     size_t direct_n_points = 0;
+    int unpackable_rest = 0;                  // calls left before candidates are tried again after shifts they cannot hold
 
     BatchVerletCache() = default;
     BatchVerletCache(const BatchVerletCache&) = delete;
@@ -2705,16 +2706,17 @@ void direct_batch(
 }
 
 /// Candidates beyond which a batch is searched directly on every call (see VERLET_MAX_CANDIDATES): the filter of a
-/// batch reads 36 bytes per candidate and two points on top of writing the rows, in two passes, and takes 0.05 ms
-/// and 36 ns per thousand candidates (i j S d asked for, a fourth of the candidates beyond the cutoff). The direct
+/// batch reads 16 bytes per candidate and two points on top of writing the rows, in two passes, and takes 0.05 ms
+/// and 33 ns per thousand candidates (i j S d asked for, a fourth of the candidates beyond the cutoff). The direct
 /// search costs more per call and less per row. Measured, direct against filter, full lists with skin 0.5:
-/// 2,000 free molecules of 3 to 40 atoms (1.0 M rows) 0.162 / 0.095 ms; 100,000 of 3 to 8 atoms (2.8 M rows) 0.750 /
-/// 0.248 ms; 512 periodic cells of 64 atoms (3.6 M rows) 0.208 / 0.226 ms; 20,000 molecules of 3 to 40 atoms (10.2 M
-/// rows) 0.456 / 0.493 ms; 4,096 cells of 64 atoms (29 M rows) 0.818 / 1.337 ms. Sorted lists of systems of several
-/// cells are the exception: the search that writes them in order takes 0.809 ms for 1,000 cells of 200 atoms (9.5 M
-/// rows) and 2.71 ms for 4,000 of them, the filter of sorted candidates 0.503 and 1.83 ms.
+/// 2,000 free molecules of 3 to 40 atoms (1.0 M rows) 0.142 / 0.095 ms; 100,000 of 3 to 8 atoms (2.8 M rows) 0.734 /
+/// 0.234 ms; 512 periodic cells of 64 atoms (3.6 M rows) 0.201 / 0.193 ms; 20,000 molecules of 3 to 40 atoms (10.2 M
+/// rows) 0.445 / 0.460 ms; 4,096 cells of 64 atoms (29 M rows) 0.807 / 1.215 ms. Sorted lists of systems of several
+/// cells are the exception: the search that writes them in order takes 0.799 ms for 1,000 cells of 200 atoms (9.5 M
+/// rows) and 2.70 ms for 4,000 of them, the filter of sorted candidates 0.457 and 1.65 ms.
 constexpr size_t BATCH_VERLET_MAX_CANDIDATES = size_t(1) << 22;
 constexpr size_t BATCH_VERLET_MAX_CANDIDATES_SORTED_CELLS = size_t(1) << 26;
+constexpr int BATCH_VERLET_UNPACKABLE_REST = 16;
 
 /// options.skin > 0 for a batch: verlet_neighbors with one candidate list for all systems. The candidates are
 /// computed again as a whole when any system's points or box moved too far, when the division into systems or the
@@ -2765,7 +2767,7 @@ void verlet_batch(
             cache.ref_points = c.take<double>(3 * n_points);
             cache.reference = c.take<BatchVerletReference>(n_systems);
             cache.system_of_point = c.take<uint32_t>(n_points);
-            cache.system_of_row = c.take<uint32_t>(n_candidates);
+            cache.packed = c.take<BatchVerletCandidate>(n_candidates);
             cache.d_first_point = c.take<unsigned long long>(n_systems + 1);
             d_candidate_first = c.take<unsigned long long>(n_systems + 1);
         };
@@ -2795,23 +2797,28 @@ void verlet_batch(
             const uint32_t blocks = static_cast<uint32_t>(std::min<size_t>(4096, (n_points + VERLET_BLOCK - 1) / VERLET_BLOCK));
             hipLaunchKernelGGL(
                 verlet_batch_owner_kernel, dim3(blocks), dim3(VERLET_BLOCK), 0, stream, cache.d_first_point,
-                static_cast<uint32_t>(n_systems), n_points, cache.system_of_point, static_cast<const int32_t*>(nullptr),
-                cache.reference
+                static_cast<uint32_t>(n_systems), n_points, cache.system_of_point
             );
         }
+        cache.status->unusable = 0; // (pinned; raised by a shift that the candidates of the filter cannot hold)
         if (n_candidates > 0) {
             const uint32_t blocks = static_cast<uint32_t>(std::min<size_t>(4096, (n_candidates + VERLET_BLOCK - 1) / VERLET_BLOCK));
             hipLaunchKernelGGL(
-                verlet_batch_owner_kernel, dim3(blocks), dim3(VERLET_BLOCK), 0, stream, d_candidate_first,
-                static_cast<uint32_t>(n_systems), n_candidates, cache.system_of_row,
-                reinterpret_cast<const int32_t*>(cache.candidates.shifts), cache.reference
+                verlet_batch_pack_kernel, dim3(blocks), dim3(VERLET_BLOCK), 0, stream,
+                reinterpret_cast<const unsigned long long*>(cache.candidates.pairs),
+                reinterpret_cast<const int32_t*>(cache.candidates.shifts), n_candidates, d_candidate_first,
+                cache.d_first_point, static_cast<uint32_t>(n_systems), cache.packed, cache.reference,
+                &cache.status->unusable
             );
         }
         // the snapshot is complete before the call returns: the caller may change points and boxes right after
         HIP_CHECK(hipGetLastError());
         HIP_CHECK(hipStreamSynchronize(stream));
+        // (the rows the candidates were packed from stay where they are, although nothing reads them again: with
+        // arrays to allocate anew, a call that computes the candidates again took a third longer, 0.40 against 0.30 ms
+        // for 2,000 molecules and 1.58 against 1.16 ms for 100,000)
         cache.options = options;
-        cache.valid = true;
+        cache.valid = cache.status->unusable == 0;
         fresh = true;
     };
     const char* forced = std::getenv("VESIN_HIP_VERLET");
@@ -2838,11 +2845,21 @@ void verlet_batch(
         direct_batch(points, first_point, n_systems, boxes, periodic, plain, neighbors, first_pair, extras, stream);
         cache.direct = too_long_for_a_filter(neighbors.length);
         cache.direct_n_points = n_points;
+        if (cache.unpackable_rest > 0) {
+            cache.unpackable_rest -= 1;
+            cache.direct = true;
+        }
+        if (!cache.direct) {
+            rebuild();
+            if (!cache.valid) {
+                // shifts of a million boxes: such a batch is searched directly for a while
+                cache.direct = true;
+                cache.unpackable_rest = BATCH_VERLET_UNPACKABLE_REST;
+            }
+        }
         if (cache.direct) {
             cache.drop_candidates();
             cache.first_point.clear();
-        } else {
-            rebuild();
         }
         return;
     }
@@ -2882,7 +2899,7 @@ void verlet_batch(
         hipLaunchKernelGGL(
             verlet_batch_limits_kernel, dim3(system_blocks), dim3(VERLET_BLOCK), 0, stream,
             reinterpret_cast<const double*>(boxes), reinterpret_cast<const bool*>(periodic), cache.reference,
-            static_cast<uint32_t>(n_systems), options.skin, limits, cache.status
+            cache.d_first_point, static_cast<uint32_t>(n_systems), options.skin, limits, cache.status
         );
         if (n_points > 0) {
             const uint32_t blocks = static_cast<uint32_t>((n_points + VERLET_BLOCK - 1) / VERLET_BLOCK);
@@ -2894,13 +2911,11 @@ void verlet_batch(
         }
         if (n_candidates > 0) {
             BatchVerletFilterArgs fargs;
-            fargs.candidate_pairs = reinterpret_cast<const unsigned long long*>(cache.candidates.pairs);
-            fargs.candidate_shifts = reinterpret_cast<const int32_t*>(cache.candidates.shifts);
-            fargs.system_of_row = cache.system_of_row;
+            fargs.candidates = cache.packed;
+            fargs.system_of_point = cache.system_of_point;
             fargs.n_candidates = n_candidates;
             fargs.n_chunks = n_chunks;
             fargs.points = reinterpret_cast<const double*>(points);
-            fargs.first_point = cache.d_first_point;
             fargs.limits = limits;
             fargs.cutoff_sq = options.cutoff * options.cutoff;
             fargs.chunk_rows = chunk_rows;
@@ -2933,6 +2948,17 @@ void verlet_batch(
                 std::fprintf(stderr, "batch with a skin: some system moved too far, the candidates are computed again\n");
             }
             rebuild();
+            if (!cache.valid) {
+                cache.direct = true;
+                cache.unpackable_rest = BATCH_VERLET_UNPACKABLE_REST;
+                cache.direct_n_points = n_points;
+                cache.drop_candidates();
+                cache.first_point.clear();
+                VesinOptions plain = options;
+                plain.skin = 0.0;
+                direct_batch(points, first_point, n_systems, boxes, periodic, plain, neighbors, first_pair, extras, stream);
+                return;
+            }
             continue;
         }
         total = n_candidates > 0 ? cache.status->total_rows : 0;

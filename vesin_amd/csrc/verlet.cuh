@@ -33,7 +33,7 @@ struct VerletReference {
 /// Written by the kernels into pinned host memory, read by the host after the call's synchronisation.
 struct VerletStatus {
     uint32_t rebuild;              // some point, or the box, moved too far (or the periodicity changed)
-    uint32_t padding;
+    uint32_t unusable;             // (batches) some candidate has a shift that the filter's records cannot hold
     unsigned long long total_rows; // rows the filter kept (also when they did not fit the arrays)
 };
 
@@ -294,7 +294,21 @@ struct BatchVerletReference {
 struct BatchVerletLimits {
     double H[9];
     double threshold_sq;
+    unsigned long long first_point; // of the system, among the points of the batch
 };
+
+/// One candidate as the filter reads it: both points by their index in the batch and the shift, 16 bytes in place of
+/// the 40 of a row with its shift.
+struct BatchVerletCandidate {
+    uint32_t i;
+    uint32_t j;
+    uint64_t shift; // three fields of 21 bits, each shift plus 2^20
+};
+constexpr int32_t BATCH_VERLET_SHIFT_BIAS = 1 << 20;
+
+__device__ __forceinline__ int32_t unpack_candidate_shift(uint64_t packed, int direction) {
+    return static_cast<int32_t>((packed >> (21 * direction)) & 0x1FFFFFu) - BATCH_VERLET_SHIFT_BIAS;
+}
 
 __device__ __forceinline__ void masked_box(
     const double* __restrict__ box, const bool* __restrict__ periodic, double* out, unsigned char* flags
@@ -325,43 +339,70 @@ __global__ __launch_bounds__(VERLET_BLOCK) void verlet_batch_store_reference(
     reference[s] = mine;
 }
 
-/// owner[item] = the system s with firsts[s] <= item < firsts[s + 1] (`firsts` has n_systems + 1 entries, starts at
-/// 0 and never decreases), for the points and for the candidate rows of a batch. With `shifts`, the items are the
-/// candidates, and the largest |S_d| of every system's candidates is noted as verlet_shift_reach_kernel does.
+/// The system s with firsts[s] <= item < firsts[s + 1] (`firsts` has n_systems + 1 entries, starts at 0 and never
+/// decreases).
+__device__ __forceinline__ uint32_t system_holding(const unsigned long long* __restrict__ firsts, uint32_t n_systems, size_t item) {
+    uint32_t lo = 0;
+    uint32_t hi = n_systems;
+    while (hi - lo > 1) {
+        const uint32_t middle = lo + (hi - lo) / 2;
+        if (firsts[middle] <= item) {
+            lo = middle;
+        } else {
+            hi = middle;
+        }
+    }
+    return lo;
+}
+
 __global__ __launch_bounds__(VERLET_BLOCK) void verlet_batch_owner_kernel(
-    const unsigned long long* __restrict__ firsts, uint32_t n_systems, size_t n_items, uint32_t* __restrict__ owner,
-    const int32_t* __restrict__ shifts, BatchVerletReference* __restrict__ reference
+    const unsigned long long* __restrict__ first_point, uint32_t n_systems, size_t n_points,
+    uint32_t* __restrict__ system_of_point
 ) {
     const size_t stride = static_cast<size_t>(gridDim.x) * VERLET_BLOCK;
-    for (size_t item = static_cast<size_t>(blockIdx.x) * VERLET_BLOCK + threadIdx.x; item < n_items; item += stride) {
-        uint32_t lo = 0;
-        uint32_t hi = n_systems;
-        while (hi - lo > 1) {
-            const uint32_t middle = lo + (hi - lo) / 2;
-            if (firsts[middle] <= item) {
-                lo = middle;
-            } else {
-                hi = middle;
-            }
-        }
-        owner[item] = lo;
-        if (shifts != nullptr) {
+    for (size_t i = static_cast<size_t>(blockIdx.x) * VERLET_BLOCK + threadIdx.x; i < n_points; i += stride) {
+        system_of_point[i] = system_holding(first_point, n_systems, i);
+    }
+}
+
+/// The rows of the batch call at cutoff + skin become the candidates the filter reads, and the largest |S_d| of
+/// every system's candidates is noted as verlet_shift_reach_kernel does. A shift that does not fit its 21 bits
+/// raises `*out_of_range` (the candidates are of no use then).
+__global__ __launch_bounds__(VERLET_BLOCK) void verlet_batch_pack_kernel(
+    const unsigned long long* __restrict__ pairs, const int32_t* __restrict__ shifts, size_t n_candidates,
+    const unsigned long long* __restrict__ candidate_first_pair, const unsigned long long* __restrict__ first_point,
+    uint32_t n_systems, BatchVerletCandidate* __restrict__ candidates, BatchVerletReference* __restrict__ reference,
+    uint32_t* __restrict__ out_of_range
+) {
+    const size_t stride = static_cast<size_t>(gridDim.x) * VERLET_BLOCK;
+    for (size_t c = static_cast<size_t>(blockIdx.x) * VERLET_BLOCK + threadIdx.x; c < n_candidates; c += stride) {
+        const uint32_t system = system_holding(candidate_first_pair, n_systems, c);
+        const unsigned long long first = first_point[system];
+        BatchVerletCandidate packed;
+        packed.i = static_cast<uint32_t>(first + pairs[2 * c + 0]);
+        packed.j = static_cast<uint32_t>(first + pairs[2 * c + 1]);
+        packed.shift = 0;
 #pragma unroll
-            for (int d = 0; d < 3; d++) {
-                const int32_t shift = shifts[3 * item + d];
-                const unsigned int reach = static_cast<unsigned int>(shift < 0 ? -shift : shift);
-                if (reach > 1) {
-                    atomicMax(&reference[lo].largest_shift[d], reach);
-                }
+        for (int d = 0; d < 3; d++) {
+            const int32_t shift = shifts[3 * c + d];
+            const unsigned int reach = static_cast<unsigned int>(shift < 0 ? -shift : shift);
+            if (reach > 1) {
+                atomicMax(&reference[system].largest_shift[d], reach);
             }
+            if (reach >= static_cast<unsigned int>(BATCH_VERLET_SHIFT_BIAS)) {
+                *out_of_range = 1;
+            }
+            packed.shift |= static_cast<uint64_t>(static_cast<uint32_t>(shift + BATCH_VERLET_SHIFT_BIAS) & 0x1FFFFFu) << (21 * d);
         }
+        candidates[c] = packed;
     }
 }
 
 /// verlet_check_kernel's decision about the box, for every system of a batch. `status->rebuild` must be 0 at launch.
 __global__ __launch_bounds__(VERLET_BLOCK) void verlet_batch_limits_kernel(
     const double* __restrict__ boxes, const bool* __restrict__ periodic, const BatchVerletReference* __restrict__ reference,
-    uint32_t n_systems, double skin, BatchVerletLimits* __restrict__ limits, VerletStatus* __restrict__ status
+    const unsigned long long* __restrict__ first_point, uint32_t n_systems, double skin,
+    BatchVerletLimits* __restrict__ limits, VerletStatus* __restrict__ status
 ) {
     const uint32_t s = blockIdx.x * VERLET_BLOCK + threadIdx.x;
     if (s >= n_systems) {
@@ -398,6 +439,7 @@ __global__ __launch_bounds__(VERLET_BLOCK) void verlet_batch_limits_kernel(
         mine.threshold_sq = -1.0;
         status->rebuild = 1;
     }
+    mine.first_point = first_point[s];
     limits[s] = mine;
 }
 
@@ -421,18 +463,16 @@ __global__ __launch_bounds__(VERLET_BLOCK) void verlet_batch_moved_kernel(
 }
 
 struct BatchVerletFilterArgs {
-    const unsigned long long* candidate_pairs; // [n_candidates][2], indices inside the row's system
-    const int32_t* candidate_shifts;           // [n_candidates][3]
-    const uint32_t* system_of_row;             // [n_candidates]
+    const BatchVerletCandidate* candidates;    // [n_candidates]
+    const uint32_t* system_of_point;           // [n_points]
     size_t n_candidates;
     size_t n_chunks;                           // of VERLET_CHUNK candidates
     const double* points;
-    const unsigned long long* first_point;     // [n_systems + 1]
     const BatchVerletLimits* limits;
     double cutoff_sq;
     uint32_t* chunk_rows;                      // [n_chunks]: written by the counting pass
     const uint64_t* chunk_base;                // [n_chunks + 1]: their exclusive scan, read by the writing pass
-    SearchOutputs out;
+    SearchOutputs out;                         // pairs with indices inside the row's system
     size_t capacity;                           // rows the output arrays hold: a longer list is not written at all
     unsigned long long* first_pair;            // [n_systems + 1], filled by the writing pass
     uint32_t n_systems;
@@ -465,23 +505,27 @@ __global__ __launch_bounds__(VERLET_BLOCK) void verlet_batch_filter_kernel(Batch
         for (int k = 0; k < VERLET_DEPTH; k++) {
             const size_t c = first + static_cast<size_t>(k) * WAVE + lane;
             bool keep = false;
-            unsigned long long pi = 0, pj = 0;
+            uint32_t gi = 0, gj = 0;
             int32_t sx = 0, sy = 0, sz = 0;
             double vx = 0.0, vy = 0.0, vz = 0.0, dd = 0.0;
             uint32_t system = 0;
+            unsigned long long first_point = 0;
             if (c < a.n_candidates) {
-                system = a.system_of_row[c];
-                pi = a.candidate_pairs[2 * c + 0];
-                pj = a.candidate_pairs[2 * c + 1];
-                sx = a.candidate_shifts[3 * c + 0];
-                sy = a.candidate_shifts[3 * c + 1];
-                sz = a.candidate_shifts[3 * c + 2];
-                const double* H = a.limits[system].H;
+                const BatchVerletCandidate candidate = a.candidates[c];
+                gi = candidate.i;
+                gj = candidate.j;
+                sx = unpack_candidate_shift(candidate.shift, 0);
+                sy = unpack_candidate_shift(candidate.shift, 1);
+                sz = unpack_candidate_shift(candidate.shift, 2);
+                system = a.system_of_point[gi];
+                const BatchVerletLimits* of_system = a.limits + system;
+                const double* H = of_system->H;
+                first_point = of_system->first_point;
                 const double tx = static_cast<double>(sx) * H[0] + static_cast<double>(sy) * H[3] + static_cast<double>(sz) * H[6];
                 const double ty = static_cast<double>(sx) * H[1] + static_cast<double>(sy) * H[4] + static_cast<double>(sz) * H[7];
                 const double tz = static_cast<double>(sx) * H[2] + static_cast<double>(sy) * H[5] + static_cast<double>(sz) * H[8];
-                const double* ri = a.points + 3 * (a.first_point[system] + pi);
-                const double* rj = a.points + 3 * (a.first_point[system] + pj);
+                const double* ri = a.points + 3 * static_cast<size_t>(gi);
+                const double* rj = a.points + 3 * static_cast<size_t>(gj);
                 vx = (rj[0] - ri[0]) + tx;
                 vy = (rj[1] - ri[1]) + ty;
                 vz = (rj[2] - ri[2]) + tz;
@@ -493,8 +537,12 @@ __global__ __launch_bounds__(VERLET_BLOCK) void verlet_batch_filter_kernel(Batch
                 const uint64_t mine = row + __builtin_amdgcn_mbcnt_hi(
                     static_cast<uint32_t>(mask >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0u)
                 );
+                // the system of the candidate before this one: the lane below holds it, or memory does
+                uint32_t before = static_cast<uint32_t>(__shfl_up(static_cast<int>(system), 1, WAVE));
                 if (c < a.n_candidates) {
-                    const uint32_t before = c == 0 ? 0xFFFFFFFFu : a.system_of_row[c - 1];
+                    if (lane == 0) {
+                        before = c == 0 ? 0xFFFFFFFFu : a.system_of_point[a.candidates[c - 1].i];
+                    }
                     if (before != system) {
                         // (systems without candidates in between begin, and end, here as well)
                         for (uint32_t s = before + 1; s != system + 1; s++) {
@@ -508,8 +556,8 @@ __global__ __launch_bounds__(VERLET_BLOCK) void verlet_batch_filter_kernel(Batch
                     }
                 }
                 if (keep && fits) {
-                    a.out.pairs[2 * mine + 0] = pi;
-                    a.out.pairs[2 * mine + 1] = pj;
+                    a.out.pairs[2 * mine + 0] = gi - first_point;
+                    a.out.pairs[2 * mine + 1] = gj - first_point;
                     if (a.out.shifts != nullptr) {
                         a.out.shifts[3 * mine + 0] = sx;
                         a.out.shifts[3 * mine + 1] = sy;
