@@ -259,3 +259,49 @@ def test_shifts_beyond_what_the_kept_candidates_can_hold(capfd, monkeypatch):
         report = capfd.readouterr().err
         check(lists, all_points, all_boxes, flags, 2.0, True, False, f"step {step} with all shifts in range")
     assert "rows filtered from" in report
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_sequences_of_batches_with_a_skin(seed):
+    """Random batches (sizes, shapes, flags, points given boxes away) through random sequences of small moves, box
+    changes, unchanged calls and new batches on one list: every call has the rows of a direct calculation."""
+    rng = np.random.default_rng(770_000 + seed)
+    cutoff = float(rng.choice([1.5, 2.5, 3.5]))
+    skin = float(rng.choice([0.1, 0.4, 1.0]))
+    full = bool(rng.integers(0, 2))
+    is_sorted = bool(rng.integers(0, 2))
+    calculator = NeighborList(cutoff=cutoff, full_list=full, sorted=is_sorted, skin=skin)
+
+    def new_batch():
+        n_systems = int(rng.choice([1, 2, 5, 30, 120]))
+        all_points, all_boxes, all_flags, all_reach = [], [], [], []
+        for _ in range(n_systems):
+            n = int(rng.choice([0, 1, 2, 7, 40, 150, 400], p=[0.05, 0.05, 0.1, 0.3, 0.3, 0.15, 0.05]))
+            if rng.random() < 0.5:
+                flags = tuple(bool(x) for x in rng.integers(0, 2, size=3))
+            else:
+                flags = (True,) * 3 if rng.random() < 0.6 else (False,) * 3
+            edge = float(rng.choice([2.0, 5.0, 9.0])) * (1 + rng.random())
+            box = np.eye(3) * edge + 0.2 * edge * rng.normal(size=(3, 3)) * (rng.random() < 0.5)
+            reach = np.zeros((n, 3))
+            if rng.random() < 0.2:
+                reach = rng.integers(-3, 4, size=(n, 3)).astype(np.float64) * np.array(flags, dtype=np.float64)
+            all_points.append(rng.random((n, 3)) @ box)
+            all_boxes.append(box)
+            all_flags.append(flags)
+            all_reach.append(reach)
+        return all_points, all_boxes, all_flags, all_reach
+
+    all_points, all_boxes, flags, reach = new_batch()
+    for step in range(6):
+        kind = rng.random()
+        if step > 0 and kind < 0.6:
+            amplitude = skin * float(rng.choice([0.02, 0.1, 0.3]))
+            all_points = [p + amplitude * rng.normal(size=p.shape) for p in all_points]
+        elif step > 0 and kind < 0.8:
+            all_boxes = [b * (1 + 0.01 * skin * rng.normal()) for b in all_boxes]
+        elif step > 0 and kind < 0.9:
+            all_points, all_boxes, flags, reach = new_batch()
+        given = [p + r @ b for p, r, b in zip(all_points, reach, all_boxes)]
+        lists = batch(calculator, given, all_boxes, flags)
+        check(lists, given, all_boxes, flags, cutoff, full, is_sorted, f"seed {seed}, step {step}")
