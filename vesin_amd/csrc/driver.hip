@@ -347,10 +347,13 @@ struct Carver {
 constexpr int EXTENT_REST = 8;
 
 /// Candidates beyond which a cached list is not worth filtering: the direct search writes its rows at more than
-/// half the memory bandwidth, and a filter has to read every candidate on top of writing the same rows. Measured
-/// on jittered diamond (cutoff 5, skin 0.5): the filter takes 0.038 ms against 0.077 ms at 0.2 M candidates,
-/// breaks even near 1.6 M and takes twice the direct search's time at 15 M.
-constexpr size_t VERLET_MAX_CANDIDATES = size_t(1) << 20;
+/// half the memory bandwidth, and a filter has to read every candidate, twice, on top of writing the same rows.
+/// Measured on jittered diamond (cutoff 5, skin 0.5, i j S d), filter against direct search: 0.2 M candidates 0.055 /
+/// 0.074 ms, 1.6 M 0.074 / 0.102 ms, 5.5 M 0.212 / 0.167 ms, 13 M 0.430 / 0.272 ms. A sorted list costs the direct
+/// search more and the filter nothing (sorted candidates stay sorted): 1.6 M candidates 0.072 / 0.162 ms, 5.5 M
+/// 0.213 / 0.274 ms, 13 M 0.433 / 0.424 ms, 31 M 0.973 / 0.854 ms.
+constexpr size_t VERLET_MAX_CANDIDATES = size_t(1) << 21;
+constexpr size_t VERLET_MAX_CANDIDATES_SORTED = size_t(1) << 23;
 
 /// One-pass cell build: slots per cell (one tile: with two the search has as many empty tiles as full ones and
 /// loses more than the build gains) and the mean occupations between which it is tried. A cell that overflows voids
@@ -386,7 +389,6 @@ struct VerletCache {
     size_t ref_capacity = 0;
     size_t n_ref = 0;
     VerletReference* reference = nullptr; // device: box and periodicity of that call
-    VerletWork* work = nullptr;           // device
     VerletStatus* status = nullptr;       // pinned
     VesinOptions options = {};
     bool valid = false;
@@ -408,9 +410,6 @@ struct VerletCache {
         }
         if (reference != nullptr) {
             (void)hipFree(reference);
-        }
-        if (work != nullptr) {
-            (void)hipFree(work);
         }
         if (status != nullptr) {
             (void)hipHostFree(status);
@@ -2327,9 +2326,11 @@ bool compute(
 namespace {
 
 /// options.skin > 0: filter the cached candidates, after rebuilding them when they no longer cover the points
-/// (reference: vesin/src/cpu_cell_list.cpp:222-234, vesin/src/verlet.cpp). In the steady state a call is three
-/// launches (check, filter, publish) and one synchronisation; the filter writes straight into the arrays the list
-/// kept, and is repeated when they turn out too small or when the check asks for new candidates.
+/// (reference: vesin/src/cpu_cell_list.cpp:222-234, vesin/src/verlet.cpp). In the steady state a call is two
+/// launches (the check together with the filter's counting pass; the writing pass), with a scan of the counts
+/// between them for lists of more than 0.5 M candidates, and one synchronisation; the filter writes straight into the arrays the list kept, and is
+/// repeated when they turn out too small or when the check asks for new candidates. Sorted lists come from sorted
+/// candidates: the filter keeps their order.
 void verlet_neighbors(
     const double (*points)[3], size_t n_points, const double box[3][3], const bool periodic[3], VesinOptions options,
     VesinNeighborList& neighbors, HipExtras& extras, hipStream_t stream
@@ -2337,7 +2338,6 @@ void verlet_neighbors(
     if (extras.verlet == nullptr) {
         auto cache = std::make_unique<VerletCache>();
         HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&cache->reference), sizeof(VerletReference)));
-        HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&cache->work), sizeof(VerletWork)));
         HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&cache->status), sizeof(VerletStatus), hipHostMallocDefault));
         extras.verlet = cache.release();
     }
@@ -2346,14 +2346,14 @@ void verlet_neighbors(
 
     // same triggers as the reference (vesin/src/verlet.cpp:48-54, :65-71)
     const bool options_changed = cache.options.cutoff != options.cutoff || cache.options.skin != options.skin ||
-                                 cache.options.full != options.full;
+                                 cache.options.full != options.full || cache.options.sorted != options.sorted;
     bool fresh = false;
     auto rebuild = [&]() {
         cache.valid = false;
         VesinOptions build = {};
         build.cutoff = options.cutoff + options.skin;
         build.full = options.full;
-        build.sorted = false;
+        build.sorted = options.sorted; // sorted rows come from sorted candidates: the filter keeps their order
         build.algorithm = VesinCellList;
         build.n_threads = options.n_threads;
         build.return_shifts = true;
@@ -2384,7 +2384,7 @@ void verlet_neighbors(
         );
         if (cache.candidates.length > 0) {
             // (how far the shifts of the candidates reach: what the box may change by before they are computed again
-            // depends on it, see verlet_check_kernel)
+            // depends on it, see verlet_check_and_count_kernel)
             const uint32_t blocks = static_cast<uint32_t>(std::min<size_t>(1024, (cache.candidates.length + VERLET_BLOCK - 1) / VERLET_BLOCK));
             hipLaunchKernelGGL(
                 verlet_shift_reach_kernel, dim3(blocks), dim3(VERLET_BLOCK), 0, stream,
@@ -2406,7 +2406,8 @@ void verlet_neighbors(
     auto too_long_for_a_filter = [&](size_t rows) {
         const double ratio = (options.cutoff + options.skin) / options.cutoff;
         const double candidates = static_cast<double>(rows) * ratio * ratio * ratio;
-        return force_direct || (!force_cache && candidates > static_cast<double>(VERLET_MAX_CANDIDATES));
+        const size_t limit = options.sorted ? VERLET_MAX_CANDIDATES_SORTED : VERLET_MAX_CANDIDATES;
+        return force_direct || (!force_cache && candidates > static_cast<double>(limit));
     };
     if (options_changed || cache.direct_n_points != n_points) {
         cache.direct = false;
@@ -2432,56 +2433,64 @@ void verlet_neighbors(
         return;
     }
 
-    SortWorkspace sort_space = {};
-    sort_space.host_ranges = extras.mail->ranges;
-    sort_space.device_ranges = extras.mail_device->ranges;
     size_t total = 0;
-    bool through_scratch = options.sorted;
     for (int attempt = 0;; attempt++) {
         if (attempt > 4) {
             throw std::runtime_error("internal error: the Verlet filter did not settle");
         }
         const size_t n_candidates = cache.candidates.length;
+        size_outputs(neighbors, extras, 0, options);
         SearchOutputs out;
-        size_t capacity = 0;
-        if (through_scratch) {
-            // the rows are sorted afterwards: they go to scratch rows, of which there are at most as many as
-            // candidates
-            carve_sort_space(extras, std::max<size_t>(n_candidates, 1), options, out, sort_space);
-            capacity = n_candidates;
-        } else {
-            size_outputs(neighbors, extras, 0, options);
-            out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
-            out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
-            out.distances = neighbors.distances;
-            out.vectors = reinterpret_cast<double*>(neighbors.vectors);
-            capacity = extras.capacity;
-        }
+        out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
+        out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
+        out.distances = neighbors.distances;
+        out.vectors = reinterpret_cast<double*>(neighbors.vectors);
+        const size_t capacity = extras.capacity;
 
         cache.status->rebuild = 0;
         cache.status->total_rows = 0;
-        const unsigned check_blocks = static_cast<unsigned>(std::max<size_t>((n_points + VERLET_BLOCK - 1) / VERLET_BLOCK, 1));
+        const size_t check_blocks = std::max<size_t>((n_points + VERLET_BLOCK - 1) / VERLET_BLOCK, 1);
+        const size_t chunks = (n_candidates + VERLET_CHUNK - 1) / VERLET_CHUNK;
+        const size_t count_blocks = std::min<size_t>((chunks + VERLET_WAVES - 1) / VERLET_WAVES, 256 * 64);
+        const bool self_scan = chunks <= VERLET_SELF_SCAN_CHUNKS;
+
+        VerletFilterArgs fargs;
+        fargs.candidate_pairs = reinterpret_cast<const unsigned long long*>(cache.candidates.pairs);
+        fargs.candidate_shifts = reinterpret_cast<const int32_t*>(cache.candidates.shifts);
+        fargs.n_candidates = n_candidates;
+        fargs.n_chunks = chunks;
+        fargs.points = reinterpret_cast<const double*>(points);
+        fargs.box = reinterpret_cast<const double*>(box);
+        fargs.periodic = periodic;
+        fargs.cutoff_sq = options.cutoff * options.cutoff;
+        fargs.out = out;
+        fargs.capacity = capacity;
+        fargs.status = cache.status;
+        uint64_t* scan_scratch = nullptr;
+        auto carve = [&](Carver& c) {
+            fargs.chunk_rows = c.take<uint32_t>(chunks);
+            fargs.chunk_base = c.take<uint64_t>(self_scan ? 0 : chunks + 1);
+            scan_scratch = c.take<uint64_t>(self_scan ? 0 : scan_scratch_elements(chunks));
+        };
+        Carver measure(nullptr);
+        carve(measure);
+        extras.sort_work.reserve(measure.used);
+        Carver carver(extras.sort_work.ptr);
+        carve(carver);
+
+        // check and count, (scan,) write: the rows keep the order of the candidates
         hipLaunchKernelGGL(
-            verlet_check_kernel, dim3(check_blocks), dim3(VERLET_BLOCK), 0, stream,
-            reinterpret_cast<const double*>(points), cache.ref_points, n_points, reinterpret_cast<const double*>(box),
-            periodic, cache.reference, options.skin, cache.status, cache.work
+            verlet_check_and_count_kernel, dim3(static_cast<unsigned>(std::max(check_blocks, count_blocks))),
+            dim3(VERLET_BLOCK), 0, stream, cache.ref_points, n_points, cache.reference, options.skin, fargs
         );
         if (n_candidates > 0) {
-            VerletFilterArgs fargs;
-            fargs.candidate_pairs = reinterpret_cast<const unsigned long long*>(cache.candidates.pairs);
-            fargs.candidate_shifts = reinterpret_cast<const int32_t*>(cache.candidates.shifts);
-            fargs.n_candidates = n_candidates;
-            fargs.points = reinterpret_cast<const double*>(points);
-            fargs.work = cache.work;
-            fargs.cutoff_sq = options.cutoff * options.cutoff;
-            fargs.out = out;
-            fargs.capacity = capacity;
-            const size_t chunks = (n_candidates + VERLET_CHUNK - 1) / VERLET_CHUNK;
-            const size_t wanted = (chunks + VERLET_WAVES - 1) / VERLET_WAVES;
-            const unsigned blocks = static_cast<unsigned>(std::min<size_t>(wanted, 256 * 64));
-            hipLaunchKernelGGL(verlet_filter_kernel, dim3(blocks), dim3(VERLET_BLOCK), 0, stream, fargs);
+            if (self_scan) {
+                hipLaunchKernelGGL(verlet_write_kernel<true>, dim3(static_cast<unsigned>(count_blocks)), dim3(VERLET_BLOCK), 0, stream, fargs);
+            } else {
+                exclusive_scan<SCAN_U32>(fargs.chunk_rows, chunks, fargs.chunk_base, scan_scratch, stream);
+                hipLaunchKernelGGL(verlet_write_kernel<false>, dim3(static_cast<unsigned>(count_blocks)), dim3(VERLET_BLOCK), 0, stream, fargs);
+            }
         }
-        hipLaunchKernelGGL(verlet_publish, dim3(1), dim3(1), 0, stream, cache.work, cache.status);
         HIP_CHECK(hipStreamSynchronize(stream));
         HIP_CHECK(hipGetLastError());
 
@@ -2500,26 +2509,6 @@ void verlet_neighbors(
                 "Consider reducing the cutoff distance, or explicitly setting " +
                 "VESIN_CUDA_MAX_PAIRS_PER_POINT as an environment variable."
             );
-        }
-        if (through_scratch) {
-            size_outputs(neighbors, extras, total, options);
-            if (total <= 1) {
-                // nothing to sort: the one row is produced again, in place
-                if (total == 0) {
-                    break;
-                }
-                through_scratch = false;
-                continue;
-            }
-            SearchOutputs final_out;
-            final_out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
-            final_out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
-            final_out.distances = neighbors.distances;
-            final_out.vectors = reinterpret_cast<double*>(neighbors.vectors);
-            sort_pairs(out, final_out, total, n_points, sort_space, stream);
-            HIP_CHECK(hipStreamSynchronize(stream));
-            HIP_CHECK(hipGetLastError());
-            break;
         }
         if (total > extras.capacity) {
             size_outputs(neighbors, extras, total, options);

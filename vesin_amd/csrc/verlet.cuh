@@ -37,13 +37,6 @@ struct VerletStatus {
     unsigned long long total_rows; // rows the filter kept (also when they did not fit the arrays)
 };
 
-/// Work state of the filter in device memory.
-struct VerletWork {
-    unsigned long long total_rows;
-    unsigned long long padding;
-    double H[9]; // box of this call; rows of non-periodic directions are zero (their shifts are)
-};
-
 __global__ void verlet_store_reference(
     const double* __restrict__ box, const bool* __restrict__ periodic, VerletReference* __restrict__ reference
 ) {
@@ -59,7 +52,7 @@ __global__ void verlet_store_reference(
 
 /// The largest |S_d| among the candidates, per direction (launched behind verlet_store_reference). Points given far
 /// outside of the box make pairs with shifts of several boxes, and how far the image of such a pair moves when the
-/// box changes grows with the shift: see verlet_check_kernel.
+/// box changes grows with the shift: see verlet_check_and_count_kernel.
 __global__ __launch_bounds__(VERLET_BLOCK) void verlet_shift_reach_kernel(
     const int32_t* __restrict__ candidate_shifts, size_t n_candidates, VerletReference* __restrict__ reference
 ) {
@@ -109,168 +102,212 @@ __device__ inline double corner_displacements(const double* box, const double* r
     return sqrt(largest) + sqrt(second);
 }
 
-/// Decides whether the candidates still cover this call (vesin/src/verlet.cpp:60-110) and prepares the filter:
-/// the box of this call and a zeroed row counter. `status->rebuild` must be 0 at launch.
-__global__ __launch_bounds__(VERLET_BLOCK) void verlet_check_kernel(
-    const double* __restrict__ points, const double* __restrict__ ref_points, size_t n_points,
-    const double* __restrict__ box, const bool* __restrict__ periodic, const VerletReference* __restrict__ reference,
-    double skin, VerletStatus* __restrict__ status, VerletWork* __restrict__ work
-) {
-    __shared__ double threshold_sq;
-    __shared__ uint32_t box_moved_too_far;
-    if (threadIdx.x == 0) {
-        bool too_far = false;
-        for (int d = 0; d < 3; d++) {
-            too_far = too_far || ((periodic[d] ? 1 : 0) != reference->periodic[d]);
-        }
-        const double half_skin = skin / 2.0;
-        const double half_skin_sq = half_skin * half_skin;
-        double half_displacement = corner_displacements(box, reference->box) / 2.0;
-        // The reference's bound covers the images one box away: the image of a pair with shift S moves by S . (H -
-        // H_ref) when the box changes, and for |S_d| <= 1 that is at most the two largest corner displacements. Points
-        // given several boxes outside of the box make pairs with larger shifts, whose images move further: for them
-        // the bound is sum_d max|S_d| x |H_d - H_ref_d| (never smaller than needed: more rebuilds, never a missed
-        // pair). Nothing changes while the box stays as it is, or while no candidate has such a shift.
-        if (reference->largest_shift[0] > 1 || reference->largest_shift[1] > 1 || reference->largest_shift[2] > 1) {
-            double reach = 0.0;
-            for (int d = 0; d < 3; d++) {
-                double moved_sq = 0.0;
-                for (int k = 0; k < 3; k++) {
-                    const double moved = box[3 * d + k] - reference->box[3 * d + k];
-                    moved_sq += moved * moved;
-                }
-                reach += static_cast<double>(max(reference->largest_shift[d], 1u)) * sqrt(moved_sq);
-            }
-            half_displacement = fmax(half_displacement, reach / 2.0);
-        }
-        // also true when the box holds a NaN
-        too_far = too_far || !(half_displacement * half_displacement <= half_skin_sq);
-        threshold_sq = (sqrt(half_skin_sq) - half_displacement) * (sqrt(half_skin_sq) - half_displacement);
-        box_moved_too_far = too_far ? 1 : 0;
-        if (blockIdx.x == 0) {
-            if (too_far) {
-                status->rebuild = 1;
-            }
-            work->total_rows = 0;
-            for (int d = 0; d < 3; d++) {
-                for (int k = 0; k < 3; k++) {
-                    work->H[3 * d + k] = periodic[d] ? box[3 * d + k] : 0.0;
-                }
-            }
-        }
-    }
-    __syncthreads();
-    if (box_moved_too_far != 0) {
-        return;
-    }
-    const size_t i = static_cast<size_t>(blockIdx.x) * VERLET_BLOCK + threadIdx.x;
-    if (i < n_points) {
-        const double dx = points[3 * i + 0] - ref_points[3 * i + 0];
-        const double dy = points[3 * i + 1] - ref_points[3 * i + 1];
-        const double dz = points[3 * i + 2] - ref_points[3 * i + 2];
-        const double moved_sq = dx * dx + dy * dy + dz * dz;
-        // a NaN coordinate rebuilds too: the direct search then reports it the way it always does
-        if (!(moved_sq <= threshold_sq)) {
-            status->rebuild = 1;
-        }
-    }
-}
-
 struct VerletFilterArgs {
     const unsigned long long* candidate_pairs; // [n_candidates][2]
     const int32_t* candidate_shifts;           // [n_candidates][3]
     size_t n_candidates;
+    size_t n_chunks;       // of VERLET_CHUNK candidates
     const double* points;
-    VerletWork* work;
+    const double* box;     // of this call
+    const bool* periodic;
     double cutoff_sq;
+    uint32_t* chunk_rows;  // [n_chunks]: the rows every chunk keeps, written by the counting pass
+    uint64_t* chunk_base;  // [n_chunks + 1]: their exclusive scan, for lists of more than VERLET_SELF_SCAN_CHUNKS chunks
     SearchOutputs out;
-    size_t capacity; // rows the output arrays hold; a chunk that would pass it is counted but not written
+    size_t capacity;       // rows the output arrays hold: a longer list is not written at all
+    VerletStatus* status;  // pinned
 };
 
-/// One wave takes chunks of 512 candidates: tests them, takes room for the kept ones with one atomic, writes them.
-__global__ __launch_bounds__(VERLET_BLOCK) void verlet_filter_kernel(VerletFilterArgs a) {
+/// Lists of at most this many chunks (0.5 M candidates) go without a scan of their own: every wave of the writing
+/// pass adds up the counts before its chunk itself. (With 3,200 chunks that cost more than the scan's launch: 0.080
+/// against 0.073 ms per call.)
+constexpr size_t VERLET_SELF_SCAN_CHUNKS = 1024;
+
+/// The box as the filter uses it: rows of non-periodic directions are zero (their shifts are).
+__device__ __forceinline__ void filter_box(const double* __restrict__ box, const bool* __restrict__ periodic, double* H) {
+#pragma unroll
+    for (int d = 0; d < 3; d++) {
+        const bool p = periodic[d];
+#pragma unroll
+        for (int k = 0; k < 3; k++) {
+            H[3 * d + k] = p ? box[3 * d + k] : 0.0;
+        }
+    }
+}
+
+/// Tests the candidates of one chunk, 64 at a time; `visit(k, keep, mask, ...)` sees every group of 64 with the ballot
+/// of the kept ones. T = S . H, v = (r_j - r_i) + T, keep iff |v|^2 < cutoff^2: the arithmetic of the search.
+struct TestedCandidate {
+    unsigned long long i, j;
+    int32_t sx, sy, sz;
+    double vx, vy, vz, dd;
+    bool keep;
+};
+
+__device__ __forceinline__ TestedCandidate test_candidate(const VerletFilterArgs& a, const double* H, size_t c) {
+    TestedCandidate t = {};
+    if (c < a.n_candidates) {
+        t.i = a.candidate_pairs[2 * c + 0];
+        t.j = a.candidate_pairs[2 * c + 1];
+        t.sx = a.candidate_shifts[3 * c + 0];
+        t.sy = a.candidate_shifts[3 * c + 1];
+        t.sz = a.candidate_shifts[3 * c + 2];
+        const double tx = static_cast<double>(t.sx) * H[0] + static_cast<double>(t.sy) * H[3] + static_cast<double>(t.sz) * H[6];
+        const double ty = static_cast<double>(t.sx) * H[1] + static_cast<double>(t.sy) * H[4] + static_cast<double>(t.sz) * H[7];
+        const double tz = static_cast<double>(t.sx) * H[2] + static_cast<double>(t.sy) * H[5] + static_cast<double>(t.sz) * H[8];
+        t.vx = (a.points[3 * t.j + 0] - a.points[3 * t.i + 0]) + tx;
+        t.vy = (a.points[3 * t.j + 1] - a.points[3 * t.i + 1]) + ty;
+        t.vz = (a.points[3 * t.j + 2] - a.points[3 * t.i + 2]) + tz;
+        t.dd = t.vx * t.vx + t.vy * t.vy + t.vz * t.vz;
+        t.keep = t.dd < a.cutoff_sq;
+    }
+    return t;
+}
+
+/// First launch of a filtered call, two jobs. (1) Whether the candidates still cover this call
+/// (vesin/src/verlet.cpp:60-110): thread 0 of every workgroup with points evaluates the box, a thread per point how
+/// far it moved; `status->rebuild` must be 0 at launch. (2) The counting pass of the filter, in two passes that keep
+/// the order of the candidates (sorted candidates give sorted rows without a sort, and an unsorted list comes out
+/// the same way on every call): the rows every chunk of 512 candidates keeps. Neither waits for the other: when
+/// the check fails the counts are not used.
+__global__ __launch_bounds__(VERLET_BLOCK) void verlet_check_and_count_kernel(
+    const double* __restrict__ ref_points, size_t n_points, const VerletReference* __restrict__ reference, double skin,
+    VerletFilterArgs a
+) {
+    __shared__ double threshold_sq;
+    __shared__ uint32_t box_moved_too_far;
+    const size_t check_blocks = (n_points + VERLET_BLOCK - 1) / VERLET_BLOCK;
+    if (blockIdx.x < check_blocks || blockIdx.x == 0) {
+        if (threadIdx.x == 0) {
+            bool too_far = false;
+            for (int d = 0; d < 3; d++) {
+                too_far = too_far || ((a.periodic[d] ? 1 : 0) != reference->periodic[d]);
+            }
+            const double half_skin = skin / 2.0;
+            const double half_skin_sq = half_skin * half_skin;
+            double half_displacement = corner_displacements(a.box, reference->box) / 2.0;
+            // The reference's bound covers the images one box away: the image of a pair with shift S moves by S . (H -
+            // H_ref) when the box changes, and for |S_d| <= 1 that is at most the two largest corner displacements.
+            // Points given several boxes outside of the box make pairs with larger shifts, whose images move further:
+            // for them the bound is sum_d max|S_d| x |H_d - H_ref_d| (never smaller than needed: more rebuilds, never
+            // a missed pair). Nothing changes while the box stays as it is, or while no candidate has such a shift.
+            if (reference->largest_shift[0] > 1 || reference->largest_shift[1] > 1 || reference->largest_shift[2] > 1) {
+                double reach = 0.0;
+                for (int d = 0; d < 3; d++) {
+                    double moved_sq = 0.0;
+                    for (int k = 0; k < 3; k++) {
+                        const double moved = a.box[3 * d + k] - reference->box[3 * d + k];
+                        moved_sq += moved * moved;
+                    }
+                    reach += static_cast<double>(max(reference->largest_shift[d], 1u)) * sqrt(moved_sq);
+                }
+                half_displacement = fmax(half_displacement, reach / 2.0);
+            }
+            // also true when the box holds a NaN
+            too_far = too_far || !(half_displacement * half_displacement <= half_skin_sq);
+            threshold_sq = (sqrt(half_skin_sq) - half_displacement) * (sqrt(half_skin_sq) - half_displacement);
+            box_moved_too_far = too_far ? 1 : 0;
+            if (blockIdx.x == 0 && too_far) {
+                a.status->rebuild = 1;
+            }
+        }
+        __syncthreads();
+        const size_t i = static_cast<size_t>(blockIdx.x) * VERLET_BLOCK + threadIdx.x;
+        if (box_moved_too_far == 0 && i < n_points) {
+            const double dx = a.points[3 * i + 0] - ref_points[3 * i + 0];
+            const double dy = a.points[3 * i + 1] - ref_points[3 * i + 1];
+            const double dz = a.points[3 * i + 2] - ref_points[3 * i + 2];
+            const double moved_sq = dx * dx + dy * dy + dz * dz;
+            // a NaN coordinate rebuilds too: the direct search then reports it the way it always does
+            if (!(moved_sq <= threshold_sq)) {
+                a.status->rebuild = 1;
+            }
+        }
+    }
+
     const uint32_t lane = static_cast<uint32_t>(lane_id());
     const size_t wave = static_cast<size_t>(blockIdx.x) * VERLET_WAVES + threadIdx.x / WAVE;
     const size_t n_waves = static_cast<size_t>(gridDim.x) * VERLET_WAVES;
     double H[9];
-#pragma unroll
-    for (int k = 0; k < 9; k++) {
-        H[k] = a.work->H[k];
-    }
-
-    for (size_t first = wave * VERLET_CHUNK; first < a.n_candidates; first += n_waves * VERLET_CHUNK) {
-        unsigned long long pi[VERLET_DEPTH];
-        unsigned long long pj[VERLET_DEPTH];
-        int32_t sx[VERLET_DEPTH];
-        int32_t sy[VERLET_DEPTH];
-        int32_t sz[VERLET_DEPTH];
-        double vx[VERLET_DEPTH];
-        double vy[VERLET_DEPTH];
-        double vz[VERLET_DEPTH];
-        double dd[VERLET_DEPTH];
-        uint32_t kept = 0;
-        uint32_t before[VERLET_DEPTH];
-        uint32_t chunk_rows = 0;
+    filter_box(a.box, a.periodic, H);
+    for (size_t chunk = wave; chunk < a.n_chunks; chunk += n_waves) {
+        uint32_t kept_rows = 0;
 #pragma unroll
         for (int k = 0; k < VERLET_DEPTH; k++) {
-            const size_t c = first + static_cast<size_t>(k) * WAVE + lane;
-            bool keep = false;
-            if (c < a.n_candidates) {
-                pi[k] = a.candidate_pairs[2 * c + 0];
-                pj[k] = a.candidate_pairs[2 * c + 1];
-                sx[k] = a.candidate_shifts[3 * c + 0];
-                sy[k] = a.candidate_shifts[3 * c + 1];
-                sz[k] = a.candidate_shifts[3 * c + 2];
-                const double tx = static_cast<double>(sx[k]) * H[0] + static_cast<double>(sy[k]) * H[3] +
-                                  static_cast<double>(sz[k]) * H[6];
-                const double ty = static_cast<double>(sx[k]) * H[1] + static_cast<double>(sy[k]) * H[4] +
-                                  static_cast<double>(sz[k]) * H[7];
-                const double tz = static_cast<double>(sx[k]) * H[2] + static_cast<double>(sy[k]) * H[5] +
-                                  static_cast<double>(sz[k]) * H[8];
-                vx[k] = (a.points[3 * pj[k] + 0] - a.points[3 * pi[k] + 0]) + tx;
-                vy[k] = (a.points[3 * pj[k] + 1] - a.points[3 * pi[k] + 1]) + ty;
-                vz[k] = (a.points[3 * pj[k] + 2] - a.points[3 * pi[k] + 2]) + tz;
-                dd[k] = vx[k] * vx[k] + vy[k] * vy[k] + vz[k] * vz[k];
-                keep = dd[k] < a.cutoff_sq;
-            }
-            const uint64_t mask = __ballot(keep);
-            before[k] = chunk_rows + __builtin_amdgcn_mbcnt_hi(
-                static_cast<uint32_t>(mask >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0u)
-            );
-            chunk_rows += static_cast<uint32_t>(__popcll(mask));
-            kept |= (keep ? 1u : 0u) << k;
+            const TestedCandidate t = test_candidate(a, H, chunk * VERLET_CHUNK + static_cast<size_t>(k) * WAVE + lane);
+            kept_rows += static_cast<uint32_t>(__popcll(__ballot(t.keep)));
         }
-        if (chunk_rows == 0) {
-            continue;
-        }
-        unsigned long long base = 0;
         if (lane == 0) {
-            base = atomicAdd(&a.work->total_rows, static_cast<unsigned long long>(chunk_rows));
+            a.chunk_rows[chunk] = kept_rows;
         }
-        base = uniform(static_cast<uint64_t>(base));
-        if (base + chunk_rows > a.capacity) {
-            continue;
+    }
+}
+
+/// The writing pass: the same tests again, and every kept row goes where the kept rows before it end. Where these
+/// are comes from the scan of the counts (`chunk_base`), or with SELF_SCAN from the counts themselves. A list longer
+/// than `capacity` is not written at all; the total goes to `status` either way. (One pass that kept the tested
+/// candidates in registers and took room for a chunk's rows with an atomic was slower, 0.100 against 0.074 ms at
+/// 1.6 M candidates and 0.52 against 0.43 ms at 13 M.)
+template <bool SELF_SCAN>
+__global__ __launch_bounds__(VERLET_BLOCK) void verlet_write_kernel(VerletFilterArgs a) {
+    const uint32_t lane = static_cast<uint32_t>(lane_id());
+    const size_t wave = static_cast<size_t>(blockIdx.x) * VERLET_WAVES + threadIdx.x / WAVE;
+    const size_t n_waves = static_cast<size_t>(gridDim.x) * VERLET_WAVES;
+    double H[9];
+    filter_box(a.box, a.periodic, H);
+    unsigned long long total = 0;
+    unsigned long long before_mine = 0; // SELF_SCAN: the rows of the chunks before this wave's (it has one at most)
+    if (SELF_SCAN) {
+        unsigned long long all = 0;
+        unsigned long long before = 0;
+        for (size_t chunk = lane; chunk < a.n_chunks; chunk += WAVE) {
+            const unsigned long long rows = a.chunk_rows[chunk];
+            all += rows;
+            before += chunk < wave ? rows : 0;
         }
 #pragma unroll
+        for (int offset = WAVE / 2; offset > 0; offset >>= 1) {
+            all += __shfl_xor(all, offset, WAVE);
+            before += __shfl_xor(before, offset, WAVE);
+        }
+        total = all;
+        before_mine = before;
+    } else {
+        total = a.chunk_base[a.n_chunks];
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        a.status->total_rows = total;
+    }
+    if (total > a.capacity) {
+        return;
+    }
+    for (size_t chunk = wave; chunk < a.n_chunks; chunk += n_waves) {
+        uint64_t row = SELF_SCAN ? before_mine : a.chunk_base[chunk];
+#pragma unroll
         for (int k = 0; k < VERLET_DEPTH; k++) {
-            if ((kept >> k) & 1u) {
-                const size_t row = base + before[k];
-                a.out.pairs[2 * row + 0] = pi[k];
-                a.out.pairs[2 * row + 1] = pj[k];
+            const TestedCandidate t = test_candidate(a, H, chunk * VERLET_CHUNK + static_cast<size_t>(k) * WAVE + lane);
+            const uint64_t mask = __ballot(t.keep);
+            if (t.keep) {
+                const uint64_t mine = row + __builtin_amdgcn_mbcnt_hi(
+                    static_cast<uint32_t>(mask >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0u)
+                );
+                a.out.pairs[2 * mine + 0] = t.i;
+                a.out.pairs[2 * mine + 1] = t.j;
                 if (a.out.shifts != nullptr) {
-                    a.out.shifts[3 * row + 0] = sx[k];
-                    a.out.shifts[3 * row + 1] = sy[k];
-                    a.out.shifts[3 * row + 2] = sz[k];
+                    a.out.shifts[3 * mine + 0] = t.sx;
+                    a.out.shifts[3 * mine + 1] = t.sy;
+                    a.out.shifts[3 * mine + 2] = t.sz;
                 }
                 if (a.out.distances != nullptr) {
-                    a.out.distances[row] = sqrt(dd[k]);
+                    a.out.distances[mine] = sqrt(t.dd);
                 }
                 if (a.out.vectors != nullptr) {
-                    a.out.vectors[3 * row + 0] = vx[k];
-                    a.out.vectors[3 * row + 1] = vy[k];
-                    a.out.vectors[3 * row + 2] = vz[k];
+                    a.out.vectors[3 * mine + 0] = t.vx;
+                    a.out.vectors[3 * mine + 1] = t.vy;
+                    a.out.vectors[3 * mine + 2] = t.vz;
                 }
             }
+            row += static_cast<uint64_t>(__popcll(mask));
         }
     }
 }
@@ -398,7 +435,7 @@ __global__ __launch_bounds__(VERLET_BLOCK) void verlet_batch_pack_kernel(
     }
 }
 
-/// verlet_check_kernel's decision about the box, for every system of a batch. `status->rebuild` must be 0 at launch.
+/// verlet_check_and_count_kernel's decision about the box, for every system of a batch. `status->rebuild` must be 0 at launch.
 __global__ __launch_bounds__(VERLET_BLOCK) void verlet_batch_limits_kernel(
     const double* __restrict__ boxes, const bool* __restrict__ periodic, const BatchVerletReference* __restrict__ reference,
     const unsigned long long* __restrict__ first_point, uint32_t n_systems, double skin,
@@ -420,7 +457,7 @@ __global__ __launch_bounds__(VERLET_BLOCK) void verlet_batch_limits_kernel(
     const double half_skin_sq = half_skin * half_skin;
     double half_displacement = corner_displacements(mine.H, then.box) / 2.0;
     if (then.largest_shift[0] > 1 || then.largest_shift[1] > 1 || then.largest_shift[2] > 1) {
-        // candidates whose shifts reach further than one box: see verlet_check_kernel
+        // candidates whose shifts reach further than one box: see verlet_check_and_count_kernel
         double reach = 0.0;
         for (int d = 0; d < 3; d++) {
             double moved_sq = 0.0;
@@ -581,10 +618,6 @@ __global__ __launch_bounds__(VERLET_BLOCK) void verlet_batch_filter_kernel(Batch
             a.chunk_rows[chunk] = chunk_rows;
         }
     }
-}
-
-__global__ void verlet_publish(const VerletWork* __restrict__ work, VerletStatus* __restrict__ status) {
-    status->total_rows = work->total_rows;
 }
 
 } // namespace vesin_hip
