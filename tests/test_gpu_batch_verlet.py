@@ -305,3 +305,33 @@ def test_random_sequences_of_batches_with_a_skin(seed):
         given = [p + r @ b for p, r, b in zip(all_points, reach, all_boxes)]
         lists = batch(calculator, given, all_boxes, flags)
         check(lists, given, all_boxes, flags, cutoff, full, is_sorted, f"seed {seed}, step {step}")
+
+
+def test_errors_on_a_list_with_kept_candidates(monkeypatch):
+    """What a direct batch refuses, a batch with a skin refuses with the same message, also on a call that would
+    only have filtered; the list works again afterwards."""
+    rng = np.random.default_rng(37)
+    all_points, all_boxes, flags = mixed_systems(rng)
+    calculator = NeighborList(cutoff=2.5, full_list=True, skin=0.4)
+    for _ in range(2):
+        check(batch(calculator, all_points, all_boxes, flags), all_points, all_boxes, flags, 2.5, True, False, "before")
+
+    broken = [p.copy() for p in all_points]
+    broken[4][17, 2] = np.nan
+    with pytest.raises(RuntimeError, match="non-finite coordinate along axis 2"):
+        batch(calculator, broken, all_boxes, flags)
+    singular = [b.copy() for b in all_boxes]
+    singular[7][2] = singular[7][1]
+    with pytest.raises(RuntimeError, match="the box matrix is not invertible"):
+        batch(calculator, all_points, singular, flags)
+    for _ in range(2):
+        check(batch(calculator, all_points, all_boxes, flags), all_points, all_boxes, flags, 2.5, True, False, "after")
+
+    # the reference's limit on pairs per point applies to the filtered rows as to a direct search
+    total = sum(len(oracle.neighbors(p, b, list(f), 2.5, True, False, "ij")["pairs"]) for p, b, f in zip(all_points, all_boxes, flags))
+    n_points = sum(len(p) for p in all_points)
+    monkeypatch.setenv("VESIN_CUDA_MAX_PAIRS_PER_POINT", str(max(1, total // n_points - 1)))
+    with pytest.raises(RuntimeError, match="exceeds the maximum capacity"):
+        batch(calculator, all_points, all_boxes, flags)
+    monkeypatch.setenv("VESIN_CUDA_MAX_PAIRS_PER_POINT", str(total // n_points + 1))
+    check(batch(calculator, all_points, all_boxes, flags), all_points, all_boxes, flags, 2.5, True, False, "within the limit")
