@@ -167,8 +167,9 @@ int VESIN_API vesin_hip_neighbors_on_stream(
  *
  * Between the two calls the inputs (`points`, `box`, `periodic`) must stay as they are, `neighbors` must not be
  * passed to any other entry point (they refuse it; vesin_free completes the queued call first), and the values in
- * the struct are those of the call before. With options.skin > 0 the call is queued as far as the cache's own
- * bookkeeping allows, which is usually not at all. */
+ * the struct are those of the call before. With options.skin > 0 a call that only filters the kept candidates is
+ * queued whole (the word says pending when a point or the box turned out to have moved too far; collect then
+ * computes the candidates again). */
 #define VESIN_HIP_ROWS_PENDING (~0ull)
 
 int VESIN_API vesin_hip_neighbors_enqueue(

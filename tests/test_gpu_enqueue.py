@@ -192,6 +192,51 @@ def test_a_list_in_its_steady_state_is_queued_whole(cells, cutoff, full, sorted)
         lib.vesin_free(ctypes.byref(neighbors))
 
 
+@pytest.mark.parametrize("sorted", [False, True], ids=["unsorted", "sorted"])
+def test_a_list_with_a_skin_is_queued_whole_while_its_candidates_hold(sorted):
+    """options.skin > 0: a call that only filters the kept candidates is two launches, all queued; when a point has
+    moved too far the word stays pending and collect computes the candidates again."""
+    import torch
+
+    lib = get_library()
+    options = _options(5.0, True, sorted)
+    options.skin = 1.0
+    stream = torch.cuda.Stream()
+    neighbors = VesinNeighborList()
+    try:
+        inputs = _device(*configs.diamond(6, seed=60, sigma=0.02))
+        torch.cuda.synchronize()
+        for _ in range(2):
+            _blocking(lib, inputs, options, neighbors, stream.cuda_stream)  # the search and the candidates; a filter
+        room = neighbors.length
+        for step, sigma in enumerate([0.02, 0.02, 0.02, 0.6, 0.6]):
+            points, box, periodic = configs.diamond(6, seed=61 + (step if sigma < 0.1 else 3), sigma=sigma)
+            expected = oracle.neighbors(points, box, periodic, 5.0, True, sorted, "ijSdD")
+            inputs = _device(points, box, periodic)
+            torch.cuda.synchronize()
+            _busy(stream)
+            word = _enqueue(lib, inputs, options, neighbors, stream.cuda_stream)
+            queued = not stream.query()
+            with torch.cuda.stream(stream):
+                consumer = Consumer(neighbors, word, min(room, len(expected["pairs"])))
+            _collect(lib, neighbors)
+            assert queued, "the call waited for the stream instead of queueing its work"
+            stream.synchronize()
+            rows = _rows(neighbors)
+            assert_same_list(rows, expected, ordered=sorted, what=f"step {step}")
+            assert int(_view(word, (1,), "<i8", neighbors).item()) == neighbors.length
+            if step < 3 or step == 4:
+                # within the skin of the candidates (step 4: of the candidates that step 3 computed)
+                assert len(expected["pairs"]) <= room + room // 8
+                if len(expected["pairs"]) <= room:
+                    consumer.check(rows)
+            else:
+                consumer.saw_nothing()
+            room = max(room, neighbors.length)
+    finally:
+        lib.vesin_free(ctypes.byref(neighbors))
+
+
 def test_what_the_queued_part_cannot_finish_is_finished_by_collect():
     """The first call of a list (no arrays yet), rows that outgrow the arrays, and a box that is not the one of the
     call before: the consumer queued in between finds the word pending and touches nothing; after collect the list is

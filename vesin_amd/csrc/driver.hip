@@ -647,7 +647,9 @@ constexpr unsigned long long ROWS_PENDING = ~0ull;
 
 /// What tells, on the device, whether the kernels queued by a call left the complete list in the arrays.
 struct QueuedOutcome {
-    int kind;                          // 0: single-pass search, 1: small system in one launch, 2: in-order search
+    int kind;                          // 0: single-pass search, 1: small system in one launch, 2: in-order search,
+                                       // 3: kept candidates filtered (options.skin > 0)
+    const VerletStatus* filtered;      // (3) pinned host memory
     const FusedStatus* fused;          // (0)
     const DeviceStatus* build;         // (0, 2)
     const OrderedHostStatus* small;    // (1) what workgroup 0 of the launch reported
@@ -667,6 +669,14 @@ __global__ void publish_queued_length(
     QueuedOutcome outcome, const double* __restrict__ box, const bool* __restrict__ periodic, unsigned long long* word
 ) {
     if (threadIdx.x != 0 || blockIdx.x != 0) {
+        return;
+    }
+    if (outcome.kind == 3) {
+        // (the check that ran with the filter compared this call's box and points with those of the candidates)
+        const unsigned long long rows = outcome.filtered->total_rows;
+        const bool complete = outcome.filtered->rebuild == 0 && rows <= outcome.capacity &&
+                              (outcome.row_limit == 0 || rows <= outcome.row_limit);
+        *word = complete ? rows : ROWS_PENDING;
         return;
     }
     bool complete = true;
@@ -2491,7 +2501,14 @@ void verlet_neighbors(
                 hipLaunchKernelGGL(verlet_write_kernel<false>, dim3(static_cast<unsigned>(count_blocks)), dim3(VERLET_BLOCK), 0, stream, fargs);
             }
         }
-        HIP_CHECK(hipStreamSynchronize(stream));
+        // (a queued call stops here: what was launched above is all that a list in its steady state needs)
+        QueuedOutcome outcome = {};
+        outcome.kind = 3;
+        outcome.filtered = cache.status;
+        outcome.capacity = capacity;
+        outcome.row_limit = pair_limit != 0 ? n_points * pair_limit : 0;
+        const bool published_here = extras.publish_length(outcome, reinterpret_cast<const double*>(box), periodic, stream);
+        extras.wait(stream);
         HIP_CHECK(hipGetLastError());
 
         if (cache.status->rebuild != 0) {
@@ -2514,6 +2531,7 @@ void verlet_neighbors(
             size_outputs(neighbors, extras, total, options);
             continue;
         }
+        extras.queued_part_sufficed = published_here;
         break;
     }
     neighbors.length = total;
