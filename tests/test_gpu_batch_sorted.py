@@ -307,9 +307,16 @@ def test_batches_whose_systems_all_have_few_points(full, capfd, monkeypatch):
         assert len(lines) == 1 and lines[0].endswith(": used"), (call, lines)
     molecules = [(rng.normal(scale=1.5, size=(int(rng.integers(1, 33)), 3)) + rng.uniform(-40, 40, size=3), np.zeros((3, 3)),
                   (False, False, False)) for _ in range(203)]
+    # (batches of free molecules have kernels of their own from their second call on: here the general path is meant)
+    monkeypatch.setenv("VESIN_HIP_MOLECULES", "off")
     for call in range(3):
         _call_and_check(calculator, molecules, cutoff, full, "PSd", f"molecules, call {call}")
         lines = _in_order_lines(capfd)
         assert len(lines) == 1 and lines[0].endswith(": used"), (call, lines)
         assert ("grids picked on the device" in lines[0]) == (call >= 1), (call, lines)
         molecules = [(m[0] + rng.normal(scale=0.03, size=m[0].shape), m[1], m[2]) for m in molecules]
+    monkeypatch.delenv("VESIN_HIP_MOLECULES")
+    for call in range(2):
+        capfd.readouterr()
+        _call_and_check(calculator, molecules, cutoff, full, "PSd", f"molecules with their own kernels, call {call}")
+        assert "batch of free molecules" in capfd.readouterr().err

@@ -33,6 +33,7 @@
 #include "fused.cuh"
 #include "geometry.hpp"
 #include "images.cuh"
+#include "molecules.cuh"
 #include "ordered.cuh"
 #include "small.cuh"
 #include "policy.hpp"
@@ -558,6 +559,12 @@ struct BatchSetup {
     // where the first rows of the systems land before they are copied into the caller's array (pinned)
     size_t* first_pair_landing = nullptr;
     size_t first_pair_capacity = 0;
+    // batches of free molecules (molecules.cuh): work memory of their own (what the general path keeps in the list's
+    // work memory between calls stays as it is), the division into systems on the device, the kernels' report
+    DeviceBuffer molecule_work;
+    std::vector<size_t> molecule_first_point;
+    bool molecule_first_point_on_device = false;
+    MoleculeStatus* molecule_report = nullptr; // pinned
 };
 
 /// A call that stops where the host would wait for the GPU and goes on later (vesin_hip_neighbors_enqueue /
@@ -832,6 +839,10 @@ struct HipExtras {
         work.release();
         sort_work.release();
         batch.kept_boxes.release();
+        batch.molecule_work.release();
+        if (batch.molecule_report != nullptr) {
+            (void)hipHostFree(batch.molecule_report);
+        }
         if (batch.first_pair_landing != nullptr) {
             (void)hipHostFree(batch.first_pair_landing);
         }
@@ -2592,6 +2603,11 @@ void verlet_batch(
     HipExtras& extras, hipStream_t stream
 );
 
+bool molecules_batch(
+    const double (*points)[3], const size_t* first_point, size_t n_systems, const bool (*periodic)[3],
+    VesinOptions options, VesinNeighborList& neighbors, size_t* first_pair, HipExtras& extras, hipStream_t stream
+);
+
 } // namespace
 
 void neighbors_batch(
@@ -2667,6 +2683,20 @@ void direct_batch(
     const size_t n_points = first_point[n_systems];
     extras.guess.have_box = false; // the work buffers of the single-system path are about to be reused
 
+    // Free molecules of at most 64 points each, as the call before found them (same division into systems; that
+    // no system has a periodic direction is for the kernels to confirm): no cell lists, see molecules.cuh.
+    {
+        const BatchSetup& known = extras.batch;
+        const bool free_molecules =
+            known.valid && known.all_open && known.most_points <= MOLECULE_MAX_POINTS && n_points > 0 &&
+            options.algorithm != VesinCellList && !extras.fixed_memory && std::getenv("VESIN_HIP_MOLECULES") == nullptr &&
+            known.first_point.size() == n_systems + 1 &&
+            std::memcmp(known.first_point.data(), first_point, (n_systems + 1) * sizeof(size_t)) == 0;
+        if (free_molecules && molecules_batch(points, first_point, n_systems, periodic, options, neighbors, first_pair, extras, stream)) {
+            return;
+        }
+    }
+
     // The grids follow from the boxes, the flags, the division into systems, the cutoff and the algorithm alone,
     // unless some direction is open: then they also follow the points. Same inputs as the call before: same grids.
     // Whether the boxes and flags are the same is for the device to say, where they live: a call whose other inputs
@@ -2710,6 +2740,144 @@ void direct_batch(
     (void)batch_attempt(points, first_point, n_systems, boxes, periodic, options, neighbors, first_pair, extras, false, stream);
     setup.guess.have_box = setup.kept_on_device;
     setup.guess.stored(key);
+}
+
+/// A batch of free molecules through molecules_kernel: counting pass, scan over the systems, writing pass, one
+/// synchronisation. Returns false, with nothing of the result to be used, when some system turned out to have a
+/// periodic direction (the flags live on the device).
+bool molecules_batch(
+    const double (*points)[3], const size_t* first_point, size_t n_systems, const bool (*periodic)[3],
+    VesinOptions options, VesinNeighborList& neighbors, size_t* first_pair, HipExtras& extras, hipStream_t stream
+) {
+    const TraceRange whole_call("vesin_hip_neighbors_batch (free molecules)");
+    BatchSetup& setup = extras.batch;
+    const size_t n_points = first_point[n_systems];
+    const size_t pair_limit = pairs_per_point_limit();
+    if (setup.molecule_report == nullptr) {
+        HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&setup.molecule_report), sizeof(MoleculeStatus), hipHostMallocDefault));
+    }
+    if (setup.first_pair_capacity < n_systems + 1) {
+        if (setup.first_pair_landing != nullptr) {
+            (void)hipHostFree(setup.first_pair_landing);
+            setup.first_pair_landing = nullptr;
+            setup.first_pair_capacity = 0;
+        }
+        const size_t wanted = (n_systems + 1) + (n_systems + 1) / 4;
+        HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&setup.first_pair_landing), wanted * sizeof(size_t), hipHostMallocDefault));
+        setup.first_pair_capacity = wanted;
+    }
+
+    MoleculeArgs args = {};
+    uint32_t* d_first_point = nullptr;
+    uint64_t* d_first_pair = nullptr;
+    uint64_t* scan_scratch = nullptr;
+    auto carve = [&](Carver& c) {
+        d_first_point = c.take<uint32_t>(n_systems + 1);
+        args.status = c.take<MoleculeStatus>(1);
+        args.rows_of_system = c.take<uint32_t>(n_systems);
+        d_first_pair = c.take<uint64_t>(n_systems + 1);
+        scan_scratch = c.take<uint64_t>(scan_scratch_elements(n_systems));
+    };
+    Carver measure(nullptr);
+    carve(measure);
+    const uint64_t generation = setup.molecule_work.generation;
+    setup.molecule_work.reserve(measure.used);
+    Carver carver(setup.molecule_work.ptr);
+    carve(carver);
+    const bool same_division = setup.molecule_first_point_on_device && generation == setup.molecule_work.generation &&
+                               setup.molecule_first_point.size() == n_systems + 1 &&
+                               std::memcmp(setup.molecule_first_point.data(), first_point, (n_systems + 1) * sizeof(size_t)) == 0;
+    if (!same_division) {
+        setup.molecule_first_point_on_device = false;
+        setup.molecule_first_point.assign(first_point, first_point + n_systems + 1);
+        // (setup.first_point32 holds the same division, as the general path left it)
+        HIP_CHECK(hipMemcpyAsync(
+            d_first_point, setup.first_point32.data(), (n_systems + 1) * sizeof(uint32_t), hipMemcpyHostToDevice, stream
+        ));
+        setup.molecule_first_point_on_device = true;
+    }
+
+    args.points = reinterpret_cast<const double*>(points);
+    args.periodic = reinterpret_cast<const bool*>(periodic);
+    args.first_point = d_first_point;
+    args.n_systems = static_cast<uint32_t>(n_systems);
+    args.cutoff2 = options.cutoff * options.cutoff;
+    args.full = options.full ? 1 : 0;
+    args.first_pair = d_first_pair;
+    args.report = setup.molecule_report;
+
+    // lanes per system: the next power of two from the largest system on, eight at least
+    const int lanes = setup.most_points <= 8 ? 8 : setup.most_points <= 16 ? 16 : setup.most_points <= 32 ? 32 : 64;
+    const size_t per_block = static_cast<size_t>(MOLECULE_BLOCK / WAVE) * (WAVE / lanes);
+    const unsigned blocks = static_cast<unsigned>((n_systems + per_block - 1) / per_block);
+    auto launch = [&](bool write) {
+        const dim3 grid(blocks), block(MOLECULE_BLOCK);
+        switch (lanes * 2 + (write ? 1 : 0)) {
+        case 16: hipLaunchKernelGGL((molecules_kernel<8, false>), grid, block, 0, stream, args); break;
+        case 17: hipLaunchKernelGGL((molecules_kernel<8, true>), grid, block, 0, stream, args); break;
+        case 32: hipLaunchKernelGGL((molecules_kernel<16, false>), grid, block, 0, stream, args); break;
+        case 33: hipLaunchKernelGGL((molecules_kernel<16, true>), grid, block, 0, stream, args); break;
+        case 64: hipLaunchKernelGGL((molecules_kernel<32, false>), grid, block, 0, stream, args); break;
+        case 65: hipLaunchKernelGGL((molecules_kernel<32, true>), grid, block, 0, stream, args); break;
+        case 128: hipLaunchKernelGGL((molecules_kernel<64, false>), grid, block, 0, stream, args); break;
+        default: hipLaunchKernelGGL((molecules_kernel<64, true>), grid, block, 0, stream, args); break;
+        }
+    };
+
+    MoleculeStatus cleared = {};
+    cleared.first_bad = 0xFFFFFFFFu;
+    *setup.molecule_report = cleared;
+    HIP_CHECK(hipMemcpyAsync(args.status, setup.molecule_report, sizeof(MoleculeStatus), hipMemcpyHostToDevice, stream));
+    launch(false);
+    exclusive_scan<SCAN_U32>(args.rows_of_system, n_systems, d_first_pair, scan_scratch, stream);
+    size_t total = 0;
+    for (int attempt = 0;; attempt++) {
+        if (attempt > 2) {
+            throw std::runtime_error("internal error: the rows of a batch of molecules did not settle");
+        }
+        size_outputs(neighbors, extras, total, options);
+        args.out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
+        args.out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
+        args.out.distances = neighbors.distances;
+        args.out.vectors = reinterpret_cast<double*>(neighbors.vectors);
+        args.capacity = extras.capacity;
+        launch(true);
+        if (attempt == 0) {
+            HIP_CHECK(hipMemcpyAsync(
+                setup.first_pair_landing, d_first_pair, (n_systems + 1) * sizeof(size_t), hipMemcpyDeviceToHost, stream
+            ));
+        }
+        HIP_CHECK(hipStreamSynchronize(stream));
+        HIP_CHECK(hipGetLastError());
+        const MoleculeStatus found = *setup.molecule_report;
+        if (found.periodic != 0) {
+            if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
+                std::fprintf(stderr, "batch: free molecules no more, some system has a periodic direction now\n");
+            }
+            return false;
+        }
+        if (found.first_bad != 0xFFFFFFFFu) {
+            non_finite_error(points, found.first_bad);
+        }
+        total = found.total_rows;
+        if (pair_limit != 0 && total > n_points * pair_limit) {
+            throw std::runtime_error(
+                "The number of neighbor pairs exceeds the maximum capacity of " + std::to_string(n_points * pair_limit) +
+                " (max_pairs_per_point=" + std::to_string(pair_limit) + "; n_points=" + std::to_string(n_points) + "). " +
+                "Consider reducing the cutoff distance, or explicitly setting " +
+                "VESIN_CUDA_MAX_PAIRS_PER_POINT as an environment variable."
+            );
+        }
+        if (total <= extras.capacity) {
+            break;
+        }
+    }
+    neighbors.length = total;
+    std::memcpy(first_pair, setup.first_pair_landing, (n_systems + 1) * sizeof(size_t));
+    if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
+        std::fprintf(stderr, "batch of free molecules: %zu rows, %d lanes per system\n", total, lanes);
+    }
+    return true;
 }
 
 /// Candidates beyond which a batch is searched directly on every call (see VERLET_MAX_CANDIDATES): the filter of a
