@@ -72,6 +72,26 @@ def test_ase_wrapper_gives_the_full_list_ordered_by_i(with_ase, name):
     assert_same_list(actual, expected, what=name)
 
 
+@pytest.mark.gpu
+def test_ase_wrapper_keeps_its_calculators_and_hands_out_copies(with_ase):
+    """One calculator per (cutoff, device) serves all calls: systems of other sizes and shapes in turn, and the
+    arrays of an earlier call stay what they were."""
+    from vesin_amd import _ase
+
+    results = []
+    for name in ["diamond", "water", "diamond", "slab", "naphthalene", "water"]:
+        points, box, periodic = systems.read_xyz(name)
+        i, j, S, d = vesin_amd.ase_neighbor_list("ijSd", Atoms(points, box, periodic), cutoff=4.5)
+        expected = oracle.neighbors(points, box, periodic, 4.5, full=True, sorted=True)
+        results.append(((i, j, S, d), expected, name))
+    assert len([key for key in _ase._KEPT if key[0] == 4.5]) == 1
+    for (i, j, S, d), expected, name in results:
+        assert_same_list({"pairs": np.stack([i, j], axis=1), "shifts": S, "distances": d}, expected, what=name)
+    for cutoff in np.linspace(1.0, 2.0, 12):
+        vesin_amd.ase_neighbor_list("ij", Atoms(points, box, periodic), cutoff=float(cutoff))
+    assert len(_ase._KEPT) <= _ase._KEPT_MOST
+
+
 # ---------------------------------------------------------------------------------------------------------------
 # a device-array library with the surface of cupy that the adapter uses
 

