@@ -3572,7 +3572,6 @@ bool batch_attempt(
 
     // ---- cell lists of all systems, in one sequence of launches
     const uint32_t point_blocks = static_cast<uint32_t>((n_points + BLOCK - 1) / BLOCK);
-    const uint32_t bounding_blocks = std::min<uint32_t>(BOUNDING_BLOCKS, point_blocks);
     const auto* flat_points = reinterpret_cast<const double*>(points);
     {
         // one launch clears the histogram, the tiles' flags, the state of the single-pass search and the counts, and
