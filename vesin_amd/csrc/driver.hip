@@ -562,8 +562,8 @@ struct BatchSetup {
     // batches of free molecules (molecules.cuh): work memory of their own (what the general path keeps in the list's
     // work memory between calls stays as it is), the division into systems on the device, the kernels' report
     DeviceBuffer molecule_work;
-    std::vector<size_t> molecule_first_point;
-    bool molecule_first_point_on_device = false;
+    uint64_t division = 0;          // counts the divisions into systems this set-up has seen (`first_point` assigned)
+    uint64_t molecule_division = 0; // the one whose first points are in `molecule_work` (0: none)
     MoleculeStatus* molecule_report = nullptr; // pinned
 };
 
@@ -2784,17 +2784,13 @@ bool molecules_batch(
     setup.molecule_work.reserve(measure.used);
     Carver carver(setup.molecule_work.ptr);
     carve(carver);
-    const bool same_division = setup.molecule_first_point_on_device && generation == setup.molecule_work.generation &&
-                               setup.molecule_first_point.size() == n_systems + 1 &&
-                               std::memcmp(setup.molecule_first_point.data(), first_point, (n_systems + 1) * sizeof(size_t)) == 0;
-    if (!same_division) {
-        setup.molecule_first_point_on_device = false;
-        setup.molecule_first_point.assign(first_point, first_point + n_systems + 1);
-        // (setup.first_point32 holds the same division, as the general path left it)
+    // (the caller found this call's division to be the one of the set-up, whose 32-bit copy goes to the device once)
+    if (setup.molecule_division != setup.division || generation != setup.molecule_work.generation) {
+        setup.molecule_division = 0;
         HIP_CHECK(hipMemcpyAsync(
             d_first_point, setup.first_point32.data(), (n_systems + 1) * sizeof(uint32_t), hipMemcpyHostToDevice, stream
         ));
-        setup.molecule_first_point_on_device = true;
+        setup.molecule_division = setup.division;
     }
 
     args.points = reinterpret_cast<const double*>(points);
@@ -3225,6 +3221,7 @@ bool batch_attempt(
         setup.boxes.swap(setup.incoming_boxes);
         setup.periodic.swap(setup.incoming_periodic);
         setup.first_point.assign(first_point, first_point + n_systems + 1);
+        setup.division += 1;
         setup.cutoff = options.cutoff;
         setup.algorithm = static_cast<int>(options.algorithm);
         setup.full_stencil = full_stencil_only();
