@@ -1,4 +1,4 @@
-"""Batches of free molecules (no periodic direction, at most 64 points per system) have kernels of their own from the
+"""Batches of free molecules (no periodic direction, at most 256 points per system) have kernels of their own from the
 second call of a list on: no cell lists, every system's rows in (i, j) order. Per system the rows are those of a call
 on that system alone (``-m gpu``)."""
 
@@ -53,11 +53,11 @@ def random_molecules(rng, n_systems, most):
 
 @pytest.mark.parametrize("is_sorted", [False, True], ids=["unsorted", "sorted"])
 @pytest.mark.parametrize("full", [True, False], ids=["full", "half"])
-@pytest.mark.parametrize("most", [8, 16, 32, 64], ids=lambda m: f"up to {m} points")
+@pytest.mark.parametrize("most", [8, 16, 32, 64, 100, 256], ids=lambda m: f"up to {m} points")
 def test_molecules_of_every_size(most, full, is_sorted, capfd, monkeypatch):
     monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
     rng = np.random.default_rng(100 + most)
-    molecules = random_molecules(rng, 700, most)
+    molecules = random_molecules(rng, 700 if most <= 64 else 150, most)
     molecules[5] = np.zeros((0, 3))
     molecules[-1] = rng.normal(size=(most, 3))
     calculator = NeighborList(cutoff=2.4, full_list=full, sorted=is_sorted)
@@ -65,9 +65,11 @@ def test_molecules_of_every_size(most, full, is_sorted, capfd, monkeypatch):
         capfd.readouterr()
         lists = batch(calculator, molecules)
         report = capfd.readouterr().err
-        assert ("batch of free molecules" in report) == (call > 0), report
-        if call > 0:
-            assert f"{most} lanes per system" in report
+        # (with systems of more than 64 points, only sorted lists come from these kernels)
+        expected_here = call > 0 and (most <= 64 or is_sorted)
+        assert ("batch of free molecules" in report) == expected_here, report
+        if expected_here:
+            assert f"{most if most <= 64 else 256} lanes per system" in report
             check_in_order(lists, molecules, 2.4, full, f"call {call}")
         else:
             for s, rows in enumerate(lists):
@@ -96,7 +98,7 @@ def test_what_sends_a_batch_back_to_the_general_path(capfd, monkeypatch):
     rng = np.random.default_rng(11)
     molecules = random_molecules(rng, 120, 30)
     cutoff = 2.2
-    calculator = NeighborList(cutoff=cutoff, full_list=True)
+    calculator = NeighborList(cutoff=cutoff, full_list=True, sorted=True)
     for _ in range(2):
         lists = batch(calculator, molecules)
     check_in_order(lists, molecules, cutoff, True, "free molecules")
@@ -124,11 +126,11 @@ def test_what_sends_a_batch_back_to_the_general_path(capfd, monkeypatch):
         assert ("batch of free molecules" in capfd.readouterr().err) == (call == 1)
     check_in_order(lists, molecules, cutoff, True, "free again")
 
-    # another division into systems, one molecule of 65 atoms, a forced cell list: all through the general path
+    # another division into systems, one molecule of 257 atoms, a forced cell list: all through the general path
     other = random_molecules(rng, 90, 30)
-    big = other[:40] + [rng.normal(scale=2.0, size=(65, 3))] + other[40:]
+    big = other[:40] + [rng.normal(scale=3.0, size=(257, 3))] + other[40:]
     for molecules_now, options in ((other, {}), (big, {}), (other, {"algorithm": "cell_list"})):
-        calc = NeighborList(cutoff=cutoff, full_list=True, **options) if options else calculator
+        calc = NeighborList(cutoff=cutoff, full_list=True, sorted=True, **options) if options else calculator
         for call in range(2):
             capfd.readouterr()
             lists = batch(calc, molecules_now)
@@ -176,3 +178,18 @@ def test_a_hundred_thousand_tiny_molecules():
         expected = oracle.canonicalize(oracle.neighbors(molecules[s], np.zeros((3, 3)), [False] * 3, 5.0, True, False, "ijSd"))
         for key, value in lists[s].items():
             assert np.array_equal(value, expected[key]), (s, key)
+
+
+@pytest.mark.parametrize("full", [True, False], ids=["full", "half"])
+def test_molecules_of_very_different_sizes_in_one_batch(full):
+    """A few large molecules among many small ones in a sorted batch: every system gets a workgroup, most of whose
+    waves have no points."""
+    rng = np.random.default_rng(19)
+    molecules = random_molecules(rng, 400, 12)
+    for at, n in ((3, 256), (77, 65), (200, 129), (399, 193), (10, 64), (11, 1), (12, 0)):
+        molecules[at] = rng.normal(scale=1.0 + 0.25 * max(n, 1) ** (1 / 3), size=(n, 3))
+    calculator = NeighborList(cutoff=3.0, full_list=full, sorted=True)
+    for call in range(3):
+        lists = batch(calculator, molecules)
+        check_in_order(lists, molecules, 3.0, full, f"call {call}")
+        molecules = [m + 0.02 * rng.normal(size=m.shape) for m in molecules]
