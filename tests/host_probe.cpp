@@ -139,6 +139,37 @@ extern "C" void probe_wait_rest(const unsigned char* gives_up, size_t n_calls, u
     }
 }
 
+/// Runs the bookkeeping of kept candidates (vesin_hip::CandidateLifetime) over a sequence of calls with a skin:
+/// `outdated[k]` says whether candidates that exist at call k are found outdated by it. `what[k]` receives what call
+/// k does: 0 a direct search that keeps nothing, 1 a direct search followed by new candidates, 2 a filter of the kept
+/// candidates, 3 a filter that fails followed by new candidates and their filter.
+extern "C" void probe_candidate_lifetime(const unsigned char* outdated, size_t n_calls, unsigned char* what) {
+    vesin_hip::CandidateLifetime lifetime;
+    bool have = false;
+    for (size_t k = 0; k < n_calls; k++) {
+        if (!have) {
+            if (lifetime.resting()) {
+                what[k] = 0;
+            } else {
+                what[k] = 1;
+                have = true;
+            }
+            continue;
+        }
+        if (outdated[k] != 0) {
+            if (lifetime.outdated()) {
+                what[k] = 0;
+                have = false;
+                continue;
+            }
+            what[k] = 3;
+        } else {
+            what[k] = 2;
+        }
+        lifetime.served();
+    }
+}
+
 extern "C" int probe_ordered_records_fit(size_t n_points, size_t record_bytes) {
     return vesin_hip::ordered_records_fit(n_points, record_bytes) ? 1 : 0;
 }

@@ -335,3 +335,25 @@ def test_errors_on_a_list_with_kept_candidates(monkeypatch):
         batch(calculator, all_points, all_boxes, flags)
     monkeypatch.setenv("VESIN_CUDA_MAX_PAIRS_PER_POINT", str(total // n_points + 1))
     check(batch(calculator, all_points, all_boxes, flags), all_points, all_boxes, flags, 2.5, True, False, "within the limit")
+
+
+def test_candidates_that_keep_getting_outdated_are_given_up_for_a_while(capfd, monkeypatch):
+    """One system of the batch jumps at every call: after three sets of candidates that served a call each, the list
+    searches directly for 64 calls, keeping nothing, then tries candidates again. Always the same rows."""
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    rng = np.random.default_rng(41)
+    all_points, all_boxes, flags = mixed_systems(rng)
+    calculator = NeighborList(cutoff=2.0, full_list=True, skin=0.4)
+    reports = []
+    for call in range(72):
+        if call < 4:
+            all_points[7][call] += np.array([0.9, 0.0, 0.0])
+        capfd.readouterr()
+        lists = batch(calculator, all_points, all_boxes, flags, "PSd")
+        reports.append(capfd.readouterr().err)
+        if call < 6 or call > 66 or call % 16 == 0:
+            check(lists, all_points, all_boxes, flags, 2.0, True, False, f"call {call}")
+    assert "candidates are computed again" in reports[1] and "candidates are computed again" in reports[2]
+    assert "direct searches for a while" in reports[3]
+    assert not any("rows filtered from" in report for report in reports[3:69])
+    assert all("rows filtered from" in report for report in reports[69:])

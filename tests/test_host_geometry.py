@@ -39,6 +39,8 @@ def probe(tmp_path_factory):
                                     ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
     lib.probe_wait_rest.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
     lib.probe_wait_rest.restype = None
+    lib.probe_candidate_lifetime.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+    lib.probe_candidate_lifetime.restype = None
     lib.probe_ordered_share.argtypes = [ctypes.c_size_t, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_int]
     lib.probe_ordered_share.restype = ctypes.c_uint
     for name in ("probe_ordered_write_split", "probe_ordered_count_split"):
@@ -409,6 +411,34 @@ def test_a_launch_whose_waves_gave_up_is_left_alone_for_longer_and_longer(probe)
     assert used[:11].all() and not used[11:75].any() and used[75:201].all() and not used[201:265].any() and used[265:].all()
 
 
+
+
+def run_candidate_lifetime(probe, outdated):
+    outdated = np.ascontiguousarray(outdated, dtype=np.uint8)
+    what = np.zeros(len(outdated), dtype=np.uint8)
+    probe.probe_candidate_lifetime(outdated.ctypes.data, len(outdated), what.ctypes.data)
+    return what.tolist()
+
+
+def test_candidates_that_keep_getting_outdated_are_given_up_for_a_while(probe):
+    """options.skin > 0: 0 = direct search that keeps nothing, 1 = direct search and new candidates, 2 = filter,
+    3 = failed filter, new candidates, filter."""
+    # candidates that last: one set, filtered for ever; outdated every tenth call: computed again every time
+    assert run_candidate_lifetime(probe, [0] * 30) == [1] + [2] * 29
+    every_tenth = [1 if k % 10 == 0 else 0 for k in range(50)]
+    assert run_candidate_lifetime(probe, every_tenth) == [1] + [3 if k % 10 == 0 else 2 for k in range(1, 50)]
+    # outdated at every call: three sets that served one call each (the one that computed them), then 64 direct
+    # searches, then candidates once more
+    what = run_candidate_lifetime(probe, [1] * 200)
+    assert what[:4] == [1, 3, 3, 0] and what[4:68] == [0] * 64 and what[68:72] == [1, 3, 3, 0]
+    # every third call: sets that serve three calls are short-lived as well; every fourth: they are not
+    what = run_candidate_lifetime(probe, [1 if k % 3 == 0 else 0 for k in range(40)])
+    assert what[:11] == [1, 2, 2, 3, 2, 2, 3, 2, 2, 0, 0]
+    what = run_candidate_lifetime(probe, [1 if k % 4 == 0 else 0 for k in range(60)])
+    assert 0 not in what
+    # two short-lived sets, then one that lasts: the count starts over
+    outdated = [0, 1, 1, 0, 0, 0, 0, 0, 1, 1, 1, 0]
+    assert run_candidate_lifetime(probe, outdated) == [1, 3, 3, 2, 2, 2, 2, 2, 3, 3, 3, 2]
 
 
 def test_work_memory_of_the_in_order_search_is_bounded(probe):

@@ -397,6 +397,7 @@ struct VerletCache {
     /// estimate is revised with every call's row count.
     bool direct = false;
     size_t direct_n_points = 0;
+    CandidateLifetime lifetime; // ... and so are lists whose candidates keep getting outdated after a few calls
 
     VerletCache() = default;
     VerletCache(const VerletCache&) = delete;
@@ -474,6 +475,7 @@ struct BatchVerletCache {
     bool direct = false;                      // as in VerletCache
     size_t direct_n_points = 0;
     int unpackable_rest = 0;                  // calls left before candidates are tried again after shifts they cannot hold
+    CandidateLifetime lifetime;               // as in VerletCache
 
     BatchVerletCache() = default;
     BatchVerletCache(const BatchVerletCache&) = delete;
@@ -2432,23 +2434,27 @@ void verlet_neighbors(
     };
     if (options_changed || cache.direct_n_points != n_points) {
         cache.direct = false;
+        cache.lifetime.reset();
     }
+    auto drop_candidates = [&]() {
+        if (cache.valid) {
+            free_neighbors(cache.candidates);
+            cache.candidates = VesinNeighborList();
+            cache.valid = false;
+        }
+    };
     if (!cache.valid || options_changed || cache.n_ref != n_points || cache.direct) {
         // Without usable candidates this call is a direct search, whose rows are the answer. Its row count says
-        // how many candidates there would be: few enough, and they are computed now for the next calls to filter.
+        // how many candidates there would be: few enough, and they are computed now for the next calls to filter
+        // (unless the candidates of this list keep getting outdated: see CandidateLifetime).
         VesinOptions plain = options;
         plain.skin = 0.0;
         direct_neighbors(points, n_points, box, periodic, plain, neighbors, extras, stream);
         cache.direct = too_long_for_a_filter(neighbors.length);
         cache.direct_n_points = n_points;
         if (cache.direct) {
-            if (cache.valid) {
-                // the candidates of a smaller past are of no use any more
-                free_neighbors(cache.candidates);
-                cache.candidates = VesinNeighborList();
-                cache.valid = false;
-            }
-        } else {
+            drop_candidates(); // the candidates of a smaller past are of no use any more
+        } else if (force_cache || !cache.lifetime.resting()) {
             rebuild();
         }
         return;
@@ -2526,6 +2532,14 @@ void verlet_neighbors(
             if (fresh) {
                 throw std::runtime_error("internal error: fresh Verlet candidates do not cover their own points");
             }
+            if (!force_cache && cache.lifetime.outdated()) {
+                // the third set of candidates in a row that did not last: the direct search for a while
+                drop_candidates();
+                VesinOptions plain = options;
+                plain.skin = 0.0;
+                direct_neighbors(points, n_points, box, periodic, plain, neighbors, extras, stream);
+                return;
+            }
             rebuild();
             continue;
         }
@@ -2546,6 +2560,7 @@ void verlet_neighbors(
         break;
     }
     neighbors.length = total;
+    cache.lifetime.served();
     if (too_long_for_a_filter(total)) {
         cache.direct = true;
         cache.direct_n_points = n_points;
@@ -3030,6 +3045,7 @@ void verlet_batch(
     };
     if (options_changed || cache.direct_n_points != n_points) {
         cache.direct = false;
+        cache.lifetime.reset();
     }
     if (!cache.valid || options_changed || !same_division || cache.direct) {
         // (as in verlet_neighbors: this call is a direct search, and its row count says whether candidates pay)
@@ -3041,6 +3057,12 @@ void verlet_batch(
         if (cache.unpackable_rest > 0) {
             cache.unpackable_rest -= 1;
             cache.direct = true;
+        }
+        if (!cache.direct && !force_cache && cache.lifetime.resting()) {
+            // (candidates that keep getting outdated after a few calls: see CandidateLifetime)
+            cache.drop_candidates();
+            cache.first_point.clear();
+            return;
         }
         if (!cache.direct) {
             rebuild();
@@ -3137,6 +3159,17 @@ void verlet_batch(
             if (fresh) {
                 throw std::runtime_error("internal error: fresh Verlet candidates of a batch do not cover their own points");
             }
+            if (!force_cache && cache.lifetime.outdated()) {
+                if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
+                    std::fprintf(stderr, "batch with a skin: the candidates keep getting outdated, direct searches for a while\n");
+                }
+                cache.drop_candidates();
+                cache.first_point.clear();
+                VesinOptions plain = options;
+                plain.skin = 0.0;
+                direct_batch(points, first_point, n_systems, boxes, periodic, plain, neighbors, first_pair, extras, stream);
+                return;
+            }
             if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
                 std::fprintf(stderr, "batch with a skin: some system moved too far, the candidates are computed again\n");
             }
@@ -3170,6 +3203,7 @@ void verlet_batch(
         break;
     }
     neighbors.length = total;
+    cache.lifetime.served();
     if (std::getenv("VESIN_HIP_DEBUG") != nullptr) {
         std::fprintf(stderr, "batch with a skin: %zu rows filtered from %zu candidates\n", total, n_candidates);
     }

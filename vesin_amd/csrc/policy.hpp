@@ -96,6 +96,54 @@ struct WaitRest {
     }
 };
 
+/// options.skin > 0: kept candidates pay when calls that only filter them outnumber the calls that compute them
+/// again, which cost a failed filter and a search at cutoff + skin (two to three direct searches). A skin too thin
+/// for how far the points move between calls turns that around, and in a batch, where one system past its limit
+/// costs all systems their candidates, so does a large number of systems: candidates that serve fewer than
+/// CANDIDATES_SHORT_LIVED filtering calls are short-lived, and after CANDIDATES_STRIKES such sets in a row the list
+/// searches directly, keeping nothing, for CANDIDATES_REST calls before it tries candidates again. The rows are the
+/// same either way.
+constexpr int CANDIDATES_SHORT_LIVED = 4;
+constexpr int CANDIDATES_STRIKES = 3;
+constexpr int CANDIDATES_REST = 64;
+
+struct CandidateLifetime {
+    int filtered = 0; // calls that the current candidates served
+    int strikes = 0;  // short-lived sets in a row
+    int rest = 0;     // direct calls left before candidates are tried again
+
+    void served() {
+        filtered += 1;
+    }
+
+    /// The check found the candidates outdated. True: no new ones for a while.
+    bool outdated() {
+        strikes = filtered < CANDIDATES_SHORT_LIVED ? strikes + 1 : 0;
+        filtered = 0;
+        if (strikes >= CANDIDATES_STRIKES) {
+            strikes = 0;
+            rest = CANDIDATES_REST;
+            return true;
+        }
+        return false;
+    }
+
+    /// Once per call without usable candidates: true while the list stays with the direct search.
+    bool resting() {
+        if (rest > 0) {
+            rest -= 1;
+            return true;
+        }
+        return false;
+    }
+
+    void reset() {
+        filtered = 0;
+        strikes = 0;
+        rest = 0;
+    }
+};
+
 // ---------------------------------------------------------------------------------------------------------------
 // The search that writes a sorted list in order (ordered.cuh): how its work is cut into waves. Every choice gives
 // the same list; the figures are what the passes were measured at on one MI355X (256 compute units, 1024 SIMDs).
