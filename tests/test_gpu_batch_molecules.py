@@ -1,6 +1,6 @@
-"""Batches of free molecules (no periodic direction, at most 256 points per system) have kernels of their own from the
-second call of a list on: no cell lists, every system's rows in (i, j) order. Per system the rows are those of a call
-on that system alone (``-m gpu``)."""
+"""Batches of free molecules (no periodic direction, at most 64 points per system, 256 for sorted lists) have kernels of
+their own: no cell lists, every system's rows in (i, j) order. Per system the rows are those of a call on that system
+alone (``-m gpu``)."""
 
 import numpy as np
 import pytest
@@ -66,7 +66,7 @@ def test_molecules_of_every_size(most, full, is_sorted, capfd, monkeypatch):
         lists = batch(calculator, molecules)
         report = capfd.readouterr().err
         # (with systems of more than 64 points, only sorted lists come from these kernels)
-        expected_here = call > 0 and (most <= 64 or is_sorted)
+        expected_here = most <= 64 or is_sorted
         assert ("batch of free molecules" in report) == expected_here, report
         if expected_here:
             assert f"{most if most <= 64 else 256} lanes per system" in report
@@ -126,7 +126,7 @@ def test_what_sends_a_batch_back_to_the_general_path(capfd, monkeypatch):
         assert ("batch of free molecules" in capfd.readouterr().err) == (call == 1)
     check_in_order(lists, molecules, cutoff, True, "free again")
 
-    # another division into systems, one molecule of 257 atoms, a forced cell list: all through the general path
+    # another division into systems: these kernels at once; one molecule of 257 atoms, a forced cell list: the general path
     other = random_molecules(rng, 90, 30)
     big = other[:40] + [rng.normal(scale=3.0, size=(257, 3))] + other[40:]
     for molecules_now, options in ((other, {}), (big, {}), (other, {"algorithm": "cell_list"})):
@@ -135,7 +135,7 @@ def test_what_sends_a_batch_back_to_the_general_path(capfd, monkeypatch):
             capfd.readouterr()
             lists = batch(calc, molecules_now)
             report = capfd.readouterr().err
-            expected_fast = call == 1 and molecules_now is other and not options
+            expected_fast = molecules_now is other and not options
             assert ("batch of free molecules" in report) == expected_fast, (len(molecules_now), options, call)
             for s, rows in enumerate(lists):
                 expected = oracle.canonicalize(oracle.neighbors(molecules_now[s], np.zeros((3, 3)), [False] * 3, cutoff, True, False, "ijSdD"))
@@ -193,3 +193,27 @@ def test_molecules_of_very_different_sizes_in_one_batch(full):
         lists = batch(calculator, molecules)
         check_in_order(lists, molecules, 3.0, full, f"call {call}")
         molecules = [m + 0.02 * rng.normal(size=m.shape) for m in molecules]
+
+
+def test_other_molecules_with_every_call_and_a_list_that_starts_with_crystals(capfd, monkeypatch):
+    """A loader hands over other molecules with every call: every call goes through the kernels for molecules, the
+    first one of a new list included. A new list given crystals guesses wrong once and not again."""
+    monkeypatch.setenv("VESIN_HIP_DEBUG", "1")
+    rng = np.random.default_rng(23)
+    calculator = NeighborList(cutoff=2.5, full_list=False, sorted=True)
+    for call in range(6):
+        molecules = random_molecules(rng, int(rng.integers(1, 300)), int(rng.choice([6, 20, 64, 200])))
+        capfd.readouterr()
+        lists = batch(calculator, molecules)
+        assert "batch of free molecules" in capfd.readouterr().err, call
+        check_in_order(lists, molecules, 2.5, False, f"call {call}")
+
+    crystals = [rng.random((n, 3)) * 5.0 for n in (8, 20, 33)]
+    boxes = np.array([np.eye(3) * 5.0] * 3)
+    flags = np.ones((3, 3), dtype=bool)
+    another = NeighborList(cutoff=2.5, full_list=True, sorted=True)
+    for call in range(3):
+        capfd.readouterr()
+        lists = batch(another, crystals, flags=flags, boxes=boxes)
+        assert ("free molecules no more" in capfd.readouterr().err) == (call == 0)
+        check_in_order(lists, crystals, 2.5, True, f"crystals, call {call}", flags=flags, boxes=boxes)

@@ -564,8 +564,9 @@ struct BatchSetup {
     // batches of free molecules (molecules.cuh): work memory of their own (what the general path keeps in the list's
     // work memory between calls stays as it is), the division into systems on the device, the kernels' report
     DeviceBuffer molecule_work;
-    uint64_t division = 0;          // counts the divisions into systems this set-up has seen (`first_point` assigned)
-    uint64_t molecule_division = 0; // the one whose first points are in `molecule_work` (0: none)
+    std::vector<size_t> molecule_first_point;      // the division into systems whose 32-bit copy is in `molecule_work`
+    PinnedVector<uint32_t> molecule_first_point32; // (where the copy to the device starts from)
+    bool molecule_first_point_on_device = false;
     MoleculeStatus* molecule_report = nullptr; // pinned
 };
 
@@ -2619,7 +2620,7 @@ void verlet_batch(
 );
 
 bool molecules_batch(
-    const double (*points)[3], const size_t* first_point, size_t n_systems, const bool (*periodic)[3],
+    const double (*points)[3], const size_t* first_point, size_t n_systems, const bool (*periodic)[3], size_t most_points,
     VesinOptions options, VesinNeighborList& neighbors, size_t* first_pair, HipExtras& extras, hipStream_t stream
 );
 
@@ -2698,20 +2699,26 @@ void direct_batch(
     const size_t n_points = first_point[n_systems];
     extras.guess.have_box = false; // the work buffers of the single-system path are about to be reused
 
-    // Free molecules of at most 64 points each (256 for a sorted list), as the call before found them (same division
-    // into systems; that no system has a periodic direction is for the kernels to confirm): no cell lists, see
-    // molecules.cuh. With larger systems in the batch the kernels for molecules write an unsorted list no faster than
-    // the general path (2,000 molecules of 100 to 256 atoms 0.69 against 0.59 ms per call, 20,000 of 3 to 80 atoms
-    // 0.89 against 0.85 ms), and a sorted one in half the time (0.69 against 1.26 ms, 0.89 against 1.37 ms).
+    // Free molecules of at most 64 points each (256 for a sorted list): no cell lists, see molecules.cuh. That no
+    // system has a periodic direction is for the kernels to confirm, since the flags live on the device: the batch is
+    // tried as one of free molecules on a list that has not seen a batch yet or whose last batch through the general
+    // path had no periodic direction anywhere (a loader that hands over other molecules with every call stays on these
+    // kernels; a list used for crystals pays for the wrong guess once at most). With larger systems in the batch the
+    // kernels for molecules write an unsorted list no faster than the general path (2,000 molecules of 100 to 256
+    // atoms 0.69 against 0.59 ms per call, 20,000 of 3 to 80 atoms 0.89 against 0.85 ms), and a sorted one in half the
+    // time (0.69 against 1.26 ms, 0.89 against 1.37 ms).
     {
         const BatchSetup& known = extras.batch;
-        const size_t most_points = options.sorted ? MOLECULE_MAX_POINTS : MOLECULE_GROUP_POINTS;
+        size_t most_points = 0;
+        for (size_t s = 0; s < n_systems; s++) {
+            most_points = std::max(most_points, first_point[s + 1] - first_point[s]);
+        }
         const bool free_molecules =
-            known.valid && known.all_open && known.most_points <= most_points && n_points > 0 &&
-            options.algorithm != VesinCellList && !extras.fixed_memory && std::getenv("VESIN_HIP_MOLECULES") == nullptr &&
-            known.first_point.size() == n_systems + 1 &&
-            std::memcmp(known.first_point.data(), first_point, (n_systems + 1) * sizeof(size_t)) == 0;
-        if (free_molecules && molecules_batch(points, first_point, n_systems, periodic, options, neighbors, first_pair, extras, stream)) {
+            (!known.valid || known.all_open) && n_points > 0 &&
+            most_points <= (options.sorted ? MOLECULE_MAX_POINTS : MOLECULE_GROUP_POINTS) &&
+            options.algorithm != VesinCellList && !extras.fixed_memory && std::getenv("VESIN_HIP_MOLECULES") == nullptr;
+        if (free_molecules &&
+            molecules_batch(points, first_point, n_systems, periodic, most_points, options, neighbors, first_pair, extras, stream)) {
             return;
         }
     }
@@ -2761,11 +2768,11 @@ void direct_batch(
     setup.guess.stored(key);
 }
 
-/// A batch of free molecules through molecules_kernel: counting pass, scan over the systems, writing pass, one
-/// synchronisation. Returns false, with nothing of the result to be used, when some system turned out to have a
-/// periodic direction (the flags live on the device).
+/// A batch of free molecules (`most_points` at most per system) through molecules_kernel: counting pass, scan over
+/// the systems, writing pass, one synchronisation. Returns false, with nothing of the result to be used, when some
+/// system turned out to have a periodic direction (the flags live on the device).
 bool molecules_batch(
-    const double (*points)[3], const size_t* first_point, size_t n_systems, const bool (*periodic)[3],
+    const double (*points)[3], const size_t* first_point, size_t n_systems, const bool (*periodic)[3], size_t most_points,
     VesinOptions options, VesinNeighborList& neighbors, size_t* first_pair, HipExtras& extras, hipStream_t stream
 ) {
     const TraceRange whole_call("vesin_hip_neighbors_batch (free molecules)");
@@ -2791,8 +2798,8 @@ bool molecules_batch(
     uint64_t* d_first_pair = nullptr;
     uint64_t* scan_scratch = nullptr;
     // lanes per system: the next power of two from the largest system on, eight at least; a workgroup beyond 64
-    const int lanes = setup.most_points <= 8 ? 8 : setup.most_points <= 16 ? 16 : setup.most_points <= 32 ? 32
-                    : setup.most_points <= MOLECULE_GROUP_POINTS ? 64 : MOLECULE_BLOCK;
+    const int lanes = most_points <= 8 ? 8 : most_points <= 16 ? 16 : most_points <= 32 ? 32
+                    : most_points <= MOLECULE_GROUP_POINTS ? 64 : MOLECULE_BLOCK;
     const bool wide = lanes == MOLECULE_BLOCK;
     uint64_t* d_first_row = nullptr;
     auto carve = [&](Carver& c) {
@@ -2810,13 +2817,21 @@ bool molecules_batch(
     setup.molecule_work.reserve(measure.used);
     Carver carver(setup.molecule_work.ptr);
     carve(carver);
-    // (the caller found this call's division to be the one of the set-up, whose 32-bit copy goes to the device once)
-    if (setup.molecule_division != setup.division || generation != setup.molecule_work.generation) {
-        setup.molecule_division = 0;
+    // the division into systems goes to the device when it is not the one of the call before
+    const bool same_division = setup.molecule_first_point_on_device && generation == setup.molecule_work.generation &&
+                               setup.molecule_first_point.size() == n_systems + 1 &&
+                               std::memcmp(setup.molecule_first_point.data(), first_point, (n_systems + 1) * sizeof(size_t)) == 0;
+    if (!same_division) {
+        setup.molecule_first_point_on_device = false;
+        setup.molecule_first_point.assign(first_point, first_point + n_systems + 1);
+        setup.molecule_first_point32.resize(n_systems + 1);
+        for (size_t s = 0; s <= n_systems; s++) {
+            setup.molecule_first_point32[s] = static_cast<uint32_t>(first_point[s]);
+        }
         HIP_CHECK(hipMemcpyAsync(
-            d_first_point, setup.first_point32.data(), (n_systems + 1) * sizeof(uint32_t), hipMemcpyHostToDevice, stream
+            d_first_point, setup.molecule_first_point32.data(), (n_systems + 1) * sizeof(uint32_t), hipMemcpyHostToDevice, stream
         ));
-        setup.molecule_division = setup.division;
+        setup.molecule_first_point_on_device = true;
     }
 
     args.points = reinterpret_cast<const double*>(points);
@@ -2868,12 +2883,17 @@ bool molecules_batch(
         if (attempt > 2) {
             throw std::runtime_error("internal error: the rows of a batch of molecules did not settle");
         }
-        size_outputs(neighbors, extras, total, options);
+        // (a list without arrays gets them once the kernels have confirmed that these are free molecules: until then
+        // it stays as it was, for the general path to start from; the writing pass only reports)
+        const bool has_arrays = extras.capacity > 0 || attempt > 0;
+        if (has_arrays) {
+            size_outputs(neighbors, extras, total, options);
+        }
         args.out.pairs = reinterpret_cast<unsigned long long*>(neighbors.pairs);
         args.out.shifts = reinterpret_cast<int32_t*>(neighbors.shifts);
         args.out.distances = neighbors.distances;
         args.out.vectors = reinterpret_cast<double*>(neighbors.vectors);
-        args.capacity = extras.capacity;
+        args.capacity = has_arrays ? extras.capacity : 0;
         launch(true);
         if (attempt == 0) {
             HIP_CHECK(hipMemcpyAsync(
@@ -2901,9 +2921,12 @@ bool molecules_batch(
                 "VESIN_CUDA_MAX_PAIRS_PER_POINT as an environment variable."
             );
         }
-        if (total <= extras.capacity) {
+        if (total <= args.capacity) {
             break;
         }
+    }
+    if (extras.capacity == 0) {
+        size_outputs(neighbors, extras, 0, options); // (no rows at all: the arrays exist all the same)
     }
     neighbors.length = total;
     std::memcpy(first_pair, setup.first_pair_landing, (n_systems + 1) * sizeof(size_t));
@@ -3277,7 +3300,6 @@ bool batch_attempt(
         setup.boxes.swap(setup.incoming_boxes);
         setup.periodic.swap(setup.incoming_periodic);
         setup.first_point.assign(first_point, first_point + n_systems + 1);
-        setup.division += 1;
         setup.cutoff = options.cutoff;
         setup.algorithm = static_cast<int>(options.algorithm);
         setup.full_stencil = full_stencil_only();

@@ -48,7 +48,8 @@ struct MoleculeArgs {
     uint32_t* rows_of_point;       // [total_points]
     const uint64_t* first_row;     // [total_points + 1]
     SearchOutputs out;
-    size_t capacity;               // rows the output arrays hold: a longer list is not written at all
+    size_t capacity;               // rows the output arrays hold: a longer list is not written at all (and
+                                   // nothing is when the counting pass met a periodic direction)
     MoleculeStatus* status;        // device
     MoleculeStatus* report;        // pinned
 };
@@ -71,7 +72,7 @@ __global__ __launch_bounds__(MOLECULE_BLOCK) void molecules_kernel(MoleculeArgs 
             a.report->first_bad = a.status->first_bad;
             a.report->total_rows = total;
         }
-        if (total > a.capacity) {
+        if (total > a.capacity || a.status->periodic != 0) {
             return;
         }
     }
@@ -170,7 +171,7 @@ __global__ __launch_bounds__(MOLECULE_BLOCK) void molecules_wide_kernel(Molecule
             a.report->first_bad = a.status->first_bad;
             a.report->total_rows = total;
         }
-        if (total > a.capacity) {
+        if (total > a.capacity || a.status->periodic != 0) {
             return;
         }
     }
