@@ -613,3 +613,33 @@ def test_stretched_open_systems_keep_to_the_room_for_their_cells(algorithm, capf
             rows = slice(int(first_pair[s]), int(first_pair[s + 1]))
             expected = oracle.neighbors(points, np.eye(3) * 500.0, [False] * 3, cutoff, True, False, "ijSdD")
             assert_same_list({k: v[rows] for k, v in whole.items()}, expected, what=f"call {call}, system {s}")
+
+
+def test_five_thousand_systems_of_every_kind_and_other_ones_with_every_call():
+    """Enough systems for the host to go over them on several threads (boxes, grids), with open directions among
+    them (extents of the points in between), and another set of systems with every call; a singular box among them is
+    the error it always is."""
+    rng = np.random.default_rng(91)
+    calculator = NeighborList(cutoff=3.0, full_list=True)
+    for call in range(3):
+        all_points, all_boxes, all_flags = [], [], []
+        for _ in range(5000):
+            n = int(rng.integers(0, 24))
+            edge = 4.0 + 4.0 * rng.random()
+            box = np.eye(3) * edge + 0.2 * rng.normal(size=(3, 3))
+            kind = rng.integers(0, 4)
+            flags = [(True, True, True), (True, True, False), (False, False, False), (True, True, True)][kind]
+            all_points.append(rng.random((n, 3)) @ box)
+            all_boxes.append(box)
+            all_flags.append(flags)
+        if call == 2:
+            all_boxes[4321] = all_boxes[4321].copy()
+            all_boxes[4321][2] = all_boxes[4321][0]
+            all_flags[4321] = (True, True, True)
+            with pytest.raises(RuntimeError, match="the box matrix is not invertible"):
+                run_batch(calculator, all_points, all_boxes, periodic=np.array(all_flags))
+            continue
+        lists = run_batch(calculator, all_points, all_boxes, periodic=np.array(all_flags))
+        for s in rng.choice(5000, size=150, replace=False):
+            expected = oracle.neighbors(all_points[s], all_boxes[s], list(all_flags[s]), 3.0, True, False, "ijSdD")
+            assert_same_list(lists[s], expected, what=f"call {call}, system {s}")
