@@ -2618,23 +2618,27 @@ void verlet_neighbors(
     }
 }
 
-/// first_pair[s] = first output row of system s (offsets are kept per tile-major work item), first_pair[n] = total.
+/// first_pair[s] = first output row of system s (offsets are kept per tile-major work item), first_pair[n] = total;
+/// for the device and, in `landing`, for the host.
 __global__ void system_rows_kernel(
     const uint64_t* __restrict__ cell_scan, const uint32_t* __restrict__ cell_base, const uint64_t* __restrict__ offsets,
     uint32_t n_systems, uint32_t n_slices, uint32_t n_slots, const FusedStatus* __restrict__ single_pass,
-    unsigned long long* __restrict__ first_pair
+    unsigned long long* __restrict__ first_pair, unsigned long long* __restrict__ landing
 ) {
     const uint32_t s = blockIdx.x * BLOCK + threadIdx.x;
     if (s > n_systems) {
         return;
     }
+    unsigned long long first = 0;
     if (s == n_systems) {
         // after the single-pass search `offsets` holds the first row of every work item, the total is in its status
-        first_pair[s] = single_pass != nullptr ? single_pass->total_rows : offsets[n_slots];
-        return;
+        first = single_pass != nullptr ? single_pass->total_rows : offsets[n_slots];
+    } else {
+        const uint32_t first_tile = static_cast<uint32_t>(cell_scan[cell_base[s]] >> 32);
+        first = offsets[static_cast<size_t>(first_tile) * n_slices];
     }
-    const uint32_t first_tile = static_cast<uint32_t>(cell_scan[cell_base[s]] >> 32);
-    first_pair[s] = offsets[static_cast<size_t>(first_tile) * n_slices];
+    first_pair[s] = first;
+    landing[s] = first; // (pinned host memory: what the host reads after the call's synchronisation)
 }
 
 template <bool WRITE>
@@ -4007,11 +4011,8 @@ bool batch_attempt(
         hipLaunchKernelGGL(
             system_rows_kernel, dim3(system_blocks), dim3(BLOCK), 0, stream,
             cell_scan, d_cell_base, offsets, static_cast<uint32_t>(n_systems), n_slices, static_cast<uint32_t>(n_slots),
-            fused_status, d_first_pair
+            fused_status, d_first_pair, reinterpret_cast<unsigned long long*>(setup.first_pair_landing)
         );
-        HIP_CHECK(hipMemcpyAsync(
-            setup.first_pair_landing, d_first_pair, (n_systems + 1) * sizeof(size_t), hipMemcpyDeviceToHost, stream
-        ));
         HIP_CHECK(hipStreamSynchronize(stream));
         if (speculate && (extras.mail->batch_changed != 0 || (device_grids && extras.mail->batch_total_cells > total_cells))) {
             // other boxes than the grids were picked from, or (which open_grids_kernel rules out) more cells than
@@ -4095,11 +4096,8 @@ bool batch_attempt(
     hipLaunchKernelGGL(
         system_rows_kernel, dim3(system_blocks), dim3(BLOCK), 0, stream,
         cell_scan, d_cell_base, offsets, static_cast<uint32_t>(n_systems), n_slices, static_cast<uint32_t>(n_slots),
-        static_cast<const FusedStatus*>(nullptr), d_first_pair
+        static_cast<const FusedStatus*>(nullptr), d_first_pair, reinterpret_cast<unsigned long long*>(setup.first_pair_landing)
     );
-    HIP_CHECK(hipMemcpyAsync(
-        setup.first_pair_landing, d_first_pair, (n_systems + 1) * sizeof(size_t), hipMemcpyDeviceToHost, stream
-    ));
     if (sorting) {
         // every system's rows stay in their range and come out ordered by (i, j, shift) inside it: the order of
         // vesin_neighbors on that system alone
