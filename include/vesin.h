@@ -306,6 +306,42 @@ int VESIN_API vesin_hip_pairs_backward(
     const char** error_message
 );
 
+/* Output arrays from the caller's allocator, and handing them over without a copy. No counterpart in the
+ * reference, whose callers copy the rows out of the list's arrays when they want to keep them beyond the next
+ * call (python/vesin/vesin/_neighbors.py:343-381 and :513-574, vesin-torch/src/vesin_torch.cpp:214-256): for a
+ * list of a million points that copy takes as long as the search.
+ *
+ * vesin_hip_set_output_allocator makes `neighbors` take the memory of pairs / shifts / distances / vectors from
+ * `allocate` and give it back through `release` (both called with `context`, with the list's GPU current, from
+ * inside calls on this list and from vesin_free; `allocate` returns device memory of that GPU, usable on any of
+ * its streams, or NULL when it has none). Arrays the list holds at that moment go back to where they came from.
+ * NULL for both restores hipMalloc / hipFree. The list may be zeroed (no call yet): `device` is then the device it
+ * will be used with.
+ *
+ * vesin_hip_detach_outputs makes the arrays `neighbors` points to the caller's: read the four pointers and `length`
+ * from the struct first; afterwards they are NULL in the struct, the list will never touch or release that memory
+ * again, and the caller releases every non-NULL array itself, the way `release` would (hipFree without an
+ * allocator). `*capacity` (may be NULL) receives the rows each array has room for. The next call on the list
+ * allocates arrays of that size again before it starts, so it runs as a call on a list that kept its arrays. Fails
+ * while a call queued with vesin_hip_neighbors_enqueue is pending. */
+typedef void* (*VesinHipAllocate)(size_t bytes, void* context);
+typedef void (*VesinHipRelease)(void* pointer, void* context);
+
+int VESIN_API vesin_hip_set_output_allocator(
+    struct VesinNeighborList* neighbors,
+    struct VesinDevice device,
+    VesinHipAllocate allocate,
+    VesinHipRelease release,
+    void* context,
+    const char** error_message
+);
+
+int VESIN_API vesin_hip_detach_outputs(struct VesinNeighborList* neighbors, size_t* capacity, const char** error_message);
+
+/* Rows every output array of `neighbors` has room for (0 for a list without arrays): what a caller compares `length`
+ * with before it takes arrays over that are much larger than their rows. */
+size_t VESIN_API vesin_hip_output_capacity(const struct VesinNeighborList* neighbors);
+
 void VESIN_API vesin_hip_enable_timings(int enabled);
 int VESIN_API vesin_hip_last_timings(const struct VesinNeighborList* neighbors, struct VesinHipTimings* timings);
 

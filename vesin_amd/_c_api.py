@@ -176,6 +176,23 @@ def get_library():
             ctypes.c_void_p,
             ctypes.POINTER(ctypes.c_char_p),
         ]
+        lib.vesin_hip_set_output_allocator.restype = ctypes.c_int
+        lib.vesin_hip_set_output_allocator.argtypes = [
+            ctypes.POINTER(VesinNeighborList),
+            VesinDevice,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.POINTER(ctypes.c_char_p),
+        ]
+        lib.vesin_hip_detach_outputs.restype = ctypes.c_int
+        lib.vesin_hip_detach_outputs.argtypes = [
+            ctypes.POINTER(VesinNeighborList),
+            ctypes.POINTER(ctypes.c_size_t),
+            ctypes.POINTER(ctypes.c_char_p),
+        ]
+        lib.vesin_hip_output_capacity.restype = ctypes.c_size_t
+        lib.vesin_hip_output_capacity.argtypes = [ctypes.POINTER(VesinNeighborList)]
         lib.vesin_hip_enable_timings.restype = None
         lib.vesin_hip_enable_timings.argtypes = [ctypes.c_int]
         lib.vesin_hip_last_timings.restype = ctypes.c_int

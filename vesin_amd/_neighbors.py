@@ -13,6 +13,13 @@ The calculation always runs on a GPU through ``vesin_neighbors`` with ``device =
 * numpy arrays (or anything numpy can convert) are uploaded to ``device`` (default ``cuda:0``) and the results come
   back as numpy arrays.
 
+With ``copy=True`` (the default) the reference copies every array out of the list's memory
+(python/vesin/vesin/_neighbors.py:343-381, 513-574). Here the list takes its arrays from PyTorch's caching allocator
+(``vesin_hip_set_output_allocator``, through the two functions ``lib/libvesin_torch.so`` exports) and the tensors that
+go to the caller take them over (``vesin_hip_detach_outputs``): nothing is copied, the next call gets arrays of the
+same size from the allocator's cache. Arrays with room for more than twice their rows are copied as before, and so is
+everything when ``lib/libvesin_torch.so`` was not built.
+
 torch is only used to hold device memory; nothing is computed with it.
 """
 
@@ -33,6 +40,32 @@ from ._c_api import (
     VesinUnknownDevice,
     get_library,
 )
+
+_HANDOVER = None
+
+
+def _torch_handover():
+    """What taking arrays over needs, or False when ``lib/libvesin_torch.so`` is not there: the library itself (for
+    its ``vesin_amd_torch_release``), the addresses of its allocate and release functions, and the operator that
+    makes a tensor the owner of an array from that allocator."""
+    global _HANDOVER
+    if _HANDOVER is None:
+        try:
+            import torch
+
+            from .torchscript import TORCH_LIB_PATH, load_torch_library
+
+            load_torch_library()
+            hooks = ctypes.CDLL(TORCH_LIB_PATH)
+            hooks.vesin_amd_torch_release.restype = None
+            hooks.vesin_amd_torch_release.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+            allocate = ctypes.cast(hooks.vesin_amd_torch_allocate, ctypes.c_void_p).value
+            release = ctypes.cast(hooks.vesin_amd_torch_release, ctypes.c_void_p).value
+            _HANDOVER = (hooks, allocate, release, torch.ops.vesin_amd.adopt)
+        except Exception:
+            _HANDOVER = False
+    return _HANDOVER
+
 
 _ALGORITHMS = {
     "auto": VesinAutoAlgorithm,
@@ -122,6 +155,54 @@ class NeighborList:
             raise ValueError("n_threads must be zero or a positive integer")
         self.device = device
         self._neighbors = VesinNeighborList()
+        # whether results with ``copy=True`` take the list's arrays over instead of copying them
+        self.hand_over = True
+        self._allocator_set = False
+
+    def _torch_allocator(self, c_device):
+        """Make the list take its arrays from PyTorch's caching allocator (once per list); returns what
+        ``_torch_handover`` does, or None when arrays are not handed over."""
+        if not self.hand_over:
+            return None
+        handover = _torch_handover()
+        if not handover:
+            return None
+        if not self._allocator_set:
+            error_message = ctypes.c_char_p()
+            status = self._lib.vesin_hip_set_output_allocator(
+                ctypes.byref(self._neighbors), c_device, handover[1], handover[2], None, ctypes.byref(error_message)
+            )
+            if status != 0:
+                raise RuntimeError(error_message.value.decode("utf8"))
+            self._allocator_set = True
+        return handover
+
+    def _take_arrays(self, handover):
+        """The arrays of the list become the caller's (None when they stay: no allocator, no rows, or room for more
+        than twice the rows): returns a function ``(pointer, shape, dtype, index) -> tensor`` that makes a tensor the
+        owner of one of them, and a function that releases those no tensor took."""
+        n_pairs = self._neighbors.length
+        if not handover or not self._allocator_set or n_pairs == 0:
+            return None
+        if 2 * n_pairs < self._lib.vesin_hip_output_capacity(ctypes.byref(self._neighbors)):
+            return None
+        arrays = [self._neighbors.pairs, self._neighbors.shifts, self._neighbors.distances, self._neighbors.vectors]
+        error_message = ctypes.c_char_p()
+        if self._lib.vesin_hip_detach_outputs(ctypes.byref(self._neighbors), None, ctypes.byref(error_message)) != 0:
+            return None
+        hooks, adopt = handover[0], handover[3]
+        left = {pointer for pointer in arrays if pointer}
+
+        def owned(pointer, shape, dtype, index):
+            left.discard(pointer)
+            return adopt(pointer, list(shape), dtype, index)
+
+        def release_rest():
+            for pointer in left:
+                hooks.vesin_amd_torch_release(pointer, None)
+            left.clear()
+
+        return owned, release_rest
 
     def __del__(self):
         if hasattr(self, "_lib") and hasattr(self, "_neighbors"):
@@ -267,6 +348,8 @@ class NeighborList:
             # the list lives on another GPU: release it and start from a zeroed struct
             self._lib.vesin_free(ctypes.byref(self._neighbors))
             ctypes.memset(ctypes.byref(self._neighbors), 0, ctypes.sizeof(self._neighbors))
+            self._allocator_set = False
+        handover = self._torch_allocator(c_device) if copy else None
 
         # inputs may still be in flight on torch's current stream. The library works on the null stream, which waits
         # for everything earlier on torch's default stream by itself; only a stream of the caller's own does not
@@ -292,11 +375,12 @@ class NeighborList:
             raise RuntimeError(error_message.value.decode("utf8"))
 
         n_pairs = self._neighbors.length
+        pointers = (self._neighbors.pairs, self._neighbors.shifts, self._neighbors.distances, self._neighbors.vectors)
+        taken = self._take_arrays(handover) if copy else None
         if not copy:
             # views of arrays that did not move, asked for in the same way: the tuple of the call before
             result_key = (
-                quantities, n_pairs, self._neighbors.pairs, self._neighbors.shifts, self._neighbors.distances,
-                self._neighbors.vectors, float_dtype, index,
+                quantities, n_pairs, *pointers, float_dtype, index,
                 # (distances and vectors in another precision are converted copies, made again on every call)
                 namespace is None and is_torch and float_dtype == torch.float64,
             )
@@ -310,6 +394,8 @@ class NeighborList:
         def wrap(pointer, shape, typestr, dtype):
             if n_pairs == 0:
                 return torch.empty(shape, dtype=dtype, device=device_str)
+            if taken is not None:
+                return taken[0](pointer, shape, dtype, index)
             if copy:
                 return torch.as_tensor(_DeviceView(pointer, shape, typestr, self), device=device_str).clone()
             # the arrays are kept between calls: the same pointer and shape give the same view (views refer to
@@ -323,13 +409,15 @@ class NeighborList:
 
         pairs = shifts = distances = vectors = None
         if any(q in quantities for q in "ijP"):
-            pairs = wrap(self._neighbors.pairs, (n_pairs, 2), "<u8", torch.uint64)
+            pairs = wrap(pointers[0], (n_pairs, 2), "<u8", torch.uint64)
         if "S" in quantities:
-            shifts = wrap(self._neighbors.shifts, (n_pairs, 3), "<i4", torch.int32)
+            shifts = wrap(pointers[1], (n_pairs, 3), "<i4", torch.int32)
         if "d" in quantities:
-            distances = wrap(self._neighbors.distances, (n_pairs,), "<f8", torch.float64).to(float_dtype)
+            distances = wrap(pointers[2], (n_pairs,), "<f8", torch.float64).to(float_dtype)
         if "D" in quantities:
-            vectors = wrap(self._neighbors.vectors, (n_pairs, 3), "<f8", torch.float64).to(float_dtype)
+            vectors = wrap(pointers[3], (n_pairs, 3), "<f8", torch.float64).to(float_dtype)
+        if taken is not None:
+            taken[1]()  # (the pairs of a call that asked for none of "ijP")
 
         data = []
         for quantity in quantities:
@@ -394,6 +482,11 @@ class NeighborList:
         options.skin = self.skin
 
         index = device.index if device.index is not None else torch.cuda.current_device()
+        if self._neighbors.device.type != VesinUnknownDevice and self._neighbors.device.device_id != index:
+            self._lib.vesin_free(ctypes.byref(self._neighbors))
+            ctypes.memset(ctypes.byref(self._neighbors), 0, ctypes.sizeof(self._neighbors))
+            self._allocator_set = False
+        handover = self._torch_allocator(VesinDevice(VesinCUDA, index)) if copy else None
         torch.cuda.current_stream(device).synchronize()
         first_pair = np.zeros(n_systems + 1, dtype=np.uint64)
         error_message = ctypes.c_char_p()
@@ -412,12 +505,23 @@ class NeighborList:
         if status != 0:
             raise RuntimeError(error_message.value.decode("utf8"))
 
+        return self._results(quantities, index, copy, handover), first_pair
+
+    def _results(self, quantities, index, copy, handover):
+        """The requested quantities of the call that just ended, as torch tensors: views of the list's arrays, or
+        (``copy``) tensors of their own, which take the arrays over when they can."""
+        import torch
+
         n_pairs = self._neighbors.length
         device_str = f"cuda:{index}"
+        pointers = (self._neighbors.pairs, self._neighbors.shifts, self._neighbors.distances, self._neighbors.vectors)
+        taken = self._take_arrays(handover) if copy else None
 
         def wrap(pointer, shape, typestr, dtype):
             if n_pairs == 0:
                 return torch.empty(shape, dtype=dtype, device=device_str)
+            if taken is not None:
+                return taken[0](pointer, shape, dtype, index)
             view = torch.as_tensor(_DeviceView(pointer, shape, typestr, self), device=device_str)
             return view.clone() if copy else view
 
@@ -425,7 +529,7 @@ class NeighborList:
         pairs = None
         for quantity in quantities:
             if quantity in "ijP" and pairs is None:
-                pairs = wrap(self._neighbors.pairs, (n_pairs, 2), "<u8", torch.uint64)
+                pairs = wrap(pointers[0], (n_pairs, 2), "<u8", torch.uint64)
             if quantity == "P":
                 data.append(pairs)
             elif quantity == "i":
@@ -433,12 +537,14 @@ class NeighborList:
             elif quantity == "j":
                 data.append(pairs[:, 1])
             elif quantity == "S":
-                data.append(wrap(self._neighbors.shifts, (n_pairs, 3), "<i4", torch.int32))
+                data.append(wrap(pointers[1], (n_pairs, 3), "<i4", torch.int32))
             elif quantity == "d":
-                data.append(wrap(self._neighbors.distances, (n_pairs,), "<f8", torch.float64))
+                data.append(wrap(pointers[2], (n_pairs,), "<f8", torch.float64))
             elif quantity == "D":
-                data.append(wrap(self._neighbors.vectors, (n_pairs, 3), "<f8", torch.float64))
-        return tuple(data), first_pair
+                data.append(wrap(pointers[3], (n_pairs, 3), "<f8", torch.float64))
+        if taken is not None:
+            taken[1]()
+        return tuple(data)
 
     def enqueue(self, points, box, periodic, quantities: str = "ij"):
         """``compute`` in two halves (``vesin_hip_neighbors_enqueue``): queues the calculation on torch's current
@@ -473,6 +579,11 @@ class NeighborList:
         options.return_distances = "d" in quantities
         options.return_vectors = "D" in quantities
         options.skin = self.skin
+        if self._neighbors.device.type != VesinUnknownDevice and self._neighbors.device.device_id != index:
+            self._lib.vesin_free(ctypes.byref(self._neighbors))
+            ctypes.memset(ctypes.byref(self._neighbors), 0, ctypes.sizeof(self._neighbors))
+            self._allocator_set = False
+        self._torch_allocator(VesinDevice(VesinCUDA, index))
         word = ctypes.c_void_p()
         error_message = ctypes.c_char_p()
         status = self._lib.vesin_hip_neighbors_enqueue(
@@ -499,33 +610,8 @@ class NeighborList:
         error_message = ctypes.c_char_p()
         if self._lib.vesin_hip_neighbors_collect(ctypes.byref(self._neighbors), ctypes.byref(error_message)) != 0:
             raise RuntimeError(error_message.value.decode("utf8"))
-        n_pairs = self._neighbors.length
-        device_str = f"cuda:{index}"
-
-        def wrap(pointer, shape, typestr, dtype):
-            if n_pairs == 0:
-                return torch.empty(shape, dtype=dtype, device=device_str)
-            view = torch.as_tensor(_DeviceView(pointer, shape, typestr, self), device=device_str)
-            return view.clone() if copy else view
-
-        data = []
-        pairs = None
-        for quantity in quantities:
-            if quantity in "ijP" and pairs is None:
-                pairs = wrap(self._neighbors.pairs, (n_pairs, 2), "<u8", torch.uint64)
-            if quantity == "P":
-                data.append(pairs)
-            elif quantity == "i":
-                data.append(pairs[:, 0])
-            elif quantity == "j":
-                data.append(pairs[:, 1])
-            elif quantity == "S":
-                data.append(wrap(self._neighbors.shifts, (n_pairs, 3), "<i4", torch.int32))
-            elif quantity == "d":
-                data.append(wrap(self._neighbors.distances, (n_pairs,), "<f8", torch.float64))
-            elif quantity == "D":
-                data.append(wrap(self._neighbors.vectors, (n_pairs, 3), "<f8", torch.float64))
-        return tuple(data)
+        handover = _torch_handover() if copy and self.hand_over and self._allocator_set else None
+        return self._results(quantities, index, copy, handover)
 
     def timings(self):
         """Per-stage GPU times (ms) of the last ``compute``; needs ``enable_timings(True)`` beforehand."""

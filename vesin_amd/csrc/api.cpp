@@ -414,6 +414,85 @@ extern "C" void vesin_free(VesinNeighborList* neighbors) {
     std::memset(static_cast<void*>(neighbors), 0, sizeof(VesinNeighborList));
 }
 
+extern "C" int vesin_hip_set_output_allocator(
+    VesinNeighborList* neighbors,
+    VesinDevice device,
+    VesinHipAllocate allocate,
+    VesinHipRelease release,
+    void* context,
+    const char** error_message
+) {
+    if (error_message == nullptr) {
+        return EXIT_FAILURE;
+    }
+    if (neighbors == nullptr) {
+        return fail(error_message, "`neighbors` can not be a NULL pointer");
+    }
+    if (device.type != VesinCUDA) {
+        return fail(error_message, "output arrays are only allocated for a GPU device (VesinCUDA, i.e. HIP on ROCm)");
+    }
+    if (neighbors->device.type != VesinUnknownDevice &&
+        (neighbors->device.type != device.type || neighbors->device.device_id != device.device_id)) {
+        return fail(error_message, "`neighbors` device and data `device` do not match, free the neighbors first");
+    }
+    try {
+        const bool fresh = neighbors->device.type == VesinUnknownDevice;
+        neighbors->device = device;
+        try {
+            vesin_hip::set_output_allocator(*neighbors, allocate, release, context);
+        } catch (...) {
+            if (fresh && neighbors->opaque == nullptr) {
+                neighbors->device.type = VesinUnknownDevice;
+                neighbors->device.device_id = 0;
+            }
+            throw;
+        }
+    } catch (const std::bad_alloc&) {
+        LAST_ERROR = "failed to allocate memory";
+        *error_message = LAST_ERROR.c_str();
+        return EXIT_FAILURE;
+    } catch (const std::exception& e) {
+        LAST_ERROR = e.what();
+        *error_message = LAST_ERROR.c_str();
+        return EXIT_FAILURE;
+    } catch (...) {
+        return fail(error_message, "fatal error: unknown type thrown as exception");
+    }
+    return EXIT_SUCCESS;
+}
+
+extern "C" int vesin_hip_detach_outputs(VesinNeighborList* neighbors, size_t* capacity, const char** error_message) {
+    if (error_message == nullptr) {
+        return EXIT_FAILURE;
+    }
+    if (neighbors == nullptr) {
+        return fail(error_message, "`neighbors` can not be a NULL pointer");
+    }
+    if (neighbors->device.type != VesinCUDA && neighbors->device.type != VesinUnknownDevice) {
+        return fail(error_message, "the arrays of this list are not this library's");
+    }
+    try {
+        const size_t rows = vesin_hip::detach_outputs(*neighbors);
+        if (capacity != nullptr) {
+            *capacity = rows;
+        }
+    } catch (const std::exception& e) {
+        LAST_ERROR = e.what();
+        *error_message = LAST_ERROR.c_str();
+        return EXIT_FAILURE;
+    } catch (...) {
+        return fail(error_message, "fatal error: unknown type thrown as exception");
+    }
+    return EXIT_SUCCESS;
+}
+
+extern "C" size_t vesin_hip_output_capacity(const VesinNeighborList* neighbors) {
+    if (neighbors == nullptr || neighbors->device.type != VesinCUDA) {
+        return 0;
+    }
+    return vesin_hip::output_capacity(*neighbors);
+}
+
 extern "C" void vesin_hip_enable_timings(int enabled) {
     vesin_hip::enable_timings(enabled != 0);
 }

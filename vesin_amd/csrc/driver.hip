@@ -16,6 +16,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <thread>
+#include <type_traits>
 
 #include <algorithm>
 #include <atomic>
@@ -796,6 +797,11 @@ struct HipExtras {
     /// array, the output arrays are the caller's, and nothing of it is ever freed or grown.
     bool fixed_memory = false;
     size_t capacity = 0;              // rows every allocated output array can hold
+    /// Where the output arrays come from and go back to when the caller said so (vesin_hip_set_output_allocator);
+    /// hipMalloc and hipFree otherwise.
+    VesinHipAllocate allocate = nullptr;
+    VesinHipRelease release = nullptr;
+    void* allocator_context = nullptr;
     unsigned char last_box[BOX_BYTES] = {}; // box and periodicity of the last call that read them
     BoxGuess guess;                   // when a call starts from that box without reading this call's first
     int single_pass_rest = 0;         // calls left before the single-pass search is tried again after it did not fit
@@ -968,19 +974,23 @@ int device_of(const void* ptr) {
     return attributes.device;
 }
 
-void free_outputs(VesinNeighborList& neighbors) {
-    if (neighbors.pairs != nullptr) {
-        (void)hipFree(neighbors.pairs);
+/// An output array goes back to where it came from: the allocator of the list's caller, or the HIP runtime.
+void release_output(const HipExtras* extras, void* pointer) {
+    if (pointer == nullptr) {
+        return;
     }
-    if (neighbors.shifts != nullptr) {
-        (void)hipFree(neighbors.shifts);
+    if (extras != nullptr && extras->release != nullptr) {
+        extras->release(pointer, extras->allocator_context);
+    } else {
+        (void)hipFree(pointer);
     }
-    if (neighbors.distances != nullptr) {
-        (void)hipFree(neighbors.distances);
-    }
-    if (neighbors.vectors != nullptr) {
-        (void)hipFree(neighbors.vectors);
-    }
+}
+
+void free_outputs(VesinNeighborList& neighbors, const HipExtras* extras) {
+    release_output(extras, neighbors.pairs);
+    release_output(extras, neighbors.shifts);
+    release_output(extras, neighbors.distances);
+    release_output(extras, neighbors.vectors);
     neighbors.pairs = nullptr;
     neighbors.shifts = nullptr;
     neighbors.distances = nullptr;
@@ -1011,7 +1021,7 @@ void size_outputs(VesinNeighborList& neighbors, HipExtras& extras, size_t rows, 
         return;
     }
     if (rows > extras.capacity) {
-        free_outputs(neighbors);
+        free_outputs(neighbors, &extras);
         size_t capacity = rows + rows / 8;
         if (capacity < 1024) {
             capacity = 1024;
@@ -1023,20 +1033,27 @@ void size_outputs(VesinNeighborList& neighbors, HipExtras& extras, size_t rows, 
     }
     const size_t capacity = extras.capacity;
 
-    auto drop = [](auto*& pointer) {
-        if (pointer != nullptr) {
-            (void)hipFree(pointer);
-            pointer = nullptr;
-        }
+    auto drop = [&](auto*& pointer) {
+        release_output(&extras, pointer);
+        pointer = nullptr;
     };
     auto ensure = [&](auto*& pointer, size_t bytes) {
-        if (pointer == nullptr && hipMalloc(reinterpret_cast<void**>(&pointer), bytes) != hipSuccess) {
+        if (pointer != nullptr) {
+            return;
+        }
+        void* memory = nullptr;
+        if (extras.allocate != nullptr) {
+            memory = extras.allocate(bytes, extras.allocator_context);
+        } else if (hipMalloc(&memory, bytes) != hipSuccess) {
             (void)hipGetLastError();
-            pointer = nullptr;
-            free_outputs(neighbors);
+            memory = nullptr;
+        }
+        if (memory == nullptr) {
+            free_outputs(neighbors, &extras);
             extras.capacity = 0;
             throw std::bad_alloc();
         }
+        pointer = static_cast<std::remove_reference_t<decltype(pointer)>>(memory);
     };
 
     ensure(neighbors.pairs, capacity * 2 * sizeof(size_t));
@@ -1203,6 +1220,14 @@ void run_call(
     direct_neighbors(points, n_points, box, periodic, options, neighbors, extras, stream);
 }
 
+/// A list whose arrays were handed to the caller (vesin_hip_detach_outputs) gets arrays of the same size again
+/// before the call starts: every path that writes into kept arrays finds them as it left them.
+void restore_outputs(VesinNeighborList& neighbors, HipExtras& extras, const VesinOptions& options) {
+    if (!extras.fixed_memory && extras.capacity > 0 && neighbors.pairs == nullptr) {
+        size_outputs(neighbors, extras, 0, options);
+    }
+}
+
 void refuse_while_queued(const HipExtras& extras) {
     if (extras.enqueued) {
         throw std::runtime_error(
@@ -1257,6 +1282,7 @@ void neighbors(
     const DeviceGuard guard(device_id);
     HipExtras& extras = extras_of(neighbors);
     refuse_while_queued(extras);
+    restore_outputs(neighbors, extras, options);
     HOST_LAP(1);
     run_call(points, n_points, box, periodic, options, neighbors, extras, stream);
     HOST_LAP(5);
@@ -1281,6 +1307,7 @@ const unsigned long long* neighbors_enqueue(
     const DeviceGuard guard(device_id);
     HipExtras& extras = extras_of(neighbors);
     refuse_while_queued(extras);
+    restore_outputs(neighbors, extras, options);
     if (extras.d_queued_length == nullptr) {
         HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&extras.d_queued_length), 256));
     }
@@ -2728,6 +2755,7 @@ void neighbors_batch(
     const DeviceGuard guard(device_id);
     HipExtras& extras = extras_of(neighbors);
     refuse_while_queued(extras);
+    restore_outputs(neighbors, extras, options);
     extras.timings_valid = false;
     hipStream_t stream = static_cast<hipStream_t>(caller_stream);
     if (options.skin > 0.0) {
@@ -4283,9 +4311,57 @@ void free_neighbors(VesinNeighborList& neighbors) {
             }
         }
     }
-    free_outputs(neighbors);
+    free_outputs(neighbors, static_cast<const HipExtras*>(neighbors.opaque));
     delete static_cast<HipExtras*>(neighbors.opaque);
     neighbors.opaque = nullptr;
+}
+
+void set_output_allocator(VesinNeighborList& neighbors, VesinHipAllocate allocate, VesinHipRelease release, void* context) {
+    if ((allocate == nullptr) != (release == nullptr)) {
+        throw std::runtime_error("`allocate` and `release` come together: both functions, or NULL for both");
+    }
+    int device_count = 0;
+    if (hipGetDeviceCount(&device_count) != hipSuccess || device_count == 0) {
+        (void)hipGetLastError();
+        throw std::runtime_error("no HIP device is available to this process");
+    }
+    if (neighbors.device.device_id < 0 || neighbors.device.device_id >= device_count) {
+        throw std::runtime_error("invalid GPU device_id " + std::to_string(neighbors.device.device_id));
+    }
+    const DeviceGuard guard(neighbors.device.device_id);
+    HipExtras& extras = extras_of(neighbors);
+    refuse_while_queued(extras);
+    // what the list holds goes back the way it came; the next call makes arrays of the same size with the new functions
+    free_outputs(neighbors, &extras);
+    extras.allocate = allocate;
+    extras.release = release;
+    extras.allocator_context = context;
+}
+
+size_t detach_outputs(VesinNeighborList& neighbors) {
+    auto* extras = static_cast<HipExtras*>(neighbors.opaque);
+    if (extras == nullptr) {
+        // no call yet: there is nothing to hand over
+        neighbors.pairs = nullptr;
+        neighbors.shifts = nullptr;
+        neighbors.distances = nullptr;
+        neighbors.vectors = nullptr;
+        return 0;
+    }
+    if (extras->fixed_memory) {
+        throw std::runtime_error("internal error: the arrays of this list are the caller's already");
+    }
+    refuse_while_queued(*extras);
+    neighbors.pairs = nullptr;
+    neighbors.shifts = nullptr;
+    neighbors.distances = nullptr;
+    neighbors.vectors = nullptr;
+    return extras->capacity;
+}
+
+size_t output_capacity(const VesinNeighborList& neighbors) {
+    const auto* extras = static_cast<const HipExtras*>(neighbors.opaque);
+    return extras == nullptr || neighbors.pairs == nullptr ? 0 : extras->capacity;
 }
 
 void pairs_backward(

@@ -94,6 +94,17 @@ void pairs_backward(
 /// Free the outputs and the private state of a GPU list (does not zero the struct).
 void free_neighbors(VesinNeighborList& neighbors);
 
+/// The output arrays of this list come from `allocate` and go back through `release` from now on (NULL for both:
+/// hipMalloc and hipFree); arrays the list holds are released the way they were allocated.
+void set_output_allocator(VesinNeighborList& neighbors, VesinHipAllocate allocate, VesinHipRelease release, void* context);
+
+/// The arrays the list points to become the caller's: the pointers are cleared, the rows they have room for returned;
+/// the next call allocates arrays of that size again before it starts.
+size_t detach_outputs(VesinNeighborList& neighbors);
+
+/// Rows the output arrays of the list have room for.
+size_t output_capacity(const VesinNeighborList& neighbors);
+
 void enable_timings(bool enabled);
 bool last_timings(const VesinNeighborList& neighbors, VesinHipTimings& timings);
 

@@ -6,7 +6,11 @@
 //   - pairs are handed out as int64 views of the size_t arrays the kernels wrote (every index is below 2^63, so
 //     the bits are the same): no conversion pass over 16 bytes per pair (the reference converts, :225-226);
 //   - the kernels run on the caller's current stream (vesin_hip_neighbors_on_stream), ordered after whatever
-//     produced the inputs there, instead of on the null stream.
+//     produced the inputs there, instead of on the null stream;
+//   - with `copy=true` (the default) the rows are not copied out of the list's arrays (the reference clones every
+//     array, :214-256): the list takes its arrays from PyTorch's caching allocator (vesin_hip_set_output_allocator)
+//     and the tensors that go to the caller take them over (vesin_hip_detach_outputs), the next call gets new ones
+//     from the allocator's cache. Arrays much larger than their rows are copied as before.
 // The gradient of distances and vectors with respect to points and box (reference :403-479) is one HIP kernel
 // of the library (vesin_hip_pairs_backward) instead of a chain of tensor operations.
 
@@ -18,11 +22,47 @@
 
 #include <torch/torch.h>
 
+#include <c10/hip/HIPCachingAllocator.h>
 #include <c10/hip/HIPStream.h>
 
 #include "vesin.h"
 
+// What vesin_hip_set_output_allocator is given: device memory from PyTorch's caching allocator (of the current
+// device, for the current stream, like the memory of any tensor made now). Exported for callers that bind the C ABI
+// themselves (the ctypes caller of this package passes their addresses on).
+extern "C" __attribute__((visibility("default"))) void* vesin_amd_torch_allocate(size_t bytes, void* /*context*/) {
+    try {
+        return c10::hip::HIPCachingAllocator::raw_alloc(bytes);
+    } catch (...) {
+        return nullptr; // (the library reports "failed to allocate memory")
+    }
+}
+
+extern "C" __attribute__((visibility("default"))) void vesin_amd_torch_release(void* pointer, void* /*context*/) {
+    try {
+        c10::hip::HIPCachingAllocator::raw_delete(pointer);
+    } catch (...) {
+    }
+}
+
 namespace vesin_amd_torch {
+
+/// A tensor over `rows` rows at the start of an array that came from vesin_amd_torch_allocate; the array goes back to
+/// the allocator with the tensor's storage.
+static torch::Tensor adopt_array(void* data, std::vector<int64_t> shape, torch::ScalarType dtype, const torch::Device& device) {
+    return torch::from_blob(
+        data, shape, [](void* pointer) { vesin_amd_torch_release(pointer, nullptr); },
+        torch::TensorOptions().device(device).dtype(dtype)
+    );
+}
+
+/// The same for callers outside of this file (`torch.ops.vesin_amd.adopt`).
+static torch::Tensor adopt(int64_t pointer, std::vector<int64_t> shape, torch::ScalarType dtype, int64_t device_index) {
+    return adopt_array(
+        reinterpret_cast<void*>(static_cast<uintptr_t>(pointer)), std::move(shape), dtype,
+        torch::Device(torch::kCUDA, static_cast<c10::DeviceIndex>(device_index))
+    );
+}
 
 static VesinDevice to_vesin(const torch::Device& device) {
     if (device.is_cuda()) {
@@ -228,6 +268,17 @@ public:
 
         if (list_.device.type != VesinUnknownDevice && list_.device.type != device.type) {
             vesin_free(&list_);
+            from_torch_allocator_ = false;
+        }
+        if (!from_torch_allocator_ && device.type == VesinCUDA) {
+            const char* error_message = nullptr;
+            const auto status = vesin_hip_set_output_allocator(
+                &list_, device, vesin_amd_torch_allocate, vesin_amd_torch_release, nullptr, &error_message
+            );
+            if (status != EXIT_SUCCESS) {
+                throw std::runtime_error(std::string("failed to compute neighbors: ") + error_message);
+            }
+            from_torch_allocator_ = true;
         }
 
         auto points_data = points.detach().contiguous();
@@ -253,26 +304,48 @@ public:
         const auto on_device = torch::TensorOptions().device(points.device());
         // what the backward step will read must outlive the next calculation on this list: never a view then
         const bool own_copy = copy || through_autograd;
+        // Instead of a copy the tensors take the arrays over, unless those are much larger than their rows (a list
+        // that saw a large system keeps large arrays: a caller who collects the lists of many small systems would
+        // hold all that room).
+        void* const arrays[4] = {list_.pairs, list_.shifts, list_.distances, list_.vectors};
+        bool hand_over = false;
+        if (own_copy && from_torch_allocator_ && length > 0 &&
+            static_cast<size_t>(length) >= vesin_hip_output_capacity(&list_) / 2) {
+            const char* detach_message = nullptr;
+            hand_over = vesin_hip_detach_outputs(&list_, nullptr, &detach_message) == EXIT_SUCCESS;
+        }
         const auto wrap = [&](void* data, std::vector<int64_t> shape, torch::ScalarType dtype) {
             if (length == 0 || data == nullptr) {
                 return torch::empty(shape, on_device.dtype(dtype));
+            }
+            if (hand_over) {
+                return adopt_array(data, shape, dtype, points.device());
             }
             auto view = torch::from_blob(data, shape, on_device.dtype(dtype));
             return own_copy ? view.clone() : view;
         };
 
-        auto pairs = wrap(list_.pairs, {length, 2}, torch::kInt64);
+        auto pairs = wrap(arrays[0], {length, 2}, torch::kInt64);
         auto shifts = torch::Tensor();
         if (options.return_shifts) {
-            shifts = wrap(list_.shifts, {length, 3}, torch::kInt32);
+            shifts = wrap(arrays[1], {length, 3}, torch::kInt32);
         }
         auto distances = torch::Tensor();
         if (options.return_distances) {
-            distances = wrap(list_.distances, {length}, torch::kFloat64);
+            distances = wrap(arrays[2], {length}, torch::kFloat64);
         }
         auto vectors = torch::Tensor();
         if (options.return_vectors) {
-            vectors = wrap(list_.vectors, {length, 3}, torch::kFloat64);
+            vectors = wrap(arrays[3], {length, 3}, torch::kFloat64);
+        }
+        if (hand_over) {
+            // (an array that no tensor took: there is none today, every array the list holds was asked for)
+            const bool taken[4] = {true, shifts.defined(), distances.defined(), vectors.defined()};
+            for (int k = 0; k < 4; k++) {
+                if (arrays[k] != nullptr && !taken[k]) {
+                    vesin_amd_torch_release(arrays[k], nullptr);
+                }
+            }
         }
 
         if (through_autograd) {
@@ -322,9 +395,14 @@ private:
     std::string algorithm_;
     int64_t n_threads_;
     VesinNeighborList list_ = VesinNeighborList();
+    bool from_torch_allocator_ = false; // the arrays of list_ come from PyTorch's caching allocator
 };
 
 } // namespace vesin_amd_torch
+
+TORCH_LIBRARY(vesin_amd, m) {
+    m.def("adopt(int pointer, int[] shape, ScalarType dtype, int device) -> Tensor", &vesin_amd_torch::adopt);
+}
 
 TORCH_LIBRARY(vesin, m) {
     using vesin_amd_torch::NeighborListHolder;
