@@ -279,6 +279,30 @@ int VESIN_API vesin_hip_neighbors_batch_on_stream(
     const char** error_message
 );
 
+/* vesin_hip_neighbors_batch_on_stream in two halves, like vesin_hip_neighbors_enqueue: everything the batch can do
+ * before the host needs an answer from the GPU is queued on `stream` (for a list that saw the same division into
+ * systems before: the whole calculation), and the call returns; vesin_hip_neighbors_collect on the same list
+ * completes it (waits for the queued kernels, starts over with what they reported when the boxes or the systems were
+ * not those of the call before, grows the arrays) and reports its errors. No counterpart in the reference.
+ * Between the two calls `points`, `boxes`, `periodic` and the host array `first_point` must stay as they are;
+ * `first_pair` (host) is written by vesin_hip_neighbors_collect; the list is refused by every other entry point.
+ * The word at `*device_length` says VESIN_HIP_ROWS_PENDING until vesin_hip_neighbors_collect has set it to `length`:
+ * unlike a single system, a batch does not tell work queued behind it how many rows it found. */
+int VESIN_API vesin_hip_neighbors_batch_enqueue(
+    const double (*points)[3],
+    const size_t* first_point,
+    size_t n_systems,
+    const double (*boxes)[3][3],
+    const bool (*periodic)[3],
+    struct VesinDevice device,
+    struct VesinOptions options,
+    struct VesinNeighborList* neighbors,
+    size_t* first_pair,
+    void* stream,
+    const unsigned long long** device_length,
+    const char** error_message
+);
+
 /* Gradient of the pair geometry: given dE/d(distances) and dE/d(vectors) of some scalar E for the rows of a list,
  * ADD dE/d(points) and dE/d(box) to `points_grad` and `box_grad` (the caller zeroes them, or accumulates):
  *     g_k = vectors_grad[k] + distances_grad[k] * vectors[k] / distances[k]

@@ -116,6 +116,21 @@ def get_library():
             ctypes.c_void_p,
             ctypes.POINTER(ctypes.c_char_p),
         ]
+        lib.vesin_hip_neighbors_batch_enqueue.restype = ctypes.c_int
+        lib.vesin_hip_neighbors_batch_enqueue.argtypes = [
+            ctypes.c_void_p,
+            ctypes.POINTER(ctypes.c_size_t),
+            ctypes.c_size_t,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            VesinDevice,
+            VesinOptions,
+            ctypes.POINTER(VesinNeighborList),
+            ctypes.POINTER(ctypes.c_size_t),
+            ctypes.c_void_p,
+            ctypes.POINTER(ctypes.c_void_p),
+            ctypes.POINTER(ctypes.c_char_p),
+        ]
         lib.vesin_hip_pairs_backward.restype = ctypes.c_int
         lib.vesin_hip_pairs_backward.argtypes = [
             ctypes.c_void_p,

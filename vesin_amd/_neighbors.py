@@ -448,8 +448,37 @@ class NeighborList:
         """
         import torch
 
+        device, index, first_point, n_systems, points, boxes, periodic, options = self._batch_arguments(
+            points, first_point, boxes, periodic, quantities
+        )
+        handover = self._torch_allocator(VesinDevice(VesinCUDA, index)) if copy else None
+        torch.cuda.current_stream(device).synchronize()
+        first_pair = np.zeros(n_systems + 1, dtype=np.uint64)
+        error_message = ctypes.c_char_p()
+        status = self._lib.vesin_hip_neighbors_batch(
+            points.data_ptr() if points.shape[0] > 0 else boxes.data_ptr(),
+            first_point.ctypes.data_as(ctypes.POINTER(ctypes.c_size_t)),
+            n_systems,
+            boxes.data_ptr(),
+            periodic.data_ptr(),
+            VesinDevice(VesinCUDA, index),
+            options,
+            ctypes.byref(self._neighbors),
+            first_pair.ctypes.data_as(ctypes.POINTER(ctypes.c_size_t)),
+            ctypes.byref(error_message),
+        )
+        if status != 0:
+            raise RuntimeError(error_message.value.decode("utf8"))
+
+        return self._results(quantities, index, copy, handover), first_pair
+
+    def _batch_arguments(self, points, first_point, boxes, periodic, quantities):
+        """The inputs of a batch as the library takes them (tensors on the points' device, the division into systems
+        as a numpy array, the options), on a list of that device."""
+        import torch
+
         if not isinstance(points, torch.Tensor) or points.device.type != "cuda":
-            raise RuntimeError("compute_batch takes torch tensors on a cuda (HIP) device")
+            raise RuntimeError("a batch takes torch tensors on a cuda (HIP) device")
         device = points.device
         first_point = np.ascontiguousarray(first_point, dtype=np.uint64)
         n_systems = len(first_point) - 1
@@ -486,26 +515,7 @@ class NeighborList:
             self._lib.vesin_free(ctypes.byref(self._neighbors))
             ctypes.memset(ctypes.byref(self._neighbors), 0, ctypes.sizeof(self._neighbors))
             self._allocator_set = False
-        handover = self._torch_allocator(VesinDevice(VesinCUDA, index)) if copy else None
-        torch.cuda.current_stream(device).synchronize()
-        first_pair = np.zeros(n_systems + 1, dtype=np.uint64)
-        error_message = ctypes.c_char_p()
-        status = self._lib.vesin_hip_neighbors_batch(
-            points.data_ptr() if points.shape[0] > 0 else boxes.data_ptr(),
-            first_point.ctypes.data_as(ctypes.POINTER(ctypes.c_size_t)),
-            n_systems,
-            boxes.data_ptr(),
-            periodic.data_ptr(),
-            VesinDevice(VesinCUDA, index),
-            options,
-            ctypes.byref(self._neighbors),
-            first_pair.ctypes.data_as(ctypes.POINTER(ctypes.c_size_t)),
-            ctypes.byref(error_message),
-        )
-        if status != 0:
-            raise RuntimeError(error_message.value.decode("utf8"))
-
-        return self._results(quantities, index, copy, handover), first_pair
+        return device, index, first_point, n_systems, points, boxes, periodic, options
 
     def _results(self, quantities, index, copy, handover):
         """The requested quantities of the call that just ended, as torch tensors: views of the list's arrays, or
@@ -597,9 +607,45 @@ class NeighborList:
         self._queued = (quantities, index, points, box, periodic)
         return torch.as_tensor(_DeviceView(word.value, (1,), "<i8", self), device=f"cuda:{index}")
 
+    def enqueue_batch(self, points, first_point, boxes, periodic=True, quantities: str = "ij"):
+        """``compute_batch`` in two halves (``vesin_hip_neighbors_batch_enqueue``): queues the batch on torch's
+        current stream and returns without waiting for the GPU; ``collect`` completes it and returns what
+        ``compute_batch`` would have, ``(outputs, first_pair)``. The inputs must not be changed in between. The
+        tensor returned here holds -1 until ``collect`` has set it to the number of rows."""
+        import torch
+
+        if self.__dict__.get("_queued") is not None:
+            raise RuntimeError("this calculator has a call pending: collect() it first")
+        device, index, first_point, n_systems, points, boxes, periodic, options = self._batch_arguments(
+            points, first_point, boxes, periodic, quantities
+        )
+        self._torch_allocator(VesinDevice(VesinCUDA, index))
+        first_pair = np.zeros(n_systems + 1, dtype=np.uint64)
+        word = ctypes.c_void_p()
+        error_message = ctypes.c_char_p()
+        status = self._lib.vesin_hip_neighbors_batch_enqueue(
+            points.data_ptr() if points.shape[0] > 0 else boxes.data_ptr(),
+            first_point.ctypes.data_as(ctypes.POINTER(ctypes.c_size_t)),
+            n_systems,
+            boxes.data_ptr(),
+            periodic.data_ptr(),
+            VesinDevice(VesinCUDA, index),
+            options,
+            ctypes.byref(self._neighbors),
+            first_pair.ctypes.data_as(ctypes.POINTER(ctypes.c_size_t)),
+            torch.cuda.current_stream(device).cuda_stream,
+            ctypes.byref(word),
+            ctypes.byref(error_message),
+        )
+        if status != 0:
+            raise RuntimeError(error_message.value.decode("utf8"))
+        # (the inputs and the two host arrays are referred to until the call is collected)
+        self._queued = (quantities, index, points, boxes, periodic, first_point, first_pair)
+        return torch.as_tensor(_DeviceView(word.value, (1,), "<i8", self), device=f"cuda:{index}")
+
     def collect(self, copy: bool = True):
-        """Completes the call that ``enqueue`` started (``vesin_hip_neighbors_collect``) and returns the quantities
-        it asked for, as ``compute`` would have. Errors of the calculation are raised here."""
+        """Completes the call that ``enqueue`` or ``enqueue_batch`` started (``vesin_hip_neighbors_collect``) and
+        returns what ``compute`` or ``compute_batch`` would have. Errors of the calculation are raised here."""
         import torch
 
         queued = self.__dict__.get("_queued")
@@ -611,7 +657,8 @@ class NeighborList:
         if self._lib.vesin_hip_neighbors_collect(ctypes.byref(self._neighbors), ctypes.byref(error_message)) != 0:
             raise RuntimeError(error_message.value.decode("utf8"))
         handover = _torch_handover() if copy and self.hand_over and self._allocator_set else None
-        return self._results(quantities, index, copy, handover)
+        results = self._results(quantities, index, copy, handover)
+        return (results, queued[6]) if len(queued) == 7 else results
 
     def timings(self):
         """Per-stage GPU times (ms) of the last ``compute``; needs ``enable_timings(True)`` beforehand."""

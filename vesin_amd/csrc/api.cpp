@@ -256,7 +256,8 @@ static int neighbors_batch_on(
     VesinNeighborList* neighbors,
     size_t* first_pair,
     void* stream,
-    const char** error_message
+    const char** error_message,
+    const unsigned long long** device_length = nullptr
 ) {
     if (error_message == nullptr) {
         return EXIT_FAILURE;
@@ -302,7 +303,13 @@ static int neighbors_batch_on(
         if (neighbors->device.type == VesinUnknownDevice) {
             neighbors->device = device;
         }
-        vesin_hip::neighbors_batch(points, first_point, n_systems, boxes, periodic, options, *neighbors, first_pair, stream);
+        if (device_length != nullptr) {
+            *device_length = vesin_hip::neighbors_batch_enqueue(
+                points, first_point, n_systems, boxes, periodic, options, *neighbors, first_pair, stream
+            );
+        } else {
+            vesin_hip::neighbors_batch(points, first_point, n_systems, boxes, periodic, options, *neighbors, first_pair, stream);
+        }
     } catch (const std::bad_alloc&) {
         LAST_ERROR = "failed to allocate memory";
         *error_message = LAST_ERROR.c_str();
@@ -349,6 +356,32 @@ extern "C" int vesin_hip_neighbors_batch_on_stream(
 ) {
     return neighbors_batch_on(
         points, first_point, n_systems, boxes, periodic, device, options, neighbors, first_pair, stream, error_message
+    );
+}
+
+extern "C" int vesin_hip_neighbors_batch_enqueue(
+    const double (*points)[3],
+    const size_t* first_point,
+    size_t n_systems,
+    const double (*boxes)[3][3],
+    const bool (*periodic)[3],
+    VesinDevice device,
+    VesinOptions options,
+    VesinNeighborList* neighbors,
+    size_t* first_pair,
+    void* stream,
+    const unsigned long long** device_length,
+    const char** error_message
+) {
+    if (error_message == nullptr) {
+        return EXIT_FAILURE;
+    }
+    if (device_length == nullptr) {
+        return fail(error_message, "`device_length` can not be a NULL pointer");
+    }
+    return neighbors_batch_on(
+        points, first_point, n_systems, boxes, periodic, device, options, neighbors, first_pair, stream, error_message,
+        device_length
     );
 }
 

@@ -865,6 +865,13 @@ struct HipExtras {
                 ));
             }
         }
+        sync(stream);
+    }
+
+    /// Wait for the stream; a queued call (see SuspendedCall) stops at its first wait instead and, once resumed, waits
+    /// for what it had queued up to there only. Not for use inside a `catch` block: a call must not stop with an
+    /// exception in flight.
+    void sync(hipStream_t stream) {
         if (queued != nullptr && queued->stop_at_next_wait) {
             queued->stop_at_next_wait = false;
             HIP_CHECK(hipEventRecord(queued->reached, stream));
@@ -1237,6 +1244,25 @@ void refuse_while_queued(const HipExtras& extras) {
     }
 }
 
+/// What a list needs before a call is queued on it: the device word (saying that the rows are pending) and the stack
+/// the call runs on.
+void begin_queued(HipExtras& extras, hipStream_t stream) {
+    if (extras.d_queued_length == nullptr) {
+        HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&extras.d_queued_length), 256));
+    }
+    if (extras.queued == nullptr) {
+        extras.queued = new SuspendedCall();
+    }
+    // whatever was queued behind an earlier call has read its word by the time this one is overwritten: same stream,
+    // or the caller's own ordering between streams
+    hipLaunchKernelGGL(set_queued_length, dim3(1), dim3(1), 0, stream, extras.d_queued_length, ROWS_PENDING);
+    HIP_CHECK(hipGetLastError());
+    extras.length_published = false;
+    extras.queued_part_sufficed = false;
+    extras.enqueued = true;
+    extras.queued_stream = stream;
+}
+
 /// After the queued call ran to its end: hand on its error, and make the device word say what `length` says unless
 /// the queued kernels did that themselves.
 void finish_queued(VesinNeighborList& neighbors, HipExtras& extras, hipStream_t stream) {
@@ -1308,20 +1334,7 @@ const unsigned long long* neighbors_enqueue(
     HipExtras& extras = extras_of(neighbors);
     refuse_while_queued(extras);
     restore_outputs(neighbors, extras, options);
-    if (extras.d_queued_length == nullptr) {
-        HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&extras.d_queued_length), 256));
-    }
-    if (extras.queued == nullptr) {
-        extras.queued = new SuspendedCall();
-    }
-    // whatever was queued behind an earlier call has read its word by the time this one is overwritten: same stream,
-    // or the caller's own ordering between streams
-    hipLaunchKernelGGL(set_queued_length, dim3(1), dim3(1), 0, stream, extras.d_queued_length, ROWS_PENDING);
-    HIP_CHECK(hipGetLastError());
-    extras.length_published = false;
-    extras.queued_part_sufficed = false;
-    extras.enqueued = true;
-    extras.queued_stream = stream;
+    begin_queued(extras, stream);
     VesinNeighborList* list = &neighbors;
     HipExtras* state = &extras;
     extras.queued->start([=]() { run_call(points, n_points, box, periodic, options, *list, *state, stream); });
@@ -2707,18 +2720,13 @@ bool molecules_batch(
 
 } // namespace
 
-void neighbors_batch(
-    const double (*points)[3],
-    const size_t* first_point,
-    size_t n_systems,
-    const double (*boxes)[3][3],
-    const bool (*periodic)[3],
-    VesinOptions options,
-    VesinNeighborList& neighbors,
-    size_t* first_pair,
-    void* caller_stream
+namespace {
+
+/// What every batched entry point checks before anything is queued.
+void check_batch_inputs(
+    const double (*points)[3], const size_t* first_point, size_t n_systems, const double (*boxes)[3][3],
+    const bool (*periodic)[3], int device_id
 ) {
-    const int device_id = neighbors.device.device_id;
     int device_count = 0;
     if (hipGetDeviceCount(&device_count) != hipSuccess || device_count == 0) {
         (void)hipGetLastError();
@@ -2751,13 +2759,15 @@ void neighbors_batch(
     if (device_of(periodic) != device_id) {
         throw std::runtime_error("`periodic` pointer is not allocated on the GPU of the neighbor list");
     }
+}
 
-    const DeviceGuard guard(device_id);
-    HipExtras& extras = extras_of(neighbors);
-    refuse_while_queued(extras);
-    restore_outputs(neighbors, extras, options);
+/// A batch on a list that has its state and whose inputs were checked, with the list's device current.
+void run_batch(
+    const double (*points)[3], const size_t* first_point, size_t n_systems, const double (*boxes)[3][3],
+    const bool (*periodic)[3], VesinOptions options, VesinNeighborList& neighbors, size_t* first_pair,
+    HipExtras& extras, hipStream_t stream
+) {
     extras.timings_valid = false;
-    hipStream_t stream = static_cast<hipStream_t>(caller_stream);
     if (options.skin > 0.0) {
         verlet_batch(points, first_point, n_systems, boxes, periodic, options, neighbors, first_pair, extras, stream);
         return;
@@ -2768,6 +2778,62 @@ void neighbors_batch(
         extras.verlet_batch = nullptr;
     }
     direct_batch(points, first_point, n_systems, boxes, periodic, options, neighbors, first_pair, extras, stream);
+}
+
+} // namespace
+
+void neighbors_batch(
+    const double (*points)[3],
+    const size_t* first_point,
+    size_t n_systems,
+    const double (*boxes)[3][3],
+    const bool (*periodic)[3],
+    VesinOptions options,
+    VesinNeighborList& neighbors,
+    size_t* first_pair,
+    void* caller_stream
+) {
+    const int device_id = neighbors.device.device_id;
+    check_batch_inputs(points, first_point, n_systems, boxes, periodic, device_id);
+    const DeviceGuard guard(device_id);
+    HipExtras& extras = extras_of(neighbors);
+    refuse_while_queued(extras);
+    restore_outputs(neighbors, extras, options);
+    run_batch(
+        points, first_point, n_systems, boxes, periodic, options, neighbors, first_pair, extras,
+        static_cast<hipStream_t>(caller_stream)
+    );
+}
+
+const unsigned long long* neighbors_batch_enqueue(
+    const double (*points)[3],
+    const size_t* first_point,
+    size_t n_systems,
+    const double (*boxes)[3][3],
+    const bool (*periodic)[3],
+    VesinOptions options,
+    VesinNeighborList& neighbors,
+    size_t* first_pair,
+    void* caller_stream
+) {
+    hipStream_t stream = static_cast<hipStream_t>(caller_stream);
+    const int device_id = neighbors.device.device_id;
+    check_batch_inputs(points, first_point, n_systems, boxes, periodic, device_id);
+    const DeviceGuard guard(device_id);
+    HipExtras& extras = extras_of(neighbors);
+    refuse_while_queued(extras);
+    restore_outputs(neighbors, extras, options);
+    begin_queued(extras, stream);
+    VesinNeighborList* list = &neighbors;
+    HipExtras* state = &extras;
+    extras.queued->start([=]() {
+        run_batch(points, first_point, n_systems, boxes, periodic, options, *list, first_pair, *state, stream);
+    });
+    if (extras.queued->finished) {
+        // an error before the first wait
+        finish_queued(neighbors, extras, stream);
+    }
+    return extras.d_queued_length;
 }
 
 namespace {
@@ -2830,7 +2896,7 @@ void direct_batch(
         } catch (...) {
             // the error may be a consequence of boxes that changed
             failure = std::current_exception();
-            HIP_CHECK(hipStreamSynchronize(stream));
+            HIP_CHECK(hipStreamSynchronize(stream)); // (not extras.sync: a queued call does not stop inside a handler)
             right = extras.mail->batch_changed == 0;
             if (right) {
                 std::rethrow_exception(failure);
@@ -2982,7 +3048,7 @@ bool molecules_batch(
                 setup.first_pair_landing, d_first_pair, (n_systems + 1) * sizeof(size_t), hipMemcpyDeviceToHost, stream
             ));
         }
-        HIP_CHECK(hipStreamSynchronize(stream));
+        extras.sync(stream);
         HIP_CHECK(hipGetLastError());
         const MoleculeStatus found = *setup.molecule_report;
         if (found.periodic != 0) {
@@ -3126,7 +3192,7 @@ void verlet_batch(
         }
         // the snapshot is complete before the call returns: the caller may change points and boxes right after
         HIP_CHECK(hipGetLastError());
-        HIP_CHECK(hipStreamSynchronize(stream));
+        extras.sync(stream);
         // (the rows the candidates were packed from stay where they are, although nothing reads them again: with
         // arrays to allocate anew, a call that computes the candidates again took a third longer, 0.40 against 0.30 ms
         // for 2,000 molecules and 1.58 against 1.16 ms for 100,000)
@@ -3257,7 +3323,7 @@ void verlet_batch(
                 cache.first_pair_landing.data(), d_first_pair, (n_systems + 1) * sizeof(size_t), hipMemcpyDeviceToHost, stream
             ));
         }
-        HIP_CHECK(hipStreamSynchronize(stream));
+        extras.sync(stream);
         HIP_CHECK(hipGetLastError());
 
         if (cache.status->rebuild != 0) {
@@ -3361,7 +3427,7 @@ bool batch_attempt(
         HIP_CHECK(hipMemcpyAsync(
             setup.incoming_periodic.data(), periodic, setup.incoming_periodic.size(), hipMemcpyDeviceToHost, stream
         ));
-        HIP_CHECK(hipStreamSynchronize(stream));
+        extras.sync(stream);
         same_setup =
             setup.valid && !setup.any_open_direction && setup.cutoff == options.cutoff &&
             setup.algorithm == static_cast<int>(options.algorithm) && setup.full_stencil == full_stencil_only() &&
@@ -3478,7 +3544,7 @@ bool batch_attempt(
             HIP_CHECK(hipMemcpyAsync(
                 bounds.data(), d_bounds, n_systems * sizeof(BlockBounds), hipMemcpyDeviceToHost, stream
             ));
-            HIP_CHECK(hipStreamSynchronize(stream));
+            extras.sync(stream);
             unsigned int bad = 0xFFFFFFFFu;
             for (const BlockBounds& found : bounds) {
                 bad = std::min(bad, found.first_bad_coordinate);
@@ -3963,7 +4029,7 @@ bool batch_attempt(
         HIP_CHECK(hipMemcpyAsync(
             setup.first_pair_landing, d_first_pair, (n_systems + 1) * sizeof(size_t), hipMemcpyDeviceToHost, stream
         ));
-        HIP_CHECK(hipStreamSynchronize(stream));
+        extras.sync(stream);
         if (setup_changed()) {
             return false;
         }
@@ -3995,7 +4061,7 @@ bool batch_attempt(
                 if (total > 0) {
                     launch_write(nullptr);
                 }
-                HIP_CHECK(hipStreamSynchronize(stream));
+                extras.sync(stream);
             }
             HIP_CHECK(hipGetLastError());
             std::memcpy(first_pair, setup.first_pair_landing, (n_systems + 1) * sizeof(size_t));
@@ -4041,7 +4107,7 @@ bool batch_attempt(
             cell_scan, d_cell_base, offsets, static_cast<uint32_t>(n_systems), n_slices, static_cast<uint32_t>(n_slots),
             fused_status, d_first_pair, reinterpret_cast<unsigned long long*>(setup.first_pair_landing)
         );
-        HIP_CHECK(hipStreamSynchronize(stream));
+        extras.sync(stream);
         if (speculate && (extras.mail->batch_changed != 0 || (device_grids && extras.mail->batch_total_cells > total_cells))) {
             // other boxes than the grids were picked from, or (which open_grids_kernel rules out) more cells than
             // the buffers were sized for: nothing of this attempt is used, the host picks the grids
@@ -4083,7 +4149,7 @@ bool batch_attempt(
     launch_search_batch<false>(options.full, args, stream);
     exclusive_scan<SCAN_U32>(counts, n_slots, offsets, scan_scratch, stream);
     hipLaunchKernelGGL(publish_status, dim3(1), dim3(1), 0, stream, extras.d_status, offsets + n_slots, &extras.mail_device->status);
-    HIP_CHECK(hipStreamSynchronize(stream));
+    extras.sync(stream);
     if (speculate && (extras.mail->batch_changed != 0 || (device_grids && extras.mail->batch_total_cells > total_cells))) {
         return false;
     }
@@ -4135,7 +4201,7 @@ bool batch_attempt(
         rows_of_systems.n_systems = static_cast<uint32_t>(n_systems);
         sort_pairs(unsorted, final_out, total, n_points, sort_space, stream, rows_of_systems);
     }
-    HIP_CHECK(hipStreamSynchronize(stream));
+    extras.sync(stream);
     HIP_CHECK(hipGetLastError());
     std::memcpy(first_pair, setup.first_pair_landing, (n_systems + 1) * sizeof(size_t));
     neighbors.length = total;

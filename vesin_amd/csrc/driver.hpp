@@ -52,6 +52,21 @@ void neighbors_batch(
     void* stream
 );
 
+/// `neighbors_batch` that comes back as soon as the host would have to wait for the GPU, like `neighbors_enqueue`;
+/// `neighbors_collect` ends it. `first_point` is read and `first_pair` written until then. The device word says that
+/// the rows are pending until `neighbors_collect` has set it.
+const unsigned long long* neighbors_batch_enqueue(
+    const double (*points)[3],
+    const size_t* first_point,
+    size_t n_systems,
+    const double (*boxes)[3][3],
+    const bool (*periodic)[3],
+    VesinOptions options,
+    VesinNeighborList& neighbors,
+    size_t* first_pair,
+    void* stream
+);
+
 /// `neighbors` without any allocation: the rows go to the caller's arrays (device memory of GPU `device_id` holding
 /// `capacity` rows each; the ones that `options` does not request are not touched), the work memory is a fixed
 /// array every GPU holds while the library is loaded. Throws when the system or its list does not fit; `length` then
