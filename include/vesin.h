@@ -286,8 +286,17 @@ int VESIN_API vesin_hip_neighbors_batch_on_stream(
  * not those of the call before, grows the arrays) and reports its errors. No counterpart in the reference.
  * Between the two calls `points`, `boxes`, `periodic` and the host array `first_point` must stay as they are;
  * `first_pair` (host) is written by vesin_hip_neighbors_collect; the list is refused by every other entry point.
- * The word at `*device_length` says VESIN_HIP_ROWS_PENDING until vesin_hip_neighbors_collect has set it to `length`:
- * unlike a single system, a batch does not tell work queued behind it how many rows it found. */
+ * As for a single system, work queued on `stream` behind this call finds the number of rows in the word at
+ * `*device_length` when the queued kernels left the complete list in the arrays: a batch with the division into
+ * systems, the boxes and the options of the call before, unsorted and without a skin (free molecules of up to 64
+ * points each also with other molecules in every call, sorted or not). In every other case the word says
+ * VESIN_HIP_ROWS_PENDING until vesin_hip_neighbors_collect has set it to `length`.
+ *
+ * vesin_hip_batch_first_pair_on_device returns where the kernels of the last batch on the list (queued or not) left
+ * the first row of every system: n_systems + 1 64-bit words in the memory of the GPU, the last one the number of
+ * rows; what `first_pair` receives on the host, for work on the GPU that goes through the rows system by system.
+ * Valid when the device word of a queued batch holds a number of rows, or after the batch has returned or was
+ * collected, until the next call on the list. NULL when the last call was no batch or had no points. */
 int VESIN_API vesin_hip_neighbors_batch_enqueue(
     const double (*points)[3],
     const size_t* first_point,
@@ -302,6 +311,8 @@ int VESIN_API vesin_hip_neighbors_batch_enqueue(
     const unsigned long long** device_length,
     const char** error_message
 );
+
+const unsigned long long* VESIN_API vesin_hip_batch_first_pair_on_device(const struct VesinNeighborList* neighbors);
 
 /* Gradient of the pair geometry: given dE/d(distances) and dE/d(vectors) of some scalar E for the rows of a list,
  * ADD dE/d(points) and dE/d(box) to `points_grad` and `box_grad` (the caller zeroes them, or accumulates):

@@ -61,7 +61,7 @@ def test_ctypes_mirror_has_the_same_layout():
 def test_library_exports_every_declared_symbol():
     with open(HEADER) as fd:
         text = fd.read()
-    declared = re.findall(r"^\w[\w ]*\bVESIN_API\s+(\w+)\s*\(", text, flags=re.M)
+    declared = re.findall(r"^\w[\w *]*\bVESIN_API\s+(\w+)\s*\(", text, flags=re.M)
     assert set(declared) >= {"vesin_neighbors", "vesin_free"}
     lib = _c_api.get_library()
     for name in declared:

@@ -95,8 +95,11 @@ def test_a_batch_in_two_halves_gives_the_rows_of_the_blocking_call(full, is_sort
         lists = _per_system(outputs, first_pair)
         _check(lists, *systems, cutoff, full, is_sorted, f"step {step}")
         stream.synchronize()
-        assert int(seen.item()) == -1, "a batch does not publish its length before collect"
+        # (systems with open directions beside periodic ones: the host picks the grids from the points of every call,
+        # so the queued part never is the whole call)
+        assert int(seen.item()) == -1
         assert int(word.item()) == int(first_pair[-1])
+        assert np.array_equal(calculator.first_pair_on_device().cpu().numpy().astype(np.uint64), first_pair)
         assert float(busy[-1]) == float(1 << 20)
         # the blocking call on the same list gives the same rows (and leaves the list fit for the next queued call)
         again, first_again = calculator.compute_batch(*inputs, quantities="PSdD")
@@ -123,9 +126,22 @@ def test_free_molecules_and_a_skin(is_sorted):
                 move = 0.04 if step < 3 else 0.6
                 systems = ([p + move * rng.normal(size=p.shape) for p in systems[0]], boxes, flags)
             inputs = _on_device(*systems)
-            calculator.enqueue_batch(*inputs, quantities="PSdD")
+            word = calculator.enqueue_batch(*inputs, quantities="PSdD")
+            seen = word.clone()  # queued behind the batch, no host synchronisation in between
+            on_device = calculator.first_pair_on_device()
+            seen_first_pair = on_device.clone() if on_device is not None else None
             outputs, first_pair = calculator.collect()
             _check(_per_system(outputs, first_pair), *systems, cutoff, True, is_sorted, f"skin {skin} step {step}")
+            total = int(first_pair[-1])
+            assert int(word.item()) == total
+            assert int(seen.item()) in (-1, total), f"skin {skin} step {step}"
+            if skin == 0.0 and step == 1:
+                # other molecules than those of the call before, and still the whole call is queued: work behind it
+                # finds the number of rows and every system's first row on the device
+                assert int(seen.item()) == total
+            if int(seen.item()) == total and skin == 0.0:
+                assert np.array_equal(seen_first_pair.cpu().numpy().astype(np.uint64), first_pair)
+            assert np.array_equal(calculator.first_pair_on_device().cpu().numpy().astype(np.uint64), first_pair)
 
 
 def test_errors_other_threads_and_lists_dropped_with_a_batch_pending():
@@ -195,7 +211,28 @@ def test_the_small_cell_batch_queued():
     inputs = _on_device(all_points, all_boxes, flags)
     for is_sorted in (False, True):
         calculator = NeighborList(cutoff=cutoff, full_list=True, sorted=is_sorted)
-        for call in range(3):
-            calculator.enqueue_batch(*inputs, quantities="PSdD")
+        counts = []
+        for call in range(4):
+            word = calculator.enqueue_batch(*inputs, quantities="PSdD")
+            seen = word.clone()
+            on_device = calculator.first_pair_on_device()
+            seen_first_pair = on_device.clone() if on_device is not None else None
             outputs, first_pair = calculator.collect()
             _check(_per_system(outputs, first_pair), all_points, all_boxes, flags, cutoff, True, is_sorted, f"call {call}")
+            counts.append(int(seen.item()))
+            assert int(word.item()) == int(first_pair[-1])
+            if counts[-1] != -1:
+                assert np.array_equal(seen_first_pair.cpu().numpy().astype(np.uint64), first_pair)
+        total = int(first_pair[-1])
+        if is_sorted:
+            # (the search that writes the rows in order has a second wait: its queued part is never the whole call)
+            assert counts == [-1] * 4
+        else:
+            # the list's first batch sizes the arrays; from then on the same systems and boxes are queued whole
+            assert counts == [-1, total, total, total]
+    # a call on a single system in between: no batch, nothing to point at
+    points, box, periodic, _ = configs.config3(0)
+    import torch
+
+    calculator.compute(torch.tensor(points, device="cuda:0"), torch.tensor(box, device="cuda:0"), True, "P")
+    assert calculator.first_pair_on_device() is None

@@ -131,6 +131,8 @@ def get_library():
             ctypes.POINTER(ctypes.c_void_p),
             ctypes.POINTER(ctypes.c_char_p),
         ]
+        lib.vesin_hip_batch_first_pair_on_device.restype = ctypes.c_void_p
+        lib.vesin_hip_batch_first_pair_on_device.argtypes = [ctypes.POINTER(VesinNeighborList)]
         lib.vesin_hip_pairs_backward.restype = ctypes.c_int
         lib.vesin_hip_pairs_backward.argtypes = [
             ctypes.c_void_p,

@@ -515,6 +515,7 @@ class NeighborList:
             self._lib.vesin_free(ctypes.byref(self._neighbors))
             ctypes.memset(ctypes.byref(self._neighbors), 0, ctypes.sizeof(self._neighbors))
             self._allocator_set = False
+        self._last_batch_systems = n_systems
         return device, index, first_point, n_systems, points, boxes, periodic, options
 
     def _results(self, quantities, index, copy, handover):
@@ -642,6 +643,20 @@ class NeighborList:
         # (the inputs and the two host arrays are referred to until the call is collected)
         self._queued = (quantities, index, points, boxes, periodic, first_point, first_pair)
         return torch.as_tensor(_DeviceView(word.value, (1,), "<i8", self), device=f"cuda:{index}")
+
+    def first_pair_on_device(self):
+        """The first row of every system of the last batch as the kernels left it on the GPU
+        (``vesin_hip_batch_first_pair_on_device``): a tensor of n_systems + 1 int64 that refers to the calculator's
+        memory and holds these values until the next call; None when the last call was no batch or had no points. For
+        work queued behind ``enqueue_batch`` that goes through the rows system by system without the host."""
+        import torch
+
+        pointer = self._lib.vesin_hip_batch_first_pair_on_device(ctypes.byref(self._neighbors))
+        n_systems = self.__dict__.get("_last_batch_systems")
+        if not pointer or n_systems is None:
+            return None
+        index = self._neighbors.device.device_id
+        return torch.as_tensor(_DeviceView(pointer, (n_systems + 1,), "<i8", self), device=f"cuda:{index}")
 
     def collect(self, copy: bool = True):
         """Completes the call that ``enqueue`` or ``enqueue_batch`` started (``vesin_hip_neighbors_collect``) and

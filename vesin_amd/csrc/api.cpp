@@ -519,6 +519,13 @@ extern "C" int vesin_hip_detach_outputs(VesinNeighborList* neighbors, size_t* ca
     return EXIT_SUCCESS;
 }
 
+extern "C" const unsigned long long* vesin_hip_batch_first_pair_on_device(const VesinNeighborList* neighbors) {
+    if (neighbors == nullptr || neighbors->device.type != VesinCUDA) {
+        return nullptr;
+    }
+    return vesin_hip::batch_first_pair_on_device(*neighbors);
+}
+
 extern "C" size_t vesin_hip_output_capacity(const VesinNeighborList* neighbors) {
     if (neighbors == nullptr || neighbors->device.type != VesinCUDA) {
         return 0;

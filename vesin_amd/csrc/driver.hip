@@ -779,6 +779,44 @@ __global__ void publish_queued_length(
     *word = complete ? rows : ROWS_PENDING;
 }
 
+/// publish_queued_length for a batch through the single-pass search: the list is complete in the arrays when the
+/// search found nothing it could not handle and, for a call that started from the grids of the call before, the
+/// boxes turned out to be the same (and the cells of grids picked on the device fit their room): what the host checks
+/// after its wait, in the same words.
+__global__ void publish_queued_batch_length(
+    const Mailbox* mail, int speculated, int device_grids, unsigned long long total_cells, unsigned long long row_limit,
+    unsigned long long* word
+) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) {
+        return;
+    }
+    const FusedStatus found = mail->fused;
+    bool complete = found.first_bad_coordinate == 0xFFFFFFFFu && found.general == 0 && found.deferred == 0 &&
+                    found.overflow == 0 && found.chain_timeout == 0;
+    if (speculated != 0) {
+        complete = complete && mail->batch_changed == 0 && (device_grids == 0 || mail->batch_total_cells <= total_cells);
+    }
+    if (row_limit != 0 && found.total_rows > row_limit) {
+        complete = false;
+    }
+    *word = complete ? found.total_rows : ROWS_PENDING;
+}
+
+/// The same for a batch of free molecules: `status` is what the kernels gathered, `total_rows` the end of the scan over
+/// the systems' rows.
+__global__ void publish_queued_molecules_length(
+    const MoleculeStatus* status, const unsigned long long* total_rows, unsigned long long capacity,
+    unsigned long long row_limit, unsigned long long* word
+) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) {
+        return;
+    }
+    const unsigned long long rows = *total_rows;
+    const bool complete = status->periodic == 0 && status->first_bad == 0xFFFFFFFFu && rows <= capacity &&
+                          (row_limit == 0 || rows <= row_limit);
+    *word = complete ? rows : ROWS_PENDING;
+}
+
 __global__ void set_queued_length(unsigned long long* word, unsigned long long value) {
     if (threadIdx.x == 0 && blockIdx.x == 0) {
         *word = value;
@@ -844,6 +882,9 @@ struct HipExtras {
     bool enqueued = false;            // a call was queued and not collected yet
     hipStream_t queued_stream = nullptr;
     unsigned long long* d_queued_length = nullptr;
+    /// Where the systems' first rows of the last batch are on the device (n_systems + 1 words, the last one the number
+    /// of rows), until the next call on the list; nullptr when the last call was no batch.
+    const unsigned long long* batch_first_pair_device = nullptr;
     bool length_published = false;    // the kernels of the queued part were followed by the one that fills that word
     bool queued_part_sufficed = false; // ... and the host found, like that kernel, that they left the complete list
 
@@ -886,6 +927,12 @@ struct HipExtras {
     /// queued call is told, if this is the part of the call that is queued (only such calls pay for the launch).
     /// Returns whether it did: the caller then says, once it has looked, whether the host came to the same conclusion
     /// (`queued_part_sufficed`).
+    /// Whether the next wait is the one a queued call stops at: what is queued before it may be followed by a kernel
+    /// that fills the device word.
+    bool before_the_stop_of_a_queued_call() const {
+        return queued != nullptr && queued->stop_at_next_wait;
+    }
+
     bool publish_length(const QueuedOutcome& outcome, const double* box, const bool* periodic, hipStream_t stream) {
         if (queued != nullptr && queued->stop_at_next_wait) {
             hipLaunchKernelGGL(publish_queued_length, dim3(1), dim3(1), 0, stream, outcome, box, periodic, d_queued_length);
@@ -1215,6 +1262,7 @@ void run_call(
 ) {
     const TraceRange whole_call(options.skin > 0.0 ? "vesin_neighbors (skin)" : "vesin_neighbors");
     extras.timings_valid = false;
+    extras.batch_first_pair_device = nullptr;
     if (options.skin > 0.0) {
         verlet_neighbors(points, n_points, box, periodic, options, neighbors, extras, stream);
         return;
@@ -3027,6 +3075,8 @@ bool molecules_batch(
         exclusive_scan<SCAN_U32>(args.rows_of_system, n_systems, d_first_pair, scan_scratch, stream);
     }
     size_t total = 0;
+    extras.batch_first_pair_device = reinterpret_cast<const unsigned long long*>(d_first_pair);
+    bool published_here = false;
     for (int attempt = 0;; attempt++) {
         if (attempt > 2) {
             throw std::runtime_error("internal error: the rows of a batch of molecules did not settle");
@@ -3047,6 +3097,16 @@ bool molecules_batch(
             HIP_CHECK(hipMemcpyAsync(
                 setup.first_pair_landing, d_first_pair, (n_systems + 1) * sizeof(size_t), hipMemcpyDeviceToHost, stream
             ));
+            if (has_arrays && extras.before_the_stop_of_a_queued_call()) {
+                hipLaunchKernelGGL(
+                    publish_queued_molecules_length, dim3(1), dim3(1), 0, stream, args.status,
+                    reinterpret_cast<const unsigned long long*>(d_first_pair + n_systems),
+                    static_cast<unsigned long long>(args.capacity),
+                    static_cast<unsigned long long>(pair_limit != 0 ? n_points * pair_limit : 0), extras.d_queued_length
+                );
+                extras.length_published = true;
+                published_here = true;
+            }
         }
         extras.sync(stream);
         HIP_CHECK(hipGetLastError());
@@ -3070,6 +3130,7 @@ bool molecules_batch(
             );
         }
         if (total <= args.capacity) {
+            extras.queued_part_sufficed = published_here && attempt == 0;
             break;
         }
     }
@@ -3312,6 +3373,7 @@ void verlet_batch(
             fargs.out.vectors = reinterpret_cast<double*>(neighbors.vectors);
             fargs.capacity = extras.capacity;
             fargs.first_pair = d_first_pair;
+            extras.batch_first_pair_device = d_first_pair;
             fargs.n_systems = static_cast<uint32_t>(n_systems);
             fargs.status = cache.status;
             const size_t wanted = (n_chunks + VERLET_WAVES - 1) / VERLET_WAVES;
@@ -3680,6 +3742,7 @@ bool batch_attempt(
         for (size_t s = 0; s <= n_systems; s++) {
             first_pair[s] = 0;
         }
+        extras.batch_first_pair_device = nullptr; // (no kernel ran)
         return true;
     }
     // the first rows of the systems come to pinned memory and go on to the caller's array from there
@@ -3813,6 +3876,7 @@ bool batch_attempt(
     extras.work.reserve(measure.used);
     Carver carver(extras.work.ptr);
     carve(carver);
+    extras.batch_first_pair_device = d_first_pair;
 
     if (try_in_order && !(same_setup && setup.on_device && setup.work_generation == extras.work.generation &&
                           setup.d_pair_base == d_pair_base)) {
@@ -4107,6 +4171,17 @@ bool batch_attempt(
             cell_scan, d_cell_base, offsets, static_cast<uint32_t>(n_systems), n_slices, static_cast<uint32_t>(n_slots),
             fused_status, d_first_pair, reinterpret_cast<unsigned long long*>(setup.first_pair_landing)
         );
+        extras.batch_first_pair_device = d_first_pair;
+        bool published_here = false;
+        if (extras.before_the_stop_of_a_queued_call()) {
+            hipLaunchKernelGGL(
+                publish_queued_batch_length, dim3(1), dim3(1), 0, stream, extras.mail_device, speculate ? 1 : 0,
+                device_grids ? 1 : 0, static_cast<unsigned long long>(total_cells),
+                static_cast<unsigned long long>(pair_limit != 0 ? n_points * pair_limit : 0), extras.d_queued_length
+            );
+            extras.length_published = true;
+            published_here = true;
+        }
         extras.sync(stream);
         if (speculate && (extras.mail->batch_changed != 0 || (device_grids && extras.mail->batch_total_cells > total_cells))) {
             // other boxes than the grids were picked from, or (which open_grids_kernel rules out) more cells than
@@ -4137,6 +4212,7 @@ bool batch_attempt(
             std::memcpy(first_pair, setup.first_pair_landing, (n_systems + 1) * sizeof(size_t));
             neighbors.length = result.total_rows;
             setup.chain_rest.went_through();
+            extras.queued_part_sufficed = published_here;
             return true;
         }
         if (result.chain_timeout != 0) {
@@ -4423,6 +4499,11 @@ size_t detach_outputs(VesinNeighborList& neighbors) {
     neighbors.distances = nullptr;
     neighbors.vectors = nullptr;
     return extras->capacity;
+}
+
+const unsigned long long* batch_first_pair_on_device(const VesinNeighborList& neighbors) {
+    const auto* extras = static_cast<const HipExtras*>(neighbors.opaque);
+    return extras == nullptr ? nullptr : extras->batch_first_pair_device;
 }
 
 size_t output_capacity(const VesinNeighborList& neighbors) {

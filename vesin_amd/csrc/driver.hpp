@@ -117,6 +117,10 @@ void set_output_allocator(VesinNeighborList& neighbors, VesinHipAllocate allocat
 /// the next call allocates arrays of that size again before it starts.
 size_t detach_outputs(VesinNeighborList& neighbors);
 
+/// Where the kernels of the last batch on this list left the first row of every system (n_systems + 1 words in
+/// device memory, the last one the number of rows); nullptr when the last call was no batch or had no points.
+const unsigned long long* batch_first_pair_on_device(const VesinNeighborList& neighbors);
+
 /// Rows the output arrays of the list have room for.
 size_t output_capacity(const VesinNeighborList& neighbors);
 
