@@ -173,3 +173,103 @@ def test_random_batches_on_one_reused_list(seed):
                     assert np.array_equal(actual[key], in_order[key]), (what, key)
             else:
                 assert_same_list(actual, expected, what=what)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_every_kind_of_call_on_one_calculator(seed):
+    """Every way of calling one calculator, in random order: ``compute`` with copies (which take the list's arrays
+    over) and with views, batches, queued calls and queued batches, with ``sorted``, ``full_list`` and ``skin``
+    changing in between. Every result against the oracle; what a queued call said on the device is either pending or
+    the number of rows; results of earlier calls are checked again later (arrays that were handed over stay what
+    they were whatever the list goes on to do)."""
+    import torch
+
+    rng = np.random.default_rng(430_000 + seed)
+    cutoff = float(rng.choice([1.5, 2.5, 3.7]))
+    calc = NeighborList(cutoff=cutoff, full_list=True)
+    kept = []  # (tensors, expected dict, ordered, what)
+    single = None
+    batch = None
+    for step in range(14):
+        if rng.random() < 0.25:
+            calc.sorted = bool(rng.integers(0, 2))
+        if rng.random() < 0.15:
+            calc.full_list = bool(rng.integers(0, 2))
+        if rng.random() < 0.15:
+            calc.skin = float(rng.choice([0.0, 0.0, 0.4]))
+        full, is_sorted = calc.full_list, calc.sorted
+        kinds = ["compute", "views", "batch", "enqueue", "enqueue_batch"]
+        kind = rng.choice(kinds, p=[0.3, 0.1, 0.25, 0.2, 0.15])
+        letters = "PSdD"
+        what = f"seed {seed} step {step} {kind} sorted={is_sorted} full={full} skin={calc.skin}"
+        if kind in ("compute", "views", "enqueue"):
+            if single is None or rng.random() < 0.5:
+                single = random_system(rng, larger=seed % 5 == 4 and rng.random() < 0.3)
+            else:
+                moved = single[0] + rng.normal(scale=rng.choice([0.01, 0.3]), size=single[0].shape)
+                single = (moved, single[1], single[2])
+            points, box, periodic = single
+            tp = torch.as_tensor(points, device="cuda:0")
+            tb = torch.as_tensor(box, device="cuda:0")
+            expected = oracle.neighbors(points, box, periodic, cutoff, full, False, "ijSdD")
+            if kind == "enqueue":
+                flags = torch.as_tensor(np.array(periodic, dtype=bool), device="cuda:0")
+                word = calc.enqueue(tp.contiguous(), tb.contiguous(), flags, letters)
+                seen = word.clone()
+                outputs = calc.collect(copy=bool(rng.integers(0, 2)))
+                assert int(seen.item()) in (-1, len(outputs[0])), what
+                assert int(word.item()) == len(outputs[0]), what
+            else:
+                outputs = calc.compute(tp, tb, periodic, letters, copy=(kind == "compute"))
+            actual = {NAMES[q]: t.cpu().numpy() for q, t in zip(letters, outputs)}
+            assert_same_list(actual, expected, ordered=is_sorted, what=what + f" n={len(points)} periodic={periodic}")
+            if kind == "compute" and len(kept) < 6:
+                kept.append((outputs, [expected], None, is_sorted, what))
+        else:
+            if batch is None or rng.random() < 0.5:
+                batch = []
+                free = rng.random() < 0.3
+                for _ in range(int(rng.integers(1, 9))):
+                    p, b, f = random_system(rng)
+                    if free:
+                        f = [False] * 3
+                        p = p[: int(rng.integers(1, 60))]
+                    batch.append([p, b, f])
+            else:
+                for s in batch:
+                    s[0] = s[0] + rng.normal(scale=rng.choice([0.01, 0.3]), size=s[0].shape)
+            first_point = np.cumsum([0] + [len(s[0]) for s in batch])
+            args = (
+                torch.as_tensor(np.concatenate([s[0] for s in batch]).reshape(-1, 3), device="cuda:0"),
+                first_point,
+                torch.as_tensor(np.stack([s[1] for s in batch]), device="cuda:0"),
+                np.array([s[2] for s in batch], dtype=bool),
+            )
+            if kind == "enqueue_batch":
+                word = calc.enqueue_batch(*args, letters)
+                seen = word.clone()
+                outputs, first_pair = calc.collect(copy=bool(rng.integers(0, 2)))
+                assert int(seen.item()) in (-1, int(first_pair[-1])), what
+                assert int(word.item()) == int(first_pair[-1]), what
+                on_device = calc.first_pair_on_device()
+                if first_point[-1] > 0:
+                    assert np.array_equal(on_device.cpu().numpy().astype(np.uint64), first_pair), what
+            else:
+                copy = bool(rng.integers(0, 2))
+                outputs, first_pair = calc.compute_batch(*args, letters, copy=copy)
+            whole = {NAMES[q]: t.cpu().numpy() for q, t in zip(letters, outputs)}
+            assert first_pair[0] == 0 and first_pair[-1] == len(whole["pairs"]), what
+            exps = []
+            for k, (p, b, f) in enumerate(batch):
+                rows = slice(int(first_pair[k]), int(first_pair[k + 1]))
+                exp = oracle.neighbors(p, b, f, cutoff, full, False, "ijSdD")
+                exps.append(exp)
+                assert_same_list(
+                    {key: v[rows] for key, v in whole.items()}, exp, ordered=is_sorted,
+                    what=what + f" system {k} n={len(p)} periodic={f}",
+                )
+        # results of earlier calls that were copies (or took the arrays over) are what they were
+        if kept and rng.random() < 0.4:
+            outputs, exps, fp, was_sorted, was = kept[int(rng.integers(0, len(kept)))]
+            actual = {NAMES[q]: t.cpu().numpy() for q, t in zip("PSdD", outputs)}
+            assert_same_list(actual, exps[0], ordered=was_sorted, what="kept result of " + was + " after " + what)
