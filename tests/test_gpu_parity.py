@@ -275,3 +275,40 @@ def test_same_output_twice(monkeypatch):
     second = gpu_neighbors(points, box, periodic, 5.0, True, False, "ijSdD")
     for key in first:
         assert np.array_equal(first[key], second[key]), key
+
+
+@pytest.mark.parametrize("n_points", [300, 6000], ids=["one launch", "searches of the large systems"])
+@pytest.mark.parametrize("periodic", [True, False], ids=["periodic", "open"])
+def test_zeros_of_both_signs_keep_their_sign_in_the_vectors(n_points, periodic):
+    """Coordinates that are +0.0 and -0.0: a component of r_j - r_i is then -0.0 or +0.0 depending on which zero is
+    whose, and the reference adds the shift vector to it, whose components for a zero shift are zeros of a sign that
+    follows the signs of the box (vesin/src/cpu_cell_list.cpp:135-138, vesin/src/types.hpp:232-243): the vectors of
+    the rows must have the reference's bits, signs of zero included, on every path (first call of a list and
+    reused list, sorted and not, full and half)."""
+    rng = np.random.default_rng(202)
+    edge = 9.0 if n_points == 300 else 24.0
+    # (a column of the box with negative entries only makes that component of the zero shift's vector -0.0, and only
+    # then does a difference of -0.0 keep its sign)
+    box = np.diag([edge, -edge, edge]) + np.array([[0.0, -0.3, 0.0], [0.5, 0.0, 0.0], [0.0, -0.4, 0.0]])
+    points = rng.random((n_points, 3)) @ np.abs(box)
+    # a cluster of points on the planes through the origin, zeros of both signs among their coordinates
+    for k in range(60):
+        axis = k % 3
+        points[k] = rng.random(3) * 1.5
+        points[k, axis] = 0.0 if k % 2 == 0 else -0.0
+        if k % 5 == 0:
+            points[k, (axis + 1) % 3] = -0.0
+    cutoff = 2.5
+    for full in (True, False):
+        for is_sorted in (False, True):
+            expected = oracle.canonicalize(oracle.neighbors(points, box, periodic, cutoff, full, False, "ijSdD"))
+            actual = gpu_neighbors(points, box, periodic, cutoff, full=full, sorted=is_sorted)
+            what = f"full={full} sorted={is_sorted}"
+            assert_same_list(actual, expected, ordered=is_sorted, what=what)
+            actual = oracle.canonicalize(actual)
+            negative_zeros = np.signbit(expected["vectors"]) & (expected["vectors"] == 0.0)
+            positive_zeros = ~np.signbit(expected["vectors"]) & (expected["vectors"] == 0.0)
+            assert np.any(positive_zeros) and (np.any(negative_zeros) or not periodic), "the case lost its point"
+            assert np.array_equal(
+                actual["vectors"].view(np.uint64), expected["vectors"].view(np.uint64)
+            ), f"{what}: vectors differ in the sign of a zero"
