@@ -23,8 +23,8 @@ The line carries, next to the throughput:
   and one thread on a bounded sample of the same workload.
 
 ``--config NAME`` makes another configuration the workload of the line (profiling runs use it):
-config0, config1 (default), config1_shuffled, config1_sorted, config2, config3, config3_sorted, config3_single, config4a,
-config4b.
+config0, config1 (default), config1_shuffled, config1_sorted, config1_vectors, config2, config3, config3_sorted,
+config3_single, config4a, config4b.
 """
 
 import argparse
@@ -51,7 +51,7 @@ SEARCH_KERNEL_TRAFFIC = {
 }
 KERNEL_SOURCES = ["device_common.cuh", "geometry.hpp", "cells.cuh", "search.cuh", "fused.cuh"]
 
-CONFIG_NAMES = ["config0", "config1", "config1_shuffled", "config1_sorted", "config2", "config3", "config3_sorted", "config3_single", "config4a",
+CONFIG_NAMES = ["config0", "config1", "config1_shuffled", "config1_sorted", "config1_vectors", "config2", "config3", "config3_sorted", "config3_single", "config4a",
                 "config4b"]
 DESCRIPTIONS = {
     "config0": "config0: 216 atoms, cutoff 5 A, full, sorted, i j S d",
@@ -60,6 +60,7 @@ DESCRIPTIONS = {
     "config1_shuffled": "config1 with its atoms in random order",
     "config1_box_changes": "config1 with a box that differs from the call before on every call",
     "config1_sorted": "config1 with sorted=true (rows in the order of i, j, S)",
+    "config1_vectors": "config1 returning i j S d D (vectors beside the distances: 60 bytes per row)",
     "config2": "config2: 100000 atoms, triclinic, cutoff 6 A, half, sorted, i j S d D",
     "config3": "config3: 4096 replicas of 64 atoms, box 7.134 A, cutoff 10 A, full, i j S d, one batched call",
     "config3_sorted": "config3 with sorted=true (every replica's rows in the order of i, j, S)",
@@ -94,6 +95,9 @@ def host_system(name, replicas=50):
     if name == "config1_sorted":
         points, box, periodic, options = configs.config1(replicas)
         return points, box, periodic, dict(options, sorted=True)
+    if name == "config1_vectors":
+        points, box, periodic, options = configs.config1(replicas)
+        return points, box, periodic, dict(options, quantities="ijSdD")
     if name == "config2":
         return configs.config2()
     if name == "config3_single":
@@ -380,7 +384,7 @@ def other_configs(args, torch, np):
     names = [name for name in ["config0", "config2", "config3", "config3_sorted", "config3_single", "config4a", "config4b"]
              if name != args.config]
     if args.config == "config1":
-        names += ["config1_shuffled", "config1_box_changes", "config1_sorted"]
+        names += ["config1_shuffled", "config1_box_changes", "config1_sorted", "config1_vectors"]
     for name in names:
         workload = Workload(name, args.replicas)
         measured = measure(workload, 20, 5, torch, np)

@@ -67,7 +67,9 @@ struct FusedArgs {
     uint32_t wait_ticks; // and the time it waits at most, in ticks of the 100 MHz clock
 };
 
-/// LDS of one wave.
+/// LDS of one wave. STAGED: with room to line up the vectors of 64 rows on their way to memory (the kernels of calls
+/// that return vectors; the others keep the LDS, and the code, they had without it).
+template <bool STAGED>
 struct FusedWaveShared: SearchTables {
     double tile_x[TILE_POINTS], tile_y[TILE_POINTS], tile_z[TILE_POINTS];
     uint32_t tile_index[TILE_POINTS];
@@ -76,10 +78,12 @@ struct FusedWaveShared: SearchTables {
     uint32_t cand_index[FUSED_SLOTS];
     int32_t cand_shift[FUSED_SLOTS]; // packed: cell shift minus the candidate's own wrap shift
     uint16_t ring[RING];
+    __attribute__((aligned(16))) double vector_stage[STAGED ? 3 * WAVE : 2];
 };
 
+template <bool STAGED>
 struct FusedShared {
-    FusedWaveShared wave[SEARCH_WAVES];
+    FusedWaveShared<STAGED> wave[SEARCH_WAVES];
     uint32_t rows[SEARCH_WAVES];
     uint64_t base;     // first output row of the workgroup
     uint32_t writable; // the workgroup's rows fit the output arrays
@@ -225,6 +229,37 @@ __device__ __forceinline__ uint32_t sweep_columns_wrapped(
     return total;
 }
 
+/// The vectors of n <= 64 consecutive rows (lane l holds row l) go to memory as 16-byte pieces of consecutive
+/// addresses, one piece per lane and store instruction, after they were lined up in the wave's LDS. Stored row by row
+/// instead (16 + 8 bytes per lane, 24 bytes apart), every store instruction leaves holes in the cache lines it
+/// touches for the next one to fill, and rows with vectors reached 3.0 TB/s where rows without reach 4.5.
+__device__ __forceinline__ void store_vector_rows(
+    double* stage, char* rows, uint32_t n, bool active, uint32_t lane, double x, double y, double z
+) {
+    // (the lanes of a wave read what other lanes wrote: the LDS serves a wave's accesses in the order they were
+    // issued, which a fence of wavefront scope tells the compiler to keep; nothing waits for the row stores in flight)
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    if (active) {
+        stage[3 * lane + 0] = x;
+        stage[3 * lane + 1] = y;
+        stage[3 * lane + 2] = z;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    const uint32_t bytes = n * 24u;
+    if (lane * 16u + 16u <= bytes) {
+        stream_store(rows + lane * 16u, VectorHead{stage[2 * lane], stage[2 * lane + 1]});
+    }
+    if (1024u + lane * 16u + 16u <= bytes) {
+        stream_store(rows + 1024u + lane * 16u, VectorHead{stage[2 * WAVE + 2 * lane], stage[2 * WAVE + 2 * lane + 1]});
+    }
+    if ((n & 1u) != 0 && lane == 0) {
+        // an odd number of rows ends with half a piece
+        stream_store(rows + bytes - 8u, stage[3 * n - 1]);
+    }
+}
+
 /// Constants of the replay phase of one work item.
 struct ReplayContext {
     double zero_tx, zero_ty, zero_tz;
@@ -242,9 +277,9 @@ struct ReplayState {
 };
 
 /// Redeem n <= 64 tickets: same rows as `redeem` of the two-pass search, candidates and tile points read from LDS.
-template <bool FULL>
+template <bool FULL, bool STAGED>
 __device__ __forceinline__ void redeem_fused(
-    uint32_t n, ReplayState& state, FusedWaveShared& sh, const SearchOutputs& out, const GridParams& g,
+    uint32_t n, ReplayState& state, FusedWaveShared<STAGED>& sh, const SearchOutputs& out, const GridParams& g,
     const ReplayContext& ctx
 ) {
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
@@ -284,9 +319,16 @@ __device__ __forceinline__ void redeem_fused(
             mz = -tz;
         }
     }
-    const double vx = (xj - xi) + tx;
-    const double vy = (yj - yi) + ty;
-    const double vz = (zj - zi) + tz;
+    // A half list that returns vectors computes only the orientation it keeps, from its own operands (both
+    // orientations alive until the vectors are stored cost registers the kernel does not have). The other one has
+    // the same components up to their signs (r_i - r_j = -(r_j - r_i) exactly, the shift vector of -S is minus that
+    // of S, and the vector of the zero shift only decides the sign of a zero), so the squared distance, a sum of
+    // squares in the same order, is the same either way.
+    const bool flip = !FULL && (oi > oj || (oi == oj && !half_keeps_self_image(sx, sy, sz)));
+    const bool kept_only = !FULL && STAGED;
+    const double vx = kept_only ? ((flip ? xi : xj) - (flip ? xj : xi)) + (flip ? mx : tx) : (xj - xi) + tx;
+    const double vy = kept_only ? ((flip ? yi : yj) - (flip ? yj : yi)) + (flip ? my : ty) : (yj - yi) + ty;
+    const double vz = kept_only ? ((flip ? zi : zj) - (flip ? zj : zi)) + (flip ? mz : tz) : (zj - zi) + tz;
     const double wx = (xi - xj) + mx;
     const double wy = (yi - yj) + my;
     const double wz = (zi - zj) + mz;
@@ -311,7 +353,7 @@ __device__ __forceinline__ void redeem_fused(
                 stream_store(distance_rows + ulane * 8u, d);
                 stream_store(distance_rows + n * 8u + ulane * 8u, d);
             }
-            if (out.vectors != nullptr) {
+            if (!STAGED && out.vectors != nullptr) {
                 char* vector_rows = reinterpret_cast<char*>(out.vectors) + cursor * 24;
                 stream_store(vector_rows + ulane * 24u, VectorHead{vx, vy});
                 stream_store(vector_rows + ulane * 24u + 16u, vz);
@@ -319,9 +361,13 @@ __device__ __forceinline__ void redeem_fused(
                 stream_store(vector_rows + n * 24u + ulane * 24u + 16u, wz);
             }
         }
+        if (STAGED && out.vectors != nullptr) {
+            char* vector_rows = reinterpret_cast<char*>(out.vectors) + cursor * 24;
+            store_vector_rows(sh.vector_stage, vector_rows, n, active, ulane, vx, vy, vz);
+            store_vector_rows(sh.vector_stage, vector_rows + n * 24u, n, active, ulane, wx, wy, wz);
+        }
         state.out_cursor += 2 * n;
     } else {
-        const bool flip = oi > oj || (oi == oj && !half_keeps_self_image(sx, sy, sz));
         if (active) {
             stream_store(reinterpret_cast<char*>(out.pairs) + cursor * 16 + ulane * 16u, PairRow{flip ? oj : oi, flip ? oi : oj});
             if (out.shifts != nullptr) {
@@ -333,11 +379,14 @@ __device__ __forceinline__ void redeem_fused(
             if (out.distances != nullptr) {
                 stream_store(reinterpret_cast<char*>(out.distances) + cursor * 8 + ulane * 8u, sqrt(d2));
             }
-            if (out.vectors != nullptr) {
+            if (!STAGED && out.vectors != nullptr) {
                 char* row = reinterpret_cast<char*>(out.vectors) + cursor * 24 + ulane * 24u;
                 stream_store(row, VectorHead{flip ? wx : vx, flip ? wy : vy});
                 stream_store(row + 16u, flip ? wz : vz);
             }
+        }
+        if (STAGED && out.vectors != nullptr) {
+            store_vector_rows(sh.vector_stage, reinterpret_cast<char*>(out.vectors) + cursor * 24, n, active, ulane, vx, vy, vz);
         }
         state.out_cursor += n;
     }
@@ -519,19 +568,20 @@ __device__ __forceinline__ uint64_t chain_position(
 /// BATCH: many systems in one launch (see search_kernel_batch): the grid is the one of the tile's system, tiles are
 /// taken in their order (systems stay together) and every work item reports its first row, from which the host
 /// learns where each system's rows start. Only used with ORDERED.
+/// STAGED: for calls that return vectors: their rows are lined up in LDS before they are stored (store_vector_rows).
 ///
 /// Five waves per SIMD: the kernel needs 96 vector registers for that (the 32 hit columns among them), one fewer
 /// than the compiler takes when left alone, which would be four waves (measured: the clustered 500,000-atom system
 /// 0.59 -> 0.54 ms, the batch of 4096 small cells 1.78 -> 1.75 ms, the 1,000,000-atom lattice unchanged, being bound
 /// by its row stores; six waves with 8 columns instead of 32 made that one slower).
-template <bool FULL, bool ORDERED, bool BATCH = false>
+template <bool FULL, bool ORDERED, bool BATCH = false, bool STAGED = false>
 __global__ __launch_bounds__(SEARCH_BLOCK) __attribute__((amdgpu_waves_per_eu(5, 5))) void fused_search_kernel(FusedArgs fargs, GridParams single_grid) {
     constexpr int R = 2;
-    __shared__ FusedShared shared;
+    __shared__ FusedShared<STAGED> shared;
     const SearchArgs& args = fargs.search;
     const int lane = lane_id();
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
-    FusedWaveShared& sh = shared.wave[wave];
+    FusedWaveShared<STAGED>& sh = shared.wave[wave];
     GridParams batch_grid;
     const GridParams& g = BATCH ? batch_grid : single_grid;
     // fixed-capacity layout (never in a batch): every cell has the same number of tiles, some of them empty
@@ -795,7 +845,7 @@ __global__ __launch_bounds__(SEARCH_BLOCK) __attribute__((amdgpu_waves_per_eu(5,
         const uint32_t half = unit & 1;
         if (half == 0 ? state.tail < filled[0] : state.tail < filled[1]) {
             // pending tickets still point into the records about to be replaced
-            redeem_fused<FULL>(state.head - state.tail, state, sh, args.out, g, ctx);
+            redeem_fused<FULL, STAGED>(state.head - state.tail, state, sh, args.out, g, ctx);
         }
         const uint32_t k = (item.unit_begin + unit) * WAVE + lane;
         const UnitCandidates u = locate_unit(sh, item.n_batch, item.n_candidates, k, sorted);
@@ -824,7 +874,7 @@ __global__ __launch_bounds__(SEARCH_BLOCK) __attribute__((amdgpu_waves_per_eu(5,
             }
             state.head += __popcll(mask);
             while (state.head - state.tail >= state.batch) {
-                redeem_fused<FULL>(state.batch, state, sh, args.out, g, ctx);
+                redeem_fused<FULL, STAGED>(state.batch, state, sh, args.out, g, ctx);
             }
         }
         if (half == 0) {
@@ -834,7 +884,7 @@ __global__ __launch_bounds__(SEARCH_BLOCK) __attribute__((amdgpu_waves_per_eu(5,
         }
     }
     if (state.head != state.tail) {
-        redeem_fused<FULL>(state.head - state.tail, state, sh, args.out, g, ctx);
+        redeem_fused<FULL, STAGED>(state.head - state.tail, state, sh, args.out, g, ctx);
     }
 }
 
