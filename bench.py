@@ -16,8 +16,8 @@ The line carries, next to the throughput:
   may legitimately differ from the CPU path's);
 * ``other_configs``: the same figures for the other configurations of the baseline (the 216-atom sorted case, the
   triclinic sorted half list, the batch of 4096 small cells, the clustered system without and with periodic
-  directions) and for two variants of the headline workload (atoms in random order; a box that changes with every
-  call). They are parity cases (tests/test_gpu_parity.py), timed here for the record, each next to the CPU path;
+  directions) and for four variants of the headline workload (atoms in random order; a box that changes with every
+  call; sorted=true; vectors returned as well). They are parity cases (tests/test_gpu_parity.py), timed here for the record, each next to the CPU path;
 * ``cpu_baseline``: the reference's CPU path (the compiled reference in oracle/_ref when present, otherwise the C
   restatement in oracle/) timed in the same run on the host cores, in a child process with a time limit: all cores,
   and one thread on a bounded sample of the same workload.
