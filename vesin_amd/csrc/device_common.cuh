@@ -149,6 +149,44 @@ __device__ __forceinline__ void stream_store(void* address, T value) {
     __builtin_nontemporal_store(value, reinterpret_cast<T*>(address));
 }
 
+/// The vectors of up to 64 consecutive rows (lane l holds row l of a block that starts on a multiple of 64 rows; the
+/// rows of lanes [lo, hi) are there) go to memory as 16-byte pieces of consecutive addresses, one piece per lane and
+/// store instruction, after they were lined up in LDS (`stage`: 192 doubles of the wave's own); a first or last row
+/// that starts or ends in the middle of a piece stores that half on its own. Stored row by row (16 + 8 bytes per lane,
+/// 24 bytes apart), every store instruction leaves holes in the cache lines it touches for the next one to fill, and
+/// kernels that are held up by their stores write the vectors at half the rate of their other rows.
+__device__ __forceinline__ void store_vector_block(
+    double* stage, char* block, uint32_t lo, uint32_t hi, bool active, uint32_t lane, double x, double y, double z
+) {
+    // (the lanes of a wave read what other lanes wrote: the LDS serves a wave's accesses in the order they were
+    // issued, which a fence of wavefront scope tells the compiler to keep; nothing waits for the row stores in flight)
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    if (active) {
+        stage[3 * lane + 0] = x;
+        stage[3 * lane + 1] = y;
+        stage[3 * lane + 2] = z;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    const uint32_t begin = 24u * lo;
+    const uint32_t end = 24u * hi;
+#pragma unroll
+    for (uint32_t turn = 0; turn < 2; turn++) {
+        const uint32_t piece = turn * WAVE + lane; // 96 pieces of 16 bytes make 64 rows
+        const uint32_t at = 16u * piece;
+        if (piece < 3 * WAVE / 2) {
+            if (at >= begin && at + 16u <= end) {
+                stream_store(block + at, VectorHead{stage[2 * piece], stage[2 * piece + 1]});
+            } else if (at + 8u == begin && at + 16u <= end) {
+                stream_store(block + at + 8u, stage[2 * piece + 1]);
+            } else if (at >= begin && at + 8u == end) {
+                stream_store(block + at, stage[2 * piece]);
+            }
+        }
+    }
+}
+
 } // namespace vesin_hip
 
 #endif

@@ -4044,8 +4044,13 @@ bool batch_attempt(
             if (in_order_images) {
                 iargs.publish_to = in_order_tiles ? nullptr : publish_to;
                 iargs.build_status = extras.d_status;
-                auto kernel = few_points ? (options.full ? image_write_kernel<true, true> : image_write_kernel<false, true>)
-                                         : (options.full ? image_write_kernel<true, false> : image_write_kernel<false, false>);
+                // (calls that return vectors take the kernels that line them up in LDS before they store them)
+                const bool staged = iargs.out.vectors != nullptr;
+                auto kernel =
+                    staged ? (few_points ? (options.full ? image_write_kernel<true, true, true> : image_write_kernel<false, true, true>)
+                                         : (options.full ? image_write_kernel<true, false, true> : image_write_kernel<false, false, true>))
+                           : (few_points ? (options.full ? image_write_kernel<true, true> : image_write_kernel<false, true>)
+                                         : (options.full ? image_write_kernel<true, false> : image_write_kernel<false, false>));
                 hipLaunchKernelGGL(kernel, image_grid, dim3(IMAGE_BLOCK), 0, stream, iargs);
             }
             if (in_order_tiles) {

@@ -103,11 +103,14 @@ struct ImageCountShared: ImageShared<POINTS> {
     float lo32, hi32;
 };
 
-template <uint32_t POINTS, int WAVES>
+/// STAGED: with room to line up the vectors of 64 rows per wave (the kernels of calls that return vectors).
+template <uint32_t POINTS, int WAVES, bool STAGED>
 struct ImageWriteShared: ImageShared<POINTS> {
     // (first point << 16) | (second point << 8) | image, at the place of the row: what a run of consecutive rows left
     // short of a multiple of 64, and the rows of the points behind it
     uint32_t rows[WAVES][IMAGE_ROWS + WAVE];
+    // the vectors of 64 consecutive rows on their way to memory (store_vector_block), per wave
+    __attribute__((aligned(16))) double vector_stage[WAVES][STAGED ? 3 * WAVE : 2];
 };
 
 /// The system's points by index, and the images that can hold a neighbour in the order of their cell shift.
@@ -482,61 +485,73 @@ __global__ __launch_bounds__(IMAGE_BLOCK) void image_count_kernel(ImageArgs args
 /// Stores the first `count` rows lined up in `rows` as the rows `first_row` ... of the list: 64 consecutive rows per
 /// step, each step ending on a multiple of 64 rows (whole cache lines in every output array; the first step stores
 /// fewer).
-template <typename Shared>
+template <bool STAGED, typename Shared>
 __device__ __forceinline__ void store_image_rows(
-    const Shared& sh, const uint32_t* rows, const GridParams& g, const SearchOutputs& out, bool moved_apart,
-    uint32_t count, uint64_t first_row, int lane
+    const Shared& sh, const uint32_t* rows, double* vector_stage, const GridParams& g, const SearchOutputs& out,
+    bool moved_apart, uint32_t count, uint64_t first_row, int lane
 ) {
     const uint32_t skew = static_cast<uint32_t>(first_row % WAVE);
     for (uint32_t r0 = 0; r0 < count + skew; r0 += WAVE) {
         const uint32_t r = r0 + lane - skew;
-        if (r >= count) {
-            continue; // (before the first row as well: unsigned)
+        const bool active = r < count; // (false before the first row as well: unsigned)
+        double vx = 0.0, vy = 0.0, vz = 0.0;
+        if (active) {
+            const uint32_t ticket = rows[r];
+            const uint32_t i = ticket >> 16;
+            const uint32_t j = (ticket >> 8) & 0xffu;
+            const uint32_t e = ticket & 0xffu;
+            int32_t sx, sy, sz;
+            unpack_shift(sh.q[e], sx, sy, sz);
+            double tx = sh.tx[e];
+            double ty = sh.ty[e];
+            double tz = sh.tz[e];
+            if (moved_apart) {
+                sx += sh.wx[i] - sh.wx[j];
+                sy += sh.wy[i] - sh.wy[j];
+                sz += sh.wz[i] - sh.wz[j];
+                shift_vector(g, sx, sy, sz, tx, ty, tz);
+            }
+            vx = (sh.x[j] - sh.x[i]) + tx;
+            vy = (sh.y[j] - sh.y[i]) + ty;
+            vz = (sh.z[j] - sh.z[i]) + tz;
+            const uint64_t row = first_row + r;
+            stream_store(out.pairs + 2 * row, PairRow{i, j});
+            if (out.shifts != nullptr) {
+                stream_store(out.shifts + 3 * row, ShiftRow{sx, sy, sz});
+            }
+            if (out.distances != nullptr) {
+                stream_store(out.distances + row, sqrt(vx * vx + vy * vy + vz * vz));
+            }
+            if (!STAGED && out.vectors != nullptr) {
+                stream_store(out.vectors + 3 * row, VectorHead{vx, vy});
+                stream_store(out.vectors + 3 * row + 2, vz);
+            }
         }
-        const uint32_t ticket = rows[r];
-        const uint32_t i = ticket >> 16;
-        const uint32_t j = (ticket >> 8) & 0xffu;
-        const uint32_t e = ticket & 0xffu;
-        int32_t sx, sy, sz;
-        unpack_shift(sh.q[e], sx, sy, sz);
-        double tx = sh.tx[e];
-        double ty = sh.ty[e];
-        double tz = sh.tz[e];
-        if (moved_apart) {
-            sx += sh.wx[i] - sh.wx[j];
-            sy += sh.wy[i] - sh.wy[j];
-            sz += sh.wz[i] - sh.wz[j];
-            shift_vector(g, sx, sy, sz, tx, ty, tz);
-        }
-        const double vx = (sh.x[j] - sh.x[i]) + tx;
-        const double vy = (sh.y[j] - sh.y[i]) + ty;
-        const double vz = (sh.z[j] - sh.z[i]) + tz;
-        const uint64_t row = first_row + r;
-        stream_store(out.pairs + 2 * row, PairRow{i, j});
-        if (out.shifts != nullptr) {
-            stream_store(out.shifts + 3 * row, ShiftRow{sx, sy, sz});
-        }
-        if (out.distances != nullptr) {
-            stream_store(out.distances + row, sqrt(vx * vx + vy * vy + vz * vz));
-        }
-        if (out.vectors != nullptr) {
-            stream_store(out.vectors + 3 * row, VectorHead{vx, vy});
-            stream_store(out.vectors + 3 * row + 2, vz);
+        if (STAGED && out.vectors != nullptr) {
+            // the block of 64 rows this step falls into, and its lanes that hold a row
+            const uint64_t block_row = first_row + r0 - skew;
+            const uint32_t lo = r0 == 0 ? skew : 0u;
+            const uint32_t hi = min(static_cast<uint32_t>(WAVE), count + skew - r0);
+            store_vector_block(
+                vector_stage, reinterpret_cast<char*>(out.vectors + 3 * block_row), lo, hi, active,
+                static_cast<uint32_t>(lane), vx, vy, vz
+            );
         }
     }
 }
 
 /// WRITE: one workgroup per system, every wave a run of consecutive first points: their rows are consecutive rows of
 /// the list, lined up in LDS one point after the other and stored whenever they reach a multiple of 64 rows.
-template <bool FULL, bool FEW>
+/// STAGED: for calls that return vectors, which are lined up in LDS before they are stored (store_vector_block).
+template <bool FULL, bool FEW, bool STAGED = false>
 __global__ __launch_bounds__(IMAGE_BLOCK) void image_write_kernel(ImageArgs args) {
     constexpr uint32_t POINTS = FEW ? IMAGE_FEW_POINTS : IMAGE_MAX_POINTS;
     constexpr uint32_t WAVES = FEW ? 1 : IMAGE_WAVES; // of a system
-    __shared__ ImageWriteShared<POINTS, WAVES> shared[FEW ? IMAGE_WAVES : 1];
+    __shared__ ImageWriteShared<POINTS, WAVES, STAGED> shared[FEW ? IMAGE_WAVES : 1];
     const int lane = lane_id();
     const uint32_t wave_of_block = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     const uint32_t wave = FEW ? 0 : wave_of_block;    // within its system
-    ImageWriteShared<POINTS, WAVES>& sh = shared[FEW ? wave_of_block : 0];
+    ImageWriteShared<POINTS, WAVES, STAGED>& sh = shared[FEW ? wave_of_block : 0];
     if (args.publish_to != nullptr && blockIdx.x == 0 && threadIdx.x == 0) {
         OrderedHostStatus report;
         report.found = *args.status;
@@ -569,6 +584,7 @@ __global__ __launch_bounds__(IMAGE_BLOCK) void image_write_kernel(ImageArgs args
     const uint32_t words = args.words;
     const uint64_t* system_hits = args.hits + args.pair_base[system] * words;
     uint32_t* rows = sh.rows[wave];
+    double* vector_stage = sh.vector_stage[wave];
     const SearchOutputs& out = args.out;
 
     const uint32_t per_wave = (n + WAVES - 1) / WAVES;
@@ -638,7 +654,7 @@ __global__ __launch_bounds__(IMAGE_BLOCK) void image_write_kernel(ImageArgs args
             if (whole > staged_row) {
                 // everything up to the last multiple of 64 rows; what is left moves to the front
                 const uint32_t count = static_cast<uint32_t>(whole - staged_row);
-                store_image_rows(sh, rows, g, out, moved_apart, count, staged_row, lane);
+                store_image_rows<STAGED>(sh, rows, vector_stage, g, out, moved_apart, count, staged_row, lane);
                 const uint32_t left = staged - count; // < 64
                 const uint32_t ticket = rows[min(count + lane, IMAGE_ROWS + WAVE - 1)];
                 wave_sync();
@@ -652,7 +668,7 @@ __global__ __launch_bounds__(IMAGE_BLOCK) void image_write_kernel(ImageArgs args
         }
     }
     if (staged != 0) {
-        store_image_rows(sh, rows, g, out, moved_apart, staged, staged_row, lane);
+        store_image_rows<STAGED>(sh, rows, vector_stage, g, out, moved_apart, staged, staged_row, lane);
     }
 }
 
