@@ -42,12 +42,12 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes moved by ONE launch of the single-pass search kernel on the 1M-atom workload, from rocprofv3 --pmc
-# FETCH_SIZE and WRITE_SIZE runs scaled by a device copy of known size (167.2 MB fetched + 3238.3 MB written). The figure belongs to the kernel sources whose
+# FETCH_SIZE and WRITE_SIZE runs scaled by a device copy of known size (166.7 MB fetched + 3238.2 MB written). The figure belongs to the kernel sources whose
 # digest is recorded with it: a run with other sources reports no traffic instead of a stale one.
 SEARCH_KERNEL_TRAFFIC = {
-    "bytes": 3_405_500_000,
+    "bytes": 3_405_000_000,
     "profile": "profiles/fused_search_config1_pmc.txt",
-    "kernel_sources_sha256": "aa14adad1821bdfd20b33d8334a2a86d73a63bd6115e3892d3d8722046b462cc",
+    "kernel_sources_sha256": "328c98660c2d928e30d4d9bc2d87d4aae0645b39d27bfb959108c77a834d4a2f",
 }
 KERNEL_SOURCES = ["device_common.cuh", "geometry.hpp", "cells.cuh", "search.cuh", "fused.cuh"]
 
