@@ -468,7 +468,9 @@ class NeighborList:
             ctypes.byref(error_message),
         )
         if status != 0:
+            self._last_batch_systems = None
             raise RuntimeError(error_message.value.decode("utf8"))
+        self._last_batch_systems = n_systems
 
         return self._results(quantities, index, copy, handover), first_pair
 
@@ -515,7 +517,6 @@ class NeighborList:
             self._lib.vesin_free(ctypes.byref(self._neighbors))
             ctypes.memset(ctypes.byref(self._neighbors), 0, ctypes.sizeof(self._neighbors))
             self._allocator_set = False
-        self._last_batch_systems = n_systems
         return device, index, first_point, n_systems, points, boxes, periodic, options
 
     def _results(self, quantities, index, copy, handover):
@@ -639,7 +640,9 @@ class NeighborList:
             ctypes.byref(error_message),
         )
         if status != 0:
+            self._last_batch_systems = None
             raise RuntimeError(error_message.value.decode("utf8"))
+        self._last_batch_systems = n_systems
         # (the inputs and the two host arrays are referred to until the call is collected)
         self._queued = (quantities, index, points, boxes, periodic, first_point, first_pair)
         return torch.as_tensor(_DeviceView(word.value, (1,), "<i8", self), device=f"cuda:{index}")
@@ -670,6 +673,7 @@ class NeighborList:
         quantities, index = queued[0], queued[1]
         error_message = ctypes.c_char_p()
         if self._lib.vesin_hip_neighbors_collect(ctypes.byref(self._neighbors), ctypes.byref(error_message)) != 0:
+            self._last_batch_systems = None
             raise RuntimeError(error_message.value.decode("utf8"))
         handover = _torch_handover() if copy and self.hand_over and self._allocator_set else None
         results = self._results(quantities, index, copy, handover)

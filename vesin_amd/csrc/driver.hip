@@ -2830,6 +2830,7 @@ void run_batch(
     HipExtras& extras, hipStream_t stream
 ) {
     extras.timings_valid = false;
+    extras.batch_first_pair_device = nullptr; // (until the kernels of this call have a place for the systems' first rows)
     if (options.skin > 0.0) {
         verlet_batch(points, first_point, n_systems, boxes, periodic, options, neighbors, first_pair, extras, stream);
         return;
