@@ -296,7 +296,8 @@ int VESIN_API vesin_hip_neighbors_batch_on_stream(
  * the first row of every system: n_systems + 1 64-bit words in the memory of the GPU, the last one the number of
  * rows; what `first_pair` receives on the host, for work on the GPU that goes through the rows system by system.
  * Valid when the device word of a queued batch holds a number of rows, or after the batch has returned or was
- * collected, until the next call on the list. NULL when the last call was no batch or had no points. */
+ * collected, until the next call on the list. NULL when the last call was no batch or had no points, and while a
+ * queued batch has not got as far as its kernels (then the device word says pending, too). */
 int VESIN_API vesin_hip_neighbors_batch_enqueue(
     const double (*points)[3],
     const size_t* first_point,
